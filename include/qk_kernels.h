@@ -1,0 +1,154 @@
+/* qk_kernels.h -- operator-level C ABI of libqk.so (MI355X / gfx950).
+ *
+ * The reference has no exported per-kernel API: each of its kernels is a compute
+ * pipeline with a fixed contract -- storage buffers in binding order, a small
+ * push-constant block, the dispatch z axis as the slot/token index -- consumed by
+ * makePipe()/disp() (reference src/main.cpp:779-816, 4186-4193).  This header states
+ * those contracts as plain C entry points over device pointers so the engine, the
+ * benchmark and the tests drive the kernels without a model file.  Each function
+ * cites the reference pipeline(s) it stands for (paths relative to the reference tree).
+ *
+ * Conventions
+ *  - every pointer is a DEVICE pointer unless its name ends in _host;
+ *  - `stream` is a hipStream_t passed as void* (NULL = the default stream); all work
+ *    is enqueued on it and nothing synchronises unless stated;
+ *  - weights are raw GGUF blocks, row-major, rows of K elements, tensor base aligned
+ *    to 16 bytes; activations and outputs are fp32;
+ *  - return 0 on success, a negative QKK_E* code otherwise; qkk_last_error() returns
+ *    the message of the calling thread's last failure;
+ *  - there is no CPU fallback: without a HIP device every compute entry point fails
+ *    with QKK_EDEVICE.
+ */
+#ifndef QK_KERNELS_H
+#define QK_KERNELS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define QKK_MAX_SLOTS 16u   /* decode slots per step (reference include/qk.h:21) */
+#define QKK_MAX_USED 16u    /* picks per token (reference shaders/moe_select.comp:8) */
+#define QKK_MAX_EXPERTS 512u
+
+/* ggml tensor type ids (reference src/gguf.h:17-21) */
+enum qkk_type {
+    QKK_F32 = 0,
+    QKK_F16 = 1,
+    QKK_Q8_0 = 8,
+    QKK_Q6_K = 14,
+    QKK_IQ3_XXS = 18,
+    QKK_IQ4_XS = 23,
+};
+
+enum qkk_status {
+    QKK_OK = 0,
+    QKK_EINVAL = -1,   /* null pointer, zero size, misaligned tensor */
+    QKK_ESHAPE = -2,   /* shape the kernels do not cover (K not a block multiple, ...) */
+    QKK_ETYPE = -3,    /* tensor type not supported by this entry point */
+    QKK_EDEVICE = -4,  /* no HIP device / launch failure */
+    QKK_EWORKSPACE = -5 /* workspace too small */
+};
+
+/* Router output of one slot, 160 bytes: the SelT every MoE pipeline binds
+ * (reference shaders/moe_select.comp:15). */
+typedef struct qkk_sel {
+    uint32_t ids[16];
+    float w[16];
+    float w_shared;
+    float pad[7];
+} qkk_sel;
+
+/* One MoE layer's device tensors (reference src/main.cpp:1258-1263, MoeT). */
+typedef struct qkk_moe_layer {
+    uint32_t n_embd, n_ff, n_expert, n_used;
+    int32_t gu_type;   /* QKK_IQ3_XXS */
+    int32_t down_type; /* QKK_IQ4_XS or QKK_Q6_K */
+    const float *gate_inp;       /* [n_expert][n_embd] f32 */
+    const float *gate_inp_shexp; /* [n_embd] f32 */
+    const void *gate_exps;       /* [n_expert][n_ff] rows of n_embd */
+    const void *up_exps;         /* [n_expert][n_ff] rows of n_embd */
+    const void *down_exps;       /* [n_expert][n_embd] rows of n_ff */
+    const void *gate_shexp;      /* Q8_0 [n_ff] rows of n_embd */
+    const void *up_shexp;        /* Q8_0 [n_ff] rows of n_embd */
+    const void *down_shexp;      /* Q8_0 [n_embd] rows of n_ff */
+} qkk_moe_layer;
+
+const char *qkk_last_error(void);
+
+/* Library / device probe. Returns the number of HIP devices (0 when none), fills
+ * arch_host (e.g. "gfx950") when non-NULL. Never fails. */
+int qkk_device_info(char *arch_host, size_t arch_len, uint32_t *n_cu_host);
+
+/* Bytes of one row of k elements of `type`; 0 if unsupported (reference src/gguf.h:36-46). */
+size_t qkk_row_bytes(int type, uint64_t k);
+
+/* out[i] = fp32 value of element i of a block stream, evaluated in the reference's
+ * order with no contraction, so the result is bit-identical to its CPU dequantisation
+ * (reference src/quants.h:70-165). Debug / verification kernel. n_elems must be a
+ * multiple of the block size. */
+int qkk_dequant(int type, const void *W, float *out, uint64_t n_elems, void *stream);
+
+/* Y[b][m] = W[m] . X[b], b < batch <= 16.  Stands for gemv_{f16,q8_0,q6_k,iq4_xs,iq3_xxs}.comp
+ * (reference shaders/gemv_q8_0.comp:29-71, gemv_q6_k.comp:35-96, gemv_iq4_xs.comp:34-77,
+ * gemv_iq3_xxs.comp:30-78, gemv_f16.comp:21-44) and, for QKK_F32, moe_logits.comp:18-37.
+ * X is [batch][K], Y is [batch][M]. */
+int qkk_gemv(int type, const void *W, const float *X, float *Y, uint32_t M, uint32_t K,
+             uint32_t batch, void *stream);
+
+/* Workspace for qkk_moe_decode with up to n_slots slots. */
+size_t qkk_moe_workspace_bytes(const qkk_moe_layer *L_host, uint32_t n_slots);
+
+/* Fused MoE step for n_slots activation rows (reference src/main.cpp:4379-4402 without
+ * the residual/RMS half of add_rms3): router logits, top-n_used select and softmax over
+ * the picks, sigmoid shared gate, routed gate/up with SiLU, routed down, shared expert,
+ * weighted combine.  Stands for moe_logits / moe_select / moe_gateup_iq3 / moe_gateup_q8 /
+ * moe_down_{iq4,q6k} / moe_down_q8b and the a+b sum of add_rms3.comp:27-31.
+ *   X   [n_slots][n_embd]          in
+ *   Y   [n_slots][n_embd]          out: routed + shared contribution (no residual)
+ *   sel [n_slots]                  out: picks in pick order, weights, shared gate
+ *   workspace                      qkk_moe_workspace_bytes(), 256-byte aligned, must be
+ *                                  zero-filled once before its first use; calls sharing
+ *                                  a workspace must not overlap in time.
+ * Expert weights are read once per step however many slots pick the same expert. */
+int qkk_moe_decode(const qkk_moe_layer *L_host, const float *X, float *Y, qkk_sel *sel,
+                   void *workspace, size_t workspace_bytes, uint32_t n_slots, void *stream);
+
+/* Counting sort of (token, pick) pairs by expert (reference shaders/moe_group_pairs.comp:19-51):
+ * offsets[n_expert+1], pairs[n_tokens*n_used] = (token<<4)|pick, ascending inside an expert. */
+int qkk_moe_group_pairs(const qkk_sel *sel, uint32_t n_tokens, uint32_t n_expert, uint32_t n_used,
+                        uint32_t *offsets, uint32_t *pairs, void *stream);
+
+/* LM head + greedy sample (reference src/main.cpp:4406-4419: gemv_q6_k TPR=128, argmax1.comp,
+ * argmax2.comp): tok[b] = argmax_m W[m] . X[b], ties to the lower id.  W is Q6_K [V][K].
+ * logits (optional, [batch][V]) receives the fp32 logits when non-NULL.
+ * workspace: qkk_head_workspace_bytes(V, batch) bytes, zero-filled once before first use. */
+size_t qkk_head_workspace_bytes(uint32_t V, uint32_t batch);
+int qkk_head_argmax(const void *W, const float *X, uint32_t *tok, float *logits, uint32_t V,
+                    uint32_t K, uint32_t batch, void *workspace, size_t workspace_bytes,
+                    void *stream);
+
+/* Two-pass argmax over fp32 rows (reference shaders/argmax1.comp:17-40, argmax2.comp:16-30):
+ * tok[b] = first index of the maximum of logits[b][0..n). */
+int qkk_argmax(const float *logits, uint32_t *tok, uint32_t n, uint32_t batch, void *stream);
+
+/* Batched-prefill dense projection Y[n][m] = X[n] . W[m], W in Q8_0 (reference
+ * shaders/gemm_q8_0.comp:32-101, gemm_q8_0_coopmat2.comp:42-148): fp16 tiles dequantised
+ * in LDS, MFMA with fp32 accumulation.  X [N][K] fp32, Y [N][M] fp32. */
+int qkk_gemm_q8_0(const void *W, const float *X, float *Y, uint32_t M, uint32_t K, uint32_t N,
+                  void *stream);
+
+/* Batched-prefill MoE for n_tokens rows (reference src/main.cpp:5050-5198: moe_logits_gemm,
+ * moe_select, moe_group_pairs, moe_gateup_iq3_grouped_coopmat, moe_down_*_grouped_coopmat,
+ * moe_gateup_q8_coopmat, moe_down_q8_coopmat, the routed fold of add_rms3_grouped.comp:22-27).
+ * Same tensors and outputs as qkk_moe_decode, n_tokens <= 4096. */
+size_t qkk_moe_prefill_workspace_bytes(const qkk_moe_layer *L_host, uint32_t n_tokens);
+int qkk_moe_prefill(const qkk_moe_layer *L_host, const float *X, float *Y, qkk_sel *sel,
+                    void *workspace, size_t workspace_bytes, uint32_t n_tokens, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

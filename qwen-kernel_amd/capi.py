@@ -1,0 +1,206 @@
+"""ctypes binding of include/qk_kernels.h.  Arguments are torch CUDA tensors (device
+memory) or plain ints; every wrapper passes raw device pointers and the current torch
+stream to the C entry point and raises QkError on a negative status."""
+import ctypes as C
+import os
+
+F32, F16, Q8_0, Q6_K, IQ3_XXS, IQ4_XS = 0, 1, 8, 14, 18, 23
+BLOCK = {F32: (1, 4), F16: (1, 2), Q8_0: (32, 34), Q6_K: (256, 210), IQ4_XS: (256, 136), IQ3_XXS: (256, 98)}
+TYPE_NAMES = {F32: "f32", F16: "f16", Q8_0: "q8_0", Q6_K: "q6_k", IQ4_XS: "iq4_xs", IQ3_XXS: "iq3_xxs"}
+
+
+class QkError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__(f"libqk status {code}: {msg}")
+        self.code = code
+
+
+class QkSel(C.Structure):
+    _fields_ = [("ids", C.c_uint32 * 16), ("w", C.c_float * 16), ("w_shared", C.c_float), ("pad", C.c_float * 7)]
+
+
+class _Layer(C.Structure):
+    _fields_ = [("n_embd", C.c_uint32), ("n_ff", C.c_uint32), ("n_expert", C.c_uint32), ("n_used", C.c_uint32),
+                ("gu_type", C.c_int32), ("down_type", C.c_int32),
+                ("gate_inp", C.c_void_p), ("gate_inp_shexp", C.c_void_p), ("gate_exps", C.c_void_p),
+                ("up_exps", C.c_void_p), ("down_exps", C.c_void_p), ("gate_shexp", C.c_void_p),
+                ("up_shexp", C.c_void_p), ("down_shexp", C.c_void_p)]
+
+
+def lib_path():
+    return os.path.join(os.path.dirname(os.path.abspath(__file__)), "libqk.so")
+
+
+_lib = None
+
+
+def lib():
+    """Loads libqk.so from the package directory; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        p = lib_path()
+        if not os.path.exists(p):
+            raise QkError(-4, f"{p} is missing: build it with `make -C qwen-kernel_amd` "
+                              "(or __graft_entry__.build()); there is no fallback path")
+        L = C.CDLL(p)
+        L.qkk_last_error.restype = C.c_char_p
+        L.qkk_row_bytes.restype = C.c_size_t
+        L.qkk_row_bytes.argtypes = [C.c_int, C.c_uint64]
+        L.qkk_moe_workspace_bytes.restype = C.c_size_t
+        L.qkk_moe_workspace_bytes.argtypes = [C.c_void_p, C.c_uint32]
+        L.qkk_moe_prefill_workspace_bytes.restype = C.c_size_t
+        L.qkk_moe_prefill_workspace_bytes.argtypes = [C.c_void_p, C.c_uint32]
+        L.qkk_head_workspace_bytes.restype = C.c_size_t
+        L.qkk_head_workspace_bytes.argtypes = [C.c_uint32, C.c_uint32]
+        L.qkk_device_info.argtypes = [C.c_char_p, C.c_size_t, C.POINTER(C.c_uint32)]
+        vp, u32, u64, sz = C.c_void_p, C.c_uint32, C.c_uint64, C.c_size_t
+        L.qkk_dequant.argtypes = [C.c_int, vp, vp, u64, vp]
+        L.qkk_gemv.argtypes = [C.c_int, vp, vp, vp, u32, u32, u32, vp]
+        L.qkk_moe_decode.argtypes = [vp, vp, vp, vp, vp, sz, u32, vp]
+        L.qkk_moe_group_pairs.argtypes = [vp, u32, u32, u32, vp, vp, vp]
+        L.qkk_head_argmax.argtypes = [vp, vp, vp, vp, u32, u32, u32, vp, sz, vp]
+        L.qkk_argmax.argtypes = [vp, vp, u32, u32, vp]
+        L.qkk_gemm_q8_0.argtypes = [vp, vp, vp, u32, u32, u32, vp]
+        L.qkk_moe_prefill.argtypes = [vp, vp, vp, vp, vp, sz, u32, vp]
+        _lib = L
+    return _lib
+
+
+def _check(rc):
+    if rc < 0:
+        raise QkError(rc, lib().qkk_last_error().decode())
+    return rc
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(0)
+
+
+def _stream():
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def device_info():
+    buf = C.create_string_buffer(64)
+    ncu = C.c_uint32(0)
+    n = lib().qkk_device_info(buf, 64, C.byref(ncu))
+    return {"devices": n, "arch": buf.value.decode(), "cus": ncu.value}
+
+
+def row_bytes(type_, k):
+    return lib().qkk_row_bytes(type_, k)
+
+
+def dequant(type_, W, n_elems, out=None):
+    import torch
+    if out is None:
+        out = torch.empty(n_elems, dtype=torch.float32, device=W.device)
+    _check(lib().qkk_dequant(type_, _ptr(W), _ptr(out), n_elems, _stream()))
+    return out
+
+
+def gemv(type_, W, X, M, K, out=None):
+    """Y[b][m] = W[m] . X[b]; X is [batch, K] (or [K]) fp32 on the device."""
+    import torch
+    batch = 1 if X.dim() == 1 else X.shape[0]
+    if out is None:
+        out = torch.empty((batch, M), dtype=torch.float32, device=X.device)
+    _check(lib().qkk_gemv(type_, _ptr(W), _ptr(X), _ptr(out), M, K, batch, _stream()))
+    return out if X.dim() == 2 else out[0]
+
+
+class MoeLayer:
+    """Device tensors of one MoE layer plus the C struct that names them."""
+
+    def __init__(self, n_embd, n_ff, n_expert, n_used, down_type, gate_inp, gate_inp_shexp, gate_exps, up_exps,
+                 down_exps, gate_shexp, up_shexp, down_shexp, gu_type=IQ3_XXS):
+        self.tensors = dict(gate_inp=gate_inp, gate_inp_shexp=gate_inp_shexp, gate_exps=gate_exps,
+                            up_exps=up_exps, down_exps=down_exps, gate_shexp=gate_shexp, up_shexp=up_shexp,
+                            down_shexp=down_shexp)
+        self.n_embd, self.n_ff, self.n_expert, self.n_used = n_embd, n_ff, n_expert, n_used
+        self.gu_type, self.down_type = gu_type, down_type
+        self.c = _Layer(n_embd, n_ff, n_expert, n_used, gu_type, down_type,
+                        *[t.data_ptr() for t in (gate_inp, gate_inp_shexp, gate_exps, up_exps, down_exps,
+                                                 gate_shexp, up_shexp, down_shexp)])
+
+    def active_bytes(self, n_distinct_experts=None):
+        """Weight bytes one decode step must read (reference src/main.cpp:1239-1241)."""
+        u = self.n_used if n_distinct_experts is None else n_distinct_experts
+        H, F = self.n_embd, self.n_ff
+        per_expert = 2 * F * row_bytes(self.gu_type, H) + H * row_bytes(self.down_type, F)
+        shared = 2 * F * row_bytes(Q8_0, H) + H * row_bytes(Q8_0, F)
+        return self.n_expert * H * 4 + H * 4 + u * per_expert + shared
+
+
+def moe_workspace_bytes(layer, n_slots):
+    return lib().qkk_moe_workspace_bytes(C.byref(layer.c), n_slots)
+
+
+def moe_decode(layer, X, workspace, Y=None, sel=None):
+    """Fused MoE step. X [n_slots, n_embd] fp32. Returns (Y, sel) where sel is a uint8 tensor
+    [n_slots, 160] holding QkSel records."""
+    import torch
+    n = X.shape[0]
+    if Y is None:
+        Y = torch.empty_like(X)
+    if sel is None:
+        sel = torch.zeros((n, 160), dtype=torch.uint8, device=X.device)
+    _check(lib().qkk_moe_decode(C.byref(layer.c), _ptr(X), _ptr(Y), _ptr(sel), _ptr(workspace),
+                                workspace.numel() * workspace.element_size(), n, _stream()))
+    return Y, sel
+
+
+def moe_prefill_workspace_bytes(layer, n_tokens):
+    return lib().qkk_moe_prefill_workspace_bytes(C.byref(layer.c), n_tokens)
+
+
+def moe_prefill(layer, X, workspace, Y=None, sel=None):
+    import torch
+    n = X.shape[0]
+    if Y is None:
+        Y = torch.empty_like(X)
+    if sel is None:
+        sel = torch.zeros((n, 160), dtype=torch.uint8, device=X.device)
+    _check(lib().qkk_moe_prefill(C.byref(layer.c), _ptr(X), _ptr(Y), _ptr(sel), _ptr(workspace),
+                                 workspace.numel() * workspace.element_size(), n, _stream()))
+    return Y, sel
+
+
+def moe_group_pairs(sel, n_tokens, n_expert, n_used):
+    import torch
+    offsets = torch.empty(n_expert + 1, dtype=torch.int32, device=sel.device)
+    pairs = torch.empty(n_tokens * n_used, dtype=torch.int32, device=sel.device)
+    _check(lib().qkk_moe_group_pairs(_ptr(sel), n_tokens, n_expert, n_used, _ptr(offsets), _ptr(pairs), _stream()))
+    return offsets, pairs
+
+
+def head_workspace_bytes(V, batch):
+    return lib().qkk_head_workspace_bytes(V, batch)
+
+
+def head_argmax(W, X, V, K, workspace, want_logits=False):
+    import torch
+    batch = X.shape[0]
+    tok = torch.empty(batch, dtype=torch.int32, device=X.device)
+    logits = torch.empty((batch, V), dtype=torch.float32, device=X.device) if want_logits else None
+    _check(lib().qkk_head_argmax(_ptr(W), _ptr(X), _ptr(tok), _ptr(logits), V, K, batch, _ptr(workspace),
+                                 workspace.numel() * workspace.element_size(), _stream()))
+    return tok, logits
+
+
+def argmax(logits):
+    import torch
+    batch, n = logits.shape
+    tok = torch.empty(batch, dtype=torch.int32, device=logits.device)
+    _check(lib().qkk_argmax(_ptr(logits), _ptr(tok), n, batch, _stream()))
+    return tok
+
+
+def gemm_q8_0(W, X, M, K, out=None):
+    import torch
+    N = X.shape[0]
+    if out is None:
+        out = torch.empty((N, M), dtype=torch.float32, device=X.device)
+    _check(lib().qkk_gemm_q8_0(_ptr(W), _ptr(X), _ptr(out), M, K, N, _stream()))
+    return out

@@ -1,0 +1,327 @@
+// qk_device.h -- device-side helpers shared by the gfx950 kernels: wave64 reductions
+// on DPP, unaligned block-stream loads, half conversion, per-format lane tasks.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "qk_formats.h"
+
+namespace qk {
+
+constexpr int WAVE = 64;
+
+// ---- loads -----------------------------------------------------------------------
+// GGUF blocks are 2-byte (Q8_0, Q6_K, IQ3_XXS) or 8-byte (IQ4_XS) aligned.  gfx950
+// global loads accept any byte alignment, so a block field is fetched with the widest
+// load that covers it; memcpy keeps the access well-defined for the compiler.
+template <typename T>
+__device__ __forceinline__ T ldg(const uint8_t* p)
+{
+    T v;
+    __builtin_memcpy(&v, p, sizeof(T));
+    return v;
+}
+
+__device__ __forceinline__ float h2f(uint16_t h)
+{
+    _Float16 v;
+    __builtin_memcpy(&v, &h, 2);
+    return (float)v;
+}
+
+template <int TYPE>
+__host__ __device__ constexpr size_t qkk_row_bytes_dev(uint64_t k)
+{
+    return TYPE == 8 ? k / 32 * Q8_0_BYTES
+         : TYPE == 14 ? k / 256 * Q6_K_BYTES
+         : TYPE == 23 ? k / 256 * IQ4_XS_BYTES
+         : TYPE == 18 ? k / 256 * IQ3_XXS_BYTES
+         : TYPE == 1 ? k * 2 : k * 4;
+}
+
+// ---- wave64 reductions -------------------------------------------------------------
+// Butterfly inside each row of 16 lanes on DPP (quad_perm xor1, xor2, row_half_mirror,
+// row_mirror): after these four steps every lane of a row holds the row's sum.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v)
+{
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+template <int CTRL>
+__device__ __forceinline__ int dpp_i(int v)
+{
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
+}
+constexpr int DPP_XOR1 = 0xB1;         // quad_perm [1,0,3,2]
+constexpr int DPP_XOR2 = 0x4E;         // quad_perm [2,3,0,1]
+constexpr int DPP_HALF_MIRROR = 0x141; // lanes 0..7 reversed inside each 8
+constexpr int DPP_MIRROR = 0x140;      // lanes 0..15 reversed inside each 16
+
+// Sum over groups of N adjacent lanes (N = 4, 8 or 16); every lane gets its group's sum.
+template <int N>
+__device__ __forceinline__ float group_sum(float v)
+{
+    v += dpp_f<DPP_XOR1>(v);
+    v += dpp_f<DPP_XOR2>(v);
+    if (N >= 8) v += dpp_f<DPP_HALF_MIRROR>(v);
+    if (N >= 16) v += dpp_f<DPP_MIRROR>(v);
+    return v;
+}
+
+__device__ __forceinline__ float readlane_f(float v, int lane)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// Sum over the whole wave; the result is wave-uniform.
+__device__ __forceinline__ float wave_sum(float v)
+{
+    v = group_sum<16>(v);
+    return (readlane_f(v, 0) + readlane_f(v, 16)) + (readlane_f(v, 32) + readlane_f(v, 48));
+}
+
+// Sum over groups of N adjacent lanes for N = 32 (two rows).
+__device__ __forceinline__ float group_sum32(float v)
+{
+    v = group_sum<16>(v);
+    // lanes 0..31 want rows 0+1, lanes 32..63 rows 2+3: swap rows with ds_swizzle-free DPP
+    // row_shr is row-local, so fetch the partner row through bpermute.
+    const int lane = (int)__lane_id();
+    const float o = __builtin_bit_cast(
+        float, __builtin_amdgcn_ds_bpermute((lane ^ 16) << 2, __builtin_bit_cast(int, v)));
+    return v + o;
+}
+
+template <int N>
+__device__ __forceinline__ float lanes_sum(float v)
+{
+    if constexpr (N == 64) return wave_sum(v);
+    else if constexpr (N == 32) return group_sum32(v);
+    else return group_sum<N>(v);
+}
+
+__device__ __forceinline__ float wave_max(float v)
+{
+    v = fmaxf(v, dpp_f<DPP_XOR1>(v));
+    v = fmaxf(v, dpp_f<DPP_XOR2>(v));
+    v = fmaxf(v, dpp_f<DPP_HALF_MIRROR>(v));
+    v = fmaxf(v, dpp_f<DPP_MIRROR>(v));
+    return fmaxf(fmaxf(readlane_f(v, 0), readlane_f(v, 16)),
+                 fmaxf(readlane_f(v, 32), readlane_f(v, 48)));
+}
+
+__device__ __forceinline__ uint32_t wave_min_u32(uint32_t v)
+{
+    int x = (int)v; // callers pass values < 2^31
+    x = min(x, dpp_i<DPP_XOR1>(x));
+    x = min(x, dpp_i<DPP_XOR2>(x));
+    x = min(x, dpp_i<DPP_HALF_MIRROR>(x));
+    x = min(x, dpp_i<DPP_MIRROR>(x));
+    const int a = min(__builtin_amdgcn_readlane(x, 0), __builtin_amdgcn_readlane(x, 16));
+    const int b = min(__builtin_amdgcn_readlane(x, 32), __builtin_amdgcn_readlane(x, 48));
+    return (uint32_t)min(a, b);
+}
+
+// ---- per-format lane tasks -----------------------------------------------------------
+// Every quantised format is cut so that ONE LANE owns 32 weights of a row per pass and a
+// wave covers 2048 consecutive weights: Q8_0 one block per lane; IQ4_XS one 32-weight
+// sub-block; IQ3_XXS one 32-weight group (8 grid bytes + its aux word); Q6_K four runs of
+// 8 weights that share 8 qh bytes.  XS is the lane's slice of the activation row.
+
+struct XSlice {
+    float v[32];
+};
+
+// Where the lane's 32 activations live, as four runs of 8 floats: offset of run c.
+template <int TYPE>
+__device__ __forceinline__ int xrun_offset(int lane_in_row, int c)
+{
+    if constexpr (TYPE == 14) { // Q6_K: block = lane/8, half n = (lane%8)/4, l0 = 8*(lane%4)
+        const int b = lane_in_row >> 3, n = (lane_in_row >> 2) & 1, l0 = (lane_in_row & 3) * 8;
+        return b * 256 + n * 128 + c * 32 + l0;
+    } else {
+        return lane_in_row * 32 + c * 8;
+    }
+}
+
+template <int TYPE>
+__device__ __forceinline__ void load_xslice(XSlice& xs, const float* __restrict__ x, int lane_in_row)
+{
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        const float4* p = (const float4*)(x + xrun_offset<TYPE>(lane_in_row, c));
+        const float4 a = p[0], b = p[1];
+        xs.v[c * 8 + 0] = a.x; xs.v[c * 8 + 1] = a.y; xs.v[c * 8 + 2] = a.z; xs.v[c * 8 + 3] = a.w;
+        xs.v[c * 8 + 4] = b.x; xs.v[c * 8 + 5] = b.y; xs.v[c * 8 + 6] = b.z; xs.v[c * 8 + 7] = b.w;
+    }
+}
+
+// IQ3_XXS codebook in device memory (one copy per translation unit; 1 KiB).
+static __device__ const uint32_t g_iq3xxs_grid[256] = {QK_IQ3XXS_GRID_ROWS};
+
+// LDS tables used by the IQ formats.
+struct IqTables {
+    uint32_t grid[256];
+    float iq4[16];
+};
+
+// Bytes of weights one lane fetches per pass, held in registers between the load and the
+// arithmetic so several rows can be in flight.
+template <int TYPE>
+struct LaneW;
+
+template <>
+struct LaneW<8> { // Q8_0
+    uint32_t q[8];
+    uint16_t d;
+    __device__ __forceinline__ void load(const uint8_t* row, int lane_in_row)
+    {
+        const uint8_t* p = row + (size_t)lane_in_row * Q8_0_BYTES;
+        d = ldg<uint16_t>(p);
+        const uint4 a = ldg<uint4>(p + 2), b = ldg<uint4>(p + 18);
+        q[0] = a.x; q[1] = a.y; q[2] = a.z; q[3] = a.w;
+        q[4] = b.x; q[5] = b.y; q[6] = b.z; q[7] = b.w;
+    }
+    __device__ __forceinline__ float dot(const XSlice& xs, const float*, const IqTables*, int) const
+    {
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) s += (float)(int8_t)(q[i] >> (8 * j)) * xs.v[i * 4 + j];
+        }
+        return h2f(d) * s;
+    }
+};
+
+template <>
+struct LaneW<14> { // Q6_K
+    uint2 qa, qb, qh;
+    uint32_t sc4; // the four sub-scales of this lane's runs, one per byte
+    uint16_t d;
+    __device__ __forceinline__ void load(const uint8_t* row, int lane_in_row)
+    {
+        const int b = lane_in_row >> 3, n = (lane_in_row >> 2) & 1, l0 = (lane_in_row & 3) * 8;
+        const uint8_t* p = row + (size_t)b * Q6_K_BYTES;
+        qa = ldg<uint2>(p + 64 * n + l0);
+        qb = ldg<uint2>(p + 64 * n + 32 + l0);
+        qh = ldg<uint2>(p + Q6_K_QH + 32 * n + l0);
+        // scales 8n + is + {0,2,4,6}, is = l0/16: fetch the 8 scales of this half
+        const uint2 s8 = ldg<uint2>(p + Q6_K_SC + 8 * n);
+        const int is = l0 >> 4;
+        const uint32_t lo = is ? (s8.x >> 8) : s8.x, hi = is ? (s8.y >> 8) : s8.y;
+        sc4 = (lo & 0xFFu) | ((lo >> 8) & 0xFF00u) | ((hi & 0xFFu) << 16) | ((hi << 8) & 0xFF000000u);
+        d = ldg<uint16_t>(p + Q6_K_D);
+    }
+    // xsum[c] = sum of run c of the activations (the -32 offset is applied through it)
+    __device__ __forceinline__ float dot(const XSlice& xs, const float* xsum, const IqTables*, int) const
+    {
+        float tot = 0.f;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const uint2 ql = (c & 1) ? qb : qa;
+            const int sh = 2 * c;
+            float s = 0.f;
+#pragma unroll
+            for (int w = 0; w < 2; w++) {
+                const uint32_t l4 = w ? ql.y : ql.x, h4 = w ? qh.y : qh.x;
+                const uint32_t nib = (c >= 2 ? (l4 >> 4) : l4) & 0x0F0F0F0Fu;
+                const uint32_t q4 = nib | (((h4 >> sh) << 4) & 0x30303030u);
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    s += (float)((q4 >> (8 * j)) & 0xFFu) * xs.v[c * 8 + w * 4 + j];
+            }
+            const float scv = (float)(int8_t)(sc4 >> (8 * c));
+            tot += scv * (s - 32.f * xsum[c]);
+        }
+        return h2f(d) * tot;
+    }
+};
+
+template <>
+struct LaneW<23> { // IQ4_XS
+    uint4 q;
+    uint2 hdr; // d | scales_h<<16, scales_l[4]
+    __device__ __forceinline__ void load(const uint8_t* row, int lane_in_row)
+    {
+        const int b = lane_in_row >> 3, ib = lane_in_row & 7;
+        const uint8_t* p = row + (size_t)b * IQ4_XS_BYTES;
+        hdr = ldg<uint2>(p);
+        q = ldg<uint4>(p + IQ4_XS_QS + 16 * ib);
+    }
+    __device__ __forceinline__ float dot(const XSlice& xs, const float*, const IqTables* tab, int lane_in_row) const
+    {
+        const float* lut = tab->iq4; // the codebook as floats in LDS
+        const int ib = lane_in_row & 7;
+        const uint32_t sh = hdr.x >> 16;
+        const int ls = (int)(((hdr.y >> (4 * ib)) & 0xFu) | (((sh >> (2 * ib)) & 3u) << 4)) - 32;
+        const uint32_t qq[4] = {q.x, q.y, q.z, q.w};
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint32_t byte = (qq[i] >> (8 * j)) & 0xFFu;
+                s += lut[byte & 15u] * xs.v[i * 4 + j];
+                s += lut[byte >> 4] * xs.v[16 + i * 4 + j];
+            }
+        }
+        return h2f((uint16_t)hdr.x) * (float)ls * s;
+    }
+};
+
+template <>
+struct LaneW<18> { // IQ3_XXS
+    uint2 g;      // 8 grid indices
+    uint32_t aux; // 4 x 7-bit sign selectors + 4-bit scale
+    uint16_t d;
+    __device__ __forceinline__ void load(const uint8_t* row, int lane_in_row)
+    {
+        const int b = lane_in_row >> 3, ib = lane_in_row & 7;
+        const uint8_t* p = row + (size_t)b * IQ3_XXS_BYTES;
+        d = ldg<uint16_t>(p);
+        g = ldg<uint2>(p + IQ3_XXS_QS + 8 * ib);
+        aux = ldg<uint32_t>(p + IQ3_XXS_AUX + 4 * ib);
+    }
+    __device__ __forceinline__ float dot(const XSlice& xs, const float*, const IqTables* tab, int) const
+    {
+        const uint32_t* grid = tab->grid; // 256 codewords in LDS
+        float s = 0.f;
+#pragma unroll
+        for (int l = 0; l < 4; l++) {
+            const uint32_t s7 = (aux >> (7 * l)) & 127u;
+            const uint32_t sg = s7 | ((__builtin_popcount(s7) & 1u) << 7);
+            const uint32_t gw = l < 2 ? g.x : g.y;
+#pragma unroll
+            for (int hh = 0; hh < 2; hh++) {
+                const uint32_t cw = grid[(gw >> (16 * (l & 1) + 8 * hh)) & 0xFFu];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const float mag = (float)((cw >> (8 * j)) & 0xFFu);
+                    const uint32_t neg = (sg << (31 - (4 * hh + j))) & 0x80000000u;
+                    const float xv = __builtin_bit_cast(
+                        float, __builtin_bit_cast(uint32_t, xs.v[l * 8 + hh * 4 + j]) ^ neg);
+                    s += mag * xv;
+                }
+            }
+        }
+        return h2f(d) * (0.5f + (float)(aux >> 28)) * 0.5f * s;
+    }
+};
+
+__device__ __forceinline__ void fill_iq_tables(IqTables& t, const uint32_t* __restrict__ grid_g,
+                                               int tid, int nthreads)
+{
+    constexpr int8_t kv[16] = {QK_IQ4NL_VALUES};
+    for (int i = tid; i < 256; i += nthreads) t.grid[i] = grid_g[i];
+    if (tid < 16) {
+        float v = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; i++) v = tid == i ? (float)kv[i] : v;
+        t.iq4[tid] = v;
+    }
+}
+
+
+} // namespace qk

@@ -1,0 +1,383 @@
+// qk_moe.hip -- fused Qwen3-MoE decode step for gfx950.
+//
+// Three launches per step:
+//   1. route:   router logits (F32 rows) + shared-expert gate dot + shared gate/up (Q8_0);
+//               the block that finishes last picks the top-n_used experts and writes Sel.
+//   2. gate/up: routed IQ3_XXS gate and up rows of the picked experts, SiLU gating -> h.
+//   3. down:    routed down rows (IQ4_XS or Q6_K) weighted by the router, shared down row
+//               (Q8_0) weighted by the sigmoid gate, summed into y.
+#include "qk_device.h"
+#include "qk_host.h"
+
+namespace qk {
+
+struct MoeDims {
+    uint32_t H, F, E, k;
+};
+
+// Workspace layout (floats unless noted), per slot s:
+//   logits  [E + 1]  (entry E = shared gate dot), stride LSTRIDE
+//   h       [(k + 1) * F]
+//   counter u32 (one per slot), after everything else
+__host__ __device__ inline uint32_t lstride(uint32_t E) { return (E + 1 + 63) & ~63u; }
+
+struct MoeWs {
+    float* logits;
+    float* h;
+    uint32_t* counter;
+};
+
+static size_t ws_bytes(const MoeDims& d, uint32_t n_slots)
+{
+    return ((size_t)n_slots * lstride(d.E) + (size_t)n_slots * (d.k + 1) * d.F) * 4 + 256;
+}
+
+static MoeWs ws_carve(void* ws, const MoeDims& d, uint32_t n_slots)
+{
+    MoeWs w;
+    // counters first so they stay 256-byte aligned with the buffer
+    w.counter = (uint32_t*)ws;
+    w.logits = (float*)((uint8_t*)ws + 256);
+    w.h = w.logits + (size_t)n_slots * lstride(d.E);
+    return w;
+}
+
+// ---- selector --------------------------------------------------------------------------
+// One wave; lane L owns logits L, L+64, ...  Picks n_used times the maximum, lower id on
+// ties; non-finite logits count as -3.4e38 (reference shaders/moe_select.comp:28-34, 53-63).
+__device__ static void select_wave(const float* __restrict__ logits, uint32_t E, uint32_t k,
+                                   qkk_sel* __restrict__ out)
+{
+    constexpr float FLOOR = -3.4e38f;
+    const int lane = threadIdx.x & 63;
+    float v[QKK_MAX_EXPERTS / 64];
+#pragma unroll
+    for (int i = 0; i < (int)(QKK_MAX_EXPERTS / 64); i++) {
+        const uint32_t e = lane + 64 * i;
+        float l = e < E ? logits[e] : FLOOR;
+        if (isnan(l) || isinf(l)) l = FLOOR;
+        v[i] = l;
+    }
+    float picked = 0.f, top = 0.f, wsum = 0.f, myw = 0.f;
+    uint32_t myid = 0;
+    for (uint32_t r = 0; r < k; r++) {
+        float bv = v[0];
+        uint32_t bi = lane;
+#pragma unroll
+        for (int i = 1; i < (int)(QKK_MAX_EXPERTS / 64); i++)
+            if (v[i] > bv) { bv = v[i]; bi = lane + 64 * i; }
+        const float m = wave_max(bv);
+        const uint32_t id = wave_min_u32(bv == m ? bi : 0x7FFFFFFFu);
+        // retire the winner
+#pragma unroll
+        for (int i = 0; i < (int)(QKK_MAX_EXPERTS / 64); i++)
+            if ((uint32_t)(lane + 64 * i) == id) v[i] = FLOOR;
+        if (r == 0) top = m;
+        picked = expf(m - top);
+        wsum += picked;
+        if ((uint32_t)lane == r) { myw = picked; myid = min(id, E - 1); }
+    }
+    if ((uint32_t)lane < k) {
+        out->ids[lane] = myid;
+        out->w[lane] = myw / wsum;
+    }
+}
+
+// ---- launch 1: router + shared gate/up + select ---------------------------------------
+// Wave tasks: [0, E] F32 rows (E = the shared gate row), then F shared gate/up row pairs.
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ gate_inp,
+                                                        const float* __restrict__ gate_inp_shexp,
+                                                        const uint8_t* __restrict__ gate_shexp,
+                                                        const uint8_t* __restrict__ up_shexp,
+                                                        const float* __restrict__ X, MoeWs ws,
+                                                        qkk_sel* __restrict__ sel, MoeDims d)
+{
+    __shared__ uint32_t s_last;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t slot = blockIdx.y;
+    const float* x = X + (size_t)slot * d.H;
+    float* logits = ws.logits + (size_t)slot * lstride(d.E);
+    float* h = ws.h + (size_t)slot * (d.k + 1) * d.F;
+    const uint32_t n_dense = d.E + 1, n_tasks = n_dense + d.F;
+    const uint32_t q8_row = d.H / 32 * Q8_0_BYTES;
+
+    for (uint32_t t = blockIdx.x * 4 + wave; t < n_tasks; t += gridDim.x * 4) {
+        if (t < n_dense) {
+            const float4* row = (const float4*)(t < d.E ? gate_inp + (size_t)t * d.H : gate_inp_shexp);
+            const float4* xv = (const float4*)x;
+            float a0 = 0.f, a1 = 0.f;
+            for (uint32_t c = lane; c < d.H / 4; c += 64) {
+                const float4 w = row[c], xx = xv[c];
+                a0 += w.x * xx.x + w.y * xx.y;
+                a1 += w.z * xx.z + w.w * xx.w;
+            }
+            const float s = wave_sum(a0 + a1);
+            if (lane == 0) logits[t] = s;
+        } else {
+            const uint32_t r = t - n_dense;
+            float g = 0.f, u = 0.f;
+            for (uint32_t b0 = 0; b0 < d.H / 32; b0 += 64) {
+                if (b0 + lane < d.H / 32) {
+                    XSlice xs;
+                    load_xslice<QKK_Q8_0>(xs, x + b0 * 32, lane);
+                    LaneW<QKK_Q8_0> wg, wu;
+                    wg.load(gate_shexp + (size_t)r * q8_row + (size_t)b0 * Q8_0_BYTES, lane);
+                    wu.load(up_shexp + (size_t)r * q8_row + (size_t)b0 * Q8_0_BYTES, lane);
+                    g += wg.dot(xs, nullptr, nullptr, lane);
+                    u += wu.dot(xs, nullptr, nullptr, lane);
+                }
+            }
+            g = wave_sum(g);
+            u = wave_sum(u);
+            if (lane == 0) h[(size_t)d.k * d.F + r] = (g / (1.f + expf(-g))) * u;
+        }
+    }
+
+    // last block of this slot runs the selector
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) s_last = atomicAdd(&ws.counter[slot], 1u) == gridDim.x - 1 ? 1u : 0u;
+    __syncthreads();
+    if (s_last && wave == 0) {
+        __threadfence();
+        const volatile float* vl = logits;
+        // logits were written by other blocks: read them past the caches
+        __shared__ float s_log[QKK_MAX_EXPERTS + 1];
+        for (uint32_t e = lane; e <= d.E; e += 64) s_log[e] = vl[e];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        select_wave(s_log, d.E, d.k, &sel[slot]);
+        if (lane == 0) {
+            sel[slot].w_shared = 1.f / (1.f + expf(-s_log[d.E]));
+            ws.counter[slot] = 0u; // ready for the next step
+        }
+    }
+}
+
+// ---- launch 2: routed gate/up + SiLU ---------------------------------------------------
+// Wave task = (pick s, RIF consecutive FFN rows); gate and up rows of one FFN row are
+// fetched together.  IQ3_XXS rows of H = 2048*PASSES weights.
+template <int TYPE, int PASSES, int RIF>
+__global__ __launch_bounds__(256) void moe_gateup_kernel(const uint8_t* __restrict__ gate_exps,
+                                                         const uint8_t* __restrict__ up_exps,
+                                                         const float* __restrict__ X, MoeWs ws,
+                                                         const qkk_sel* __restrict__ sel, MoeDims d)
+{
+    __shared__ IqTables tab;
+    fill_iq_tables(tab, g_iq3xxs_grid, threadIdx.x, 256);
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t slot = blockIdx.y;
+    const float* x = X + (size_t)slot * d.H;
+    float* h = ws.h + (size_t)slot * (d.k + 1) * d.F;
+    const uint32_t row_bytes = (uint32_t)qkk_row_bytes_dev<TYPE>(d.H);
+    const uint32_t pass_bytes = row_bytes / PASSES;
+
+    XSlice xs[PASSES];
+#pragma unroll
+    for (int p = 0; p < PASSES; p++) load_xslice<TYPE>(xs[p], x + p * 2048, lane);
+
+    const uint32_t groups = (d.F + RIF - 1) / RIF; // row groups per pick
+    for (uint32_t t = blockIdx.x * 4 + wave; t < d.k * groups; t += gridDim.x * 4) {
+        const uint32_t s = t / groups, r0 = (t % groups) * RIF;
+        const uint32_t e = min(sel[slot].ids[s], d.E - 1);
+        const uint8_t* gbase = gate_exps + ((size_t)e * d.F) * row_bytes;
+        const uint8_t* ubase = up_exps + ((size_t)e * d.F) * row_bytes;
+        LaneW<TYPE> wg[RIF][PASSES], wu[RIF][PASSES];
+#pragma unroll
+        for (int i = 0; i < RIF; i++) {
+            const uint32_t r = min(r0 + i, d.F - 1);
+#pragma unroll
+            for (int p = 0; p < PASSES; p++) {
+                wg[i][p].load(gbase + (size_t)r * row_bytes + (size_t)p * pass_bytes, lane);
+                wu[i][p].load(ubase + (size_t)r * row_bytes + (size_t)p * pass_bytes, lane);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < RIF; i++) {
+            float g = 0.f, u = 0.f;
+#pragma unroll
+            for (int p = 0; p < PASSES; p++) {
+                g += wg[i][p].dot(xs[p], nullptr, &tab, lane);
+                u += wu[i][p].dot(xs[p], nullptr, &tab, lane);
+            }
+            g = wave_sum(g);
+            u = wave_sum(u);
+            if (lane == 0 && r0 + i < d.F) h[(size_t)s * d.F + r0 + i] = (g / (1.f + expf(-g))) * u;
+        }
+    }
+}
+
+// ---- launch 3: routed down + shared down + combine ---------------------------------------
+// Wave task = RIF consecutive outputs o.  F = 32*LPR: LPR lanes cover one down row, so
+// 64/LPR picks are processed side by side; the shared Q8_0 row rides on lane group 0.
+template <int TYPE, int LPR, int ROUNDS, int RIF>
+__global__ __launch_bounds__(256) void moe_down_kernel(const uint8_t* __restrict__ down_exps,
+                                                       const uint8_t* __restrict__ down_shexp,
+                                                       MoeWs ws, const qkk_sel* __restrict__ sel,
+                                                       float* __restrict__ Y, MoeDims d)
+{
+    __shared__ IqTables tab;
+    fill_iq_tables(tab, g_iq3xxs_grid, threadIdx.x, 256);
+    __syncthreads();
+    constexpr int GROUPS = WAVE / LPR;
+    constexpr uint32_t rounds = ROUNDS; // ROUNDS * GROUPS >= n_used; surplus lanes carry weight 0
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lir = lane % LPR, grp = lane / LPR;
+    const uint32_t slot = blockIdx.y;
+    const float* h = ws.h + (size_t)slot * (d.k + 1) * d.F;
+    float* y = Y + (size_t)slot * d.H;
+    const uint32_t row_bytes = (uint32_t)qkk_row_bytes_dev<TYPE>(d.F);
+    const uint32_t q8_row = d.F / 32 * Q8_0_BYTES;
+
+    // h slices and weights of this lane's picks
+    XSlice hs[ROUNDS];
+    float hsum[ROUNDS][4];
+    float wt[ROUNDS];
+    const uint8_t* ebase[ROUNDS];
+#pragma unroll
+    for (int q = 0; q < ROUNDS; q++) {
+        const uint32_t s = q * GROUPS + grp;
+        const bool on = (uint32_t)q < rounds && s < d.k;
+        const uint32_t sc = on ? s : 0;
+        wt[q] = on ? sel[slot].w[sc] : 0.f;
+        ebase[q] = down_exps + (size_t)min(sel[slot].ids[sc], d.E - 1) * d.H * row_bytes;
+        if ((uint32_t)q < rounds) {
+            load_xslice<TYPE>(hs[q], h + (size_t)sc * d.F, lir);
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                float a = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; i++) a += hs[q].v[c * 8 + i];
+                hsum[q][c] = a;
+            }
+        }
+    }
+    XSlice hsh; // shared expert's h, lane group 0 only
+    load_xslice<QKK_Q8_0>(hsh, h + (size_t)d.k * d.F, lir);
+    const float wsh = grp == 0 ? sel[slot].w_shared : 0.f;
+
+    for (uint32_t o0 = (blockIdx.x * 4 + wave) * RIF; o0 < d.H; o0 += gridDim.x * 4 * RIF) {
+        LaneW<TYPE> w[RIF][ROUNDS];
+        LaneW<QKK_Q8_0> wq[RIF];
+#pragma unroll
+        for (int i = 0; i < RIF; i++) {
+            const uint32_t o = min(o0 + i, d.H - 1);
+#pragma unroll
+            for (int q = 0; q < ROUNDS; q++)
+                if ((uint32_t)q < rounds) w[i][q].load(ebase[q] + (size_t)o * row_bytes, lir);
+            wq[i].load(down_shexp + (size_t)o * q8_row, lir);
+        }
+#pragma unroll
+        for (int i = 0; i < RIF; i++) {
+            float acc = wsh * wq[i].dot(hsh, nullptr, nullptr, lir);
+#pragma unroll
+            for (int q = 0; q < ROUNDS; q++)
+                if ((uint32_t)q < rounds) acc += wt[q] * w[i][q].dot(hs[q], hsum[q], &tab, lir);
+            acc = wave_sum(acc);
+            if (lane == 0 && o0 + i < d.H) y[o0 + i] = acc;
+        }
+    }
+}
+
+} // namespace qk
+
+using namespace qk;
+
+static int check_layer(const qkk_moe_layer* L, const char* who)
+{
+    if (!L) return fail(QKK_EINVAL, "%s: null layer", who);
+    if (!L->gate_inp || !L->gate_inp_shexp || !L->gate_exps || !L->up_exps || !L->down_exps ||
+        !L->gate_shexp || !L->up_shexp || !L->down_shexp)
+        return fail(QKK_EINVAL, "%s: null tensor pointer", who);
+    if (L->gu_type != QKK_IQ3_XXS) return fail(QKK_ETYPE, "%s: gate/up experts must be IQ3_XXS", who);
+    if (L->down_type != QKK_IQ4_XS && L->down_type != QKK_Q6_K)
+        return fail(QKK_ETYPE, "%s: down experts must be IQ4_XS or Q6_K", who);
+    if (L->n_embd != 2048 && L->n_embd != 4096)
+        return fail(QKK_ESHAPE, "%s: n_embd %u not supported (2048 or 4096)", who, L->n_embd);
+    if ((L->n_ff != 512 && L->n_ff != 256 && L->n_ff != 1024) || (L->n_ff == 1024 && L->n_used > 16))
+        return fail(QKK_ESHAPE, "%s: n_ff %u not supported (256, 512 or 1024)", who, L->n_ff);
+    if (L->n_expert < 1 || L->n_expert > QKK_MAX_EXPERTS)
+        return fail(QKK_ESHAPE, "%s: n_expert %u outside 1..%u", who, L->n_expert, QKK_MAX_EXPERTS);
+    if (L->n_used < 1 || L->n_used > QKK_MAX_USED || L->n_used > L->n_expert)
+        return fail(QKK_ESHAPE, "%s: n_used %u outside 1..min(16, n_expert)", who, L->n_used);
+    const void* t[] = {L->gate_inp, L->gate_inp_shexp, L->gate_exps, L->up_exps,
+                       L->down_exps, L->gate_shexp, L->up_shexp, L->down_shexp};
+    for (const void* p : t)
+        if (!aligned16(p)) return fail(QKK_EINVAL, "%s: tensors must be 16-byte aligned", who);
+    return QKK_OK;
+}
+
+template <int TYPE, int LPR, int ROUNDS, int RIF>
+static void launch_down2(const qkk_moe_layer* L, const MoeWs& ws, const qkk_sel* sel, float* Y,
+                         const MoeDims& d, uint32_t n_slots, hipStream_t st)
+{
+    const uint32_t waves = (d.H + RIF - 1) / RIF;
+    hipLaunchKernelGGL((moe_down_kernel<TYPE, LPR, ROUNDS, RIF>), dim3((waves + 3) / 4, n_slots), dim3(256), 0, st,
+                       (const uint8_t*)L->down_exps, (const uint8_t*)L->down_shexp, ws, sel, Y, d);
+}
+
+// Picks processed side by side = 64/LPR; ROUNDS covers n_used with the fewest passes and
+// the rows in flight shrink as ROUNDS grows so the lane's registers hold them.
+template <int TYPE, int LPR>
+static void launch_down(const qkk_moe_layer* L, const MoeWs& ws, const qkk_sel* sel, float* Y,
+                        const MoeDims& d, uint32_t n_slots, hipStream_t st)
+{
+    const uint32_t need = (d.k + 64 / LPR - 1) / (64 / LPR);
+    if (need <= 1) launch_down2<TYPE, LPR, 1, 4>(L, ws, sel, Y, d, n_slots, st);
+    else if (need <= 2) launch_down2<TYPE, LPR, 2, 4>(L, ws, sel, Y, d, n_slots, st);
+    else if (need <= 4) launch_down2<TYPE, LPR, 4, 2>(L, ws, sel, Y, d, n_slots, st);
+    else launch_down2<TYPE, LPR, 8, 1>(L, ws, sel, Y, d, n_slots, st);
+}
+
+template <int TYPE>
+static void launch_down(const qkk_moe_layer* L, const MoeWs& ws, const qkk_sel* sel, float* Y,
+                        const MoeDims& d, uint32_t n_slots, hipStream_t st)
+{
+    if (d.F == 512) launch_down<TYPE, 16>(L, ws, sel, Y, d, n_slots, st);
+    else if (d.F == 256) launch_down<TYPE, 8>(L, ws, sel, Y, d, n_slots, st);
+    else launch_down<TYPE, 32>(L, ws, sel, Y, d, n_slots, st);
+}
+
+extern "C" {
+
+size_t qkk_moe_workspace_bytes(const qkk_moe_layer* L, uint32_t n_slots)
+{
+    if (!L || n_slots == 0) return 0;
+    const MoeDims d{L->n_embd, L->n_ff, L->n_expert, L->n_used};
+    return ws_bytes(d, n_slots);
+}
+
+int qkk_moe_decode(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* sel, void* workspace,
+                   size_t workspace_bytes, uint32_t n_slots, void* stream)
+{
+    if (int rc = check_layer(L, "qkk_moe_decode")) return rc;
+    if (!X || !Y || !sel || !workspace) return fail(QKK_EINVAL, "qkk_moe_decode: null pointer");
+    if (n_slots < 1 || n_slots > 65535) return fail(QKK_ESHAPE, "qkk_moe_decode: n_slots %u outside 1..65535", n_slots);
+    if (!aligned16(X) || !aligned16(Y) || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+        return fail(QKK_EINVAL, "qkk_moe_decode: X/Y must be 16-byte and workspace 256-byte aligned");
+    const MoeDims d{L->n_embd, L->n_ff, L->n_expert, L->n_used};
+    if (workspace_bytes < ws_bytes(d, n_slots))
+        return fail(QKK_EWORKSPACE, "qkk_moe_decode: workspace %zu < %zu bytes", workspace_bytes, ws_bytes(d, n_slots));
+    if (int rc = require_device()) return rc;
+    hipStream_t st = as_stream(stream);
+    const MoeWs ws = ws_carve(workspace, d, n_slots);
+
+    const uint32_t t1 = d.E + 1 + d.F;
+    hipLaunchKernelGGL(moe_route_kernel, dim3((t1 + 3) / 4, n_slots), dim3(256), 0, st, L->gate_inp,
+                       L->gate_inp_shexp, (const uint8_t*)L->gate_shexp, (const uint8_t*)L->up_shexp, X, ws,
+                       sel, d);
+    constexpr int GU_RIF = 4;
+    const uint32_t t2 = d.k * ((d.F + GU_RIF - 1) / GU_RIF);
+    if (d.H == 2048)
+        hipLaunchKernelGGL((moe_gateup_kernel<QKK_IQ3_XXS, 1, GU_RIF>), dim3((t2 + 3) / 4, n_slots), dim3(256), 0,
+                           st, (const uint8_t*)L->gate_exps, (const uint8_t*)L->up_exps, X, ws, sel, d);
+    else
+        hipLaunchKernelGGL((moe_gateup_kernel<QKK_IQ3_XXS, 2, 2>), dim3((d.k * ((d.F + 1) / 2) + 3) / 4, n_slots),
+                           dim3(256), 0, st, (const uint8_t*)L->gate_exps, (const uint8_t*)L->up_exps, X, ws, sel, d);
+    if (L->down_type == QKK_IQ4_XS) launch_down<QKK_IQ4_XS>(L, ws, sel, Y, d, n_slots, st);
+    else launch_down<QKK_Q6_K>(L, ws, sel, Y, d, n_slots, st);
+    return check_launch("qkk_moe_decode");
+}
+
+} // extern "C"

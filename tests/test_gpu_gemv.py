@@ -1,0 +1,73 @@
+"""Quantised GEMVs through the C ABI against the oracle (dequantise row, dot in double).
+Bar: max|got-ref| / max|ref| <= 1e-3 (accumulation order differs); the reference's own
+scale-aware metric (<= 1e-2) is checked as well."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+TYPES = {"q8_0": 8, "q6_k": 14, "iq4_xs": 23, "iq3_xxs": 18, "f16": 1, "f32": 0}
+TOL = 1e-3
+
+
+def run_case(qk, orc, dev, name, M, K, batch, seed=42):
+    import torch
+    print(f"[case] gemv {name} M={M} K={K} batch={batch} seed={seed}", flush=True)
+    t = TYPES[name]
+    W = qk.synth.tensor_host(t, M, K, seed)
+    x = np.random.default_rng(seed + 1).standard_normal((batch, K)).astype(np.float32)
+    got = qk.gemv(t, torch.from_numpy(W).to(dev), torch.from_numpy(x).to(dev), M, K).cpu().numpy()
+    want = orc.gemv(t, W, x, M, K)
+    assert got.shape == want.shape
+    assert orc.rel_maxabs_err(got, want) <= TOL
+    assert orc.max_rel_err(got, want) <= 1e-2
+    return got
+
+
+@pytest.mark.parametrize("name", ["q8_0", "q6_k", "iq4_xs", "iq3_xxs"])
+@pytest.mark.parametrize("M,K,batch", [(8192, 2048, 1), (1000, 2048, 3), (515, 4096, 2), (2048, 512, 1),
+                                       (333, 512, 2), (64, 8192, 1), (37, 1024, 1), (50, 256, 1),
+                                       (21, 768, 2), (9, 2304, 1), (1, 2048, 1)])
+def test_gemv_quantised(qk, orc, dev, name, M, K, batch):
+    run_case(qk, orc, dev, name, M, K, batch)
+
+
+@pytest.mark.parametrize("M,K", [(64, 32), (33, 96), (10, 2080)])
+def test_gemv_q8_0_short_rows(qk, orc, dev, M, K):
+    run_case(qk, orc, dev, "q8_0", M, K, 1)
+
+
+@pytest.mark.parametrize("name", ["f16", "f32"])
+@pytest.mark.parametrize("M,K,batch", [(4096, 4096, 1), (257, 2048, 2), (256, 2048, 16), (5, 72, 1)])
+def test_gemv_dense(qk, orc, dev, name, M, K, batch):
+    run_case(qk, orc, dev, name, M, K, batch)
+
+
+def test_gemv_is_deterministic(qk, orc, dev):
+    a = run_case(qk, orc, dev, "iq3_xxs", 4096, 2048, 1, seed=9)
+    b = run_case(qk, orc, dev, "iq3_xxs", 4096, 2048, 1, seed=9)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+def test_gemv_zero_scales_give_zero(qk, dev):
+    import torch
+    W = qk.synth.tensor_host(qk.Q6_K, 64, 2048, 3).reshape(-1, 210).copy()
+    W[:, 208:210] = 0
+    x = torch.randn(2048, device=dev)
+    y = qk.gemv(qk.Q6_K, torch.from_numpy(W.reshape(-1)).to(dev), x, 64, 2048)
+    assert torch.all(y == 0)
+
+
+def test_gemv_argument_errors(qk, dev):
+    import torch
+    W = torch.zeros(34 * 64, dtype=torch.uint8, device=dev)
+    x = torch.zeros(2048, device=dev)
+    with pytest.raises(qk.QkError) as e:
+        qk.gemv(qk.Q6_K, W, x, 1, 100)
+    assert e.value.code == -2
+    with pytest.raises(qk.QkError) as e:
+        qk.gemv(77, W, x, 1, 2048)
+    assert e.value.code == -3
+    with pytest.raises(qk.QkError) as e:
+        qk.gemv(qk.Q8_0, W[2:], x, 1, 32)   # misaligned tensor base
+    assert e.value.code == -1

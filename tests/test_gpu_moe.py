@@ -1,0 +1,145 @@
+"""Fused MoE decode step through the C ABI against the oracle's restatement of the
+reference's CPU MoE.  Selected expert ids must match exactly and in pick order; router
+weights within 1e-4 (the reference's bar); outputs within 1e-3 relative max-abs."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+def sel_fields(sel):
+    raw = sel.cpu().numpy()
+    ids = raw.view(np.uint32).reshape(-1, 40)[:, :16]
+    w = raw.view(np.float32).reshape(-1, 40)[:, 16:32]
+    wsh = raw.view(np.float32).reshape(-1, 40)[:, 32]
+    return ids, w, wsh
+
+
+def pick_inputs(orc, hl, n, seed, min_gap=2e-3):
+    """n activation rows whose top-k margin is comfortably above fp32 dot-product noise."""
+    rng = np.random.default_rng(seed)
+    rows, refs = [], []
+    while len(rows) < n:
+        x = rng.standard_normal(hl.n_embd).astype(np.float32)
+        r = orc.moe_ref(hl, x)
+        picked = sorted(r["sel"].w[:hl.n_used], reverse=True)
+        # margins between consecutive picks decide the ORDER, the gap decides the SET
+        lw = np.log(np.array(picked))
+        if r["sel"].gap > min_gap and np.min(-np.diff(lw)) > min_gap:
+            rows.append(x)
+            refs.append(r)
+    return np.stack(rows), refs
+
+
+@pytest.fixture(scope="module")
+def layer_iq4(qk):
+    return qk.synth.HostLayer(seed=100, down_type=qk.IQ4_XS)
+
+
+@pytest.fixture(scope="module")
+def layer_q6k(qk):
+    return qk.synth.HostLayer(seed=200, down_type=qk.Q6_K)
+
+
+def check(qk, orc, dev, hl, X, refs):
+    import torch
+    layer = hl.to_device(dev)
+    n = X.shape[0]
+    ws = torch.zeros(qk.moe_workspace_bytes(layer, n), dtype=torch.uint8, device=dev)
+    Y, sel = qk.moe_decode(layer, torch.from_numpy(X).to(dev), ws)
+    torch.cuda.synchronize()
+    Y = Y.cpu().numpy()
+    ids, w, wsh = sel_fields(sel)
+    k = hl.n_used
+    for s in range(n):
+        r = refs[s]
+        assert list(ids[s, :k]) == list(r["sel"].ids[:k]), f"slot {s}"
+        assert np.max(np.abs(w[s, :k] - np.array(r["sel"].w[:k]))) <= 1e-4
+        assert abs(wsh[s] - r["sel"].w_shared) <= 1e-4
+        assert orc.rel_maxabs_err(Y[s], r["y"]) <= TOL, f"slot {s}"
+        assert orc.max_rel_err(Y[s], r["y"]) <= 1e-2
+    return layer, ws, Y, sel
+
+
+def test_moe_decode_bs1_iq4_down(qk, orc, dev, layer_iq4):
+    print("[case] moe bs=1 E=256 k=8 IQ4_XS down", flush=True)
+    X, refs = pick_inputs(orc, layer_iq4, 1, seed=1)
+    check(qk, orc, dev, layer_iq4, X, refs)
+
+
+def test_moe_decode_bs16_q6k_down(qk, orc, dev, layer_q6k):
+    print("[case] moe bs=16 E=256 k=8 Q6_K down", flush=True)
+    X, refs = pick_inputs(orc, layer_q6k, 16, seed=2)
+    check(qk, orc, dev, layer_q6k, X, refs)
+
+
+def test_moe_decode_bs3_iq4_down_repeatable(qk, orc, dev, layer_iq4):
+    import torch
+    print("[case] moe bs=3 repeat on one workspace", flush=True)
+    X, refs = pick_inputs(orc, layer_iq4, 3, seed=3)
+    layer, ws, Y, sel = check(qk, orc, dev, layer_iq4, X, refs)
+    # same workspace, second and third call: bit-identical output (the race canary)
+    for _ in range(2):
+        Y2, sel2 = qk.moe_decode(layer, torch.from_numpy(X).to(dev), ws)
+        torch.cuda.synchronize()
+        assert np.array_equal(Y2.cpu().numpy().view(np.uint32), Y.view(np.uint32))
+        assert torch.equal(sel2, sel)
+
+
+def test_moe_identical_slots_share_experts(qk, orc, dev, layer_q6k):
+    print("[case] moe bs=4 identical rows", flush=True)
+    X, refs = pick_inputs(orc, layer_q6k, 1, seed=4)
+    X4 = np.repeat(X, 4, axis=0)
+    _, _, Y, _ = check(qk, orc, dev, layer_q6k, X4, refs * 4)
+    for s in range(1, 4):
+        assert np.array_equal(Y[s].view(np.uint32), Y[0].view(np.uint32))
+
+
+@pytest.mark.parametrize("E,k,F,down", [(8, 2, 256, "iq4"), (32, 8, 512, "q6k"), (64, 10, 512, "iq4"),
+                                         (512, 16, 512, "iq4"), (16, 16, 256, "q6k"), (4, 1, 1024, "iq4")])
+def test_moe_decode_other_shapes(qk, orc, dev, E, k, F, down):
+    print(f"[case] moe E={E} k={k} F={F} down={down}", flush=True)
+    hl = qk.synth.HostLayer(seed=300 + E + k, n_ff=F, n_expert=E, n_used=k,
+                            down_type=qk.IQ4_XS if down == "iq4" else qk.Q6_K)
+    X, refs = pick_inputs(orc, hl, 2, seed=5, min_gap=(2e-3 if k < E else -1.0))
+    check(qk, orc, dev, hl, X, refs)
+
+
+def test_moe_nan_activations_keep_ids_in_range(qk, dev, layer_iq4):
+    import torch
+    print("[case] moe NaN activations", flush=True)
+    layer = layer_iq4.to_device(dev)
+    X = torch.full((2, 2048), float("nan"), device=dev)
+    X[1] = float("inf")
+    ws = torch.zeros(qk.moe_workspace_bytes(layer, 2), dtype=torch.uint8, device=dev)
+    Y, sel = qk.moe_decode(layer, X, ws)
+    torch.cuda.synchronize()
+    ids, _, _ = sel_fields(sel)
+    assert np.all(ids[:, :8] < 256)
+
+
+def test_moe_argument_errors(qk, dev, layer_iq4):
+    import torch
+    layer = layer_iq4.to_device(dev)
+    X = torch.zeros((1, 2048), device=dev)
+    small = torch.zeros(256, dtype=torch.uint8, device=dev)
+    with pytest.raises(qk.QkError) as e:
+        qk.moe_decode(layer, X, small)
+    assert e.value.code == -5
+
+
+def test_group_pairs_matches_oracle(qk, orc, dev):
+    import torch
+    print("[case] group pairs", flush=True)
+    rng = np.random.default_rng(6)
+    for n_tokens, E, k in [(16, 256, 8), (128, 256, 8), (3, 8, 2), (512, 256, 8), (1, 512, 16)]:
+        sel = np.zeros((n_tokens, 40), dtype=np.uint32)
+        for t in range(n_tokens):
+            sel[t, :k] = rng.choice(E, size=k, replace=False)
+        sel[0, 0] = E + 3
+        sb = sel.view(np.uint8).reshape(n_tokens, 160)
+        off, pairs = qk.moe_group_pairs(torch.from_numpy(sb.copy()).to(dev), n_tokens, E, k)
+        woff, wpairs = orc.group_pairs(sb, n_tokens, E, k)
+        assert np.array_equal(off.cpu().numpy().view(np.uint32), woff)
+        assert np.array_equal(pairs.cpu().numpy().view(np.uint32), wpairs)
