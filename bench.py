@@ -1,0 +1,280 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-weight decode hot path on one MI355X.
+
+Headline workload (config.workload = "moe_decode_bs1"): one fused Qwen3-MoE decode layer,
+hidden 2048, 256 experts, top-8, IQ3_XXS gate/up, IQ4_XS down, Q8_0 shared expert, bs=1.
+A "step" is one call of qkk_moe_decode().  Steps run over a ring of distinct synthetic
+layers whose total size exceeds the 256 MB last-level cache (as the 40 layers of a real
+decode do), captured in a HIP graph; inputs are resident in HBM before the timed region.
+`value` is algorithmic bytes per step / step time, in GB/s.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--ring R]
+                  [--extras/--no-extras] [--cpu/--no-cpu]
+
+Prints ONE JSON line.  --gpus above 1 is refused: this build drives one GPU.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+import __graft_entry__ as entry  # noqa: E402
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def gpu_time_ms(fn, reps):
+    """Mean milliseconds of fn() over reps calls, HIP events on the current stream."""
+    import torch
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    a.record()
+    for _ in range(reps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / reps
+
+
+class Graphed:
+    """A list of launches captured once into a HIP graph on a side stream."""
+
+    def __init__(self, launches):
+        import torch
+        self.n = len(launches)
+        self.stream = torch.cuda.Stream()
+        with torch.cuda.stream(self.stream):
+            for f in launches:  # eager warm-up (also first-touch of every buffer)
+                f()
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph, stream=self.stream):
+            for f in launches:
+                f()
+        torch.cuda.synchronize()
+
+    def replay(self):
+        self.graph.replay()
+
+
+def run_ring(launches, steps, warmup):
+    """Times `steps` launches (a multiple of the ring) bracketed by synchronize.  Returns
+    (ms_per_step wall, ms_per_step by events)."""
+    import torch
+    g = Graphed(launches)
+    reps = max(1, steps // g.n)
+    for _ in range(max(1, warmup // g.n)):
+        g.replay()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    a.record()
+    for _ in range(reps):
+        g.replay()
+    b.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    n = reps * g.n
+    return (t1 - t0) * 1e3 / n, a.elapsed_time(b) / n, n
+
+
+# ---- workloads -------------------------------------------------------------------------------
+
+def moe_workload(qk, n_slots, down_type, ring, steps, warmup, seed=1234):
+    import torch
+    dev = "cuda:0"
+    layers = [qk.synth.device_layer(seed + 16 * i, down_type=down_type, device=dev) for i in range(ring)]
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    X = torch.randn((ring, n_slots, 2048), device=dev, generator=g)
+    Y = torch.empty_like(X)
+    sel = torch.zeros((ring, n_slots, 160), dtype=torch.uint8, device=dev)
+    ws = torch.zeros(qk.moe_workspace_bytes(layers[0], n_slots), dtype=torch.uint8, device=dev)
+
+    def step(i, stages=None):
+        return lambda: qk.moe_decode(layers[i], X[i], ws, Y[i], sel[i], stages=stages)
+
+    wall, ev, n = run_ring([step(i) for i in range(ring)], steps, warmup)
+    # distinct experts touched per step (bs=1: n_used)
+    ids = sel.cpu().numpy().view("uint32").reshape(ring, n_slots, 40)[:, :, :8]
+    distinct = [len(set(ids[i].reshape(-1).tolist())) for i in range(ring)]
+    u = sum(distinct) / len(distinct)
+    L = layers[0]
+    act = n_slots * (2048 * 4 * 2 + 160)  # x in, y out, sel out
+    bytes_step = L.active_bytes(u) + act
+    # per-stage kernel time: the same ring, one stage per launch
+    stage_ms = {}
+    for name, mask in (("route", 1), ("gateup", 2), ("down", 4)):
+        _, sev, _ = run_ring([step(i, mask) for i in range(ring)], max(ring * 5, steps // 2), ring)
+        stage_ms[name] = sev
+    H, F = 2048, 512
+    gu_bytes = u * 2 * F * qk.row_bytes(qk.IQ3_XXS, H) + n_slots * (H * 4 + 9 * F * 4)
+    return dict(ms_wall=wall, ms_event=ev, steps=n, bytes_step=bytes_step, distinct_experts=u, stage_ms=stage_ms,
+                gateup_bytes=gu_bytes, ring=ring, ring_bytes=ring * L.active_bytes(L.n_expert))
+
+
+def gemv_workload(qk, type_, M, K, batch, steps, warmup, seed=99):
+    import torch
+    dev = "cuda:0"
+    rb = qk.row_bytes(type_, K)
+    ring = max(2, int(320e6 // (M * rb)) + 1)
+    be = qk.capi.BLOCK[type_][0]
+    if type_ == qk.F16:
+        Ws = [(torch.randn(M * K, device=dev) * 0.05).to(torch.float16) for _ in range(ring)]
+    else:
+        Ws = [qk.synth.blocks_device(type_, M * (K // be), seed + i, dev).reshape(-1) for i in range(ring)]
+    X = torch.randn((ring, batch, K), device=dev)
+    Y = torch.empty((ring, batch, M), device=dev)
+    wall, ev, n = run_ring([(lambda i=i: qk.gemv(type_, Ws[i], X[i], M, K, out=Y[i])) for i in range(ring)],
+                           steps, warmup)
+    return dict(ms_wall=wall, ms_event=ev, steps=n, bytes_step=M * rb + batch * (K + M) * 4, ring=ring)
+
+
+def head_workload(qk, V, K, batch, steps, warmup, seed=77):
+    import torch
+    dev = "cuda:0"
+    ring = 2
+    Ws = [qk.synth.blocks_device(qk.Q6_K, V * (K // 256), seed + i, dev).reshape(-1) for i in range(ring)]
+    X = torch.randn((ring, batch, K), device=dev)
+    ws = torch.zeros(qk.head_workspace_bytes(V, batch), dtype=torch.uint8, device=dev)
+    toks = []
+
+    def step(i):
+        def f():
+            toks.append(qk.head_argmax(Ws[i], X[i], V, K, ws)[0])
+        return f
+
+    # head_argmax allocates its small token tensor: do that outside the capture
+    import ctypes as C
+    tok = torch.zeros((ring, batch), dtype=torch.int32, device=dev)
+    L = qk.lib()
+
+    def raw(i):
+        def f():
+            rc = L.qkk_head_argmax(C.c_void_p(Ws[i].data_ptr()), C.c_void_p(X[i].data_ptr()),
+                                   C.c_void_p(tok[i].data_ptr()), None, V, K, batch, C.c_void_p(ws.data_ptr()),
+                                   ws.numel(), C.c_void_p(torch.cuda.current_stream().cuda_stream))
+            assert rc == 0, L.qkk_last_error()
+        return f
+
+    wall, ev, n = run_ring([raw(i) for i in range(ring)], steps, warmup)
+    return dict(ms_wall=wall, ms_event=ev, steps=n, bytes_step=V * qk.row_bytes(qk.Q6_K, K) + batch * (K * 4 + 4),
+                ring=ring)
+
+
+def cpu_baseline(qk, orc, budget_s=12.0):
+    """The oracle's scalar fused-MoE step (the reference's moeCpuRef restated) on one host
+    core, on the same layer shape, a fresh activation row per step."""
+    import numpy as np
+    hl = qk.synth.HostLayer(seed=4321)
+    rng = np.random.default_rng(5)
+    xs = rng.standard_normal((64, 2048)).astype(np.float32)
+    orc.moe_ref(hl, xs[0])  # touch
+    t0 = time.perf_counter()
+    n = 0
+    while True:
+        orc.moe_ref(hl, xs[(n + 1) % 64])
+        n += 1
+        if time.perf_counter() - t0 > budget_s or n >= 400:
+            break
+    dt = (time.perf_counter() - t0) / n
+    layer_bytes = 256 * 2048 * 4 + 2048 * 4 + 8 * (2 * 512 * 784 + 2048 * 272) + 2 * 512 * 2176 + 2048 * 544
+    return dict(value=layer_bytes / dt / 1e9, unit="GB/s", cores=1, kind="port",
+                sample=f"{n} fused MoE decode steps (bs=1, one synthetic layer, fresh x per step), "
+                       f"{dt * 1e6:.0f} us/step, oracle moe_ref single-threaded",
+                us_per_step=dt * 1e6)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--workload", default="moe_decode_bs1")
+    ap.add_argument("--ring", type=int, default=40)
+    ap.add_argument("--extras", dest="extras", action="store_true", default=True)
+    ap.add_argument("--no-extras", dest="extras", action="store_false")
+    ap.add_argument("--cpu", dest="cpu", action="store_true", default=True)
+    ap.add_argument("--no-cpu", dest="cpu", action="store_false")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build drives ONE GPU (one process, one device); "
+                 "--gpus N with N > 1 is not supported")
+    import torch
+    qk = entry.load_package()
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no HIP device; libqk.so has no CPU path")
+    qk.lib()
+    info = qk.device_info()
+    log(f"[bench] device {info}")
+
+    steps = max(a.ring, a.steps // a.ring * a.ring)
+    res = {}
+    if a.workload == "moe_decode_bs1":
+        m = moe_workload(qk, 1, qk.IQ4_XS, a.ring, steps, a.warmup)
+    elif a.workload == "moe_decode_bs16":
+        m = moe_workload(qk, 16, qk.Q6_K, min(a.ring, 8), steps, a.warmup)
+    else:
+        sys.exit(f"unknown workload {a.workload}")
+    log(f"[bench] {a.workload}: {m['ms_wall'] * 1e3:.2f} us/step wall, {m['ms_event'] * 1e3:.2f} us/step events, "
+        f"stages {m['stage_ms']}")
+    gbps = m["bytes_step"] / (m["ms_wall"] * 1e-3) / 1e9
+    dom = max(m["stage_ms"], key=m["stage_ms"].get)
+    gu_ms = m["stage_ms"]["gateup"]
+    roof = dict(bound="hbm", kernel="moe_gateup_kernel (routed IQ3_XXS gate/up + SiLU)",
+                achieved=m["gateup_bytes"] / (gu_ms * 1e-3) / 1e9, peak=HBM_PEAK_GBPS, unit="GB/s",
+                frac=m["gateup_bytes"] / (gu_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, traffic=None,
+                bytes_per_launch=m["gateup_bytes"], us_per_launch=gu_ms * 1e3, longest_stage=dom)
+    out = dict(metric="fused_moe_decode_step_hbm_gbps", value=gbps, unit="GB/s", n_gpus=1, steps=m["steps"],
+               warmup=a.warmup, ms_per_step=m["ms_wall"], higher_is_better=True, scaling="weak", vs_baseline=None,
+               dtype="f32", data="synthetic",
+               config=dict(workload=a.workload, n_embd=2048, n_ff=512, n_expert=256, n_used=8,
+                           gate_up="IQ3_XXS", down="IQ4_XS" if a.workload.endswith("bs1") else "Q6_K",
+                           shared="Q8_0", slots=1 if a.workload.endswith("bs1") else 16, ring_layers=m["ring"],
+                           ring_bytes=m["ring_bytes"], timing="hipGraph replay of the ring"),
+               us_per_step=m["ms_wall"] * 1e3, us_per_step_events=m["ms_event"] * 1e3,
+               bytes_per_step=m["bytes_step"], frac_of_hbm_peak=gbps / HBM_PEAK_GBPS,
+               distinct_experts_per_step=m["distinct_experts"],
+               stage_us={k: v * 1e3 for k, v in m["stage_ms"].items()}, roofline=roof, device=info)
+
+    if a.extras:
+        ex = {}
+        es, ew = 400, 40
+        for name, t in (("q8_0", qk.Q8_0), ("q6_k", qk.Q6_K), ("iq4_xs", qk.IQ4_XS), ("iq3_xxs", qk.IQ3_XXS),
+                        ("f16", qk.F16)):
+            g = gemv_workload(qk, t, 8192, 2048, 1, es, ew)
+            ex[f"gemv_{name}_8192x2048"] = dict(us=g["ms_event"] * 1e3, gbps=g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9,
+                                                frac=g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9 / HBM_PEAK_GBPS)
+            log(f"[bench] gemv {name}: {ex[f'gemv_{name}_8192x2048']}")
+            torch.cuda.empty_cache()
+        for b in (1, 16):
+            h = head_workload(qk, 151936, 2048, b, 40, 8)
+            ex[f"head_q6k_151936_bs{b}"] = dict(us=h["ms_event"] * 1e3, gbps=h["bytes_step"] / (h["ms_event"] * 1e-3) / 1e9,
+                                                frac=h["bytes_step"] / (h["ms_event"] * 1e-3) / 1e9 / HBM_PEAK_GBPS)
+            log(f"[bench] head bs{b}: {ex[f'head_q6k_151936_bs{b}']}")
+            torch.cuda.empty_cache()
+        if a.workload == "moe_decode_bs1":
+            m16 = moe_workload(qk, 16, qk.Q6_K, 4, 200, 20)
+            ex["moe_decode_bs16_q6k_down"] = dict(us=m16["ms_event"] * 1e3, distinct_experts=m16["distinct_experts"],
+                                                  gbps=m16["bytes_step"] / (m16["ms_event"] * 1e-3) / 1e9,
+                                                  frac=m16["bytes_step"] / (m16["ms_event"] * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                                                  stage_us={k: v * 1e3 for k, v in m16["stage_ms"].items()})
+            log(f"[bench] moe bs16: {ex['moe_decode_bs16_q6k_down']}")
+        out["extras"] = ex
+
+    if a.cpu:
+        orc = entry.load_oracle()
+        out["cpu_baseline"] = cpu_baseline(qk, orc)
+        log(f"[bench] cpu baseline: {out['cpu_baseline']}")
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

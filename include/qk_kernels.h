@@ -116,6 +116,18 @@ size_t qkk_moe_workspace_bytes(const qkk_moe_layer *L_host, uint32_t n_slots);
 int qkk_moe_decode(const qkk_moe_layer *L_host, const float *X, float *Y, qkk_sel *sel,
                    void *workspace, size_t workspace_bytes, uint32_t n_slots, void *stream);
 
+/* The same step cut at its launch boundaries, for per-stage timing (the reference times its
+ * MoE stages separately under QK_STEP_PROF, src/main.cpp:4173-4185, 4591-4632).  `stages` is
+ * a mask of QKK_STAGE_*; a stage reads what the earlier stages of a previous call left in
+ * sel / workspace. */
+#define QKK_STAGE_ROUTE 1u  /* router logits, shared gate/up, select   */
+#define QKK_STAGE_GATEUP 2u /* routed gate/up + SiLU                     */
+#define QKK_STAGE_DOWN 4u   /* routed + shared down, weighted combine    */
+#define QKK_STAGE_ALL 7u
+int qkk_moe_decode_stages(const qkk_moe_layer *L_host, const float *X, float *Y, qkk_sel *sel,
+                          void *workspace, size_t workspace_bytes, uint32_t n_slots, uint32_t stages,
+                          void *stream);
+
 /* Counting sort of (token, pick) pairs by expert (reference shaders/moe_group_pairs.comp:19-51):
  * offsets[n_expert+1], pairs[n_tokens*n_used] = (token<<4)|pick, ascending inside an expert. */
 int qkk_moe_group_pairs(const qkk_sel *sel, uint32_t n_tokens, uint32_t n_expert, uint32_t n_used,

@@ -57,6 +57,7 @@ def lib():
         L.qkk_dequant.argtypes = [C.c_int, vp, vp, u64, vp]
         L.qkk_gemv.argtypes = [C.c_int, vp, vp, vp, u32, u32, u32, vp]
         L.qkk_moe_decode.argtypes = [vp, vp, vp, vp, vp, sz, u32, vp]
+        L.qkk_moe_decode_stages.argtypes = [vp, vp, vp, vp, vp, sz, u32, u32, vp]
         L.qkk_moe_group_pairs.argtypes = [vp, u32, u32, u32, vp, vp, vp]
         L.qkk_head_argmax.argtypes = [vp, vp, vp, vp, u32, u32, u32, vp, sz, vp]
         L.qkk_argmax.argtypes = [vp, vp, u32, u32, vp]
@@ -137,17 +138,23 @@ def moe_workspace_bytes(layer, n_slots):
     return lib().qkk_moe_workspace_bytes(C.byref(layer.c), n_slots)
 
 
-def moe_decode(layer, X, workspace, Y=None, sel=None):
+def moe_decode(layer, X, workspace, Y=None, sel=None, stages=None):
     """Fused MoE step. X [n_slots, n_embd] fp32. Returns (Y, sel) where sel is a uint8 tensor
-    [n_slots, 160] holding QkSel records."""
+    [n_slots, 160] holding QkSel records.  stages: optional mask of the launches to run
+    (1 route, 2 gate/up, 4 down) for per-stage timing."""
     import torch
     n = X.shape[0]
     if Y is None:
         Y = torch.empty_like(X)
     if sel is None:
         sel = torch.zeros((n, 160), dtype=torch.uint8, device=X.device)
-    _check(lib().qkk_moe_decode(C.byref(layer.c), _ptr(X), _ptr(Y), _ptr(sel), _ptr(workspace),
-                                workspace.numel() * workspace.element_size(), n, _stream()))
+    wsb = workspace.numel() * workspace.element_size()
+    if stages is None:
+        _check(lib().qkk_moe_decode(C.byref(layer.c), _ptr(X), _ptr(Y), _ptr(sel), _ptr(workspace), wsb, n,
+                                    _stream()))
+    else:
+        _check(lib().qkk_moe_decode_stages(C.byref(layer.c), _ptr(X), _ptr(Y), _ptr(sel), _ptr(workspace), wsb,
+                                           n, stages, _stream()))
     return Y, sel
 
 

@@ -36,6 +36,19 @@ int require_device()
     return QKK_OK;
 }
 
+uint32_t persistent_blocks()
+{
+    static uint32_t cached = 0;
+    if (cached == 0) {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+        cached = (uint32_t)cus * 4u;
+    }
+    return cached;
+}
+
 int check_launch(const char* what)
 {
     const hipError_t e = hipGetLastError();
@@ -135,7 +148,7 @@ template <int TYPE, int LPR, int PASSES, int RIF>
 __global__ __launch_bounds__(256) void gemv_q_kernel(const uint8_t* __restrict__ W,
                                                      const float* __restrict__ X,
                                                      float* __restrict__ Y, uint32_t M, uint32_t K,
-                                                     uint32_t row_bytes, uint32_t rows_per_wave)
+                                                     uint32_t row_bytes)
 {
     __shared__ IqTables tab;
     if constexpr (TYPE == QKK_IQ3_XXS || TYPE == QKK_IQ4_XS) {
@@ -163,10 +176,9 @@ __global__ __launch_bounds__(256) void gemv_q_kernel(const uint8_t* __restrict__
     }
     const uint32_t pass_bytes = row_bytes / PASSES;
 
-    const uint32_t wave_id = blockIdx.x * 4 + wave;
-    const uint32_t first = wave_id * rows_per_wave;
-    const uint32_t last = min(first + rows_per_wave, M);
-    for (uint32_t r0 = first; r0 < last; r0 += GROUPS * RIF) {
+    // chunks of GROUPS*RIF rows are dealt round-robin to the waves of the (persistent) grid
+    constexpr uint32_t CHUNK = GROUPS * RIF;
+    for (uint32_t r0 = (blockIdx.x * 4 + wave) * CHUNK; r0 < M; r0 += gridDim.x * 4 * CHUNK) {
         LaneW<TYPE> w[RIF][PASSES];
 #pragma unroll
         for (int i = 0; i < RIF; i++) {
@@ -183,7 +195,7 @@ __global__ __launch_bounds__(256) void gemv_q_kernel(const uint8_t* __restrict__
             for (int p = 0; p < PASSES; p++) acc += w[i][p].dot(xs[p], xsum[p], &tab, lir);
             acc = lanes_sum<LPR>(acc);
             const uint32_t r = r0 + i * GROUPS + grp;
-            if (lir == 0 && r < last) y[r] = acc;
+            if (lir == 0 && r < M) y[r] = acc;
         }
     }
 }
@@ -238,17 +250,14 @@ __global__ __launch_bounds__(256) void gemv_q_generic_kernel(const uint8_t* __re
 template <typename T> // T = _Float16 or float
 __global__ __launch_bounds__(256) void gemv_dense_kernel(const T* __restrict__ W,
                                                          const float* __restrict__ X,
-                                                         float* __restrict__ Y, uint32_t M, uint32_t K,
-                                                         uint32_t rows_per_wave)
+                                                         float* __restrict__ Y, uint32_t M, uint32_t K)
 {
     constexpr int PER = 16 / sizeof(T); // elements per 16-byte chunk
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float* x = X + (size_t)blockIdx.y * K;
     float* y = Y + (size_t)blockIdx.y * M;
-    const uint32_t first = (blockIdx.x * 4 + wave) * rows_per_wave;
-    const uint32_t last = min(first + rows_per_wave, M);
     const uint32_t chunks = K / PER;
-    for (uint32_t r = first; r < last; r++) {
+    for (uint32_t r = blockIdx.x * 4 + wave; r < M; r += gridDim.x * 4) {
         const uint4* row = (const uint4*)(W + (size_t)r * K);
         float acc0 = 0.f, acc1 = 0.f;
         for (uint32_t c = lane; c < chunks; c += 64) {
@@ -277,14 +286,11 @@ template <int TYPE, int LPR, int PASSES, int RIF>
 static void launch_q(const void* W, const float* X, float* Y, uint32_t M, uint32_t K, uint32_t batch,
                      uint32_t row_bytes, hipStream_t st)
 {
-    constexpr uint32_t GROUPS = WAVE / LPR;
-    // rows per wave: a multiple of the rows in flight, sized so the grid has >= ~2048 waves
-    uint32_t rpw = GROUPS * RIF;
-    while ((uint64_t)(M + rpw - 1) / rpw > 8192 && rpw < 64 * GROUPS * RIF) rpw *= 2;
-    const uint32_t waves = (M + rpw - 1) / rpw;
-    const dim3 grid((waves + 3) / 4, batch);
+    constexpr uint32_t CHUNK = WAVE / LPR * RIF;
+    const uint32_t waves = (M + CHUNK - 1) / CHUNK;
+    const dim3 grid(std::min((waves + 3) / 4, persistent_blocks()), batch);
     hipLaunchKernelGGL((gemv_q_kernel<TYPE, LPR, PASSES, RIF>), grid, dim3(256), 0, st,
-                       (const uint8_t*)W, X, Y, M, K, row_bytes, rpw);
+                       (const uint8_t*)W, X, Y, M, K, row_bytes);
 }
 
 template <int TYPE>
@@ -399,14 +405,11 @@ int qkk_gemv(int type, const void* W, const float* X, float* Y, uint32_t M, uint
     case QKK_F32: {
         const uint32_t per = type == QKK_F16 ? 8 : 4;
         if (K % per) return fail(QKK_ESHAPE, "qkk_gemv: K=%u must be a multiple of %u for dense rows", K, per);
-        uint32_t rpw = 1;
-        while ((uint64_t)(M + rpw - 1) / rpw > 16384 && rpw < 64) rpw *= 2;
-        const uint32_t waves = (M + rpw - 1) / rpw;
-        const dim3 grid((waves + 3) / 4, batch);
+        const dim3 grid(std::min((M + 3) / 4, persistent_blocks()), batch);
         if (type == QKK_F16)
-            hipLaunchKernelGGL(gemv_dense_kernel<_Float16>, grid, dim3(256), 0, st, (const _Float16*)W, X, Y, M, K, rpw);
+            hipLaunchKernelGGL(gemv_dense_kernel<_Float16>, grid, dim3(256), 0, st, (const _Float16*)W, X, Y, M, K);
         else
-            hipLaunchKernelGGL(gemv_dense_kernel<float>, grid, dim3(256), 0, st, (const float*)W, X, Y, M, K, rpw);
+            hipLaunchKernelGGL(gemv_dense_kernel<float>, grid, dim3(256), 0, st, (const float*)W, X, Y, M, K);
         return check_launch("qkk_gemv");
     }
     default: return fail(QKK_ETYPE, "qkk_gemv: unsupported tensor type %d", type);

@@ -8,6 +8,8 @@
 #include "qk_device.h"
 #include "qk_host.h"
 
+#include <algorithm>
+
 namespace qk {
 
 constexpr float ARG_FLOOR = -3.4e38f;
@@ -52,8 +54,7 @@ __global__ __launch_bounds__(256) void head_q6k_kernel(const uint8_t* __restrict
                                                        const float* __restrict__ X,
                                                        float* __restrict__ logits_out,
                                                        uint32_t* __restrict__ tok, HeadWs ws, uint32_t V,
-                                                       uint32_t K, uint32_t row_bytes,
-                                                       uint32_t rows_per_wave)
+                                                       uint32_t K, uint32_t row_bytes)
 {
     __shared__ float s_v[256];
     __shared__ uint32_t s_i[256];
@@ -76,12 +77,10 @@ __global__ __launch_bounds__(256) void head_q6k_kernel(const uint8_t* __restrict
         }
     }
     const uint32_t pass_bytes = row_bytes / PASSES;
-    const uint32_t first = (blockIdx.x * 4 + wave) * rows_per_wave;
-    const uint32_t last = min(first + rows_per_wave, V);
-
     float bv = ARG_FLOOR;
     uint32_t bi = 0xFFFFFFFFu;
-    for (uint32_t r0 = first; r0 < last; r0 += RIF) {
+    // chunks of RIF rows dealt round-robin to the waves; a wave's rows ascend
+    for (uint32_t r0 = (blockIdx.x * 4 + wave) * RIF; r0 < V; r0 += gridDim.x * 4 * RIF) {
         LaneW<QKK_Q6_K> w[RIF][PASSES];
 #pragma unroll
         for (int i = 0; i < RIF; i++) {
@@ -97,7 +96,7 @@ __global__ __launch_bounds__(256) void head_q6k_kernel(const uint8_t* __restrict
             for (int p = 0; p < PASSES; p++) acc += w[i][p].dot(xs[p], xsum[p], nullptr, lane);
             acc = wave_sum(acc);
             const uint32_t r = r0 + i;
-            if (r < last) {
+            if (r < V) {
                 if (logits_out && lane == 0) logits_out[(size_t)b * V + r] = acc;
                 if (acc > bv) { bv = acc; bi = r; } // rows ascend: strict '>' keeps the lowest id
             }
@@ -153,16 +152,10 @@ __global__ __launch_bounds__(256) void argmax_kernel(const float* __restrict__ l
     if (threadIdx.x == 0) tok[blockIdx.x] = s_i[0] == 0xFFFFFFFFu ? 0u : s_i[0];
 }
 
-static uint32_t head_rows_per_wave(uint32_t V, uint32_t rif)
-{
-    uint32_t rpw = rif;
-    while ((uint64_t)(V + rpw - 1) / rpw > 8192 && rpw < 64 * rif) rpw *= 2;
-    return rpw;
-}
 static uint32_t head_blocks(uint32_t V, uint32_t rif)
 {
-    const uint32_t rpw = head_rows_per_wave(V, rif);
-    return ((V + rpw - 1) / rpw + 3) / 4;
+    const uint32_t waves = (V + rif - 1) / rif;
+    return std::min((waves + 3) / 4, persistent_blocks());
 }
 constexpr uint32_t HEAD_RIF = 4;
 
@@ -194,7 +187,7 @@ int qkk_head_argmax(const void* W, const float* X, uint32_t* tok, float* logits,
     if (int rc = require_device()) return rc;
     hipStream_t st = as_stream(stream);
     const uint32_t rif = K == 2048 ? HEAD_RIF : 2;
-    const uint32_t rpw = head_rows_per_wave(V, rif), blocks = head_blocks(V, rif);
+    const uint32_t blocks = head_blocks(V, rif);
     HeadWs ws;
     ws.counter = (uint32_t*)workspace;
     ws.cand_v = (float*)((uint8_t*)workspace + 256);
@@ -202,10 +195,10 @@ int qkk_head_argmax(const void* W, const float* X, uint32_t* tok, float* logits,
     const uint32_t rb = (uint32_t)qkk_row_bytes(QKK_Q6_K, K);
     if (K == 2048)
         hipLaunchKernelGGL((head_q6k_kernel<1, HEAD_RIF>), dim3(blocks, batch), dim3(256), 0, st, (const uint8_t*)W,
-                           X, logits, tok, ws, V, K, rb, rpw);
+                           X, logits, tok, ws, V, K, rb);
     else
         hipLaunchKernelGGL((head_q6k_kernel<2, 2>), dim3(blocks, batch), dim3(256), 0, st, (const uint8_t*)W, X,
-                           logits, tok, ws, V, K, rb, rpw);
+                           logits, tok, ws, V, K, rb);
     return check_launch("qkk_head_argmax");
 }
 

@@ -14,6 +14,10 @@ int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 // Device probe shared by every launcher: QKK_OK when a HIP device is current.
 int require_device();
 
+// Blocks of 256 threads that fill the device four deep (16 waves per CU): the grid size of
+// the streaming kernels, which loop over their work with a grid stride.
+uint32_t persistent_blocks();
+
 // Converts the last launch error (if any) into a QKK_EDEVICE failure.
 int check_launch(const char* what);
 

@@ -84,7 +84,10 @@ __device__ static void select_wave(const float* __restrict__ logits, uint32_t E,
 }
 
 // ---- launch 1: router + shared gate/up + select ---------------------------------------
-// Wave tasks: [0, E] F32 rows (E = the shared gate row), then F shared gate/up row pairs.
+// One wave per task, no loop: tasks [0, E] are F32 rows (row E = the shared gate row), tasks
+// after that are shared-expert gate/up row pairs.  Every load of a task is issued before its
+// arithmetic, so a task costs one memory round trip.  H = 256*NCH.
+template <int NCH>
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ gate_inp,
                                                         const float* __restrict__ gate_inp_shexp,
                                                         const uint8_t* __restrict__ gate_shexp,
@@ -92,7 +95,9 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
                                                         const float* __restrict__ X, MoeWs ws,
                                                         qkk_sel* __restrict__ sel, MoeDims d)
 {
+    constexpr int P = NCH / 8; // 2048-weight passes per Q8_0 row
     __shared__ uint32_t s_last;
+    __shared__ float s_log[QKK_MAX_EXPERTS + 1];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t slot = blockIdx.y;
     const float* x = X + (size_t)slot * d.H;
@@ -100,49 +105,56 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     float* h = ws.h + (size_t)slot * (d.k + 1) * d.F;
     const uint32_t n_dense = d.E + 1, n_tasks = n_dense + d.F;
     const uint32_t q8_row = d.H / 32 * Q8_0_BYTES;
+    const uint32_t t = blockIdx.x * 4 + wave;
 
-    for (uint32_t t = blockIdx.x * 4 + wave; t < n_tasks; t += gridDim.x * 4) {
-        if (t < n_dense) {
-            const float4* row = (const float4*)(t < d.E ? gate_inp + (size_t)t * d.H : gate_inp_shexp);
-            const float4* xv = (const float4*)x;
-            float a0 = 0.f, a1 = 0.f;
-            for (uint32_t c = lane; c < d.H / 4; c += 64) {
-                const float4 w = row[c], xx = xv[c];
-                a0 += w.x * xx.x + w.y * xx.y;
-                a1 += w.z * xx.z + w.w * xx.w;
-            }
-            const float s = wave_sum(a0 + a1);
-            if (lane == 0) logits[t] = s;
-        } else {
-            const uint32_t r = t - n_dense;
-            float g = 0.f, u = 0.f;
-            for (uint32_t b0 = 0; b0 < d.H / 32; b0 += 64) {
-                if (b0 + lane < d.H / 32) {
-                    XSlice xs;
-                    load_xslice<QKK_Q8_0>(xs, x + b0 * 32, lane);
-                    LaneW<QKK_Q8_0> wg, wu;
-                    wg.load(gate_shexp + (size_t)r * q8_row + (size_t)b0 * Q8_0_BYTES, lane);
-                    wu.load(up_shexp + (size_t)r * q8_row + (size_t)b0 * Q8_0_BYTES, lane);
-                    g += wg.dot(xs, nullptr, nullptr, lane);
-                    u += wu.dot(xs, nullptr, nullptr, lane);
-                }
-            }
-            g = wave_sum(g);
-            u = wave_sum(u);
-            if (lane == 0) h[(size_t)d.k * d.F + r] = (g / (1.f + expf(-g))) * u;
+    if (t < n_dense) {
+        const float4* row = (const float4*)(t < d.E ? gate_inp + (size_t)t * d.H : gate_inp_shexp);
+        const float4* xv = (const float4*)x;
+        float4 w[NCH], xx[NCH];
+#pragma unroll
+        for (int i = 0; i < NCH; i++) w[i] = row[lane + 64 * i];
+#pragma unroll
+        for (int i = 0; i < NCH; i++) xx[i] = xv[lane + 64 * i];
+        float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            a0 += w[i].x * xx[i].x + w[i].y * xx[i].y;
+            a1 += w[i].z * xx[i].z + w[i].w * xx[i].w;
         }
+        const float s = wave_sum(a0 + a1);
+        if (lane == 0) logits[t] = s;
+    } else if (t < n_tasks) {
+        const uint32_t r = t - n_dense;
+        LaneW<QKK_Q8_0> wg[P], wu[P];
+        XSlice xs[P];
+#pragma unroll
+        for (int p = 0; p < P; p++) {
+            wg[p].load(gate_shexp + (size_t)r * q8_row + (size_t)p * 64 * Q8_0_BYTES, lane);
+            wu[p].load(up_shexp + (size_t)r * q8_row + (size_t)p * 64 * Q8_0_BYTES, lane);
+        }
+#pragma unroll
+        for (int p = 0; p < P; p++) load_xslice<QKK_Q8_0>(xs[p], x + p * 2048, lane);
+        float g = 0.f, u = 0.f;
+#pragma unroll
+        for (int p = 0; p < P; p++) {
+            g += wg[p].dot(xs[p], nullptr, nullptr, lane);
+            u += wu[p].dot(xs[p], nullptr, nullptr, lane);
+        }
+        g = wave_sum(g);
+        u = wave_sum(u);
+        if (lane == 0) h[(size_t)d.k * d.F + r] = (g / (1.f + expf(-g))) * u;
     }
 
-    // last block of this slot runs the selector
-    __threadfence();
+    // the block of this slot that finishes last runs the selector
     __syncthreads();
-    if (threadIdx.x == 0) s_last = atomicAdd(&ws.counter[slot], 1u) == gridDim.x - 1 ? 1u : 0u;
+    if (threadIdx.x == 0) {
+        __threadfence(); // publish this block's logits / h before the count
+        s_last = atomicAdd(&ws.counter[slot], 1u) == gridDim.x - 1 ? 1u : 0u;
+    }
     __syncthreads();
     if (s_last && wave == 0) {
-        __threadfence();
+        __threadfence(); // see the other blocks' logits
         const volatile float* vl = logits;
-        // logits were written by other blocks: read them past the caches
-        __shared__ float s_log[QKK_MAX_EXPERTS + 1];
         for (uint32_t e = lane; e <= d.E; e += 64) s_log[e] = vl[e];
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -348,36 +360,66 @@ size_t qkk_moe_workspace_bytes(const qkk_moe_layer* L, uint32_t n_slots)
     return ws_bytes(d, n_slots);
 }
 
-int qkk_moe_decode(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* sel, void* workspace,
-                   size_t workspace_bytes, uint32_t n_slots, void* stream)
+static int moe_decode_impl(const char* who, const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* sel,
+                           void* workspace, size_t workspace_bytes, uint32_t n_slots, uint32_t stages,
+                           void* stream)
 {
-    if (int rc = check_layer(L, "qkk_moe_decode")) return rc;
-    if (!X || !Y || !sel || !workspace) return fail(QKK_EINVAL, "qkk_moe_decode: null pointer");
-    if (n_slots < 1 || n_slots > 65535) return fail(QKK_ESHAPE, "qkk_moe_decode: n_slots %u outside 1..65535", n_slots);
+    if (int rc = check_layer(L, who)) return rc;
+    if (!X || !Y || !sel || !workspace) return fail(QKK_EINVAL, "%s: null pointer", who);
+    if (n_slots < 1 || n_slots > 65535) return fail(QKK_ESHAPE, "%s: n_slots %u outside 1..65535", who, n_slots);
     if (!aligned16(X) || !aligned16(Y) || (reinterpret_cast<uintptr_t>(workspace) & 255u))
-        return fail(QKK_EINVAL, "qkk_moe_decode: X/Y must be 16-byte and workspace 256-byte aligned");
+        return fail(QKK_EINVAL, "%s: X/Y must be 16-byte and workspace 256-byte aligned", who);
     const MoeDims d{L->n_embd, L->n_ff, L->n_expert, L->n_used};
     if (workspace_bytes < ws_bytes(d, n_slots))
-        return fail(QKK_EWORKSPACE, "qkk_moe_decode: workspace %zu < %zu bytes", workspace_bytes, ws_bytes(d, n_slots));
+        return fail(QKK_EWORKSPACE, "%s: workspace %zu < %zu bytes", who, workspace_bytes, ws_bytes(d, n_slots));
     if (int rc = require_device()) return rc;
     hipStream_t st = as_stream(stream);
     const MoeWs ws = ws_carve(workspace, d, n_slots);
 
-    const uint32_t t1 = d.E + 1 + d.F;
-    hipLaunchKernelGGL(moe_route_kernel, dim3((t1 + 3) / 4, n_slots), dim3(256), 0, st, L->gate_inp,
-                       L->gate_inp_shexp, (const uint8_t*)L->gate_shexp, (const uint8_t*)L->up_shexp, X, ws,
-                       sel, d);
-    constexpr int GU_RIF = 4;
-    const uint32_t t2 = d.k * ((d.F + GU_RIF - 1) / GU_RIF);
-    if (d.H == 2048)
-        hipLaunchKernelGGL((moe_gateup_kernel<QKK_IQ3_XXS, 1, GU_RIF>), dim3((t2 + 3) / 4, n_slots), dim3(256), 0,
-                           st, (const uint8_t*)L->gate_exps, (const uint8_t*)L->up_exps, X, ws, sel, d);
-    else
-        hipLaunchKernelGGL((moe_gateup_kernel<QKK_IQ3_XXS, 2, 2>), dim3((d.k * ((d.F + 1) / 2) + 3) / 4, n_slots),
-                           dim3(256), 0, st, (const uint8_t*)L->gate_exps, (const uint8_t*)L->up_exps, X, ws, sel, d);
-    if (L->down_type == QKK_IQ4_XS) launch_down<QKK_IQ4_XS>(L, ws, sel, Y, d, n_slots, st);
-    else launch_down<QKK_Q6_K>(L, ws, sel, Y, d, n_slots, st);
-    return check_launch("qkk_moe_decode");
+    if (stages & QKK_STAGE_ROUTE) {
+        const uint32_t t1 = d.E + 1 + d.F;
+        if (d.H == 2048)
+            hipLaunchKernelGGL(moe_route_kernel<8>, dim3((t1 + 3) / 4, n_slots), dim3(256), 0, st, L->gate_inp,
+                               L->gate_inp_shexp, (const uint8_t*)L->gate_shexp, (const uint8_t*)L->up_shexp,
+                               X, ws, sel, d);
+        else
+            hipLaunchKernelGGL(moe_route_kernel<16>, dim3((t1 + 3) / 4, n_slots), dim3(256), 0, st, L->gate_inp,
+                               L->gate_inp_shexp, (const uint8_t*)L->gate_shexp, (const uint8_t*)L->up_shexp,
+                               X, ws, sel, d);
+    }
+    if (stages & QKK_STAGE_GATEUP) {
+        constexpr int GU_RIF = 4;
+        const uint32_t t2 = d.k * ((d.F + GU_RIF - 1) / GU_RIF);
+        if (d.H == 2048)
+            hipLaunchKernelGGL((moe_gateup_kernel<QKK_IQ3_XXS, 1, GU_RIF>), dim3((t2 + 3) / 4, n_slots),
+                               dim3(256), 0, st, (const uint8_t*)L->gate_exps, (const uint8_t*)L->up_exps, X,
+                               ws, sel, d);
+        else
+            hipLaunchKernelGGL((moe_gateup_kernel<QKK_IQ3_XXS, 2, 2>),
+                               dim3((d.k * ((d.F + 1) / 2) + 3) / 4, n_slots), dim3(256), 0, st,
+                               (const uint8_t*)L->gate_exps, (const uint8_t*)L->up_exps, X, ws, sel, d);
+    }
+    if (stages & QKK_STAGE_DOWN) {
+        if (L->down_type == QKK_IQ4_XS) launch_down<QKK_IQ4_XS>(L, ws, sel, Y, d, n_slots, st);
+        else launch_down<QKK_Q6_K>(L, ws, sel, Y, d, n_slots, st);
+    }
+    return check_launch(who);
+}
+
+int qkk_moe_decode(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* sel, void* workspace,
+                   size_t workspace_bytes, uint32_t n_slots, void* stream)
+{
+    return moe_decode_impl("qkk_moe_decode", L, X, Y, sel, workspace, workspace_bytes, n_slots, QKK_STAGE_ALL,
+                           stream);
+}
+
+int qkk_moe_decode_stages(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* sel, void* workspace,
+                          size_t workspace_bytes, uint32_t n_slots, uint32_t stages, void* stream)
+{
+    if ((stages & ~QKK_STAGE_ALL) || stages == 0)
+        return fail(QKK_EINVAL, "qkk_moe_decode_stages: stage mask 0x%x outside 1..7", stages);
+    return moe_decode_impl("qkk_moe_decode_stages", L, X, Y, sel, workspace, workspace_bytes, n_slots, stages,
+                           stream);
 }
 
 } // extern "C"

@@ -26,7 +26,8 @@ def pick_inputs(orc, hl, n, seed, min_gap=2e-3):
         picked = sorted(r["sel"].w[:hl.n_used], reverse=True)
         # margins between consecutive picks decide the ORDER, the gap decides the SET
         lw = np.log(np.array(picked))
-        if r["sel"].gap > min_gap and np.min(-np.diff(lw)) > min_gap:
+        order_margin = np.min(-np.diff(lw)) if hl.n_used > 1 else np.inf
+        if r["sel"].gap > min_gap and order_margin > min_gap:
             rows.append(x)
             refs.append(r)
     return np.stack(rows), refs
