@@ -175,6 +175,13 @@ template <>
 struct LaneW<8> { // Q8_0
     uint32_t q[8];
     uint16_t d;
+    // Optimisation barrier: keeps the compiler from hoisting this row's decoded weights out
+    // of a loop over activation rows (that would hold 32 floats per row in registers).
+    __device__ __forceinline__ void touch()
+    {
+#pragma unroll
+        for (int i = 0; i < 8; i++) asm volatile("" : "+v"(q[i]));
+    }
     __device__ __forceinline__ void load(const uint8_t* row, int lane_in_row)
     {
         const uint8_t* p = row + (size_t)lane_in_row * Q8_0_BYTES;
@@ -200,6 +207,10 @@ struct LaneW<14> { // Q6_K
     uint2 qa, qb, qh;
     uint32_t sc4; // the four sub-scales of this lane's runs, one per byte
     uint16_t d;
+    __device__ __forceinline__ void touch()
+    {
+        asm volatile("" : "+v"(qa.x), "+v"(qa.y), "+v"(qb.x), "+v"(qb.y), "+v"(qh.x), "+v"(qh.y));
+    }
     __device__ __forceinline__ void load(const uint8_t* row, int lane_in_row)
     {
         const int b = lane_in_row >> 3, n = (lane_in_row >> 2) & 1, l0 = (lane_in_row & 3) * 8;
@@ -243,6 +254,7 @@ template <>
 struct LaneW<23> { // IQ4_XS
     uint4 q;
     uint2 hdr; // d | scales_h<<16, scales_l[4]
+    __device__ __forceinline__ void touch() { asm volatile("" : "+v"(q.x), "+v"(q.y), "+v"(q.z), "+v"(q.w)); }
     __device__ __forceinline__ void load(const uint8_t* row, int lane_in_row)
     {
         const int b = lane_in_row >> 3, ib = lane_in_row & 7;
@@ -276,6 +288,7 @@ struct LaneW<18> { // IQ3_XXS
     uint2 g;      // 8 grid indices
     uint32_t aux; // 4 x 7-bit sign selectors + 4-bit scale
     uint16_t d;
+    __device__ __forceinline__ void touch() { asm volatile("" : "+v"(g.x), "+v"(g.y), "+v"(aux)); }
     __device__ __forceinline__ void load(const uint8_t* row, int lane_in_row)
     {
         const int b = lane_in_row >> 3, ib = lane_in_row & 7;

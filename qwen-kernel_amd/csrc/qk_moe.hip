@@ -6,82 +6,9 @@
 //   2. gate/up: routed IQ3_XXS gate and up rows of the picked experts, SiLU gating -> h.
 //   3. down:    routed down rows (IQ4_XS or Q6_K) weighted by the router, shared down row
 //               (Q8_0) weighted by the sigmoid gate, summed into y.
-#include "qk_device.h"
-#include "qk_host.h"
+#include "qk_moe_common.h"
 
 namespace qk {
-
-struct MoeDims {
-    uint32_t H, F, E, k;
-};
-
-// Workspace layout (floats unless noted), per slot s:
-//   logits  [E + 1]  (entry E = shared gate dot), stride LSTRIDE
-//   h       [(k + 1) * F]
-//   counter u32 (one per slot), after everything else
-__host__ __device__ inline uint32_t lstride(uint32_t E) { return (E + 1 + 63) & ~63u; }
-
-struct MoeWs {
-    float* logits;
-    float* h;
-    uint32_t* counter;
-};
-
-static size_t ws_bytes(const MoeDims& d, uint32_t n_slots)
-{
-    return ((size_t)n_slots * lstride(d.E) + (size_t)n_slots * (d.k + 1) * d.F) * 4 + 256;
-}
-
-static MoeWs ws_carve(void* ws, const MoeDims& d, uint32_t n_slots)
-{
-    MoeWs w;
-    // counters first so they stay 256-byte aligned with the buffer
-    w.counter = (uint32_t*)ws;
-    w.logits = (float*)((uint8_t*)ws + 256);
-    w.h = w.logits + (size_t)n_slots * lstride(d.E);
-    return w;
-}
-
-// ---- selector --------------------------------------------------------------------------
-// One wave; lane L owns logits L, L+64, ...  Picks n_used times the maximum, lower id on
-// ties; non-finite logits count as -3.4e38 (reference shaders/moe_select.comp:28-34, 53-63).
-__device__ static void select_wave(const float* __restrict__ logits, uint32_t E, uint32_t k,
-                                   qkk_sel* __restrict__ out)
-{
-    constexpr float FLOOR = -3.4e38f;
-    const int lane = threadIdx.x & 63;
-    float v[QKK_MAX_EXPERTS / 64];
-#pragma unroll
-    for (int i = 0; i < (int)(QKK_MAX_EXPERTS / 64); i++) {
-        const uint32_t e = lane + 64 * i;
-        float l = e < E ? logits[e] : FLOOR;
-        if (isnan(l) || isinf(l)) l = FLOOR;
-        v[i] = l;
-    }
-    float picked = 0.f, top = 0.f, wsum = 0.f, myw = 0.f;
-    uint32_t myid = 0;
-    for (uint32_t r = 0; r < k; r++) {
-        float bv = v[0];
-        uint32_t bi = lane;
-#pragma unroll
-        for (int i = 1; i < (int)(QKK_MAX_EXPERTS / 64); i++)
-            if (v[i] > bv) { bv = v[i]; bi = lane + 64 * i; }
-        const float m = wave_max(bv);
-        const uint32_t id = wave_min_u32(bv == m ? bi : 0x7FFFFFFFu);
-        // retire the winner
-#pragma unroll
-        for (int i = 0; i < (int)(QKK_MAX_EXPERTS / 64); i++)
-            if ((uint32_t)(lane + 64 * i) == id) v[i] = FLOOR;
-        if (r == 0) top = m;
-        picked = expf(m - top);
-        wsum += picked;
-        if ((uint32_t)lane == r) { myw = picked; myid = min(id, E - 1); }
-    }
-    if ((uint32_t)lane < k) {
-        out->ids[lane] = myid;
-        out->w[lane] = myw / wsum;
-    }
-}
 
 // ---- launch 1: router + shared gate/up + select ---------------------------------------
 // One wave per task, no loop: tasks [0, E] are F32 rows (row E = the shared gate row), tasks
@@ -154,8 +81,14 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     __syncthreads();
     if (s_last && wave == 0) {
         __threadfence(); // see the other blocks' logits
-        const volatile float* vl = logits;
-        for (uint32_t e = lane; e <= d.E; e += 64) s_log[e] = vl[e];
+        // plain loads after the acquire fence, all issued before the first use
+        float lv[QKK_MAX_EXPERTS / 64 + 1];
+#pragma unroll
+        for (int i = 0; i <= (int)(QKK_MAX_EXPERTS / 64); i++)
+            lv[i] = (uint32_t)(lane + 64 * i) <= d.E ? logits[lane + 64 * i] : 0.f;
+#pragma unroll
+        for (int i = 0; i <= (int)(QKK_MAX_EXPERTS / 64); i++)
+            if ((uint32_t)(lane + 64 * i) <= d.E) s_log[lane + 64 * i] = lv[i];
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         select_wave(s_log, d.E, d.k, &sel[slot]);
@@ -294,6 +227,10 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const uint8_t* __restrict
 
 } // namespace qk
 
+namespace qk {
+int moe_grouped_launch(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* sel, void* workspace,
+                       uint32_t N, uint32_t stages, hipStream_t st);
+}
 using namespace qk;
 
 static int check_layer(const qkk_moe_layer* L, const char* who)
@@ -366,7 +303,7 @@ static int moe_decode_impl(const char* who, const qkk_moe_layer* L, const float*
 {
     if (int rc = check_layer(L, who)) return rc;
     if (!X || !Y || !sel || !workspace) return fail(QKK_EINVAL, "%s: null pointer", who);
-    if (n_slots < 1 || n_slots > 65535) return fail(QKK_ESHAPE, "%s: n_slots %u outside 1..65535", who, n_slots);
+    if (n_slots < 1 || n_slots > 4096) return fail(QKK_ESHAPE, "%s: %u rows outside 1..4096", who, n_slots);
     if (!aligned16(X) || !aligned16(Y) || (reinterpret_cast<uintptr_t>(workspace) & 255u))
         return fail(QKK_EINVAL, "%s: X/Y must be 16-byte and workspace 256-byte aligned", who);
     const MoeDims d{L->n_embd, L->n_ff, L->n_expert, L->n_used};
@@ -374,6 +311,7 @@ static int moe_decode_impl(const char* who, const qkk_moe_layer* L, const float*
         return fail(QKK_EWORKSPACE, "%s: workspace %zu < %zu bytes", who, workspace_bytes, ws_bytes(d, n_slots));
     if (int rc = require_device()) return rc;
     hipStream_t st = as_stream(stream);
+    if (n_slots >= 2) return moe_grouped_launch(L, X, Y, sel, workspace, n_slots, stages, st);
     const MoeWs ws = ws_carve(workspace, d, n_slots);
 
     if (stages & QKK_STAGE_ROUTE) {

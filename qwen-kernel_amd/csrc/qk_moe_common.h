@@ -1,0 +1,103 @@
+// qk_moe_common.h -- pieces shared by the single-slot and the grouped MoE paths: dimensions,
+// workspace carving, the wave-level top-k selector.
+#pragma once
+#include "qk_device.h"
+#include "qk_host.h"
+
+namespace qk {
+
+struct MoeDims {
+    uint32_t H, F, E, k;
+};
+
+// Workspace layout (floats unless noted), per slot s:
+//   logits  [E + 1]  (entry E = shared gate dot), stride LSTRIDE
+//   h       [(k + 1) * F]
+//   counter u32 (one per slot), after everything else
+__host__ __device__ inline uint32_t lstride(uint32_t E) { return (E + 1 + 63) & ~63u; }
+
+// One record per expert that at least one token picked: where its pairs are.
+struct ActiveExpert {
+    uint32_t expert, first, count, pad;
+};
+
+struct MoeWs {
+    uint32_t* counter;    // [64] arrival counters; [0] is zero between steps
+    float* logits;        // [n][lstride(E)]
+    float* h;             // [n][k+1][F]
+    // grouped path only (n >= 2)
+    uint32_t* n_active;   // [1] (+3 pad)
+    ActiveExpert* active; // [E]
+    uint32_t* offsets;    // [E+1]
+    uint32_t* pairs;      // [n*k] (token<<4)|pick
+    float* contrib;       // [n][k][H]
+};
+
+static inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+static inline size_t ws_bytes(const MoeDims& d, uint32_t n)
+{
+    size_t b = 256 + align256((size_t)n * lstride(d.E) * 4) + align256((size_t)n * (d.k + 1) * d.F * 4);
+    if (n >= 2)
+        b += 256 + align256((size_t)d.E * sizeof(ActiveExpert)) + align256((size_t)(d.E + 1) * 4) +
+             align256((size_t)n * d.k * 4) + align256((size_t)n * d.k * d.H * 4);
+    return b;
+}
+
+static inline MoeWs ws_carve(void* ws, const MoeDims& d, uint32_t n)
+{
+    MoeWs w;
+    uint8_t* p = (uint8_t*)ws;
+    w.counter = (uint32_t*)p; p += 256;
+    w.logits = (float*)p; p += align256((size_t)n * lstride(d.E) * 4);
+    w.h = (float*)p; p += align256((size_t)n * (d.k + 1) * d.F * 4);
+    w.n_active = (uint32_t*)p; p += 256;
+    w.active = (ActiveExpert*)p; p += align256((size_t)d.E * sizeof(ActiveExpert));
+    w.offsets = (uint32_t*)p; p += align256((size_t)(d.E + 1) * 4);
+    w.pairs = (uint32_t*)p; p += align256((size_t)n * d.k * 4);
+    w.contrib = (float*)p;
+    return w;
+}
+
+// ---- selector --------------------------------------------------------------------------
+// One wave; lane L owns logits L, L+64, ...  Picks n_used times the maximum, lower id on
+// ties; non-finite logits count as -3.4e38 (reference shaders/moe_select.comp:28-34, 53-63).
+__device__ static inline void select_wave(const float* __restrict__ logits, uint32_t E, uint32_t k,
+                                   qkk_sel* __restrict__ out)
+{
+    constexpr float FLOOR = -3.4e38f;
+    const int lane = threadIdx.x & 63;
+    float v[QKK_MAX_EXPERTS / 64];
+#pragma unroll
+    for (int i = 0; i < (int)(QKK_MAX_EXPERTS / 64); i++) {
+        const uint32_t e = lane + 64 * i;
+        float l = e < E ? logits[e] : FLOOR;
+        if (isnan(l) || isinf(l)) l = FLOOR;
+        v[i] = l;
+    }
+    float picked = 0.f, top = 0.f, wsum = 0.f, myw = 0.f;
+    uint32_t myid = 0;
+    for (uint32_t r = 0; r < k; r++) {
+        float bv = v[0];
+        uint32_t bi = lane;
+#pragma unroll
+        for (int i = 1; i < (int)(QKK_MAX_EXPERTS / 64); i++)
+            if (v[i] > bv) { bv = v[i]; bi = lane + 64 * i; }
+        const float m = wave_max(bv);
+        const uint32_t id = wave_min_u32(bv == m ? bi : 0x7FFFFFFFu);
+        // retire the winner
+#pragma unroll
+        for (int i = 0; i < (int)(QKK_MAX_EXPERTS / 64); i++)
+            if ((uint32_t)(lane + 64 * i) == id) v[i] = FLOOR;
+        if (r == 0) top = m;
+        picked = expf(m - top);
+        wsum += picked;
+        if ((uint32_t)lane == r) { myw = picked; myid = min(id, E - 1); }
+    }
+    if ((uint32_t)lane < k) {
+        out->ids[lane] = myid;
+        out->w[lane] = myw / wsum;
+    }
+}
+
+} // namespace qk

@@ -43,6 +43,117 @@ __global__ __launch_bounds__(1024) void group_pairs_kernel(const qkk_sel* __rest
     }
 }
 
+
+// ---- MFMA building blocks -------------------------------------------------------------------
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+// v_mfma_f32_16x16x32_f16: lane l feeds A[l%16][8*(l/16)+e] and B[8*(l/16)+e][l%16], e < 8,
+// and receives D[4*(l/16)+e][l%16], e < 4.
+__device__ __forceinline__ float4v mfma16(half8 a, half8 b, float4v c)
+{
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+
+// Eight int8 weights (two dwords) times the block scale -> eight halves.  Each byte q becomes
+// the half 1024 + (q + 128) by pasting it under the exponent 0x64, then -1152 gives q exactly
+// and one rounded multiply by d gives half(d*q): the same value as converting the fp32
+// product d*q to half (the product is exact in fp32), which is what the reference stages
+// (reference shaders/gemm_q8_0_coopmat2.comp:60-106).
+__device__ __forceinline__ half8 q8_to_half8(uint32_t q0, uint32_t q1, _Float16 d)
+{
+    const uint32_t u0 = q0 ^ 0x80808080u, u1 = q1 ^ 0x80808080u;
+    uint32_t w[4];
+    w[0] = 0x64006400u | (u0 & 0xFFu) | ((u0 & 0xFF00u) << 8);
+    w[1] = 0x64006400u | ((u0 >> 16) & 0xFFu) | ((u0 >> 8) & 0xFF0000u);
+    w[2] = 0x64006400u | (u1 & 0xFFu) | ((u1 & 0xFF00u) << 8);
+    w[3] = 0x64006400u | ((u1 >> 16) & 0xFFu) | ((u1 >> 8) & 0xFF0000u);
+    const half2v off = {(_Float16)-1152.f, (_Float16)-1152.f}, dd = {d, d};
+    half8 r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const half2v v = (__builtin_bit_cast(half2v, w[i]) + off) * dd;
+        r[2 * i] = v[0];
+        r[2 * i + 1] = v[1];
+    }
+    return r;
+}
+
+// ---- dense Q8_0 projection -------------------------------------------------------------------
+// Block = 4 waves; wave w owns rows m0+16w..+15 and all NT token tiles of 16.  Per K step of
+// 32 (one Q8_0 block per row) a lane fetches its 8 weights straight from the block stream --
+// every weight is used by exactly one wave, so weights never pass through LDS -- while the
+// activation tile [16*NT tokens][32] is split into half hi + half lo (x = hi + lo to ~2^-22)
+// and staged in LDS for all four waves.  Loads for step s+1 are in flight during the MFMAs
+// of step s.
+template <int NT>
+__global__ __launch_bounds__(256) void gemm_q8_0_kernel(const uint8_t* __restrict__ W,
+                                                        const float* __restrict__ X, float* __restrict__ Y,
+                                                        uint32_t M, uint32_t K, uint32_t N)
+{
+    constexpr int BN = 16 * NT;
+    constexpr int FPT = BN * 32 / 256; // floats of the activation tile staged per thread (4..16)
+    __shared__ __attribute__((aligned(16))) _Float16 sX[2][2][BN][32];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int i = lane & 15, g = lane >> 4;
+    const uint32_t row_bytes = K / 32 * Q8_0_BYTES;
+    const uint32_t m0 = blockIdx.x * 64 + wave * 16;
+    const uint32_t n0 = blockIdx.y * BN;
+    const uint8_t* wrow = W + (size_t)min(m0 + i, M - 1) * row_bytes + 2 + 8 * g;
+    const int xn = tid * FPT / 32, xk = tid * FPT % 32;
+    const float* xsrc = X + (size_t)min(n0 + xn, N - 1) * K + xk;
+    const uint32_t steps = K / 32;
+
+    float4v acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) acc[t] = float4v{0.f, 0.f, 0.f, 0.f};
+
+    uint2 aq = ldg<uint2>(wrow);
+    uint16_t ad = ldg<uint16_t>(wrow - 2 - 8 * g);
+    float xr[FPT];
+#pragma unroll
+    for (int e = 0; e < FPT; e += 4) *(float4*)&xr[e] = *(const float4*)(xsrc + e);
+
+    for (uint32_t ks = 0; ks < steps; ks++) {
+        const int buf = ks & 1;
+#pragma unroll
+        for (int e = 0; e < FPT; e++) {
+            const _Float16 hi = (_Float16)xr[e];
+            sX[buf][0][xn][xk + e] = hi;
+            sX[buf][1][xn][xk + e] = (_Float16)(xr[e] - (float)hi);
+        }
+        const half8 a = q8_to_half8(aq.x, aq.y, __builtin_bit_cast(_Float16, ad));
+        __syncthreads();
+        if (ks + 1 < steps) {
+            aq = ldg<uint2>(wrow + (size_t)(ks + 1) * Q8_0_BYTES);
+            ad = ldg<uint16_t>(wrow + (size_t)(ks + 1) * Q8_0_BYTES - 2 - 8 * g);
+#pragma unroll
+            for (int e = 0; e < FPT; e += 4) *(float4*)&xr[e] = *(const float4*)(xsrc + (size_t)(ks + 1) * 32 + e);
+        }
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const half8 bh = *(const half8*)&sX[buf][0][16 * t + i][8 * g];
+            const half8 bl = *(const half8*)&sX[buf][1][16 * t + i][8 * g];
+            acc[t] = mfma16(a, bh, acc[t]);
+            acc[t] = mfma16(a, bl, acc[t]);
+        }
+    }
+    // D[4g+e][i]: rows are weight rows (m), columns tokens (n)
+    const uint32_t m = m0 + 4 * g;
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        const uint32_t n = n0 + 16 * t + i;
+        if (n >= N) continue;
+        float* dst = Y + (size_t)n * M + m;
+        if (m + 3 < M && (M & 3u) == 0) *(float4*)dst = float4{acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
+        else
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (m + e < M) dst[e] = acc[t][e];
+    }
+}
+
 } // namespace qk
 
 using namespace qk;
@@ -63,14 +174,31 @@ int qkk_moe_group_pairs(const qkk_sel* sel, uint32_t n_tokens, uint32_t n_expert
     return check_launch("qkk_moe_group_pairs");
 }
 
-int qkk_gemm_q8_0(const void*, const float*, float*, uint32_t, uint32_t, uint32_t, void*)
+int qkk_gemm_q8_0(const void* W, const float* X, float* Y, uint32_t M, uint32_t K, uint32_t N, void* stream)
 {
-    return fail(QKK_ESHAPE, "qkk_gemm_q8_0: not built yet");
+    if (!W || !X || !Y) return fail(QKK_EINVAL, "qkk_gemm_q8_0: null pointer");
+    if (M == 0 || K == 0 || N == 0) return fail(QKK_EINVAL, "qkk_gemm_q8_0: M, K and N must be positive");
+    if (K % 32) return fail(QKK_ESHAPE, "qkk_gemm_q8_0: K=%u is not a multiple of 32", K);
+    if (!aligned16(W) || !aligned16(X) || !aligned16(Y))
+        return fail(QKK_EINVAL, "qkk_gemm_q8_0: W, X and Y must be 16-byte aligned");
+    if ((uint64_t)(N + 127) / 128 > 65535) return fail(QKK_ESHAPE, "qkk_gemm_q8_0: N=%u too large", N);
+    if (int rc = require_device()) return rc;
+    hipStream_t st = as_stream(stream);
+    const uint8_t* w = (const uint8_t*)W;
+    const uint32_t mb = (M + 63) / 64;
+    if (N > 64) hipLaunchKernelGGL(gemm_q8_0_kernel<8>, dim3(mb, (N + 127) / 128), dim3(256), 0, st, w, X, Y, M, K, N);
+    else if (N > 32) hipLaunchKernelGGL(gemm_q8_0_kernel<4>, dim3(mb, 1), dim3(256), 0, st, w, X, Y, M, K, N);
+    else hipLaunchKernelGGL(gemm_q8_0_kernel<2>, dim3(mb, 1), dim3(256), 0, st, w, X, Y, M, K, N);
+    return check_launch("qkk_gemm_q8_0");
 }
-size_t qkk_moe_prefill_workspace_bytes(const qkk_moe_layer*, uint32_t) { return 0; }
-int qkk_moe_prefill(const qkk_moe_layer*, const float*, float*, qkk_sel*, void*, size_t, uint32_t, void*)
+size_t qkk_moe_prefill_workspace_bytes(const qkk_moe_layer* L, uint32_t n_tokens)
 {
-    return fail(QKK_ESHAPE, "qkk_moe_prefill: not built yet");
+    return qkk_moe_workspace_bytes(L, n_tokens);
+}
+int qkk_moe_prefill(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* sel, void* workspace,
+                    size_t workspace_bytes, uint32_t n_tokens, void* stream)
+{
+    return qkk_moe_decode(L, X, Y, sel, workspace, workspace_bytes, n_tokens, stream);
 }
 
 } // extern "C"

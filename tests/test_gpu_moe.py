@@ -20,8 +20,12 @@ def pick_inputs(orc, hl, n, seed, min_gap=2e-3):
     """n activation rows whose top-k margin is comfortably above fp32 dot-product noise."""
     rng = np.random.default_rng(seed)
     rows, refs = [], []
+    gi64 = hl.gate_inp.astype(np.float64)
     while len(rows) < n:
         x = rng.standard_normal(hl.n_embd).astype(np.float32)
+        top = np.sort(gi64 @ x.astype(np.float64))[::-1][:hl.n_used + 1]
+        if hl.n_used < hl.n_expert and np.min(-np.diff(top)) <= min_gap:
+            continue   # cheap pre-check of the margins before the full CPU reference
         r = orc.moe_ref(hl, x)
         picked = sorted(r["sel"].w[:hl.n_used], reverse=True)
         # margins between consecutive picks decide the ORDER, the gap decides the SET

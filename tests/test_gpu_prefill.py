@@ -1,0 +1,86 @@
+"""Batched-prefill entry points against the oracle: the MoE step over a chunk of tokens
+(per token identical to the decode step: exact expert ids in pick order, outputs within 1e-3
+relative max-abs) and the Q8_0 dense projection GEMM (reference bar for fp16-input tiles:
+max error < 2e-3 * rms, src/main.cpp:5659-5662)."""
+import numpy as np
+import pytest
+
+from test_gpu_moe import pick_inputs, sel_fields
+
+pytestmark = pytest.mark.gpu
+
+
+def prefill_case(qk, orc, dev, hl, n_tokens, seed):
+    import torch
+    X, refs = pick_inputs(orc, hl, n_tokens, seed=seed)
+    layer = hl.to_device(dev)
+    ws = torch.zeros(qk.moe_prefill_workspace_bytes(layer, n_tokens), dtype=torch.uint8, device=dev)
+    Y, sel = qk.moe_prefill(layer, torch.from_numpy(X).to(dev), ws)
+    torch.cuda.synchronize()
+    Y = Y.cpu().numpy()
+    ids, w, wsh = sel_fields(sel)
+    k = hl.n_used
+    worst = 0.0
+    for t in range(n_tokens):
+        r = refs[t]
+        assert list(ids[t, :k]) == list(r["sel"].ids[:k]), f"token {t}"
+        assert np.max(np.abs(w[t, :k] - np.array(r["sel"].w[:k]))) <= 1e-4
+        assert abs(wsh[t] - r["sel"].w_shared) <= 1e-4
+        worst = max(worst, orc.rel_maxabs_err(Y[t], r["y"]))
+    assert worst <= 1e-3, worst
+    # second call on the same workspace: identical bits
+    Y2, _ = qk.moe_prefill(layer, torch.from_numpy(X).to(dev), ws)
+    torch.cuda.synchronize()
+    assert np.array_equal(Y2.cpu().numpy().view(np.uint32), Y.view(np.uint32))
+
+
+def test_moe_prefill_128_tokens_iq4_down(qk, orc, dev):
+    print("[case] moe prefill 128 tokens IQ4_XS down", flush=True)
+    hl = qk.synth.HostLayer(seed=100, down_type=qk.IQ4_XS)
+    prefill_case(qk, orc, dev, hl, 128, seed=21)
+
+
+def test_moe_prefill_40_tokens_q6k_down(qk, orc, dev):
+    print("[case] moe prefill 40 tokens Q6_K down", flush=True)
+    hl = qk.synth.HostLayer(seed=200, down_type=qk.Q6_K)
+    prefill_case(qk, orc, dev, hl, 40, seed=22)
+
+
+def test_moe_prefill_small_layer_many_pairs_per_expert(qk, orc, dev):
+    print("[case] moe prefill 96 tokens on 16 experts", flush=True)
+    hl = qk.synth.HostLayer(seed=300, n_expert=16, n_used=4, down_type=qk.IQ4_XS)
+    prefill_case(qk, orc, dev, hl, 96, seed=23)
+
+
+@pytest.mark.parametrize("M,K,N", [(8192, 2048, 128), (100, 96, 5), (64, 32, 33), (130, 2048, 200), (4096, 4096, 48),
+                                   (7, 64, 1), (1024, 512, 16)])
+def test_gemm_q8_0(qk, orc, dev, M, K, N):
+    import torch
+    print(f"[case] gemm q8_0 M={M} K={K} N={N}", flush=True)
+    W = qk.synth.tensor_host(qk.Q8_0, M, K, seed=7, d_scale=1e-2)
+    X = np.random.default_rng(8).uniform(-1, 1, (N, K)).astype(np.float32)
+    Y = qk.gemm_q8_0(torch.from_numpy(W).to(dev), torch.from_numpy(X).to(dev), M, K).cpu().numpy()
+    want = orc.gemm_q8_0(W, X, M, K)
+    assert Y.shape == want.shape == (N, M)
+    assert orc.max_err_over_rms(Y, want) < 2e-3      # the reference's bar for fp16-input tiles
+    assert orc.rel_maxabs_err(Y, want) <= 1e-3
+
+
+def test_gemm_q8_0_matches_gemv_rows(qk, dev):
+    """The GEMM and the GEMV read the same blocks: row by row they agree to fp16-weight rounding."""
+    import torch
+    M, K, N = 512, 2048, 16
+    W = torch.from_numpy(qk.synth.tensor_host(qk.Q8_0, M, K, seed=9)).to(dev)
+    X = torch.randn((N, K), device=dev)
+    a = qk.gemm_q8_0(W, X, M, K)
+    b = qk.gemv(qk.Q8_0, W, X, M, K)
+    assert torch.max(torch.abs(a - b)) <= 1e-3 * torch.max(torch.abs(b))
+
+
+def test_gemm_argument_errors(qk, dev):
+    import torch
+    W = torch.zeros(34 * 4, dtype=torch.uint8, device=dev)
+    X = torch.zeros((2, 40), device=dev)
+    with pytest.raises(qk.QkError) as e:
+        qk.gemm_q8_0(W, X, 1, 40)
+    assert e.value.code == -2
