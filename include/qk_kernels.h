@@ -119,7 +119,7 @@ int qkk_moe_decode(const qkk_moe_layer *L_host, const float *X, float *Y, qkk_se
 /* The same step cut at its launch boundaries, for per-stage timing (the reference times its
  * MoE stages separately under QK_STEP_PROF, src/main.cpp:4173-4185, 4591-4632).  `stages` is
  * a mask of QKK_STAGE_*; a stage reads what the earlier stages of a previous call left in
- * sel / workspace. */
+ * sel / workspace.  With all three stages it is the three-launch form of the step. */
 #define QKK_STAGE_ROUTE 1u  /* router logits, shared gate/up, select   */
 #define QKK_STAGE_GATEUP 2u /* routed gate/up + SiLU                     */
 #define QKK_STAGE_DOWN 4u   /* routed + shared down, weighted combine    */

@@ -1,16 +1,21 @@
 // qk_moe.hip -- fused Qwen3-MoE decode step for gfx950.
 //
-// Three launches per step:
-//   1. route:   router logits (F32 rows) + shared-expert gate dot + shared gate/up (Q8_0);
-//               the block that finishes last picks the top-n_used experts and writes Sel.
-//   2. gate/up: routed IQ3_XXS gate and up rows of the picked experts, SiLU gating -> h.
+// One activation row, three launches per step:
+//   1. route:   router logits (F32 rows) + shared-expert gate dot + shared gate/up (Q8_0).
+//   2. gate/up: every workgroup picks the top-n_used experts from the logits, then the routed
+//               IQ3_XXS gate and up rows of the picks, SiLU gating -> h; writes the router record.
 //   3. down:    routed down rows (IQ4_XS or Q6_K) weighted by the router, shared down row
 //               (Q8_0) weighted by the sigmoid gate, summed into y.
+// On this device a dependent memory access costs 2-3 us when the line is cold (each step
+// touches a different layer's weights) while a kernel boundary costs well under 1 us, so each
+// launch is arranged as two round trips at most and nothing synchronises inside a kernel.
+// (A single-launch form with device-wide barriers was measured at ~5 us per barrier and
+// dropped.)  Several rows go through the expert-major path in qk_moe_grouped.hip.
 #include "qk_moe_common.h"
 
 namespace qk {
 
-// ---- launch 1: router + shared gate/up + select ---------------------------------------
+// ---- launch 1: router logits + shared gate/up ---------------------------------------------
 // One wave per task, no loop: tasks [0, E] are F32 rows (row E = the shared gate row), tasks
 // after that are shared-expert gate/up row pairs.  Every load of a task is issued before its
 // arithmetic, so a task costs one memory round trip.  H = 256*NCH.
@@ -19,17 +24,10 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
                                                         const float* __restrict__ gate_inp_shexp,
                                                         const uint8_t* __restrict__ gate_shexp,
                                                         const uint8_t* __restrict__ up_shexp,
-                                                        const float* __restrict__ X, MoeWs ws,
-                                                        qkk_sel* __restrict__ sel, MoeDims d)
+                                                        const float* __restrict__ x, MoeWs ws, MoeDims d)
 {
     constexpr int P = NCH / 8; // 2048-weight passes per Q8_0 row
-    __shared__ uint32_t s_last;
-    __shared__ float s_log[QKK_MAX_EXPERTS + 1];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t slot = blockIdx.y;
-    const float* x = X + (size_t)slot * d.H;
-    float* logits = ws.logits + (size_t)slot * lstride(d.E);
-    float* h = ws.h + (size_t)slot * (d.k + 1) * d.F;
     const uint32_t n_dense = d.E + 1, n_tasks = n_dense + d.F;
     const uint32_t q8_row = d.H / 32 * Q8_0_BYTES;
     const uint32_t t = blockIdx.x * 4 + wave;
@@ -49,7 +47,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
             a1 += w[i].z * xx[i].z + w[i].w * xx[i].w;
         }
         const float s = wave_sum(a0 + a1);
-        if (lane == 0) logits[t] = s;
+        if (lane == 0) ws.logits[t] = s;
     } else if (t < n_tasks) {
         const uint32_t r = t - n_dense;
         LaneW<QKK_Q8_0> wg[P], wu[P];
@@ -69,63 +67,67 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
         }
         g = wave_sum(g);
         u = wave_sum(u);
-        if (lane == 0) h[(size_t)d.k * d.F + r] = (g / (1.f + expf(-g))) * u;
+        if (lane == 0) ws.h[(size_t)d.k * d.F + r] = (g / (1.f + expf(-g))) * u;
     }
+}
 
-    // the block of this slot that finishes last runs the selector
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        __threadfence(); // publish this block's logits / h before the count
-        s_last = atomicAdd(&ws.counter[slot], 1u) == gridDim.x - 1 ? 1u : 0u;
-    }
-    __syncthreads();
-    if (s_last && wave == 0) {
-        __threadfence(); // see the other blocks' logits
-        // plain loads after the acquire fence, all issued before the first use
-        float lv[QKK_MAX_EXPERTS / 64 + 1];
+// ---- launch 2: select + routed gate/up + SiLU --------------------------------------------
+// Every workgroup picks the top-n_used experts itself from the E logits of launch 1 (one wave,
+// ~1 us) instead of waiting for a selector launch: the logits, the activation slice and the
+// codebook are fetched in one round trip, the picked rows in a second.  Workgroup 0 also
+// writes the router record.  Wave task = (pick s, RIF consecutive FFN rows); gate and up rows
+// of one FFN row are fetched together.  IQ3_XXS rows of H = 2048*PASSES weights.
+template <int TYPE, int PASSES, int RIF>
+__global__ __launch_bounds__(256) void moe_gateup_kernel(const uint8_t* __restrict__ gate_exps,
+                                                         const uint8_t* __restrict__ up_exps,
+                                                         const float* __restrict__ x, MoeWs ws,
+                                                         qkk_sel* __restrict__ sel, MoeDims d)
+{
+    __shared__ IqTables tab;
+    __shared__ float s_log[QKK_MAX_EXPERTS + 8];
+    __shared__ qkk_sel s_sel;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t row_bytes = (uint32_t)qkk_row_bytes_dev<TYPE>(d.H);
+    const uint32_t pass_bytes = row_bytes / PASSES;
+
+    // round trip 1: codebook word, logits (wave 0), activation slice
+    const uint32_t grid_word = g_iq3xxs_grid[threadIdx.x];
+    float lv[QKK_MAX_EXPERTS / 64 + 1];
+    if (wave == 0) {
 #pragma unroll
         for (int i = 0; i <= (int)(QKK_MAX_EXPERTS / 64); i++)
-            lv[i] = (uint32_t)(lane + 64 * i) <= d.E ? logits[lane + 64 * i] : 0.f;
+            lv[i] = (uint32_t)(lane + 64 * i) <= d.E ? ws.logits[lane + 64 * i] : 0.f;
+    }
+    XSlice xs[PASSES];
+#pragma unroll
+    for (int p = 0; p < PASSES; p++) load_xslice<TYPE>(xs[p], x + p * 2048, lane);
+
+    tab.grid[threadIdx.x] = grid_word;
+    if (wave == 0) {
 #pragma unroll
         for (int i = 0; i <= (int)(QKK_MAX_EXPERTS / 64); i++)
             if ((uint32_t)(lane + 64 * i) <= d.E) s_log[lane + 64 * i] = lv[i];
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        select_wave(s_log, d.E, d.k, &sel[slot]);
-        if (lane == 0) {
-            sel[slot].w_shared = 1.f / (1.f + expf(-s_log[d.E]));
-            ws.counter[slot] = 0u; // ready for the next step
+        select_wave(s_log, d.E, d.k, &s_sel);
+        if (lane == 0) s_sel.w_shared = 1.f / (1.f + expf(-s_log[d.E]));
+    }
+    __syncthreads();
+    if (blockIdx.x == 0 && threadIdx.x < 33) {
+        if (threadIdx.x < 16) {
+            if (threadIdx.x < d.k) {
+                sel->ids[threadIdx.x] = s_sel.ids[threadIdx.x];
+                sel->w[threadIdx.x] = s_sel.w[threadIdx.x];
+            }
+        } else if (threadIdx.x == 32) {
+            sel->w_shared = s_sel.w_shared;
         }
     }
-}
-
-// ---- launch 2: routed gate/up + SiLU ---------------------------------------------------
-// Wave task = (pick s, RIF consecutive FFN rows); gate and up rows of one FFN row are
-// fetched together.  IQ3_XXS rows of H = 2048*PASSES weights.
-template <int TYPE, int PASSES, int RIF>
-__global__ __launch_bounds__(256) void moe_gateup_kernel(const uint8_t* __restrict__ gate_exps,
-                                                         const uint8_t* __restrict__ up_exps,
-                                                         const float* __restrict__ X, MoeWs ws,
-                                                         const qkk_sel* __restrict__ sel, MoeDims d)
-{
-    __shared__ IqTables tab;
-    fill_iq_tables(tab, g_iq3xxs_grid, threadIdx.x, 256);
-    __syncthreads();
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t slot = blockIdx.y;
-    const float* x = X + (size_t)slot * d.H;
-    float* h = ws.h + (size_t)slot * (d.k + 1) * d.F;
-    const uint32_t row_bytes = (uint32_t)qkk_row_bytes_dev<TYPE>(d.H);
-    const uint32_t pass_bytes = row_bytes / PASSES;
-
-    XSlice xs[PASSES];
-#pragma unroll
-    for (int p = 0; p < PASSES; p++) load_xslice<TYPE>(xs[p], x + p * 2048, lane);
 
     const uint32_t groups = (d.F + RIF - 1) / RIF; // row groups per pick
     for (uint32_t t = blockIdx.x * 4 + wave; t < d.k * groups; t += gridDim.x * 4) {
         const uint32_t s = t / groups, r0 = (t % groups) * RIF;
-        const uint32_t e = min(sel[slot].ids[s], d.E - 1);
+        const uint32_t e = min(s_sel.ids[s], d.E - 1);
         const uint8_t* gbase = gate_exps + ((size_t)e * d.F) * row_bytes;
         const uint8_t* ubase = up_exps + ((size_t)e * d.F) * row_bytes;
         LaneW<TYPE> wg[RIF][PASSES], wu[RIF][PASSES];
@@ -148,7 +150,7 @@ __global__ __launch_bounds__(256) void moe_gateup_kernel(const uint8_t* __restri
             }
             g = wave_sum(g);
             u = wave_sum(u);
-            if (lane == 0 && r0 + i < d.F) h[(size_t)s * d.F + r0 + i] = (g / (1.f + expf(-g))) * u;
+            if (lane == 0 && r0 + i < d.F) ws.h[(size_t)s * d.F + r0 + i] = (g / (1.f + expf(-g))) * u;
         }
     }
 }
@@ -156,72 +158,74 @@ __global__ __launch_bounds__(256) void moe_gateup_kernel(const uint8_t* __restri
 // ---- launch 3: routed down + shared down + combine ---------------------------------------
 // Wave task = RIF consecutive outputs o.  F = 32*LPR: LPR lanes cover one down row, so
 // 64/LPR picks are processed side by side; the shared Q8_0 row rides on lane group 0.
+// Round trip 1 fetches everything that does not depend on the picks (router record, h slices,
+// shared rows, codebook); round trip 2 the picked experts' rows.
 template <int TYPE, int LPR, int ROUNDS, int RIF>
 __global__ __launch_bounds__(256) void moe_down_kernel(const uint8_t* __restrict__ down_exps,
                                                        const uint8_t* __restrict__ down_shexp,
                                                        MoeWs ws, const qkk_sel* __restrict__ sel,
-                                                       float* __restrict__ Y, MoeDims d)
+                                                       float* __restrict__ y, MoeDims d)
 {
     __shared__ IqTables tab;
-    fill_iq_tables(tab, g_iq3xxs_grid, threadIdx.x, 256);
-    __syncthreads();
     constexpr int GROUPS = WAVE / LPR;
-    constexpr uint32_t rounds = ROUNDS; // ROUNDS * GROUPS >= n_used; surplus lanes carry weight 0
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lir = lane % LPR, grp = lane / LPR;
-    const uint32_t slot = blockIdx.y;
-    const float* h = ws.h + (size_t)slot * (d.k + 1) * d.F;
-    float* y = Y + (size_t)slot * d.H;
+    const float* h = ws.h;
     const uint32_t row_bytes = (uint32_t)qkk_row_bytes_dev<TYPE>(d.F);
     const uint32_t q8_row = d.F / 32 * Q8_0_BYTES;
+    const uint32_t o0 = (blockIdx.x * 4 + wave) * RIF; // the grid covers every output once
 
-    // h slices and weights of this lane's picks
-    XSlice hs[ROUNDS];
-    float hsum[ROUNDS][4];
+    // round trip 1
+    uint32_t eid[ROUNDS];
     float wt[ROUNDS];
-    const uint8_t* ebase[ROUNDS];
 #pragma unroll
     for (int q = 0; q < ROUNDS; q++) {
         const uint32_t s = q * GROUPS + grp;
-        const bool on = (uint32_t)q < rounds && s < d.k;
-        const uint32_t sc = on ? s : 0;
-        wt[q] = on ? sel[slot].w[sc] : 0.f;
-        ebase[q] = down_exps + (size_t)min(sel[slot].ids[sc], d.E - 1) * d.H * row_bytes;
-        if ((uint32_t)q < rounds) {
-            load_xslice<TYPE>(hs[q], h + (size_t)sc * d.F, lir);
-#pragma unroll
-            for (int c = 0; c < 4; c++) {
-                float a = 0.f;
-#pragma unroll
-                for (int i = 0; i < 8; i++) a += hs[q].v[c * 8 + i];
-                hsum[q][c] = a;
-            }
-        }
+        const uint32_t sc = s < d.k ? s : 0;
+        eid[q] = sel->ids[sc];
+        wt[q] = sel->w[sc];
     }
-    XSlice hsh; // shared expert's h, lane group 0 only
+    float wsh = sel->w_shared;
+    XSlice hs[ROUNDS], hsh;
+#pragma unroll
+    for (int q = 0; q < ROUNDS; q++) {
+        const uint32_t s = q * GROUPS + grp;
+        load_xslice<TYPE>(hs[q], h + (size_t)(s < d.k ? s : 0) * d.F, lir);
+    }
     load_xslice<QKK_Q8_0>(hsh, h + (size_t)d.k * d.F, lir);
-    const float wsh = grp == 0 ? sel[slot].w_shared : 0.f;
+    LaneW<QKK_Q8_0> wq[RIF];
+#pragma unroll
+    for (int i = 0; i < RIF; i++) wq[i].load(down_shexp + (size_t)min(o0 + i, d.H - 1) * q8_row, lir);
+    fill_iq_tables(tab, g_iq3xxs_grid, threadIdx.x, 256);
 
-    for (uint32_t o0 = (blockIdx.x * 4 + wave) * RIF; o0 < d.H; o0 += gridDim.x * 4 * RIF) {
-        LaneW<TYPE> w[RIF][ROUNDS];
-        LaneW<QKK_Q8_0> wq[RIF];
+    // round trip 2
+    LaneW<TYPE> w[RIF][ROUNDS];
 #pragma unroll
-        for (int i = 0; i < RIF; i++) {
-            const uint32_t o = min(o0 + i, d.H - 1);
+    for (int q = 0; q < ROUNDS; q++) {
+        const uint8_t* base = down_exps + (size_t)min(eid[q], d.E - 1) * d.H * row_bytes;
+        if (q * GROUPS + grp >= (int)d.k) wt[q] = 0.f;
 #pragma unroll
-            for (int q = 0; q < ROUNDS; q++)
-                if ((uint32_t)q < rounds) w[i][q].load(ebase[q] + (size_t)o * row_bytes, lir);
-            wq[i].load(down_shexp + (size_t)o * q8_row, lir);
+        for (int i = 0; i < RIF; i++) w[i][q].load(base + (size_t)min(o0 + i, d.H - 1) * row_bytes, lir);
+    }
+    if (grp != 0) wsh = 0.f;
+    float hsum[ROUNDS][4];
+#pragma unroll
+    for (int q = 0; q < ROUNDS; q++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            float a = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) a += hs[q].v[c * 8 + i];
+            hsum[q][c] = a;
         }
+    __syncthreads(); // codebook in LDS
 #pragma unroll
-        for (int i = 0; i < RIF; i++) {
-            float acc = wsh * wq[i].dot(hsh, nullptr, nullptr, lir);
+    for (int i = 0; i < RIF; i++) {
+        float acc = wsh * wq[i].dot(hsh, nullptr, nullptr, lir);
 #pragma unroll
-            for (int q = 0; q < ROUNDS; q++)
-                if ((uint32_t)q < rounds) acc += wt[q] * w[i][q].dot(hs[q], hsum[q], &tab, lir);
-            acc = wave_sum(acc);
-            if (lane == 0 && o0 + i < d.H) y[o0 + i] = acc;
-        }
+        for (int q = 0; q < ROUNDS; q++) acc += wt[q] * w[i][q].dot(hs[q], hsum[q], &tab, lir);
+        acc = wave_sum(acc);
+        if (lane == 0 && o0 + i < d.H) y[o0 + i] = acc;
     }
 }
 
@@ -262,7 +266,7 @@ static void launch_down2(const qkk_moe_layer* L, const MoeWs& ws, const qkk_sel*
                          const MoeDims& d, uint32_t n_slots, hipStream_t st)
 {
     const uint32_t waves = (d.H + RIF - 1) / RIF;
-    hipLaunchKernelGGL((moe_down_kernel<TYPE, LPR, ROUNDS, RIF>), dim3((waves + 3) / 4, n_slots), dim3(256), 0, st,
+    hipLaunchKernelGGL((moe_down_kernel<TYPE, LPR, ROUNDS, RIF>), dim3((waves + 3) / 4), dim3(256), 0, st,
                        (const uint8_t*)L->down_exps, (const uint8_t*)L->down_shexp, ws, sel, Y, d);
 }
 
@@ -317,24 +321,24 @@ static int moe_decode_impl(const char* who, const qkk_moe_layer* L, const float*
     if (stages & QKK_STAGE_ROUTE) {
         const uint32_t t1 = d.E + 1 + d.F;
         if (d.H == 2048)
-            hipLaunchKernelGGL(moe_route_kernel<8>, dim3((t1 + 3) / 4, n_slots), dim3(256), 0, st, L->gate_inp,
+            hipLaunchKernelGGL(moe_route_kernel<8>, dim3((t1 + 3) / 4), dim3(256), 0, st, L->gate_inp,
                                L->gate_inp_shexp, (const uint8_t*)L->gate_shexp, (const uint8_t*)L->up_shexp,
-                               X, ws, sel, d);
+                               X, ws, d);
         else
-            hipLaunchKernelGGL(moe_route_kernel<16>, dim3((t1 + 3) / 4, n_slots), dim3(256), 0, st, L->gate_inp,
+            hipLaunchKernelGGL(moe_route_kernel<16>, dim3((t1 + 3) / 4), dim3(256), 0, st, L->gate_inp,
                                L->gate_inp_shexp, (const uint8_t*)L->gate_shexp, (const uint8_t*)L->up_shexp,
-                               X, ws, sel, d);
+                               X, ws, d);
     }
     if (stages & QKK_STAGE_GATEUP) {
         constexpr int GU_RIF = 4;
         const uint32_t t2 = d.k * ((d.F + GU_RIF - 1) / GU_RIF);
         if (d.H == 2048)
-            hipLaunchKernelGGL((moe_gateup_kernel<QKK_IQ3_XXS, 1, GU_RIF>), dim3((t2 + 3) / 4, n_slots),
+            hipLaunchKernelGGL((moe_gateup_kernel<QKK_IQ3_XXS, 1, GU_RIF>), dim3((t2 + 3) / 4),
                                dim3(256), 0, st, (const uint8_t*)L->gate_exps, (const uint8_t*)L->up_exps, X,
                                ws, sel, d);
         else
             hipLaunchKernelGGL((moe_gateup_kernel<QKK_IQ3_XXS, 2, 2>),
-                               dim3((d.k * ((d.F + 1) / 2) + 3) / 4, n_slots), dim3(256), 0, st,
+                               dim3((d.k * ((d.F + 1) / 2) + 3) / 4), dim3(256), 0, st,
                                (const uint8_t*)L->gate_exps, (const uint8_t*)L->up_exps, X, ws, sel, d);
     }
     if (stages & QKK_STAGE_DOWN) {

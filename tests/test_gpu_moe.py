@@ -47,13 +47,14 @@ def layer_q6k(qk):
     return qk.synth.HostLayer(seed=200, down_type=qk.Q6_K)
 
 
-def check(qk, orc, dev, hl, X, refs):
+def check(qk, orc, dev, hl, X, refs, stages=None):
     import torch
     layer = hl.to_device(dev)
     n = X.shape[0]
     ws = torch.zeros(qk.moe_workspace_bytes(layer, n), dtype=torch.uint8, device=dev)
-    Y, sel = qk.moe_decode(layer, torch.from_numpy(X).to(dev), ws)
+    Y, sel = qk.moe_decode(layer, torch.from_numpy(X).to(dev), ws, stages=stages)
     torch.cuda.synchronize()
+    assert np.all(sel.cpu().numpy().view(np.uint32).reshape(-1, 40)[:, 33:] == 0)   # padding untouched
     Y = Y.cpu().numpy()
     ids, w, wsh = sel_fields(sel)
     k = hl.n_used
@@ -71,6 +72,39 @@ def test_moe_decode_bs1_iq4_down(qk, orc, dev, layer_iq4):
     print("[case] moe bs=1 E=256 k=8 IQ4_XS down", flush=True)
     X, refs = pick_inputs(orc, layer_iq4, 1, seed=1)
     check(qk, orc, dev, layer_iq4, X, refs)
+
+
+def test_moe_decode_bs1_three_launch_form(qk, orc, dev, layer_iq4, layer_q6k):
+    print("[case] moe bs=1 via qkk_moe_decode_stages(ALL)", flush=True)
+    for hl in (layer_iq4, layer_q6k):
+        X, refs = pick_inputs(orc, hl, 1, seed=11)
+        check(qk, orc, dev, hl, X, refs, stages=7)
+
+
+def test_moe_decode_bs1_q6k_down(qk, orc, dev, layer_q6k):
+    print("[case] moe bs=1 E=256 k=8 Q6_K down", flush=True)
+    X, refs = pick_inputs(orc, layer_q6k, 1, seed=12)
+    check(qk, orc, dev, layer_q6k, X, refs)
+
+
+def test_moe_decode_bs1_many_steps_one_workspace(qk, orc, dev, layer_iq4):
+    """Back-to-back steps on one workspace: no state may leak from one step into the next."""
+    import torch
+    print("[case] moe bs=1 x 50 steps on one workspace", flush=True)
+    X, refs = pick_inputs(orc, layer_iq4, 5, seed=13)
+    layer = layer_iq4.to_device(dev)
+    ws = torch.zeros(qk.moe_workspace_bytes(layer, 1), dtype=torch.uint8, device=dev)
+    Xd = torch.from_numpy(X).to(dev)
+    for it in range(50):
+        i = it % 5
+        Y, sel = qk.moe_decode(layer, Xd[i:i + 1], ws)
+        if it >= 45:
+            torch.cuda.synchronize()
+            ids, _, _ = sel_fields(sel)
+            assert list(ids[0, :8]) == list(refs[i]["sel"].ids[:8])
+            assert orc.rel_maxabs_err(Y.cpu().numpy()[0], refs[i]["y"]) <= TOL
+    torch.cuda.synchronize()
+    assert int(ws[:256].view(torch.int32).abs().sum()) == 0   # arrival counters are back at zero
 
 
 def test_moe_decode_bs16_q6k_down(qk, orc, dev, layer_q6k):
