@@ -24,9 +24,10 @@ sys.path.insert(0, ROOT)
 import __graft_entry__ as entry  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/);
-# None until a counter run of the same command has been recorded.
-TRAFFIC = {}
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what
+# the same counters read for a plain 256 MiB copy (see profiles/); None where no counter run
+# of that kernel has been recorded.
+TRAFFIC = {"moe_gateup_kernel": 6451726}  # profiles/moe_decode_bs1_hbm_traffic.txt
 
 
 def log(*a):
@@ -204,6 +205,8 @@ def main():
     ap.add_argument("--ring", type=int, default=40)
     ap.add_argument("--extras", dest="extras", action="store_true", default=True)
     ap.add_argument("--no-extras", dest="extras", action="store_false")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one plain 256 MiB device copy (calibrates FETCH_SIZE/WRITE_SIZE counter runs)")
     ap.add_argument("--cpu", dest="cpu", action="store_true", default=True)
     ap.add_argument("--no-cpu", dest="cpu", action="store_false")
     a = ap.parse_args()
@@ -218,8 +221,14 @@ def main():
     info = qk.device_info()
     log(f"[bench] device {info}")
 
+    if a.copy_probe:
+        src = torch.full((64 << 20,), 1.0, device="cuda:0")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)  # 256 MiB read + 256 MiB written: the counters' yardstick
+        torch.cuda.synchronize()
+        del src, dst
     steps = max(a.ring, a.steps // a.ring * a.ring)
-    res = {}
     if a.workload == "moe_decode_bs1":
         m = moe_workload(qk, 1, qk.IQ4_XS, a.ring, steps, a.warmup)
     elif a.workload == "moe_decode_bs16":
@@ -229,19 +238,15 @@ def main():
     log(f"[bench] {a.workload}: {m['ms_wall'] * 1e3:.2f} us/step wall, {m['ms_event'] * 1e3:.2f} us/step events, "
         f"stages {m['stage_ms']}")
     gbps = m["bytes_step"] / (m["ms_wall"] * 1e-3) / 1e9
-    if a.workload == "moe_decode_bs1":
-        # the bs=1 step is ONE launch (moe_fused_kernel): its launch duration is the step time
-        # measured with HIP events on the launch stream over the timed region
-        ach = m["bytes_step"] / (m["ms_event"] * 1e-3) / 1e9
-        roof = dict(bound="hbm", kernel="moe_fused_kernel (whole bs=1 MoE step, one launch)", achieved=ach,
-                    peak=HBM_PEAK_GBPS, unit="GB/s", frac=ach / HBM_PEAK_GBPS, traffic=TRAFFIC.get("moe_fused_kernel"),
-                    bytes_per_launch=m["bytes_step"], us_per_launch=m["ms_event"] * 1e3)
-    else:
-        gu_ms = m["stage_ms"]["gateup"]
-        ach = m["gateup_bytes"] / (gu_ms * 1e-3) / 1e9
-        roof = dict(bound="hbm", kernel="moe_gateup_grouped_kernel (expert-major IQ3_XXS gate/up + SiLU)",
-                    achieved=ach, peak=HBM_PEAK_GBPS, unit="GB/s", frac=ach / HBM_PEAK_GBPS, traffic=None,
-                    bytes_per_launch=m["gateup_bytes"], us_per_launch=gu_ms * 1e3)
+    # dominant kernel = the routed gate/up launch (most bytes of the step); its average launch
+    # duration is measured live with HIP events on the launch stream over a replay of that
+    # stage alone on the same ring (profiles/ holds the rocprofv3 figure for the same kernel)
+    gu_ms = m["stage_ms"]["gateup"]
+    ach = m["gateup_bytes"] / (gu_ms * 1e-3) / 1e9
+    kname = "moe_gateup_kernel" if a.workload == "moe_decode_bs1" else "moe_gateup_grouped_kernel"
+    roof = dict(bound="hbm", kernel=kname + " (select + routed IQ3_XXS gate/up + SiLU)", achieved=ach,
+                peak=HBM_PEAK_GBPS, unit="GB/s", frac=ach / HBM_PEAK_GBPS, traffic=TRAFFIC.get(kname),
+                bytes_per_launch=m["gateup_bytes"], us_per_launch=gu_ms * 1e3)
     out = dict(metric="fused_moe_decode_step_hbm_gbps", value=gbps, unit="GB/s", n_gpus=1, steps=m["steps"],
                warmup=a.warmup, ms_per_step=m["ms_wall"], higher_is_better=True, scaling="weak", vs_baseline=None,
                dtype="f32", data="synthetic",
