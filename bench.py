@@ -173,6 +173,37 @@ def head_workload(qk, V, K, batch, steps, warmup, seed=77):
                 ring=ring)
 
 
+def gemm_workload(qk, M, K, N, steps, warmup, seed=55):
+    import torch
+    dev = "cuda:0"
+    ring = max(2, int(320e6 // (M * K // 32 * 34)) + 1)
+    Ws = [qk.synth.blocks_device(qk.Q8_0, M * K // 32, seed + i, dev).reshape(-1) for i in range(ring)]
+    X = torch.rand((ring, N, K), device=dev) * 2 - 1
+    Y = torch.empty((ring, N, M), device=dev)
+    wall, ev, n = run_ring([(lambda i=i: qk.gemm_q8_0(Ws[i], X[i], M, K, out=Y[i])) for i in range(ring)],
+                           steps, warmup)
+    return dict(ms_event=ev, flops=2.0 * M * K * N, bytes_step=M * K // 32 * 34 + N * K * 4 + N * M * 4)
+
+
+def prefill_moe_workload(qk, n_tokens, steps, warmup, seed=4242):
+    import torch
+    dev = "cuda:0"
+    ring = 2
+    layers = [qk.synth.device_layer(seed + 16 * i, down_type=qk.IQ4_XS, device=dev) for i in range(ring)]
+    X = torch.randn((ring, n_tokens, 2048), device=dev)
+    Y = torch.empty_like(X)
+    sel = torch.zeros((ring, n_tokens, 160), dtype=torch.uint8, device=dev)
+    ws = torch.zeros(qk.moe_prefill_workspace_bytes(layers[0], n_tokens), dtype=torch.uint8, device=dev)
+    wall, ev, n = run_ring([(lambda i=i: qk.moe_prefill(layers[i], X[i], ws, Y[i], sel[i])) for i in range(ring)],
+                           steps, warmup)
+    ids = sel.cpu().numpy().view("uint32").reshape(ring, n_tokens, 40)[:, :, :8]
+    u = sum(len(set(ids[i].reshape(-1).tolist())) for i in range(ring)) / ring
+    L = layers[0]
+    H, F = 2048, 512
+    flops = 2.0 * n_tokens * 8 * (2 * F * H + H * F) + 2.0 * n_tokens * (256 * H + 3 * F * H)
+    return dict(ms_event=ev, distinct_experts=u, bytes_step=L.active_bytes(u) + n_tokens * 2 * H * 4, flops=flops)
+
+
 def cpu_baseline(qk, orc, budget_s=12.0):
     """The oracle's scalar fused-MoE step (the reference's moeCpuRef restated) on one host
     core, on the same layer shape, a fresh activation row per step."""
@@ -282,6 +313,20 @@ def main():
                                                   frac=m16["bytes_step"] / (m16["ms_event"] * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                                                   stage_us={k: v * 1e3 for k, v in m16["stage_ms"].items()})
             log(f"[bench] moe bs16: {ex['moe_decode_bs16_q6k_down']}")
+            torch.cuda.empty_cache()
+            g = gemm_workload(qk, 8192, 2048, 128, 200, 20)
+            ex["prefill_gemm_q8_0_8192x2048x128"] = dict(us=g["ms_event"] * 1e3, tflops=g["flops"] / (g["ms_event"] * 1e-3) / 1e12,
+                                                         frac_mfma_peak=g["flops"] / (g["ms_event"] * 1e-3) / 2.5e15,
+                                                         gbps=g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9)
+            log(f"[bench] prefill gemm: {ex['prefill_gemm_q8_0_8192x2048x128']}")
+            torch.cuda.empty_cache()
+            pm = prefill_moe_workload(qk, 128, 20, 4)
+            ex["prefill_moe_128_tokens"] = dict(us=pm["ms_event"] * 1e3, tok_per_s=128 / (pm["ms_event"] * 1e-3),
+                                                distinct_experts=pm["distinct_experts"],
+                                                gbps=pm["bytes_step"] / (pm["ms_event"] * 1e-3) / 1e9,
+                                                frac=pm["bytes_step"] / (pm["ms_event"] * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                                                tflops=pm["flops"] / (pm["ms_event"] * 1e-3) / 1e12)
+            log(f"[bench] prefill moe: {ex['prefill_moe_128_tokens']}")
         out["extras"] = ex
 
     if a.cpu:

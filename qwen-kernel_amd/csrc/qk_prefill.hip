@@ -81,76 +81,105 @@ __device__ __forceinline__ half8 q8_to_half8(uint32_t q0, uint32_t q1, _Float16 
 }
 
 // ---- dense Q8_0 projection -------------------------------------------------------------------
-// Block = 4 waves; wave w owns rows m0+16w..+15 and all NT token tiles of 16.  Per K step of
-// 32 (one Q8_0 block per row) a lane fetches its 8 weights straight from the block stream --
-// every weight is used by exactly one wave, so weights never pass through LDS -- while the
-// activation tile [16*NT tokens][32] is split into half hi + half lo (x = hi + lo to ~2^-22)
-// and staged in LDS for all four waves.  Loads for step s+1 are in flight during the MFMAs
-// of step s.
-template <int NT>
+// Workgroup tile: 64 weight rows x 16*NT tokens, four waves as 2 (row halves) x 2 (token
+// halves); a wave owns two 16-row tiles and NT/2 token tiles, so every activation fragment it
+// reads from LDS feeds two MFMAs.  Per K step of 32 (one Q8_0 block per row) a lane fetches
+// its 8 weights straight from the block stream in the MFMA A layout -- weights never pass
+// through LDS -- while the activation tile [16*NT tokens][32] is split into half hi + half lo
+// (x = hi + lo to ~2^-22; SPLIT=false keeps hi only, the reference's single-f16 staging) and
+// staged in LDS for all four waves.  Global loads run D steps ahead of the MFMAs in registers.
+template <int NT, bool SPLIT, int D>
 __global__ __launch_bounds__(256) void gemm_q8_0_kernel(const uint8_t* __restrict__ W,
                                                         const float* __restrict__ X, float* __restrict__ Y,
                                                         uint32_t M, uint32_t K, uint32_t N)
 {
-    constexpr int BN = 16 * NT;
+    constexpr int BN = 16 * NT, NTW = NT / 2; // D: steps of look-ahead; K/32 must be a multiple of D
     constexpr int FPT = BN * 32 / 256; // floats of the activation tile staged per thread (4..16)
     __shared__ __attribute__((aligned(16))) _Float16 sX[2][2][BN][32];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int i = lane & 15, g = lane >> 4;
+    const int i = lane & 15, g = lane >> 4, wm = wave & 1, wn = wave >> 1;
     const uint32_t row_bytes = K / 32 * Q8_0_BYTES;
-    const uint32_t m0 = blockIdx.x * 64 + wave * 16;
+    const uint32_t m_base = blockIdx.x * 64 + wm * 32;
     const uint32_t n0 = blockIdx.y * BN;
-    const uint8_t* wrow = W + (size_t)min(m0 + i, M - 1) * row_bytes + 2 + 8 * g;
+    const uint8_t* wrow[2];
+#pragma unroll
+    for (int mt = 0; mt < 2; mt++) wrow[mt] = W + (size_t)min(m_base + 16 * mt + i, M - 1) * row_bytes;
     const int xn = tid * FPT / 32, xk = tid * FPT % 32;
     const float* xsrc = X + (size_t)min(n0 + xn, N - 1) * K + xk;
     const uint32_t steps = K / 32;
 
-    float4v acc[NT];
+    float4v acc[2][NTW];
 #pragma unroll
-    for (int t = 0; t < NT; t++) acc[t] = float4v{0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+        for (int t = 0; t < NTW; t++) acc[mt][t] = float4v{0.f, 0.f, 0.f, 0.f};
 
-    uint2 aq = ldg<uint2>(wrow);
-    uint16_t ad = ldg<uint16_t>(wrow - 2 - 8 * g);
-    float xr[FPT];
+    uint2 aq[D][2];
+    uint32_t ad[D][2]; // dword holding the block scale in its low half (a full-register load)
+    float xr[D][FPT];
+    auto fetch = [&](int slot, uint32_t ks) {
 #pragma unroll
-    for (int e = 0; e < FPT; e += 4) *(float4*)&xr[e] = *(const float4*)(xsrc + e);
-
-    for (uint32_t ks = 0; ks < steps; ks++) {
-        const int buf = ks & 1;
-#pragma unroll
-        for (int e = 0; e < FPT; e++) {
-            const _Float16 hi = (_Float16)xr[e];
-            sX[buf][0][xn][xk + e] = hi;
-            sX[buf][1][xn][xk + e] = (_Float16)(xr[e] - (float)hi);
-        }
-        const half8 a = q8_to_half8(aq.x, aq.y, __builtin_bit_cast(_Float16, ad));
-        __syncthreads();
-        if (ks + 1 < steps) {
-            aq = ldg<uint2>(wrow + (size_t)(ks + 1) * Q8_0_BYTES);
-            ad = ldg<uint16_t>(wrow + (size_t)(ks + 1) * Q8_0_BYTES - 2 - 8 * g);
-#pragma unroll
-            for (int e = 0; e < FPT; e += 4) *(float4*)&xr[e] = *(const float4*)(xsrc + (size_t)(ks + 1) * 32 + e);
+        for (int mt = 0; mt < 2; mt++) {
+            const uint8_t* p = wrow[mt] + (size_t)ks * Q8_0_BYTES;
+            aq[slot][mt] = ldg<uint2>(p + 2 + 8 * g);
+            ad[slot][mt] = ldg<uint32_t>(p);
         }
 #pragma unroll
-        for (int t = 0; t < NT; t++) {
-            const half8 bh = *(const half8*)&sX[buf][0][16 * t + i][8 * g];
-            const half8 bl = *(const half8*)&sX[buf][1][16 * t + i][8 * g];
-            acc[t] = mfma16(a, bh, acc[t]);
-            acc[t] = mfma16(a, bl, acc[t]);
+        for (int e = 0; e < FPT; e += 4) *(float4*)&xr[slot][e] = *(const float4*)(xsrc + (size_t)ks * 32 + e);
+    };
+#pragma unroll
+    for (int j = 0; j < D; j++) fetch(j, j);
+
+    // no branches inside the loop: the look-ahead fetch past the end re-reads the last step,
+    // so the compiler can count outstanding loads exactly instead of draining them every step
+    int buf = 0;
+    for (uint32_t ks0 = 0; ks0 < steps; ks0 += D) {
+#pragma unroll
+        for (int j = 0; j < D; j++) {
+            const uint32_t ks = ks0 + j;
+#pragma unroll
+            for (int e = 0; e < FPT; e++) {
+                const _Float16 hi = (_Float16)xr[j][e];
+                sX[buf][0][xn][xk + e] = hi;
+                if (SPLIT) sX[buf][1][xn][xk + e] = (_Float16)(xr[j][e] - (float)hi);
+            }
+            half8 a[2];
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++)
+                a[mt] = q8_to_half8(aq[j][mt].x, aq[j][mt].y, __builtin_bit_cast(_Float16, (uint16_t)ad[j][mt]));
+            __syncthreads();
+            fetch(j, min(ks + D, steps - 1));
+#pragma unroll
+            for (int t = 0; t < NTW; t++) {
+                const int T = wn * NTW + t;
+                const half8 bh = *(const half8*)&sX[buf][0][16 * T + i][8 * g];
+#pragma unroll
+                for (int mt = 0; mt < 2; mt++) acc[mt][t] = mfma16(a[mt], bh, acc[mt][t]);
+                if (SPLIT) {
+                    const half8 bl = *(const half8*)&sX[buf][1][16 * T + i][8 * g];
+#pragma unroll
+                    for (int mt = 0; mt < 2; mt++) acc[mt][t] = mfma16(a[mt], bl, acc[mt][t]);
+                }
+            }
+            buf ^= 1;
         }
     }
     // D[4g+e][i]: rows are weight rows (m), columns tokens (n)
-    const uint32_t m = m0 + 4 * g;
 #pragma unroll
-    for (int t = 0; t < NT; t++) {
-        const uint32_t n = n0 + 16 * t + i;
-        if (n >= N) continue;
-        float* dst = Y + (size_t)n * M + m;
-        if (m + 3 < M && (M & 3u) == 0) *(float4*)dst = float4{acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
-        else
+    for (int mt = 0; mt < 2; mt++) {
+        const uint32_t m = m_base + 16 * mt + 4 * g;
 #pragma unroll
-            for (int e = 0; e < 4; e++)
-                if (m + e < M) dst[e] = acc[t][e];
+        for (int t = 0; t < NTW; t++) {
+            const uint32_t n = n0 + 16 * (wn * NTW + t) + i;
+            if (n >= N) continue;
+            float* dst = Y + (size_t)n * M + m;
+            if (m + 3 < M && (M & 3u) == 0)
+                *(float4*)dst = float4{acc[mt][t][0], acc[mt][t][1], acc[mt][t][2], acc[mt][t][3]};
+            else
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (m + e < M) dst[e] = acc[mt][t][e];
+        }
     }
 }
 
@@ -186,9 +215,16 @@ int qkk_gemm_q8_0(const void* W, const float* X, float* Y, uint32_t M, uint32_t 
     hipStream_t st = as_stream(stream);
     const uint8_t* w = (const uint8_t*)W;
     const uint32_t mb = (M + 63) / 64;
-    if (N > 64) hipLaunchKernelGGL(gemm_q8_0_kernel<8>, dim3(mb, (N + 127) / 128), dim3(256), 0, st, w, X, Y, M, K, N);
-    else if (N > 32) hipLaunchKernelGGL(gemm_q8_0_kernel<4>, dim3(mb, 1), dim3(256), 0, st, w, X, Y, M, K, N);
-    else hipLaunchKernelGGL(gemm_q8_0_kernel<2>, dim3(mb, 1), dim3(256), 0, st, w, X, Y, M, K, N);
+    const bool deep = (K / 32) % 4 == 0;
+#define QK_GEMM_LAUNCH(NT_, D_, GY_)                                                                         \
+    hipLaunchKernelGGL((gemm_q8_0_kernel<NT_, true, D_>), dim3(mb, GY_), dim3(256), 0, st, w, X, Y, M, K, N)
+    // 64 tokens per workgroup measured fastest at N = 128 (twice the workgroups of the 128-token
+    // tile: the K loop is latency-bound per workgroup, so more of them in flight wins)
+    const int nt = N > 32 ? 4 : 2;
+    const uint32_t gy = (N + 16 * nt - 1) / (16 * nt);
+    if (nt == 4) { if (deep) QK_GEMM_LAUNCH(4, 4, gy); else QK_GEMM_LAUNCH(4, 1, gy); }
+    else { if (deep) QK_GEMM_LAUNCH(2, 4, gy); else QK_GEMM_LAUNCH(2, 1, gy); }
+#undef QK_GEMM_LAUNCH
     return check_launch("qkk_gemm_q8_0");
 }
 size_t qkk_moe_prefill_workspace_bytes(const qkk_moe_layer* L, uint32_t n_tokens)
