@@ -39,6 +39,33 @@ __host__ __device__ constexpr size_t qkk_row_bytes_dev(uint64_t k)
          : TYPE == 1 ? k * 2 : k * 4;
 }
 
+// ---- publishing results to other workgroups of the same launch -----------------------------
+// A release fence at device scope writes back the whole L2 of the XCD (buffer_wbl2); issued
+// once per workgroup by a thousand workgroups it costs tens of microseconds.  Values another
+// workgroup of the same launch will read are therefore stored with device-scope atomic stores
+// (written through to memory), the arrival is counted with a relaxed device-scope atomic after
+// the stores have completed, and only the single workgroup that reads them executes an acquire
+// fence (cache invalidate).
+__device__ __forceinline__ void publish(float* p, float v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void publish(uint32_t* p, uint32_t v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Called by ONE thread after a __syncthreads() that follows the workgroup's publish() calls.
+// Returns true for the workgroup that arrives last; that one may then read what the others
+// published.
+__device__ __forceinline__ bool arrive_last(uint32_t* counter, uint32_t n_workgroups)
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); // the stores above have completed
+    const bool last =
+        __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == n_workgroups - 1;
+    if (last) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    return last;
+}
+
 // ---- wave64 reductions -------------------------------------------------------------
 // Butterfly inside each row of 16 lanes on DPP (quad_perm xor1, xor2, row_half_mirror,
 // row_mirror): after these four steps every lane of a row holds the row's sum.

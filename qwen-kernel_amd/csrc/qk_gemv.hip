@@ -144,7 +144,9 @@ __global__ __launch_bounds__(256) void dequant_f16_kernel(const uint16_t* __rest
 // LPR   lanes per row (8..64): a row of K = 32*LPR*PASSES weights.
 // PASSES how many 32*LPR slices a row has; x slices for all passes stay in registers.
 // RIF   rows in flight per lane group: loads of RIF rows are issued before any arithmetic.
-template <int TYPE, int LPR, int PASSES, int RIF>
+// DEEP  true: two register sets, the next chunk's loads in flight during the arithmetic of the
+//       current one (large matrices); false: one chunk at a time (a wave has one or two chunks).
+template <int TYPE, int LPR, int PASSES, int RIF, bool DEEP>
 __global__ __launch_bounds__(256) void gemv_q_kernel(const uint8_t* __restrict__ W,
                                                      const float* __restrict__ X,
                                                      float* __restrict__ Y, uint32_t M, uint32_t K,
@@ -176,26 +178,46 @@ __global__ __launch_bounds__(256) void gemv_q_kernel(const uint8_t* __restrict__
     }
     const uint32_t pass_bytes = row_bytes / PASSES;
 
-    // chunks of GROUPS*RIF rows are dealt round-robin to the waves of the (persistent) grid
+    // chunks of GROUPS*RIF rows are dealt round-robin to the waves of the (persistent) grid;
+    // the loads of a wave's next chunk are issued before the arithmetic of the current one
+    // (two register sets, loop unrolled by two, no branch around the loads: chunks past the
+    // end re-read the last row and their results are dropped)
     constexpr uint32_t CHUNK = GROUPS * RIF;
-    for (uint32_t r0 = (blockIdx.x * 4 + wave) * CHUNK; r0 < M; r0 += gridDim.x * 4 * CHUNK) {
-        LaneW<TYPE> w[RIF][PASSES];
+    const uint32_t stride = gridDim.x * 4 * CHUNK;
+    LaneW<TYPE> w[DEEP ? 2 : 1][RIF][PASSES];
+    auto fetch = [&](int set, uint32_t r0) {
 #pragma unroll
         for (int i = 0; i < RIF; i++) {
-            // rows past the end re-read the last row; their result is discarded
             const uint32_t r = min(r0 + i * GROUPS + grp, M - 1);
 #pragma unroll
             for (int p = 0; p < PASSES; p++)
-                w[i][p].load(W + (size_t)r * row_bytes + (size_t)p * pass_bytes, lir);
+                w[set][i][p].load(W + (size_t)r * row_bytes + (size_t)p * pass_bytes, lir);
         }
+    };
+    auto reduce = [&](int set, uint32_t r0) {
 #pragma unroll
         for (int i = 0; i < RIF; i++) {
             float acc = 0.f;
 #pragma unroll
-            for (int p = 0; p < PASSES; p++) acc += w[i][p].dot(xs[p], xsum[p], &tab, lir);
+            for (int p = 0; p < PASSES; p++) acc += w[set][i][p].dot(xs[p], xsum[p], &tab, lir);
             acc = lanes_sum<LPR>(acc);
             const uint32_t r = r0 + i * GROUPS + grp;
             if (lir == 0 && r < M) y[r] = acc;
+        }
+    };
+    uint32_t r0 = (blockIdx.x * 4 + wave) * CHUNK;
+    if constexpr (DEEP) {
+        fetch(0, r0);
+        for (; r0 < M; r0 += 2 * stride) {
+            fetch(1, r0 + stride);
+            reduce(0, r0);
+            fetch(0, r0 + 2 * stride);
+            reduce(1, r0 + stride);
+        }
+    } else {
+        for (; r0 < M; r0 += stride) {
+            fetch(0, r0);
+            reduce(0, r0);
         }
     }
 }
@@ -289,8 +311,12 @@ static void launch_q(const void* W, const float* X, float* Y, uint32_t M, uint32
     constexpr uint32_t CHUNK = WAVE / LPR * RIF;
     const uint32_t waves = (M + CHUNK - 1) / CHUNK;
     const dim3 grid(std::min((waves + 3) / 4, persistent_blocks()), batch);
-    hipLaunchKernelGGL((gemv_q_kernel<TYPE, LPR, PASSES, RIF>), grid, dim3(256), 0, st,
-                       (const uint8_t*)W, X, Y, M, K, row_bytes);
+    if (waves > 4 * grid.x * 4) // at least four chunks per wave: worth the second register set
+        hipLaunchKernelGGL((gemv_q_kernel<TYPE, LPR, PASSES, RIF, true>), grid, dim3(256), 0, st,
+                           (const uint8_t*)W, X, Y, M, K, row_bytes);
+    else
+        hipLaunchKernelGGL((gemv_q_kernel<TYPE, LPR, PASSES, RIF, false>), grid, dim3(256), 0, st,
+                           (const uint8_t*)W, X, Y, M, K, row_bytes);
 }
 
 template <int TYPE>

@@ -7,6 +7,7 @@
 // (reference shaders/argmax1.comp:25-33, argmax2.comp:20-28).
 #include "qk_device.h"
 #include "qk_host.h"
+#include "qk_mfma.h"
 
 #include <algorithm>
 
@@ -79,21 +80,25 @@ __global__ __launch_bounds__(256) void head_q6k_kernel(const uint8_t* __restrict
     const uint32_t pass_bytes = row_bytes / PASSES;
     float bv = ARG_FLOOR;
     uint32_t bi = 0xFFFFFFFFu;
-    // chunks of RIF rows dealt round-robin to the waves; a wave's rows ascend
-    for (uint32_t r0 = (blockIdx.x * 4 + wave) * RIF; r0 < V; r0 += gridDim.x * 4 * RIF) {
-        LaneW<QKK_Q6_K> w[RIF][PASSES];
+    // chunks of RIF rows dealt round-robin to the waves; a wave's rows ascend.  The next
+    // chunk's loads are issued before the arithmetic of the current one.
+    const uint32_t stride = gridDim.x * 4 * RIF;
+    LaneW<QKK_Q6_K> w[2][RIF][PASSES];
+    auto fetch = [&](int set, uint32_t r0) {
 #pragma unroll
         for (int i = 0; i < RIF; i++) {
             const uint32_t r = min(r0 + i, V - 1);
 #pragma unroll
             for (int p = 0; p < PASSES; p++)
-                w[i][p].load(W + (size_t)r * row_bytes + (size_t)p * pass_bytes, lane);
+                w[set][i][p].load(W + (size_t)r * row_bytes + (size_t)p * pass_bytes, lane);
         }
+    };
+    auto reduce = [&](int set, uint32_t r0) {
 #pragma unroll
         for (int i = 0; i < RIF; i++) {
             float acc = 0.f;
 #pragma unroll
-            for (int p = 0; p < PASSES; p++) acc += w[i][p].dot(xs[p], xsum[p], nullptr, lane);
+            for (int p = 0; p < PASSES; p++) acc += w[set][i][p].dot(xs[p], xsum[p], nullptr, lane);
             acc = wave_sum(acc);
             const uint32_t r = r0 + i;
             if (r < V) {
@@ -101,6 +106,14 @@ __global__ __launch_bounds__(256) void head_q6k_kernel(const uint8_t* __restrict
                 if (acc > bv) { bv = acc; bi = r; } // rows ascend: strict '>' keeps the lowest id
             }
         }
+    };
+    uint32_t r0 = (blockIdx.x * 4 + wave) * RIF;
+    fetch(0, r0);
+    for (; r0 < V; r0 += 2 * stride) {
+        fetch(1, r0 + stride);
+        reduce(0, r0);
+        fetch(0, r0 + 2 * stride);
+        reduce(1, r0 + stride);
     }
 
     // fold the four waves of the block
@@ -109,14 +122,12 @@ __global__ __launch_bounds__(256) void head_q6k_kernel(const uint8_t* __restrict
     if (threadIdx.x == 0) {
         for (int wv = 1; wv < 4; wv++)
             if (better(s_v[wv], s_i[wv], bv, bi)) { bv = s_v[wv]; bi = s_i[wv]; }
-        ws.cand_v[(size_t)b * gridDim.x + blockIdx.x] = bv;
-        ws.cand_i[(size_t)b * gridDim.x + blockIdx.x] = bi;
-        __threadfence();
-        s_last = atomicAdd(&ws.counter[b], 1u) == gridDim.x - 1 ? 1u : 0u;
+        publish(&ws.cand_v[(size_t)b * gridDim.x + blockIdx.x], bv);
+        publish(&ws.cand_i[(size_t)b * gridDim.x + blockIdx.x], bi);
+        s_last = arrive_last(&ws.counter[b], gridDim.x) ? 1u : 0u;
     }
     __syncthreads();
     if (s_last) {
-        __threadfence();
         const uint32_t t = fold_candidates(ws.cand_v + (size_t)b * gridDim.x, ws.cand_i + (size_t)b * gridDim.x,
                                            gridDim.x, s_v, s_i);
         if (threadIdx.x == 0) {
@@ -152,6 +163,171 @@ __global__ __launch_bounds__(256) void argmax_kernel(const float* __restrict__ l
     if (threadIdx.x == 0) tok[blockIdx.x] = s_i[0] == 0xFFFFFFFFu ? 0u : s_i[0];
 }
 
+// ---- batched head: 2..16 rows of X against the Q6_K matrix on MFMA --------------------------
+// The weights cross HBM once for the whole batch.  Workgroup = 16 waves sharing the batch's
+// activations in LDS (hi/lo half planes in fragment order, 128 KiB for K = 2048); each wave
+// streams 16-row tiles of W.  One Q6_K scale group (16 weights) is one 16x16x16 MFMA with the
+// 6-bit integers as the weight operand; d*scale is applied to the MFMA result in fp32.
+// Lane (row = l%16, g = l/16) fetches, per 256-weight block, the twelve dwords holding its
+// 64 weights (4 per scale group), the 16 scales and d.
+__device__ __forceinline__ void dpp_better(float& v, uint32_t& i)
+{
+#define QK_STEP(CTRL)                                                                             \
+    {                                                                                             \
+        const float ov = dpp_f<CTRL>(v);                                                          \
+        const uint32_t oi = (uint32_t)dpp_i<CTRL>((int)i);                                        \
+        if (better(ov, oi, v, i)) { v = ov; i = oi; }                                             \
+    }
+    QK_STEP(DPP_XOR1) QK_STEP(DPP_XOR2) QK_STEP(DPP_HALF_MIRROR) QK_STEP(DPP_MIRROR)
+#undef QK_STEP
+}
+
+struct Q6Frag { // one lane's share of a Q6_K block in the B-operand cut
+    uint32_t ql[2][2][2], qh[2][2];
+    uint4 sc;
+    uint16_t d;
+    __device__ __forceinline__ void load(const uint8_t* p, int g)
+    {
+#pragma unroll
+        for (int n = 0; n < 2; n++)
+#pragma unroll
+            for (int hf = 0; hf < 2; hf++) {
+#pragma unroll
+                for (int cb = 0; cb < 2; cb++) ql[n][cb][hf] = ldg<uint32_t>(p + 64 * n + 32 * cb + 16 * hf + 4 * g);
+                qh[n][hf] = ldg<uint32_t>(p + Q6_K_QH + 32 * n + 16 * hf + 4 * g);
+            }
+        sc = ldg<uint4>(p + Q6_K_SC);
+        d = ldg<uint16_t>(p + Q6_K_D);
+    }
+    // weights of scale group kk (0..15) as four exact halves (q - 32), and d*scale
+    __device__ __forceinline__ half4 group(int kk, float& scale) const
+    {
+        const int n = kk >> 3, c = (kk >> 1) & 3, hf = kk & 1;
+        const uint32_t l4 = ql[n][c & 1][hf];
+        const uint32_t nib = (c >= 2 ? (l4 >> 4) : l4) & 0x0F0F0F0Fu;
+        const uint32_t q4 = nib | (((qh[n][hf] >> (2 * c)) << 4) & 0x30303030u);
+        const uint32_t sw = kk < 4 ? sc.x : kk < 8 ? sc.y : kk < 12 ? sc.z : sc.w;
+        scale = h2f(d) * (float)(int8_t)(sw >> (8 * (kk & 3)));
+        return bytes_to_half4(q4, 32.f);
+    }
+};
+
+template <int KBLOCKS> // K = 256*KBLOCKS
+__global__ __launch_bounds__(1024) void head_q6k_mfma_kernel(const uint8_t* __restrict__ W,
+                                                             const float* __restrict__ X,
+                                                             float* __restrict__ logits_out,
+                                                             uint32_t* __restrict__ tok, HeadWs ws, uint32_t V,
+                                                             uint32_t batch)
+{
+    constexpr uint32_t K = 256 * KBLOCKS, ROW = Q6_K_BYTES * KBLOCKS;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    _Float16* s_hi = (_Float16*)smem;
+    _Float16* s_lo = s_hi + 16 * K;
+    __shared__ float s_v[16][16];
+    __shared__ uint32_t s_i[16][16];
+    __shared__ uint32_t s_last;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int j = lane & 15, g = lane >> 4;
+
+    stage_tokens<16>(s_hi, s_lo, X, K, batch, [](uint32_t r) { return r; }, tid, 1024);
+    __syncthreads();
+
+    float bv[4];
+    uint32_t bi[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) { bv[e] = ARG_FLOOR; bi[e] = 0xFFFFFFFFu; }
+
+    // Tiles of 16 rows are dealt round-robin to the waves; within a tile the blocks are walked
+    // with the next block's loads in flight during the MFMAs of the current one.
+    const uint32_t tiles = (V + 15) / 16;
+    const uint32_t tstride = gridDim.x * 16;
+    uint32_t mt = blockIdx.x * 16 + wave;
+    Q6Frag f[2];
+    auto fetch = [&](int set, uint32_t tile, int blk) {
+        f[set].load(W + (size_t)min(tile * 16 + j, V - 1) * ROW + (size_t)blk * Q6_K_BYTES, g);
+    };
+    auto consume = [&](int set, int blk, float4v& acc) {
+#pragma unroll
+        for (int kk = 0; kk < 16; kk++) {
+            float sc;
+            const half4 b = f[set].group(kk, sc);
+            const uint32_t frag = (uint32_t)blk * 16 + kk;
+            const half4 ah = *(const half4*)(s_hi + ((size_t)frag * 64 + lane) * 4);
+            const half4 al = *(const half4*)(s_lo + ((size_t)frag * 64 + lane) * 4);
+            float4v part = mfma16x16(ah, b, float4v{0.f, 0.f, 0.f, 0.f});
+            part = mfma16x16(al, b, part);
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[e] += sc * part[e];
+        }
+    };
+    fetch(0, mt, 0);
+    for (; mt < tiles; mt += tstride) {
+        float4v acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+        for (int blk = 0; blk < KBLOCKS; blk += 2) {
+            fetch(1, mt, blk + 1);
+            consume(0, blk, acc);
+            // block after next: of this tile, or the first block of the wave's next tile
+            const bool wrap = blk + 2 >= KBLOCKS;
+            fetch(0, wrap ? mt + tstride : mt, wrap ? 0 : blk + 2);
+            consume(1, blk + 1, acc);
+        }
+        const uint32_t row = mt * 16 + j;
+        if (row < V) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const uint32_t t = 4 * g + e;
+                if (t < batch) {
+                    if (logits_out) logits_out[(size_t)t * V + row] = acc[e];
+                    if (acc[e] > bv[e]) { bv[e] = acc[e]; bi[e] = row; } // a lane's rows ascend
+                }
+            }
+        }
+    }
+    // per token: fold the 16 rows of the lane group, then the 16 waves, then the workgroups
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        dpp_better(bv[e], bi[e]);
+        if (j == 0) { s_v[wave][4 * g + e] = bv[e]; s_i[wave][4 * g + e] = bi[e]; }
+    }
+    __syncthreads();
+    if (tid < 16 && (uint32_t)tid < batch) {
+        float v = s_v[0][tid];
+        uint32_t i = s_i[0][tid];
+        for (int w = 1; w < 16; w++)
+            if (better(s_v[w][tid], s_i[w][tid], v, i)) { v = s_v[w][tid]; i = s_i[w][tid]; }
+        publish(&ws.cand_v[(size_t)tid * gridDim.x + blockIdx.x], v);
+        publish(&ws.cand_i[(size_t)tid * gridDim.x + blockIdx.x], i);
+    }
+    __syncthreads();
+    if (tid == 0) s_last = arrive_last(&ws.counter[0], gridDim.x) ? 1u : 0u;
+    __syncthreads();
+    if (s_last) {
+        // one wave per token folds the workgroups' candidates
+        if ((uint32_t)wave < batch) {
+            float v = ARG_FLOOR;
+            uint32_t i = 0xFFFFFFFFu;
+            for (uint32_t c = lane; c < gridDim.x; c += 64) {
+                const float cv = ws.cand_v[(size_t)wave * gridDim.x + c];
+                const uint32_t ci = ws.cand_i[(size_t)wave * gridDim.x + c];
+                if (better(cv, ci, v, i)) { v = cv; i = ci; }
+            }
+            dpp_better(v, i);
+            // four rows of 16 lanes remain
+            float fv = readlane_f(v, 0);
+            uint32_t fi = (uint32_t)__builtin_amdgcn_readlane((int)i, 0);
+#pragma unroll
+            for (int r = 16; r < 64; r += 16) {
+                const float ov = readlane_f(v, r);
+                const uint32_t oi = (uint32_t)__builtin_amdgcn_readlane((int)i, r);
+                if (better(ov, oi, fv, fi)) { fv = ov; fi = oi; }
+            }
+            if (lane == 0) tok[wave] = fi == 0xFFFFFFFFu ? 0u : fi;
+        }
+        if (tid == 0) ws.counter[0] = 0u;
+    }
+}
+
 static uint32_t head_blocks(uint32_t V, uint32_t rif)
 {
     const uint32_t waves = (V + rif - 1) / rif;
@@ -168,7 +344,7 @@ extern "C" {
 size_t qkk_head_workspace_bytes(uint32_t V, uint32_t batch)
 {
     if (V == 0 || batch == 0) return 0;
-    const size_t blocks = head_blocks(V, 1); // upper bound over the kernels' RIF choices
+    const size_t blocks = std::max<size_t>(head_blocks(V, 1), persistent_blocks() / 4); // upper bound over the kernels
     return 256 + (size_t)batch * blocks * 8;
 }
 
@@ -186,6 +362,22 @@ int qkk_head_argmax(const void* W, const float* X, uint32_t* tok, float* logits,
                     qkk_head_workspace_bytes(V, batch));
     if (int rc = require_device()) return rc;
     hipStream_t st = as_stream(stream);
+    if (batch >= 2 && batch <= 16 && K == 2048) {
+        HeadWs ws;
+        const uint32_t blocks = persistent_blocks() / 4; // one 16-wave workgroup per CU
+        ws.counter = (uint32_t*)workspace;
+        ws.cand_v = (float*)((uint8_t*)workspace + 256);
+        ws.cand_i = (uint32_t*)(ws.cand_v + (size_t)batch * blocks);
+        const size_t lds = (size_t)2 * 16 * K * sizeof(_Float16);
+        static bool attr_done = false;
+        if (!attr_done) {
+            (void)hipFuncSetAttribute((const void*)head_q6k_mfma_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 4096);
+            attr_done = true;
+        }
+        hipLaunchKernelGGL(head_q6k_mfma_kernel<8>, dim3(blocks), dim3(1024), lds, st, (const uint8_t*)W, X, logits,
+                           tok, ws, V, batch);
+        return check_launch("qkk_head_argmax");
+    }
     const uint32_t rif = K == 2048 ? HEAD_RIF : 2;
     const uint32_t blocks = head_blocks(V, rif);
     HeadWs ws;

@@ -146,7 +146,7 @@ __global__ __launch_bounds__(512) void moe_route_multi_kernel(const float* __res
                 a1 += w[i].z * xx[j][i].z + w[i].w * xx[j][i].w;
             }
             const float s = wave_sum(a0 + a1);
-            if (lane == 0 && t0 + j < N) ws.logits[(size_t)(t0 + j) * LS + t] = s;
+            if (lane == 0 && t0 + j < N) publish(&ws.logits[(size_t)(t0 + j) * LS + t], s);
         }
     } else if (t0 < N) {
         const uint32_t r = t - n_dense;
@@ -180,14 +180,12 @@ __global__ __launch_bounds__(512) void moe_route_multi_kernel(const float* __res
     }
     if (!select_here) return;
 
+    // only the logits are read back inside this launch (by the selecting workgroup); the
+    // shared-expert h is read by the next launch
     __syncthreads();
-    if (threadIdx.x == 0) {
-        __threadfence();
-        s_last = atomicAdd(&ws.counter[0], 1u) == gridDim.x - 1 ? 1u : 0u;
-    }
+    if (threadIdx.x == 0) s_last = arrive_last(&ws.counter[0], gridDim.x) ? 1u : 0u;
     __syncthreads();
     if (s_last) {
-        __threadfence();
         select_and_group<NW>(ws, sel, d, N, s_log, s_cnt, s_cur);
         if (threadIdx.x == 0) ws.counter[0] = 0u;
     }
