@@ -229,7 +229,7 @@ __global__ __launch_bounds__(1024) void head_q6k_mfma_kernel(const uint8_t* __re
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int j = lane & 15, g = lane >> 4;
 
-    stage_tokens<16>(s_hi, s_lo, X, K, batch, [](uint32_t r) { return r; }, tid, 1024);
+    stage_tokens<16>(s_hi, s_lo, X, K, K, batch, [](uint32_t r) { return r; }, tid, 1024);
     __syncthreads();
 
     float bv[4];

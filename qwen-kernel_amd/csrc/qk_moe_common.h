@@ -30,7 +30,7 @@ struct MoeWs {
     ActiveExpert* active; // [E]
     uint32_t* offsets;    // [E+1]
     uint32_t* pairs;      // [n*k] (token<<4)|pick
-    float* contrib;       // [n][k][H]
+    float* contrib;       // [n][k+1][H], slot k = shared expert
 };
 
 static inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -40,7 +40,7 @@ static inline size_t ws_bytes(const MoeDims& d, uint32_t n)
     size_t b = 256 + align256((size_t)n * lstride(d.E) * 4) + align256((size_t)n * (d.k + 1) * d.F * 4);
     if (n >= 2)
         b += 256 + align256((size_t)d.E * sizeof(ActiveExpert)) + align256((size_t)(d.E + 1) * 4) +
-             align256((size_t)n * d.k * 4) + align256((size_t)n * d.k * d.H * 4);
+             align256((size_t)n * d.k * 4) + align256((size_t)n * (d.k + 1) * d.H * 4);
     return b;
 }
 

@@ -1,14 +1,12 @@
-// qk_moe_grouped.hip -- expert-major MoE step for several tokens (decode slots or a prefill
-// chunk) on VALU.
+// qk_moe_grouped.hip -- routing for several tokens (decode slots or a prefill chunk): router
+// logits, top-k selection and the grouping of (token, pick) pairs by expert.
 //
-// Each expert picked by at least one token is visited once: its gate/up rows and its down
-// rows are fetched once and applied to every (token, pick) pair routed to it, so the
-// expert's bytes cross HBM once however many tokens share it
-// (the expert-major order of reference shaders/moe_gateup_iq3_grouped.comp:30-114 and
+// Each expert picked by at least one token is then visited once by the MFMA kernels of
+// qk_moe_mfma.hip: its gate/up rows and its down rows cross HBM once however many tokens
+// share it (the expert-major order of reference shaders/moe_gateup_iq3_grouped.comp:30-114 and
 // moe_down_iq4_grouped.comp:24-75, driven by the pair lists of moe_group_pairs.comp).
-// Launches: route (router logits, shared gate/up, and -- in the block that finishes last --
-// top-k selection and pair grouping), grouped gate/up, grouped down into per-pair
-// contributions, fold (+ shared down).
+// Launches of a step: route (router logits and -- in the workgroup that finishes last --
+// selection + grouping; a launch of its own above 64 tokens), gate/up, down, fold.
 #include "qk_moe_common.h"
 
 #include <algorithm>
@@ -100,33 +98,29 @@ __device__ static void select_and_group(const MoeWs& ws, qkk_sel* __restrict__ s
     }
 }
 
-// ---- launch 1: router + shared gate/up for N tokens ----------------------------------------
-// One wave per task = (router row | shared row pair) x (group of TG tokens).  All loads of a
-// task -- its weights and the TG activation slices -- are issued together: one memory round
-// trip per task.  Weights are re-read once per token group (from L2 after the first).
+// ---- launch 1: router logits for N tokens ----------------------------------------------------
+// One wave per task = (router row, group of TG tokens); row E is the shared-gate row.  All loads
+// of a task -- the row and the TG activation rows -- are issued together: one memory round trip
+// per task.  The router matrix is re-read once per token group (from L2 after the first).
 template <int NCH>
 __global__ __launch_bounds__(512) void moe_route_multi_kernel(const float* __restrict__ gate_inp,
                                                               const float* __restrict__ gate_inp_shexp,
-                                                              const uint8_t* __restrict__ gate_shexp,
-                                                              const uint8_t* __restrict__ up_shexp,
                                                               const float* __restrict__ X, MoeWs ws,
                                                               qkk_sel* __restrict__ sel, MoeDims d, uint32_t N,
                                                               uint32_t select_here)
 {
-    constexpr int P = NCH / 8;
     constexpr int TG = NCH <= 8 ? 4 : 2; // tokens per task
     constexpr int NW = 8;                // waves per block
     __shared__ uint32_t s_last;
     __shared__ float s_log[NW * (QKK_MAX_EXPERTS + 8)];
     __shared__ uint32_t s_cnt[QKK_MAX_EXPERTS + 1], s_cur[QKK_MAX_EXPERTS + 1];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t n_dense = d.E + 1, n_rows = n_dense + d.F;
-    const uint32_t q8_row = d.H / 32 * Q8_0_BYTES;
+    const uint32_t n_rows = d.E + 1;
     const uint32_t task = blockIdx.x * NW + wave;
     const uint32_t t = task % n_rows, t0 = (task / n_rows) * TG;
     const uint32_t LS = lstride(d.E);
 
-    if (t0 < N && t < n_dense) {
+    if (t0 < N) {
         const float4* row = (const float4*)(t < d.E ? gate_inp + (size_t)t * d.H : gate_inp_shexp);
         float4 w[NCH], xx[TG][NCH];
 #pragma unroll
@@ -148,40 +142,9 @@ __global__ __launch_bounds__(512) void moe_route_multi_kernel(const float* __res
             const float s = wave_sum(a0 + a1);
             if (lane == 0 && t0 + j < N) publish(&ws.logits[(size_t)(t0 + j) * LS + t], s);
         }
-    } else if (t0 < N) {
-        const uint32_t r = t - n_dense;
-        LaneW<QKK_Q8_0> wg[P], wu[P];
-        XSlice xs[TG][P];
-#pragma unroll
-        for (int p = 0; p < P; p++) {
-            wg[p].load(gate_shexp + (size_t)r * q8_row + (size_t)p * 64 * Q8_0_BYTES, lane);
-            wu[p].load(up_shexp + (size_t)r * q8_row + (size_t)p * 64 * Q8_0_BYTES, lane);
-        }
-#pragma unroll
-        for (int j = 0; j < TG; j++)
-#pragma unroll
-            for (int p = 0; p < P; p++)
-                load_xslice<QKK_Q8_0>(xs[j][p], X + (size_t)min(t0 + j, N - 1) * d.H + p * 2048, lane);
-#pragma unroll
-        for (int j = 0; j < TG; j++) {
-            float g = 0.f, u = 0.f;
-#pragma unroll
-            for (int p = 0; p < P; p++) {
-                wg[p].touch();
-                wu[p].touch();
-                g += wg[p].dot(xs[j][p], nullptr, nullptr, lane);
-                u += wu[p].dot(xs[j][p], nullptr, nullptr, lane);
-            }
-            g = wave_sum(g);
-            u = wave_sum(u);
-            if (lane == 0 && t0 + j < N)
-                ws.h[((size_t)(t0 + j) * (d.k + 1) + d.k) * d.F + r] = (g / (1.f + expf(-g))) * u;
-        }
     }
     if (!select_here) return;
 
-    // only the logits are read back inside this launch (by the selecting workgroup); the
-    // shared-expert h is read by the next launch
     __syncthreads();
     if (threadIdx.x == 0) s_last = arrive_last(&ws.counter[0], gridDim.x) ? 1u : 0u;
     __syncthreads();
@@ -200,225 +163,29 @@ __global__ __launch_bounds__(1024) void moe_select_group_kernel(MoeWs ws, qkk_se
     select_and_group<16>(ws, sel, d, N, s_log, s_cnt, s_cur);
 }
 
-// ---- launch 2: expert-major gate/up -----------------------------------------------------------
-template <int TYPE, int PASSES, int RIF>
-__global__ __launch_bounds__(256) void moe_gateup_grouped_kernel(const uint8_t* __restrict__ gate_exps,
-                                                                 const uint8_t* __restrict__ up_exps,
-                                                                 const float* __restrict__ X, MoeWs ws, MoeDims d)
-{
-    __shared__ IqTables tab;
-    fill_iq_tables(tab, g_iq3xxs_grid, threadIdx.x, 256);
-    __syncthreads();
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t row_bytes = (uint32_t)qkk_row_bytes_dev<TYPE>(d.H);
-    const uint32_t pass_bytes = row_bytes / PASSES;
-    const uint32_t groups = (d.F + RIF - 1) / RIF;
-    const uint32_t n_tasks = *ws.n_active * groups;
-    for (uint32_t task = blockIdx.x * 4 + wave; task < n_tasks; task += gridDim.x * 4) {
-        const ActiveExpert a = ws.active[task / groups];
-        const uint32_t r0 = (task % groups) * RIF;
-        const uint8_t* gbase = gate_exps + ((size_t)a.expert * d.F) * row_bytes;
-        const uint8_t* ubase = up_exps + ((size_t)a.expert * d.F) * row_bytes;
-        LaneW<TYPE> wg[RIF][PASSES], wu[RIF][PASSES];
-#pragma unroll
-        for (int i = 0; i < RIF; i++) {
-            const uint32_t r = min(r0 + i, d.F - 1);
-#pragma unroll
-            for (int p = 0; p < PASSES; p++) {
-                wg[i][p].load(gbase + (size_t)r * row_bytes + (size_t)p * pass_bytes, lane);
-                wu[i][p].load(ubase + (size_t)r * row_bytes + (size_t)p * pass_bytes, lane);
-            }
-        }
-        for (uint32_t q = 0; q < a.count; q++) {
-            const uint32_t pr = ws.pairs[a.first + q];
-            const uint32_t tok = pr >> 4, s = pr & 15u;
-            XSlice xs[PASSES];
-#pragma unroll
-            for (int p = 0; p < PASSES; p++) load_xslice<TYPE>(xs[p], X + (size_t)tok * d.H + p * 2048, lane);
-#pragma unroll
-            for (int i = 0; i < RIF; i++) {
-#pragma unroll
-                for (int p = 0; p < PASSES; p++) {
-                    wg[i][p].touch();
-                    wu[i][p].touch();
-                }
-                float g = 0.f, u = 0.f;
-#pragma unroll
-                for (int p = 0; p < PASSES; p++) {
-                    g += wg[i][p].dot(xs[p], nullptr, &tab, lane);
-                    u += wu[i][p].dot(xs[p], nullptr, &tab, lane);
-                }
-                g = wave_sum(g);
-                u = wave_sum(u);
-                if (lane == 0 && r0 + i < d.F)
-                    ws.h[((size_t)tok * (d.k + 1) + s) * d.F + r0 + i] = (g / (1.f + expf(-g))) * u;
-            }
-        }
-    }
-}
+void moe_mfma_launch(const qkk_moe_layer* L, const float* X, float* Y, const qkk_sel* sel, const MoeWs& ws,
+                     const MoeDims& d, uint32_t N, uint32_t stages, hipStream_t st);
 
-// ---- launch 3: expert-major down into per-pair contributions -----------------------------------
-// contrib[(token*k + pick)*H + o] = w[token][pick] * (D_expert[o] . h[token][pick])
-// (reference shaders/moe_down_iq4_grouped.comp:67-72).  F = 32*LPR.
-template <int TYPE, int LPR, int RIF>
-__global__ __launch_bounds__(256) void moe_down_grouped_kernel(const uint8_t* __restrict__ down_exps, MoeWs ws,
-                                                               const qkk_sel* __restrict__ sel, MoeDims d)
-{
-    __shared__ IqTables tab;
-    fill_iq_tables(tab, g_iq3xxs_grid, threadIdx.x, 256);
-    __syncthreads();
-    constexpr int GROUPS = WAVE / LPR;
-    constexpr uint32_t CHUNK = GROUPS * RIF;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int lir = lane % LPR, grp = lane / LPR;
-    const uint32_t row_bytes = (uint32_t)qkk_row_bytes_dev<TYPE>(d.F);
-    const uint32_t chunks = (d.H + CHUNK - 1) / CHUNK;
-    const uint32_t n_tasks = *ws.n_active * chunks;
-    for (uint32_t task = blockIdx.x * 4 + wave; task < n_tasks; task += gridDim.x * 4) {
-        const ActiveExpert a = ws.active[task / chunks];
-        const uint32_t o0 = (task % chunks) * CHUNK;
-        const uint8_t* base = down_exps + (size_t)a.expert * d.H * row_bytes;
-        LaneW<TYPE> w[RIF];
-#pragma unroll
-        for (int i = 0; i < RIF; i++)
-            w[i].load(base + (size_t)min(o0 + i * GROUPS + grp, d.H - 1) * row_bytes, lir);
-        for (uint32_t q = 0; q < a.count; q++) {
-            const uint32_t pr = ws.pairs[a.first + q];
-            const uint32_t tok = pr >> 4, s = pr & 15u;
-            const float wt = sel[tok].w[s];
-            XSlice hs;
-            load_xslice<TYPE>(hs, ws.h + ((size_t)tok * (d.k + 1) + s) * d.F, lir);
-            float hsum[4];
-#pragma unroll
-            for (int c = 0; c < 4; c++) {
-                float v = 0.f;
-#pragma unroll
-                for (int i = 0; i < 8; i++) v += hs.v[c * 8 + i];
-                hsum[c] = v;
-            }
-#pragma unroll
-            for (int i = 0; i < RIF; i++) {
-                float acc = wt * w[i].dot(hs, hsum, &tab, lir);
-                acc = lanes_sum<LPR>(acc);
-                const uint32_t o = o0 + i * GROUPS + grp;
-                if (lir == 0 && o < d.H) ws.contrib[((size_t)tok * d.k + s) * d.H + o] = acc;
-            }
-        }
-    }
-}
-
-// ---- launch 4: fold the contributions, add the shared expert -------------------------------------
-// Y[t][o] = sum_s contrib[t][s][o] + w_shared[t] * (Ds[o] . h[t][k]); the shared down rows stay
-// in registers while the wave walks the tokens.
-template <int LPR, int RIF>
-__global__ __launch_bounds__(256) void moe_fold_shared_kernel(const uint8_t* __restrict__ down_shexp, MoeWs ws,
-                                                              const qkk_sel* __restrict__ sel,
-                                                              float* __restrict__ Y, MoeDims d, uint32_t N)
-{
-    constexpr int GROUPS = WAVE / LPR;
-    constexpr uint32_t CHUNK = GROUPS * RIF;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int lir = lane % LPR, grp = lane / LPR;
-    const uint32_t q8_row = d.F / 32 * Q8_0_BYTES;
-    for (uint32_t o0 = (blockIdx.x * 4 + wave) * CHUNK; o0 < d.H; o0 += gridDim.x * 4 * CHUNK) {
-        LaneW<QKK_Q8_0> w[RIF];
-#pragma unroll
-        for (int i = 0; i < RIF; i++)
-            w[i].load(down_shexp + (size_t)min(o0 + i * GROUPS + grp, d.H - 1) * q8_row, lir);
-        for (uint32_t t = 0; t < N; t++) {
-            XSlice hs;
-            load_xslice<QKK_Q8_0>(hs, ws.h + ((size_t)t * (d.k + 1) + d.k) * d.F, lir);
-            const float wsh = sel[t].w_shared;
-            float part[RIF];
-#pragma unroll
-            for (int i = 0; i < RIF; i++) {
-                const uint32_t o = min(o0 + i * GROUPS + grp, d.H - 1);
-                float c = 0.f;
-                for (uint32_t s = lir; s < d.k; s += LPR) c += ws.contrib[((size_t)t * d.k + s) * d.H + o];
-                part[i] = c;
-            }
-#pragma unroll
-            for (int i = 0; i < RIF; i++) {
-                float acc = wsh * w[i].dot(hs, nullptr, nullptr, lir) + part[i];
-                acc = lanes_sum<LPR>(acc);
-                const uint32_t o = o0 + i * GROUPS + grp;
-                if (lir == 0 && o < d.H) Y[(size_t)t * d.H + o] = acc;
-            }
-        }
-    }
-}
-
-template <int TYPE, int LPR>
-static void launch_down_grouped(const qkk_moe_layer* L, const MoeWs& ws, const qkk_sel* sel, const MoeDims& d,
-                                uint32_t max_active, hipStream_t st)
-{
-    constexpr int RIF = 4;
-    const uint32_t chunks = (d.H + (64 / LPR) * RIF - 1) / ((64 / LPR) * RIF);
-    const uint32_t blocks = std::min((max_active * chunks + 3) / 4, persistent_blocks());
-    hipLaunchKernelGGL((moe_down_grouped_kernel<TYPE, LPR, RIF>), dim3(blocks), dim3(256), 0, st,
-                       (const uint8_t*)L->down_exps, ws, sel, d);
-}
-
-template <int LPR>
-static void launch_fold(const qkk_moe_layer* L, const MoeWs& ws, const qkk_sel* sel, float* Y, const MoeDims& d,
-                        uint32_t N, hipStream_t st)
-{
-    constexpr int RIF = 2;
-    const uint32_t chunks = (d.H + (64 / LPR) * RIF - 1) / ((64 / LPR) * RIF);
-    hipLaunchKernelGGL((moe_fold_shared_kernel<LPR, RIF>), dim3((chunks + 3) / 4), dim3(256), 0, st,
-                       (const uint8_t*)L->down_shexp, ws, sel, Y, d, N);
-}
-
-// Host entry of the grouped path (arguments already validated).
+// Host entry of the path for N >= 2 rows (arguments already validated).
 int moe_grouped_launch(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* sel, void* workspace,
                        uint32_t N, uint32_t stages, hipStream_t st)
 {
     const MoeDims d{L->n_embd, L->n_ff, L->n_expert, L->n_used};
     const MoeWs ws = ws_carve(workspace, d, N);
-    const uint32_t t1 = d.E + 1 + d.F;
-    const uint32_t inline_sel = N <= SELECT_INLINE_MAX ? 1u : 0u;
-    const uint8_t* gs = (const uint8_t*)L->gate_shexp;
-    const uint8_t* us = (const uint8_t*)L->up_shexp;
-    if (!(stages & QKK_STAGE_ROUTE)) {
-    } else if (d.H == 2048) {
-        const uint32_t tasks = t1 * ((N + 3) / 4);
-        hipLaunchKernelGGL(moe_route_multi_kernel<8>, dim3((tasks + 7) / 8), dim3(512), 0, st, L->gate_inp,
-                           L->gate_inp_shexp, gs, us, X, ws, sel, d, N, inline_sel);
-    } else {
-        const uint32_t tasks = t1 * ((N + 1) / 2);
-        hipLaunchKernelGGL(moe_route_multi_kernel<16>, dim3((tasks + 7) / 8), dim3(512), 0, st, L->gate_inp,
-                           L->gate_inp_shexp, gs, us, X, ws, sel, d, N, inline_sel);
+    if (stages & QKK_STAGE_ROUTE) {
+        const uint32_t inline_sel = N <= SELECT_INLINE_MAX ? 1u : 0u;
+        if (d.H == 2048) {
+            const uint32_t tasks = (d.E + 1) * ((N + 3) / 4);
+            hipLaunchKernelGGL(moe_route_multi_kernel<8>, dim3((tasks + 7) / 8), dim3(512), 0, st, L->gate_inp,
+                               L->gate_inp_shexp, X, ws, sel, d, N, inline_sel);
+        } else {
+            const uint32_t tasks = (d.E + 1) * ((N + 1) / 2);
+            hipLaunchKernelGGL(moe_route_multi_kernel<16>, dim3((tasks + 7) / 8), dim3(512), 0, st, L->gate_inp,
+                               L->gate_inp_shexp, X, ws, sel, d, N, inline_sel);
+        }
+        if (!inline_sel) hipLaunchKernelGGL(moe_select_group_kernel, dim3(1), dim3(1024), 0, st, ws, sel, d, N);
     }
-    if ((stages & QKK_STAGE_ROUTE) && !inline_sel) hipLaunchKernelGGL(moe_select_group_kernel, dim3(1), dim3(1024), 0, st, ws, sel, d, N);
-
-    const uint32_t max_active = std::min<uint64_t>(d.E, (uint64_t)N * d.k);
-    const uint8_t* ge = (const uint8_t*)L->gate_exps;
-    const uint8_t* ue = (const uint8_t*)L->up_exps;
-    if (!(stages & QKK_STAGE_GATEUP)) {
-    } else if (d.H == 2048) {
-        constexpr int RIF = 4;
-        const uint32_t blocks = std::min((max_active * ((d.F + RIF - 1) / RIF) + 3) / 4, persistent_blocks());
-        hipLaunchKernelGGL((moe_gateup_grouped_kernel<QKK_IQ3_XXS, 1, RIF>), dim3(blocks), dim3(256), 0, st, ge, ue,
-                           X, ws, d);
-    } else {
-        constexpr int RIF = 2;
-        const uint32_t blocks = std::min((max_active * ((d.F + RIF - 1) / RIF) + 3) / 4, persistent_blocks());
-        hipLaunchKernelGGL((moe_gateup_grouped_kernel<QKK_IQ3_XXS, 2, RIF>), dim3(blocks), dim3(256), 0, st, ge, ue,
-                           X, ws, d);
-    }
-    if (!(stages & QKK_STAGE_DOWN)) return check_launch("moe grouped path");
-    if (L->down_type == QKK_IQ4_XS) {
-        if (d.F == 512) launch_down_grouped<QKK_IQ4_XS, 16>(L, ws, sel, d, max_active, st);
-        else if (d.F == 256) launch_down_grouped<QKK_IQ4_XS, 8>(L, ws, sel, d, max_active, st);
-        else launch_down_grouped<QKK_IQ4_XS, 32>(L, ws, sel, d, max_active, st);
-    } else {
-        if (d.F == 512) launch_down_grouped<QKK_Q6_K, 16>(L, ws, sel, d, max_active, st);
-        else if (d.F == 256) launch_down_grouped<QKK_Q6_K, 8>(L, ws, sel, d, max_active, st);
-        else launch_down_grouped<QKK_Q6_K, 32>(L, ws, sel, d, max_active, st);
-    }
-    if (d.F == 512) launch_fold<16>(L, ws, sel, Y, d, N, st);
-    else if (d.F == 256) launch_fold<8>(L, ws, sel, Y, d, N, st);
-    else launch_fold<32>(L, ws, sel, Y, d, N, st);
+    moe_mfma_launch(L, X, Y, sel, ws, d, N, stages, st);
     return check_launch("moe grouped path");
 }
 
