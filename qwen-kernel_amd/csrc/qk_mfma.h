@@ -5,8 +5,8 @@
 // The lane that decodes row l%16 for B therefore also owns that row's outputs, and per-block
 // scales are applied lane-locally in fp32 AFTER the MFMA: the weight operand holds only the
 // block's small integers (exact in half), the activation operand is split x = hi + lo (two
-// halves, x exact to ~2^-22).  Kernels that fold a block's integer sub-scale into the weight
-// operand (to make a lane's weight bytes contiguous) round that product to half once.
+// halves, x exact to ~2^-22).  Kernels that fold a block's sub-scale into the weight operand (to
+// make a lane's weight bytes contiguous) carry the rounding residual in a second operand.
 #pragma once
 #include "qk_device.h"
 
@@ -66,95 +66,6 @@ __device__ __forceinline__ void stage_tokens(_Float16* __restrict__ s_hi, _Float
             s_hi[off + e] = hi;
             s_lo[off + e] = (_Float16)(f[e] - (float)hi);
         }
-    }
-}
-
-// Same LDS layouts as stage_tokens, written for speed: every thread converts whole lane
-// pieces (KE = 8 halves for K=32 fragments, 4 for K=16), all global loads of a thread are in
-// flight together, and consecutive threads write consecutive LDS pieces.  KT = staged width;
-// up to 16 rows, rows >= n_rows read as zero; row r of the tile is X + row_of(r)*stride.
-template <int KE, int KT, int NTHREADS, typename RowOf>
-__device__ __forceinline__ void stage_rows(_Float16* __restrict__ s_hi, _Float16* __restrict__ s_lo,
-                                           const float* __restrict__ X, uint32_t stride, uint32_t n_rows,
-                                           RowOf row_of, int tid)
-{
-    constexpr int PIECES = 16 * KT / KE, IT = (PIECES + NTHREADS - 1) / NTHREADS;
-    float v[IT][KE];
-#pragma unroll
-    for (int it = 0; it < IT; it++) {
-        const uint32_t q = min((uint32_t)(tid + it * NTHREADS), (uint32_t)PIECES - 1);
-        const uint32_t row = q & 15u, g = (q >> 4) & 3u, step = q >> 6;
-        const float* src = X + (size_t)row_of(min(row, n_rows - 1)) * stride + step * (4 * KE) + g * KE;
-#pragma unroll
-        for (int c = 0; c < KE / 4; c++) {
-            const float4 f = *(const float4*)(src + 4 * c);
-            v[it][4 * c] = f.x; v[it][4 * c + 1] = f.y; v[it][4 * c + 2] = f.z; v[it][4 * c + 3] = f.w;
-        }
-    }
-#pragma unroll
-    for (int it = 0; it < IT; it++) {
-        const uint32_t q = tid + it * NTHREADS;
-        if (PIECES % NTHREADS != 0 && q >= (uint32_t)PIECES) break;
-        const float keep = (q & 15u) < n_rows ? 1.f : 0.f;
-        _Float16 hi[KE], lo[KE];
-#pragma unroll
-        for (int e = 0; e < KE; e++) {
-            const float x = v[it][e] * keep;
-            hi[e] = (_Float16)x;
-            lo[e] = (_Float16)(x - (float)hi[e]);
-        }
-        if constexpr (KE == 8) {
-            *(half8*)(s_hi + (size_t)q * 8) = half8{hi[0], hi[1], hi[2], hi[3], hi[4], hi[5], hi[6], hi[7]};
-            *(half8*)(s_lo + (size_t)q * 8) = half8{lo[0], lo[1], lo[2], lo[3], lo[4], lo[5], lo[6], lo[7]};
-        } else {
-            *(half4*)(s_hi + (size_t)q * 4) = half4{hi[0], hi[1], hi[2], hi[3]};
-            *(half4*)(s_lo + (size_t)q * 4) = half4{lo[0], lo[1], lo[2], lo[3]};
-        }
-    }
-}
-
-// Staging for fragments that span one 256-weight super-block (8 steps of K = 32) in which a
-// lane group does not take every fourth run of 8 weights but a cut that makes its share of
-// the weight bytes contiguous in the block:
-//   LAYOUT 0: group g holds weights [64g, 64g+64), step i the eight at 64g + 8i
-//   LAYOUT 1 (Q6_K): group g holds, of the 128-weight half g/2, the 16-weight scale groups of
-//             parity g%2; step i the eight at 128(g/2) + 32(i/2) + 16(g%2) + 8(i%2)
-// (the four lane groups of one MFMA then lie in different scale groups, so all scales below
-// the super-block's are folded into the weight operand).  LDS order is
-// [fragment][step][lane = 16g + row][8 halves]; KT = staged width, up to 16 rows, rows >=
-// n_rows read as zero; row r of the tile is X + row_of(r)*stride.
-template <int LAYOUT, int KT, int NTHREADS, typename RowOf>
-__device__ __forceinline__ void stage_rows256(_Float16* __restrict__ s_hi, _Float16* __restrict__ s_lo,
-                                              const float* __restrict__ X, uint32_t stride, uint32_t n_rows,
-                                              RowOf row_of, int tid)
-{
-    constexpr int PIECES = 16 * KT / 8, IT = (PIECES + NTHREADS - 1) / NTHREADS;
-    float4 v[IT][2];
-#pragma unroll
-    for (int it = 0; it < IT; it++) {
-        const uint32_t q = min((uint32_t)(tid + it * NTHREADS), (uint32_t)PIECES - 1);
-        const uint32_t row = q & 15u, g = (q >> 4) & 3u, i = (q >> 6) & 7u, frag = q >> 9;
-        const uint32_t k = frag * 256 + (LAYOUT == 0 ? 64 * g + 8 * i
-                                                     : 128 * (g >> 1) + 32 * (i >> 1) + 16 * (g & 1) + 8 * (i & 1));
-        const float* src = X + (size_t)row_of(min(row, n_rows - 1)) * stride + k;
-        v[it][0] = *(const float4*)src;
-        v[it][1] = *(const float4*)(src + 4);
-    }
-#pragma unroll
-    for (int it = 0; it < IT; it++) {
-        const uint32_t q = tid + it * NTHREADS;
-        if (PIECES % NTHREADS != 0 && q >= (uint32_t)PIECES) break;
-        const float keep = (q & 15u) < n_rows ? 1.f : 0.f;
-        const float f[8] = {v[it][0].x, v[it][0].y, v[it][0].z, v[it][0].w, v[it][1].x, v[it][1].y, v[it][1].z, v[it][1].w};
-        half8 hi, lo;
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-            const float x = f[e] * keep;
-            hi[e] = (_Float16)x;
-            lo[e] = (_Float16)(x - (float)hi[e]);
-        }
-        *(half8*)(s_hi + (size_t)q * 8) = hi;
-        *(half8*)(s_lo + (size_t)q * 8) = lo;
     }
 }
 

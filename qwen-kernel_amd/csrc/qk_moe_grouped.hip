@@ -171,18 +171,14 @@ int moe_grouped_launch(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel
                        uint32_t N, uint32_t stages, hipStream_t st)
 {
     const MoeDims d{L->n_embd, L->n_ff, L->n_expert, L->n_used};
+    // the matrix-core kernels split n_embd over the eight waves of a workgroup, 256 weights each
+    if (d.H != 2048) return fail(QKK_ESHAPE, "moe: several rows need n_embd = 2048 (got %u)", d.H);
     const MoeWs ws = ws_carve(workspace, d, N);
     if (stages & QKK_STAGE_ROUTE) {
         const uint32_t inline_sel = N <= SELECT_INLINE_MAX ? 1u : 0u;
-        if (d.H == 2048) {
-            const uint32_t tasks = (d.E + 1) * ((N + 3) / 4);
-            hipLaunchKernelGGL(moe_route_multi_kernel<8>, dim3((tasks + 7) / 8), dim3(512), 0, st, L->gate_inp,
-                               L->gate_inp_shexp, X, ws, sel, d, N, inline_sel);
-        } else {
-            const uint32_t tasks = (d.E + 1) * ((N + 1) / 2);
-            hipLaunchKernelGGL(moe_route_multi_kernel<16>, dim3((tasks + 7) / 8), dim3(512), 0, st, L->gate_inp,
-                               L->gate_inp_shexp, X, ws, sel, d, N, inline_sel);
-        }
+        const uint32_t tasks = (d.E + 1) * ((N + 3) / 4);
+        hipLaunchKernelGGL(moe_route_multi_kernel<8>, dim3((tasks + 7) / 8), dim3(512), 0, st, L->gate_inp,
+                           L->gate_inp_shexp, X, ws, sel, d, N, inline_sel);
         if (!inline_sel) hipLaunchKernelGGL(moe_select_group_kernel, dim3(1), dim3(1024), 0, st, ws, sel, d, N);
     }
     moe_mfma_launch(L, X, Y, sel, ws, d, N, stages, st);

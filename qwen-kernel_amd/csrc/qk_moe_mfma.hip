@@ -2,13 +2,13 @@
 // (decode slots or a prefill chunk).
 //
 // A work item is one expert with the (token, pick) pairs routed to it, or the shared expert
-// with 16 consecutive tokens, cut into sub-items by weight-row tiles.  A workgroup of 8 waves
-// takes a sub-item: it gathers 16 of the item's activation rows into LDS as half hi + half lo
-// planes in MFMA fragment order, then every wave streams its weight rows ONCE from HBM and
-// applies them to all 16 rows with v_mfma_f32_16x16x32_f16; the activation fragments a wave
-// reads from LDS are shared by all the weight tiles it holds.  Orientation, exactness and
-// post-scaling: see qk_mfma.h -- the weight operand carries the block's integers, block scales
-// are applied to the MFMA result in fp32.
+// with 16 consecutive tokens, cut into sub-items by weight rows.  A workgroup of 8 waves takes
+// a sub-item: its weight rows are one contiguous byte range, which the workgroup copies to LDS
+// in double-buffered batches with coalesced 16-byte loads; the waves split K (each keeps its
+// 256-wide slice of the 16 activation rows in registers as hi + lo half operands), decode
+// their fragments from LDS into v_mfma_f32_16x16x32_f16 weight operands, and their partial
+// 16x16 results are summed through LDS in a fixed order.  Each weight byte is read from HBM
+// once per 16 rows; the L1 sees each line once.  Orientation and exactness: see qk_mfma.h.
 // (reference shaders/moe_gateup_iq3_grouped_coopmat.comp:46-217, moe_down_iq4_grouped_coopmat.comp:45-166,
 //  moe_gateup_q8_coopmat.comp, moe_down_q8_coopmat.comp.)
 #include "qk_mfma.h"
@@ -20,12 +20,18 @@ namespace qk {
 
 struct MfmaTables {
     uint32_t grid[256]; // IQ3_XXS codewords, four magnitudes per dword
+    uint2 sign[128];    // IQ3_XXS sign selector -> 0xFF in the bytes of the eight weights to negate
     uint32_t iq4[4];    // IQ4 codebook, sixteen int8 in four dwords
 };
 
 __device__ static void fill_mfma_tables(MfmaTables& t, int tid, int nthreads)
 {
     for (int i = tid; i < 256; i += nthreads) t.grid[i] = g_iq3xxs_grid[i];
+    for (int i = tid; i < 128; i += nthreads) {
+        const uint32_t s8 = (uint32_t)i | ((__builtin_popcount(i) & 1u) << 7); // eighth sign = parity
+        const uint32_t a = ((s8 & 15u) * 0x00204081u) & 0x01010101u, b = ((s8 >> 4) * 0x00204081u) & 0x01010101u;
+        t.sign[i] = uint2{(a << 8) - a, (b << 8) - b};
+    }
     if (tid < 4) {
         constexpr int8_t kv[16] = {QK_IQ4NL_VALUES};
         uint32_t w = 0;
@@ -37,10 +43,12 @@ __device__ static void fill_mfma_tables(MfmaTables& t, int tid, int nthreads)
 }
 
 // ---- a lane's share of one 256-weight fragment of row (l%16), in the B-operand cut -----------------
-// What limits these kernels is the number of L1 accesses, one per lane and load instruction,
-// so lane group g = l/16 owns 64 of the fragment's 256 weights chosen so that its bytes are
-// CONTIGUOUS in the block (LAYOUT, see stage_rows256) and fetches them with two or three wide
-// loads.  Step i of 8 feeds eight of them to one K = 32 MFMA.  The four lane groups of a step
+// Lane group g = l/16 owns 64 of the fragment's 256 weights, chosen so that its bytes are
+// CONTIGUOUS in the block and a fragment is two or three wide (LDS) reads:
+//   LAYOUT 0: weights [64g, 64g+64), step i the eight at 64g + 8i
+//   LAYOUT 1 (Q6_K): of the 128-weight half g/2 the 16-weight scale groups of parity g%2;
+//             step i the eight at 128(g/2) + 32(i/2) + 16(g%2) + 8(i%2)
+// Step i of 8 feeds eight of them to one K = 32 MFMA.  The four lane groups of a step
 // then lie in different sub-blocks, so step(i, g, tab, lo) returns the weights times the
 // sub-block scale as halves; post() is what remains, one fp32 factor per row and fragment,
 // applied to the MFMA result.  Where that product does not fit a half exactly (SPLIT), `lo`
@@ -103,23 +111,20 @@ struct BFrag<QKK_IQ3_XXS> { // group g owns sub-blocks 2g, 2g+1: 16 grid indices
         aux = ldg<uint2>(p + IQ3_XXS_AUX + 8 * g);
     }
     __device__ __forceinline__ float post() const { return h2f(d) * 0.25f; } // d * (2s+1)/4, 2s+1 in the operand
-    // four magnitudes (bytes of cw, each <= 62) with sign bits s4 -> four halves +-mag, exact:
-    // the byte 0x80 +- mag under the exponent byte 0x64 is the half 1152 +- mag
-    __device__ __forceinline__ static half4 signed4(uint32_t cw, uint32_t s4)
+    // four magnitudes (bytes of cw, each <= 62), m = 0xFF in the bytes to negate -> four halves
+    // +-mag, exact: the byte 0x80 +- mag under the exponent byte 0x64 is the half 1152 +- mag
+    __device__ __forceinline__ static half4 signed4(uint32_t cw, uint32_t m)
     {
-        const uint32_t t = ((s4 & 15u) * 0x00204081u) & 0x01010101u;
-        const uint32_t m = (t << 8) - t;                               // 0xFF in the bytes to negate
         const uint32_t pos = cw + 0x80808080u, neg = 0x80808080u - cw; // no carry between bytes
         return bytes_to_half4((neg & m) | (pos & ~m), 128.f);
     }
     __device__ __forceinline__ half8 step(int i, int, const MfmaTables& tab, half8&) const
     {
         const uint32_t a = (i >> 2) ? aux.y : aux.x;
-        const uint32_t s7 = (a >> (7 * (i & 3))) & 127u;
-        const uint32_t s8 = s7 | ((__builtin_popcount(s7) & 1u) << 7);
+        const uint2 m = tab.sign[(a >> (7 * (i & 3))) & 127u];
         const uint32_t w = (i >> 1) == 0 ? idx.x : (i >> 1) == 1 ? idx.y : (i >> 1) == 2 ? idx.z : idx.w;
         const uint32_t pr = w >> (16 * (i & 1));
-        const half4 lo = signed4(tab.grid[pr & 255u], s8), hi = signed4(tab.grid[(pr >> 8) & 255u], s8 >> 4);
+        const half4 lo = signed4(tab.grid[pr & 255u], m.x), hi = signed4(tab.grid[(pr >> 8) & 255u], m.y);
         return scale8(lo, hi, (_Float16)(float)((a >> 27) | 1u));
     }
 };
@@ -193,81 +198,179 @@ struct BFrag<QKK_Q6_K> { // group g owns, of half g/2, l = 16(g%2)..16(g%2)+15 o
     }
 };
 
-// Fragment number `fi` of the staged tile for NT weight tiles at once: the activation
-// fragments are read from LDS once per step and reused by all NT tiles; the eight steps chain
-// through the MFMA accumulator and the row's factor is applied once.
-template <int TYPE, int NT>
-__device__ __forceinline__ void mac_multi(const BFrag<TYPE>* f, const _Float16* __restrict__ s_hi,
-                                          const _Float16* __restrict__ s_lo, uint32_t fi, int lane, int g,
-                                          const MfmaTables& tab, float4v* acc)
+// ---- cooperative streaming ----------------------------------------------------------------------------
+// The weight rows of a sub-item are ONE contiguous byte range per tensor (consecutive rows of a
+// row-major tensor), so the workgroup copies it to LDS in batches with fully coalesced 16-byte
+// loads, double-buffered: the L1 sees every line once.  The eight waves split K: wave w owns
+// fragment w % KS of every row (its slice of the 16 activation rows stays in registers as the
+// MFMA A operand, hi + lo halves) and, when KS < 8, tile group w / KS.  Per batch every wave
+// reads its fragments of the batch's tiles from LDS, runs the MFMAs, writes its partial
+// 16x16 results to LDS; after a barrier the partials are summed in wave order (a fixed order:
+// results are bit-reproducible) and handed to the epilogue.
+constexpr int CW = 8;       // waves per workgroup
+constexpr int CT = 64 * CW; // threads per workgroup
+
+// ALT: the NS = 2 tensors take turns, batch 2q = tiles of tensor 0, batch 2q+1 = the same rows
+// of tensor 1 (for blocks too large to double-buffer both tensors' tiles together).
+template <int TYPE, int KS, int NS, int TG, bool ALT = false>
+struct CoopGeom {
+    static constexpr int G = CW / KS;                   // tile groups
+    static constexpr int BT = G * TG;                   // row tiles per tensor and batch
+    static constexpr int NSB = ALT ? 1 : NS;            // tensors per batch
+    static constexpr uint32_t RB = (uint32_t)qkk_row_bytes_dev<TYPE>(256 * KS);
+    static constexpr uint32_t TBYTES = 16 * RB;         // one tile of 16 rows: contiguous
+    static constexpr uint32_t BBYTES = NSB * BT * TBYTES; // one batch in LDS
+    static constexpr uint32_t PART_BYTES = NSB * BT * KS * 64 * 16;
+    static constexpr uint32_t LDS_BYTES = 2 * BBYTES + 2 * PART_BYTES; // both double-buffered
+    static_assert(BBYTES % 16 == 0 && CW % KS == 0 && (!ALT || NS == 2), "geometry");
+};
+
+// The A operand of one wave: rows row_of(0..np-1) (rows >= np read as zero), K slice
+// [k0, k0+256) in the cut of `LAYOUT` (see BFrag), split into hi + lo halves.
+struct AFrag {
+    half8 hi[8], lo[8];
+};
+
+template <int LAYOUT, typename RowOf>
+__device__ __forceinline__ void load_afrag(AFrag& a, const float* __restrict__ X, uint32_t stride, uint32_t k0,
+                                           uint32_t np, RowOf row_of, int lane)
 {
-    float4v part[NT];
-#pragma unroll
-    for (int t = 0; t < NT; t++) part[t] = float4v{0.f, 0.f, 0.f, 0.f};
+    const uint32_t j = lane & 15, g = lane >> 4;
+    const float keep = j < np ? 1.f : 0.f;
+    const float* src = X + (size_t)row_of(min(j, np - 1)) * stride + k0;
+    float4 v[8][2];
 #pragma unroll
     for (int i = 0; i < 8; i++) {
-        const size_t off = ((size_t)(fi * 8 + i) * 64 + lane) * 8;
-        const half8 ah = *(const half8*)(s_hi + off), al = *(const half8*)(s_lo + off);
-#pragma unroll
-        for (int t = 0; t < NT; t++) {
-            half8 bl;
-            const half8 b = f[t].step(i, g, tab, bl);
-            part[t] = mfma16x32(ah, b, part[t]);
-            part[t] = mfma16x32(al, b, part[t]);
-            if constexpr (BFrag<TYPE>::SPLIT) part[t] = mfma16x32(ah, bl, part[t]);
-        }
-        __builtin_amdgcn_sched_barrier(0); // keep the decode of later steps from piling up in registers
+        const uint32_t k = LAYOUT == 0 ? 64 * g + 8 * i : 128 * (g >> 1) + 32 * (i >> 1) + 16 * (g & 1) + 8 * (i & 1);
+        v[i][0] = *(const float4*)(src + k);
+        v[i][1] = *(const float4*)(src + k + 4);
     }
 #pragma unroll
-    for (int t = 0; t < NT; t++) {
-        const float sc = f[t].post();
+    for (int i = 0; i < 8; i++) {
+        const float f[8] = {v[i][0].x, v[i][0].y, v[i][0].z, v[i][0].w, v[i][1].x, v[i][1].y, v[i][1].z, v[i][1].w};
 #pragma unroll
-        for (int e = 0; e < 4; e++) acc[t][e] += sc * part[t][e];
+        for (int e = 0; e < 8; e++) {
+            const float x = f[e] * keep;
+            a.hi[i][e] = (_Float16)x;
+            a.lo[i][e] = (_Float16)(x - (float)a.hi[i][e]);
+        }
     }
 }
 
-// Streams NT weight rows per lane (rowp[t] = this lane's row of tile t, at the first staged
-// weight) over `nfrag` fragments of the staged activation tile through a ring of DEPTH
-// fragment sets.  prime() issues the first DEPTH loads and needs nothing from LDS, so it is
-// called BEFORE the activation rows are staged: HBM latency overlaps the staging.  In run()
-// the loads of fragment b+DEPTH are issued as soon as fragment b has been consumed; loads
-// past the end re-read the last fragment (no branch around a load).
-template <int TYPE, int NT, int DEPTH>
-struct Stream {
-    using F = BFrag<TYPE>;
-    F f[DEPTH][NT];
-    __device__ __forceinline__ void prime(const uint8_t* const* rowp, uint32_t nfrag, int g)
-    {
+// Streams n_batches batches of BT row tiles starting at base0 / base1 (tensor 0 / 1, first row
+// of the sub-item) and calls epi(tile, lane, e, sum0, sum1) for every output: tile = row tile
+// within the sub-item, lane%16 = row within the tile, 4*(lane/16)+e = activation row, sum_s =
+// tensor s's dot product.  One barrier per batch: batch b+1 is written to the other LDS buffer
+// as soon as this wave is done with batch b (nobody reads that buffer any more), the partials
+// alternate between two buffers as well, so fast waves run ahead into the next batch.
+template <int TYPE, int KS, int NS, int TG, bool ALT, typename RowOf, typename Epi>
+__device__ __forceinline__ void coop_stream(const uint8_t* __restrict__ base0, const uint8_t* __restrict__ base1,
+                                            uint32_t n_batches, const float* __restrict__ A_src, uint32_t a_stride,
+                                            uint32_t np, RowOf row_of, uint8_t* smem, const MfmaTables& tab, int tid,
+                                            Epi epi)
+{
+    using Geo = CoopGeom<TYPE, KS, NS, TG, ALT>;
+    constexpr int BT = Geo::BT, NSB = Geo::NSB, NTL = NSB * TG; // tiles per wave and batch
+    constexpr uint32_t RB = Geo::RB, TBYTES = Geo::TBYTES, BBYTES = Geo::BBYTES, PBYTES = Geo::PART_BYTES;
+    constexpr int PIECES = BBYTES / 16, PPT = BT * TBYTES / 16, NLD = (PIECES + CT - 1) / CT;
+    constexpr int OUTS = (BT * 256 + CT - 1) / CT; // outputs per thread and batch
+    const int lane = tid & 63, wave = tid >> 6, kw = wave % KS, tg = wave / KS, j = lane & 15, g = lane >> 4;
+    const uint32_t steps = ALT ? 2 * n_batches : n_batches; // LDS batches
+
+    // piece p of a batch: 16 bytes at offset (p % PPT)*16 of tensor p / PPT; LDS keeps the same order
+    const uint8_t* src[NLD];
 #pragma unroll
-        for (int dd = 0; dd < DEPTH; dd++)
-#pragma unroll
-            for (int t = 0; t < NT; t++) f[dd][t].load(rowp[t], min((uint32_t)dd, nfrag - 1), g);
+    for (int n = 0; n < NLD; n++) {
+        const uint32_t p = min((uint32_t)(tid + CT * n), (uint32_t)PIECES - 1);
+        src[n] = ((NSB > 1 && p >= (uint32_t)PPT) ? base1 : base0) + (size_t)(p % PPT) * 16;
     }
-    __device__ __forceinline__ void run(const uint8_t* const* rowp, uint32_t nfrag, const _Float16* s_hi,
-                                        const _Float16* s_lo, int lane, int g, const MfmaTables& tab, float4v* acc)
-    {
+    const size_t alt_delta = ALT ? (size_t)(base1 - base0) : 0;
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    u32x4 ld[NLD];
+    const auto adv_of = [&](uint32_t nx) -> size_t {
+        nx = min(nx, steps - 1); // past the end: a harmless re-read
+        return ALT ? (size_t)(nx >> 1) * (BT * TBYTES) + (nx & 1u) * alt_delta : (size_t)nx * (BT * TBYTES);
+    };
+#pragma unroll
+    for (int n = 0; n < NLD; n++) ld[n] = *(const u32x4*)src[n];
+    AFrag a; // fetched and converted while the first batch is in flight
+    load_afrag<BFrag<TYPE>::LAYOUT>(a, A_src, a_stride, 256 * kw, np, row_of, lane);
+#pragma unroll
+    for (int n = 0; n < NLD; n++)
+        if (PIECES % CT == 0 || n + 1 < NLD || tid + CT * n < PIECES) *(u32x4*)(smem + (size_t)(tid + CT * n) * 16) = ld[n];
+    __syncthreads();
+    float saved[OUTS]; // ALT: tensor 0's sums wait here for tensor 1's
+#pragma unroll
+    for (int o = 0; o < OUTS; o++) saved[o] = 0.f;
+
 #pragma unroll 1
-        for (uint32_t b = 0; b < nfrag; b += DEPTH) {
+    for (uint32_t b = 0; b < steps; b++) {
+        const uint32_t buf = b & 1u;
+        {   // next batch: lands during the MFMA phase
+            const size_t adv = adv_of(b + 1);
 #pragma unroll
-            for (int dd = 0; dd < DEPTH; dd++) {
-                if (DEPTH == 1 || b + dd < nfrag) mac_multi<TYPE, NT>(f[dd], s_hi, s_lo, b + dd, lane, g, tab, acc);
+            for (int n = 0; n < NLD; n++) ld[n] = *(const u32x4*)(src[n] + adv);
+        }
+        // this wave's fragments of the batch: tiles tg*TG .. +TG of every tensor in it
+        BFrag<TYPE> f[NTL];
 #pragma unroll
-                for (int t = 0; t < NT; t++)
-                    f[dd][t].load(rowp[t], min(b + dd + DEPTH, nfrag - 1), g);
+        for (int s = 0; s < NSB; s++)
+#pragma unroll
+            for (int t = 0; t < TG; t++)
+                f[s * TG + t].load(smem + buf * BBYTES + ((size_t)(s * BT + tg * TG + t) * 16 + j) * RB, kw, g);
+        float4v acc[NTL];
+#pragma unroll
+        for (int t = 0; t < NTL; t++) acc[t] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+#pragma unroll
+            for (int t = 0; t < NTL; t++) {
+                half8 bl;
+                const half8 bh = f[t].step(i, g, tab, bl);
+                acc[t] = mfma16x32(a.hi[i], bh, acc[t]);
+                acc[t] = mfma16x32(a.lo[i], bh, acc[t]);
+                if constexpr (BFrag<TYPE>::SPLIT) acc[t] = mfma16x32(a.hi[i], bl, acc[t]);
             }
+            __builtin_amdgcn_sched_barrier(0); // keep the decode of later steps from piling up in registers
+        }
+        float* part = (float*)(smem + 2 * BBYTES + buf * PBYTES); // [NSB*BT][KS][64 lanes][4]
+#pragma unroll
+        for (int s = 0; s < NSB; s++)
+#pragma unroll
+            for (int t = 0; t < TG; t++) {
+                const float sc = f[s * TG + t].post();
+                const float4v r = acc[s * TG + t];
+                *(float4*)(part + (((size_t)(s * BT + tg * TG + t) * KS + kw) * 64 + lane) * 4) =
+                    float4{sc * r[0], sc * r[1], sc * r[2], sc * r[3]};
+            }
+#pragma unroll
+        for (int n = 0; n < NLD; n++)
+            if (PIECES % CT == 0 || n + 1 < NLD || tid + CT * n < PIECES)
+                *(u32x4*)(smem + (buf ^ 1u) * BBYTES + (size_t)(tid + CT * n) * 16) = ld[n];
+        __syncthreads(); // partials of batch b complete, batch b+1 in place
+#pragma unroll
+        for (int oo = 0; oo < OUTS; oo++) {
+            const uint32_t o = tid + CT * oo;
+            if (BT * 256 % CT != 0 && o >= (uint32_t)BT * 256) break;
+            const uint32_t bt = o >> 8, e = (o >> 6) & 3u, ln = o & 63u;
+            float sum0 = 0.f, sum1 = 0.f;
+#pragma unroll
+            for (int w = 0; w < KS; w++) {
+                sum0 += part[(((size_t)bt * KS + w) * 64 + ln) * 4 + e];
+                if (NSB > 1) sum1 += part[(((size_t)(BT + bt) * KS + w) * 64 + ln) * 4 + e];
+            }
+            if (!ALT) epi(b * BT + bt, ln, e, sum0, sum1);
+            else if (b & 1u) epi((b >> 1) * BT + bt, ln, e, saved[oo], sum0);
+            else saved[oo] = sum0;
         }
     }
-};
+    __syncthreads(); // the buffers are free for the next call
+}
 
-constexpr int GU_WAVES = 8; // waves per gate/up workgroup
-constexpr int GU_TPW = 2;   // row tiles per wave: its gate and up tile share every activation fragment
-constexpr int DN_WAVES = 8;
-constexpr int DN_TPW = 4;   // row tiles per wave in the down launch
-
-// Work items: first the shared expert's tiles of 16 consecutive tokens (they cannot be split
-// by pairs, so they start first), then the routed experts with their pair lists.  Every item
-// is cut into sub-items that take different weight-row tiles, so one expert's rows are
-// streamed by several workgroups (each stages the item's activation rows itself).
+// Work items: first the shared expert's tiles of 16 consecutive tokens (one dense expert for
+// every token: its items are the long ones, so they start first), then the routed experts with
+// their pair lists.  Every item is cut into sub-items of `nb` batches of weight rows, so one
+// expert's rows are streamed by several workgroups (each loads the activation rows itself).
 struct Item {
     bool shared;
     uint32_t expert, first, count; // routed: pairs [first, first+count) of ws.pairs; shared: tokens
@@ -296,81 +399,32 @@ __device__ __forceinline__ Item get_item(const MoeWs& ws, uint32_t index, uint32
 }
 
 // ---- gate/up + SiLU --------------------------------------------------------------------------------
-// One sub-item: GU_WAVES*GU_TPW row tiles of gate and up for up to 16 staged rows.  H = 2048*NCHUNK.
-// TYPE = format of the gate/up tensors of this item (IQ3_XXS experts, Q8_0 shared expert).
-// TPW = row tiles per wave (their gate and up rows share every activation fragment).
-template <int TYPE, int NCHUNK, int TPW, int DEPTH>
-__device__ __forceinline__ void gateup_tile(const uint8_t* __restrict__ gate, const uint8_t* __restrict__ up,
-                                            size_t row_bytes, const float* __restrict__ X, float* __restrict__ h,
-                                            const MoeDims& d, uint32_t tile0, uint32_t np, _Float16* s_hi,
-                                            _Float16* s_lo, const uint32_t* s_tok, const uint32_t* s_slot,
-                                            const MfmaTables& tab, int tid)
-{
-    constexpr int NT = 2 * TPW; // weight tiles per lane: gate q0, up q0, gate q1, up q1 ...
-    constexpr uint32_t NFRAG = 2048 / 256; // fragments per staged chunk
-    const int lane = tid & 63, j = lane & 15, g = lane >> 4;
-    const uint8_t* rowp[NT];
-#pragma unroll
-    for (int q = 0; q < TPW; q++) {
-        const size_t ro = (size_t)((tile0 + GU_WAVES * q) * 16 + j) * row_bytes;
-        rowp[2 * q] = gate + ro;
-        rowp[2 * q + 1] = up + ro;
-    }
-    float4v acc[NT];
-#pragma unroll
-    for (int t = 0; t < NT; t++) acc[t] = float4v{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 1
-    for (int ch = 0; ch < NCHUNK; ch++) {
-        Stream<TYPE, NT, DEPTH> st;
-        if (ch) {
-            __syncthreads(); // the previous chunk's fragments are consumed
-#pragma unroll
-            for (int t = 0; t < NT; t++) rowp[t] += qkk_row_bytes_dev<TYPE>(2048);
-        }
-        st.prime(rowp, NFRAG, g); // in flight while the activation rows are staged
-        stage_rows256<BFrag<TYPE>::LAYOUT, 2048, 64 * GU_WAVES>(s_hi, s_lo, X + ch * 2048, d.H, np,
-                                                               [&](uint32_t r) { return s_tok[r]; }, tid);
-        __syncthreads();
-        st.run(rowp, NFRAG, s_hi, s_lo, lane, g, tab, acc);
-    }
-    // lane holds rows (tile0 + GU_WAVES*q)*16 + j for staged rows 4g+e
-#pragma unroll
-    for (int q = 0; q < TPW; q++) {
-        const uint32_t row = (tile0 + GU_WAVES * q) * 16 + j;
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const uint32_t r = 4 * g + e;
-            if (r < np) {
-                const float gg = acc[2 * q][e], uu = acc[2 * q + 1][e];
-                h[((size_t)s_tok[r] * (d.k + 1) + s_slot[r]) * d.F + row] = (gg / (1.f + expf(-gg))) * uu;
-            }
-        }
-    }
-}
+// n_embd = 2048: the eight waves take one 256-weight fragment each.  Routed experts: batches of
+// one row tile of gate and of up (IQ3_XXS); shared expert (Q8_0): one row tile, gate and up in turns.
+constexpr int GU_TG_R = 1, GU_TG_S = 1;
+using GuGeoR = CoopGeom<QKK_IQ3_XXS, 8, 2, GU_TG_R>;
+using GuGeoS = CoopGeom<QKK_Q8_0, 8, 2, GU_TG_S, true>;
+constexpr uint32_t GU_LDS = GuGeoR::LDS_BYTES > GuGeoS::LDS_BYTES ? GuGeoR::LDS_BYTES : GuGeoS::LDS_BYTES;
 
-template <int NCHUNK>
-__global__ __launch_bounds__(64 * GU_WAVES) void moe_gateup_mfma_kernel(const uint8_t* __restrict__ gate_exps,
-                                                                        const uint8_t* __restrict__ up_exps,
-                                                                        const uint8_t* __restrict__ gate_shexp,
-                                                                        const uint8_t* __restrict__ up_shexp,
-                                                                        const float* __restrict__ X, MoeWs ws,
-                                                                        MoeDims d, uint32_t N)
+__global__ __launch_bounds__(CT) void moe_gateup_mfma_kernel(const uint8_t* __restrict__ gate_exps,
+                                                             const uint8_t* __restrict__ up_exps,
+                                                             const uint8_t* __restrict__ gate_shexp,
+                                                             const uint8_t* __restrict__ up_shexp,
+                                                             const float* __restrict__ X, MoeWs ws, MoeDims d,
+                                                             uint32_t N, uint32_t nb_r, uint32_t nb_s)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    _Float16* s_hi = (_Float16*)smem;
-    _Float16* s_lo = s_hi + 16 * 2048;
     __shared__ MfmaTables tab;
     __shared__ uint32_t s_tok[16], s_slot[16];
-    const int tid = threadIdx.x, wave = tid >> 6;
+    const int tid = threadIdx.x;
     const uint32_t F = d.F, H = d.H;
-    fill_mfma_tables(tab, tid, 64 * GU_WAVES);
+    fill_mfma_tables(tab, tid, CT);
     const uint32_t n_active = *ws.n_active;
-    const uint32_t subs_sh = F / (16 * GU_WAVES), subs = F / (16 * GU_WAVES * GU_TPW);
+    const uint32_t subs_sh = F / (16 * GuGeoS::BT * nb_s), subs = F / (16 * GuGeoR::BT * nb_r);
     const uint32_t n_items = item_count(n_active, N, subs_sh, subs);
 
     for (uint32_t w = blockIdx.x; w < n_items; w += gridDim.x) {
         const Item it = get_item(ws, w, subs_sh, subs, N);
-        const uint32_t tile0 = it.sub * GU_WAVES * (it.shared ? 1 : GU_TPW) + wave; // this wave: tile0 + GU_WAVES*q
         for (uint32_t t0 = 0; t0 < it.count; t0 += 16) {
             const uint32_t np = it.shared ? it.count : min(16u, it.count - t0);
             __syncthreads(); // previous tile fully consumed
@@ -384,80 +438,62 @@ __global__ __launch_bounds__(64 * GU_WAVES) void moe_gateup_mfma_kernel(const ui
                 s_slot[tid] = slot;
             }
             __syncthreads();
+            const auto row_of = [&](uint32_t r) { return s_tok[r]; };
             if (it.shared) {
-                gateup_tile<QKK_Q8_0, NCHUNK, 1, 3>(gate_shexp, up_shexp, (size_t)H / 32 * Q8_0_BYTES, X, ws.h, d, tile0, np,
-                                                 s_hi, s_lo, s_tok, s_slot, tab, tid);
+                const uint32_t row0 = it.sub * nb_s * GuGeoS::BT * 16;
+                coop_stream<QKK_Q8_0, 8, 2, GU_TG_S, true>(gate_shexp + (size_t)row0 * GuGeoS::RB, up_shexp + (size_t)row0 * GuGeoS::RB, nb_s, X, H, np, row_of, smem, tab, tid,
+                    [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1) {
+                        const uint32_t r = 4 * (ln >> 4) + e;
+                        if (r < np)
+                            ws.h[((size_t)s_tok[r] * (d.k + 1) + s_slot[r]) * F + row0 + tile * 16 + (ln & 15u)] =
+                                (sum0 / (1.f + expf(-sum0))) * sum1;
+                    });
                 break;
             }
-            const size_t rb = (size_t)H / 256 * IQ3_XXS_BYTES, eo = (size_t)it.expert * F * rb;
-            gateup_tile<QKK_IQ3_XXS, NCHUNK, GU_TPW, 3>(gate_exps + eo, up_exps + eo, rb, X, ws.h, d, tile0, np, s_hi, s_lo,
-                                                s_tok, s_slot, tab, tid);
+            const uint32_t row0 = it.sub * nb_r * GuGeoR::BT * 16;
+            const size_t eo = ((size_t)it.expert * F + row0) * GuGeoR::RB;
+            coop_stream<QKK_IQ3_XXS, 8, 2, GU_TG_R, false>(gate_exps + eo, up_exps + eo, nb_r, X, H, np, row_of, smem, tab, tid,
+                [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1) {
+                    const uint32_t r = 4 * (ln >> 4) + e;
+                    if (r < np)
+                        ws.h[((size_t)s_tok[r] * (d.k + 1) + s_slot[r]) * F + row0 + tile * 16 + (ln & 15u)] =
+                            (sum0 / (1.f + expf(-sum0))) * sum1;
+                });
         }
     }
 }
 
 // ---- down: per-pair contributions -----------------------------------------------------------------
 // contrib[(token*(k+1) + slot)*H + o] = weight * (D[o] . h[token][slot]); slot k = shared expert.
-// A sub-item is DN_WAVES*DN_TPW row tiles of 16.  FB = F/256.
-template <int TYPE, int FB, int NT, int DEPTH>
-__device__ __forceinline__ void down_tile(const uint8_t* __restrict__ W, const float* __restrict__ h,
-                                          float* __restrict__ contrib, const MoeDims& d, uint32_t tile0, uint32_t np,
-                                          _Float16* s_hi, _Float16* s_lo, const uint32_t* s_tok, const uint32_t* s_slot,
-                                          const float* s_wt, const MfmaTables& tab, int tid)
-{
-    constexpr uint32_t NFRAG = FB;
-    const size_t RB = qkk_row_bytes_dev<TYPE>(256 * FB);
-    const int lane = tid & 63, j = lane & 15, g = lane >> 4;
-    const auto row_of = [&](uint32_t r) { return s_tok[r] * (d.k + 1) + s_slot[r]; };
-#pragma unroll 1
-    for (int q0 = 0; q0 < DN_TPW; q0 += NT) {
-        const uint8_t* rowp[NT];
-#pragma unroll
-        for (int q = 0; q < NT; q++) rowp[q] = W + (size_t)((tile0 + DN_WAVES * (q0 + q)) * 16 + j) * RB;
-        Stream<TYPE, NT, DEPTH> st;
-        st.prime(rowp, NFRAG, g);
-        if (q0 == 0) {
-            stage_rows256<BFrag<TYPE>::LAYOUT, 256 * FB, 64 * DN_WAVES>(s_hi, s_lo, h, d.F, np, row_of, tid);
-            __syncthreads();
-        }
-        float4v acc[NT];
-#pragma unroll
-        for (int q = 0; q < NT; q++) acc[q] = float4v{0.f, 0.f, 0.f, 0.f};
-        st.run(rowp, NFRAG, s_hi, s_lo, lane, g, tab, acc);
-#pragma unroll
-        for (int q = 0; q < NT; q++) {
-            const uint32_t row = (tile0 + DN_WAVES * (q0 + q)) * 16 + j;
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const uint32_t r = 4 * g + e;
-                if (r < np) contrib[((size_t)s_tok[r] * (d.k + 1) + s_slot[r]) * d.H + row] = s_wt[r] * acc[q][e];
-            }
-        }
-    }
-}
+// K = F = 256*FB: FB waves split K, 8/FB tile groups split the batch's tiles.
+template <int TYPE_DN, int FB>
+struct DnGeo {
+    static constexpr int TG_R = TYPE_DN == QKK_Q6_K ? 1 : 2, TG_S = 1;
+    using R = CoopGeom<TYPE_DN, FB, 1, TG_R>;
+    using S = CoopGeom<QKK_Q8_0, FB, 1, TG_S>;
+    static constexpr uint32_t LDS = R::LDS_BYTES > S::LDS_BYTES ? R::LDS_BYTES : S::LDS_BYTES;
+};
 
 template <int TYPE_DN, int FB>
-__global__ __launch_bounds__(64 * DN_WAVES) void moe_down_mfma_kernel(const uint8_t* __restrict__ down_exps,
-                                                                      const uint8_t* __restrict__ down_shexp,
-                                                                      MoeWs ws, const qkk_sel* __restrict__ sel,
-                                                                      MoeDims d, uint32_t N)
+__global__ __launch_bounds__(CT) void moe_down_mfma_kernel(const uint8_t* __restrict__ down_exps,
+                                                           const uint8_t* __restrict__ down_shexp, MoeWs ws,
+                                                           const qkk_sel* __restrict__ sel, MoeDims d, uint32_t N,
+                                                           uint32_t nb_r, uint32_t nb_s)
 {
+    using Geo = DnGeo<TYPE_DN, FB>;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    _Float16* s_hi = (_Float16*)smem;
-    _Float16* s_lo = s_hi + 16 * 256 * FB;
     __shared__ MfmaTables tab;
     __shared__ uint32_t s_tok[16], s_slot[16];
     __shared__ float s_wt[16];
-    const int tid = threadIdx.x, wave = tid >> 6;
-    const uint32_t H = d.H;
-    fill_mfma_tables(tab, tid, 64 * DN_WAVES);
+    const int tid = threadIdx.x;
+    const uint32_t F = d.F, H = d.H;
+    fill_mfma_tables(tab, tid, CT);
     const uint32_t n_active = *ws.n_active;
-    const uint32_t subs = H / (16 * DN_WAVES * DN_TPW);
-    const uint32_t n_items = item_count(n_active, N, subs, subs);
+    const uint32_t subs_sh = H / (16 * Geo::S::BT * nb_s), subs = H / (16 * Geo::R::BT * nb_r);
+    const uint32_t n_items = item_count(n_active, N, subs_sh, subs);
 
     for (uint32_t w = blockIdx.x; w < n_items; w += gridDim.x) {
-        const Item it = get_item(ws, w, subs, subs, N);
-        const uint32_t tile0 = it.sub * DN_WAVES * DN_TPW + wave; // this wave: tile0 + DN_WAVES*q
+        const Item it = get_item(ws, w, subs_sh, subs, N);
         for (uint32_t t0 = 0; t0 < it.count; t0 += 16) {
             const uint32_t np = it.shared ? it.count : min(16u, it.count - t0);
             __syncthreads();
@@ -474,14 +510,26 @@ __global__ __launch_bounds__(64 * DN_WAVES) void moe_down_mfma_kernel(const uint
                 s_tok[tid] = tok; s_slot[tid] = slot; s_wt[tid] = wt;
             }
             __syncthreads();
+            const auto row_of = [&](uint32_t r) { return s_tok[r] * (d.k + 1) + s_slot[r]; };
             if (it.shared) {
-                down_tile<QKK_Q8_0, FB, 2, (FB < 2 ? 1 : 2)>(down_shexp, ws.h, ws.contrib, d, tile0, np, s_hi, s_lo, s_tok,
-                                                            s_slot, s_wt, tab, tid);
+                const uint32_t row0 = it.sub * nb_s * Geo::S::BT * 16;
+                coop_stream<QKK_Q8_0, FB, 1, Geo::TG_S, false>(down_shexp + (size_t)row0 * Geo::S::RB, nullptr, nb_s, ws.h, F, np, row_of, smem, tab, tid,
+                    [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1) {
+                        const uint32_t r = 4 * (ln >> 4) + e;
+                        if (r < np)
+                            ws.contrib[((size_t)s_tok[r] * (d.k + 1) + s_slot[r]) * H + row0 + tile * 16 + (ln & 15u)] =
+                                s_wt[r] * sum0;
+                    });
                 break;
             }
-            const size_t RB = qkk_row_bytes_dev<TYPE_DN>(256 * FB);
-            down_tile<TYPE_DN, FB, 2, (FB < 2 ? 1 : 2)>(down_exps + (size_t)it.expert * H * RB, ws.h, ws.contrib, d,
-                                                            tile0, np, s_hi, s_lo, s_tok, s_slot, s_wt, tab, tid);
+            const uint32_t row0 = it.sub * nb_r * Geo::R::BT * 16;
+            coop_stream<TYPE_DN, FB, 1, Geo::TG_R, false>(down_exps + ((size_t)it.expert * H + row0) * Geo::R::RB, nullptr, nb_r, ws.h, F, np, row_of, smem, tab, tid,
+                [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1) {
+                    const uint32_t r = 4 * (ln >> 4) + e;
+                    if (r < np)
+                        ws.contrib[((size_t)s_tok[r] * (d.k + 1) + s_slot[r]) * H + row0 + tile * 16 + (ln & 15u)] =
+                            s_wt[r] * sum0;
+                });
         }
     }
 }
@@ -502,61 +550,59 @@ __global__ __launch_bounds__(256) void moe_fold_kernel(MoeWs ws, float* __restri
 }
 
 // ---- host -----------------------------------------------------------------------------------------------
-static void set_lds_attr(const void* fn)
+static void set_lds_attr(const void* fn, uint32_t bytes)
 {
-    (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 140 * 1024);
+    (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
 }
 
-static void launch_gateup(const qkk_moe_layer* L, const float* X, const MoeWs& ws, const MoeDims& d, uint32_t N,
-                          uint32_t blocks, hipStream_t st)
+// batches per sub-item: the largest power of two <= total that still gives every CU about two items
+static uint32_t pick_nb(uint32_t total_batches, uint32_t experts)
 {
-    const size_t lds = (size_t)2 * 16 * 2048 * sizeof(_Float16);
-    const uint8_t *ge = (const uint8_t*)L->gate_exps, *ue = (const uint8_t*)L->up_exps,
-                  *gs = (const uint8_t*)L->gate_shexp, *us = (const uint8_t*)L->up_shexp;
-    if (d.H == 2048) {
-        static bool once = (set_lds_attr((const void*)moe_gateup_mfma_kernel<1>), true);
-        (void)once;
-        hipLaunchKernelGGL(moe_gateup_mfma_kernel<1>, dim3(blocks), dim3(64 * GU_WAVES), lds, st, ge, ue, gs, us, X, ws, d, N);
-    } else {
-        static bool once = (set_lds_attr((const void*)moe_gateup_mfma_kernel<2>), true);
-        (void)once;
-        hipLaunchKernelGGL(moe_gateup_mfma_kernel<2>, dim3(blocks), dim3(64 * GU_WAVES), lds, st, ge, ue, gs, us, X, ws, d, N);
-    }
+    uint32_t nb = total_batches;
+    while (nb > 1 && (uint64_t)experts * (total_batches / nb) < 2ull * persistent_blocks() / 4) nb /= 2;
+    return nb;
 }
 
 template <int TYPE, int FB>
 static void launch_down(const qkk_moe_layer* L, const MoeWs& ws, const qkk_sel* sel, const MoeDims& d, uint32_t N,
-                        uint32_t blocks, hipStream_t st)
+                        uint32_t experts, hipStream_t st)
 {
-    const size_t lds = (size_t)2 * 16 * 256 * FB * sizeof(_Float16);
-    static bool once = (set_lds_attr((const void*)moe_down_mfma_kernel<TYPE, FB>), true);
+    using Geo = DnGeo<TYPE, FB>;
+    static bool once = (set_lds_attr((const void*)moe_down_mfma_kernel<TYPE, FB>, Geo::LDS), true);
     (void)once;
-    hipLaunchKernelGGL((moe_down_mfma_kernel<TYPE, FB>), dim3(blocks), dim3(64 * DN_WAVES), lds, st,
-                       (const uint8_t*)L->down_exps, (const uint8_t*)L->down_shexp, ws, sel, d, N);
+    const uint32_t tot_r = d.H / (16 * Geo::R::BT), tot_s = d.H / (16 * Geo::S::BT);
+    const uint32_t nb_r = pick_nb(tot_r, experts), nb_s = std::min(tot_s, std::max(1u, nb_r * Geo::R::BT / Geo::S::BT / 2));
+    const uint32_t items = experts * (tot_r / nb_r) + (N + 15) / 16 * (tot_s / nb_s);
+    const uint32_t blocks = std::min(items, persistent_blocks() / 4);
+    hipLaunchKernelGGL((moe_down_mfma_kernel<TYPE, FB>), dim3(blocks), dim3(CT), Geo::LDS, st,
+                       (const uint8_t*)L->down_exps, (const uint8_t*)L->down_shexp, ws, sel, d, N, nb_r, nb_s);
 }
 
 // Gate/up, down and fold for N >= 2 rows; the router record and the pair lists are in place.
 void moe_mfma_launch(const qkk_moe_layer* L, const float* X, float* Y, const qkk_sel* sel, const MoeWs& ws,
                      const MoeDims& d, uint32_t N, uint32_t stages, hipStream_t st)
 {
-    const uint32_t max_items = (uint32_t)std::min<uint64_t>(d.E, (uint64_t)N * d.k) + (N + 15) / 16;
-    // down: 8-wave workgroups, several share a CU (the staged tile is 16*F*4 bytes)
-    const uint32_t blocks = std::min(max_items * (d.H / (16 * DN_WAVES * DN_TPW)), persistent_blocks() / 2);
+    const uint32_t experts = (uint32_t)std::min<uint64_t>(d.E, (uint64_t)N * d.k); // upper bound of the active ones
     if (stages & QKK_STAGE_GATEUP) {
-        const uint32_t gu_items = (uint32_t)std::min<uint64_t>(d.E, (uint64_t)N * d.k) * (d.F / (16 * GU_WAVES * GU_TPW)) +
-                                  (N + 15) / 16 * (d.F / (16 * GU_WAVES));
-        const uint32_t gu_blocks = std::min(gu_items, persistent_blocks() / 4);
-        launch_gateup(L, X, ws, d, N, gu_blocks, st);
+        static bool once = (set_lds_attr((const void*)moe_gateup_mfma_kernel, GU_LDS), true);
+        (void)once;
+        const uint32_t tot_r = d.F / (16 * GuGeoR::BT), tot_s = d.F / (16 * GuGeoS::BT);
+        const uint32_t nb_r = pick_nb(tot_r, experts), nb_s = std::min(tot_s, std::max(1u, nb_r * GuGeoR::BT / GuGeoS::BT / 2));
+        const uint32_t items = experts * (tot_r / nb_r) + (N + 15) / 16 * (tot_s / nb_s);
+        const uint32_t blocks = std::min(items, persistent_blocks() / 4);
+        hipLaunchKernelGGL(moe_gateup_mfma_kernel, dim3(blocks), dim3(CT), GU_LDS, st, (const uint8_t*)L->gate_exps,
+                           (const uint8_t*)L->up_exps, (const uint8_t*)L->gate_shexp, (const uint8_t*)L->up_shexp, X, ws, d,
+                           N, nb_r, nb_s);
     }
     if (stages & QKK_STAGE_DOWN) {
         if (L->down_type == QKK_IQ4_XS) {
-            if (d.F == 256) launch_down<QKK_IQ4_XS, 1>(L, ws, sel, d, N, blocks, st);
-            else if (d.F == 512) launch_down<QKK_IQ4_XS, 2>(L, ws, sel, d, N, blocks, st);
-            else launch_down<QKK_IQ4_XS, 4>(L, ws, sel, d, N, blocks, st);
+            if (d.F == 256) launch_down<QKK_IQ4_XS, 1>(L, ws, sel, d, N, experts, st);
+            else if (d.F == 512) launch_down<QKK_IQ4_XS, 2>(L, ws, sel, d, N, experts, st);
+            else launch_down<QKK_IQ4_XS, 4>(L, ws, sel, d, N, experts, st);
         } else {
-            if (d.F == 256) launch_down<QKK_Q6_K, 1>(L, ws, sel, d, N, blocks, st);
-            else if (d.F == 512) launch_down<QKK_Q6_K, 2>(L, ws, sel, d, N, blocks, st);
-            else launch_down<QKK_Q6_K, 4>(L, ws, sel, d, N, blocks, st);
+            if (d.F == 256) launch_down<QKK_Q6_K, 1>(L, ws, sel, d, N, experts, st);
+            else if (d.F == 512) launch_down<QKK_Q6_K, 2>(L, ws, sel, d, N, experts, st);
+            else launch_down<QKK_Q6_K, 4>(L, ws, sel, d, N, experts, st);
         }
         const uint32_t fb = (uint32_t)std::min<uint64_t>(((uint64_t)N * d.H / 4 + 255) / 256, persistent_blocks());
         hipLaunchKernelGGL(moe_fold_kernel, dim3(fb), dim3(256), 0, st, ws, Y, d, N);
