@@ -6,24 +6,24 @@
 // share it (the expert-major order of reference shaders/moe_gateup_iq3_grouped.comp:30-114 and
 // moe_down_iq4_grouped.comp:24-75, driven by the pair lists of moe_group_pairs.comp).
 // Launches of a step: route (router logits and -- in the workgroup that finishes last --
-// selection + grouping; a launch of its own above 64 tokens), gate/up, down, fold.
+// selection + grouping; above 32 tokens a launch of its own that selects one token per wave
+// and groups in its last workgroup), gate/up, down, fold.
 #include "qk_moe_common.h"
 
 #include <algorithm>
 
 namespace qk {
 
-constexpr uint32_t SELECT_INLINE_MAX = 64; // up to this many tokens the route launch also selects
+constexpr uint32_t SELECT_INLINE_MAX = 32; // up to this many tokens the route launch also selects
 
-// ---- selection + grouping by one workgroup of NW waves ------------------------------------
-template <int NW>
-__device__ static void select_and_group(const MoeWs& ws, qkk_sel* __restrict__ sel, MoeDims d, uint32_t N,
-                                        float* s_log, uint32_t* s_cnt, uint32_t* s_cur)
+// ---- selection: one wave takes the tokens first, first+stride, ... ----------------------------
+// (logits written by other workgroups: the caller's acquire fence, or a kernel boundary, precedes)
+__device__ static void select_tokens(const MoeWs& ws, qkk_sel* __restrict__ sel, MoeDims d, uint32_t N,
+                                     uint32_t first, uint32_t stride, float* my_log, bool publish_ids)
 {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    float* my_log = s_log + (size_t)wave * (QKK_MAX_EXPERTS + 8);
-    for (uint32_t t = wave; t < N; t += NW) {
-        // the caller's acquire fence precedes this: plain loads, all issued before the first use
+    const int lane = threadIdx.x & 63;
+    for (uint32_t t = first; t < N; t += stride) {
+        // plain loads, all issued before the first use
         const float* gl = ws.logits + (size_t)t * lstride(d.E);
         float lv[QKK_MAX_EXPERTS / 64 + 1];
 #pragma unroll
@@ -36,8 +36,17 @@ __device__ static void select_and_group(const MoeWs& ws, qkk_sel* __restrict__ s
         __builtin_amdgcn_wave_barrier();
         select_wave(my_log, d.E, d.k, &sel[t]);
         if (lane == 0) sel[t].w_shared = 1.f / (1.f + expf(-my_log[d.E]));
+        // the grouping workgroup of the same launch reads the ids: write them through
+        if (publish_ids && (uint32_t)lane < d.k) publish(&sel[t].ids[lane], sel[t].ids[lane]);
         __builtin_amdgcn_wave_barrier();
     }
+}
+
+// ---- grouping of the N*k (token, pick) pairs by expert, by one workgroup of NW waves ----------
+template <int NW>
+__device__ static void group_pairs_wg(const MoeWs& ws, qkk_sel* __restrict__ sel, MoeDims d, uint32_t N,
+                                      uint32_t* s_cnt, uint32_t* s_cur)
+{
     for (uint32_t e = threadIdx.x; e <= QKK_MAX_EXPERTS; e += NW * 64) s_cnt[e] = 0;
     __threadfence_block();
     __syncthreads();
@@ -149,18 +158,29 @@ __global__ __launch_bounds__(512) void moe_route_multi_kernel(const float* __res
     if (threadIdx.x == 0) s_last = arrive_last(&ws.counter[0], gridDim.x) ? 1u : 0u;
     __syncthreads();
     if (s_last) {
-        select_and_group<NW>(ws, sel, d, N, s_log, s_cnt, s_cur);
+        select_tokens(ws, sel, d, N, wave, NW, s_log + (size_t)wave * (QKK_MAX_EXPERTS + 8), false);
+        group_pairs_wg<NW>(ws, sel, d, N, s_cnt, s_cur);
         if (threadIdx.x == 0) ws.counter[0] = 0u;
     }
 }
 
-// Selection + grouping as a launch of its own (many tokens).
+// Selection + grouping as a launch of its own (many tokens): one token per wave, sixteen per
+// workgroup; the workgroup that finishes last groups the pairs.
 __global__ __launch_bounds__(1024) void moe_select_group_kernel(MoeWs ws, qkk_sel* __restrict__ sel, MoeDims d,
                                                                 uint32_t N)
 {
     __shared__ float s_log[16 * (QKK_MAX_EXPERTS + 8)];
     __shared__ uint32_t s_cnt[QKK_MAX_EXPERTS + 1], s_cur[QKK_MAX_EXPERTS + 1];
-    select_and_group<16>(ws, sel, d, N, s_log, s_cnt, s_cur);
+    __shared__ uint32_t s_last;
+    const int wave = threadIdx.x >> 6;
+    select_tokens(ws, sel, d, N, blockIdx.x * 16 + wave, gridDim.x * 16, s_log + (size_t)wave * (QKK_MAX_EXPERTS + 8), true);
+    __syncthreads();
+    if (threadIdx.x == 0) s_last = arrive_last(&ws.counter[0], gridDim.x) ? 1u : 0u;
+    __syncthreads();
+    if (s_last) {
+        group_pairs_wg<16>(ws, sel, d, N, s_cnt, s_cur);
+        if (threadIdx.x == 0) ws.counter[0] = 0u;
+    }
 }
 
 void moe_mfma_launch(const qkk_moe_layer* L, const float* X, float* Y, const qkk_sel* sel, const MoeWs& ws,
@@ -179,7 +199,7 @@ int moe_grouped_launch(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel
         const uint32_t tasks = (d.E + 1) * ((N + 3) / 4);
         hipLaunchKernelGGL(moe_route_multi_kernel<8>, dim3((tasks + 7) / 8), dim3(512), 0, st, L->gate_inp,
                            L->gate_inp_shexp, X, ws, sel, d, N, inline_sel);
-        if (!inline_sel) hipLaunchKernelGGL(moe_select_group_kernel, dim3(1), dim3(1024), 0, st, ws, sel, d, N);
+        if (!inline_sel) hipLaunchKernelGGL(moe_select_group_kernel, dim3((N + 15) / 16), dim3(1024), 0, st, ws, sel, d, N);
     }
     moe_mfma_launch(L, X, Y, sel, ws, d, N, stages, st);
     return check_launch("moe grouped path");
