@@ -264,6 +264,8 @@ def main():
         m = moe_workload(qk, 1, qk.IQ4_XS, a.ring, steps, a.warmup)
     elif a.workload == "moe_decode_bs16":
         m = moe_workload(qk, 16, qk.Q6_K, min(a.ring, 8), steps, a.warmup)
+    elif a.workload == "moe_prefill_128":
+        m = moe_workload(qk, 128, qk.IQ4_XS, min(a.ring, 4), min(steps, 400), min(a.warmup, 40))
     else:
         sys.exit(f"unknown workload {a.workload}")
     log(f"[bench] {a.workload}: {m['ms_wall'] * 1e3:.2f} us/step wall, {m['ms_event'] * 1e3:.2f} us/step events, "
@@ -274,7 +276,7 @@ def main():
     # stage alone on the same ring (profiles/ holds the rocprofv3 figure for the same kernel)
     gu_ms = m["stage_ms"]["gateup"]
     ach = m["gateup_bytes"] / (gu_ms * 1e-3) / 1e9
-    kname = "moe_gateup_kernel" if a.workload == "moe_decode_bs1" else "moe_gateup_grouped_kernel"
+    kname = "moe_gateup_kernel" if a.workload == "moe_decode_bs1" else "moe_gateup_mfma_kernel"
     roof = dict(bound="hbm", kernel=kname + " (select + routed IQ3_XXS gate/up + SiLU)", achieved=ach,
                 peak=HBM_PEAK_GBPS, unit="GB/s", frac=ach / HBM_PEAK_GBPS, traffic=TRAFFIC.get(kname),
                 bytes_per_launch=m["gateup_bytes"], us_per_launch=gu_ms * 1e3)
@@ -282,8 +284,9 @@ def main():
                warmup=a.warmup, ms_per_step=m["ms_wall"], higher_is_better=True, scaling="weak", vs_baseline=None,
                dtype="f32", data="synthetic",
                config=dict(workload=a.workload, n_embd=2048, n_ff=512, n_expert=256, n_used=8,
-                           gate_up="IQ3_XXS", down="IQ4_XS" if a.workload.endswith("bs1") else "Q6_K",
-                           shared="Q8_0", slots=1 if a.workload.endswith("bs1") else 16, ring_layers=m["ring"],
+                           gate_up="IQ3_XXS", down="Q6_K" if a.workload.endswith("bs16") else "IQ4_XS",
+                           shared="Q8_0", slots={"moe_decode_bs1": 1, "moe_decode_bs16": 16}.get(a.workload, 128),
+                           ring_layers=m["ring"],
                            ring_bytes=m["ring_bytes"], timing="hipGraph replay of the ring"),
                us_per_step=m["ms_wall"] * 1e3, us_per_step_events=m["ms_event"] * 1e3,
                bytes_per_step=m["bytes_step"], frac_of_hbm_peak=gbps / HBM_PEAK_GBPS,

@@ -5,9 +5,9 @@
 // writes one candidate, and the block that finishes last folds all candidates into the
 // token id.  Ties go to the lower id; a logit must beat -3.4e38 to be chosen
 // (reference shaders/argmax1.comp:25-33, argmax2.comp:20-28).
+#include "qk_coop.h"
 #include "qk_device.h"
 #include "qk_host.h"
-#include "qk_mfma.h"
 
 #include <algorithm>
 
@@ -182,120 +182,61 @@ __device__ __forceinline__ void dpp_better(float& v, uint32_t& i)
 #undef QK_STEP
 }
 
-struct Q6Frag { // one lane's share of a Q6_K block in the B-operand cut
-    uint32_t ql[2][2][2], qh[2][2];
-    uint4 sc;
-    uint16_t d;
-    __device__ __forceinline__ void load(const uint8_t* p, int g)
-    {
-#pragma unroll
-        for (int n = 0; n < 2; n++)
-#pragma unroll
-            for (int hf = 0; hf < 2; hf++) {
-#pragma unroll
-                for (int cb = 0; cb < 2; cb++) ql[n][cb][hf] = ldg<uint32_t>(p + 64 * n + 32 * cb + 16 * hf + 4 * g);
-                qh[n][hf] = ldg<uint32_t>(p + Q6_K_QH + 32 * n + 16 * hf + 4 * g);
-            }
-        sc = ldg<uint4>(p + Q6_K_SC);
-        d = ldg<uint16_t>(p + Q6_K_D);
-    }
-    // weights of scale group kk (0..15) as four exact halves (q - 32), and d*scale
-    __device__ __forceinline__ half4 group(int kk, float& scale) const
-    {
-        const int n = kk >> 3, c = (kk >> 1) & 3, hf = kk & 1;
-        const uint32_t l4 = ql[n][c & 1][hf];
-        const uint32_t nib = (c >= 2 ? (l4 >> 4) : l4) & 0x0F0F0F0Fu;
-        const uint32_t q4 = nib | (((qh[n][hf] >> (2 * c)) << 4) & 0x30303030u);
-        const uint32_t sw = kk < 4 ? sc.x : kk < 8 ? sc.y : kk < 12 ? sc.z : sc.w;
-        scale = h2f(d) * (float)(int8_t)(sw >> (8 * (kk & 3)));
-        return bytes_to_half4(q4, 32.f);
-    }
-};
+// ---- batch 2..16, K = 2048: the cooperative matrix-core stream (qk_coop.h) ------------------------
+// The head is one dense "expert" of V rows applied to `batch` activation rows: every workgroup
+// streams a contiguous range of row tiles, two per batch, and each thread keeps the best
+// (logit, id) of the outputs it reduces (its rows ascend, so `>` keeps the lowest id).
+constexpr int HEAD_TG = 2;
+using HeadGeo = CoopGeom<QKK_Q6_K, 8, 1, HEAD_TG>;
 
-template <int KBLOCKS> // K = 256*KBLOCKS
-__global__ __launch_bounds__(1024) void head_q6k_mfma_kernel(const uint8_t* __restrict__ W,
-                                                             const float* __restrict__ X,
-                                                             float* __restrict__ logits_out,
-                                                             uint32_t* __restrict__ tok, HeadWs ws, uint32_t V,
-                                                             uint32_t batch)
+__global__ __launch_bounds__(CT) void head_q6k_coop_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X,
+                                                           float* __restrict__ logits_out, uint32_t* __restrict__ tok,
+                                                           HeadWs ws, uint32_t V, uint32_t batch)
 {
-    constexpr uint32_t K = 256 * KBLOCKS, ROW = Q6_K_BYTES * KBLOCKS;
+    constexpr uint32_t K = 2048, ROW = HeadGeo::RB, BT = HeadGeo::BT;
+    static_assert(BT * 256 <= CT, "one output per thread and batch");
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    _Float16* s_hi = (_Float16*)smem;
-    _Float16* s_lo = s_hi + 16 * K;
-    __shared__ float s_v[16][16];
-    __shared__ uint32_t s_i[16][16];
+    __shared__ MfmaTables tab;
     __shared__ uint32_t s_last;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int j = lane & 15, g = lane >> 4;
+    fill_mfma_tables(tab, tid, CT);
 
-    stage_tokens<16>(s_hi, s_lo, X, K, K, batch, [](uint32_t r) { return r; }, tid, 1024);
+    // batches [b0, b1) of the tensor's `total`, an even split (b1 <= total for every workgroup)
+    const uint32_t total = (V + 16 * BT - 1) / (16 * BT);
+    const uint32_t b0 = (uint32_t)((uint64_t)blockIdx.x * total / gridDim.x);
+    const uint32_t b1 = (uint32_t)((uint64_t)(blockIdx.x + 1) * total / gridDim.x);
+    const uint32_t row0 = b0 * BT * 16;
+    const uint32_t nb = row0 < V ? b1 - b0 : 0u;
+    float bv = ARG_FLOOR;
+    uint32_t bi = 0xFFFFFFFFu;
     __syncthreads();
-
-    float bv[4];
-    uint32_t bi[4];
-#pragma unroll
-    for (int e = 0; e < 4; e++) { bv[e] = ARG_FLOOR; bi[e] = 0xFFFFFFFFu; }
-
-    // Tiles of 16 rows are dealt round-robin to the waves; within a tile the blocks are walked
-    // with the next block's loads in flight during the MFMAs of the current one.
-    const uint32_t tiles = (V + 15) / 16;
-    const uint32_t tstride = gridDim.x * 16;
-    uint32_t mt = blockIdx.x * 16 + wave;
-    Q6Frag f[2];
-    auto fetch = [&](int set, uint32_t tile, int blk) {
-        f[set].load(W + (size_t)min(tile * 16 + j, V - 1) * ROW + (size_t)blk * Q6_K_BYTES, g);
-    };
-    auto consume = [&](int set, int blk, float4v& acc) {
-#pragma unroll
-        for (int kk = 0; kk < 16; kk++) {
-            float sc;
-            const half4 b = f[set].group(kk, sc);
-            const uint32_t frag = (uint32_t)blk * 16 + kk;
-            const half4 ah = *(const half4*)(s_hi + ((size_t)frag * 64 + lane) * 4);
-            const half4 al = *(const half4*)(s_lo + ((size_t)frag * 64 + lane) * 4);
-            float4v part = mfma16x16(ah, b, float4v{0.f, 0.f, 0.f, 0.f});
-            part = mfma16x16(al, b, part);
-#pragma unroll
-            for (int e = 0; e < 4; e++) acc[e] += sc * part[e];
-        }
-    };
-    fetch(0, mt, 0);
-    for (; mt < tiles; mt += tstride) {
-        float4v acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 1
-        for (int blk = 0; blk < KBLOCKS; blk += 2) {
-            fetch(1, mt, blk + 1);
-            consume(0, blk, acc);
-            // block after next: of this tile, or the first block of the wave's next tile
-            const bool wrap = blk + 2 >= KBLOCKS;
-            fetch(0, wrap ? mt + tstride : mt, wrap ? 0 : blk + 2);
-            consume(1, blk + 1, acc);
-        }
-        const uint32_t row = mt * 16 + j;
-        if (row < V) {
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const uint32_t t = 4 * g + e;
-                if (t < batch) {
-                    if (logits_out) logits_out[(size_t)t * V + row] = acc[e];
-                    if (acc[e] > bv[e]) { bv[e] = acc[e]; bi[e] = row; } // a lane's rows ascend
+    if (nb) {
+        coop_stream<QKK_Q6_K, 8, 1, HEAD_TG, false, true>(
+            W + (size_t)row0 * ROW, nullptr, nb, X, K, batch, [](uint32_t r) { return r; }, smem, tab, tid,
+            [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float) {
+                const uint32_t t = 4 * (ln >> 4) + e, row = row0 + tile * 16 + (ln & 15u);
+                if (t < batch && row < V) {
+                    if (logits_out) logits_out[(size_t)t * V + row] = sum0;
+                    if (sum0 > bv) { bv = sum0; bi = row; }
                 }
-            }
-        }
+            },
+            (size_t)V * ROW - 16 - (size_t)row0 * ROW);
     }
-    // per token: fold the 16 rows of the lane group, then the 16 waves, then the workgroups
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-        dpp_better(bv[e], bi[e]);
-        if (j == 0) { s_v[wave][4 * g + e] = bv[e]; s_i[wave][4 * g + e] = bi[e]; }
-    }
+    // per token: the 32 threads that reduce its outputs (16 rows x BT tiles), then the workgroups
+    float* s_v = (float*)smem;
+    uint32_t* s_i = (uint32_t*)(smem + CT * 4);
+    s_v[tid] = bv;
+    s_i[tid] = bi;
     __syncthreads();
-    if (tid < 16 && (uint32_t)tid < batch) {
-        float v = s_v[0][tid];
-        uint32_t i = s_i[0][tid];
-        for (int w = 1; w < 16; w++)
-            if (better(s_v[w][tid], s_i[w][tid], v, i)) { v = s_v[w][tid]; i = s_i[w][tid]; }
+    if ((uint32_t)tid < batch) {
+        float v = ARG_FLOOR;
+        uint32_t i = 0xFFFFFFFFu;
+        const uint32_t g = tid >> 2, e = tid & 3u;
+        for (uint32_t bt = 0; bt < BT; bt++)
+            for (uint32_t j = 0; j < 16; j++) {
+                const uint32_t o = bt * 256 + e * 64 + g * 16 + j;
+                if (better(s_v[o], s_i[o], v, i)) { v = s_v[o]; i = s_i[o]; }
+            }
         publish(&ws.cand_v[(size_t)tid * gridDim.x + blockIdx.x], v);
         publish(&ws.cand_i[(size_t)tid * gridDim.x + blockIdx.x], i);
     }
@@ -304,12 +245,12 @@ __global__ __launch_bounds__(1024) void head_q6k_mfma_kernel(const uint8_t* __re
     __syncthreads();
     if (s_last) {
         // one wave per token folds the workgroups' candidates
-        if ((uint32_t)wave < batch) {
+        for (uint32_t t = wave; t < batch; t += CW) {
             float v = ARG_FLOOR;
             uint32_t i = 0xFFFFFFFFu;
             for (uint32_t c = lane; c < gridDim.x; c += 64) {
-                const float cv = ws.cand_v[(size_t)wave * gridDim.x + c];
-                const uint32_t ci = ws.cand_i[(size_t)wave * gridDim.x + c];
+                const float cv = ws.cand_v[(size_t)t * gridDim.x + c];
+                const uint32_t ci = ws.cand_i[(size_t)t * gridDim.x + c];
                 if (better(cv, ci, v, i)) { v = cv; i = ci; }
             }
             dpp_better(v, i);
@@ -322,7 +263,7 @@ __global__ __launch_bounds__(1024) void head_q6k_mfma_kernel(const uint8_t* __re
                 const uint32_t oi = (uint32_t)__builtin_amdgcn_readlane((int)i, r);
                 if (better(ov, oi, fv, fi)) { fv = ov; fi = oi; }
             }
-            if (lane == 0) tok[wave] = fi == 0xFFFFFFFFu ? 0u : fi;
+            if (lane == 0) tok[t] = fi == 0xFFFFFFFFu ? 0u : fi;
         }
         if (tid == 0) ws.counter[0] = 0u;
     }
@@ -364,18 +305,18 @@ int qkk_head_argmax(const void* W, const float* X, uint32_t* tok, float* logits,
     hipStream_t st = as_stream(stream);
     if (batch >= 2 && batch <= 16 && K == 2048) {
         HeadWs ws;
-        const uint32_t blocks = persistent_blocks() / 4; // one 16-wave workgroup per CU
+        const uint32_t blocks = persistent_blocks() / 4; // one workgroup per CU (LDS)
         ws.counter = (uint32_t*)workspace;
         ws.cand_v = (float*)((uint8_t*)workspace + 256);
         ws.cand_i = (uint32_t*)(ws.cand_v + (size_t)batch * blocks);
-        const size_t lds = (size_t)2 * 16 * K * sizeof(_Float16);
         static bool attr_done = false;
         if (!attr_done) {
-            (void)hipFuncSetAttribute((const void*)head_q6k_mfma_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 4096);
+            (void)hipFuncSetAttribute((const void*)head_q6k_coop_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      (int)HeadGeo::LDS_BYTES);
             attr_done = true;
         }
-        hipLaunchKernelGGL(head_q6k_mfma_kernel<8>, dim3(blocks), dim3(1024), lds, st, (const uint8_t*)W, X, logits,
-                           tok, ws, V, batch);
+        hipLaunchKernelGGL(head_q6k_coop_kernel, dim3(blocks), dim3(CT), HeadGeo::LDS_BYTES, st, (const uint8_t*)W, X,
+                           logits, tok, ws, V, batch);
         return check_launch("qkk_head_argmax");
     }
     const uint32_t rif = K == 2048 ? HEAD_RIF : 2;
