@@ -208,7 +208,9 @@ constexpr int CT = 64 * CW; // threads per workgroup
 
 // ALT: the NS = 2 tensors take turns, batch 2q = tiles of tensor 0, batch 2q+1 = the same rows
 // of tensor 1 (for blocks too large to double-buffer both tensors' tiles together).
-template <int TYPE, int KS, int NS, int TG, bool ALT = false>
+// NA: tiles of 16 activation rows a wave keeps as A operands (every weight fragment is decoded once
+// and applied to all of them).
+template <int TYPE, int KS, int NS, int TG, bool ALT = false, int NA = 1>
 struct CoopGeom {
     static constexpr int G = CW / KS;                   // tile groups
     static constexpr int BT = G * TG;                   // row tiles per tensor and batch
@@ -216,7 +218,7 @@ struct CoopGeom {
     static constexpr uint32_t RB = (uint32_t)qkk_row_bytes_dev<TYPE>(256 * KS);
     static constexpr uint32_t TBYTES = 16 * RB;         // one tile of 16 rows: contiguous
     static constexpr uint32_t BBYTES = NSB * BT * TBYTES; // one batch in LDS
-    static constexpr uint32_t PART_BYTES = NSB * BT * KS * 64 * 16;
+    static constexpr uint32_t PART_BYTES = NSB * BT * KS * NA * 64 * 16;
     static constexpr uint32_t LDS_BYTES = 2 * BBYTES + 2 * PART_BYTES; // both double-buffered
     static_assert(BBYTES % 16 == 0 && CW % KS == 0 && (!ALT || NS == 2), "geometry");
 };
@@ -229,9 +231,9 @@ struct AFrag {
 
 template <int LAYOUT, typename RowOf>
 __device__ __forceinline__ void load_afrag(AFrag& a, const float* __restrict__ X, uint32_t stride, uint32_t k0,
-                                           uint32_t np, RowOf row_of, int lane)
+                                           uint32_t np, RowOf row_of, int lane, uint32_t first_row = 0)
 {
-    const uint32_t j = lane & 15, g = lane >> 4;
+    const uint32_t j = first_row + (lane & 15), g = lane >> 4;
     const float keep = j < np ? 1.f : 0.f;
     const float* src = X + (size_t)row_of(min(j, np - 1)) * stride + k0;
     float4 v[8][2];
@@ -254,24 +256,24 @@ __device__ __forceinline__ void load_afrag(AFrag& a, const float* __restrict__ X
 }
 
 // Streams n_batches batches of BT row tiles starting at base0 / base1 (tensor 0 / 1, first row
-// of the sub-item) and calls epi(tile, lane, e, sum0, sum1) for every output: tile = row tile
-// within the sub-item, lane%16 = row within the tile, 4*(lane/16)+e = activation row, sum_s =
-// tensor s's dot product.  One barrier per batch: batch b+1 is written to the other LDS buffer
+// of the sub-item) and calls epi(tile, lane, e, sum0, sum1, na) for every output: tile = row tile
+// within the sub-item, lane%16 = row within the tile, 16*na + 4*(lane/16)+e = activation row,
+// sum_s = tensor s's dot product.  One barrier per batch: batch b+1 is written to the other LDS buffer
 // as soon as this wave is done with batch b (nobody reads that buffer any more), the partials
 // alternate between two buffers as well, so fast waves run ahead into the next batch.
 // CLAMP: `limit` is the offset from base0 of the tensor's last 16 bytes; loads beyond it re-read
 // those (the caller ignores the rows that do not exist).
-template <int TYPE, int KS, int NS, int TG, bool ALT, bool CLAMP, typename RowOf, typename Epi>
+template <int TYPE, int KS, int NS, int TG, bool ALT, bool CLAMP, int NA = 1, typename RowOf, typename Epi>
 __device__ __forceinline__ void coop_stream(const uint8_t* __restrict__ base0, const uint8_t* __restrict__ base1,
                                             uint32_t n_batches, const float* __restrict__ A_src, uint32_t a_stride,
                                             uint32_t np, RowOf row_of, uint8_t* smem, const MfmaTables& tab, int tid,
                                             Epi epi, size_t limit = 0)
 {
-    using Geo = CoopGeom<TYPE, KS, NS, TG, ALT>;
+    using Geo = CoopGeom<TYPE, KS, NS, TG, ALT, NA>;
     constexpr int BT = Geo::BT, NSB = Geo::NSB, NTL = NSB * TG; // tiles per wave and batch
     constexpr uint32_t RB = Geo::RB, TBYTES = Geo::TBYTES, BBYTES = Geo::BBYTES, PBYTES = Geo::PART_BYTES;
     constexpr int PIECES = BBYTES / 16, PPT = BT * TBYTES / 16, NLD = (PIECES + CT - 1) / CT;
-    constexpr int OUTS = (BT * 256 + CT - 1) / CT; // outputs per thread and batch
+    constexpr int OUTS = (NA * BT * 256 + CT - 1) / CT; // outputs per thread and batch
     const int lane = tid & 63, wave = tid >> 6, kw = wave % KS, tg = wave / KS, j = lane & 15, g = lane >> 4;
     const uint32_t steps = ALT ? 2 * n_batches : n_batches; // LDS batches
 
@@ -294,8 +296,9 @@ __device__ __forceinline__ void coop_stream(const uint8_t* __restrict__ base0, c
     };
 #pragma unroll
     for (int n = 0; n < NLD; n++) ld[n] = *(const u32x4*)src[n];
-    AFrag a; // fetched and converted while the first batch is in flight
-    load_afrag<BFrag<TYPE>::LAYOUT>(a, A_src, a_stride, 256 * kw, np, row_of, lane);
+    AFrag a[NA]; // fetched and converted while the first batch is in flight
+#pragma unroll
+    for (int na = 0; na < NA; na++) load_afrag<BFrag<TYPE>::LAYOUT>(a[na], A_src, a_stride, 256 * kw, np, row_of, lane, 16 * na);
 #pragma unroll
     for (int n = 0; n < NLD; n++)
         if (PIECES % CT == 0 || n + 1 < NLD || tid + CT * n < PIECES) *(u32x4*)(smem + (size_t)(tid + CT * n) * 16) = ld[n];
@@ -319,30 +322,38 @@ __device__ __forceinline__ void coop_stream(const uint8_t* __restrict__ base0, c
 #pragma unroll
             for (int t = 0; t < TG; t++)
                 f[s * TG + t].load(smem + buf * BBYTES + ((size_t)(s * BT + tg * TG + t) * 16 + j) * RB, kw, g);
-        float4v acc[NTL];
+        float4v acc[NTL][NA];
 #pragma unroll
-        for (int t = 0; t < NTL; t++) acc[t] = float4v{0.f, 0.f, 0.f, 0.f};
+        for (int t = 0; t < NTL; t++)
+#pragma unroll
+            for (int na = 0; na < NA; na++) acc[t][na] = float4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < 8; i++) {
 #pragma unroll
             for (int t = 0; t < NTL; t++) {
                 half8 bl;
                 const half8 bh = f[t].step(i, g, tab, bl);
-                acc[t] = mfma16x32(a.hi[i], bh, acc[t]);
-                acc[t] = mfma16x32(a.lo[i], bh, acc[t]);
-                if constexpr (BFrag<TYPE>::SPLIT) acc[t] = mfma16x32(a.hi[i], bl, acc[t]);
+#pragma unroll
+                for (int na = 0; na < NA; na++) {
+                    acc[t][na] = mfma16x32(a[na].hi[i], bh, acc[t][na]);
+                    acc[t][na] = mfma16x32(a[na].lo[i], bh, acc[t][na]);
+                    if constexpr (BFrag<TYPE>::SPLIT) acc[t][na] = mfma16x32(a[na].hi[i], bl, acc[t][na]);
+                }
             }
             __builtin_amdgcn_sched_barrier(0); // keep the decode of later steps from piling up in registers
         }
-        float* part = (float*)(smem + 2 * BBYTES + buf * PBYTES); // [NSB*BT][KS][64 lanes][4]
+        float* part = (float*)(smem + 2 * BBYTES + buf * PBYTES); // [NA][NSB*BT][KS][64 lanes][4]
 #pragma unroll
         for (int s = 0; s < NSB; s++)
 #pragma unroll
             for (int t = 0; t < TG; t++) {
                 const float sc = f[s * TG + t].post();
-                const float4v r = acc[s * TG + t];
-                *(float4*)(part + (((size_t)(s * BT + tg * TG + t) * KS + kw) * 64 + lane) * 4) =
-                    float4{sc * r[0], sc * r[1], sc * r[2], sc * r[3]};
+#pragma unroll
+                for (int na = 0; na < NA; na++) {
+                    const float4v r = acc[s * TG + t][na];
+                    *(float4*)(part + ((((size_t)na * NSB * BT + s * BT + tg * TG + t) * KS + kw) * 64 + lane) * 4) =
+                        float4{sc * r[0], sc * r[1], sc * r[2], sc * r[3]};
+                }
             }
 #pragma unroll
         for (int n = 0; n < NLD; n++)
@@ -352,16 +363,17 @@ __device__ __forceinline__ void coop_stream(const uint8_t* __restrict__ base0, c
 #pragma unroll
         for (int oo = 0; oo < OUTS; oo++) {
             const uint32_t o = tid + CT * oo;
-            if (BT * 256 % CT != 0 && o >= (uint32_t)BT * 256) break;
-            const uint32_t bt = o >> 8, e = (o >> 6) & 3u, ln = o & 63u;
+            if (NA * BT * 256 % CT != 0 && o >= (uint32_t)NA * BT * 256) break;
+            const uint32_t na = o / (BT * 256), bt = (o >> 8) % BT, e = (o >> 6) & 3u, ln = o & 63u;
+            const float* pa = part + (size_t)na * (NSB * BT * KS * 256);
             float sum0 = 0.f, sum1 = 0.f;
 #pragma unroll
             for (int w = 0; w < KS; w++) {
-                sum0 += part[(((size_t)bt * KS + w) * 64 + ln) * 4 + e];
-                if (NSB > 1) sum1 += part[(((size_t)(BT + bt) * KS + w) * 64 + ln) * 4 + e];
+                sum0 += pa[(((size_t)bt * KS + w) * 64 + ln) * 4 + e];
+                if (NSB > 1) sum1 += pa[(((size_t)(BT + bt) * KS + w) * 64 + ln) * 4 + e];
             }
-            if (!ALT) epi(b * BT + bt, ln, e, sum0, sum1);
-            else if (b & 1u) epi((b >> 1) * BT + bt, ln, e, saved[oo], sum0);
+            if (!ALT) epi(b * BT + bt, ln, e, sum0, sum1, na);
+            else if (b & 1u) epi((b >> 1) * BT + bt, ln, e, saved[oo], sum0, na);
             else saved[oo] = sum0;
         }
     }

@@ -213,7 +213,7 @@ __global__ __launch_bounds__(CT) void head_q6k_coop_kernel(const uint8_t* __rest
     if (nb) {
         coop_stream<QKK_Q6_K, 8, 1, HEAD_TG, false, true>(
             W + (size_t)row0 * ROW, nullptr, nb, X, K, batch, [](uint32_t r) { return r; }, smem, tab, tid,
-            [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float) {
+            [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float, uint32_t) {
                 const uint32_t t = 4 * (ln >> 4) + e, row = row0 + tile * 16 + (ln & 15u);
                 if (t < batch && row < V) {
                     if (logits_out) logits_out[(size_t)t * V + row] = sum0;

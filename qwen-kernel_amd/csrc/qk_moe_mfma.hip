@@ -93,7 +93,7 @@ __global__ __launch_bounds__(CT) void moe_gateup_mfma_kernel(const uint8_t* __re
             if (it.shared) {
                 const uint32_t row0 = it.sub * nb_s * GuGeoS::BT * 16;
                 coop_stream<QKK_Q8_0, 8, 2, GU_TG_S, true, false>(gate_shexp + (size_t)row0 * GuGeoS::RB, up_shexp + (size_t)row0 * GuGeoS::RB, nb_s, X, H, np, row_of, smem, tab, tid,
-                    [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1) {
+                    [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1, uint32_t) {
                         const uint32_t r = 4 * (ln >> 4) + e;
                         if (r < np)
                             ws.h[((size_t)s_tok[r] * (d.k + 1) + s_slot[r]) * F + row0 + tile * 16 + (ln & 15u)] =
@@ -104,7 +104,7 @@ __global__ __launch_bounds__(CT) void moe_gateup_mfma_kernel(const uint8_t* __re
             const uint32_t row0 = it.sub * nb_r * GuGeoR::BT * 16;
             const size_t eo = ((size_t)it.expert * F + row0) * GuGeoR::RB;
             coop_stream<QKK_IQ3_XXS, 8, 2, GU_TG_R, false, false>(gate_exps + eo, up_exps + eo, nb_r, X, H, np, row_of, smem, tab, tid,
-                [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1) {
+                [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1, uint32_t) {
                     const uint32_t r = 4 * (ln >> 4) + e;
                     if (r < np)
                         ws.h[((size_t)s_tok[r] * (d.k + 1) + s_slot[r]) * F + row0 + tile * 16 + (ln & 15u)] =
@@ -165,7 +165,7 @@ __global__ __launch_bounds__(CT) void moe_down_mfma_kernel(const uint8_t* __rest
             if (it.shared) {
                 const uint32_t row0 = it.sub * nb_s * Geo::S::BT * 16;
                 coop_stream<QKK_Q8_0, FB, 1, Geo::TG_S, false, false>(down_shexp + (size_t)row0 * Geo::S::RB, nullptr, nb_s, ws.h, F, np, row_of, smem, tab, tid,
-                    [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1) {
+                    [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1, uint32_t) {
                         const uint32_t r = 4 * (ln >> 4) + e;
                         if (r < np)
                             ws.contrib[((size_t)s_tok[r] * (d.k + 1) + s_slot[r]) * H + row0 + tile * 16 + (ln & 15u)] =
@@ -175,7 +175,7 @@ __global__ __launch_bounds__(CT) void moe_down_mfma_kernel(const uint8_t* __rest
             }
             const uint32_t row0 = it.sub * nb_r * Geo::R::BT * 16;
             coop_stream<TYPE_DN, FB, 1, Geo::TG_R, false, false>(down_exps + ((size_t)it.expert * H + row0) * Geo::R::RB, nullptr, nb_r, ws.h, F, np, row_of, smem, tab, tid,
-                [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1) {
+                [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1, uint32_t) {
                     const uint32_t r = 4 * (ln >> 4) + e;
                     if (r < np)
                         ws.contrib[((size_t)s_tok[r] * (d.k + 1) + s_slot[r]) * H + row0 + tile * 16 + (ln & 15u)] =
