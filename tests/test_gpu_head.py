@@ -38,7 +38,8 @@ def test_head_full_vocab_bs16(qk, orc, dev):
     head_case(qk, orc, dev, 151936, 2048, 16, seed=11)
 
 
-@pytest.mark.parametrize("V,K,batch", [(1000, 2048, 2), (4097, 2048, 1), (3, 2048, 1), (777, 4096, 3)])
+@pytest.mark.parametrize("V,K,batch", [(1000, 2048, 2), (4097, 2048, 1), (3, 2048, 1), (777, 4096, 3), (4097, 2048, 16),
+                                           (33, 2048, 5), (16, 2048, 9)])
 def test_head_ragged(qk, orc, dev, V, K, batch):
     head_case(qk, orc, dev, V, K, batch, seed=12 + V)
 

@@ -53,6 +53,7 @@ def test_moe_prefill_small_layer_many_pairs_per_expert(qk, orc, dev):
 
 
 @pytest.mark.parametrize("M,K,N", [(8192, 2048, 128), (100, 96, 5), (64, 32, 33), (130, 2048, 200), (4096, 4096, 48),
+                                   (300, 256, 40), (96, 512, 64), (1000, 1024, 17), (17, 2048, 8), (2048, 2048, 7),
                                    (7, 64, 1), (1024, 512, 16)])
 def test_gemm_q8_0(qk, orc, dev, M, K, N):
     import torch
