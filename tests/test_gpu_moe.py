@@ -168,6 +168,30 @@ def test_moe_argument_errors(qk, dev, layer_iq4):
     assert e.value.code == -5
 
 
+def test_moe_several_rows_need_n_embd_2048(qk, dev):
+    """One row works at n_embd = 4096; several rows are refused with a shape error, not run wrong."""
+    import torch
+    hl = qk.synth.HostLayer(seed=55, n_embd=4096, n_ff=256, n_expert=4, n_used=2)
+    layer = hl.to_device(dev)
+    X = torch.zeros((3, 4096), device=dev)
+    ws = torch.zeros(qk.moe_workspace_bytes(layer, 3), dtype=torch.uint8, device=dev)
+    with pytest.raises(qk.QkError) as e:
+        qk.moe_decode(layer, X, ws)
+    assert e.value.code == -2 and "2048" in str(e.value)
+
+
+def test_moe_decode_bs17_two_shared_tiles(qk, orc, dev, layer_iq4):
+    """17 rows: the shared expert needs a second, one-row tile; workspace reused for a smaller call."""
+    import torch
+    print("[case] moe bs=17 then bs=2 on one workspace", flush=True)
+    X, refs = pick_inputs(orc, layer_iq4, 17, seed=31)
+    layer, ws, Y, sel = check(qk, orc, dev, layer_iq4, X, refs)
+    Y2, sel2 = qk.moe_decode(layer, torch.from_numpy(X[:2]).to(dev), ws)
+    torch.cuda.synchronize()
+    for s in range(2):
+        assert orc.rel_maxabs_err(Y2.cpu().numpy()[s], refs[s]["y"]) <= TOL
+
+
 def test_group_pairs_matches_oracle(qk, orc, dev):
     import torch
     print("[case] group pairs", flush=True)
