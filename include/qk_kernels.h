@@ -112,7 +112,8 @@ size_t qkk_moe_workspace_bytes(const qkk_moe_layer *L_host, uint32_t n_slots);
  *   workspace                      qkk_moe_workspace_bytes(), 256-byte aligned, must be
  *                                  zero-filled once before its first use; calls sharing
  *                                  a workspace must not overlap in time.
- * Expert weights are read once per step however many slots pick the same expert. */
+ * With n_slots >= 2 every picked expert's weights are read once per 16 rows that picked it
+ * (matrix-core path); that path needs n_embd = 2048 and returns QKK_ESHAPE otherwise. */
 int qkk_moe_decode(const qkk_moe_layer *L_host, const float *X, float *Y, qkk_sel *sel,
                    void *workspace, size_t workspace_bytes, uint32_t n_slots, void *stream);
 
@@ -147,8 +148,9 @@ int qkk_head_argmax(const void *W, const float *X, uint32_t *tok, float *logits,
 int qkk_argmax(const float *logits, uint32_t *tok, uint32_t n, uint32_t batch, void *stream);
 
 /* Batched-prefill dense projection Y[n][m] = X[n] . W[m], W in Q8_0 (reference
- * shaders/gemm_q8_0.comp:32-101, gemm_q8_0_coopmat2.comp:42-148): fp16 tiles dequantised
- * in LDS, MFMA with fp32 accumulation.  X [N][K] fp32, Y [N][M] fp32. */
+ * shaders/gemm_q8_0.comp:32-101, gemm_q8_0_coopmat2.comp:42-148): Q8_0 rows streamed through
+ * LDS, MFMA on half operands with fp32 accumulation (activations and weights kept exact to
+ * ~2^-22 by hi/lo splits).  X [N][K] fp32, Y [N][M] fp32, K a multiple of 32. */
 int qkk_gemm_q8_0(const void *W, const float *X, float *Y, uint32_t M, uint32_t K, uint32_t N,
                   void *stream);
 
