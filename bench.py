@@ -303,6 +303,13 @@ def main():
                                                 frac=g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9 / HBM_PEAK_GBPS)
             log(f"[bench] gemv {name}: {ex[f'gemv_{name}_8192x2048']}")
             torch.cuda.empty_cache()
+            if t != qk.F16:  # the same projection for 16 decode slots: weights read once
+                g = gemv_workload(qk, t, 8192, 2048, 16, es, ew)
+                ex[f"gemv_{name}_8192x2048_bs16"] = dict(us=g["ms_event"] * 1e3,
+                                                         gbps=g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9,
+                                                         frac=g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9 / HBM_PEAK_GBPS)
+                log(f"[bench] gemv {name} bs16: {ex[f'gemv_{name}_8192x2048_bs16']}")
+                torch.cuda.empty_cache()
         for b in (1, 16):
             h = head_workload(qk, 151936, 2048, b, 40, 8)
             ex[f"head_q6k_151936_bs{b}"] = dict(us=h["ms_event"] * 1e3, gbps=h["bytes_step"] / (h["ms_event"] * 1e-3) / 1e9,

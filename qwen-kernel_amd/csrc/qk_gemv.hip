@@ -344,6 +344,12 @@ static int dispatch_q(const void* W, const float* X, float* Y, uint32_t M, uint3
 
 using namespace qk;
 
+namespace qk {
+bool coop_gemm_launch(int type, const uint8_t* W, const float* X, float* Y, uint32_t M, uint32_t K, uint32_t N,
+                      hipStream_t st);
+constexpr uint32_t COOP_MIN_BATCH = 3;
+} // namespace qk
+
 extern "C" {
 
 const char* qkk_last_error(void) { return t_err; }
@@ -422,6 +428,10 @@ int qkk_gemv(int type, const void* W, const float* X, float* Y, uint32_t M, uint
                     "qkk_gemv: type %d with K=%u is not supported", type, K);
     if (int rc = require_device()) return rc;
     hipStream_t st = as_stream(stream);
+    // several rows: read the weights once for all of them on the matrix cores (needs Y aligned
+    // like any output of that path); one row, or a shape that path does not cover: one pass per row
+    if (batch >= COOP_MIN_BATCH && aligned16(Y) && coop_gemm_launch(type, (const uint8_t*)W, X, Y, M, K, batch, st))
+        return check_launch("qkk_gemv");
     switch (type) {
     case QKK_Q8_0: return dispatch_q<QKK_Q8_0>(W, X, Y, M, K, batch, st);
     case QKK_Q6_K: return dispatch_q<QKK_Q6_K>(W, X, Y, M, K, batch, st);

@@ -2,7 +2,6 @@
 // projection GEMM (cooperative matrix-core stream for K = 256..2048 and N >= 8, a lane-direct
 // MFMA kernel otherwise); the grouped-expert MoE entry point forwards to the expert-major
 // kernels of qk_moe_grouped.hip / qk_moe_mfma.hip.
-#include "qk_coop.h"
 #include "qk_device.h"
 #include "qk_host.h"
 
@@ -187,55 +186,9 @@ __global__ __launch_bounds__(256) void gemm_q8_0_kernel(const uint8_t* __restric
     }
 }
 
-// ---- Q8_0 GEMM for K = 256..2048 on the cooperative stream (qk_coop.h) -----------------------------
-// Y[n][m] = W[m] . X[n]: the projection is one dense "expert" of M rows.  A workgroup takes a
-// range of row tiles and GEMM_NA*16 tokens; every weight fragment is decoded once and applied to
-// all GEMM_NA activation tiles the wave keeps in registers.
-constexpr int GEMM_NA = 2;
-template <int KS>
-using GemmGeo = CoopGeom<QKK_Q8_0, KS, 1, 1, false, GEMM_NA>;
-
-template <int KS>
-__global__ __launch_bounds__(CT) void gemm_q8_0_coop_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X,
-                                                            float* __restrict__ Y, uint32_t M, uint32_t N,
-                                                            uint32_t ranges)
-{
-    using Geo = GemmGeo<KS>;
-    constexpr uint32_t K = 256 * KS, RB = Geo::RB, BT = Geo::BT;
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    __shared__ MfmaTables tab; // unused by Q8_0
-    const int tid = threadIdx.x;
-    const uint32_t groups = (N + 16 * GEMM_NA - 1) / (16 * GEMM_NA);
-    const uint32_t q = blockIdx.x % groups, r = blockIdx.x / groups;
-    // batches [b0, b1) of the tensor's `total`, an even split over the ranges (b1 <= total)
-    const uint32_t total = (M + 16 * BT - 1) / (16 * BT);
-    const uint32_t b0 = (uint32_t)((uint64_t)r * total / ranges), b1 = (uint32_t)((uint64_t)(r + 1) * total / ranges);
-    const uint32_t row0 = b0 * BT * 16, tok0 = q * 16 * GEMM_NA;
-    if (b1 <= b0 || row0 >= M || tok0 >= N) return;
-    const uint32_t np = min((uint32_t)(16 * GEMM_NA), N - tok0);
-    coop_stream<QKK_Q8_0, KS, 1, 1, false, true, GEMM_NA>(
-        W + (size_t)row0 * RB, nullptr, b1 - b0, X + (size_t)tok0 * K, K, np, [](uint32_t t) { return t; }, smem, tab, tid,
-        [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float, uint32_t na) {
-            const uint32_t t = 16 * na + 4 * (ln >> 4) + e, row = row0 + tile * 16 + (ln & 15u);
-            if (t < np && row < M) Y[(size_t)(tok0 + t) * M + row] = sum0;
-        },
-        (size_t)M * RB - 16 - (size_t)row0 * RB);
-}
-
-template <int KS>
-static void launch_gemm_coop(const uint8_t* W, const float* X, float* Y, uint32_t M, uint32_t N, hipStream_t st)
-{
-    using Geo = GemmGeo<KS>;
-    static bool once = ((void)hipFuncSetAttribute((const void*)gemm_q8_0_coop_kernel<KS>,
-                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)Geo::LDS_BYTES), true);
-    (void)once;
-    const uint32_t groups = (N + 16 * GEMM_NA - 1) / (16 * GEMM_NA);
-    const uint32_t total = (M + 16 * Geo::BT - 1) / (16 * Geo::BT);
-    // one workgroup per CU (LDS), at least four batches each where the tensor allows
-    const uint32_t want = std::max(1u, (persistent_blocks() / 4) / groups);
-    const uint32_t ranges = std::max(1u, std::min(want, (total + 3) / 4));
-    hipLaunchKernelGGL(gemm_q8_0_coop_kernel<KS>, dim3(groups * ranges), dim3(CT), Geo::LDS_BYTES, st, W, X, Y, M, N, ranges);
-}
+// Cooperative matrix-core GEMM for K = 256..2048 (qk_gemm_coop.hip); false if the shape is not covered.
+bool coop_gemm_launch(int type, const uint8_t* W, const float* X, float* Y, uint32_t M, uint32_t K, uint32_t N,
+                      hipStream_t st);
 
 } // namespace qk
 
@@ -268,13 +221,7 @@ int qkk_gemm_q8_0(const void* W, const float* X, float* Y, uint32_t M, uint32_t 
     if (int rc = require_device()) return rc;
     hipStream_t st = as_stream(stream);
     const uint8_t* w = (const uint8_t*)W;
-    if (N >= 8 && (K == 256 || K == 512 || K == 1024 || K == 2048)) {
-        if (K == 256) launch_gemm_coop<1>(w, X, Y, M, N, st);
-        else if (K == 512) launch_gemm_coop<2>(w, X, Y, M, N, st);
-        else if (K == 1024) launch_gemm_coop<4>(w, X, Y, M, N, st);
-        else launch_gemm_coop<8>(w, X, Y, M, N, st);
-        return check_launch("qkk_gemm_q8_0");
-    }
+    if (N >= 8 && coop_gemm_launch(QKK_Q8_0, w, X, Y, M, K, N, st)) return check_launch("qkk_gemm_q8_0");
     const uint32_t mb = (M + 63) / 64;
     const bool deep = (K / 32) % 4 == 0;
 #define QK_GEMM_LAUNCH(NT_, D_, GY_)                                                                         \

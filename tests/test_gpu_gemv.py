@@ -32,6 +32,15 @@ def test_gemv_quantised(qk, orc, dev, name, M, K, batch):
     run_case(qk, orc, dev, name, M, K, batch)
 
 
+@pytest.mark.parametrize("name", ["q8_0", "q6_k", "iq4_xs", "iq3_xxs"])
+@pytest.mark.parametrize("M,K,batch", [(8192, 2048, 16), (1000, 2048, 5), (130, 1024, 16), (96, 512, 4),
+                                       (77, 512, 3), (48, 256, 32), (2048, 2048, 40), (33, 2048, 17)])
+def test_gemv_quantised_several_rows(qk, orc, dev, name, M, K, batch):
+    """batch >= 3 takes the matrix-core path where the shape allows (K = 256..2048 and the tensor
+    ending on a 16-byte boundary), one pass per row otherwise: same bar either way."""
+    run_case(qk, orc, dev, name, M, K, batch, seed=77)
+
+
 @pytest.mark.parametrize("M,K", [(64, 32), (33, 96), (10, 2080)])
 def test_gemv_q8_0_short_rows(qk, orc, dev, M, K):
     run_case(qk, orc, dev, "q8_0", M, K, 1)
