@@ -210,7 +210,8 @@ constexpr int CT = 64 * CW; // threads per workgroup
 // of tensor 1 (for blocks too large to double-buffer both tensors' tiles together).
 // NA: tiles of 16 activation rows a wave keeps as A operands (every weight fragment is decoded once
 // and applied to all of them).
-template <int TYPE, int KS, int NS, int TG, bool ALT = false, int NA = 1>
+// PB: partial-result buffers, 2 (one barrier per batch) or 1 (two barriers, less LDS).
+template <int TYPE, int KS, int NS, int TG, bool ALT = false, int NA = 1, int PB = 2>
 struct CoopGeom {
     static constexpr int G = CW / KS;                   // tile groups
     static constexpr int BT = G * TG;                   // row tiles per tensor and batch
@@ -219,7 +220,7 @@ struct CoopGeom {
     static constexpr uint32_t TBYTES = 16 * RB;         // one tile of 16 rows: contiguous
     static constexpr uint32_t BBYTES = NSB * BT * TBYTES; // one batch in LDS
     static constexpr uint32_t PART_BYTES = NSB * BT * KS * NA * 64 * 16;
-    static constexpr uint32_t LDS_BYTES = 2 * BBYTES + 2 * PART_BYTES; // both double-buffered
+    static constexpr uint32_t LDS_BYTES = 2 * BBYTES + PB * PART_BYTES;
     static_assert(BBYTES % 16 == 0 && CW % KS == 0 && (!ALT || NS == 2), "geometry");
 };
 
@@ -263,13 +264,13 @@ __device__ __forceinline__ void load_afrag(AFrag& a, const float* __restrict__ X
 // alternate between two buffers as well, so fast waves run ahead into the next batch.
 // CLAMP: `limit` is the offset from base0 of the tensor's last 16 bytes; loads beyond it re-read
 // those (the caller ignores the rows that do not exist).
-template <int TYPE, int KS, int NS, int TG, bool ALT, bool CLAMP, int NA = 1, typename RowOf, typename Epi>
+template <int TYPE, int KS, int NS, int TG, bool ALT, bool CLAMP, int NA = 1, int PB = 2, typename RowOf, typename Epi>
 __device__ __forceinline__ void coop_stream(const uint8_t* __restrict__ base0, const uint8_t* __restrict__ base1,
                                             uint32_t n_batches, const float* __restrict__ A_src, uint32_t a_stride,
                                             uint32_t np, RowOf row_of, uint8_t* smem, const MfmaTables& tab, int tid,
                                             Epi epi, size_t limit = 0)
 {
-    using Geo = CoopGeom<TYPE, KS, NS, TG, ALT, NA>;
+    using Geo = CoopGeom<TYPE, KS, NS, TG, ALT, NA, PB>;
     constexpr int BT = Geo::BT, NSB = Geo::NSB, NTL = NSB * TG; // tiles per wave and batch
     constexpr uint32_t RB = Geo::RB, TBYTES = Geo::TBYTES, BBYTES = Geo::BBYTES, PBYTES = Geo::PART_BYTES;
     constexpr int PIECES = BBYTES / 16, PPT = BT * TBYTES / 16, NLD = (PIECES + CT - 1) / CT;
@@ -342,7 +343,7 @@ __device__ __forceinline__ void coop_stream(const uint8_t* __restrict__ base0, c
             }
             __builtin_amdgcn_sched_barrier(0); // keep the decode of later steps from piling up in registers
         }
-        float* part = (float*)(smem + 2 * BBYTES + buf * PBYTES); // [NA][NSB*BT][KS][64 lanes][4]
+        float* part = (float*)(smem + 2 * BBYTES + (PB > 1 ? buf : 0u) * PBYTES); // [NA][NSB*BT][KS][64 lanes][4]
 #pragma unroll
         for (int s = 0; s < NSB; s++)
 #pragma unroll
@@ -376,6 +377,7 @@ __device__ __forceinline__ void coop_stream(const uint8_t* __restrict__ base0, c
             else if (b & 1u) epi((b >> 1) * BT + bt, ln, e, saved[oo], sum0, na);
             else saved[oo] = sum0;
         }
+        if (PB == 1) __syncthreads(); // the single partial buffer is free again
     }
     __syncthreads(); // the buffers are free for the next call
 }

@@ -53,8 +53,9 @@ __device__ __forceinline__ Item get_item(const MoeWs& ws, uint32_t index, uint32
 // n_embd = 2048: the eight waves take one 256-weight fragment each.  Routed experts: batches of
 // one row tile of gate and of up (IQ3_XXS); shared expert (Q8_0): one row tile, gate and up in turns.
 constexpr int GU_TG_R = 1, GU_TG_S = 1;
-using GuGeoR = CoopGeom<QKK_IQ3_XXS, 8, 2, GU_TG_R>;
-using GuGeoS = CoopGeom<QKK_Q8_0, 8, 2, GU_TG_S, true>;
+constexpr int GU_PB = 2; // partial buffers (2: one barrier per batch)
+using GuGeoR = CoopGeom<QKK_IQ3_XXS, 8, 2, GU_TG_R, false, 1, GU_PB>;
+using GuGeoS = CoopGeom<QKK_Q8_0, 8, 2, GU_TG_S, true, 1, GU_PB>;
 constexpr uint32_t GU_LDS = GuGeoR::LDS_BYTES > GuGeoS::LDS_BYTES ? GuGeoR::LDS_BYTES : GuGeoS::LDS_BYTES;
 
 __global__ __launch_bounds__(CT) void moe_gateup_mfma_kernel(const uint8_t* __restrict__ gate_exps,
@@ -92,7 +93,7 @@ __global__ __launch_bounds__(CT) void moe_gateup_mfma_kernel(const uint8_t* __re
             const auto row_of = [&](uint32_t r) { return s_tok[r]; };
             if (it.shared) {
                 const uint32_t row0 = it.sub * nb_s * GuGeoS::BT * 16;
-                coop_stream<QKK_Q8_0, 8, 2, GU_TG_S, true, false>(gate_shexp + (size_t)row0 * GuGeoS::RB, up_shexp + (size_t)row0 * GuGeoS::RB, nb_s, X, H, np, row_of, smem, tab, tid,
+                coop_stream<QKK_Q8_0, 8, 2, GU_TG_S, true, false, 1, GU_PB>(gate_shexp + (size_t)row0 * GuGeoS::RB, up_shexp + (size_t)row0 * GuGeoS::RB, nb_s, X, H, np, row_of, smem, tab, tid,
                     [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1, uint32_t) {
                         const uint32_t r = 4 * (ln >> 4) + e;
                         if (r < np)
@@ -103,7 +104,7 @@ __global__ __launch_bounds__(CT) void moe_gateup_mfma_kernel(const uint8_t* __re
             }
             const uint32_t row0 = it.sub * nb_r * GuGeoR::BT * 16;
             const size_t eo = ((size_t)it.expert * F + row0) * GuGeoR::RB;
-            coop_stream<QKK_IQ3_XXS, 8, 2, GU_TG_R, false, false>(gate_exps + eo, up_exps + eo, nb_r, X, H, np, row_of, smem, tab, tid,
+            coop_stream<QKK_IQ3_XXS, 8, 2, GU_TG_R, false, false, 1, GU_PB>(gate_exps + eo, up_exps + eo, nb_r, X, H, np, row_of, smem, tab, tid,
                 [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1, uint32_t) {
                     const uint32_t r = 4 * (ln >> 4) + e;
                     if (r < np)
@@ -235,12 +236,17 @@ void moe_mfma_launch(const qkk_moe_layer* L, const float* X, float* Y, const qkk
 {
     const uint32_t experts = (uint32_t)std::min<uint64_t>(d.E, (uint64_t)N * d.k); // upper bound of the active ones
     if (stages & QKK_STAGE_GATEUP) {
-        static bool once = (set_lds_attr((const void*)moe_gateup_mfma_kernel, GU_LDS), true);
-        (void)once;
+        static const uint32_t per_cu = [] { // workgroups that fit a CU at once (registers, LDS)
+            set_lds_attr((const void*)moe_gateup_mfma_kernel, GU_LDS);
+            int n = 1;
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void*)moe_gateup_mfma_kernel, CT, GU_LDS) != hipSuccess || n < 1)
+                n = 1;
+            return (uint32_t)std::min(n, 2);
+        }();
         const uint32_t tot_r = d.F / (16 * GuGeoR::BT), tot_s = d.F / (16 * GuGeoS::BT);
         const uint32_t nb_r = pick_nb(tot_r, experts), nb_s = std::min(tot_s, std::max(1u, nb_r * GuGeoR::BT / GuGeoS::BT / 2));
         const uint32_t items = experts * (tot_r / nb_r) + (N + 15) / 16 * (tot_s / nb_s);
-        const uint32_t blocks = std::min(items, persistent_blocks() / 4);
+        const uint32_t blocks = std::min(items, per_cu * (persistent_blocks() / 4));
         hipLaunchKernelGGL(moe_gateup_mfma_kernel, dim3(blocks), dim3(CT), GU_LDS, st, (const uint8_t*)L->gate_exps,
                            (const uint8_t*)L->up_exps, (const uint8_t*)L->gate_shexp, (const uint8_t*)L->up_shexp, X, ws, d,
                            N, nb_r, nb_s);
