@@ -183,8 +183,38 @@ __global__ __launch_bounds__(1024) void moe_select_group_kernel(MoeWs ws, qkk_se
     }
 }
 
-void moe_mfma_launch(const qkk_moe_layer* L, const float* X, float* Y, const qkk_sel* sel, const MoeWs& ws,
-                     const MoeDims& d, uint32_t N, uint32_t stages, hipStream_t st);
+void moe_mfma_launch_shared(const qkk_moe_layer* L, const float* X, const qkk_sel* sel, const MoeWs& ws,
+                            const MoeDims& d, uint32_t N, uint32_t stages, hipStream_t st);
+void moe_mfma_launch_routed(const qkk_moe_layer* L, const float* X, const qkk_sel* sel, const MoeWs& ws,
+                            const MoeDims& d, uint32_t N, uint32_t stages, hipStream_t st);
+void moe_mfma_launch_fold(float* Y, const qkk_sel* sel, const MoeWs& ws, const MoeDims& d, uint32_t N, hipStream_t st);
+void moe_mfma_launch_fused(const qkk_moe_layer* L, const float* X, const qkk_sel* sel, const MoeWs& ws,
+                           const MoeDims& d, uint32_t N, uint32_t stages, hipStream_t st);
+constexpr uint32_t FUSED_MAX_ROWS = 32; // up to here the shared expert rides in the routed experts' launches
+
+// The shared expert's chain runs on a side stream of the library, forked from and joined back into
+// the caller's stream with events (capturable: under stream capture the side stream joins the
+// caller's graph).  One per device, created on first use, default priority.
+struct SideStream {
+    hipStream_t stream = nullptr;
+    hipEvent_t fork = nullptr, join = nullptr;
+};
+static SideStream* side_stream()
+{
+    static SideStream per_device[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    SideStream& s = per_device[dev];
+    if (!s.stream) {
+        if (hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking) != hipSuccess ||
+            hipEventCreateWithFlags(&s.fork, hipEventDisableTiming) != hipSuccess ||
+            hipEventCreateWithFlags(&s.join, hipEventDisableTiming) != hipSuccess) {
+            s.stream = nullptr;
+            return nullptr;
+        }
+    }
+    return &s;
+}
 
 // Host entry of the path for N >= 2 rows (arguments already validated).
 int moe_grouped_launch(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* sel, void* workspace,
@@ -194,6 +224,18 @@ int moe_grouped_launch(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel
     // the matrix-core kernels split n_embd over the eight waves of a workgroup, 256 weights each
     if (d.H != 2048) return fail(QKK_ESHAPE, "moe: several rows need n_embd = 2048 (got %u)", d.H);
     const MoeWs ws = ws_carve(workspace, d, N);
+    const uint32_t experts_stages = stages & (QKK_STAGE_GATEUP | QKK_STAGE_DOWN);
+    const bool split = N > FUSED_MAX_ROWS;
+    // fork: the shared expert needs only X (and its own h), so it starts right away
+    SideStream* side = experts_stages && split ? side_stream() : nullptr;
+    if (experts_stages && split) {
+        if (side && hipEventRecord(side->fork, st) == hipSuccess && hipStreamWaitEvent(side->stream, side->fork, 0) == hipSuccess)
+            moe_mfma_launch_shared(L, X, sel, ws, d, N, stages, side->stream);
+        else {
+            side = nullptr; // no side stream: same work, in line
+            moe_mfma_launch_shared(L, X, sel, ws, d, N, stages, st);
+        }
+    }
     if (stages & QKK_STAGE_ROUTE) {
         const uint32_t inline_sel = N <= SELECT_INLINE_MAX ? 1u : 0u;
         const uint32_t tasks = (d.E + 1) * ((N + 3) / 4);
@@ -201,7 +243,15 @@ int moe_grouped_launch(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel
                            L->gate_inp_shexp, X, ws, sel, d, N, inline_sel);
         if (!inline_sel) hipLaunchKernelGGL(moe_select_group_kernel, dim3((N + 15) / 16), dim3(1024), 0, st, ws, sel, d, N);
     }
-    moe_mfma_launch(L, X, Y, sel, ws, d, N, stages, st);
+    if (experts_stages) {
+        if (split) moe_mfma_launch_routed(L, X, sel, ws, d, N, stages, st);
+        else moe_mfma_launch_fused(L, X, sel, ws, d, N, stages, st);
+    }
+    if (side) { // join
+        if (hipEventRecord(side->join, side->stream) != hipSuccess || hipStreamWaitEvent(st, side->join, 0) != hipSuccess)
+            return fail(QKK_EDEVICE, "moe: joining the shared-expert stream failed");
+    }
+    if (stages & QKK_STAGE_DOWN) moe_mfma_launch_fold(Y, sel, ws, d, N, st);
     return check_launch("moe grouped path");
 }
 

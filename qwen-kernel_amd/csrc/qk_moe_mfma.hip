@@ -18,24 +18,182 @@
 
 namespace qk {
 
-// Work items: first the shared expert's tiles of 16 consecutive tokens (one dense expert for
-// every token: its items are the long ones, so they start first), then the routed experts with
-// their pair lists.  Every item is cut into sub-items of `nb` batches of weight rows, so one
-// expert's rows are streamed by several workgroups (each loads the activation rows itself).
+// Work items.  The shared expert is one dense expert for every token: its items are tiles of 16
+// consecutive tokens; it depends on nothing the router produces, so its launches run on a side
+// stream next to the router and the routed experts.  A routed item is one active expert with its
+// pair list.  Every item is cut into sub-items of `nb` batches of weight rows, so one expert's
+// rows are streamed by several workgroups (each loads the activation rows itself).
 struct Item {
+    uint32_t expert, first, count; // routed: pairs [first, first+count) of ws.pairs; shared: tokens
+    uint32_t sub;
+};
+
+template <bool SHARED>
+__device__ __forceinline__ uint32_t item_count(const MoeWs& ws, uint32_t N, uint32_t subs)
+{
+    return (SHARED ? (N + 15) / 16 : *ws.n_active) * subs;
+}
+
+template <bool SHARED>
+__device__ __forceinline__ Item get_item(const MoeWs& ws, uint32_t index, uint32_t subs, uint32_t N)
+{
+    Item it;
+    const uint32_t w = index / subs;
+    it.sub = index % subs;
+    if (SHARED) {
+        it.expert = 0; it.first = w * 16u; it.count = min(16u, N - it.first);
+    } else {
+        const ActiveExpert a = ws.active[w];
+        it.expert = a.expert; it.first = a.first; it.count = a.count;
+    }
+    return it;
+}
+
+// rows of the staged tile: s_tok[r] = token, s_slot[r] = h / contrib slot (k = shared expert)
+template <bool SHARED>
+__device__ __forceinline__ void stage_pairs(const MoeWs& ws, const Item& it, uint32_t t0, uint32_t np, uint32_t k,
+                                            uint32_t* s_tok, uint32_t* s_slot, int tid)
+{
+    if (tid < 16) {
+        uint32_t tok = 0, slot = 0;
+        if ((uint32_t)tid < np) {
+            if (SHARED) { tok = it.first + tid; slot = k; }
+            else { const uint32_t pr = ws.pairs[it.first + t0 + tid]; tok = pr >> 4; slot = pr & 15u; }
+        }
+        s_tok[tid] = tok;
+        s_slot[tid] = slot;
+    }
+}
+
+// ---- gate/up + SiLU --------------------------------------------------------------------------------
+// n_embd = 2048: the eight waves take one 256-weight fragment each.  A batch is one row tile; the
+// gate tile and the up tile of the same rows take turns (ALT), which keeps the routed kernel at
+// 121 VGPRs and 41 KB of LDS: two workgroups per CU.
+template <bool SHARED>
+using GuGeo = CoopGeom<SHARED ? QKK_Q8_0 : QKK_IQ3_XXS, 8, 2, 1, true>;
+
+template <bool SHARED>
+__global__ __launch_bounds__(CT, SHARED ? 2 : 4) void moe_gateup_mfma_kernel(const uint8_t* __restrict__ gate,
+                                                                             const uint8_t* __restrict__ up,
+                                                                             const float* __restrict__ X, MoeWs ws,
+                                                                             MoeDims d, uint32_t N, uint32_t nb)
+{
+    using Geo = GuGeo<SHARED>;
+    constexpr int TYPE = SHARED ? QKK_Q8_0 : QKK_IQ3_XXS;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    __shared__ MfmaTables tab;
+    __shared__ uint32_t s_tok[16], s_slot[16];
+    const int tid = threadIdx.x;
+    const uint32_t F = d.F, H = d.H;
+    fill_mfma_tables(tab, tid, CT);
+    const uint32_t subs = F / (16 * Geo::BT * nb);
+    const uint32_t n_items = item_count<SHARED>(ws, N, subs);
+
+    for (uint32_t w = blockIdx.x; w < n_items; w += gridDim.x) {
+        const Item it = get_item<SHARED>(ws, w, subs, N);
+        const uint32_t row0 = it.sub * nb * Geo::BT * 16;
+        const size_t off = ((size_t)it.expert * F + row0) * Geo::RB;
+        for (uint32_t t0 = 0; t0 < it.count; t0 += 16) {
+            const uint32_t np = min(16u, it.count - t0);
+            __syncthreads(); // previous tile fully consumed
+            stage_pairs<SHARED>(ws, it, t0, np, d.k, s_tok, s_slot, tid);
+            __syncthreads();
+            coop_stream<TYPE, 8, 2, 1, true, false>(gate + off, up + off, nb, X, H, np, [&](uint32_t r) { return s_tok[r]; },
+                smem, tab, tid, [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1, uint32_t) {
+                    const uint32_t r = 4 * (ln >> 4) + e;
+                    if (r < np)
+                        ws.h[((size_t)s_tok[r] * (d.k + 1) + s_slot[r]) * F + row0 + tile * 16 + (ln & 15u)] =
+                            (sum0 / (1.f + expf(-sum0))) * sum1;
+                });
+        }
+    }
+}
+
+// ---- down: per-pair contributions -----------------------------------------------------------------
+// contrib[(token*(k+1) + slot)*H + o] = weight * (D[o] . h[token][slot]) for the routed slots; slot k
+// (shared expert) holds the unweighted product, its sigmoid gate is applied by the fold (so the
+// shared expert does not wait for the router).  K = F = 256*FB: FB waves split K, 8/FB tile groups
+// split the batch's tiles.
+template <int TYPE, int FB>
+using DnGeo = CoopGeom<TYPE, FB, 1, (TYPE == QKK_IQ4_XS ? 2 : 1)>;
+
+template <int TYPE, int FB, bool SHARED>
+__global__ __launch_bounds__(CT) void moe_down_mfma_kernel(const uint8_t* __restrict__ down, MoeWs ws,
+                                                           const qkk_sel* __restrict__ sel, MoeDims d, uint32_t N,
+                                                           uint32_t nb)
+{
+    using Geo = DnGeo<TYPE, FB>;
+    constexpr int TG = TYPE == QKK_IQ4_XS ? 2 : 1;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    __shared__ MfmaTables tab;
+    __shared__ uint32_t s_tok[16], s_slot[16];
+    __shared__ float s_wt[16];
+    const int tid = threadIdx.x;
+    const uint32_t F = d.F, H = d.H;
+    fill_mfma_tables(tab, tid, CT);
+    const uint32_t subs = H / (16 * Geo::BT * nb);
+    const uint32_t n_items = item_count<SHARED>(ws, N, subs);
+
+    for (uint32_t w = blockIdx.x; w < n_items; w += gridDim.x) {
+        const Item it = get_item<SHARED>(ws, w, subs, N);
+        const uint32_t row0 = it.sub * nb * Geo::BT * 16;
+        const uint8_t* base = down + ((size_t)it.expert * H + row0) * Geo::RB;
+        for (uint32_t t0 = 0; t0 < it.count; t0 += 16) {
+            const uint32_t np = min(16u, it.count - t0);
+            __syncthreads();
+            stage_pairs<SHARED>(ws, it, t0, np, d.k, s_tok, s_slot, tid);
+            __syncthreads();
+            if (tid < 16) s_wt[tid] = (SHARED || (uint32_t)tid >= np) ? 1.f : sel[s_tok[tid]].w[s_slot[tid]];
+            __syncthreads();
+            coop_stream<TYPE, FB, 1, TG, false, false>(base, nullptr, nb, ws.h, F, np,
+                [&](uint32_t r) { return s_tok[r] * (d.k + 1) + s_slot[r]; }, smem, tab, tid,
+                [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float, uint32_t) {
+                    const uint32_t r = 4 * (ln >> 4) + e;
+                    if (r < np)
+                        ws.contrib[((size_t)s_tok[r] * (d.k + 1) + s_slot[r]) * H + row0 + tile * 16 + (ln & 15u)] =
+                            s_wt[r] * sum0;
+                });
+        }
+    }
+}
+
+// ---- fold: Y[t][o] = sum over the k routed slots in slot order + shared gate * shared slot ---------------
+__global__ __launch_bounds__(256) void moe_fold_kernel(MoeWs ws, const qkk_sel* __restrict__ sel,
+                                                       float* __restrict__ Y, MoeDims d, uint32_t N)
+{
+    const uint32_t quads = d.H / 4;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < (size_t)N * quads; i += (size_t)gridDim.x * 256) {
+        const uint32_t t = (uint32_t)(i / quads), o = (uint32_t)(i % quads) * 4;
+        float4 s = float4{0.f, 0.f, 0.f, 0.f};
+        for (uint32_t sl = 0; sl < d.k; sl++) {
+            const float4 c = *(const float4*)(ws.contrib + ((size_t)t * (d.k + 1) + sl) * d.H + o);
+            s.x += c.x; s.y += c.y; s.z += c.z; s.w += c.w;
+        }
+        const float g = sel[t].w_shared;
+        const float4 c = *(const float4*)(ws.contrib + ((size_t)t * (d.k + 1) + d.k) * d.H + o);
+        s.x += g * c.x; s.y += g * c.y; s.z += g * c.z; s.w += g * c.w;
+        *(float4*)(Y + (size_t)t * d.H + o) = s;
+    }
+}
+
+// ==== few rows (up to FUSED_MAX_ROWS): one gate/up and one down launch take the shared expert's and
+// the routed experts' items together (a HIP graph runs the side stream's launches of so short a
+// step one after the other, which costs more than it saves).  Items: first the shared expert's
+// tiles, then the routed experts.
+struct ItemF {
     bool shared;
     uint32_t expert, first, count; // routed: pairs [first, first+count) of ws.pairs; shared: tokens
     uint32_t sub;
 };
 
-__device__ __forceinline__ uint32_t item_count(uint32_t n_active, uint32_t N, uint32_t subs_shared, uint32_t subs)
+__device__ __forceinline__ uint32_t item_count_f(uint32_t n_active, uint32_t N, uint32_t subs_shared, uint32_t subs)
 {
     return (N + 15) / 16 * subs_shared + n_active * subs;
 }
 
-__device__ __forceinline__ Item get_item(const MoeWs& ws, uint32_t index, uint32_t subs_shared, uint32_t subs, uint32_t N)
+__device__ __forceinline__ ItemF get_item_f(const MoeWs& ws, uint32_t index, uint32_t subs_shared, uint32_t subs, uint32_t N)
 {
-    Item it;
+    ItemF it;
     const uint32_t n_sh = (N + 15) / 16 * subs_shared;
     if (index < n_sh) {
         it.sub = index % subs_shared;
@@ -52,13 +210,13 @@ __device__ __forceinline__ Item get_item(const MoeWs& ws, uint32_t index, uint32
 // ---- gate/up + SiLU --------------------------------------------------------------------------------
 // n_embd = 2048: the eight waves take one 256-weight fragment each.  Routed experts: batches of
 // one row tile of gate and of up (IQ3_XXS); shared expert (Q8_0): one row tile, gate and up in turns.
-constexpr int GU_TG_R = 1, GU_TG_S = 1;
-constexpr int GU_PB = 2; // partial buffers (2: one barrier per batch)
-using GuGeoR = CoopGeom<QKK_IQ3_XXS, 8, 2, GU_TG_R, false, 1, GU_PB>;
-using GuGeoS = CoopGeom<QKK_Q8_0, 8, 2, GU_TG_S, true, 1, GU_PB>;
-constexpr uint32_t GU_LDS = GuGeoR::LDS_BYTES > GuGeoS::LDS_BYTES ? GuGeoR::LDS_BYTES : GuGeoS::LDS_BYTES;
+constexpr int FU_TG_R = 1, FU_TG_S = 1;
+constexpr int FU_PB = 2; // partial buffers (2: one barrier per batch)
+using FuGeoR = CoopGeom<QKK_IQ3_XXS, 8, 2, FU_TG_R, false, 1, FU_PB>;
+using FuGeoS = CoopGeom<QKK_Q8_0, 8, 2, FU_TG_S, true, 1, FU_PB>;
+constexpr uint32_t FU_LDS = FuGeoR::LDS_BYTES > FuGeoS::LDS_BYTES ? FuGeoR::LDS_BYTES : FuGeoS::LDS_BYTES;
 
-__global__ __launch_bounds__(CT) void moe_gateup_mfma_kernel(const uint8_t* __restrict__ gate_exps,
+__global__ __launch_bounds__(CT) void moe_gateup_fused_kernel(const uint8_t* __restrict__ gate_exps,
                                                              const uint8_t* __restrict__ up_exps,
                                                              const uint8_t* __restrict__ gate_shexp,
                                                              const uint8_t* __restrict__ up_shexp,
@@ -72,11 +230,11 @@ __global__ __launch_bounds__(CT) void moe_gateup_mfma_kernel(const uint8_t* __re
     const uint32_t F = d.F, H = d.H;
     fill_mfma_tables(tab, tid, CT);
     const uint32_t n_active = *ws.n_active;
-    const uint32_t subs_sh = F / (16 * GuGeoS::BT * nb_s), subs = F / (16 * GuGeoR::BT * nb_r);
-    const uint32_t n_items = item_count(n_active, N, subs_sh, subs);
+    const uint32_t subs_sh = F / (16 * FuGeoS::BT * nb_s), subs = F / (16 * FuGeoR::BT * nb_r);
+    const uint32_t n_items = item_count_f(n_active, N, subs_sh, subs);
 
     for (uint32_t w = blockIdx.x; w < n_items; w += gridDim.x) {
-        const Item it = get_item(ws, w, subs_sh, subs, N);
+        const ItemF it = get_item_f(ws, w, subs_sh, subs, N);
         for (uint32_t t0 = 0; t0 < it.count; t0 += 16) {
             const uint32_t np = it.shared ? it.count : min(16u, it.count - t0);
             __syncthreads(); // previous tile fully consumed
@@ -92,8 +250,8 @@ __global__ __launch_bounds__(CT) void moe_gateup_mfma_kernel(const uint8_t* __re
             __syncthreads();
             const auto row_of = [&](uint32_t r) { return s_tok[r]; };
             if (it.shared) {
-                const uint32_t row0 = it.sub * nb_s * GuGeoS::BT * 16;
-                coop_stream<QKK_Q8_0, 8, 2, GU_TG_S, true, false, 1, GU_PB>(gate_shexp + (size_t)row0 * GuGeoS::RB, up_shexp + (size_t)row0 * GuGeoS::RB, nb_s, X, H, np, row_of, smem, tab, tid,
+                const uint32_t row0 = it.sub * nb_s * FuGeoS::BT * 16;
+                coop_stream<QKK_Q8_0, 8, 2, FU_TG_S, true, false, 1, FU_PB>(gate_shexp + (size_t)row0 * FuGeoS::RB, up_shexp + (size_t)row0 * FuGeoS::RB, nb_s, X, H, np, row_of, smem, tab, tid,
                     [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1, uint32_t) {
                         const uint32_t r = 4 * (ln >> 4) + e;
                         if (r < np)
@@ -102,9 +260,9 @@ __global__ __launch_bounds__(CT) void moe_gateup_mfma_kernel(const uint8_t* __re
                     });
                 break;
             }
-            const uint32_t row0 = it.sub * nb_r * GuGeoR::BT * 16;
-            const size_t eo = ((size_t)it.expert * F + row0) * GuGeoR::RB;
-            coop_stream<QKK_IQ3_XXS, 8, 2, GU_TG_R, false, false, 1, GU_PB>(gate_exps + eo, up_exps + eo, nb_r, X, H, np, row_of, smem, tab, tid,
+            const uint32_t row0 = it.sub * nb_r * FuGeoR::BT * 16;
+            const size_t eo = ((size_t)it.expert * F + row0) * FuGeoR::RB;
+            coop_stream<QKK_IQ3_XXS, 8, 2, FU_TG_R, false, false, 1, FU_PB>(gate_exps + eo, up_exps + eo, nb_r, X, H, np, row_of, smem, tab, tid,
                 [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1, uint32_t) {
                     const uint32_t r = 4 * (ln >> 4) + e;
                     if (r < np)
@@ -119,7 +277,7 @@ __global__ __launch_bounds__(CT) void moe_gateup_mfma_kernel(const uint8_t* __re
 // contrib[(token*(k+1) + slot)*H + o] = weight * (D[o] . h[token][slot]); slot k = shared expert.
 // K = F = 256*FB: FB waves split K, 8/FB tile groups split the batch's tiles.
 template <int TYPE_DN, int FB>
-struct DnGeo {
+struct DnGeoF {
     static constexpr int TG_R = TYPE_DN == QKK_Q6_K ? 1 : 2, TG_S = 1;
     using R = CoopGeom<TYPE_DN, FB, 1, TG_R>;
     using S = CoopGeom<QKK_Q8_0, FB, 1, TG_S>;
@@ -127,12 +285,12 @@ struct DnGeo {
 };
 
 template <int TYPE_DN, int FB>
-__global__ __launch_bounds__(CT) void moe_down_mfma_kernel(const uint8_t* __restrict__ down_exps,
+__global__ __launch_bounds__(CT) void moe_down_fused_kernel(const uint8_t* __restrict__ down_exps,
                                                            const uint8_t* __restrict__ down_shexp, MoeWs ws,
                                                            const qkk_sel* __restrict__ sel, MoeDims d, uint32_t N,
                                                            uint32_t nb_r, uint32_t nb_s)
 {
-    using Geo = DnGeo<TYPE_DN, FB>;
+    using Geo = DnGeoF<TYPE_DN, FB>;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ MfmaTables tab;
     __shared__ uint32_t s_tok[16], s_slot[16];
@@ -142,10 +300,10 @@ __global__ __launch_bounds__(CT) void moe_down_mfma_kernel(const uint8_t* __rest
     fill_mfma_tables(tab, tid, CT);
     const uint32_t n_active = *ws.n_active;
     const uint32_t subs_sh = H / (16 * Geo::S::BT * nb_s), subs = H / (16 * Geo::R::BT * nb_r);
-    const uint32_t n_items = item_count(n_active, N, subs_sh, subs);
+    const uint32_t n_items = item_count_f(n_active, N, subs_sh, subs);
 
     for (uint32_t w = blockIdx.x; w < n_items; w += gridDim.x) {
-        const Item it = get_item(ws, w, subs_sh, subs, N);
+        const ItemF it = get_item_f(ws, w, subs_sh, subs, N);
         for (uint32_t t0 = 0; t0 < it.count; t0 += 16) {
             const uint32_t np = it.shared ? it.count : min(16u, it.count - t0);
             __syncthreads();
@@ -153,7 +311,7 @@ __global__ __launch_bounds__(CT) void moe_down_mfma_kernel(const uint8_t* __rest
                 uint32_t tok = 0, slot = 0;
                 float wt = 0.f;
                 if ((uint32_t)tid < np) {
-                    if (it.shared) { tok = it.first + tid; slot = d.k; wt = sel[tok].w_shared; }
+                    if (it.shared) { tok = it.first + tid; slot = d.k; wt = 1.f; } // gate applied by the fold
                     else {
                         const uint32_t pr = ws.pairs[it.first + t0 + tid];
                         tok = pr >> 4; slot = pr & 15u; wt = sel[tok].w[slot];
@@ -186,84 +344,126 @@ __global__ __launch_bounds__(CT) void moe_down_mfma_kernel(const uint8_t* __rest
     }
 }
 
-// ---- fold: Y[t][o] = sum over the k+1 slots, in slot order --------------------------------------------
-__global__ __launch_bounds__(256) void moe_fold_kernel(MoeWs ws, float* __restrict__ Y, MoeDims d, uint32_t N)
-{
-    const uint32_t quads = d.H / 4;
-    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < (size_t)N * quads; i += (size_t)gridDim.x * 256) {
-        const uint32_t t = (uint32_t)(i / quads), o = (uint32_t)(i % quads) * 4;
-        float4 s = float4{0.f, 0.f, 0.f, 0.f};
-        for (uint32_t sl = 0; sl <= d.k; sl++) {
-            const float4 c = *(const float4*)(ws.contrib + ((size_t)t * (d.k + 1) + sl) * d.H + o);
-            s.x += c.x; s.y += c.y; s.z += c.z; s.w += c.w;
-        }
-        *(float4*)(Y + (size_t)t * d.H + o) = s;
-    }
-}
-
 // ---- host -----------------------------------------------------------------------------------------------
-static void set_lds_attr(const void* fn, uint32_t bytes)
+// workgroups of `fn` that fit a CU at once (registers, LDS): one or two; also raises its LDS limit
+static uint32_t per_cu_of(const void* fn, uint32_t lds)
 {
-    (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    (void)hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    int n = 1;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, fn, CT, lds) != hipSuccess || n < 1) n = 1;
+    return (uint32_t)std::min(n, 2);
 }
 
 // batches per sub-item: the largest power of two <= total that still gives every CU about two items
-static uint32_t pick_nb(uint32_t total_batches, uint32_t experts)
+static uint32_t pick_nb(uint32_t total_batches, uint32_t items)
 {
     uint32_t nb = total_batches;
-    while (nb > 1 && (uint64_t)experts * (total_batches / nb) < 2ull * persistent_blocks() / 4) nb /= 2;
+    while (nb > 1 && (uint64_t)items * (total_batches / nb) < 2ull * persistent_blocks() / 4) nb /= 2;
     return nb;
 }
 
 template <int TYPE, int FB>
-static void launch_down(const qkk_moe_layer* L, const MoeWs& ws, const qkk_sel* sel, const MoeDims& d, uint32_t N,
-                        uint32_t experts, hipStream_t st)
+static void launch_down_fused(const qkk_moe_layer* L, const MoeWs& ws, const qkk_sel* sel, const MoeDims& d, uint32_t N,
+                              uint32_t experts, hipStream_t st)
 {
-    using Geo = DnGeo<TYPE, FB>;
-    static bool once = (set_lds_attr((const void*)moe_down_mfma_kernel<TYPE, FB>, Geo::LDS), true);
-    (void)once;
+    using Geo = DnGeoF<TYPE, FB>;
+    static const uint32_t per_cu = per_cu_of((const void*)moe_down_fused_kernel<TYPE, FB>, Geo::LDS);
+    (void)per_cu;
     const uint32_t tot_r = d.H / (16 * Geo::R::BT), tot_s = d.H / (16 * Geo::S::BT);
     const uint32_t nb_r = pick_nb(tot_r, experts), nb_s = std::min(tot_s, std::max(1u, nb_r * Geo::R::BT / Geo::S::BT / 2));
     const uint32_t items = experts * (tot_r / nb_r) + (N + 15) / 16 * (tot_s / nb_s);
-    const uint32_t blocks = std::min(items, persistent_blocks() / 4);
-    hipLaunchKernelGGL((moe_down_mfma_kernel<TYPE, FB>), dim3(blocks), dim3(CT), Geo::LDS, st,
-                       (const uint8_t*)L->down_exps, (const uint8_t*)L->down_shexp, ws, sel, d, N, nb_r, nb_s);
+    hipLaunchKernelGGL((moe_down_fused_kernel<TYPE, FB>), dim3(std::min(items, persistent_blocks() / 4)), dim3(CT), Geo::LDS,
+                       st, (const uint8_t*)L->down_exps, (const uint8_t*)L->down_shexp, ws, sel, d, N, nb_r, nb_s);
 }
 
-// Gate/up, down and fold for N >= 2 rows; the router record and the pair lists are in place.
-void moe_mfma_launch(const qkk_moe_layer* L, const float* X, float* Y, const qkk_sel* sel, const MoeWs& ws,
-                     const MoeDims& d, uint32_t N, uint32_t stages, hipStream_t st)
+// Gate/up and down for few rows: shared and routed items in one launch each.
+void moe_mfma_launch_fused(const qkk_moe_layer* L, const float* X, const qkk_sel* sel, const MoeWs& ws,
+                           const MoeDims& d, uint32_t N, uint32_t stages, hipStream_t st)
 {
     const uint32_t experts = (uint32_t)std::min<uint64_t>(d.E, (uint64_t)N * d.k); // upper bound of the active ones
     if (stages & QKK_STAGE_GATEUP) {
-        static const uint32_t per_cu = [] { // workgroups that fit a CU at once (registers, LDS)
-            set_lds_attr((const void*)moe_gateup_mfma_kernel, GU_LDS);
-            int n = 1;
-            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void*)moe_gateup_mfma_kernel, CT, GU_LDS) != hipSuccess || n < 1)
-                n = 1;
-            return (uint32_t)std::min(n, 2);
-        }();
-        const uint32_t tot_r = d.F / (16 * GuGeoR::BT), tot_s = d.F / (16 * GuGeoS::BT);
-        const uint32_t nb_r = pick_nb(tot_r, experts), nb_s = std::min(tot_s, std::max(1u, nb_r * GuGeoR::BT / GuGeoS::BT / 2));
+        static const uint32_t per_cu = per_cu_of((const void*)moe_gateup_fused_kernel, FU_LDS);
+        (void)per_cu;
+        const uint32_t tot_r = d.F / (16 * FuGeoR::BT), tot_s = d.F / (16 * FuGeoS::BT);
+        const uint32_t nb_r = pick_nb(tot_r, experts), nb_s = std::min(tot_s, std::max(1u, nb_r * FuGeoR::BT / FuGeoS::BT / 2));
         const uint32_t items = experts * (tot_r / nb_r) + (N + 15) / 16 * (tot_s / nb_s);
-        const uint32_t blocks = std::min(items, per_cu * (persistent_blocks() / 4));
-        hipLaunchKernelGGL(moe_gateup_mfma_kernel, dim3(blocks), dim3(CT), GU_LDS, st, (const uint8_t*)L->gate_exps,
-                           (const uint8_t*)L->up_exps, (const uint8_t*)L->gate_shexp, (const uint8_t*)L->up_shexp, X, ws, d,
-                           N, nb_r, nb_s);
+        hipLaunchKernelGGL(moe_gateup_fused_kernel, dim3(std::min(items, persistent_blocks() / 4)), dim3(CT), FU_LDS, st,
+                           (const uint8_t*)L->gate_exps, (const uint8_t*)L->up_exps, (const uint8_t*)L->gate_shexp,
+                           (const uint8_t*)L->up_shexp, X, ws, d, N, nb_r, nb_s);
     }
     if (stages & QKK_STAGE_DOWN) {
         if (L->down_type == QKK_IQ4_XS) {
-            if (d.F == 256) launch_down<QKK_IQ4_XS, 1>(L, ws, sel, d, N, experts, st);
-            else if (d.F == 512) launch_down<QKK_IQ4_XS, 2>(L, ws, sel, d, N, experts, st);
-            else launch_down<QKK_IQ4_XS, 4>(L, ws, sel, d, N, experts, st);
+            if (d.F == 256) launch_down_fused<QKK_IQ4_XS, 1>(L, ws, sel, d, N, experts, st);
+            else if (d.F == 512) launch_down_fused<QKK_IQ4_XS, 2>(L, ws, sel, d, N, experts, st);
+            else launch_down_fused<QKK_IQ4_XS, 4>(L, ws, sel, d, N, experts, st);
         } else {
-            if (d.F == 256) launch_down<QKK_Q6_K, 1>(L, ws, sel, d, N, experts, st);
-            else if (d.F == 512) launch_down<QKK_Q6_K, 2>(L, ws, sel, d, N, experts, st);
-            else launch_down<QKK_Q6_K, 4>(L, ws, sel, d, N, experts, st);
+            if (d.F == 256) launch_down_fused<QKK_Q6_K, 1>(L, ws, sel, d, N, experts, st);
+            else if (d.F == 512) launch_down_fused<QKK_Q6_K, 2>(L, ws, sel, d, N, experts, st);
+            else launch_down_fused<QKK_Q6_K, 4>(L, ws, sel, d, N, experts, st);
         }
-        const uint32_t fb = (uint32_t)std::min<uint64_t>(((uint64_t)N * d.H / 4 + 255) / 256, persistent_blocks());
-        hipLaunchKernelGGL(moe_fold_kernel, dim3(fb), dim3(256), 0, st, ws, Y, d, N);
     }
+}
+
+template <bool SHARED>
+static void launch_gateup(const qkk_moe_layer* L, const float* X, const MoeWs& ws, const MoeDims& d, uint32_t N,
+                          uint32_t items, hipStream_t st)
+{
+    using Geo = GuGeo<SHARED>;
+    static const uint32_t per_cu = per_cu_of((const void*)moe_gateup_mfma_kernel<SHARED>, Geo::LDS_BYTES);
+    const uint32_t tot = d.F / (16 * Geo::BT), nb = pick_nb(tot, items);
+    const uint32_t blocks = std::min(items * (tot / nb), per_cu * (persistent_blocks() / 4));
+    hipLaunchKernelGGL(moe_gateup_mfma_kernel<SHARED>, dim3(blocks), dim3(CT), Geo::LDS_BYTES, st,
+                       (const uint8_t*)(SHARED ? L->gate_shexp : L->gate_exps),
+                       (const uint8_t*)(SHARED ? L->up_shexp : L->up_exps), X, ws, d, N, nb);
+}
+
+template <int TYPE, int FB, bool SHARED>
+static void launch_down(const void* W, const MoeWs& ws, const qkk_sel* sel, const MoeDims& d, uint32_t N,
+                        uint32_t items, hipStream_t st)
+{
+    using Geo = DnGeo<TYPE, FB>;
+    static const uint32_t per_cu = per_cu_of((const void*)moe_down_mfma_kernel<TYPE, FB, SHARED>, Geo::LDS_BYTES);
+    const uint32_t tot = d.H / (16 * Geo::BT), nb = pick_nb(tot, items);
+    const uint32_t blocks = std::min(items * (tot / nb), per_cu * (persistent_blocks() / 4));
+    hipLaunchKernelGGL((moe_down_mfma_kernel<TYPE, FB, SHARED>), dim3(blocks), dim3(CT), Geo::LDS_BYTES, st,
+                       (const uint8_t*)W, ws, sel, d, N, nb);
+}
+
+template <int TYPE, bool SHARED>
+static void launch_down_f(const void* W, const MoeWs& ws, const qkk_sel* sel, const MoeDims& d, uint32_t N,
+                          uint32_t items, hipStream_t st)
+{
+    if (d.F == 256) launch_down<TYPE, 1, SHARED>(W, ws, sel, d, N, items, st);
+    else if (d.F == 512) launch_down<TYPE, 2, SHARED>(W, ws, sel, d, N, items, st);
+    else launch_down<TYPE, 4, SHARED>(W, ws, sel, d, N, items, st);
+}
+
+// The shared expert's launches of a step (side stream): gate/up, then down.
+void moe_mfma_launch_shared(const qkk_moe_layer* L, const float* X, const qkk_sel* sel, const MoeWs& ws,
+                            const MoeDims& d, uint32_t N, uint32_t stages, hipStream_t st)
+{
+    const uint32_t tiles = (N + 15) / 16;
+    if (stages & QKK_STAGE_GATEUP) launch_gateup<true>(L, X, ws, d, N, tiles, st);
+    if (stages & QKK_STAGE_DOWN) launch_down_f<QKK_Q8_0, true>(L->down_shexp, ws, sel, d, N, tiles, st);
+}
+
+// The routed experts' launches of a step; the router record and the pair lists are in place.
+void moe_mfma_launch_routed(const qkk_moe_layer* L, const float* X, const qkk_sel* sel, const MoeWs& ws,
+                            const MoeDims& d, uint32_t N, uint32_t stages, hipStream_t st)
+{
+    const uint32_t experts = (uint32_t)std::min<uint64_t>(d.E, (uint64_t)N * d.k); // upper bound of the active ones
+    if (stages & QKK_STAGE_GATEUP) launch_gateup<false>(L, X, ws, d, N, experts, st);
+    if (stages & QKK_STAGE_DOWN) {
+        if (L->down_type == QKK_IQ4_XS) launch_down_f<QKK_IQ4_XS, false>(L->down_exps, ws, sel, d, N, experts, st);
+        else launch_down_f<QKK_Q6_K, false>(L->down_exps, ws, sel, d, N, experts, st);
+    }
+}
+
+// Sum of the k+1 slots (after both chains).
+void moe_mfma_launch_fold(float* Y, const qkk_sel* sel, const MoeWs& ws, const MoeDims& d, uint32_t N, hipStream_t st)
+{
+    const uint32_t fb = (uint32_t)std::min<uint64_t>(((uint64_t)N * d.H / 4 + 255) / 256, persistent_blocks());
+    hipLaunchKernelGGL(moe_fold_kernel, dim3(fb), dim3(256), 0, st, ws, sel, Y, d, N);
 }
 
 } // namespace qk

@@ -52,6 +52,42 @@ def test_moe_prefill_small_layer_many_pairs_per_expert(qk, orc, dev):
     prefill_case(qk, orc, dev, hl, 96, seed=23)
 
 
+def test_moe_step_in_hip_graph_matches_eager(qk, dev):
+    """The many-row step forks the shared expert onto a side stream of the library and joins it back
+    with events: captured into a HIP graph it must replay to the eager result every time, with
+    eager work of the program between the replays; likewise the few-row step (no fork)."""
+    import torch
+    print("[case] moe step captured in a HIP graph, 40 and 5 rows", flush=True)
+    hl = qk.synth.HostLayer(seed=400, n_expert=32, n_used=4, down_type=qk.IQ4_XS)
+    layer = hl.to_device(dev)
+    for n in (40, 5):
+        rng = np.random.default_rng(50 + n)
+        Xs = [torch.from_numpy(rng.standard_normal((n, 2048)).astype(np.float32)).to(dev) for _ in range(3)]
+        ws = torch.zeros(qk.moe_workspace_bytes(layer, n), dtype=torch.uint8, device=dev)
+        eager = []
+        for X in Xs:
+            Y, sel = qk.moe_decode(layer, X, ws)
+            torch.cuda.synchronize()
+            eager.append((Y.clone(), sel.clone()))
+        Xg = Xs[0].clone()
+        Yg = torch.empty_like(Xg)
+        selg = torch.zeros((n, 160), dtype=torch.uint8, device=dev)
+        side = torch.cuda.Stream()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            qk.moe_decode(layer, Xg, ws, Yg, selg)
+        torch.cuda.synchronize()
+        for rep in range(6):
+            i = rep % 3
+            Xg.copy_(Xs[i])
+            scratch = (Xs[i] * 2).sum()      # unrelated eager work between replays
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(Yg, eager[i][0]), (n, rep)
+            assert torch.equal(selg, eager[i][1]), (n, rep)
+            assert torch.isfinite(scratch)
+
+
 @pytest.mark.parametrize("M,K,N", [(8192, 2048, 128), (100, 96, 5), (64, 32, 33), (130, 2048, 200), (4096, 4096, 48),
                                    (300, 256, 40), (96, 512, 64), (1000, 1024, 17), (17, 2048, 8), (2048, 2048, 7),
                                    (7, 64, 1), (1024, 512, 16)])
