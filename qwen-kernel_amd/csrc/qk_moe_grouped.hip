@@ -164,6 +164,50 @@ __global__ __launch_bounds__(512) void moe_route_multi_kernel(const float* __res
     }
 }
 
+// ---- router logits for many tokens --------------------------------------------------------------
+// Workgroup = 8 router rows x 16 tokens: the 16 activation rows are staged in LDS once and every
+// wave holds one router row in registers, so a row and an activation row cross the L1 once per
+// workgroup instead of once per dot product.  Same arithmetic, in the same order, as
+// moe_route_multi_kernel: a token's logits do not depend on how many tokens ride along.
+constexpr uint32_t LOGITS_TILE_TOKENS = 16;
+__global__ __launch_bounds__(512) void moe_logits_tiled_kernel(const float* __restrict__ gate_inp,
+                                                               const float* __restrict__ gate_inp_shexp,
+                                                               const float* __restrict__ X, MoeWs ws, MoeDims d,
+                                                               uint32_t N)
+{
+    extern __shared__ __attribute__((aligned(16))) float s_x[]; // [16][2048]
+    constexpr int NCH = 8;                                      // n_embd = 2048: eight float4 per lane
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t n_rows = d.E + 1, rgroups = (n_rows + 7) / 8;
+    const uint32_t r = (blockIdx.x % rgroups) * 8 + wave, t0 = (blockIdx.x / rgroups) * LOGITS_TILE_TOKENS;
+    const uint32_t nt = min(LOGITS_TILE_TOKENS, N - t0);
+    const uint32_t LS = lstride(d.E);
+
+    const float4* xs = (const float4*)(X + (size_t)t0 * 2048); // nt consecutive rows: one contiguous range
+    float4 xv[LOGITS_TILE_TOKENS];
+#pragma unroll
+    for (uint32_t i = 0; i < LOGITS_TILE_TOKENS; i++) xv[i] = xs[min(threadIdx.x + 512 * i, nt * 512 - 1)];
+    float4 w[NCH];
+    const float4* row = (const float4*)(r < d.E ? gate_inp + (size_t)r * 2048 : gate_inp_shexp);
+#pragma unroll
+    for (int i = 0; i < NCH; i++) w[i] = row[lane + 64 * i];
+#pragma unroll
+    for (uint32_t i = 0; i < LOGITS_TILE_TOKENS; i++) ((float4*)s_x)[threadIdx.x + 512 * i] = xv[i];
+    __syncthreads();
+    if (r >= n_rows) return;
+    for (uint32_t t = 0; t < nt; t++) {
+        float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const float4 x = ((const float4*)s_x)[t * 512 + lane + 64 * i];
+            a0 += w[i].x * x.x + w[i].y * x.y;
+            a1 += w[i].z * x.z + w[i].w * x.w;
+        }
+        const float sum = wave_sum(a0 + a1);
+        if (lane == 0) ws.logits[(size_t)(t0 + t) * LS + r] = sum;
+    }
+}
+
 // Selection + grouping as a launch of its own (many tokens): one token per wave, sixteen per
 // workgroup; the workgroup that finishes last groups the pairs.
 __global__ __launch_bounds__(1024) void moe_select_group_kernel(MoeWs ws, qkk_sel* __restrict__ sel, MoeDims d,
@@ -237,11 +281,20 @@ int moe_grouped_launch(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel
         }
     }
     if (stages & QKK_STAGE_ROUTE) {
-        const uint32_t inline_sel = N <= SELECT_INLINE_MAX ? 1u : 0u;
-        const uint32_t tasks = (d.E + 1) * ((N + 3) / 4);
-        hipLaunchKernelGGL(moe_route_multi_kernel<8>, dim3((tasks + 7) / 8), dim3(512), 0, st, L->gate_inp,
-                           L->gate_inp_shexp, X, ws, sel, d, N, inline_sel);
-        if (!inline_sel) hipLaunchKernelGGL(moe_select_group_kernel, dim3((N + 15) / 16), dim3(1024), 0, st, ws, sel, d, N);
+        if (N <= SELECT_INLINE_MAX) { // logits, and selection + grouping in the last workgroup
+            const uint32_t tasks = (d.E + 1) * ((N + 3) / 4);
+            hipLaunchKernelGGL(moe_route_multi_kernel<8>, dim3((tasks + 7) / 8), dim3(512), 0, st, L->gate_inp,
+                               L->gate_inp_shexp, X, ws, sel, d, N, 1u);
+        } else { // tiled logits, then selection one token per wave + grouping
+            constexpr uint32_t lds = LOGITS_TILE_TOKENS * 2048 * sizeof(float);
+            static bool once = ((void)hipFuncSetAttribute((const void*)moe_logits_tiled_kernel,
+                                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
+            (void)once;
+            const uint32_t grid = (d.E + 1 + 7) / 8 * ((N + LOGITS_TILE_TOKENS - 1) / LOGITS_TILE_TOKENS);
+            hipLaunchKernelGGL(moe_logits_tiled_kernel, dim3(grid), dim3(512), lds, st, L->gate_inp, L->gate_inp_shexp, X,
+                               ws, d, N);
+            hipLaunchKernelGGL(moe_select_group_kernel, dim3((N + 15) / 16), dim3(1024), 0, st, ws, sel, d, N);
+        }
     }
     if (experts_stages) {
         if (split) moe_mfma_launch_routed(L, X, sel, ws, d, N, stages, st);
