@@ -54,6 +54,9 @@ class Graphed:
         import torch
         self.n = len(launches)
         self.stream = torch.cuda.Stream()
+        # the tensors were filled (and the workspace cleared) on the current stream: without this
+        # the warm-up below can start on memory those launches have not written yet
+        self.stream.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(self.stream):
             for f in launches:  # eager warm-up (also first-touch of every buffer)
                 f()

@@ -110,8 +110,12 @@ size_t qkk_moe_workspace_bytes(const qkk_moe_layer *L_host, uint32_t n_slots);
  *   Y   [n_slots][n_embd]          out: routed + shared contribution (no residual)
  *   sel [n_slots]                  out: picks in pick order, weights, shared gate
  *   workspace                      qkk_moe_workspace_bytes(), 256-byte aligned, must be
- *                                  zero-filled once before its first use; calls sharing
- *                                  a workspace must not overlap in time.
+ *                                  zero-filled once before its first use (a fill issued on
+ *                                  another stream must have completed, or `stream` must wait
+ *                                  for it); calls sharing a workspace must not overlap in
+ *                                  time.  A workspace that breaks this gives wrong results,
+ *                                  never an access outside the tensors: the kernels clamp
+ *                                  every index they take from it.
  * With n_slots >= 2 every picked expert's weights are read once per 16 rows that picked it
  * (matrix-core path); that path needs n_embd = 2048 and returns QKK_ESHAPE otherwise. */
 int qkk_moe_decode(const qkk_moe_layer *L_host, const float *X, float *Y, qkk_sel *sel,

@@ -59,6 +59,32 @@ static inline MoeWs ws_carve(void* ws, const MoeDims& d, uint32_t n)
     return w;
 }
 
+// ---- what the grouping left in the workspace, bounded by the shapes ------------------------------
+// The expert kernels index tensors with these words.  A workspace that holds something else (first
+// 256 bytes never cleared, a gate/up or down stage run before any routing, another stream still
+// writing it) must give wrong numbers, never an access outside the tensors: every word is clamped
+// to its range on the way in.
+__device__ __forceinline__ uint32_t active_count(const MoeWs& ws, const MoeDims& d) { return min(*ws.n_active, d.E); }
+
+__device__ __forceinline__ ActiveExpert active_expert(const MoeWs& ws, uint32_t w, const MoeDims& d, uint32_t N)
+{
+    ActiveExpert a = ws.active[w]; // w < active_count() <= E
+    const uint32_t np = N * d.k;
+    a.expert = min(a.expert, d.E - 1);
+    a.first = min(a.first, np);
+    a.count = min(a.count, np - a.first);
+    return a;
+}
+
+// pair p of ws.pairs -> (token, pick)
+__device__ __forceinline__ void pair_at(const MoeWs& ws, uint32_t p, const MoeDims& d, uint32_t N, uint32_t& tok,
+                                        uint32_t& slot)
+{
+    const uint32_t pr = ws.pairs[p];
+    tok = min(pr >> 4, N - 1);
+    slot = min(pr & 15u, d.k - 1);
+}
+
 // ---- selector --------------------------------------------------------------------------
 // One wave; lane L owns logits L, L+64, ...  Picks n_used times the maximum, lower id on
 // ties; non-finite logits count as -3.4e38 (reference shaders/moe_select.comp:28-34, 53-63).

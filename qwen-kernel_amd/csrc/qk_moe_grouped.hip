@@ -103,7 +103,7 @@ __device__ static void group_pairs_wg(const MoeWs& ws, qkk_sel* __restrict__ sel
     for (uint32_t p = threadIdx.x; p < np; p += NW * 64) {
         const uint32_t t = p / d.k, s = p % d.k;
         const uint32_t e = min(vs[t].ids[s], d.E - 1);
-        ws.pairs[atomicAdd(&s_cur[e], 1u)] = (t << 4) | s;
+        ws.pairs[min(atomicAdd(&s_cur[e], 1u), np - 1)] = (t << 4) | s; // in range even if sel changes under us
     }
 }
 

@@ -29,13 +29,13 @@ struct Item {
 };
 
 template <bool SHARED>
-__device__ __forceinline__ uint32_t item_count(const MoeWs& ws, uint32_t N, uint32_t subs)
+__device__ __forceinline__ uint32_t item_count(const MoeWs& ws, const MoeDims& d, uint32_t N, uint32_t subs)
 {
-    return (SHARED ? (N + 15) / 16 : *ws.n_active) * subs;
+    return (SHARED ? (N + 15) / 16 : active_count(ws, d)) * subs;
 }
 
 template <bool SHARED>
-__device__ __forceinline__ Item get_item(const MoeWs& ws, uint32_t index, uint32_t subs, uint32_t N)
+__device__ __forceinline__ Item get_item(const MoeWs& ws, uint32_t index, uint32_t subs, const MoeDims& d, uint32_t N)
 {
     Item it;
     const uint32_t w = index / subs;
@@ -43,7 +43,7 @@ __device__ __forceinline__ Item get_item(const MoeWs& ws, uint32_t index, uint32
     if (SHARED) {
         it.expert = 0; it.first = w * 16u; it.count = min(16u, N - it.first);
     } else {
-        const ActiveExpert a = ws.active[w];
+        const ActiveExpert a = active_expert(ws, w, d, N);
         it.expert = a.expert; it.first = a.first; it.count = a.count;
     }
     return it;
@@ -51,14 +51,14 @@ __device__ __forceinline__ Item get_item(const MoeWs& ws, uint32_t index, uint32
 
 // rows of the staged tile: s_tok[r] = token, s_slot[r] = h / contrib slot (k = shared expert)
 template <bool SHARED>
-__device__ __forceinline__ void stage_pairs(const MoeWs& ws, const Item& it, uint32_t t0, uint32_t np, uint32_t k,
-                                            uint32_t* s_tok, uint32_t* s_slot, int tid)
+__device__ __forceinline__ void stage_pairs(const MoeWs& ws, const Item& it, uint32_t t0, uint32_t np,
+                                            const MoeDims& d, uint32_t N, uint32_t* s_tok, uint32_t* s_slot, int tid)
 {
     if (tid < 16) {
         uint32_t tok = 0, slot = 0;
         if ((uint32_t)tid < np) {
-            if (SHARED) { tok = it.first + tid; slot = k; }
-            else { const uint32_t pr = ws.pairs[it.first + t0 + tid]; tok = pr >> 4; slot = pr & 15u; }
+            if (SHARED) { tok = it.first + tid; slot = d.k; }
+            else pair_at(ws, it.first + t0 + tid, d, N, tok, slot);
         }
         s_tok[tid] = tok;
         s_slot[tid] = slot;
@@ -87,16 +87,16 @@ __global__ __launch_bounds__(CT, SHARED ? 2 : 4) void moe_gateup_mfma_kernel(con
     const uint32_t F = d.F, H = d.H;
     fill_mfma_tables(tab, tid, CT);
     const uint32_t subs = F / (16 * Geo::BT * nb);
-    const uint32_t n_items = item_count<SHARED>(ws, N, subs);
+    const uint32_t n_items = item_count<SHARED>(ws, d, N, subs);
 
     for (uint32_t w = blockIdx.x; w < n_items; w += gridDim.x) {
-        const Item it = get_item<SHARED>(ws, w, subs, N);
+        const Item it = get_item<SHARED>(ws, w, subs, d, N);
         const uint32_t row0 = it.sub * nb * Geo::BT * 16;
         const size_t off = ((size_t)it.expert * F + row0) * Geo::RB;
         for (uint32_t t0 = 0; t0 < it.count; t0 += 16) {
             const uint32_t np = min(16u, it.count - t0);
             __syncthreads(); // previous tile fully consumed
-            stage_pairs<SHARED>(ws, it, t0, np, d.k, s_tok, s_slot, tid);
+            stage_pairs<SHARED>(ws, it, t0, np, d, N, s_tok, s_slot, tid);
             __syncthreads();
             coop_stream<TYPE, 8, 2, 1, true, false>(gate + off, up + off, nb, X, H, np, [&](uint32_t r) { return s_tok[r]; },
                 smem, tab, tid, [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1, uint32_t) {
@@ -132,16 +132,16 @@ __global__ __launch_bounds__(CT) void moe_down_mfma_kernel(const uint8_t* __rest
     const uint32_t F = d.F, H = d.H;
     fill_mfma_tables(tab, tid, CT);
     const uint32_t subs = H / (16 * Geo::BT * nb);
-    const uint32_t n_items = item_count<SHARED>(ws, N, subs);
+    const uint32_t n_items = item_count<SHARED>(ws, d, N, subs);
 
     for (uint32_t w = blockIdx.x; w < n_items; w += gridDim.x) {
-        const Item it = get_item<SHARED>(ws, w, subs, N);
+        const Item it = get_item<SHARED>(ws, w, subs, d, N);
         const uint32_t row0 = it.sub * nb * Geo::BT * 16;
         const uint8_t* base = down + ((size_t)it.expert * H + row0) * Geo::RB;
         for (uint32_t t0 = 0; t0 < it.count; t0 += 16) {
             const uint32_t np = min(16u, it.count - t0);
             __syncthreads();
-            stage_pairs<SHARED>(ws, it, t0, np, d.k, s_tok, s_slot, tid);
+            stage_pairs<SHARED>(ws, it, t0, np, d, N, s_tok, s_slot, tid);
             __syncthreads();
             if (tid < 16) s_wt[tid] = (SHARED || (uint32_t)tid >= np) ? 1.f : sel[s_tok[tid]].w[s_slot[tid]];
             __syncthreads();
@@ -191,7 +191,8 @@ __device__ __forceinline__ uint32_t item_count_f(uint32_t n_active, uint32_t N, 
     return (N + 15) / 16 * subs_shared + n_active * subs;
 }
 
-__device__ __forceinline__ ItemF get_item_f(const MoeWs& ws, uint32_t index, uint32_t subs_shared, uint32_t subs, uint32_t N)
+__device__ __forceinline__ ItemF get_item_f(const MoeWs& ws, uint32_t index, uint32_t subs_shared, uint32_t subs,
+                                            const MoeDims& d, uint32_t N)
 {
     ItemF it;
     const uint32_t n_sh = (N + 15) / 16 * subs_shared;
@@ -201,7 +202,7 @@ __device__ __forceinline__ ItemF get_item_f(const MoeWs& ws, uint32_t index, uin
     } else {
         const uint32_t w = (index - n_sh) / subs;
         it.sub = (index - n_sh) % subs;
-        const ActiveExpert a = ws.active[w];
+        const ActiveExpert a = active_expert(ws, w, d, N);
         it.shared = false; it.expert = a.expert; it.first = a.first; it.count = a.count;
     }
     return it;
@@ -229,12 +230,12 @@ __global__ __launch_bounds__(CT) void moe_gateup_fused_kernel(const uint8_t* __r
     const int tid = threadIdx.x;
     const uint32_t F = d.F, H = d.H;
     fill_mfma_tables(tab, tid, CT);
-    const uint32_t n_active = *ws.n_active;
+    const uint32_t n_active = active_count(ws, d);
     const uint32_t subs_sh = F / (16 * FuGeoS::BT * nb_s), subs = F / (16 * FuGeoR::BT * nb_r);
     const uint32_t n_items = item_count_f(n_active, N, subs_sh, subs);
 
     for (uint32_t w = blockIdx.x; w < n_items; w += gridDim.x) {
-        const ItemF it = get_item_f(ws, w, subs_sh, subs, N);
+        const ItemF it = get_item_f(ws, w, subs_sh, subs, d, N);
         for (uint32_t t0 = 0; t0 < it.count; t0 += 16) {
             const uint32_t np = it.shared ? it.count : min(16u, it.count - t0);
             __syncthreads(); // previous tile fully consumed
@@ -242,7 +243,7 @@ __global__ __launch_bounds__(CT) void moe_gateup_fused_kernel(const uint8_t* __r
                 uint32_t tok = 0, slot = 0;
                 if ((uint32_t)tid < np) {
                     if (it.shared) { tok = it.first + tid; slot = d.k; }
-                    else { const uint32_t pr = ws.pairs[it.first + t0 + tid]; tok = pr >> 4; slot = pr & 15u; }
+                    else pair_at(ws, it.first + t0 + tid, d, N, tok, slot);
                 }
                 s_tok[tid] = tok;
                 s_slot[tid] = slot;
@@ -298,12 +299,12 @@ __global__ __launch_bounds__(CT) void moe_down_fused_kernel(const uint8_t* __res
     const int tid = threadIdx.x;
     const uint32_t F = d.F, H = d.H;
     fill_mfma_tables(tab, tid, CT);
-    const uint32_t n_active = *ws.n_active;
+    const uint32_t n_active = active_count(ws, d);
     const uint32_t subs_sh = H / (16 * Geo::S::BT * nb_s), subs = H / (16 * Geo::R::BT * nb_r);
     const uint32_t n_items = item_count_f(n_active, N, subs_sh, subs);
 
     for (uint32_t w = blockIdx.x; w < n_items; w += gridDim.x) {
-        const ItemF it = get_item_f(ws, w, subs_sh, subs, N);
+        const ItemF it = get_item_f(ws, w, subs_sh, subs, d, N);
         for (uint32_t t0 = 0; t0 < it.count; t0 += 16) {
             const uint32_t np = it.shared ? it.count : min(16u, it.count - t0);
             __syncthreads();
@@ -313,8 +314,8 @@ __global__ __launch_bounds__(CT) void moe_down_fused_kernel(const uint8_t* __res
                 if ((uint32_t)tid < np) {
                     if (it.shared) { tok = it.first + tid; slot = d.k; wt = 1.f; } // gate applied by the fold
                     else {
-                        const uint32_t pr = ws.pairs[it.first + t0 + tid];
-                        tok = pr >> 4; slot = pr & 15u; wt = sel[tok].w[slot];
+                        pair_at(ws, it.first + t0 + tid, d, N, tok, slot);
+                        wt = sel[tok].w[slot];
                     }
                 }
                 s_tok[tid] = tok; s_slot[tid] = slot; s_wt[tid] = wt;

@@ -192,6 +192,37 @@ def test_moe_decode_bs17_two_shared_tiles(qk, orc, dev, layer_iq4):
         assert orc.rel_maxabs_err(Y2.cpu().numpy()[s], refs[s]["y"]) <= TOL
 
 
+@pytest.mark.parametrize("n", [3, 40])
+def test_moe_stale_workspace_stays_in_bounds(qk, orc, dev, layer_iq4, n):
+    """Gate/up and down run on a workspace that no routing launch has written (arbitrary bytes, then
+    small integers that look like indices but fit nothing): the numbers mean nothing, but every word the
+    kernels take from the workspace is clamped to the tensors' ranges, so the launches complete.  The
+    same workspace, cleared, then gives the right step."""
+    import torch
+    print(f"[case] moe stale workspace, {n} rows", flush=True)
+    X, refs = pick_inputs(orc, layer_iq4, n, seed=40 + n)
+    layer = layer_iq4.to_device(dev)
+    nbytes = qk.moe_workspace_bytes(layer, n)
+    Xd = torch.from_numpy(X).to(dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(n)
+    fills = [torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device=dev, generator=g),
+             torch.randint(0, 64, (nbytes // 4,), dtype=torch.int32, device=dev, generator=g).view(torch.uint8)]
+    ws = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+    for fill in fills:
+        ws.copy_(fill)
+        qk.moe_decode(layer, Xd, ws, stages=6)
+        torch.cuda.synchronize()
+    ws.zero_()
+    Y, sel = qk.moe_decode(layer, Xd, ws)
+    torch.cuda.synchronize()
+    ids, _, _ = sel_fields(sel)
+    Y = Y.cpu().numpy()
+    for s in range(n):
+        assert list(ids[s, :8]) == list(refs[s]["sel"].ids[:8]), f"slot {s}"
+        assert orc.rel_maxabs_err(Y[s], refs[s]["y"]) <= TOL, f"slot {s}"
+
+
 def test_group_pairs_matches_oracle(qk, orc, dev):
     import torch
     print("[case] group pairs", flush=True)
