@@ -313,6 +313,15 @@ def main():
                                                          frac=g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9 / HBM_PEAK_GBPS)
                 log(f"[bench] gemv {name} bs16: {ex[f'gemv_{name}_8192x2048_bs16']}")
                 torch.cuda.empty_cache()
+        # the other dense projections of a decode step at the reference's shapes (src/main.cpp:4310-4335)
+        for M, K in ((4096, 2048), (2048, 4096), (512, 2048)):
+            for b in (1, 16):
+                g = gemv_workload(qk, qk.Q8_0, M, K, b, es, ew)
+                key = f"gemv_q8_0_{M}x{K}" + ("_bs16" if b > 1 else "")
+                ex[key] = dict(us=g["ms_event"] * 1e3, gbps=g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9,
+                               frac=g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9 / HBM_PEAK_GBPS)
+                log(f"[bench] {key}: {ex[key]}")
+                torch.cuda.empty_cache()
         for b in (1, 16):
             h = head_workload(qk, 151936, 2048, b, 40, 8)
             ex[f"head_q6k_151936_bs{b}"] = dict(us=h["ms_event"] * 1e3, gbps=h["bytes_step"] / (h["ms_event"] * 1e-3) / 1e9,

@@ -264,16 +264,22 @@ __device__ __forceinline__ void load_afrag(AFrag& a, const float* __restrict__ X
 // alternate between two buffers as well, so fast waves run ahead into the next batch.
 // CLAMP: `limit` is the offset from base0 of the tensor's last 16 bytes; loads beyond it re-read
 // those (the caller ignores the rows that do not exist).
-template <int TYPE, int KS, int NS, int TG, bool ALT, bool CLAMP, int NA = 1, int PB = 2, typename RowOf, typename Epi>
+// STRIDED: the rows are longer than 256*KS weights and this call takes the RB bytes at base0 of
+// each (a K range of every row): consecutive rows lie row_stride bytes apart, a row's piece is
+// still contiguous and a multiple of 16 bytes, and LDS receives the pieces packed as before.
+template <int TYPE, int KS, int NS, int TG, bool ALT, bool CLAMP, int NA = 1, int PB = 2, bool STRIDED = false,
+          typename RowOf, typename Epi>
 __device__ __forceinline__ void coop_stream(const uint8_t* __restrict__ base0, const uint8_t* __restrict__ base1,
                                             uint32_t n_batches, const float* __restrict__ A_src, uint32_t a_stride,
                                             uint32_t np, RowOf row_of, uint8_t* smem, const MfmaTables& tab, int tid,
-                                            Epi epi, size_t limit = 0)
+                                            Epi epi, size_t limit = 0, uint32_t row_stride = 0)
 {
     using Geo = CoopGeom<TYPE, KS, NS, TG, ALT, NA, PB>;
     constexpr int BT = Geo::BT, NSB = Geo::NSB, NTL = NSB * TG; // tiles per wave and batch
     constexpr uint32_t RB = Geo::RB, TBYTES = Geo::TBYTES, BBYTES = Geo::BBYTES, PBYTES = Geo::PART_BYTES;
     constexpr int PIECES = BBYTES / 16, PPT = BT * TBYTES / 16, NLD = (PIECES + CT - 1) / CT;
+    constexpr uint32_t PPR = RB / 16; // STRIDED: pieces per row
+    static_assert(!STRIDED || (RB % 16 == 0 && !ALT && NSB == 1), "strided rows: whole 16-byte pieces, one tensor");
     constexpr int OUTS = (NA * BT * 256 + CT - 1) / CT; // outputs per thread and batch
     const int lane = tid & 63, wave = tid >> 6, kw = wave % KS, tg = wave / KS, j = lane & 15, g = lane >> 4;
     const uint32_t steps = ALT ? 2 * n_batches : n_batches; // LDS batches
@@ -284,16 +290,18 @@ __device__ __forceinline__ void coop_stream(const uint8_t* __restrict__ base0, c
 #pragma unroll
     for (int n = 0; n < NLD; n++) {
         const uint32_t p = min((uint32_t)(tid + CT * n), (uint32_t)PIECES - 1);
-        size_t off = (size_t)(p % PPT) * 16;
+        const uint32_t pp = p % PPT;
+        size_t off = STRIDED ? (size_t)(pp / PPR) * row_stride + (size_t)(pp % PPR) * 16 : (size_t)pp * 16;
         if (CLAMP) { off = min(off, limit); room[n] = limit - off; }
         src[n] = ((NSB > 1 && p >= (uint32_t)PPT) ? base1 : base0) + off;
     }
     const size_t alt_delta = ALT ? (size_t)(base1 - base0) : 0;
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     u32x4 ld[NLD];
+    const size_t batch_bytes = STRIDED ? (size_t)(BT * 16) * row_stride : (size_t)(BT * TBYTES);
     const auto adv_of = [&](uint32_t nx) -> size_t {
         nx = min(nx, steps - 1); // past the end: a harmless re-read
-        return ALT ? (size_t)(nx >> 1) * (BT * TBYTES) + (nx & 1u) * alt_delta : (size_t)nx * (BT * TBYTES);
+        return ALT ? (size_t)(nx >> 1) * batch_bytes + (nx & 1u) * alt_delta : (size_t)nx * batch_bytes;
     };
 #pragma unroll
     for (int n = 0; n < NLD; n++) ld[n] = *(const u32x4*)src[n];

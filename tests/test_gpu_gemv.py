@@ -34,11 +34,28 @@ def test_gemv_quantised(qk, orc, dev, name, M, K, batch):
 
 @pytest.mark.parametrize("name", ["q8_0", "q6_k", "iq4_xs", "iq3_xxs"])
 @pytest.mark.parametrize("M,K,batch", [(8192, 2048, 16), (1000, 2048, 5), (130, 1024, 16), (96, 512, 4),
-                                       (77, 512, 3), (48, 256, 32), (2048, 2048, 40), (33, 2048, 17)])
+                                       (77, 512, 3), (48, 256, 32), (2048, 2048, 40), (33, 2048, 17),
+                                       (2048, 4096, 16), (100, 4096, 5), (33, 4096, 40)])
 def test_gemv_quantised_several_rows(qk, orc, dev, name, M, K, batch):
-    """batch >= 3 takes the matrix-core path where the shape allows (K = 256..2048 and the tensor
-    ending on a 16-byte boundary), one pass per row otherwise: same bar either way."""
+    """batch >= 3 takes the matrix-core path where the shape allows (K = 256..2048, or 4096 in two
+    passes over the rows' halves, and the tensor ending on a 16-byte boundary), one pass per row
+    otherwise: same bar either way."""
     run_case(qk, orc, dev, name, M, K, batch, seed=77)
+
+
+@pytest.mark.parametrize("M,K", [(8192, 2048), (4096, 2048), (2048, 4096), (512, 2048)])
+@pytest.mark.parametrize("batch", [1, 16])
+def test_gemv_q8_0_engine_shapes(qk, orc, dev, M, K, batch):
+    """The dense projections of a decode step at the shapes the reference dispatches them
+    (src/main.cpp:4310-4335, 4195-4196), for one slot and for sixteen."""
+    run_case(qk, orc, dev, "q8_0", M, K, batch, seed=5)
+
+
+def test_gemv_two_pass_k_is_deterministic(qk, orc, dev):
+    """K = 4096 for several rows adds the second half's sum to the first's in a fixed order."""
+    a = run_case(qk, orc, dev, "q6_k", 784, 4096, 9, seed=12)
+    b = run_case(qk, orc, dev, "q6_k", 784, 4096, 9, seed=12)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
 
 
 @pytest.mark.parametrize("M,K", [(64, 32), (33, 96), (10, 2080)])
