@@ -82,9 +82,11 @@ static void launch(const uint8_t* W, const float* X, float* Y, uint32_t M, uint3
     }();
     const uint32_t groups = (N + 16 * NA - 1) / (16 * NA);
     const uint32_t total = (M + 16 * Geo::BT - 1) / (16 * Geo::BT);
-    // fill the CUs once; at least two batches per workgroup where the tensor allows
+    // fill the CUs once; a tensor with no more batches than CUs gets a workgroup per batch (the fixed
+    // cost of a workgroup dominates there), a larger one at least two batches per workgroup
     const uint32_t want = std::max(1u, per_cu * (persistent_blocks() / 4) / groups);
-    const uint32_t ranges = std::max(1u, std::min(want, (total + 1) / 2));
+    const uint32_t minb = total <= persistent_blocks() / 4 ? 1u : 2u;
+    const uint32_t ranges = std::max(1u, std::min(want, (total + minb - 1) / minb));
     hipLaunchKernelGGL((gemm_coop_kernel<TYPE, KS, NA, KP>), dim3(groups * ranges), dim3(CT), Geo::LDS_BYTES, st, W, X, Y,
                        M, N, ranges);
 }
