@@ -38,6 +38,29 @@ __device__ static void fill_mfma_tables(MfmaTables& t, int tid, int nthreads)
     }
 }
 
+// Only what BFrag<TYPE> reads: the IQ3_XXS grid and signs, the IQ4_XS codebook, nothing for the others.
+template <int TYPE>
+__device__ static void fill_mfma_tables_for(MfmaTables& t, int tid, int nthreads)
+{
+    if constexpr (TYPE == QKK_IQ3_XXS) {
+        for (int i = tid; i < 256; i += nthreads) t.grid[i] = g_iq3xxs_grid[i];
+        for (int i = tid; i < 128; i += nthreads) {
+            const uint32_t s8 = (uint32_t)i | ((__builtin_popcount(i) & 1u) << 7);
+            const uint32_t a = ((s8 & 15u) * 0x00204081u) & 0x01010101u, b = ((s8 >> 4) * 0x00204081u) & 0x01010101u;
+            t.sign[i] = uint2{(a << 8) - a, (b << 8) - b};
+        }
+    } else if constexpr (TYPE == QKK_IQ4_XS) {
+        if (tid < 4) {
+            constexpr int8_t kv[16] = {QK_IQ4NL_VALUES};
+            uint32_t w = 0;
+#pragma unroll
+            for (int i = 0; i < 16; i++)
+                if (i / 4 == tid) w |= (uint32_t)(uint8_t)kv[i] << (8 * (i % 4));
+            t.iq4[tid] = w;
+        }
+    }
+}
+
 // ---- a lane's share of one 256-weight fragment of row (l%16), in the B-operand cut -----------------
 // Lane group g = l/16 owns 64 of the fragment's 256 weights, chosen so that its bytes are
 // CONTIGUOUS in the block and a fragment is two or three wide (LDS) reads:

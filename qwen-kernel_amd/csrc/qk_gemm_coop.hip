@@ -29,7 +29,7 @@ __global__ __launch_bounds__(CT) void gemm_coop_kernel(const uint8_t* __restrict
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ MfmaTables tab;
     const int tid = threadIdx.x;
-    fill_mfma_tables(tab, tid, CT);
+    fill_mfma_tables_for<TYPE>(tab, tid, CT); // in place before the stream's first barrier
     const uint32_t groups = (N + 16 * NA - 1) / (16 * NA);
     const uint32_t q = blockIdx.x % groups, r = blockIdx.x / groups;
     // batches [b0, b1) of the tensor's `total`, an even split over the ranges (b1 <= total)
@@ -37,7 +37,6 @@ __global__ __launch_bounds__(CT) void gemm_coop_kernel(const uint8_t* __restrict
     const uint32_t b0 = (uint32_t)((uint64_t)r * total / ranges), b1 = (uint32_t)((uint64_t)(r + 1) * total / ranges);
     const uint32_t row0 = b0 * BT * 16, tok0 = q * 16 * NA;
     if (b1 <= b0 || row0 >= M || tok0 >= N) return; // the whole workgroup
-    __syncthreads();
     const uint32_t np = min((uint32_t)(16 * NA), N - tok0);
     if constexpr (KP == 1) {
         coop_stream<TYPE, KS, 1, 1, false, true, NA>(
