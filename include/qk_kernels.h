@@ -166,6 +166,36 @@ size_t qkk_moe_prefill_workspace_bytes(const qkk_moe_layer *L_host, uint32_t n_t
 int qkk_moe_prefill(const qkk_moe_layer *L_host, const float *X, float *Y, qkk_sel *sel,
                     void *workspace, size_t workspace_bytes, uint32_t n_tokens, void *stream);
 
+/* ---- layer glue: the fp32 steps between the projections of a layer ---------------------------
+ * Rows are activation rows (the reference's z = slot), n floats each, contiguous.  Outputs may be
+ * the inputs (in place); w must not overlap an output.  eps >= 0 (the reference passes 1e-6,
+ * src/main.cpp:4194).
+ *   qkk_rmsnorm      out = x * scale * w,  scale = 1/sqrt(mean(x^2) + eps)
+ *                    (reference shaders/rmsnorm.comp:19-32)
+ *   qkk_add_rmsnorm  y = a + b;  xn = y * scale(y) * w   (residual add + the layer's FFN norm;
+ *                    reference shaders/add_rmsnorm.comp:23-40; add_rmsnorm_route.comp is the same
+ *                    arithmetic plus a counter reset this library does not need)
+ *   qkk_add_rms3     s = (a + b) + c;  xn = s * scale(s) * w   (layer tail: residual + routed +
+ *                    shared, normalised with the NEXT layer's weight; reference
+ *                    shaders/add_rms3.comp:24-41).  qkk_moe_decode already returns routed + shared
+ *                    as one row, so a caller of this library uses qkk_add_rmsnorm for the tail.
+ *   qkk_vec_add      out = a + b   (reference shaders/vec_add.comp:13-14) */
+int qkk_rmsnorm(const float *x, const float *w, float *out, uint32_t n, uint32_t rows, float eps,
+                void *stream);
+int qkk_add_rmsnorm(const float *a, const float *b, const float *w, float *y, float *xn, uint32_t n,
+                    uint32_t rows, float eps, void *stream);
+int qkk_add_rms3(const float *a, const float *b, const float *c, const float *w, float *s, float *xn,
+                 uint32_t n, uint32_t rows, float eps, void *stream);
+int qkk_vec_add(const float *a, const float *b, float *out, uint64_t n, void *stream);
+
+/* Embedding lookup (reference shaders/embed_q6k.comp:27-49, embed_q8_0.comp:24-34; the reference
+ * dispatches Q6_K or Q8_0, src/main.cpp:3678): x[r][0..kdim) = the dequantised row
+ * ids[idx + per_req * r] of the token-embedding tensor W [n_vocab][kdim], r < rows; bit-identical
+ * to qkk_dequant of that row.  ids is a device array of n_ids token ids; an id >= n_vocab reads
+ * the last row. */
+int qkk_embed(int type, const void *W, uint32_t n_vocab, uint32_t kdim, const uint32_t *ids,
+              uint32_t n_ids, uint32_t idx, uint32_t per_req, float *x, uint32_t rows, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -14,6 +14,8 @@
  *   pair grouping .................................... shaders/moe_group_pairs.comp
  *   batched GEMM reference and acceptance ............ src/main.cpp:5561-5570, 5653-5662
  *   scale-aware acceptance metric .................... src/main.cpp:548-565
+ *   RMS norm (with the shaders' fp32 residual sums) .. src/main.cpp:1685-1690, shaders/add_rms3.comp:29-40
+ *   embedding lookup ................................. shaders/embed_q6k.comp:27-49
  *
  * How each part is pinned (tests/test_oracle.py, tests/test_golden.py):
  *   qko_f16_to_f32 / qko_f32_to_f16 .. all 65,536 halves and a float sweep against the
@@ -31,6 +33,10 @@
  *       softmax-weighted MLP.
  *   qko_group_pairs ................... against a numpy stable sort.
  *   qko_argmax ........................ against numpy argmax, with duplicated maxima.
+ *   qko_add_rms ....................... against a numpy float64 evaluation; unit weights give
+ *       mean(xn^2) = ms/(ms+eps); scaling the inputs by 2 leaves xn unchanged at eps = 0
+ *       (exact in binary floating point); the stored sum is bitwise numpy's float32 (a+b)+c.
+ *   qko_embed ......................... bitwise qko_dequant_row of the chosen rows.
  * Agreement of these formats with upstream ggml is pinned in the reference only by
  * model-level token parity, which needs a model file that is absent here: parity
  * with upstream ggml is unpinned; parity with the reference's header is pinned.
@@ -433,4 +439,43 @@ double qko_max_err_over_rms(const float *got, const float *ref, size_t n)
         if (e > worst) worst = e;
     }
     return rms > 0 ? worst / rms : worst;
+}
+
+/* ---- layer glue ---------------------------------------------------------------- */
+/* v = a [+ b [+ c]] in float, left to right, as the shaders form it
+ * (shaders/add_rmsnorm.comp:28, add_rms3.comp:29); the norm as the CPU checker computes it,
+ * in double: sc = 1/sqrt(sum(v^2)/n + eps), xn = (float)(v * sc * w) (src/main.cpp:1685-1690). */
+void qko_add_rms(const float *a, const float *b, const float *c, const float *w, float *sum_out,
+                 float *xn, uint32_t n, float eps)
+{
+    double ss = 0;
+    for (uint32_t i = 0; i < n; i++) {
+        float v = a[i];
+        if (b) v = v + b[i];
+        if (c) v = v + c[i];
+        ss += (double)v * v;
+    }
+    const double sc = 1.0 / sqrt(ss / n + eps);
+    for (uint32_t i = 0; i < n; i++) {
+        float v = a[i];
+        if (b) v = v + b[i];
+        if (c) v = v + c[i];
+        if (sum_out) sum_out[i] = v;
+        xn[i] = (float)(v * sc * w[i]);
+    }
+}
+
+/* x[r] = dequantised row ids[idx + per_req*r] of W [n_vocab][kdim]
+ * (shaders/embed_q6k.comp:27-49, embed_q8_0.comp:24-34). */
+int qko_embed(int type, const void *W, uint32_t n_vocab, uint32_t kdim, const uint32_t *ids,
+              uint32_t idx, uint32_t per_req, float *x, uint32_t rows)
+{
+    const size_t rb = qko_row_bytes(type, kdim);
+    if (!rb) return -1;
+    for (uint32_t r = 0; r < rows; r++) {
+        const uint32_t tok = ids[idx + per_req * r];
+        if (tok >= n_vocab) return -2;
+        if (qko_dequant_row(type, (const uint8_t *)W + (size_t)tok * rb, x + (size_t)r * kdim, kdim)) return -1;
+    }
+    return 0;
 }

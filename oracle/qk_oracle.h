@@ -114,6 +114,16 @@ double qko_max_rel_err(const float *got, const float *ref, size_t n);
 /* max|got-ref| / rms(ref): the batched-GEMM acceptance metric (src/main.cpp:5653-5662). */
 double qko_max_err_over_rms(const float *got, const float *ref, size_t n);
 
+/* v = a [+ b [+ c]] in float (b, c may be NULL; shaders/add_rmsnorm.comp:28, add_rms3.comp:29),
+ * sum_out (optional) = v, xn = (float)(v * sc * w) with sc = 1/sqrt(sum(v^2)/n + eps) in double
+ * (src/main.cpp:1685-1690). */
+void qko_add_rms(const float *a, const float *b, const float *c, const float *w, float *sum_out,
+                 float *xn, uint32_t n, float eps);
+
+/* Embedding lookup (shaders/embed_q6k.comp:27-49). Returns 0, -1 bad type/kdim, -2 id out of range. */
+int qko_embed(int type, const void *W, uint32_t n_vocab, uint32_t kdim, const uint32_t *ids,
+              uint32_t idx, uint32_t per_req, float *x, uint32_t rows);
+
 #ifdef __cplusplus
 }
 #endif

@@ -59,6 +59,9 @@ def lib():
         L.qko_max_rel_err.argtypes = [vp, vp, C.c_size_t]
         L.qko_max_err_over_rms.restype = C.c_double
         L.qko_max_err_over_rms.argtypes = [vp, vp, C.c_size_t]
+        L.qko_add_rms.restype = None
+        L.qko_add_rms.argtypes = [vp, vp, vp, vp, vp, vp, u32, C.c_float]
+        L.qko_embed.argtypes = [C.c_int, vp, u32, u32, vp, u32, u32, vp, u32]
         _lib = L
     return _lib
 
@@ -118,6 +121,34 @@ def gemv(type_, W, x, M, K):
     if rc:
         raise ValueError(f"gemv rc={rc}")
     return y if x.ndim == 2 else y[0]
+
+
+def add_rms(a, w, eps, b=None, c=None, want_sum=False):
+    """Rows of a (+b (+c)) summed in float32, RMS-normed in double with weight w.  Returns xn, or
+    (sum, xn)."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    rows = a.reshape(-1, a.shape[-1])
+    n = rows.shape[1]
+    bb = None if b is None else np.ascontiguousarray(b, dtype=np.float32).reshape(-1, n)
+    cc = None if c is None else np.ascontiguousarray(c, dtype=np.float32).reshape(-1, n)
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    s = np.empty_like(rows)
+    xn = np.empty_like(rows)
+    for r in range(rows.shape[0]):
+        lib().qko_add_rms(_p(rows[r]), None if bb is None else _p(bb[r]), None if cc is None else _p(cc[r]), _p(w),
+                          _p(s[r]), _p(xn[r]), n, eps)
+    s, xn = s.reshape(a.shape), xn.reshape(a.shape)
+    return (s, xn) if want_sum else xn
+
+
+def embed(type_, W, n_vocab, kdim, ids, idx, per_req, rows):
+    W = np.ascontiguousarray(W).reshape(-1)
+    ids = np.ascontiguousarray(ids, dtype=np.uint32)
+    x = np.empty((rows, kdim), dtype=np.float32)
+    rc = lib().qko_embed(type_, _p(W), n_vocab, kdim, _p(ids), idx, per_req, _p(x), rows)
+    if rc:
+        raise ValueError(f"embed rc={rc}")
+    return x
 
 
 def argmax(v):

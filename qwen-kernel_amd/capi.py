@@ -63,6 +63,12 @@ def lib():
         L.qkk_argmax.argtypes = [vp, vp, u32, u32, vp]
         L.qkk_gemm_q8_0.argtypes = [vp, vp, vp, u32, u32, u32, vp]
         L.qkk_moe_prefill.argtypes = [vp, vp, vp, vp, vp, sz, u32, vp]
+        f32 = C.c_float
+        L.qkk_rmsnorm.argtypes = [vp, vp, vp, u32, u32, f32, vp]
+        L.qkk_add_rmsnorm.argtypes = [vp, vp, vp, vp, vp, u32, u32, f32, vp]
+        L.qkk_add_rms3.argtypes = [vp, vp, vp, vp, vp, vp, u32, u32, f32, vp]
+        L.qkk_vec_add.argtypes = [vp, vp, vp, u64, vp]
+        L.qkk_embed.argtypes = [C.c_int, vp, u32, u32, vp, u32, u32, u32, vp, u32, vp]
         _lib = L
     return _lib
 
@@ -210,4 +216,57 @@ def gemm_q8_0(W, X, M, K, out=None):
     if out is None:
         out = torch.empty((N, M), dtype=torch.float32, device=X.device)
     _check(lib().qkk_gemm_q8_0(_ptr(W), _ptr(X), _ptr(out), M, K, N, _stream()))
+    return out
+
+
+def _rows(t):
+    return (1, t.shape[0]) if t.dim() == 1 else (t.shape[0], t.shape[1])
+
+
+def rmsnorm(x, w, eps=1e-6, out=None):
+    """out = x * w / sqrt(mean(x^2) + eps) per row of x ([rows, n] or [n])."""
+    import torch
+    rows, n = _rows(x)
+    if out is None:
+        out = torch.empty_like(x)
+    _check(lib().qkk_rmsnorm(_ptr(x), _ptr(w), _ptr(out), n, rows, eps, _stream()))
+    return out
+
+
+def add_rmsnorm(a, b, w, eps=1e-6, y=None, xn=None):
+    """y = a + b; xn = rmsnorm(y) * w.  Returns (y, xn)."""
+    import torch
+    rows, n = _rows(a)
+    y = torch.empty_like(a) if y is None else y
+    xn = torch.empty_like(a) if xn is None else xn
+    _check(lib().qkk_add_rmsnorm(_ptr(a), _ptr(b), _ptr(w), _ptr(y), _ptr(xn), n, rows, eps, _stream()))
+    return y, xn
+
+
+def add_rms3(a, b, c, w, eps=1e-6, s=None, xn=None):
+    """s = (a + b) + c; xn = rmsnorm(s) * w.  Returns (s, xn)."""
+    import torch
+    rows, n = _rows(a)
+    s = torch.empty_like(a) if s is None else s
+    xn = torch.empty_like(a) if xn is None else xn
+    _check(lib().qkk_add_rms3(_ptr(a), _ptr(b), _ptr(c), _ptr(w), _ptr(s), _ptr(xn), n, rows, eps, _stream()))
+    return s, xn
+
+
+def vec_add(a, b, out=None):
+    import torch
+    if out is None:
+        out = torch.empty_like(a)
+    _check(lib().qkk_vec_add(_ptr(a), _ptr(b), _ptr(out), a.numel(), _stream()))
+    return out
+
+
+def embed(type_, W, n_vocab, kdim, ids, rows, idx=0, per_req=1, out=None):
+    """x[r] = dequantised row ids[idx + per_req*r] of the embedding tensor W; ids is a uint32/int32
+    device tensor."""
+    import torch
+    if out is None:
+        out = torch.empty((rows, kdim), dtype=torch.float32, device=W.device)
+    _check(lib().qkk_embed(type_, _ptr(W), n_vocab, kdim, _ptr(ids), ids.numel(), idx, per_req, _ptr(out), rows,
+                           _stream()))
     return out

@@ -133,6 +133,22 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
     out[i] = dequant_elem<TYPE>(W + blk * BLOCK_BYTES, (int)(i % BLOCK_ELEMS));
 }
 
+// Embedding lookup: row ids[idx + per_req * rq] of the token-embedding tensor, dequantised with the
+// same element routine (bit-exact), into activation row rq (reference shaders/embed_q6k.comp:27-49,
+// embed_q8_0.comp:24-34).  A token id outside the vocabulary reads the last row instead of memory
+// outside the tensor.
+template <int TYPE, int BLOCK_ELEMS, int BLOCK_BYTES>
+__global__ __launch_bounds__(256) void embed_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict__ ids,
+                                                    uint32_t idx, uint32_t per_req, float* __restrict__ x,
+                                                    uint32_t kdim, uint32_t n_vocab)
+{
+    const uint32_t rq = blockIdx.y;
+    const uint32_t tok = min(ids[idx + per_req * rq], n_vocab - 1);
+    const uint8_t* row = W + (size_t)tok * (kdim / BLOCK_ELEMS) * BLOCK_BYTES;
+    for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < kdim; i += gridDim.x * 256)
+        x[(size_t)rq * kdim + i] = dequant_elem<TYPE>(row + (size_t)(i / BLOCK_ELEMS) * BLOCK_BYTES, (int)(i % BLOCK_ELEMS));
+}
+
 __global__ __launch_bounds__(256) void dequant_f16_kernel(const uint16_t* __restrict__ W,
                                                           float* __restrict__ out, uint64_t n)
 {
@@ -412,6 +428,38 @@ int qkk_dequant(int type, const void* W, float* out, uint64_t n, void* stream)
     default: return fail(QKK_ETYPE, "qkk_dequant: unsupported tensor type %d", type);
     }
     return check_launch("qkk_dequant");
+}
+
+int qkk_embed(int type, const void* W, uint32_t n_vocab, uint32_t kdim, const uint32_t* ids, uint32_t n_ids,
+              uint32_t idx, uint32_t per_req, float* x, uint32_t rows, void* stream)
+{
+    if (!W || !ids || !x) return fail(QKK_EINVAL, "qkk_embed: null pointer");
+    if (n_vocab == 0 || kdim == 0 || rows == 0) return fail(QKK_EINVAL, "qkk_embed: n_vocab, kdim and rows must be positive");
+    if (rows > 65535) return fail(QKK_ESHAPE, "qkk_embed: %u rows exceeds 65535", rows);
+    if ((uint64_t)idx + (uint64_t)per_req * (rows - 1) >= n_ids)
+        return fail(QKK_ESHAPE, "qkk_embed: ids[%u + %u*%u] is outside the %u ids", idx, per_req, rows - 1, n_ids);
+    if (type != QKK_Q8_0 && type != QKK_Q6_K && type != QKK_IQ4_XS && type != QKK_IQ3_XXS)
+        return fail(QKK_ETYPE, "qkk_embed: unsupported tensor type %d", type);
+    if (qkk_row_bytes(type, kdim) == 0) return fail(QKK_ESHAPE, "qkk_embed: type %d with kdim=%u is not supported", type, kdim);
+    if (int rc = require_device()) return rc;
+    const dim3 grid(std::min((kdim + 255) / 256, 64u), rows);
+    hipStream_t st = as_stream(stream);
+    const uint8_t* w = (const uint8_t*)W;
+    switch (type) {
+    case QKK_Q8_0:
+        hipLaunchKernelGGL((embed_kernel<QKK_Q8_0, 32, Q8_0_BYTES>), grid, dim3(256), 0, st, w, ids, idx, per_req, x, kdim, n_vocab);
+        break;
+    case QKK_Q6_K:
+        hipLaunchKernelGGL((embed_kernel<QKK_Q6_K, 256, Q6_K_BYTES>), grid, dim3(256), 0, st, w, ids, idx, per_req, x, kdim, n_vocab);
+        break;
+    case QKK_IQ4_XS:
+        hipLaunchKernelGGL((embed_kernel<QKK_IQ4_XS, 256, IQ4_XS_BYTES>), grid, dim3(256), 0, st, w, ids, idx, per_req, x, kdim, n_vocab);
+        break;
+    default:
+        hipLaunchKernelGGL((embed_kernel<QKK_IQ3_XXS, 256, IQ3_XXS_BYTES>), grid, dim3(256), 0, st, w, ids, idx, per_req, x, kdim, n_vocab);
+        break;
+    }
+    return check_launch("qkk_embed");
 }
 
 int qkk_gemv(int type, const void* W, const float* X, float* Y, uint32_t M, uint32_t K, uint32_t batch,

@@ -348,3 +348,63 @@ def test_metrics(orc):
     assert np.isclose(orc.max_err_over_rms(got, ref_), 0.01 / rms, rtol=1e-5)
     assert np.isclose(orc.rel_maxabs_err(got, ref_), 0.01 / 4.0, rtol=1e-5)
     assert orc.max_rel_err(np.array([np.nan], dtype=np.float32), np.array([1.0], dtype=np.float32)) == np.inf
+
+
+# ---- layer glue -------------------------------------------------------------------------------
+
+def _rms64(v, w, eps):
+    v64 = v.astype(np.float64)
+    return v64 / np.sqrt(np.mean(v64 * v64, axis=-1, keepdims=True) + eps) * w.astype(np.float64)
+
+
+@pytest.mark.parametrize("n", [2048, 4096, 100, 7])
+def test_add_rms_vs_float64(orc, n):
+    rng = np.random.default_rng(n)
+    a, b, c = (rng.standard_normal((3, n)).astype(np.float32) * np.float32(s) for s in (1.0, 0.3, 5.0))   # three rows each
+    w = rng.uniform(0.5, 1.5, n).astype(np.float32)
+    eps = 1e-6
+    # one, two and three inputs; the stored sum is numpy's float32 sum taken left to right
+    for bb, cc in ((None, None), (b, None), (b, c)):
+        v = a if bb is None else (a + bb if cc is None else (a + bb) + cc)
+        assert v.dtype == np.float32
+        s, xn = orc.add_rms(a, w, eps, b=bb, c=cc, want_sum=True)
+        assert np.array_equal(s.view(np.uint32), v.view(np.uint32))
+        want = _rms64(v, w, eps)
+        assert np.max(np.abs(xn - want)) <= 2e-7 * np.max(np.abs(want))
+
+
+def test_add_rms_invariants(orc):
+    rng = np.random.default_rng(5)
+    n = 2048
+    a = rng.standard_normal((4, n)).astype(np.float32)
+    ones = np.ones(n, dtype=np.float32)
+    # unit weights: mean(xn^2) = ms / (ms + eps)
+    for eps in (1e-6, 0.5):
+        xn = orc.add_rms(a, ones, eps).astype(np.float64)
+        ms = np.mean(a.astype(np.float64) ** 2, axis=1)
+        assert np.allclose(np.mean(xn * xn, axis=1), ms / (ms + eps), rtol=1e-6)
+    # eps = 0: scaling the input by a power of two changes nothing, bit for bit
+    w = rng.uniform(0.5, 1.5, n).astype(np.float32)
+    x1, x2 = orc.add_rms(a, w, 0.0), orc.add_rms(a * np.float32(4.0), w, 0.0)
+    assert np.array_equal(x1.view(np.uint32), x2.view(np.uint32))
+    # a wrong operand order or a dropped input shows: b enters the norm
+    b = rng.standard_normal((4, n)).astype(np.float32)
+    assert not np.allclose(orc.add_rms(a, w, 1e-6, b=b), orc.add_rms(a, w, 1e-6))
+    # the weight multiplies the output elementwise
+    assert np.allclose(orc.add_rms(a, w, 1e-6), orc.add_rms(a, ones, 1e-6) * w, rtol=1e-6)
+
+
+def test_embed_is_dequant_of_the_chosen_rows(orc, qk):
+    rng = np.random.default_rng(9)
+    for t, be in ((qk.Q6_K, 256), (qk.Q8_0, 32)):
+        V, K = 50, 512
+        W = qk.synth.tensor_host(t, V, K, seed=3)
+        rb = orc.row_bytes(t, K)
+        ids = rng.integers(0, V, 12).astype(np.uint32)
+        got = orc.embed(t, W, V, K, ids, idx=2, per_req=3, rows=4)
+        for r in range(4):
+            tok = ids[2 + 3 * r]
+            want = orc.dequant(t, W.reshape(-1)[tok * rb:(tok + 1) * rb], K)
+            assert np.array_equal(got[r].view(np.uint32), want.view(np.uint32))
+    with pytest.raises(ValueError):
+        orc.embed(qk.Q8_0, W, V, K, np.array([V], dtype=np.uint32), 0, 1, 1)
