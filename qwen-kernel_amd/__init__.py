@@ -13,3 +13,4 @@ from .capi import (  # noqa: F401
     rmsnorm, add_rmsnorm, add_rms3, vec_add, embed,
 )
 from . import synth  # noqa: F401
+from . import gguf  # noqa: F401

@@ -223,6 +223,33 @@ def test_moe_stale_workspace_stays_in_bounds(qk, orc, dev, layer_iq4, n):
         assert orc.rel_maxabs_err(Y[s], refs[s]["y"]) <= TOL, f"slot {s}"
 
 
+def test_moe_layer_loaded_from_gguf(qk, orc, dev, tmp_path):
+    """The reference's per-layer check on a model file (`qk moe <layer>`, src/main.cpp:920-1254): the
+    layer's tensors come out of a GGUF file through the library's reader, the step runs on them,
+    and the result is held against the CPU restatement on the same bytes.  The file is synthetic
+    (no model file is available): same tensor names, types, shapes and metadata keys."""
+    import torch
+    print("[case] moe layer from a GGUF file", flush=True)
+    hl = qk.synth.HostLayer(seed=900, n_expert=16, n_used=4, down_type=qk.Q6_K)
+    path = tmp_path / "model.gguf"
+    qk.gguf.write(path, {"general.architecture": "qwen3next", "qwen3next.expert_used_count": 4},
+                  qk.gguf.layer_tensors(hl, 5))
+    with qk.gguf.File(path) as f:
+        layer = f.moe_layer(5, dev)
+    assert (layer.n_embd, layer.n_ff, layer.n_expert, layer.n_used, layer.down_type) == (2048, 512, 16, 4, qk.Q6_K)
+    for n in (1, 6):
+        X, refs = pick_inputs(orc, hl, n, seed=60 + n)
+        ws = torch.zeros(qk.moe_workspace_bytes(layer, n), dtype=torch.uint8, device=dev)
+        Y, sel = qk.moe_decode(layer, torch.from_numpy(X).to(dev), ws)
+        torch.cuda.synchronize()
+        ids, w, _ = sel_fields(sel)
+        Y = Y.cpu().numpy()
+        for s in range(n):
+            assert list(ids[s, :4]) == list(refs[s]["sel"].ids[:4])
+            assert np.max(np.abs(w[s, :4] - np.array(refs[s]["sel"].w[:4]))) <= 1e-4
+            assert orc.rel_maxabs_err(Y[s], refs[s]["y"]) <= TOL
+
+
 def test_group_pairs_matches_oracle(qk, orc, dev):
     import torch
     print("[case] group pairs", flush=True)
