@@ -121,6 +121,17 @@ size_t qkk_moe_workspace_bytes(const qkk_moe_layer *L_host, uint32_t n_slots);
 int qkk_moe_decode(const qkk_moe_layer *L_host, const float *X, float *Y, qkk_sel *sel,
                    void *workspace, size_t workspace_bytes, uint32_t n_slots, void *stream);
 
+/* The step followed by the layer tail (reference src/main.cpp:4379-4402 with add_rms3.comp:24-41,
+ * for several rows add_rms3_grouped.comp:22-50):
+ *   S[r]  = resid[r] + (routed + shared contribution of row r)    the next layer's residual input
+ *   Xn[r] = S[r] * w_next / sqrt(mean(S[r]^2) + eps)              normalised with the NEXT layer's weight
+ * X, sel, workspace, n_slots as for qkk_moe_decode.  resid may be S (in place); Xn must be a buffer
+ * of its own.  With several rows the tail runs inside the launch that sums the experts' slots, so
+ * the step's output is never written on its own; with one row it costs one more small launch. */
+int qkk_moe_decode_tail(const qkk_moe_layer *L_host, const float *X, const float *resid,
+                        const float *w_next, float eps, float *S, float *Xn, qkk_sel *sel,
+                        void *workspace, size_t workspace_bytes, uint32_t n_slots, void *stream);
+
 /* The same step cut at its launch boundaries, for per-stage timing (the reference times its
  * MoE stages separately under QK_STEP_PROF, src/main.cpp:4173-4185, 4591-4632).  `stages` is
  * a mask of QKK_STAGE_*; a stage reads what the earlier stages of a previous call left in

@@ -58,6 +58,7 @@ def lib():
         L.qkk_gemv.argtypes = [C.c_int, vp, vp, vp, u32, u32, u32, vp]
         L.qkk_moe_decode.argtypes = [vp, vp, vp, vp, vp, sz, u32, vp]
         L.qkk_moe_decode_stages.argtypes = [vp, vp, vp, vp, vp, sz, u32, u32, vp]
+        L.qkk_moe_decode_tail.argtypes = [vp, vp, vp, vp, C.c_float, vp, vp, vp, vp, sz, u32, vp]
         L.qkk_moe_group_pairs.argtypes = [vp, u32, u32, u32, vp, vp, vp]
         L.qkk_head_argmax.argtypes = [vp, vp, vp, vp, u32, u32, u32, vp, sz, vp]
         L.qkk_argmax.argtypes = [vp, vp, u32, u32, vp]
@@ -162,6 +163,21 @@ def moe_decode(layer, X, workspace, Y=None, sel=None, stages=None):
         _check(lib().qkk_moe_decode_stages(C.byref(layer.c), _ptr(X), _ptr(Y), _ptr(sel), _ptr(workspace), wsb,
                                            n, stages, _stream()))
     return Y, sel
+
+
+def moe_decode_tail(layer, X, resid, w_next, workspace, eps=1e-6, S=None, Xn=None, sel=None):
+    """The MoE step with the layer tail: S = resid + step(X), Xn = rmsnorm(S) * w_next.
+    Returns (S, Xn, sel).  S may be resid."""
+    import torch
+    n = X.shape[0]
+    S = torch.empty_like(X) if S is None else S
+    Xn = torch.empty_like(X) if Xn is None else Xn
+    if sel is None:
+        sel = torch.zeros((n, 160), dtype=torch.uint8, device=X.device)
+    _check(lib().qkk_moe_decode_tail(C.byref(layer.c), _ptr(X), _ptr(resid), _ptr(w_next), eps, _ptr(S), _ptr(Xn),
+                                     _ptr(sel), _ptr(workspace), workspace.numel() * workspace.element_size(), n,
+                                     _stream()))
+    return S, Xn, sel
 
 
 def moe_prefill_workspace_bytes(layer, n_tokens):

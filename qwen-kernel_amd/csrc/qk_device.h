@@ -128,6 +128,16 @@ __device__ __forceinline__ float lanes_sum(float v)
     else return group_sum<N>(v);
 }
 
+// Sum over a workgroup of four waves (256 threads, all of them calling) in wave order; every
+// thread returns the same bits.  s_red: four floats of LDS.
+__device__ __forceinline__ float block_sum4(float v, float* s_red)
+{
+    const float w = wave_sum(v);
+    if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = w;
+    __syncthreads();
+    return ((s_red[0] + s_red[1]) + s_red[2]) + s_red[3];
+}
+
 __device__ __forceinline__ float wave_max(float v)
 {
     v = fmaxf(v, dpp_f<DPP_XOR1>(v));

@@ -15,15 +15,6 @@
 
 namespace qk {
 
-// Sum over the workgroup's four waves in wave order; every thread returns the same bits.
-__device__ __forceinline__ float block_sum4(float v, float* s_red)
-{
-    const float w = wave_sum(v);
-    if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = w;
-    __syncthreads();
-    return ((s_red[0] + s_red[1]) + s_red[2]) + s_red[3];
-}
-
 // Rows of n floats, n % 4 == 0, n <= 1024 * VPT, all pointers 16-byte aligned.
 template <int NIN, int VPT>
 __global__ __launch_bounds__(256) void add_rmsnorm_kernel(const float* a, const float* b, const float* c,
@@ -122,6 +113,13 @@ static void launch_norm(const float* a, const float* b, const float* c, const fl
         hipLaunchKernelGGL((add_rmsnorm_kernel<NIN, 4>), grid, block, 0, st, a, b, c, w, sum_out, xn, n, eps);
     else
         hipLaunchKernelGGL((add_rmsnorm_kernel<NIN, 8>), grid, block, 0, st, a, b, c, w, sum_out, xn, n, eps);
+}
+
+// y = a + b, xn = y * scale(y) * w for `rows` rows (arguments already validated, launch not checked).
+void launch_add_rmsnorm(const float* a, const float* b, const float* w, float* y, float* xn, uint32_t n, uint32_t rows,
+                        float eps, hipStream_t st)
+{
+    launch_norm<2>(a, b, nullptr, w, y, xn, n, rows, eps, st);
 }
 
 static int norm_entry(const char* who, int nin, const float* a, const float* b, const float* c, const float* w,

@@ -233,7 +233,9 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const uint8_t* __restrict
 
 namespace qk {
 int moe_grouped_launch(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* sel, void* workspace,
-                       uint32_t N, uint32_t stages, hipStream_t st);
+                       uint32_t N, uint32_t stages, hipStream_t st, const MoeTail* tail);
+void launch_add_rmsnorm(const float* a, const float* b, const float* w, float* y, float* xn, uint32_t n, uint32_t rows,
+                        float eps, hipStream_t st);
 }
 using namespace qk;
 
@@ -303,7 +305,7 @@ size_t qkk_moe_workspace_bytes(const qkk_moe_layer* L, uint32_t n_slots)
 
 static int moe_decode_impl(const char* who, const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* sel,
                            void* workspace, size_t workspace_bytes, uint32_t n_slots, uint32_t stages,
-                           void* stream)
+                           void* stream, const MoeTail* tail = nullptr)
 {
     if (int rc = check_layer(L, who)) return rc;
     if (!X || !Y || !sel || !workspace) return fail(QKK_EINVAL, "%s: null pointer", who);
@@ -315,7 +317,7 @@ static int moe_decode_impl(const char* who, const qkk_moe_layer* L, const float*
         return fail(QKK_EWORKSPACE, "%s: workspace %zu < %zu bytes", who, workspace_bytes, ws_bytes(d, n_slots));
     if (int rc = require_device()) return rc;
     hipStream_t st = as_stream(stream);
-    if (n_slots >= 2) return moe_grouped_launch(L, X, Y, sel, workspace, n_slots, stages, st);
+    if (n_slots >= 2) return moe_grouped_launch(L, X, Y, sel, workspace, n_slots, stages, st, tail);
     const MoeWs ws = ws_carve(workspace, d, n_slots);
 
     if (stages & QKK_STAGE_ROUTE) {
@@ -344,6 +346,8 @@ static int moe_decode_impl(const char* who, const qkk_moe_layer* L, const float*
     if (stages & QKK_STAGE_DOWN) {
         if (L->down_type == QKK_IQ4_XS) launch_down<QKK_IQ4_XS>(L, ws, sel, Y, d, n_slots, st);
         else launch_down<QKK_Q6_K>(L, ws, sel, Y, d, n_slots, st);
+        // one row: the step's output went to tail->Xn (see qkk_moe_decode_tail); add and norm in place
+        if (tail) launch_add_rmsnorm(tail->resid, Y, tail->w_next, tail->S, tail->Xn, d.H, 1, tail->eps, st);
     }
     return check_launch(who);
 }
@@ -353,6 +357,22 @@ int qkk_moe_decode(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* se
 {
     return moe_decode_impl("qkk_moe_decode", L, X, Y, sel, workspace, workspace_bytes, n_slots, QKK_STAGE_ALL,
                            stream);
+}
+
+int qkk_moe_decode_tail(const qkk_moe_layer* L, const float* X, const float* resid, const float* w_next, float eps,
+                        float* S, float* Xn, qkk_sel* sel, void* workspace, size_t workspace_bytes, uint32_t n_slots,
+                        void* stream)
+{
+    if (!resid || !w_next || !S || !Xn) return fail(QKK_EINVAL, "qkk_moe_decode_tail: null pointer");
+    if (!aligned16(resid) || !aligned16(w_next) || !aligned16(S) || !aligned16(Xn))
+        return fail(QKK_EINVAL, "qkk_moe_decode_tail: resid, w_next, S and Xn must be 16-byte aligned");
+    if (!(eps >= 0.f)) return fail(QKK_EINVAL, "qkk_moe_decode_tail: eps must be non-negative");
+    if (Xn == X || Xn == resid || Xn == S)
+        return fail(QKK_EINVAL, "qkk_moe_decode_tail: Xn must be a buffer of its own (it holds the step's output on the way)");
+    const MoeTail tail{resid, w_next, eps, S, Xn};
+    // the step writes its output row(s) to Xn when it has to materialise them (one row)
+    return moe_decode_impl("qkk_moe_decode_tail", L, X, Xn, sel, workspace, workspace_bytes, n_slots, QKK_STAGE_ALL, stream,
+                           &tail);
 }
 
 int qkk_moe_decode_stages(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* sel, void* workspace,

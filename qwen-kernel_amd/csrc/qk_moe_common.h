@@ -33,6 +33,15 @@ struct MoeWs {
     float* contrib;       // [n][k+1][H], slot k = shared expert
 };
 
+// Layer tail behind the step: S = resid + (routed + shared), Xn = S * scale(S) * w_next.
+struct MoeTail {
+    const float* resid;
+    const float* w_next;
+    float eps;
+    float* S;
+    float* Xn;
+};
+
 static inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 static inline size_t ws_bytes(const MoeDims& d, uint32_t n)

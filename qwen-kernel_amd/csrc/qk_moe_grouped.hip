@@ -232,6 +232,8 @@ void moe_mfma_launch_shared(const qkk_moe_layer* L, const float* X, const qkk_se
 void moe_mfma_launch_routed(const qkk_moe_layer* L, const float* X, const qkk_sel* sel, const MoeWs& ws,
                             const MoeDims& d, uint32_t N, uint32_t stages, hipStream_t st);
 void moe_mfma_launch_fold(float* Y, const qkk_sel* sel, const MoeWs& ws, const MoeDims& d, uint32_t N, hipStream_t st);
+void moe_mfma_launch_fold_norm(const float* resid, const float* w_next, float eps, float* S, float* Xn,
+                               const qkk_sel* sel, const MoeWs& ws, const MoeDims& d, uint32_t N, hipStream_t st);
 void moe_mfma_launch_fused(const qkk_moe_layer* L, const float* X, const qkk_sel* sel, const MoeWs& ws,
                            const MoeDims& d, uint32_t N, uint32_t stages, hipStream_t st);
 constexpr uint32_t FUSED_MAX_ROWS = 32; // up to here the shared expert rides in the routed experts' launches
@@ -262,7 +264,7 @@ static SideStream* side_stream()
 
 // Host entry of the path for N >= 2 rows (arguments already validated).
 int moe_grouped_launch(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* sel, void* workspace,
-                       uint32_t N, uint32_t stages, hipStream_t st)
+                       uint32_t N, uint32_t stages, hipStream_t st, const MoeTail* tail)
 {
     const MoeDims d{L->n_embd, L->n_ff, L->n_expert, L->n_used};
     // the matrix-core kernels split n_embd over the eight waves of a workgroup, 256 weights each
@@ -304,7 +306,10 @@ int moe_grouped_launch(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel
         if (hipEventRecord(side->join, side->stream) != hipSuccess || hipStreamWaitEvent(st, side->join, 0) != hipSuccess)
             return fail(QKK_EDEVICE, "moe: joining the shared-expert stream failed");
     }
-    if (stages & QKK_STAGE_DOWN) moe_mfma_launch_fold(Y, sel, ws, d, N, st);
+    if (stages & QKK_STAGE_DOWN) {
+        if (tail) moe_mfma_launch_fold_norm(tail->resid, tail->w_next, tail->eps, tail->S, tail->Xn, sel, ws, d, N, st);
+        else moe_mfma_launch_fold(Y, sel, ws, d, N, st);
+    }
     return check_launch("moe grouped path");
 }
 

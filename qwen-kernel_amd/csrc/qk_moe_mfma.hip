@@ -176,6 +176,48 @@ __global__ __launch_bounds__(256) void moe_fold_kernel(MoeWs ws, const qkk_sel* 
     }
 }
 
+// The fold with the layer tail behind it, one workgroup per token (n_embd = 2048: two quads per
+// thread):  s = (resid + sum of the routed slots in slot order) + shared gate * shared slot, stored
+// as the next residual, and xn = s * scale(s) * w with the NEXT layer's norm weight
+// (reference shaders/add_rms3_grouped.comp:22-50).  resid may be S.
+__global__ __launch_bounds__(256) void moe_fold_norm_kernel(MoeWs ws, const qkk_sel* __restrict__ sel, const float* resid,
+                                                            const float* __restrict__ w, float* S, float* __restrict__ Xn,
+                                                            MoeDims d, float eps)
+{
+    __shared__ float s_red[4];
+    const uint32_t t = blockIdx.x;
+    const float g = sel[t].w_shared;
+    float4 v[2];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const uint32_t o = 4 * (threadIdx.x + 256u * j);
+        float4 r = float4{0.f, 0.f, 0.f, 0.f};
+        for (uint32_t sl = 0; sl < d.k; sl++) {
+            const float4 c = *(const float4*)(ws.contrib + ((size_t)t * (d.k + 1) + sl) * d.H + o);
+            r.x += c.x; r.y += c.y; r.z += c.z; r.w += c.w;
+        }
+        const float4 a = *(const float4*)(resid + (size_t)t * d.H + o);
+        const float4 c = *(const float4*)(ws.contrib + ((size_t)t * (d.k + 1) + d.k) * d.H + o);
+        const float4 s = float4{(a.x + r.x) + g * c.x, (a.y + r.y) + g * c.y, (a.z + r.z) + g * c.z, (a.w + r.w) + g * c.w};
+        *(float4*)(S + (size_t)t * d.H + o) = s;
+        v[j] = s;
+        ss += s.x * s.x;
+        ss += s.y * s.y;
+        ss += s.z * s.z;
+        ss += s.w * s.w;
+    }
+    const float tot = block_sum4(ss, s_red);
+    const float scale = 1.f / sqrtf(tot / (float)d.H + eps);
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const uint32_t o = 4 * (threadIdx.x + 256u * j);
+        const float4 gw = *(const float4*)(w + o);
+        *(float4*)(Xn + (size_t)t * d.H + o) =
+            float4{v[j].x * scale * gw.x, v[j].y * scale * gw.y, v[j].z * scale * gw.z, v[j].w * scale * gw.w};
+    }
+}
+
 // ==== few rows (up to FUSED_MAX_ROWS): one gate/up and one down launch take the shared expert's and
 // the routed experts' items together (a HIP graph runs the side stream's launches of so short a
 // step one after the other, which costs more than it saves).  Items: first the shared expert's
@@ -465,6 +507,13 @@ void moe_mfma_launch_fold(float* Y, const qkk_sel* sel, const MoeWs& ws, const M
 {
     const uint32_t fb = (uint32_t)std::min<uint64_t>(((uint64_t)N * d.H / 4 + 255) / 256, persistent_blocks());
     hipLaunchKernelGGL(moe_fold_kernel, dim3(fb), dim3(256), 0, st, ws, sel, Y, d, N);
+}
+
+// The same with the residual add and the next layer's RMS norm (n_embd = 2048).
+void moe_mfma_launch_fold_norm(const float* resid, const float* w_next, float eps, float* S, float* Xn,
+                               const qkk_sel* sel, const MoeWs& ws, const MoeDims& d, uint32_t N, hipStream_t st)
+{
+    hipLaunchKernelGGL(moe_fold_norm_kernel, dim3(N), dim3(256), 0, st, ws, sel, resid, w_next, S, Xn, d, eps);
 }
 
 } // namespace qk

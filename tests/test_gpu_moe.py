@@ -250,6 +250,38 @@ def test_moe_layer_loaded_from_gguf(qk, orc, dev, tmp_path):
             assert orc.rel_maxabs_err(Y[s], refs[s]["y"]) <= TOL
 
 
+@pytest.mark.parametrize("n", [1, 2, 16, 40])
+def test_moe_decode_tail(qk, orc, dev, layer_iq4, n):
+    """Step + residual + next layer's RMS norm in one call against the oracle's step followed by its
+    norm (reference src/main.cpp:4379-4402); the plain step on the same rows gives the same picks,
+    and S - resid is that step's output up to fp32 rounding of the sum."""
+    import torch
+    print(f"[case] moe step with layer tail, {n} rows", flush=True)
+    X, refs = pick_inputs(orc, layer_iq4, n, seed=70 + n)
+    rng = np.random.default_rng(n)
+    resid = rng.standard_normal((n, 2048)).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, 2048).astype(np.float32)
+    y = np.stack([r["y"] for r in refs])
+    want_s, want_xn = orc.add_rms(resid, w, 1e-6, b=y, want_sum=True)
+    layer = layer_iq4.to_device(dev)
+    ws = torch.zeros(qk.moe_workspace_bytes(layer, n), dtype=torch.uint8, device=dev)
+    Xd, Rd, Wd = (torch.from_numpy(a).to(dev) for a in (X, resid, w))
+    S, Xn, sel = qk.moe_decode_tail(layer, Xd, Rd, Wd, ws)
+    torch.cuda.synchronize()
+    ids, _, _ = sel_fields(sel)
+    for s in range(n):
+        assert list(ids[s, :8]) == list(refs[s]["sel"].ids[:8])
+    scale_y = np.max(np.abs(y))
+    assert np.max(np.abs(S.cpu().numpy() - want_s)) <= TOL * scale_y
+    assert orc.rel_maxabs_err(Xn.cpu().numpy(), want_xn) <= TOL
+    # in place: the residual buffer receives S; same bits as out of place
+    S2, Xn2, _ = qk.moe_decode_tail(layer, Xd, Rd, Wd, ws, S=Rd)
+    torch.cuda.synchronize()
+    assert S2.data_ptr() == Rd.data_ptr() and torch.equal(S2, S) and torch.equal(Xn2, Xn)
+    with pytest.raises(qk.QkError):
+        qk.moe_decode_tail(layer, Xd, Rd, Wd, ws, Xn=Xd)
+
+
 def test_group_pairs_matches_oracle(qk, orc, dev):
     import torch
     print("[case] group pairs", flush=True)
