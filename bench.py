@@ -127,6 +127,37 @@ def moe_workload(qk, n_slots, down_type, ring, steps, warmup, seed=1234):
                 gateup_bytes=gu_bytes, ring=ring, ring_bytes=ring * L.active_bytes(L.n_expert))
 
 
+def moe_tail_workload(qk, n_slots, down_type, ring, steps, warmup, seed=1234):
+    """The step with the layer tail behind it (qkk_moe_decode_tail): residual add and the next
+    layer's RMS norm.  Same ring and inputs as moe_workload; returns microseconds per step."""
+    import torch
+    dev = "cuda:0"
+    layers = [qk.synth.device_layer(seed + 16 * i, down_type=down_type, device=dev) for i in range(ring)]
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    X = torch.randn((ring, n_slots, 2048), device=dev, generator=g)
+    R = torch.randn((ring, n_slots, 2048), device=dev, generator=g)
+    W = torch.rand((ring, 2048), device=dev, generator=g) + 0.5
+    S, Xn = torch.empty_like(X), torch.empty_like(X)
+    sel = torch.zeros((ring, n_slots, 160), dtype=torch.uint8, device=dev)
+    ws = torch.zeros(qk.moe_workspace_bytes(layers[0], n_slots), dtype=torch.uint8, device=dev)
+    _, ev, _ = run_ring([(lambda i=i: qk.moe_decode_tail(layers[i], X[i], R[i], W[i], ws, S=S[i], Xn=Xn[i], sel=sel[i]))
+                         for i in range(ring)], steps, warmup)
+    return ev * 1e3
+
+
+def norm_workload(qk, rows, steps, warmup):
+    """add_rmsnorm on `rows` rows of 2048 (ring of 64 distinct row sets)."""
+    import torch
+    dev = "cuda:0"
+    ring = 64
+    A, B = torch.randn((2, ring, rows, 2048), device=dev)
+    W = torch.rand(2048, device=dev) + 0.5
+    Y, Xn = torch.empty_like(A), torch.empty_like(A)
+    _, ev, _ = run_ring([(lambda i=i: qk.add_rmsnorm(A[i], B[i], W, y=Y[i], xn=Xn[i])) for i in range(ring)], steps, warmup)
+    return ev * 1e3
+
+
 def gemv_workload(qk, type_, M, K, batch, steps, warmup, seed=99):
     import torch
     dev = "cuda:0"
@@ -335,6 +366,14 @@ def main():
                                                   frac=m16["bytes_step"] / (m16["ms_event"] * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                                                   stage_us={k: v * 1e3 for k, v in m16["stage_ms"].items()})
             log(f"[bench] moe bs16: {ex['moe_decode_bs16_q6k_down']}")
+            torch.cuda.empty_cache()
+            # layer glue (add + RMS norm alone, and behind the step in one call)
+            ex["add_rmsnorm_2048"] = dict(us_1_row=norm_workload(qk, 1, 640, 64), us_16_rows=norm_workload(qk, 16, 640, 64))
+            ex["moe_decode_tail_bs1"] = dict(us=moe_tail_workload(qk, 1, qk.IQ4_XS, 8, 400, 40))
+            torch.cuda.empty_cache()
+            ex["moe_decode_tail_bs16_q6k_down"] = dict(us=moe_tail_workload(qk, 16, qk.Q6_K, 4, 200, 20))
+            log(f"[bench] glue: {ex['add_rmsnorm_2048']} tail bs1 {ex['moe_decode_tail_bs1']} "
+                f"bs16 {ex['moe_decode_tail_bs16_q6k_down']}")
             torch.cuda.empty_cache()
             g = gemm_workload(qk, 8192, 2048, 128, 200, 20)
             ex["prefill_gemm_q8_0_8192x2048x128"] = dict(us=g["ms_event"] * 1e3, tflops=g["flops"] / (g["ms_event"] * 1e-3) / 1e12,

@@ -157,6 +157,22 @@ __global__ __launch_bounds__(CT) void moe_down_mfma_kernel(const uint8_t* __rest
     }
 }
 
+// Sum of the k routed slots of one token at outputs o..o+3, in slot order; the loads of eight
+// slots are issued together (k is a run-time value: a plain loop would wait for each in turn).
+__device__ __forceinline__ float4 sum_routed_slots(const float* __restrict__ contrib_tok, uint32_t k, uint32_t H, uint32_t o)
+{
+    float4 r = float4{0.f, 0.f, 0.f, 0.f};
+    for (uint32_t base = 0; base < k; base += 8) {
+        float4 c[8];
+#pragma unroll
+        for (uint32_t i = 0; i < 8; i++)
+            c[i] = base + i < k ? *(const float4*)(contrib_tok + (size_t)(base + i) * H + o) : float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (uint32_t i = 0; i < 8; i++) { r.x += c[i].x; r.y += c[i].y; r.z += c[i].z; r.w += c[i].w; } // + 0 is exact
+    }
+    return r;
+}
+
 // ---- fold: Y[t][o] = sum over the k routed slots in slot order + shared gate * shared slot ---------------
 __global__ __launch_bounds__(256) void moe_fold_kernel(MoeWs ws, const qkk_sel* __restrict__ sel,
                                                        float* __restrict__ Y, MoeDims d, uint32_t N)
@@ -164,11 +180,7 @@ __global__ __launch_bounds__(256) void moe_fold_kernel(MoeWs ws, const qkk_sel* 
     const uint32_t quads = d.H / 4;
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < (size_t)N * quads; i += (size_t)gridDim.x * 256) {
         const uint32_t t = (uint32_t)(i / quads), o = (uint32_t)(i % quads) * 4;
-        float4 s = float4{0.f, 0.f, 0.f, 0.f};
-        for (uint32_t sl = 0; sl < d.k; sl++) {
-            const float4 c = *(const float4*)(ws.contrib + ((size_t)t * (d.k + 1) + sl) * d.H + o);
-            s.x += c.x; s.y += c.y; s.z += c.z; s.w += c.w;
-        }
+        float4 s = sum_routed_slots(ws.contrib + (size_t)t * (d.k + 1) * d.H, d.k, d.H, o);
         const float g = sel[t].w_shared;
         const float4 c = *(const float4*)(ws.contrib + ((size_t)t * (d.k + 1) + d.k) * d.H + o);
         s.x += g * c.x; s.y += g * c.y; s.z += g * c.z; s.w += g * c.w;
@@ -192,11 +204,7 @@ __global__ __launch_bounds__(256) void moe_fold_norm_kernel(MoeWs ws, const qkk_
 #pragma unroll
     for (int j = 0; j < 2; j++) {
         const uint32_t o = 4 * (threadIdx.x + 256u * j);
-        float4 r = float4{0.f, 0.f, 0.f, 0.f};
-        for (uint32_t sl = 0; sl < d.k; sl++) {
-            const float4 c = *(const float4*)(ws.contrib + ((size_t)t * (d.k + 1) + sl) * d.H + o);
-            r.x += c.x; r.y += c.y; r.z += c.z; r.w += c.w;
-        }
+        const float4 r = sum_routed_slots(ws.contrib + (size_t)t * (d.k + 1) * d.H, d.k, d.H, o);
         const float4 a = *(const float4*)(resid + (size_t)t * d.H + o);
         const float4 c = *(const float4*)(ws.contrib + ((size_t)t * (d.k + 1) + d.k) * d.H + o);
         const float4 s = float4{(a.x + r.x) + g * c.x, (a.y + r.y) + g * c.y, (a.z + r.z) + g * c.z, (a.w + r.w) + g * c.w};
