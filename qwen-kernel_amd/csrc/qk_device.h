@@ -128,6 +128,18 @@ __device__ __forceinline__ float lanes_sum(float v)
     else return group_sum<N>(v);
 }
 
+// Inclusive prefix sum over the 64 lanes of a wave.
+__device__ __forceinline__ uint32_t wave_incl_scan_u32(uint32_t v)
+{
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t t = __shfl_up(v, d);
+        if (lane >= d) v += t;
+    }
+    return v;
+}
+
 // Sum over a workgroup of four waves (256 threads, all of them calling) in wave order; every
 // thread returns the same bits.  s_red: four floats of LDS.
 __device__ __forceinline__ float block_sum4(float v, float* s_red)

@@ -95,44 +95,63 @@ __device__ __forceinline__ void pair_at(const MoeWs& ws, uint32_t p, const MoeDi
 }
 
 // ---- selector --------------------------------------------------------------------------
-// One wave; lane L owns logits L, L+64, ...  Picks n_used times the maximum, lower id on
-// ties; non-finite logits count as -3.4e38 (reference shaders/moe_select.comp:28-34, 53-63).
-__device__ static inline void select_wave(const float* __restrict__ logits, uint32_t E, uint32_t k,
-                                   qkk_sel* __restrict__ out)
+// One wave; lane L owns logits L, L+64, ... (NR register slots cover 64*NR experts).  Picks n_used
+// times the maximum, lower id on ties; non-finite logits count as -3.4e38; weights exp(l - l0) over
+// the picks, summed in pick order (reference shaders/moe_select.comp:28-34, 53-76).
+// The loop is a chain of dependent wave-wide steps, so it is kept short: the exponentials are taken
+// after it, by the lanes in parallel, and a tie for the maximum -- the only case that needs a second
+// wave-wide reduction -- is detected with a ballot.
+template <int NR>
+__device__ static inline void select_wave_n(const float* __restrict__ logits, uint32_t E, uint32_t k,
+                                            qkk_sel* __restrict__ out, uint32_t* ids_copy)
 {
     constexpr float FLOOR = -3.4e38f;
     const int lane = threadIdx.x & 63;
-    float v[QKK_MAX_EXPERTS / 64];
+    float v[NR];
 #pragma unroll
-    for (int i = 0; i < (int)(QKK_MAX_EXPERTS / 64); i++) {
+    for (int i = 0; i < NR; i++) {
         const uint32_t e = lane + 64 * i;
         float l = e < E ? logits[e] : FLOOR;
         if (isnan(l) || isinf(l)) l = FLOOR;
         v[i] = l;
     }
-    float picked = 0.f, top = 0.f, wsum = 0.f, myw = 0.f;
+    float top = 0.f, mym = 0.f;
     uint32_t myid = 0;
     for (uint32_t r = 0; r < k; r++) {
         float bv = v[0];
         uint32_t bi = lane;
 #pragma unroll
-        for (int i = 1; i < (int)(QKK_MAX_EXPERTS / 64); i++)
+        for (int i = 1; i < NR; i++)
             if (v[i] > bv) { bv = v[i]; bi = lane + 64 * i; }
         const float m = wave_max(bv);
-        const uint32_t id = wave_min_u32(bv == m ? bi : 0x7FFFFFFFu);
+        const uint64_t tie = __builtin_amdgcn_ballot_w64(bv == m); // never empty: m is some lane's bv
+        uint32_t id;
+        if (__builtin_popcountll(tie) == 1) // wave-uniform
+            id = (uint32_t)__builtin_amdgcn_readlane((int)bi, __builtin_ctzll(tie));
+        else
+            id = wave_min_u32(bv == m ? bi : 0x7FFFFFFFu);
         // retire the winner
 #pragma unroll
-        for (int i = 0; i < (int)(QKK_MAX_EXPERTS / 64); i++)
+        for (int i = 0; i < NR; i++)
             if ((uint32_t)(lane + 64 * i) == id) v[i] = FLOOR;
         if (r == 0) top = m;
-        picked = expf(m - top);
-        wsum += picked;
-        if ((uint32_t)lane == r) { myw = picked; myid = min(id, E - 1); }
+        if ((uint32_t)lane == r) { mym = m; myid = min(id, E - 1); }
     }
+    const float p = (uint32_t)lane < k ? expf(mym - top) : 0.f;
+    float wsum = 0.f;
+    for (uint32_t r = 0; r < k; r++) wsum += readlane_f(p, (int)r); // pick order
     if ((uint32_t)lane < k) {
         out->ids[lane] = myid;
-        out->w[lane] = myw / wsum;
+        out->w[lane] = p / wsum;
+        if (ids_copy) ids_copy[lane] = myid; // for a grouping pass in the same workgroup (LDS)
     }
+}
+
+__device__ static inline void select_wave(const float* __restrict__ logits, uint32_t E, uint32_t k,
+                                          qkk_sel* __restrict__ out, uint32_t* ids_copy = nullptr)
+{
+    if (E <= 256) select_wave_n<4>(logits, E, k, out, ids_copy);
+    else select_wave_n<QKK_MAX_EXPERTS / 64>(logits, E, k, out, ids_copy);
 }
 
 } // namespace qk

@@ -16,83 +16,84 @@ namespace qk {
 
 constexpr uint32_t SELECT_INLINE_MAX = 32; // up to this many tokens the route launch also selects
 
-// ---- selection: one wave takes the tokens first, first+stride, ... ----------------------------
+// ---- selection: one wave takes the tokens first, first+stride, ... TPW (1 or 2) at a time ---------
 // (logits written by other workgroups: the caller's acquire fence, or a kernel boundary, precedes)
+// my_log: TPW areas of LOG_AREA floats of LDS for this wave.  ids_lds: when not null the picks of
+// token t are also left at ids_lds[16*t ..] for a grouping pass by the same workgroup.
+constexpr uint32_t LOG_AREA = QKK_MAX_EXPERTS + 8;
+template <int TPW>
 __device__ static void select_tokens(const MoeWs& ws, qkk_sel* __restrict__ sel, MoeDims d, uint32_t N,
-                                     uint32_t first, uint32_t stride, float* my_log, bool publish_ids)
+                                     uint32_t first, uint32_t stride, float* my_log, uint32_t* ids_lds, bool publish_ids)
 {
     const int lane = threadIdx.x & 63;
-    for (uint32_t t = first; t < N; t += stride) {
-        // plain loads, all issued before the first use
-        const float* gl = ws.logits + (size_t)t * lstride(d.E);
-        float lv[QKK_MAX_EXPERTS / 64 + 1];
+    constexpr int NL = QKK_MAX_EXPERTS / 64 + 1;
+    for (uint32_t t0 = first; t0 < N; t0 += TPW * stride) {
+        // plain loads of the logits of all TPW tokens, issued before the first use: one round trip
+        float lg[TPW][NL];
 #pragma unroll
-        for (int i = 0; i <= (int)(QKK_MAX_EXPERTS / 64); i++)
-            lv[i] = (uint32_t)(lane + 64 * i) <= d.E ? gl[lane + 64 * i] : 0.f;
+        for (int h = 0; h < TPW; h++) {
+            const float* g = ws.logits + (size_t)min(t0 + h * stride, N - 1) * lstride(d.E);
 #pragma unroll
-        for (int i = 0; i <= (int)(QKK_MAX_EXPERTS / 64); i++)
-            if ((uint32_t)(lane + 64 * i) <= d.E) my_log[lane + 64 * i] = lv[i];
+            for (int i = 0; i < NL; i++) lg[h][i] = (uint32_t)(lane + 64 * i) <= d.E ? g[lane + 64 * i] : 0.f;
+        }
+#pragma unroll
+        for (int h = 0; h < TPW; h++)
+#pragma unroll
+            for (int i = 0; i < NL; i++)
+                if ((uint32_t)(lane + 64 * i) <= d.E) my_log[h * LOG_AREA + lane + 64 * i] = lg[h][i];
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        select_wave(my_log, d.E, d.k, &sel[t]);
-        if (lane == 0) sel[t].w_shared = 1.f / (1.f + expf(-my_log[d.E]));
-        // the grouping workgroup of the same launch reads the ids: write them through
-        if (publish_ids && (uint32_t)lane < d.k) publish(&sel[t].ids[lane], sel[t].ids[lane]);
+#pragma unroll
+        for (int h = 0; h < TPW; h++) {
+            const uint32_t t = t0 + h * stride;
+            if (t >= N) break; // the whole wave
+            const float* l = my_log + h * LOG_AREA;
+            select_wave(l, d.E, d.k, &sel[t], ids_lds ? ids_lds + 16 * t : nullptr);
+            if (lane == 0) sel[t].w_shared = 1.f / (1.f + expf(-l[d.E]));
+            // a grouping workgroup elsewhere in the launch reads the ids: write them through
+            if (publish_ids && (uint32_t)lane < d.k) publish(&sel[t].ids[lane], sel[t].ids[lane]);
+        }
         __builtin_amdgcn_wave_barrier();
     }
 }
 
 // ---- grouping of the N*k (token, pick) pairs by expert, by one workgroup of NW waves ----------
+// ids: the picks of token t at ids_lds[16*t ..] when this workgroup selected them itself (LDS), else
+// read from sel with loads that bypass the L1 (other workgroups of the launch published them).
+// One expert per thread: counts by LDS atomics, exclusive offsets by a wave scan plus the sum of
+// the earlier waves' totals, then the pairs are scattered behind per-expert LDS cursors.
 template <int NW>
-__device__ static void group_pairs_wg(const MoeWs& ws, qkk_sel* __restrict__ sel, MoeDims d, uint32_t N,
-                                      uint32_t* s_cnt, uint32_t* s_cur)
+__device__ static void group_pairs_wg(const MoeWs& ws, qkk_sel* __restrict__ sel, const uint32_t* ids_lds, MoeDims d,
+                                      uint32_t N, uint32_t* s_cnt, uint32_t* s_cur)
 {
-    for (uint32_t e = threadIdx.x; e <= QKK_MAX_EXPERTS; e += NW * 64) s_cnt[e] = 0;
-    __threadfence_block();
+    static_assert(NW * 64 >= (int)QKK_MAX_EXPERTS, "one expert per thread");
+    __shared__ uint32_t s_part[NW];
+    const uint32_t e = threadIdx.x, lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    for (uint32_t i = threadIdx.x; i <= QKK_MAX_EXPERTS; i += NW * 64) s_cnt[i] = 0;
     __syncthreads();
     const uint32_t np = N * d.k;
     const volatile qkk_sel* vs = sel;
-    for (uint32_t p = threadIdx.x; p < np; p += NW * 64)
-        atomicAdd(&s_cnt[min(vs[p / d.k].ids[p % d.k], d.E - 1)], 1u);
+    const auto id_of = [&](uint32_t p) -> uint32_t {
+        const uint32_t t = p / d.k, s = p % d.k;
+        return min(ids_lds ? ids_lds[16 * t + s] : vs[t].ids[s], d.E - 1);
+    };
+    for (uint32_t p = threadIdx.x; p < np; p += NW * 64) atomicAdd(&s_cnt[id_of(p)], 1u);
     __syncthreads();
-    // exclusive scan over the experts of (pair count, "has pairs" flag), packed count | flag<<20
-    // (count <= 4096*16 < 2^20): Hillis-Steele in LDS, two experts per thread when NW = 4
-    constexpr uint32_t PER = (QKK_MAX_EXPERTS + NW * 64 - 1) / (NW * 64);
-    uint32_t mine[PER], incl[PER];
-#pragma unroll
-    for (uint32_t j = 0; j < PER; j++) {
-        const uint32_t e = threadIdx.x + j * NW * 64;
-        const uint32_t c = e < d.E ? s_cnt[e] : 0u;
-        mine[j] = c | (c ? 1u << 20 : 0u);
-        incl[j] = mine[j];
-    }
-    for (uint32_t step = 1; step < QKK_MAX_EXPERTS; step <<= 1) {
-#pragma unroll
-        for (uint32_t j = 0; j < PER; j++) {
-            const uint32_t e = threadIdx.x + j * NW * 64;
-            if (e < QKK_MAX_EXPERTS) s_cur[e] = incl[j];
-        }
-        __syncthreads();
-#pragma unroll
-        for (uint32_t j = 0; j < PER; j++) {
-            const uint32_t e = threadIdx.x + j * NW * 64;
-            if (e < QKK_MAX_EXPERTS && e >= step) incl[j] += s_cur[e - step];
-        }
-        __syncthreads();
-    }
-#pragma unroll
-    for (uint32_t j = 0; j < PER; j++) {
-        const uint32_t e = threadIdx.x + j * NW * 64;
-        if (e >= QKK_MAX_EXPERTS) continue;
-        const uint32_t excl = incl[j] - mine[j];
-        const uint32_t off = excl & 0xFFFFFu, rank = excl >> 20, c = mine[j] & 0xFFFFFu;
-        s_cur[e] = off;
-        if (e < d.E) {
-            ws.offsets[e] = off;
-            if (c) {
-                ActiveExpert a{e, off, c, 0};
-                ws.active[rank] = a;
-            }
+    // (pair count, "has pairs" flag) packed as count | flag << 20 (count <= 4096*16 < 2^20)
+    const uint32_t c = e < d.E ? s_cnt[e] : 0u;
+    const uint32_t mine = c | (c ? 1u << 20 : 0u);
+    uint32_t incl = wave_incl_scan_u32(mine);
+    if (lane == 63) s_part[wave] = incl;
+    __syncthreads();
+    for (uint32_t w = 0; w < wave; w++) incl += s_part[w];
+    const uint32_t excl = incl - mine;
+    const uint32_t off = excl & 0xFFFFFu, rank = excl >> 20;
+    if (e < QKK_MAX_EXPERTS) s_cur[e] = off;
+    if (e < d.E) {
+        ws.offsets[e] = off;
+        if (c) {
+            ActiveExpert a{e, off, c, 0};
+            ws.active[rank] = a;
         }
         if (e == d.E - 1) {
             ws.offsets[d.E] = off + c;
@@ -102,8 +103,7 @@ __device__ static void group_pairs_wg(const MoeWs& ws, qkk_sel* __restrict__ sel
     __syncthreads();
     for (uint32_t p = threadIdx.x; p < np; p += NW * 64) {
         const uint32_t t = p / d.k, s = p % d.k;
-        const uint32_t e = min(vs[t].ids[s], d.E - 1);
-        ws.pairs[min(atomicAdd(&s_cur[e], 1u), np - 1)] = (t << 4) | s; // in range even if sel changes under us
+        ws.pairs[min(atomicAdd(&s_cur[id_of(p)], 1u), np - 1)] = (t << 4) | s; // in range even if sel changes under us
     }
 }
 
@@ -121,8 +121,9 @@ __global__ __launch_bounds__(512) void moe_route_multi_kernel(const float* __res
     constexpr int TG = NCH <= 8 ? 4 : 2; // tokens per task
     constexpr int NW = 8;                // waves per block
     __shared__ uint32_t s_last;
-    __shared__ float s_log[NW * (QKK_MAX_EXPERTS + 8)];
+    __shared__ float s_log[NW * 2 * LOG_AREA];
     __shared__ uint32_t s_cnt[QKK_MAX_EXPERTS + 1], s_cur[QKK_MAX_EXPERTS + 1];
+    __shared__ uint32_t s_ids[SELECT_INLINE_MAX * 16]; // the picks of every token, for the grouping below
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t n_rows = d.E + 1;
     const uint32_t task = blockIdx.x * NW + wave;
@@ -158,8 +159,8 @@ __global__ __launch_bounds__(512) void moe_route_multi_kernel(const float* __res
     if (threadIdx.x == 0) s_last = arrive_last(&ws.counter[0], gridDim.x) ? 1u : 0u;
     __syncthreads();
     if (s_last) {
-        select_tokens(ws, sel, d, N, wave, NW, s_log + (size_t)wave * (QKK_MAX_EXPERTS + 8), false);
-        group_pairs_wg<NW>(ws, sel, d, N, s_cnt, s_cur);
+        select_tokens<2>(ws, sel, d, N, wave, NW, s_log + (size_t)wave * 2 * LOG_AREA, s_ids, false);
+        group_pairs_wg<NW>(ws, sel, s_ids, d, N, s_cnt, s_cur);
         if (threadIdx.x == 0) ws.counter[0] = 0u;
     }
 }
@@ -213,16 +214,16 @@ __global__ __launch_bounds__(512) void moe_logits_tiled_kernel(const float* __re
 __global__ __launch_bounds__(1024) void moe_select_group_kernel(MoeWs ws, qkk_sel* __restrict__ sel, MoeDims d,
                                                                 uint32_t N)
 {
-    __shared__ float s_log[16 * (QKK_MAX_EXPERTS + 8)];
+    __shared__ float s_log[16 * LOG_AREA];
     __shared__ uint32_t s_cnt[QKK_MAX_EXPERTS + 1], s_cur[QKK_MAX_EXPERTS + 1];
     __shared__ uint32_t s_last;
     const int wave = threadIdx.x >> 6;
-    select_tokens(ws, sel, d, N, blockIdx.x * 16 + wave, gridDim.x * 16, s_log + (size_t)wave * (QKK_MAX_EXPERTS + 8), true);
+    select_tokens<1>(ws, sel, d, N, blockIdx.x * 16 + wave, gridDim.x * 16, s_log + (size_t)wave * LOG_AREA, nullptr, true);
     __syncthreads();
     if (threadIdx.x == 0) s_last = arrive_last(&ws.counter[0], gridDim.x) ? 1u : 0u;
     __syncthreads();
     if (s_last) {
-        group_pairs_wg<16>(ws, sel, d, N, s_cnt, s_cur);
+        group_pairs_wg<16>(ws, sel, nullptr, d, N, s_cnt, s_cur);
         if (threadIdx.x == 0) ws.counter[0] = 0u;
     }
 }

@@ -158,6 +158,35 @@ def test_moe_nan_activations_keep_ids_in_range(qk, dev, layer_iq4):
     assert np.all(ids[:, :8] < 256)
 
 
+@pytest.mark.parametrize("n", [1, 3])
+def test_moe_tied_logits_pick_the_lower_id(qk, orc, dev, n):
+    """Two experts with identical router rows have identical logits: when both are picked the lower
+    id comes first, when one is picked it is the lower one (reference shaders/moe_select.comp:53-59)."""
+    import torch
+    print(f"[case] moe tied logits, {n} rows", flush=True)
+    hl = qk.synth.HostLayer(seed=77, n_expert=16, n_used=4, n_ff=256)
+    rng = np.random.default_rng(5)
+    for trial in range(6):
+        x = rng.standard_normal((n, 2048)).astype(np.float32)
+        order = np.argsort(-(hl.gate_inp.astype(np.float64) @ x[0].astype(np.float64)))
+        # trial even: duplicate the top row into a higher id (both picked); odd: duplicate the 4th pick (one picked)
+        src = int(order[0] if trial % 2 == 0 else order[3])
+        dst = int(max(e for e in range(16) if e != src))
+        hl.gate_inp[dst] = hl.gate_inp[src]
+        layer = hl.to_device(dev)
+        ws = torch.zeros(qk.moe_workspace_bytes(layer, n), dtype=torch.uint8, device=dev)
+        Y, sel = qk.moe_decode(layer, torch.from_numpy(x).to(dev), ws)
+        torch.cuda.synchronize()
+        ids, _, _ = sel_fields(sel)
+        got = [int(i) for i in ids[0, :4]]
+        lo, hi = min(src, dst), max(src, dst)
+        assert lo in got, (trial, got)
+        if hi in got:
+            assert got.index(lo) + 1 == got.index(hi), (trial, got)
+        r = orc.moe_ref(hl, x[0])
+        assert got == list(r["sel"].ids[:4]) or r["sel"].gap < 1e-3, (trial, got, list(r["sel"].ids[:4]))
+
+
 def test_moe_argument_errors(qk, dev, layer_iq4):
     import torch
     layer = layer_iq4.to_device(dev)
