@@ -101,29 +101,54 @@ __device__ __forceinline__ void pair_at(const MoeWs& ws, uint32_t p, const MoeDi
 // The loop is a chain of dependent wave-wide steps, so it is kept short: the exponentials are taken
 // after it, by the lanes in parallel, and a tie for the maximum -- the only case that needs a second
 // wave-wide reduction -- is detected with a ballot.
+// Order-preserving map from non-NaN floats to signed ints (and back): the loop below compares,
+// maximises and matches integers, which lets every reduction step be one DPP instruction.
+__device__ __forceinline__ int32_t float_key(float f)
+{
+    const int32_t b = __builtin_bit_cast(int32_t, f + 0.f); // -0 -> +0: equal logits must tie
+    return b ^ ((b >> 31) & 0x7FFFFFFF);
+}
+__device__ __forceinline__ float key_float(int32_t k)
+{
+    return __builtin_bit_cast(float, k ^ ((k >> 31) & 0x7FFFFFFF));
+}
+
+// Maximum over the wave, wave-uniform.
+__device__ __forceinline__ int32_t wave_max_i32(int32_t x)
+{
+    x = max(x, dpp_i<DPP_XOR1>(x));
+    x = max(x, dpp_i<DPP_XOR2>(x));
+    x = max(x, dpp_i<DPP_HALF_MIRROR>(x));
+    x = max(x, dpp_i<DPP_MIRROR>(x));
+    const int32_t a = max(__builtin_amdgcn_readlane(x, 0), __builtin_amdgcn_readlane(x, 16));
+    const int32_t b = max(__builtin_amdgcn_readlane(x, 32), __builtin_amdgcn_readlane(x, 48));
+    return max(a, b);
+}
+
 template <int NR>
 __device__ static inline void select_wave_n(const float* __restrict__ logits, uint32_t E, uint32_t k,
                                             qkk_sel* __restrict__ out, uint32_t* ids_copy)
 {
     constexpr float FLOOR = -3.4e38f;
     const int lane = threadIdx.x & 63;
-    float v[NR];
+    int32_t v[NR];
 #pragma unroll
     for (int i = 0; i < NR; i++) {
         const uint32_t e = lane + 64 * i;
         float l = e < E ? logits[e] : FLOOR;
         if (isnan(l) || isinf(l)) l = FLOOR;
-        v[i] = l;
+        v[i] = float_key(l);
     }
-    float top = 0.f, mym = 0.f;
+    const int32_t floor_key = float_key(FLOOR);
+    int32_t top = 0, mym = 0;
     uint32_t myid = 0;
     for (uint32_t r = 0; r < k; r++) {
-        float bv = v[0];
+        int32_t bv = v[0];
         uint32_t bi = lane;
 #pragma unroll
         for (int i = 1; i < NR; i++)
             if (v[i] > bv) { bv = v[i]; bi = lane + 64 * i; }
-        const float m = wave_max(bv);
+        const int32_t m = wave_max_i32(bv);
         const uint64_t tie = __builtin_amdgcn_ballot_w64(bv == m); // never empty: m is some lane's bv
         uint32_t id;
         if (__builtin_popcountll(tie) == 1) // wave-uniform
@@ -133,11 +158,11 @@ __device__ static inline void select_wave_n(const float* __restrict__ logits, ui
         // retire the winner
 #pragma unroll
         for (int i = 0; i < NR; i++)
-            if ((uint32_t)(lane + 64 * i) == id) v[i] = FLOOR;
+            if ((uint32_t)(lane + 64 * i) == id) v[i] = floor_key;
         if (r == 0) top = m;
         if ((uint32_t)lane == r) { mym = m; myid = min(id, E - 1); }
     }
-    const float p = (uint32_t)lane < k ? expf(mym - top) : 0.f;
+    const float p = (uint32_t)lane < k ? expf(key_float(mym) - key_float(top)) : 0.f;
     float wsum = 0.f;
     for (uint32_t r = 0; r < k; r++) wsum += readlane_f(p, (int)r); // pick order
     if ((uint32_t)lane < k) {
