@@ -215,6 +215,47 @@ struct IqTables {
     float iq4[16];
 };
 
+// IQ3_XXS tables for the packed-half dot product: the codebook as four half magnitudes per
+// entry, and per 7-bit sign selector the sign bits of its eight weights in half positions
+// (bit 15 / bit 31 of four dwords; the eighth sign is the parity of the seven).
+struct Iq3HalfTables {
+    uint2 grid[256];
+    uint4 sign[128];
+};
+typedef _Float16 qk_half2 __attribute__((ext_vector_type(2)));
+
+// Thread i < 256 fills entry i of the codebook (grid_word = codebook entry i as four bytes) and,
+// for i < 128, sign entry i.
+__device__ __forceinline__ void fill_iq3_half_entry(Iq3HalfTables& t, uint32_t i, uint32_t grid_word)
+{
+    const qk_half2 a = {(_Float16)(float)(grid_word & 255u), (_Float16)(float)((grid_word >> 8) & 255u)};
+    const qk_half2 b = {(_Float16)(float)((grid_word >> 16) & 255u), (_Float16)(float)(grid_word >> 24)};
+    t.grid[i] = uint2{__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b)};
+    if (i < 128) {
+        const uint32_t s8 = i | ((__builtin_popcount(i) & 1u) << 7);
+        uint32_t w[4];
+#pragma unroll
+        for (int p = 0; p < 4; p++) w[p] = (((s8 >> (2 * p)) & 1u) << 15) | (((s8 >> (2 * p + 1)) & 1u) << 31);
+        t.sign[i] = uint4{w[0], w[1], w[2], w[3]};
+    }
+}
+
+// A lane's 32 consecutive activations as 16 pairs of halves, value = hi + lo (exact to about
+// 2^-22 of the value): the operands of v_dot2_f32_f16.
+struct XSliceH {
+    qk_half2 hi[16], lo[16];
+};
+
+__device__ __forceinline__ void split_xslice(XSliceH& h, const XSlice& xs)
+{
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const _Float16 a = (_Float16)xs.v[2 * i], b = (_Float16)xs.v[2 * i + 1];
+        h.hi[i] = qk_half2{a, b};
+        h.lo[i] = qk_half2{(_Float16)(xs.v[2 * i] - (float)a), (_Float16)(xs.v[2 * i + 1] - (float)b)};
+    }
+}
+
 // Bytes of weights one lane fetches per pass, held in registers between the load and the
 // arithmetic so several rows can be in flight.
 template <int TYPE>
@@ -369,6 +410,29 @@ struct LaneW<18> { // IQ3_XXS
             }
         }
         return h2f(d) * (0.5f + (float)(aux >> 28)) * 0.5f * s;
+    }
+    // The same product on packed halves: signed magnitudes come out of two LDS lookups and two
+    // XORs per four weights, each v_dot2_f32_f16 takes two weights (products exact, fp32 sums).
+    __device__ __forceinline__ float dot_h(const XSliceH& xh, const Iq3HalfTables* tab) const
+    {
+        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+        for (int l = 0; l < 4; l++) {
+            const uint4 sm = tab->sign[(aux >> (7 * l)) & 127u];
+            const uint32_t gw = l < 2 ? g.x : g.y;
+#pragma unroll
+            for (int hh = 0; hh < 2; hh++) {
+                const uint2 m = tab->grid[(gw >> (16 * (l & 1) + 8 * hh)) & 0xFFu];
+                const qk_half2 w01 = __builtin_bit_cast(qk_half2, m.x ^ (hh ? sm.z : sm.x));
+                const qk_half2 w23 = __builtin_bit_cast(qk_half2, m.y ^ (hh ? sm.w : sm.y));
+                const int q = l * 4 + hh * 2;
+                s0 = __builtin_amdgcn_fdot2(w01, xh.hi[q], s0, false);
+                s1 = __builtin_amdgcn_fdot2(w23, xh.hi[q + 1], s1, false);
+                s0 = __builtin_amdgcn_fdot2(w01, xh.lo[q], s0, false);
+                s1 = __builtin_amdgcn_fdot2(w23, xh.lo[q + 1], s1, false);
+            }
+        }
+        return h2f(d) * (0.5f + (float)(aux >> 28)) * 0.5f * (s0 + s1);
     }
 };
 

@@ -73,17 +73,20 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
 
 // ---- launch 2: select + routed gate/up + SiLU --------------------------------------------
 // Every workgroup picks the top-n_used experts itself from the E logits of launch 1 (one wave,
-// ~1 us) instead of waiting for a selector launch: the logits, the activation slice and the
+// ~1.7 us) instead of waiting for a selector launch: the logits, the activation slice and the
 // codebook are fetched in one round trip, the picked rows in a second.  Workgroup 0 also
 // writes the router record.  Wave task = (pick s, RIF consecutive FFN rows); gate and up rows
-// of one FFN row are fetched together.  IQ3_XXS rows of H = 2048*PASSES weights.
+// of one FFN row are fetched together.  IQ3_XXS rows of H = 2048*PASSES weights.  The arithmetic
+// after the second round trip is bound by the vector ALUs (one wave per SIMD decodes 8 rows), so
+// it runs on packed halves: two LDS lookups and two XORs per four weights, v_dot2_f32_f16 against
+// the activations split into hi + lo halves.
 template <int TYPE, int PASSES, int RIF>
 __global__ __launch_bounds__(256) void moe_gateup_kernel(const uint8_t* __restrict__ gate_exps,
                                                          const uint8_t* __restrict__ up_exps,
                                                          const float* __restrict__ x, MoeWs ws,
                                                          qkk_sel* __restrict__ sel, MoeDims d)
 {
-    __shared__ IqTables tab;
+    __shared__ Iq3HalfTables tab;
     __shared__ float s_log[QKK_MAX_EXPERTS + 8];
     __shared__ qkk_sel s_sel;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -98,11 +101,15 @@ __global__ __launch_bounds__(256) void moe_gateup_kernel(const uint8_t* __restri
         for (int i = 0; i <= (int)(QKK_MAX_EXPERTS / 64); i++)
             lv[i] = (uint32_t)(lane + 64 * i) <= d.E ? ws.logits[lane + 64 * i] : 0.f;
     }
-    XSlice xs[PASSES];
+    XSliceH xs[PASSES];
 #pragma unroll
-    for (int p = 0; p < PASSES; p++) load_xslice<TYPE>(xs[p], x + p * 2048, lane);
+    for (int p = 0; p < PASSES; p++) {
+        XSlice f;
+        load_xslice<TYPE>(f, x + p * 2048, lane);
+        split_xslice(xs[p], f);
+    }
 
-    tab.grid[threadIdx.x] = grid_word;
+    fill_iq3_half_entry(tab, threadIdx.x, grid_word);
     if (wave == 0) {
 #pragma unroll
         for (int i = 0; i <= (int)(QKK_MAX_EXPERTS / 64); i++)
@@ -145,8 +152,8 @@ __global__ __launch_bounds__(256) void moe_gateup_kernel(const uint8_t* __restri
             float g = 0.f, u = 0.f;
 #pragma unroll
             for (int p = 0; p < PASSES; p++) {
-                g += wg[i][p].dot(xs[p], nullptr, &tab, lane);
-                u += wu[i][p].dot(xs[p], nullptr, &tab, lane);
+                g += wg[i][p].dot_h(xs[p], &tab);
+                u += wu[i][p].dot_h(xs[p], &tab);
             }
             g = wave_sum(g);
             u = wave_sum(u);
