@@ -405,11 +405,13 @@ static uint32_t per_cu_of(const void* fn, uint32_t lds)
     return (uint32_t)std::min(n, 2);
 }
 
-// batches per sub-item: the largest power of two <= total that still gives every CU about two items
-static uint32_t pick_nb(uint32_t total_batches, uint32_t items)
+// batches per sub-item: the largest power of two <= total that still gives each of the `wgs`
+// workgroups the launch can run at once an item (longer streams per workgroup amortise the
+// activation load and the pipeline fill of a sub-item; fewer items than workgroups leave CUs idle)
+static uint32_t pick_nb(uint32_t total_batches, uint32_t items, uint32_t wgs)
 {
     uint32_t nb = total_batches;
-    while (nb > 1 && (uint64_t)items * (total_batches / nb) < 2ull * persistent_blocks() / 4) nb /= 2;
+    while (nb > 1 && (uint64_t)items * (total_batches / nb) < wgs) nb /= 2;
     return nb;
 }
 
@@ -421,7 +423,7 @@ static void launch_down_fused(const qkk_moe_layer* L, const MoeWs& ws, const qkk
     static const uint32_t per_cu = per_cu_of((const void*)moe_down_fused_kernel<TYPE, FB>, Geo::LDS);
     (void)per_cu;
     const uint32_t tot_r = d.H / (16 * Geo::R::BT), tot_s = d.H / (16 * Geo::S::BT);
-    const uint32_t nb_r = pick_nb(tot_r, experts), nb_s = std::min(tot_s, std::max(1u, nb_r * Geo::R::BT / Geo::S::BT / 2));
+    const uint32_t nb_r = pick_nb(tot_r, experts, persistent_blocks() / 4), nb_s = std::min(tot_s, std::max(1u, nb_r * Geo::R::BT / Geo::S::BT / 2));
     const uint32_t items = experts * (tot_r / nb_r) + (N + 15) / 16 * (tot_s / nb_s);
     hipLaunchKernelGGL((moe_down_fused_kernel<TYPE, FB>), dim3(std::min(items, persistent_blocks() / 4)), dim3(CT), Geo::LDS,
                        st, (const uint8_t*)L->down_exps, (const uint8_t*)L->down_shexp, ws, sel, d, N, nb_r, nb_s);
@@ -436,7 +438,7 @@ void moe_mfma_launch_fused(const qkk_moe_layer* L, const float* X, const qkk_sel
         static const uint32_t per_cu = per_cu_of((const void*)moe_gateup_fused_kernel, FU_LDS);
         (void)per_cu;
         const uint32_t tot_r = d.F / (16 * FuGeoR::BT), tot_s = d.F / (16 * FuGeoS::BT);
-        const uint32_t nb_r = pick_nb(tot_r, experts), nb_s = std::min(tot_s, std::max(1u, nb_r * FuGeoR::BT / FuGeoS::BT / 2));
+        const uint32_t nb_r = pick_nb(tot_r, experts, persistent_blocks() / 4), nb_s = std::min(tot_s, std::max(1u, nb_r * FuGeoR::BT / FuGeoS::BT / 2));
         const uint32_t items = experts * (tot_r / nb_r) + (N + 15) / 16 * (tot_s / nb_s);
         hipLaunchKernelGGL(moe_gateup_fused_kernel, dim3(std::min(items, persistent_blocks() / 4)), dim3(CT), FU_LDS, st,
                            (const uint8_t*)L->gate_exps, (const uint8_t*)L->up_exps, (const uint8_t*)L->gate_shexp,
@@ -461,7 +463,7 @@ static void launch_gateup(const qkk_moe_layer* L, const float* X, const MoeWs& w
 {
     using Geo = GuGeo<SHARED>;
     static const uint32_t per_cu = per_cu_of((const void*)moe_gateup_mfma_kernel<SHARED>, Geo::LDS_BYTES);
-    const uint32_t tot = d.F / (16 * Geo::BT), nb = pick_nb(tot, items);
+    const uint32_t tot = d.F / (16 * Geo::BT), nb = pick_nb(tot, items, per_cu * (persistent_blocks() / 4));
     const uint32_t blocks = std::min(items * (tot / nb), per_cu * (persistent_blocks() / 4));
     hipLaunchKernelGGL(moe_gateup_mfma_kernel<SHARED>, dim3(blocks), dim3(CT), Geo::LDS_BYTES, st,
                        (const uint8_t*)(SHARED ? L->gate_shexp : L->gate_exps),
@@ -474,7 +476,7 @@ static void launch_down(const void* W, const MoeWs& ws, const qkk_sel* sel, cons
 {
     using Geo = DnGeo<TYPE, FB>;
     static const uint32_t per_cu = per_cu_of((const void*)moe_down_mfma_kernel<TYPE, FB, SHARED>, Geo::LDS_BYTES);
-    const uint32_t tot = d.H / (16 * Geo::BT), nb = pick_nb(tot, items);
+    const uint32_t tot = d.H / (16 * Geo::BT), nb = pick_nb(tot, items, per_cu * (persistent_blocks() / 4));
     const uint32_t blocks = std::min(items * (tot / nb), per_cu * (persistent_blocks() / 4));
     hipLaunchKernelGGL((moe_down_mfma_kernel<TYPE, FB, SHARED>), dim3(blocks), dim3(CT), Geo::LDS_BYTES, st,
                        (const uint8_t*)W, ws, sel, d, N, nb);
