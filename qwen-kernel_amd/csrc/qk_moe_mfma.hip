@@ -227,35 +227,29 @@ __global__ __launch_bounds__(256) void moe_fold_norm_kernel(MoeWs ws, const qkk_
 }
 
 // ==== few rows (up to FUSED_MAX_ROWS): one gate/up and one down launch take the shared expert's and
-// the routed experts' items together (a HIP graph runs the side stream's launches of so short a
-// step one after the other, which costs more than it saves).  Items: first the shared expert's
-// tiles, then the routed experts.
-struct ItemF {
-    bool shared;
-    uint32_t expert, first, count; // routed: pairs [first, first+count) of ws.pairs; shared: tokens
-    uint32_t sub;
+// the routed experts' work together (a HIP graph runs the side stream's launches of so short a
+// step one after the other, which costs more than it saves).
+//
+// Work of a launch = the shared expert's batches (token tiles x batches of weight rows, cost CS each)
+// followed by the routed batches (active experts x batches, cost CR each).  Workgroup g of G takes
+// the batches that start inside its equal share of the total cost: every workgroup gets the same
+// work to within one batch whatever the number of active experts turns out to be (the host cannot
+// know it), and its batches are consecutive, so they form at most a few runs of one expert's rows.
+struct Share {
+    uint32_t s0, s1, r0, r1; // shared batches [s0, s1), routed batches [r0, r1)
 };
 
-__device__ __forceinline__ uint32_t item_count_f(uint32_t n_active, uint32_t N, uint32_t subs_shared, uint32_t subs)
+__device__ __forceinline__ Share my_share(uint32_t g, uint32_t G, uint32_t ns, uint32_t cs, uint32_t nr, uint32_t cr)
 {
-    return (N + 15) / 16 * subs_shared + n_active * subs;
-}
-
-__device__ __forceinline__ ItemF get_item_f(const MoeWs& ws, uint32_t index, uint32_t subs_shared, uint32_t subs,
-                                            const MoeDims& d, uint32_t N)
-{
-    ItemF it;
-    const uint32_t n_sh = (N + 15) / 16 * subs_shared;
-    if (index < n_sh) {
-        it.sub = index % subs_shared;
-        it.shared = true; it.expert = 0; it.first = index / subs_shared * 16u; it.count = min(16u, N - it.first);
-    } else {
-        const uint32_t w = (index - n_sh) / subs;
-        it.sub = (index - n_sh) % subs;
-        const ActiveExpert a = active_expert(ws, w, d, N);
-        it.shared = false; it.expert = a.expert; it.first = a.first; it.count = a.count;
-    }
-    return it;
+    const uint64_t US = (uint64_t)ns * cs, U = US + (uint64_t)nr * cr;
+    const uint64_t u0 = U * g / G, u1 = U * (g + 1) / G;
+    const auto cdiv = [](uint64_t a, uint32_t b) { return (uint32_t)((a + b - 1) / b); };
+    Share sh;
+    sh.s0 = min(cdiv(min(u0, US), cs), ns);
+    sh.s1 = min(cdiv(min(u1, US), cs), ns);
+    sh.r0 = u0 > US ? min(cdiv(u0 - US, cr), nr) : 0u;
+    sh.r1 = u1 > US ? min(cdiv(u1 - US, cr), nr) : 0u;
+    return sh;
 }
 
 // ---- gate/up + SiLU --------------------------------------------------------------------------------
@@ -266,13 +260,14 @@ constexpr int FU_PB = 2; // partial buffers (2: one barrier per batch)
 using FuGeoR = CoopGeom<QKK_IQ3_XXS, 8, 2, FU_TG_R, false, 1, FU_PB>;
 using FuGeoS = CoopGeom<QKK_Q8_0, 8, 2, FU_TG_S, true, 1, FU_PB>;
 constexpr uint32_t FU_LDS = FuGeoR::LDS_BYTES > FuGeoS::LDS_BYTES ? FuGeoR::LDS_BYTES : FuGeoS::LDS_BYTES;
+constexpr uint32_t FU_CS = 3, FU_CR = 2; // a shared batch is two LDS steps, a routed one a single larger step
 
 __global__ __launch_bounds__(CT) void moe_gateup_fused_kernel(const uint8_t* __restrict__ gate_exps,
                                                              const uint8_t* __restrict__ up_exps,
                                                              const uint8_t* __restrict__ gate_shexp,
                                                              const uint8_t* __restrict__ up_shexp,
                                                              const float* __restrict__ X, MoeWs ws, MoeDims d,
-                                                             uint32_t N, uint32_t nb_r, uint32_t nb_s)
+                                                             uint32_t N)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ MfmaTables tab;
@@ -281,46 +276,52 @@ __global__ __launch_bounds__(CT) void moe_gateup_fused_kernel(const uint8_t* __r
     const uint32_t F = d.F, H = d.H;
     fill_mfma_tables(tab, tid, CT);
     const uint32_t n_active = active_count(ws, d);
-    const uint32_t subs_sh = F / (16 * FuGeoS::BT * nb_s), subs = F / (16 * FuGeoR::BT * nb_r);
-    const uint32_t n_items = item_count_f(n_active, N, subs_sh, subs);
+    const uint32_t tot_s = F / (16 * FuGeoS::BT), tot_r = F / (16 * FuGeoR::BT); // batches per token tile / expert
+    const Share sh = my_share(blockIdx.x, gridDim.x, (N + 15) / 16 * tot_s, FU_CS, n_active * tot_r, FU_CR);
+    const auto row_of = [&](uint32_t r) { return s_tok[r]; };
 
-    for (uint32_t w = blockIdx.x; w < n_items; w += gridDim.x) {
-        const ItemF it = get_item_f(ws, w, subs_sh, subs, d, N);
-        for (uint32_t t0 = 0; t0 < it.count; t0 += 16) {
-            const uint32_t np = it.shared ? it.count : min(16u, it.count - t0);
+    for (uint32_t b = sh.s0; b < sh.s1;) { // shared expert: runs inside one token tile
+        const uint32_t tile = b / tot_s, f0 = b % tot_s, nbat = min(tot_s - f0, sh.s1 - b);
+        const uint32_t first = tile * 16u, np = min(16u, N - first), row0 = f0 * FuGeoS::BT * 16;
+        __syncthreads(); // previous run fully consumed
+        if (tid < 16) {
+            s_tok[tid] = (uint32_t)tid < np ? first + tid : 0u;
+            s_slot[tid] = d.k;
+        }
+        __syncthreads();
+        coop_stream<QKK_Q8_0, 8, 2, FU_TG_S, true, false, 1, FU_PB>(gate_shexp + (size_t)row0 * FuGeoS::RB, up_shexp + (size_t)row0 * FuGeoS::RB, nbat, X, H, np, row_of, smem, tab, tid,
+            [&](uint32_t t, uint32_t ln, uint32_t e, float sum0, float sum1, uint32_t) {
+                const uint32_t r = 4 * (ln >> 4) + e;
+                if (r < np)
+                    ws.h[((size_t)s_tok[r] * (d.k + 1) + s_slot[r]) * F + row0 + t * 16 + (ln & 15u)] =
+                        (sum0 / (1.f + expf(-sum0))) * sum1;
+            });
+        b += nbat;
+    }
+    for (uint32_t b = sh.r0; b < sh.r1;) { // routed: runs inside one active expert
+        const uint32_t w = b / tot_r, f0 = b % tot_r, nbat = min(tot_r - f0, sh.r1 - b);
+        const ActiveExpert a = active_expert(ws, w, d, N); // w < n_active
+        const uint32_t row0 = f0 * FuGeoR::BT * 16;
+        const size_t eo = ((size_t)a.expert * F + row0) * FuGeoR::RB;
+        for (uint32_t t0 = 0; t0 < a.count; t0 += 16) {
+            const uint32_t np = min(16u, a.count - t0);
             __syncthreads(); // previous tile fully consumed
             if (tid < 16) {
                 uint32_t tok = 0, slot = 0;
-                if ((uint32_t)tid < np) {
-                    if (it.shared) { tok = it.first + tid; slot = d.k; }
-                    else pair_at(ws, it.first + t0 + tid, d, N, tok, slot);
-                }
+                if ((uint32_t)tid < np) pair_at(ws, a.first + t0 + tid, d, N, tok, slot);
                 s_tok[tid] = tok;
                 s_slot[tid] = slot;
             }
             __syncthreads();
-            const auto row_of = [&](uint32_t r) { return s_tok[r]; };
-            if (it.shared) {
-                const uint32_t row0 = it.sub * nb_s * FuGeoS::BT * 16;
-                coop_stream<QKK_Q8_0, 8, 2, FU_TG_S, true, false, 1, FU_PB>(gate_shexp + (size_t)row0 * FuGeoS::RB, up_shexp + (size_t)row0 * FuGeoS::RB, nb_s, X, H, np, row_of, smem, tab, tid,
-                    [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1, uint32_t) {
-                        const uint32_t r = 4 * (ln >> 4) + e;
-                        if (r < np)
-                            ws.h[((size_t)s_tok[r] * (d.k + 1) + s_slot[r]) * F + row0 + tile * 16 + (ln & 15u)] =
-                                (sum0 / (1.f + expf(-sum0))) * sum1;
-                    });
-                break;
-            }
-            const uint32_t row0 = it.sub * nb_r * FuGeoR::BT * 16;
-            const size_t eo = ((size_t)it.expert * F + row0) * FuGeoR::RB;
-            coop_stream<QKK_IQ3_XXS, 8, 2, FU_TG_R, false, false, 1, FU_PB>(gate_exps + eo, up_exps + eo, nb_r, X, H, np, row_of, smem, tab, tid,
-                [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1, uint32_t) {
+            coop_stream<QKK_IQ3_XXS, 8, 2, FU_TG_R, false, false, 1, FU_PB>(gate_exps + eo, up_exps + eo, nbat, X, H, np, row_of, smem, tab, tid,
+                [&](uint32_t t, uint32_t ln, uint32_t e, float sum0, float sum1, uint32_t) {
                     const uint32_t r = 4 * (ln >> 4) + e;
                     if (r < np)
-                        ws.h[((size_t)s_tok[r] * (d.k + 1) + s_slot[r]) * F + row0 + tile * 16 + (ln & 15u)] =
+                        ws.h[((size_t)s_tok[r] * (d.k + 1) + s_slot[r]) * F + row0 + t * 16 + (ln & 15u)] =
                             (sum0 / (1.f + expf(-sum0))) * sum1;
                 });
         }
+        b += nbat;
     }
 }
 
@@ -333,13 +334,13 @@ struct DnGeoF {
     using R = CoopGeom<TYPE_DN, FB, 1, TG_R>;
     using S = CoopGeom<QKK_Q8_0, FB, 1, TG_S>;
     static constexpr uint32_t LDS = R::LDS_BYTES > S::LDS_BYTES ? R::LDS_BYTES : S::LDS_BYTES;
+    static constexpr uint32_t CS = 1, CR = TG_R; // cost of a batch ~ row tiles per wave
 };
 
 template <int TYPE_DN, int FB>
 __global__ __launch_bounds__(CT) void moe_down_fused_kernel(const uint8_t* __restrict__ down_exps,
                                                            const uint8_t* __restrict__ down_shexp, MoeWs ws,
-                                                           const qkk_sel* __restrict__ sel, MoeDims d, uint32_t N,
-                                                           uint32_t nb_r, uint32_t nb_s)
+                                                           const qkk_sel* __restrict__ sel, MoeDims d, uint32_t N)
 {
     using Geo = DnGeoF<TYPE_DN, FB>;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -350,48 +351,54 @@ __global__ __launch_bounds__(CT) void moe_down_fused_kernel(const uint8_t* __res
     const uint32_t F = d.F, H = d.H;
     fill_mfma_tables(tab, tid, CT);
     const uint32_t n_active = active_count(ws, d);
-    const uint32_t subs_sh = H / (16 * Geo::S::BT * nb_s), subs = H / (16 * Geo::R::BT * nb_r);
-    const uint32_t n_items = item_count_f(n_active, N, subs_sh, subs);
+    const uint32_t tot_s = H / (16 * Geo::S::BT), tot_r = H / (16 * Geo::R::BT);
+    const Share sh = my_share(blockIdx.x, gridDim.x, (N + 15) / 16 * tot_s, Geo::CS, n_active * tot_r, Geo::CR);
+    const auto row_of = [&](uint32_t r) { return s_tok[r] * (d.k + 1) + s_slot[r]; };
 
-    for (uint32_t w = blockIdx.x; w < n_items; w += gridDim.x) {
-        const ItemF it = get_item_f(ws, w, subs_sh, subs, d, N);
-        for (uint32_t t0 = 0; t0 < it.count; t0 += 16) {
-            const uint32_t np = it.shared ? it.count : min(16u, it.count - t0);
+    for (uint32_t b = sh.s0; b < sh.s1;) {
+        const uint32_t tile = b / tot_s, f0 = b % tot_s, nbat = min(tot_s - f0, sh.s1 - b);
+        const uint32_t first = tile * 16u, np = min(16u, N - first), row0 = f0 * Geo::S::BT * 16;
+        __syncthreads();
+        if (tid < 16) {
+            s_tok[tid] = (uint32_t)tid < np ? first + tid : 0u;
+            s_slot[tid] = d.k;
+            s_wt[tid] = (uint32_t)tid < np ? 1.f : 0.f; // the shared gate is applied by the fold
+        }
+        __syncthreads();
+        coop_stream<QKK_Q8_0, FB, 1, Geo::TG_S, false, false>(down_shexp + (size_t)row0 * Geo::S::RB, nullptr, nbat, ws.h, F, np, row_of, smem, tab, tid,
+            [&](uint32_t t, uint32_t ln, uint32_t e, float sum0, float, uint32_t) {
+                const uint32_t r = 4 * (ln >> 4) + e;
+                if (r < np)
+                    ws.contrib[((size_t)s_tok[r] * (d.k + 1) + s_slot[r]) * H + row0 + t * 16 + (ln & 15u)] = s_wt[r] * sum0;
+            });
+        b += nbat;
+    }
+    for (uint32_t b = sh.r0; b < sh.r1;) {
+        const uint32_t w = b / tot_r, f0 = b % tot_r, nbat = min(tot_r - f0, sh.r1 - b);
+        const ActiveExpert a = active_expert(ws, w, d, N);
+        const uint32_t row0 = f0 * Geo::R::BT * 16;
+        const uint8_t* base = down_exps + ((size_t)a.expert * H + row0) * Geo::R::RB;
+        for (uint32_t t0 = 0; t0 < a.count; t0 += 16) {
+            const uint32_t np = min(16u, a.count - t0);
             __syncthreads();
             if (tid < 16) {
                 uint32_t tok = 0, slot = 0;
                 float wt = 0.f;
                 if ((uint32_t)tid < np) {
-                    if (it.shared) { tok = it.first + tid; slot = d.k; wt = 1.f; } // gate applied by the fold
-                    else {
-                        pair_at(ws, it.first + t0 + tid, d, N, tok, slot);
-                        wt = sel[tok].w[slot];
-                    }
+                    pair_at(ws, a.first + t0 + tid, d, N, tok, slot);
+                    wt = sel[tok].w[slot];
                 }
                 s_tok[tid] = tok; s_slot[tid] = slot; s_wt[tid] = wt;
             }
             __syncthreads();
-            const auto row_of = [&](uint32_t r) { return s_tok[r] * (d.k + 1) + s_slot[r]; };
-            if (it.shared) {
-                const uint32_t row0 = it.sub * nb_s * Geo::S::BT * 16;
-                coop_stream<QKK_Q8_0, FB, 1, Geo::TG_S, false, false>(down_shexp + (size_t)row0 * Geo::S::RB, nullptr, nb_s, ws.h, F, np, row_of, smem, tab, tid,
-                    [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1, uint32_t) {
-                        const uint32_t r = 4 * (ln >> 4) + e;
-                        if (r < np)
-                            ws.contrib[((size_t)s_tok[r] * (d.k + 1) + s_slot[r]) * H + row0 + tile * 16 + (ln & 15u)] =
-                                s_wt[r] * sum0;
-                    });
-                break;
-            }
-            const uint32_t row0 = it.sub * nb_r * Geo::R::BT * 16;
-            coop_stream<TYPE_DN, FB, 1, Geo::TG_R, false, false>(down_exps + ((size_t)it.expert * H + row0) * Geo::R::RB, nullptr, nb_r, ws.h, F, np, row_of, smem, tab, tid,
-                [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1, uint32_t) {
+            coop_stream<TYPE_DN, FB, 1, Geo::TG_R, false, false>(base, nullptr, nbat, ws.h, F, np, row_of, smem, tab, tid,
+                [&](uint32_t t, uint32_t ln, uint32_t e, float sum0, float, uint32_t) {
                     const uint32_t r = 4 * (ln >> 4) + e;
                     if (r < np)
-                        ws.contrib[((size_t)s_tok[r] * (d.k + 1) + s_slot[r]) * H + row0 + tile * 16 + (ln & 15u)] =
-                            s_wt[r] * sum0;
+                        ws.contrib[((size_t)s_tok[r] * (d.k + 1) + s_slot[r]) * H + row0 + t * 16 + (ln & 15u)] = s_wt[r] * sum0;
                 });
         }
+        b += nbat;
     }
 }
 
@@ -417,42 +424,35 @@ static uint32_t pick_nb(uint32_t total_batches, uint32_t items, uint32_t wgs)
 
 template <int TYPE, int FB>
 static void launch_down_fused(const qkk_moe_layer* L, const MoeWs& ws, const qkk_sel* sel, const MoeDims& d, uint32_t N,
-                              uint32_t experts, hipStream_t st)
+                              hipStream_t st)
 {
     using Geo = DnGeoF<TYPE, FB>;
     static const uint32_t per_cu = per_cu_of((const void*)moe_down_fused_kernel<TYPE, FB>, Geo::LDS);
     (void)per_cu;
-    const uint32_t tot_r = d.H / (16 * Geo::R::BT), tot_s = d.H / (16 * Geo::S::BT);
-    const uint32_t nb_r = pick_nb(tot_r, experts, persistent_blocks() / 4), nb_s = std::min(tot_s, std::max(1u, nb_r * Geo::R::BT / Geo::S::BT / 2));
-    const uint32_t items = experts * (tot_r / nb_r) + (N + 15) / 16 * (tot_s / nb_s);
-    hipLaunchKernelGGL((moe_down_fused_kernel<TYPE, FB>), dim3(std::min(items, persistent_blocks() / 4)), dim3(CT), Geo::LDS,
-                       st, (const uint8_t*)L->down_exps, (const uint8_t*)L->down_shexp, ws, sel, d, N, nb_r, nb_s);
+    hipLaunchKernelGGL((moe_down_fused_kernel<TYPE, FB>), dim3(persistent_blocks() / 4), dim3(CT), Geo::LDS, st,
+                       (const uint8_t*)L->down_exps, (const uint8_t*)L->down_shexp, ws, sel, d, N);
 }
 
-// Gate/up and down for few rows: shared and routed items in one launch each.
+// Gate/up and down for few rows: shared and routed work in one launch each, one workgroup per CU.
 void moe_mfma_launch_fused(const qkk_moe_layer* L, const float* X, const qkk_sel* sel, const MoeWs& ws,
                            const MoeDims& d, uint32_t N, uint32_t stages, hipStream_t st)
 {
-    const uint32_t experts = (uint32_t)std::min<uint64_t>(d.E, (uint64_t)N * d.k); // upper bound of the active ones
     if (stages & QKK_STAGE_GATEUP) {
         static const uint32_t per_cu = per_cu_of((const void*)moe_gateup_fused_kernel, FU_LDS);
         (void)per_cu;
-        const uint32_t tot_r = d.F / (16 * FuGeoR::BT), tot_s = d.F / (16 * FuGeoS::BT);
-        const uint32_t nb_r = pick_nb(tot_r, experts, persistent_blocks() / 4), nb_s = std::min(tot_s, std::max(1u, nb_r * FuGeoR::BT / FuGeoS::BT / 2));
-        const uint32_t items = experts * (tot_r / nb_r) + (N + 15) / 16 * (tot_s / nb_s);
-        hipLaunchKernelGGL(moe_gateup_fused_kernel, dim3(std::min(items, persistent_blocks() / 4)), dim3(CT), FU_LDS, st,
+        hipLaunchKernelGGL(moe_gateup_fused_kernel, dim3(persistent_blocks() / 4), dim3(CT), FU_LDS, st,
                            (const uint8_t*)L->gate_exps, (const uint8_t*)L->up_exps, (const uint8_t*)L->gate_shexp,
-                           (const uint8_t*)L->up_shexp, X, ws, d, N, nb_r, nb_s);
+                           (const uint8_t*)L->up_shexp, X, ws, d, N);
     }
     if (stages & QKK_STAGE_DOWN) {
         if (L->down_type == QKK_IQ4_XS) {
-            if (d.F == 256) launch_down_fused<QKK_IQ4_XS, 1>(L, ws, sel, d, N, experts, st);
-            else if (d.F == 512) launch_down_fused<QKK_IQ4_XS, 2>(L, ws, sel, d, N, experts, st);
-            else launch_down_fused<QKK_IQ4_XS, 4>(L, ws, sel, d, N, experts, st);
+            if (d.F == 256) launch_down_fused<QKK_IQ4_XS, 1>(L, ws, sel, d, N, st);
+            else if (d.F == 512) launch_down_fused<QKK_IQ4_XS, 2>(L, ws, sel, d, N, st);
+            else launch_down_fused<QKK_IQ4_XS, 4>(L, ws, sel, d, N, st);
         } else {
-            if (d.F == 256) launch_down_fused<QKK_Q6_K, 1>(L, ws, sel, d, N, experts, st);
-            else if (d.F == 512) launch_down_fused<QKK_Q6_K, 2>(L, ws, sel, d, N, experts, st);
-            else launch_down_fused<QKK_Q6_K, 4>(L, ws, sel, d, N, experts, st);
+            if (d.F == 256) launch_down_fused<QKK_Q6_K, 1>(L, ws, sel, d, N, st);
+            else if (d.F == 512) launch_down_fused<QKK_Q6_K, 2>(L, ws, sel, d, N, st);
+            else launch_down_fused<QKK_Q6_K, 4>(L, ws, sel, d, N, st);
         }
     }
 }
