@@ -18,28 +18,40 @@
 
 namespace qk {
 
+// How a launch's batches are divided: workgroup g of G takes the batches that start inside its equal
+// share of the total cost (shared-expert batches first, cost cs each, then routed ones, cost cr each):
+// the same work for every workgroup to within one batch, whatever the number of active experts.
+struct Share {
+    uint32_t s0, s1, r0, r1; // shared batches [s0, s1), routed batches [r0, r1)
+};
+
+__device__ __forceinline__ Share my_share(uint32_t g, uint32_t G, uint32_t ns, uint32_t cs, uint32_t nr, uint32_t cr)
+{
+    const uint64_t US = (uint64_t)ns * cs, U = US + (uint64_t)nr * cr;
+    const uint64_t u0 = U * g / G, u1 = U * (g + 1) / G;
+    const auto cdiv = [](uint64_t a, uint32_t b) { return (uint32_t)((a + b - 1) / b); };
+    Share sh;
+    sh.s0 = min(cdiv(min(u0, US), cs), ns);
+    sh.s1 = min(cdiv(min(u1, US), cs), ns);
+    sh.r0 = u0 > US ? min(cdiv(u0 - US, cr), nr) : 0u;
+    sh.r1 = u1 > US ? min(cdiv(u1 - US, cr), nr) : 0u;
+    return sh;
+}
+
 // Work items.  The shared expert is one dense expert for every token: its items are tiles of 16
 // consecutive tokens; it depends on nothing the router produces, so its launches run on a side
 // stream next to the router and the routed experts.  A routed item is one active expert with its
-// pair list.  Every item is cut into sub-items of `nb` batches of weight rows, so one expert's
-// rows are streamed by several workgroups (each loads the activation rows itself).
+// pair list.  A workgroup's share of the batches falls into runs, each inside one item: the
+// workgroup loads the item's activation rows and streams the run's weight rows.
 struct Item {
     uint32_t expert, first, count; // routed: pairs [first, first+count) of ws.pairs; shared: tokens
-    uint32_t sub;
 };
 
+// item w of the launch (w < number of token tiles, or < active_count())
 template <bool SHARED>
-__device__ __forceinline__ uint32_t item_count(const MoeWs& ws, const MoeDims& d, uint32_t N, uint32_t subs)
-{
-    return (SHARED ? (N + 15) / 16 : active_count(ws, d)) * subs;
-}
-
-template <bool SHARED>
-__device__ __forceinline__ Item get_item(const MoeWs& ws, uint32_t index, uint32_t subs, const MoeDims& d, uint32_t N)
+__device__ __forceinline__ Item get_item(const MoeWs& ws, uint32_t w, const MoeDims& d, uint32_t N)
 {
     Item it;
-    const uint32_t w = index / subs;
-    it.sub = index % subs;
     if (SHARED) {
         it.expert = 0; it.first = w * 16u; it.count = min(16u, N - it.first);
     } else {
@@ -47,6 +59,29 @@ __device__ __forceinline__ Item get_item(const MoeWs& ws, uint32_t index, uint32
         it.expert = a.expert; it.first = a.first; it.count = a.count;
     }
     return it;
+}
+
+// this workgroup's batches [b0, b1) of the launch's n_items * tot
+template <bool SHARED>
+__device__ __forceinline__ void my_batches(const MoeWs& ws, const MoeDims& d, uint32_t N, uint32_t tot, uint32_t& b0,
+                                           uint32_t& b1)
+{
+    const uint32_t n_items = SHARED ? (N + 15) / 16 : active_count(ws, d);
+    // Where whole sub-items of a power-of-two length fill at least nine tenths of the grid, they are
+    // taken as they are (a run never crosses an item, so no workgroup loads two activation tiles);
+    // otherwise equal shares.
+    for (uint32_t nb = tot; nb >= 1; nb >>= 1) {
+        const uint64_t subs = (uint64_t)n_items * (tot / nb);
+        if (subs > gridDim.x) break;
+        if (subs * 10 >= (uint64_t)gridDim.x * 9 && tot % nb == 0) {
+            b0 = blockIdx.x < subs ? blockIdx.x * nb : 0u;
+            b1 = blockIdx.x < subs ? b0 + nb : 0u;
+            return;
+        }
+    }
+    const Share sh = my_share(blockIdx.x, gridDim.x, 0, 1, n_items * tot, 1);
+    b0 = sh.r0;
+    b1 = sh.r1;
 }
 
 // rows of the staged tile: s_tok[r] = token, s_slot[r] = h / contrib slot (k = shared expert)
@@ -76,7 +111,7 @@ template <bool SHARED>
 __global__ __launch_bounds__(CT, SHARED ? 2 : 4) void moe_gateup_mfma_kernel(const uint8_t* __restrict__ gate,
                                                                              const uint8_t* __restrict__ up,
                                                                              const float* __restrict__ X, MoeWs ws,
-                                                                             MoeDims d, uint32_t N, uint32_t nb)
+                                                                             MoeDims d, uint32_t N)
 {
     using Geo = GuGeo<SHARED>;
     constexpr int TYPE = SHARED ? QKK_Q8_0 : QKK_IQ3_XXS;
@@ -86,19 +121,21 @@ __global__ __launch_bounds__(CT, SHARED ? 2 : 4) void moe_gateup_mfma_kernel(con
     const int tid = threadIdx.x;
     const uint32_t F = d.F, H = d.H;
     fill_mfma_tables(tab, tid, CT);
-    const uint32_t subs = F / (16 * Geo::BT * nb);
-    const uint32_t n_items = item_count<SHARED>(ws, d, N, subs);
+    const uint32_t tot = F / (16 * Geo::BT); // batches per item
+    uint32_t b0, b1;
+    my_batches<SHARED>(ws, d, N, tot, b0, b1);
 
-    for (uint32_t w = blockIdx.x; w < n_items; w += gridDim.x) {
-        const Item it = get_item<SHARED>(ws, w, subs, d, N);
-        const uint32_t row0 = it.sub * nb * Geo::BT * 16;
+    for (uint32_t b = b0; b < b1;) {
+        const uint32_t w = b / tot, f0 = b % tot, nbat = min(tot - f0, b1 - b);
+        const Item it = get_item<SHARED>(ws, w, d, N);
+        const uint32_t row0 = f0 * Geo::BT * 16;
         const size_t off = ((size_t)it.expert * F + row0) * Geo::RB;
         for (uint32_t t0 = 0; t0 < it.count; t0 += 16) {
             const uint32_t np = min(16u, it.count - t0);
             __syncthreads(); // previous tile fully consumed
             stage_pairs<SHARED>(ws, it, t0, np, d, N, s_tok, s_slot, tid);
             __syncthreads();
-            coop_stream<TYPE, 8, 2, 1, true, false>(gate + off, up + off, nb, X, H, np, [&](uint32_t r) { return s_tok[r]; },
+            coop_stream<TYPE, 8, 2, 1, true, false>(gate + off, up + off, nbat, X, H, np, [&](uint32_t r) { return s_tok[r]; },
                 smem, tab, tid, [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float sum1, uint32_t) {
                     const uint32_t r = 4 * (ln >> 4) + e;
                     if (r < np)
@@ -106,6 +143,7 @@ __global__ __launch_bounds__(CT, SHARED ? 2 : 4) void moe_gateup_mfma_kernel(con
                             (sum0 / (1.f + expf(-sum0))) * sum1;
                 });
         }
+        b += nbat;
     }
 }
 
@@ -119,8 +157,7 @@ using DnGeo = CoopGeom<TYPE, FB, 1, (TYPE == QKK_IQ4_XS ? 2 : 1)>;
 
 template <int TYPE, int FB, bool SHARED>
 __global__ __launch_bounds__(CT) void moe_down_mfma_kernel(const uint8_t* __restrict__ down, MoeWs ws,
-                                                           const qkk_sel* __restrict__ sel, MoeDims d, uint32_t N,
-                                                           uint32_t nb)
+                                                           const qkk_sel* __restrict__ sel, MoeDims d, uint32_t N)
 {
     using Geo = DnGeo<TYPE, FB>;
     constexpr int TG = TYPE == QKK_IQ4_XS ? 2 : 1;
@@ -131,12 +168,14 @@ __global__ __launch_bounds__(CT) void moe_down_mfma_kernel(const uint8_t* __rest
     const int tid = threadIdx.x;
     const uint32_t F = d.F, H = d.H;
     fill_mfma_tables(tab, tid, CT);
-    const uint32_t subs = H / (16 * Geo::BT * nb);
-    const uint32_t n_items = item_count<SHARED>(ws, d, N, subs);
+    const uint32_t tot = H / (16 * Geo::BT);
+    uint32_t b0, b1;
+    my_batches<SHARED>(ws, d, N, tot, b0, b1);
 
-    for (uint32_t w = blockIdx.x; w < n_items; w += gridDim.x) {
-        const Item it = get_item<SHARED>(ws, w, subs, d, N);
-        const uint32_t row0 = it.sub * nb * Geo::BT * 16;
+    for (uint32_t b = b0; b < b1;) {
+        const uint32_t w = b / tot, f0 = b % tot, nbat = min(tot - f0, b1 - b);
+        const Item it = get_item<SHARED>(ws, w, d, N);
+        const uint32_t row0 = f0 * Geo::BT * 16;
         const uint8_t* base = down + ((size_t)it.expert * H + row0) * Geo::RB;
         for (uint32_t t0 = 0; t0 < it.count; t0 += 16) {
             const uint32_t np = min(16u, it.count - t0);
@@ -145,7 +184,7 @@ __global__ __launch_bounds__(CT) void moe_down_mfma_kernel(const uint8_t* __rest
             __syncthreads();
             if (tid < 16) s_wt[tid] = (SHARED || (uint32_t)tid >= np) ? 1.f : sel[s_tok[tid]].w[s_slot[tid]];
             __syncthreads();
-            coop_stream<TYPE, FB, 1, TG, false, false>(base, nullptr, nb, ws.h, F, np,
+            coop_stream<TYPE, FB, 1, TG, false, false>(base, nullptr, nbat, ws.h, F, np,
                 [&](uint32_t r) { return s_tok[r] * (d.k + 1) + s_slot[r]; }, smem, tab, tid,
                 [&](uint32_t tile, uint32_t ln, uint32_t e, float sum0, float, uint32_t) {
                     const uint32_t r = 4 * (ln >> 4) + e;
@@ -154,6 +193,7 @@ __global__ __launch_bounds__(CT) void moe_down_mfma_kernel(const uint8_t* __rest
                             s_wt[r] * sum0;
                 });
         }
+        b += nbat;
     }
 }
 
@@ -235,23 +275,6 @@ __global__ __launch_bounds__(256) void moe_fold_norm_kernel(MoeWs ws, const qkk_
 // the batches that start inside its equal share of the total cost: every workgroup gets the same
 // work to within one batch whatever the number of active experts turns out to be (the host cannot
 // know it), and its batches are consecutive, so they form at most a few runs of one expert's rows.
-struct Share {
-    uint32_t s0, s1, r0, r1; // shared batches [s0, s1), routed batches [r0, r1)
-};
-
-__device__ __forceinline__ Share my_share(uint32_t g, uint32_t G, uint32_t ns, uint32_t cs, uint32_t nr, uint32_t cr)
-{
-    const uint64_t US = (uint64_t)ns * cs, U = US + (uint64_t)nr * cr;
-    const uint64_t u0 = U * g / G, u1 = U * (g + 1) / G;
-    const auto cdiv = [](uint64_t a, uint32_t b) { return (uint32_t)((a + b - 1) / b); };
-    Share sh;
-    sh.s0 = min(cdiv(min(u0, US), cs), ns);
-    sh.s1 = min(cdiv(min(u1, US), cs), ns);
-    sh.r0 = u0 > US ? min(cdiv(u0 - US, cr), nr) : 0u;
-    sh.r1 = u1 > US ? min(cdiv(u1 - US, cr), nr) : 0u;
-    return sh;
-}
-
 // ---- gate/up + SiLU --------------------------------------------------------------------------------
 // n_embd = 2048: the eight waves take one 256-weight fragment each.  Routed experts: batches of
 // one row tile of gate and of up (IQ3_XXS); shared expert (Q8_0): one row tile, gate and up in turns.
@@ -412,16 +435,6 @@ static uint32_t per_cu_of(const void* fn, uint32_t lds)
     return (uint32_t)std::min(n, 2);
 }
 
-// batches per sub-item: the largest power of two <= total that still gives each of the `wgs`
-// workgroups the launch can run at once an item (longer streams per workgroup amortise the
-// activation load and the pipeline fill of a sub-item; fewer items than workgroups leave CUs idle)
-static uint32_t pick_nb(uint32_t total_batches, uint32_t items, uint32_t wgs)
-{
-    uint32_t nb = total_batches;
-    while (nb > 1 && (uint64_t)items * (total_batches / nb) < wgs) nb /= 2;
-    return nb;
-}
-
 template <int TYPE, int FB>
 static void launch_down_fused(const qkk_moe_layer* L, const MoeWs& ws, const qkk_sel* sel, const MoeDims& d, uint32_t N,
                               hipStream_t st)
@@ -457,17 +470,18 @@ void moe_mfma_launch_fused(const qkk_moe_layer* L, const float* X, const qkk_sel
     }
 }
 
+// grid: what the device runs at once (per_cu workgroups per CU), no more than there are batches
 template <bool SHARED>
 static void launch_gateup(const qkk_moe_layer* L, const float* X, const MoeWs& ws, const MoeDims& d, uint32_t N,
                           uint32_t items, hipStream_t st)
 {
     using Geo = GuGeo<SHARED>;
     static const uint32_t per_cu = per_cu_of((const void*)moe_gateup_mfma_kernel<SHARED>, Geo::LDS_BYTES);
-    const uint32_t tot = d.F / (16 * Geo::BT), nb = pick_nb(tot, items, per_cu * (persistent_blocks() / 4));
-    const uint32_t blocks = std::min(items * (tot / nb), per_cu * (persistent_blocks() / 4));
+    const uint32_t tot = d.F / (16 * Geo::BT);
+    const uint32_t blocks = std::min(items * tot, per_cu * (persistent_blocks() / 4));
     hipLaunchKernelGGL(moe_gateup_mfma_kernel<SHARED>, dim3(blocks), dim3(CT), Geo::LDS_BYTES, st,
                        (const uint8_t*)(SHARED ? L->gate_shexp : L->gate_exps),
-                       (const uint8_t*)(SHARED ? L->up_shexp : L->up_exps), X, ws, d, N, nb);
+                       (const uint8_t*)(SHARED ? L->up_shexp : L->up_exps), X, ws, d, N);
 }
 
 template <int TYPE, int FB, bool SHARED>
@@ -476,10 +490,10 @@ static void launch_down(const void* W, const MoeWs& ws, const qkk_sel* sel, cons
 {
     using Geo = DnGeo<TYPE, FB>;
     static const uint32_t per_cu = per_cu_of((const void*)moe_down_mfma_kernel<TYPE, FB, SHARED>, Geo::LDS_BYTES);
-    const uint32_t tot = d.H / (16 * Geo::BT), nb = pick_nb(tot, items, per_cu * (persistent_blocks() / 4));
-    const uint32_t blocks = std::min(items * (tot / nb), per_cu * (persistent_blocks() / 4));
+    const uint32_t tot = d.H / (16 * Geo::BT);
+    const uint32_t blocks = std::min(items * tot, per_cu * (persistent_blocks() / 4));
     hipLaunchKernelGGL((moe_down_mfma_kernel<TYPE, FB, SHARED>), dim3(blocks), dim3(CT), Geo::LDS_BYTES, st,
-                       (const uint8_t*)W, ws, sel, d, N, nb);
+                       (const uint8_t*)W, ws, sel, d, N);
 }
 
 template <int TYPE, bool SHARED>
