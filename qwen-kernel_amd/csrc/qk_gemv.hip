@@ -169,10 +169,11 @@ __global__ __launch_bounds__(256) void gemv_q_kernel(const uint8_t* __restrict__
                                                      uint32_t row_bytes)
 {
     __shared__ IqTables tab;
-    if constexpr (TYPE == QKK_IQ3_XXS || TYPE == QKK_IQ4_XS) {
-        fill_iq_tables(tab, g_iq3xxs_grid, threadIdx.x, 256);
-        __syncthreads();
-    }
+    constexpr bool TABLES = TYPE == QKK_IQ3_XXS || TYPE == QKK_IQ4_XS;
+    // the codebook word travels with the first round trip (activations, first rows) and goes to LDS
+    // after those loads are issued: a fill and a barrier up front would be a round trip of their own
+    uint32_t grid_word = 0;
+    if constexpr (TABLES) grid_word = g_iq3xxs_grid[threadIdx.x];
     constexpr int GROUPS = WAVE / LPR; // rows a wave works on side by side
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lir = lane % LPR, grp = lane / LPR;
@@ -222,13 +223,30 @@ __global__ __launch_bounds__(256) void gemv_q_kernel(const uint8_t* __restrict__
         }
     };
     uint32_t r0 = (blockIdx.x * 4 + wave) * CHUNK;
+    if constexpr (TABLES || DEEP) fetch(0, r0); // rows past the end re-read the last row
+    if constexpr (TABLES) {
+        tab.grid[threadIdx.x] = grid_word;
+        if (threadIdx.x < 16) {
+            constexpr int8_t kv[16] = {QK_IQ4NL_VALUES};
+            float v = 0.f;
+#pragma unroll
+            for (int i = 0; i < 16; i++) v = (int)threadIdx.x == i ? (float)kv[i] : v;
+            tab.iq4[threadIdx.x] = v;
+        }
+        __syncthreads();
+    }
     if constexpr (DEEP) {
-        fetch(0, r0);
         for (; r0 < M; r0 += 2 * stride) {
             fetch(1, r0 + stride);
             reduce(0, r0);
             fetch(0, r0 + 2 * stride);
             reduce(1, r0 + stride);
+        }
+    } else if constexpr (TABLES) { // the first chunk is already on its way
+        while (r0 < M) {
+            reduce(0, r0);
+            r0 += stride;
+            if (r0 < M) fetch(0, r0); // wave-uniform
         }
     } else {
         for (; r0 < M; r0 += stride) {
