@@ -174,16 +174,18 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const uint8_t* __restrict
                                                        MoeWs ws, const qkk_sel* __restrict__ sel,
                                                        float* __restrict__ y, MoeDims d)
 {
+    extern __shared__ __attribute__((aligned(16))) float s_h[]; // [(k+1)][F]: the gated activations of every pick
     __shared__ IqTables tab;
     constexpr int GROUPS = WAVE / LPR;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lir = lane % LPR, grp = lane / LPR;
-    const float* h = ws.h;
     const uint32_t row_bytes = (uint32_t)qkk_row_bytes_dev<TYPE>(d.F);
     const uint32_t q8_row = d.F / 32 * Q8_0_BYTES;
     const uint32_t o0 = (blockIdx.x * 4 + wave) * RIF; // the grid covers every output once
 
-    // round trip 1
+    // round trip 1: everything that does not depend on the picks.  Every wave needs all of h (each
+    // lane group one pick's row per round): fetched once per workgroup and shared through LDS --
+    // a thousand waves each reading the same 18 KB made this round trip twice as long as the next.
     uint32_t eid[ROUNDS];
     float wt[ROUNDS];
 #pragma unroll
@@ -194,17 +196,20 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const uint8_t* __restrict
         wt[q] = sel->w[sc];
     }
     float wsh = sel->w_shared;
-    XSlice hs[ROUNDS], hsh;
+    const uint32_t h_quads = (d.k + 1) * d.F / 4;
+    constexpr int HQ = 8; // quads per thread in flight: covers (16 + 1) * 1024 / 4 / 256 = 17 in three rounds
+    const float4* hg = (const float4*)ws.h;
+    float4 hq[HQ];
 #pragma unroll
-    for (int q = 0; q < ROUNDS; q++) {
-        const uint32_t s = q * GROUPS + grp;
-        load_xslice<TYPE>(hs[q], h + (size_t)(s < d.k ? s : 0) * d.F, lir);
-    }
-    load_xslice<QKK_Q8_0>(hsh, h + (size_t)d.k * d.F, lir);
+    for (int i = 0; i < HQ; i++) hq[i] = hg[min(threadIdx.x + 256u * i, h_quads - 1)];
     LaneW<QKK_Q8_0> wq[RIF];
 #pragma unroll
     for (int i = 0; i < RIF; i++) wq[i].load(down_shexp + (size_t)min(o0 + i, d.H - 1) * q8_row, lir);
     fill_iq_tables(tab, g_iq3xxs_grid, threadIdx.x, 256);
+#pragma unroll
+    for (int i = 0; i < HQ; i++)
+        if (threadIdx.x + 256u * i < h_quads) ((float4*)s_h)[threadIdx.x + 256u * i] = hq[i];
+    for (uint32_t q4 = threadIdx.x + 256u * HQ; q4 < h_quads; q4 += 256u) ((float4*)s_h)[q4] = hg[q4]; // wide layers only
 
     // round trip 2
     LaneW<TYPE> w[RIF][ROUNDS];
@@ -216,6 +221,14 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const uint8_t* __restrict
         for (int i = 0; i < RIF; i++) w[i][q].load(base + (size_t)min(o0 + i, d.H - 1) * row_bytes, lir);
     }
     if (grp != 0) wsh = 0.f;
+    __syncthreads(); // h and the codebook in LDS
+    XSlice hs[ROUNDS], hsh;
+#pragma unroll
+    for (int q = 0; q < ROUNDS; q++) {
+        const uint32_t s = q * GROUPS + grp;
+        load_xslice<TYPE>(hs[q], s_h + (size_t)(s < d.k ? s : 0) * d.F, lir);
+    }
+    load_xslice<QKK_Q8_0>(hsh, s_h + (size_t)d.k * d.F, lir);
     float hsum[ROUNDS][4];
 #pragma unroll
     for (int q = 0; q < ROUNDS; q++)
@@ -226,7 +239,6 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const uint8_t* __restrict
             for (int i = 0; i < 8; i++) a += hs[q].v[c * 8 + i];
             hsum[q][c] = a;
         }
-    __syncthreads(); // codebook in LDS
 #pragma unroll
     for (int i = 0; i < RIF; i++) {
         float acc = wsh * wq[i].dot(hsh, nullptr, nullptr, lir);
@@ -276,7 +288,11 @@ static void launch_down2(const qkk_moe_layer* L, const MoeWs& ws, const qkk_sel*
                          const MoeDims& d, uint32_t n_slots, hipStream_t st)
 {
     const uint32_t waves = (d.H + RIF - 1) / RIF;
-    hipLaunchKernelGGL((moe_down_kernel<TYPE, LPR, ROUNDS, RIF>), dim3((waves + 3) / 4), dim3(256), 0, st,
+    const uint32_t lds = (d.k + 1) * d.F * 4; // h in LDS (at most 17 * 1024 floats = 68 KB)
+    static bool raised = ((void)hipFuncSetAttribute((const void*)moe_down_kernel<TYPE, LPR, ROUNDS, RIF>,
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, 17 * 1024 * 4), true);
+    (void)raised;
+    hipLaunchKernelGGL((moe_down_kernel<TYPE, LPR, ROUNDS, RIF>), dim3((waves + 3) / 4), dim3(256), lds, st,
                        (const uint8_t*)L->down_exps, (const uint8_t*)L->down_shexp, ws, sel, Y, d);
 }
 
