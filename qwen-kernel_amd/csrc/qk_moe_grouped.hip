@@ -171,6 +171,11 @@ __global__ __launch_bounds__(512) void moe_route_multi_kernel(const float* __res
 // workgroup instead of once per dot product.  Same arithmetic, in the same order, as
 // moe_route_multi_kernel: a token's logits do not depend on how many tokens ride along.
 constexpr uint32_t LOGITS_TILE_TOKENS = 16;
+// Grid = (groups of 8 router rows) x (token tiles).  At 256 experts the shared-gate row (row E) makes
+// a 33rd, nearly empty row group; where that pushes the grid past one workgroup per CU (128 tokens:
+// 264 workgroups, a second round for eight of them) the launcher sets `ride`, and the row rides
+// along instead: in every token tile one workgroup's wave 0 takes it as a second row.
+template <bool RIDE>
 __global__ __launch_bounds__(512) void moe_logits_tiled_kernel(const float* __restrict__ gate_inp,
                                                                const float* __restrict__ gate_inp_shexp,
                                                                const float* __restrict__ X, MoeWs ws, MoeDims d,
@@ -179,33 +184,51 @@ __global__ __launch_bounds__(512) void moe_logits_tiled_kernel(const float* __re
     extern __shared__ __attribute__((aligned(16))) float s_x[]; // [16][2048]
     constexpr int NCH = 8;                                      // n_embd = 2048: eight float4 per lane
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t n_rows = d.E + 1, rgroups = (n_rows + 7) / 8;
-    const uint32_t r = (blockIdx.x % rgroups) * 8 + wave, t0 = (blockIdx.x / rgroups) * LOGITS_TILE_TOKENS;
+    const uint32_t n_rows = RIDE ? d.E : d.E + 1; // rows dealt out in groups of eight
+    const uint32_t rgroups = (n_rows + 7) / 8;
+    const uint32_t rg = blockIdx.x % rgroups, tt = blockIdx.x / rgroups;
+    const uint32_t r = rg * 8 + wave, t0 = tt * LOGITS_TILE_TOKENS;
     const uint32_t nt = min(LOGITS_TILE_TOKENS, N - t0);
     const uint32_t LS = lstride(d.E);
+    const bool extra = RIDE && wave == 0 && rg == tt % rgroups; // this wave also takes the shared-gate row
 
     const float4* xs = (const float4*)(X + (size_t)t0 * 2048); // nt consecutive rows: one contiguous range
     float4 xv[LOGITS_TILE_TOKENS];
 #pragma unroll
     for (uint32_t i = 0; i < LOGITS_TILE_TOKENS; i++) xv[i] = xs[min(threadIdx.x + 512 * i, nt * 512 - 1)];
-    float4 w[NCH];
-    const float4* row = (const float4*)(r < d.E ? gate_inp + (size_t)r * 2048 : gate_inp_shexp);
+    float4 w[NCH], w2[NCH];
+    const float4* row = (const float4*)(r < d.E ? gate_inp + (size_t)r * 2048 : gate_inp_shexp); // row E = shared gate
+    const float4* row2 = (const float4*)gate_inp_shexp;
 #pragma unroll
     for (int i = 0; i < NCH; i++) w[i] = row[lane + 64 * i];
+    if constexpr (RIDE) {
+#pragma unroll
+        for (int i = 0; i < NCH; i++) w2[i] = extra ? row2[lane + 64 * i] : float4{0.f, 0.f, 0.f, 0.f};
+    }
 #pragma unroll
     for (uint32_t i = 0; i < LOGITS_TILE_TOKENS; i++) ((float4*)s_x)[threadIdx.x + 512 * i] = xv[i];
     __syncthreads();
     if (r >= n_rows) return;
     for (uint32_t t = 0; t < nt; t++) {
-        float a0 = 0.f, a1 = 0.f;
+        float a0 = 0.f, a1 = 0.f, b0 = 0.f, b1 = 0.f;
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
             const float4 x = ((const float4*)s_x)[t * 512 + lane + 64 * i];
             a0 += w[i].x * x.x + w[i].y * x.y;
             a1 += w[i].z * x.z + w[i].w * x.w;
+            if constexpr (RIDE) {
+                if (extra) { // wave-uniform
+                    b0 += w2[i].x * x.x + w2[i].y * x.y;
+                    b1 += w2[i].z * x.z + w2[i].w * x.w;
+                }
+            }
         }
         const float sum = wave_sum(a0 + a1);
         if (lane == 0) ws.logits[(size_t)(t0 + t) * LS + r] = sum;
+        if (RIDE && extra) {
+            const float sum2 = wave_sum(b0 + b1);
+            if (lane == 0) ws.logits[(size_t)(t0 + t) * LS + d.E] = sum2;
+        }
     }
 }
 
@@ -290,12 +313,21 @@ int moe_grouped_launch(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel
                                L->gate_inp_shexp, X, ws, sel, d, N, 1u);
         } else { // tiled logits, then selection one token per wave + grouping
             constexpr uint32_t lds = LOGITS_TILE_TOKENS * 2048 * sizeof(float);
-            static bool once = ((void)hipFuncSetAttribute((const void*)moe_logits_tiled_kernel,
+            static bool once = ((void)hipFuncSetAttribute((const void*)moe_logits_tiled_kernel<false>,
+                                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
+                                (void)hipFuncSetAttribute((const void*)moe_logits_tiled_kernel<true>,
                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds), true);
             (void)once;
-            const uint32_t grid = (d.E + 1 + 7) / 8 * ((N + LOGITS_TILE_TOKENS - 1) / LOGITS_TILE_TOKENS);
-            hipLaunchKernelGGL(moe_logits_tiled_kernel, dim3(grid), dim3(512), lds, st, L->gate_inp, L->gate_inp_shexp, X,
-                               ws, d, N);
+            const uint32_t tiles = (N + LOGITS_TILE_TOKENS - 1) / LOGITS_TILE_TOKENS, cus = persistent_blocks() / 4;
+            const uint32_t g_all = (d.E + 1 + 7) / 8 * tiles, g_ride = (d.E + 7) / 8 * tiles;
+            // fewer rounds of workgroups (one per CU: the activation tile takes 128 KB of LDS) decide
+            const uint32_t ride = (g_ride + cus - 1) / cus < (g_all + cus - 1) / cus ? 1u : 0u;
+            if (ride)
+                hipLaunchKernelGGL(moe_logits_tiled_kernel<true>, dim3(g_ride), dim3(512), lds, st, L->gate_inp,
+                                   L->gate_inp_shexp, X, ws, d, N);
+            else
+                hipLaunchKernelGGL(moe_logits_tiled_kernel<false>, dim3(g_all), dim3(512), lds, st, L->gate_inp,
+                                   L->gate_inp_shexp, X, ws, d, N);
             hipLaunchKernelGGL(moe_select_group_kernel, dim3((N + 15) / 16), dim3(1024), 0, st, ws, sel, d, N);
         }
     }
