@@ -123,6 +123,8 @@ def moe_workload(qk, n_slots, down_type, ring, steps, warmup, seed=1234):
         stage_ms[name] = sev
     H, F = 2048, 512
     gu_bytes = u * 2 * F * qk.row_bytes(qk.IQ3_XXS, H) + n_slots * (H * 4 + 9 * F * 4)
+    if 2 <= n_slots <= 32:   # few rows: the same launch streams the shared expert's gate and up rows
+        gu_bytes += 2 * F * qk.row_bytes(qk.Q8_0, H) * ((n_slots + 15) // 16)
     return dict(ms_wall=wall, ms_event=ev, steps=n, bytes_step=bytes_step, distinct_experts=u, stage_ms=stage_ms,
                 gateup_bytes=gu_bytes, ring=ring, ring_bytes=ring * L.active_bytes(L.n_expert))
 
@@ -310,8 +312,11 @@ def main():
     # stage alone on the same ring (profiles/ holds the rocprofv3 figure for the same kernel)
     gu_ms = m["stage_ms"]["gateup"]
     ach = m["gateup_bytes"] / (gu_ms * 1e-3) / 1e9
-    kname = "moe_gateup_kernel" if a.workload == "moe_decode_bs1" else "moe_gateup_mfma_kernel"
-    roof = dict(bound="hbm", kernel=kname + " (select + routed IQ3_XXS gate/up + SiLU)", achieved=ach,
+    kname, kwhat = {"moe_decode_bs1": ("moe_gateup_kernel", "select + routed IQ3_XXS gate/up + SiLU"),
+                    "moe_decode_bs16": ("moe_gateup_fused_kernel", "routed IQ3_XXS + shared Q8_0 gate/up + SiLU"),
+                    "moe_prefill_128": ("moe_gateup_mfma_kernel", "routed IQ3_XXS gate/up + SiLU; the stage time also "
+                                        "covers the shared expert's launch on the side stream")}[a.workload]
+    roof = dict(bound="hbm", kernel=f"{kname} ({kwhat})", achieved=ach,
                 peak=HBM_PEAK_GBPS, unit="GB/s", frac=ach / HBM_PEAK_GBPS, traffic=TRAFFIC.get(kname),
                 bytes_per_launch=m["gateup_bytes"], us_per_launch=gu_ms * 1e3)
     out = dict(metric="fused_moe_decode_step_hbm_gbps", value=gbps, unit="GB/s", n_gpus=1, steps=m["steps"],
