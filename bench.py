@@ -27,7 +27,8 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what
 # the same counters read for a plain 256 MiB copy (see profiles/); None where no counter run
 # of that kernel has been recorded.
-TRAFFIC = {"moe_gateup_kernel": 6722776}  # profiles/moe_decode_bs1_hbm_traffic.txt
+TRAFFIC = {"moe_gateup_kernel": 6722776,          # profiles/moe_decode_bs1_hbm_traffic.txt
+           "moe_gateup_fused_kernel": 85845150}   # profiles/moe_decode_bs16_hbm_traffic.txt (103 distinct experts)
 
 
 def log(*a):
