@@ -7,12 +7,19 @@
  * Threading: every function is called from one engine thread; nothing is thread-safe;
  * qk_step_chunk blocks that thread for one chunk of device steps.
  *
- * State of this build: the engine entry points validate their arguments and report errors
- * exactly as the reference does, but qk_open() cannot run a whole model yet -- the
- * attention and gated-DeltaNet mixers between the MoE blocks are outside the path this
- * library implements -- so it fails with a message saying so.  The kernels of the path
- * (GEMVs, fused MoE step, LM head + argmax, prefill GEMMs) are reached through
- * qk_kernels.h.
+ * What qk_open() runs: a GGUF whose layers are MoE blocks only (token embedding, per layer
+ * post_attention_norm + the eight MoE tensors, output_norm, Q6_K head) -- the reference's decode
+ * step with every mixer output zero.  A file whose layers carry attention or gated-DeltaNet
+ * mixer tensors is refused with a message saying that the mixers are not part of this library.
+ * On the file it accepts, every entry point behaves as the reference's: argument checks and
+ * return codes, the serial-step state machine of qk_step_chunk (one captured hipGraph per
+ * dispatch depth), greedy sampling, EOS / max_gen / n_ctx endings.  Such a model keeps no
+ * per-position state, so snapshots validate their bounds only, as in the reference's stub
+ * engine (reference stub/qk_stub.c:95-106).  QK_LAYERS pipeline stages are refused: one GPU runs
+ * every layer.  A device failure inside qk_step_chunk / qk_stage_run / qk_stage_topk returns -6.
+ * Environment, as in the reference: QK_MAXB (batch-prefill chunk, 16..1024, default 128),
+ * QK_NO_BATCH (serial prefill of the whole prompt); and QK_NO_GRAPH (launch the step's kernels
+ * one by one instead of replaying the graph).
  */
 #ifndef QK_H
 #define QK_H

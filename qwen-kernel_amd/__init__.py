@@ -14,3 +14,4 @@ from .capi import (  # noqa: F401
 )
 from . import synth  # noqa: F401
 from . import gguf  # noqa: F401
+from . import engine  # noqa: F401

@@ -1,32 +1,451 @@
-// qk_engine.cpp -- engine-level C ABI (include/qk.h).
+// qk_engine.cpp -- engine-level C ABI (include/qk.h): the slot state machine of the reference
+// engine (reference src/main.cpp:4462-4666 stepChunk, 5447-5532 slot start / cancel / step)
+// over the kernels of this library, one hipGraph per dispatch depth in place of the
+// reference's pre-recorded command buffers (reference src/main.cpp:4186-4422).
 //
-// The reference engine runs a whole hybrid model; this library implements the quantized
-// decode hot path only (GEMVs, fused MoE step, LM head, prefill GEMMs -- see qk_kernels.h).
-// qk_open() therefore validates its arguments with the reference's limits and messages
-// (reference src/main.cpp:3575, 5396-5402) and then reports that a whole-model engine
-// cannot be built from the kernels present.  Every other entry point keeps the
-// reference's argument checks and return codes (reference src/main.cpp:5405-5532) so a
-// host that resolves the full symbol set loads this library unchanged.
-#include <stdio.h>
+// What the engine can run.  The reference model alternates a mixer (attention or gated
+// DeltaNet) with a MoE block in every layer.  The mixers are not part of this library, so
+// qk_open() refuses a file whose layers carry mixer tensors; it runs a file whose layers are
+// MoE blocks only:
+//   x      = embed(token)                                    token_embd.weight (Q6_K / Q8_0)
+//   layer: xn = rmsnorm(x, blk.l.post_attention_norm);  x = x + MoE_l(xn)
+//   token' = argmax(output.weight . rmsnorm(x, output_norm)) Q6_K head, ties to the lower id
+// -- the reference's decode step (src/main.cpp:4194-4405) with every mixer output taken as
+// zero.  Such a model keeps no per-position state, so a slot's device state is empty:
+// snapshots validate their bounds only and a batch-prefilled position has nothing to write.
+// Everything the host sees -- argument checks, return codes, which step emits which token,
+// EOS / max_gen / n_ctx endings, the finished mask -- follows the reference line by line.
+#include <stdlib.h>
+#include <string.h>
 
+#include <algorithm>
 #include <new>
+#include <string>
 #include <vector>
 
 #include "../../include/qk.h"
+#include "../../include/qk_gguf.h"
+#include "qk_host.h"
+
+namespace {
+
+constexpr uint32_t N_EMBD = 2048;           // reference src/main.cpp:3086 (compile-time there too)
+constexpr uint32_t MAX_ROWS = QKK_MAX_SLOTS; // rows one device step carries
+constexpr uint32_t N_STATE = 3;             // snapshot entries (reference default, stub/qk_stub.c:98)
+constexpr int ERR_DEVICE = -6;              // a launch, copy or synchronisation failed
+
+struct EngineLayer {
+    qkk_moe_layer moe;
+    const float* post_norm; // blk.l.post_attention_norm.weight
+};
+
+} // namespace
 
 struct qk_engine {
     uint32_t n_slots = 0, n_ctx = 0, chunk = 0;
-    uint32_t vocab = 0, eos = 0, bos = 0;
-    uint32_t layer_first = 0, layer_end = 0, n_layer = 0, n_embd = 2048;
-    uint32_t n_state = 0;
-    bool split = false;
-    struct Slot { bool active = false; };
+    uint32_t vocab = 0, eos = 248046, bos = 248044; // reference src/main.cpp:3084
+    uint32_t n_layer = 40, layer_first = 0, layer_end = 0;
+    uint32_t max_b = 128; // batch-prefill chunk width (reference src/main.cpp:3833)
+    int embd_type = 0;
+    uint32_t embd_rows = 0;
+    float eps = 1e-6f; // reference src/main.cpp:1434
+
+    // device side
+    hipStream_t st = nullptr;
+    std::vector<void*> dev_allocs;
+    const void* d_embd = nullptr;
+    const void* d_head = nullptr;
+    const float* d_onorm = nullptr;
+    std::vector<EngineLayer> layers;
+    uint32_t* d_ids = nullptr;  // [MAX_ROWS] tokens fed this step
+    uint32_t* d_tok = nullptr;  // [MAX_ROWS] tokens sampled this step
+    float* d_x = nullptr;       // [MAX_ROWS][N_EMBD] residual stream
+    float* d_xn[2] = {nullptr, nullptr}; // normalised rows, alternating between layers
+    float* d_last = nullptr;    // [N_EMBD] final normalised row of the last stage run
+    float* d_logits = nullptr;  // [vocab]
+    qkk_sel* d_sel = nullptr;
+    void* d_ws = nullptr;
+    size_t ws_bytes = 0;
+    void* d_hws = nullptr;
+    size_t hws_bytes = 0;
+    uint32_t* h_ids = nullptr; // pinned, [MAX_ROWS]
+    uint32_t* h_tok = nullptr; // pinned, [MAX_ROWS]
+    std::vector<hipGraphExec_t> graphs; // [depth - 1], empty when graphs are switched off
+    uint32_t last_run_rows = 0;
+
+    // host side (reference src/main.cpp:3153-3175, Slot)
+    struct Slot {
+        bool active = false;
+        std::vector<uint32_t> prompt;
+        uint32_t cursor = 0, pos = 0, last = 0, gen = 0, max_gen = 0;
+    };
     std::vector<Slot> slots;
+
+    ~qk_engine();
+    bool open(const char* path, const qk_config& cfg, char* err, size_t err_len);
+    bool upload(const qkg_tensor& t, const void** out, char* err, size_t err_len);
+    void* dev_alloc(size_t bytes, bool zero);
+    int launch_rows(uint32_t rows, float** final_rows);
+    int run_rows(uint32_t rows, bool graph_ok);
+    int step_chunk(uint32_t* out_tok, uint32_t* out_cnt, uint32_t* out_fin);
+    int stage_run(uint32_t slot, const uint32_t* toks, const float* hidden_in, uint32_t n, uint32_t base,
+                  float* hidden_out, uint32_t* ids_out);
+    int stage_topk(uint32_t k, uint32_t* ids, float* vals);
+    bool split() const { return layer_first != 0 || layer_end != n_layer; }
 };
 
-static void set_err(char* err, size_t n, const char* msg)
+static bool set_err(char* err, size_t n, const char* msg)
 {
     if (err && n) snprintf(err, n, "%s", msg);
+    return false;
+}
+
+qk_engine::~qk_engine()
+{
+    if (st) (void)hipStreamSynchronize(st);
+    for (hipGraphExec_t g : graphs)
+        if (g) (void)hipGraphExecDestroy(g);
+    for (void* p : dev_allocs) (void)hipFree(p);
+    if (h_ids) (void)hipHostFree(h_ids);
+    if (h_tok) (void)hipHostFree(h_tok);
+    if (st) (void)hipStreamDestroy(st);
+}
+
+// Device memory the engine owns until it closes, 256 spare bytes behind it; nullptr on failure.
+void* qk_engine::dev_alloc(size_t bytes, bool zero)
+{
+    void* p = nullptr;
+    if (hipMalloc(&p, bytes + 256) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    dev_allocs.push_back(p);
+    if (zero && hipMemset(p, 0, bytes + 256) != hipSuccess) return nullptr;
+    return p;
+}
+
+// Copies one tensor of the file into device memory of its own (256 spare bytes behind it).
+bool qk_engine::upload(const qkg_tensor& t, const void** out, char* err, size_t err_len)
+{
+    uint8_t* p = (uint8_t*)dev_alloc(t.nbytes, false);
+    if (!p) return set_err(err, err_len, "qk_open: device memory exhausted");
+    if (hipMemcpy(p, t.data, t.nbytes, hipMemcpyHostToDevice) != hipSuccess ||
+        hipMemset(p + t.nbytes, 0, 256) != hipSuccess)
+        return set_err(err, err_len, "qk_open: upload failed");
+    *out = p;
+    return true;
+}
+
+// The launches of one device step over `rows` rows: d_ids -> d_tok.  *final_rows receives the
+// buffer that holds the rows normalised with output_norm (the LM head's input).
+int qk_engine::launch_rows(uint32_t rows, float** final_rows)
+{
+    if (rows < 1 || rows > MAX_ROWS) return QKK_ESHAPE;
+    if (int rc = qkk_embed(embd_type, d_embd, embd_rows, N_EMBD, d_ids, MAX_ROWS, 0, 1, d_x, rows, st)) return rc;
+    if (int rc = qkk_rmsnorm(d_x, layers[0].post_norm, d_xn[0], N_EMBD, rows, eps, st)) return rc;
+    int cur = 0;
+    for (size_t l = 0; l < layers.size(); l++) {
+        const float* w_next = l + 1 < layers.size() ? layers[l + 1].post_norm : d_onorm;
+        if (int rc = qkk_moe_decode_tail(&layers[l].moe, d_xn[cur], d_x, w_next, eps, d_x, d_xn[cur ^ 1], d_sel, d_ws,
+                                         ws_bytes, rows, st))
+            return rc;
+        cur ^= 1;
+    }
+    if (final_rows) *final_rows = d_xn[cur];
+    return qkk_head_argmax(d_head, d_xn[cur], d_tok, nullptr, vocab, N_EMBD, rows, d_hws, hws_bytes, st);
+}
+
+// One device step: h_ids[0..rows) in, h_tok[0..rows) out, host blocked until it is done.
+int qk_engine::run_rows(uint32_t rows, bool graph_ok)
+{
+    if (hipMemcpyAsync(d_ids, h_ids, rows * sizeof(uint32_t), hipMemcpyHostToDevice, st) != hipSuccess)
+        return ERR_DEVICE;
+    if (graph_ok && rows <= graphs.size() && graphs[rows - 1]) {
+        if (hipGraphLaunch(graphs[rows - 1], st) != hipSuccess) return ERR_DEVICE;
+    } else if (launch_rows(rows, nullptr) != QKK_OK) {
+        return ERR_DEVICE;
+    }
+    if (hipMemcpyAsync(h_tok, d_tok, rows * sizeof(uint32_t), hipMemcpyDeviceToHost, st) != hipSuccess)
+        return ERR_DEVICE;
+    if (hipStreamSynchronize(st) != hipSuccess) return ERR_DEVICE;
+    return 0;
+}
+
+bool qk_engine::open(const char* path, const qk_config& cfg, char* err, size_t err_len)
+{
+    auto bad = [&](const char* m) { return set_err(err, err_len, m); };
+    n_slots = cfg.n_slots; n_ctx = cfg.n_ctx; chunk = cfg.chunk;
+    // reference src/main.cpp:3575
+    if (n_slots < 1 || n_slots > 16 || n_ctx < 64 || n_ctx > 65536 || chunk < 1 || chunk > 32)
+        return bad("qk_open: bad config");
+    qkg_file* g = qkg_open(path);
+    if (!g) return bad("qk_open: cannot open GGUF");
+    struct Closer { qkg_file* g; ~Closer() { qkg_close(g); } } closer{g};
+
+    // model shape and token ids (reference src/main.cpp:3580-3590)
+    const char* arch_c = "";
+    (void)qkg_kv_str(g, "general.architecture", &arch_c);
+    const std::string arch = arch_c ? arch_c : "";
+    uint64_t v = 0;
+    if (qkg_kv_int(g, (arch + ".block_count").c_str(), &v) == 0) n_layer = (uint32_t)v;
+    if (n_layer < 1 || n_layer > 256) return bad("qk_open: bad block_count");
+    uint32_t n_used = 8;
+    if (qkg_kv_int(g, (arch + ".expert_used_count").c_str(), &v) == 0) n_used = (uint32_t)v;
+    if (n_used < 1 || n_used > 16) return bad("qk_open: expert_used_count > 16 unsupported");
+    if (qkg_kv_int(g, "tokenizer.ggml.eos_token_id", &v) == 0) eos = (uint32_t)v;
+    if (qkg_kv_int(g, "tokenizer.ggml.bos_token_id", &v) == 0) bos = (uint32_t)v;
+    layer_end = n_layer;
+    // reference src/main.cpp:3594-3601: a:b selects a pipeline stage
+    if (const char* lay = getenv("QK_LAYERS")) {
+        unsigned a = 0, b = 0;
+        if (sscanf(lay, "%u:%u", &a, &b) == 2 && a < b && b <= n_layer) { layer_first = a; layer_end = b; }
+        else {
+            if (err && err_len)
+                snprintf(err, err_len, "qk_open: bad QK_LAYERS (want a:b with 0 <= a < b <= %u)", n_layer);
+            return false;
+        }
+        if (split()) return bad("qk_open: QK_LAYERS pipeline stages are not part of this library (one GPU runs every layer)");
+    }
+    if (const char* mb = getenv("QK_MAXB")) { // reference src/main.cpp:3834-3838
+        const long x = atol(mb);
+        if (x >= 16 && x <= 1024) max_b = (uint32_t)x;
+        else fprintf(stderr, "QK_MAXB=%s out of range [16,1024]; using %u\n", mb, max_b);
+    }
+
+    // reference src/main.cpp:3602-3609
+    qkg_tensor t_embd, t_onorm, t_head;
+    if (qkg_find(g, "token_embd.weight", &t_embd) || qkg_find(g, "output_norm.weight", &t_onorm) ||
+        qkg_find(g, "output.weight", &t_head) || (t_embd.type != QKK_Q6_K && t_embd.type != QKK_Q8_0) ||
+        t_head.type != QKK_Q6_K)
+        return bad("qk_open: missing/unexpected embd/head tensors");
+    // what the reference leaves to its shaders: shapes that fit each other
+    if (t_embd.ne[0] != N_EMBD || t_head.ne[0] != N_EMBD || t_onorm.type != QKK_F32 || t_onorm.ne[0] != N_EMBD ||
+        t_head.ne[1] < 1 || t_head.ne[1] > 0x7fffffffu || t_embd.ne[1] < t_head.ne[1] || t_embd.ne[1] > 0x7fffffffu ||
+        !t_embd.nbytes || !t_head.nbytes || !t_onorm.nbytes)
+        return bad("qk_open: missing/unexpected embd/head tensors");
+    embd_type = (int)t_embd.type;
+    embd_rows = (uint32_t)t_embd.ne[1];
+    vocab = (uint32_t)t_head.ne[1];
+
+    // the layers: MoE tensor sets (reference src/main.cpp:3611-3622, 1265-1311) and no mixer
+    std::vector<qkg_moe_tensors> mt(n_layer);
+    std::vector<qkg_tensor> pn(n_layer);
+    for (uint32_t l = 0; l < n_layer; l++) {
+        char name[96];
+        for (const char* mixer : {"attn_qkv.weight", "attn_q.weight", "attn_output.weight", "ssm_out.weight"}) {
+            snprintf(name, sizeof name, "blk.%u.%s", l, mixer);
+            qkg_tensor tmp;
+            if (qkg_find(g, name, &tmp) == 0)
+                return bad("qk_open: this libqk.so implements the quantized decode hot path only (see qk_kernels.h); "
+                           "the attention / gated-DeltaNet mixers this file's layers need are not part of it");
+        }
+        if (qkg_moe_layer(g, l, &mt[l]) != 0) {
+            if (err && err_len) snprintf(err, err_len, "qk_open: %s", qkk_last_error());
+            return false;
+        }
+        if (l == 0 && (mt[0].n_expert < n_used || mt[0].n_expert > 512 || mt[0].n_ff % 256 != 0))
+            return bad("qk_open: expert shape unsupported (n_expert <= 512, n_ff_exp % 256)");
+        if (mt[l].n_embd != N_EMBD || mt[l].n_expert != mt[0].n_expert || mt[l].n_ff != mt[0].n_ff)
+            return bad("qk_open: expert shape unsupported (n_embd 2048, uniform layers)");
+        snprintf(name, sizeof name, "blk.%u.post_attention_norm.weight", l);
+        if (qkg_find(g, name, &pn[l]) || pn[l].type != QKK_F32 || pn[l].ne[0] != N_EMBD || !pn[l].nbytes)
+            return bad("qk_open: missing/unexpected post_attention_norm tensor");
+    }
+
+    // ---- device ----
+    if (qk::require_device() != QKK_OK) return bad("qk_open: no HIP device: libqk.so has no CPU path");
+    uint64_t need = t_embd.nbytes + t_head.nbytes + (64u << 20);
+    for (uint32_t l = 0; l < n_layer; l++)
+        for (const qkg_tensor* t : {&mt[l].gate_inp, &mt[l].gate_inp_shexp, &mt[l].gate_exps, &mt[l].up_exps,
+                                    &mt[l].down_exps, &mt[l].gate_shexp, &mt[l].up_shexp, &mt[l].down_shexp})
+            need += t->nbytes + 512;
+    size_t free_b = 0, total_b = 0;
+    if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) return bad("qk_open: cannot query device memory");
+    if (need > free_b) return bad("qk_open: the model does not fit this device's free memory");
+    if (hipStreamCreateWithFlags(&st, hipStreamNonBlocking) != hipSuccess) return bad("qk_open: cannot create a stream");
+
+    const void* p = nullptr;
+    if (!upload(t_embd, &d_embd, err, err_len) || !upload(t_head, &d_head, err, err_len) ||
+        !upload(t_onorm, &p, err, err_len))
+        return false;
+    d_onorm = (const float*)p;
+    layers.resize(n_layer);
+    for (uint32_t l = 0; l < n_layer; l++) {
+        qkk_moe_layer& m = layers[l].moe;
+        m.n_embd = mt[l].n_embd; m.n_ff = mt[l].n_ff; m.n_expert = mt[l].n_expert; m.n_used = mt[l].n_used;
+        m.gu_type = mt[l].gu_type; m.down_type = mt[l].down_type;
+        const void *gi = nullptr, *gis = nullptr;
+        if (!upload(mt[l].gate_inp, &gi, err, err_len) || !upload(mt[l].gate_inp_shexp, &gis, err, err_len) ||
+            !upload(mt[l].gate_exps, &m.gate_exps, err, err_len) || !upload(mt[l].up_exps, &m.up_exps, err, err_len) ||
+            !upload(mt[l].down_exps, &m.down_exps, err, err_len) || !upload(mt[l].gate_shexp, &m.gate_shexp, err, err_len) ||
+            !upload(mt[l].up_shexp, &m.up_shexp, err, err_len) || !upload(mt[l].down_shexp, &m.down_shexp, err, err_len) ||
+            !upload(pn[l], &p, err, err_len))
+            return false;
+        m.gate_inp = (const float*)gi;
+        m.gate_inp_shexp = (const float*)gis;
+        layers[l].post_norm = (const float*)p;
+    }
+
+    for (const EngineLayer& L : layers) ws_bytes = std::max(ws_bytes, qkk_moe_workspace_bytes(&L.moe, MAX_ROWS));
+    hws_bytes = qkk_head_workspace_bytes(vocab, MAX_ROWS);
+    if (!ws_bytes || !hws_bytes) return bad("qk_open: expert shape unsupported by the kernels");
+    const size_t row_b = (size_t)MAX_ROWS * N_EMBD * sizeof(float);
+    d_ids = (uint32_t*)dev_alloc(MAX_ROWS * 4, true);
+    d_tok = (uint32_t*)dev_alloc(MAX_ROWS * 4, true);
+    d_x = (float*)dev_alloc(row_b, true);
+    d_xn[0] = (float*)dev_alloc(row_b, true);
+    d_xn[1] = (float*)dev_alloc(row_b, true);
+    d_last = (float*)dev_alloc(N_EMBD * sizeof(float), true);
+    d_logits = (float*)dev_alloc((size_t)vocab * sizeof(float), true);
+    d_sel = (qkk_sel*)dev_alloc(MAX_ROWS * sizeof(qkk_sel), true);
+    d_ws = dev_alloc(ws_bytes, true);   // the kernels' workspaces start zero-filled
+    d_hws = dev_alloc(hws_bytes, true);
+    if (!d_ids || !d_tok || !d_x || !d_xn[0] || !d_xn[1] || !d_last || !d_logits || !d_sel || !d_ws || !d_hws)
+        return bad("qk_open: device memory exhausted");
+    if (hipHostMalloc((void**)&h_ids, MAX_ROWS * 4, hipHostMallocDefault) != hipSuccess ||
+        hipHostMalloc((void**)&h_tok, MAX_ROWS * 4, hipHostMallocDefault) != hipSuccess)
+        return bad("qk_open: cannot allocate pinned memory");
+    memset(h_ids, 0, MAX_ROWS * 4);
+    memset(h_tok, 0, MAX_ROWS * 4);
+    if (hipDeviceSynchronize() != hipSuccess) return bad("qk_open: upload failed"); // fills and uploads are complete
+
+    // One graph per dispatch depth z = highest active slot + 1 (the reference records one
+    // command buffer per z, src/main.cpp:4169-4422).  Each depth runs once eagerly first, so
+    // that whatever a launcher sets up on its first call is not part of a capture.
+    const bool use_graphs = !getenv("QK_NO_GRAPH");
+    graphs.assign(use_graphs ? n_slots : 0, nullptr);
+    for (uint32_t z = 1; z <= n_slots; z++) {
+        if (run_rows(z, false) != 0) {
+            if (err && err_len) snprintf(err, err_len, "qk_open: device step failed: %s", qkk_last_error());
+            return false;
+        }
+        if (!use_graphs) continue;
+        hipGraph_t graph = nullptr;
+        if (hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal) != hipSuccess)
+            return bad("qk_open: graph capture failed");
+        const int rc = launch_rows(z, nullptr);
+        const hipError_t ec = hipStreamEndCapture(st, &graph);
+        if (rc != QKK_OK || ec != hipSuccess || !graph) {
+            if (graph) (void)hipGraphDestroy(graph);
+            return bad("qk_open: graph capture failed");
+        }
+        const hipError_t ei = hipGraphInstantiate(&graphs[z - 1], graph, nullptr, nullptr, 0);
+        (void)hipGraphDestroy(graph);
+        if (ei != hipSuccess) { graphs[z - 1] = nullptr; return bad("qk_open: graph instantiation failed"); }
+    }
+    slots.assign(n_slots, Slot{});
+    return true;
+}
+
+// reference src/main.cpp:4462-4646 with speculative decoding off: its phases 1 and 2 only move
+// tokens a verify round left over, so phase 3 (serial steps) is the whole chunk.
+int qk_engine::step_chunk(uint32_t* out_tok, uint32_t* out_cnt, uint32_t* out_fin)
+{
+    for (uint32_t s = 0; s < n_slots; s++) out_cnt[s] = 0;
+    *out_fin = 0;
+    int active_at_entry = 0;
+    for (uint32_t s = 0; s < n_slots; s++)
+        if (slots[s].active) active_at_entry++;
+    if (!active_at_entry) return 0;
+
+    auto finish = [&](uint32_t s) {
+        slots[s].active = false;
+        *out_fin |= 1u << s;
+    };
+    for (uint32_t step = 0; step < chunk; step++) {
+        uint32_t n_act = 0, max_z = 0; // max_z: highest active slot + 1, the dispatch depth
+        bool need = false;             // someone still owes prefill progress or emitted tokens
+        for (uint32_t s = 0; s < n_slots; s++) {
+            Slot& sl = slots[s];
+            if (!sl.active) { h_ids[s] = 0; continue; }
+            n_act++;
+            max_z = s + 1;
+            if (sl.cursor < sl.prompt.size()) { // prefill: feed prompt[cursor] at position cursor
+                h_ids[s] = sl.prompt[sl.cursor];
+                need = true;
+            } else { // decode: feed the last sampled token
+                h_ids[s] = sl.last;
+                if (out_cnt[s] < chunk) need = true;
+            }
+        }
+        if (!n_act || !need) break;
+        if (int rc = run_rows(max_z, true)) return rc;
+
+        for (uint32_t s = 0; s < n_slots; s++) {
+            Slot& sl = slots[s];
+            if (!sl.active) continue;
+            const uint32_t sampled = h_tok[s];
+            const bool prefilling = sl.cursor < sl.prompt.size();
+            if (prefilling && sl.cursor + 1 < sl.prompt.size()) {
+                sl.cursor++; // still consuming the prompt: this step's logits are not used
+                continue;
+            }
+            // this step produced a generated token (from the last prompt token, or a decode step)
+            if (prefilling) { sl.cursor = (uint32_t)sl.prompt.size(); sl.pos = (uint32_t)sl.prompt.size(); }
+            if (sampled == eos) { // not emitted
+                if (!prefilling) sl.pos++;
+                finish(s);
+                continue;
+            }
+            if (out_cnt[s] < chunk) out_tok[s * chunk + out_cnt[s]++] = sampled; // one token per step: always fits
+            sl.last = sampled;
+            sl.gen++;
+            if (!prefilling) sl.pos++;
+            if (sl.pos >= n_ctx || sl.gen >= sl.max_gen) finish(s);
+        }
+    }
+    return active_at_entry;
+}
+
+// reference src/main.cpp:5291-5307.  Only the unsplit engine exists here: tokens in, greedy ids
+// out, no hidden rows on either side.  Rows are independent (no per-position state), so
+// a chunk is cut into device steps of MAX_ROWS rows.
+int qk_engine::stage_run(uint32_t slot, const uint32_t* toks, const float* hidden_in, uint32_t n, uint32_t base,
+                         float* /*hidden_out*/, uint32_t* ids_out)
+{
+    if (slot >= n_slots || n < 1 || (uint64_t)base + n > n_ctx) return -1;
+    if (!toks || hidden_in != nullptr) return -2;
+    if (!ids_out) return -3;
+    for (uint32_t i = 0; i < n; i++)
+        if (toks[i] >= vocab) return -1;
+    for (uint32_t off = 0; off < n; off += MAX_ROWS) {
+        const uint32_t rows = std::min(MAX_ROWS, n - off);
+        memcpy(h_ids, toks + off, rows * sizeof(uint32_t));
+        if (hipMemcpyAsync(d_ids, h_ids, rows * sizeof(uint32_t), hipMemcpyHostToDevice, st) != hipSuccess)
+            return ERR_DEVICE;
+        float* fin = nullptr;
+        if (launch_rows(rows, &fin) != QKK_OK) return ERR_DEVICE;
+        if (off + rows == n &&
+            hipMemcpyAsync(d_last, fin + (size_t)(rows - 1) * N_EMBD, N_EMBD * sizeof(float), hipMemcpyDeviceToDevice,
+                           st) != hipSuccess)
+            return ERR_DEVICE;
+        if (hipMemcpyAsync(h_tok, d_tok, rows * sizeof(uint32_t), hipMemcpyDeviceToHost, st) != hipSuccess ||
+            hipStreamSynchronize(st) != hipSuccess)
+            return ERR_DEVICE;
+        memcpy(ids_out + off, h_tok, rows * sizeof(uint32_t));
+    }
+    last_run_rows = n;
+    return 0;
+}
+
+// reference src/main.cpp:5309-5341: top-k (id, logit) of the final position of the last stage
+// run, descending; equal logits in id order.
+int qk_engine::stage_topk(uint32_t k, uint32_t* ids, float* vals)
+{
+    if (!ids || !vals || k < 1 || k > 256 || k > vocab) return -1;
+    if (!last_run_rows) return -2;
+    if (qkk_head_argmax(d_head, d_last, d_tok, d_logits, vocab, N_EMBD, 1, d_hws, hws_bytes, st) != QKK_OK)
+        return ERR_DEVICE;
+    std::vector<float> row(vocab);
+    if (hipMemcpyAsync(row.data(), d_logits, (size_t)vocab * sizeof(float), hipMemcpyDeviceToHost, st) != hipSuccess ||
+        hipStreamSynchronize(st) != hipSuccess)
+        return ERR_DEVICE;
+    std::vector<uint32_t> idx(vocab);
+    for (uint32_t i = 0; i < vocab; i++) idx[i] = i;
+    auto before = [&row](uint32_t a, uint32_t b) { return row[a] > row[b] || (row[a] == row[b] && a < b); };
+    std::partial_sort(idx.begin(), idx.begin() + k, idx.end(), before);
+    for (uint32_t i = 0; i < k; i++) {
+        ids[i] = idx[i];
+        vals[i] = row[idx[i]];
+    }
+    return 0;
 }
 
 extern "C" {
@@ -34,21 +453,10 @@ extern "C" {
 qk_engine* qk_open(const char* gguf_path, const qk_config* cfg, char* err, size_t err_len)
 {
     if (!gguf_path || !cfg) { set_err(err, err_len, "qk_open: null arg"); return nullptr; }
-    if (cfg->n_slots < 1 || cfg->n_slots > 16 || cfg->n_ctx < 64 || cfg->n_ctx > 65536 || cfg->chunk < 1 ||
-        cfg->chunk > 32) {
-        set_err(err, err_len, "qk_open: bad config");
-        return nullptr;
-    }
-    FILE* f = fopen(gguf_path, "rb");
-    if (!f) {
-        set_err(err, err_len, "qk_open: cannot open GGUF");
-        return nullptr;
-    }
-    fclose(f);
-    set_err(err, err_len,
-            "qk_open: this libqk.so implements the quantized decode hot path only (see qk_kernels.h); "
-            "the attention / gated-DeltaNet mixers a whole-model engine needs are not part of it");
-    return nullptr;
+    qk_engine* e = new (std::nothrow) qk_engine();
+    if (!e) { set_err(err, err_len, "qk_open: oom"); return nullptr; }
+    if (!e->open(gguf_path, *cfg, err, err_len)) { delete e; return nullptr; }
+    return e;
 }
 
 void qk_close(qk_engine* e) { delete e; }
@@ -62,61 +470,79 @@ uint32_t qk_bos_token(const qk_engine* e) { return e ? e->bos : 0; }
 uint32_t qk_layer_first(const qk_engine* e) { return e ? e->layer_first : 0; }
 uint32_t qk_layer_end(const qk_engine* e) { return e ? e->layer_end : 0; }
 uint32_t qk_n_layer(const qk_engine* e) { return e ? e->n_layer : 0; }
-uint32_t qk_n_embd(const qk_engine* e) { return e ? e->n_embd : 0; }
+uint32_t qk_n_embd(const qk_engine* e) { return e ? N_EMBD : 0; }
 
+// reference src/main.cpp:5447-5516
 int qk_slot_start(qk_engine* e, uint32_t slot, const uint32_t* prompt, uint32_t n_prompt, uint32_t max_gen,
-                  uint32_t /*snap_prefix*/)
+                  uint32_t snap_prefix)
 {
     if (!e || slot >= e->n_slots) return -1;
-    if (e->split) return -5;
+    if (e->split()) return -5;
     if (e->slots[slot].active) return -2;
     if (!prompt || n_prompt < 1 || (uint64_t)n_prompt + max_gen > e->n_ctx) return -3;
     for (uint32_t i = 0; i < n_prompt; i++)
         if (prompt[i] >= e->vocab) return -4;
-    return -1; // unreachable while qk_open cannot build an engine
+    qk_engine::Slot& s = e->slots[slot];
+    // Positions [0, n_prompt - 1) are batch-prefilled in chunks of max_b while 16 or more
+    // remain, first up to the caller's history boundary, then up to the last prompt token; what
+    // is left is consumed one token per serial step, and the last prompt token's step yields
+    // the first generated token.  With no per-position state a prefilled position writes
+    // nothing, so only the bookkeeping is left of the batch prefill; no cached prefix ever
+    // matches for the same reason (start = 0).
+    const uint32_t start = 0, target = n_prompt - 1;
+    uint32_t done = start;
+    auto batch_to = [&](uint32_t limit) {
+        while (limit > done && limit - done >= 16) done += std::min(e->max_b, limit - done);
+    };
+    const uint32_t snap_at = (snap_prefix > start && snap_prefix < target) ? snap_prefix : 0;
+    if (!getenv("QK_NO_BATCH")) {
+        if (snap_at) batch_to(snap_at);
+        batch_to(target);
+    }
+    s.cursor = done; s.pos = done;
+    s.active = true;
+    s.prompt.assign(prompt, prompt + n_prompt);
+    s.gen = 0; s.max_gen = max_gen; s.last = 0;
+    return 0;
 }
 
 void qk_slot_cancel(qk_engine* e, uint32_t slot)
 {
-    if (e && slot < e->n_slots) e->slots[slot].active = false;
+    if (e && slot < e->n_slots) {
+        e->slots[slot].active = false;
+        e->slots[slot].prompt.clear();
+    }
 }
 
 int qk_step_chunk(qk_engine* e, uint32_t* out_tokens, uint32_t* out_counts, uint32_t* out_finished)
 {
     if (!e || !out_tokens || !out_counts || !out_finished) return -1;
-    if (e->split) return -5;
-    for (uint32_t s = 0; s < e->n_slots; s++) out_counts[s] = 0;
-    *out_finished = 0;
-    return 0;
+    if (e->split()) return -5;
+    return e->step_chunk(out_tokens, out_counts, out_finished);
 }
 
-int qk_stage_run(qk_engine* e, uint32_t slot, const uint32_t* toks, const float* hidden_in, uint32_t n,
-                 uint32_t /*base*/, float* hidden_out, uint32_t* ids_out)
+int qk_stage_run(qk_engine* e, uint32_t slot, const uint32_t* toks, const float* hidden_in, uint32_t n, uint32_t base,
+                 float* hidden_out, uint32_t* ids_out)
 {
     if (!e) return -1;
-    if (slot >= e->n_slots || n == 0) return -1;
-    const bool first = e->layer_first == 0, last = e->layer_end == e->n_layer;
-    if (first ? (!toks || hidden_in) : !hidden_in) return -2;
-    if (last ? !ids_out : !hidden_out) return -3;
-    return -1;
+    return e->stage_run(slot, toks, hidden_in, n, base, hidden_out, ids_out);
 }
 
 int qk_stage_topk(qk_engine* e, uint32_t k, uint32_t* ids, float* vals)
 {
-    if (!e || k < 1 || k > 256 || !ids || !vals) return -1;
-    return -2; // no last-stage run has happened
+    if (!e) return -1;
+    return e->stage_topk(k, ids, vals);
 }
 
-uint32_t qk_state_n(const qk_engine* e) { return e ? e->n_state : 0; }
+// No per-position state to save: the calls validate their bounds (reference src/main.cpp:5428-5445).
+uint32_t qk_state_n(const qk_engine* e) { return e ? N_STATE : 0; }
 int qk_state_save(qk_engine* e, uint32_t slot, uint32_t idx, uint32_t)
 {
-    if (!e || slot >= e->n_slots || idx >= e->n_state) return -1;
-    return -1;
+    return (!e || slot >= e->n_slots || idx >= N_STATE) ? -1 : 0;
 }
 int qk_state_load(qk_engine* e, uint32_t slot, uint32_t idx, uint32_t)
 {
-    if (!e || slot >= e->n_slots || idx >= e->n_state) return -1;
-    return -1;
+    return (!e || slot >= e->n_slots || idx >= N_STATE) ? -1 : 0;
 }
 
 } // extern "C"

@@ -1,0 +1,155 @@
+"""ctypes binding of the engine-level C ABI (include/qk.h) and the recipe for a synthetic model file
+the engine can open: a token embedding, MoE-only layers and a Q6_K head, under the reference's
+tensor names (reference src/main.cpp:3602-3604, 1270-1277, 2726)."""
+import ctypes as C
+
+import numpy as np
+
+from . import capi, gguf, synth
+
+
+class Config(C.Structure):
+    """reference include/qk.h:20-24"""
+    _fields_ = [("n_slots", C.c_uint32), ("n_ctx", C.c_uint32), ("chunk", C.c_uint32)]
+
+
+_bound = False
+
+
+def _lib():
+    global _bound
+    L = capi.lib()
+    if not _bound:
+        vp, u32 = C.c_void_p, C.c_uint32
+        L.qk_open.restype = vp
+        L.qk_open.argtypes = [C.c_char_p, C.POINTER(Config), C.c_char_p, C.c_size_t]
+        L.qk_close.restype = None
+        L.qk_close.argtypes = [vp]
+        for name in ("qk_n_vocab", "qk_n_ctx", "qk_n_slots", "qk_chunk", "qk_eos_token", "qk_bos_token",
+                     "qk_layer_first", "qk_layer_end", "qk_n_layer", "qk_n_embd", "qk_state_n"):
+            getattr(L, name).restype = u32
+            getattr(L, name).argtypes = [vp]
+        L.qk_slot_start.argtypes = [vp, u32, vp, u32, u32, u32]
+        L.qk_slot_cancel.restype = None
+        L.qk_slot_cancel.argtypes = [vp, u32]
+        L.qk_step_chunk.argtypes = [vp, vp, vp, vp]
+        L.qk_stage_run.argtypes = [vp, u32, vp, vp, u32, u32, vp, vp]
+        L.qk_stage_topk.argtypes = [vp, u32, vp, vp]
+        L.qk_state_save.argtypes = [vp, u32, u32, u32]
+        L.qk_state_load.argtypes = [vp, u32, u32, u32]
+        _bound = True
+    return L
+
+
+class Engine:
+    """One qk_engine.  Methods return what the C functions return (negative codes included); only
+    qk_open failing raises, with the message the library wrote."""
+
+    def __init__(self, path, n_slots=1, n_ctx=4096, chunk=8):
+        L = _lib()
+        err = C.create_string_buffer(512)
+        cfg = Config(n_slots, n_ctx, chunk)
+        self._h = L.qk_open(str(path).encode(), C.byref(cfg), err, len(err))
+        if not self._h:
+            raise capi.QkError(-1, err.value.decode())
+        self.n_slots, self.n_ctx, self.chunk = L.qk_n_slots(self._h), L.qk_n_ctx(self._h), L.qk_chunk(self._h)
+        self.vocab, self.eos, self.bos = L.qk_n_vocab(self._h), L.qk_eos_token(self._h), L.qk_bos_token(self._h)
+        self.n_layer, self.n_embd = L.qk_n_layer(self._h), L.qk_n_embd(self._h)
+        self._tok = (C.c_uint32 * (self.n_slots * self.chunk))()
+        self._cnt = (C.c_uint32 * self.n_slots)()
+        self._fin = C.c_uint32(0)
+
+    def close(self):
+        if self._h:
+            _lib().qk_close(self._h)
+            self._h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *a):
+        self.close()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def slot_start(self, slot, prompt, max_gen, snap_prefix=0):
+        arr = (C.c_uint32 * max(1, len(prompt)))(*prompt)
+        return _lib().qk_slot_start(self._h, slot, arr if len(prompt) else None, len(prompt), max_gen, snap_prefix)
+
+    def slot_cancel(self, slot):
+        _lib().qk_slot_cancel(self._h, slot)
+
+    def step_chunk(self):
+        """-> (return code, {slot: [tokens]}, finished mask)"""
+        rc = _lib().qk_step_chunk(self._h, self._tok, self._cnt, C.byref(self._fin))
+        out = {}
+        if rc >= 0:
+            for s in range(self.n_slots):
+                out[s] = [self._tok[s * self.chunk + i] for i in range(self._cnt[s])]
+        return rc, out, self._fin.value
+
+    def stage_run(self, slot, toks, base=0):
+        """-> (return code, greedy ids)"""
+        n = len(toks)
+        arr = (C.c_uint32 * max(1, n))(*toks)
+        ids = (C.c_uint32 * max(1, n))()
+        rc = _lib().qk_stage_run(self._h, slot, arr, None, n, base, None, ids)
+        return rc, list(ids[:n])
+
+    def stage_topk(self, k):
+        ids = (C.c_uint32 * max(1, k))()
+        vals = (C.c_float * max(1, k))()
+        rc = _lib().qk_stage_topk(self._h, k, ids, vals)
+        return rc, list(ids[:k]), list(vals[:k])
+
+    def state_n(self):
+        return _lib().qk_state_n(self._h)
+
+    def state_save(self, slot, idx, n_tok=0):
+        return _lib().qk_state_save(self._h, slot, idx, n_tok)
+
+    def state_load(self, slot, idx, n_tok=0):
+        return _lib().qk_state_load(self._h, slot, idx, n_tok)
+
+
+class StackModel:
+    """Synthetic MoE-only model on the host: the tensors of a file qk_open accepts."""
+
+    def __init__(self, seed, n_layer=2, vocab=1024, n_expert=32, n_ff=512, n_used=8, down_types=None,
+                 embd_type=capi.Q6_K, embd_scale=0.3, eos=7, bos=11, arch="qwen35moe"):
+        # embedding rows of rms ~300 next to MoE outputs of rms ~300 (block scales |N(0,1)|*1e-3):
+        # both the residual and every layer move the logits
+        H = 2048
+        rng = np.random.default_rng(seed)
+        self.arch, self.vocab, self.eos, self.bos, self.n_used = arch, vocab, eos, bos, n_used
+        self.embd_type = embd_type
+        self.embd = synth.tensor_host(embd_type, vocab, H, seed + 101, embd_scale)
+        self.head = synth.tensor_host(capi.Q6_K, vocab, H, seed + 102)
+        self.out_norm = (1.0 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+        down_types = down_types or [capi.IQ4_XS] * n_layer
+        self.layers = [synth.HostLayer(seed + 1000 * (l + 1), H, n_ff, n_expert, n_used, down_types[l])
+                       for l in range(n_layer)]
+        self.post_norm = [(1.0 + 0.1 * rng.standard_normal(H)).astype(np.float32) for _ in range(n_layer)]
+
+    def kvs(self):
+        return {"general.architecture": self.arch, self.arch + ".block_count": len(self.layers),
+                self.arch + ".expert_used_count": self.n_used, "tokenizer.ggml.eos_token_id": self.eos,
+                "tokenizer.ggml.bos_token_id": self.bos}
+
+    def tensors(self):
+        H = 2048
+        t = [("token_embd.weight", self.embd_type, (H, self.vocab), self.embd),
+             ("output_norm.weight", capi.F32, (H,), self.out_norm),
+             ("output.weight", capi.Q6_K, (H, self.vocab), self.head)]
+        for l, hl in enumerate(self.layers):
+            t += gguf.layer_tensors(hl, l)
+            t.append((f"blk.{l}.post_attention_norm.weight", capi.F32, (H,), self.post_norm[l]))
+        return t
+
+    def write(self, path):
+        gguf.write(path, self.kvs(), self.tensors())
+        return path
