@@ -241,6 +241,51 @@ def prefill_moe_workload(qk, n_tokens, steps, warmup, seed=4242):
     return dict(ms_event=ev, distinct_experts=u, bytes_step=L.active_bytes(u) + n_tokens * 2 * H * 4, flops=flops)
 
 
+def engine_workload(qk, n_layer, slots_list, chunks, warm_chunks, seed=31):
+    """Tokens per second through the engine ABI (qk_open / qk_slot_start / qk_step_chunk) on a
+    synthetic MoE-only model file at the full layer shape and vocabulary: host wall clock over
+    whole chunks, host synchronisation after every step included.  Two distinct layers' weights
+    alternate through the file; each layer has its own copy in device memory."""
+    import shutil
+    import tempfile
+    import time
+    model = qk.engine.StackModel(seed, n_layer=2, vocab=151936, n_expert=256, n_ff=512, n_used=8,
+                                 down_types=[qk.IQ4_XS, qk.Q6_K], eos=151935)
+    model.layers = [model.layers[l % 2] for l in range(n_layer)]
+    model.post_norm = [model.post_norm[l % 2] for l in range(n_layer)]
+    tmp = tempfile.mkdtemp(prefix="qk_bench_")
+    res = {}
+    try:
+        path = model.write(os.path.join(tmp, "stack.gguf"))
+        del model
+        for n_slots in slots_list:
+            t0 = time.perf_counter()
+            with qk.engine.Engine(path, n_slots=n_slots, n_ctx=4096, chunk=32) as eng:
+                t_open = time.perf_counter() - t0
+
+                def run(n_chunks):
+                    toks = 0
+                    for _ in range(n_chunks):
+                        for s in range(n_slots):   # a finished slot (EOS or max_gen) takes the next request
+                            eng.slot_start(s, [100 + s], 4000)
+                        rc, out, _ = eng.step_chunk()
+                        if rc < 0:
+                            sys.exit(f"bench.py: qk_step_chunk returned {rc}")
+                        toks += sum(len(v) for v in out.values())
+                    return toks
+                run(warm_chunks)
+                t0 = time.perf_counter()
+                toks = run(chunks)
+                dt = time.perf_counter() - t0
+            res[f"slots_{n_slots}"] = dict(tok_per_s=toks / dt, us_per_step=dt / (chunks * 32) * 1e6, tokens=toks,
+                                           open_s=t_open)
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+    res["config"] = dict(n_layer=n_layer, vocab=151936, chunk=32,
+                         layer="256 experts, IQ3_XXS gate/up, IQ4_XS / Q6_K down alternating, Q8_0 shared")
+    return res
+
+
 def cpu_baseline(qk, orc, budget_s=12.0):
     """The oracle's scalar fused-MoE step (the reference's moeCpuRef restated) on one host
     core, on the same layer shape, a fresh activation row per step."""
@@ -297,6 +342,12 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     steps = max(a.ring, a.steps // a.ring * a.ring)
+    if a.workload == "engine_decode":   # the engine ABI alone (for kernel traces of its graph replays)
+        r = engine_workload(qk, 8, (1, 16), 8, 2)
+        print(json.dumps(dict(metric="engine_decode_tok_per_s", value=r["slots_16"]["tok_per_s"], unit="tok/s", n_gpus=1,
+                              higher_is_better=True, data="synthetic", dtype="f32",
+                              config=dict(workload="engine_decode", **r["config"]), detail=r)), flush=True)
+        return
     if a.workload == "moe_decode_bs1":
         m = moe_workload(qk, 1, qk.IQ4_XS, a.ring, steps, a.warmup)
     elif a.workload == "moe_decode_bs16":
@@ -394,6 +445,9 @@ def main():
                                                 frac=pm["bytes_step"] / (pm["ms_event"] * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                                                 tflops=pm["flops"] / (pm["ms_event"] * 1e-3) / 1e12)
             log(f"[bench] prefill moe: {ex['prefill_moe_128_tokens']}")
+            torch.cuda.empty_cache()
+            ex["engine_decode_8_layers"] = engine_workload(qk, 8, (1, 16), 8, 2)
+            log(f"[bench] engine: {ex['engine_decode_8_layers']}")
         out["extras"] = ex
 
     if a.cpu:

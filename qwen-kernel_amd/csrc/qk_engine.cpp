@@ -87,6 +87,7 @@ struct qk_engine {
     void* dev_alloc(size_t bytes, bool zero);
     int launch_rows(uint32_t rows, float** final_rows);
     int run_rows(uint32_t rows, bool graph_ok);
+    int copy_and_launch(uint32_t rows);
     int step_chunk(uint32_t* out_tok, uint32_t* out_cnt, uint32_t* out_fin);
     int stage_run(uint32_t slot, const uint32_t* toks, const float* hidden_in, uint32_t n, uint32_t base,
                   float* hidden_out, uint32_t* ids_out);
@@ -152,19 +153,26 @@ int qk_engine::launch_rows(uint32_t rows, float** final_rows)
     return qkk_head_argmax(d_head, d_xn[cur], d_tok, nullptr, vocab, N_EMBD, rows, d_hws, hws_bytes, st);
 }
 
-// One device step: h_ids[0..rows) in, h_tok[0..rows) out, host blocked until it is done.
+// One device step: h_ids[0..rows) in, h_tok[0..rows) out, host blocked until it is done.  A
+// captured step holds the two copies as well, so a replay is one launch and one wait.
 int qk_engine::run_rows(uint32_t rows, bool graph_ok)
+{
+    if (graph_ok && rows <= graphs.size() && graphs[rows - 1]) {
+        if (hipGraphLaunch(graphs[rows - 1], st) != hipSuccess) return ERR_DEVICE;
+    } else if (copy_and_launch(rows) != 0) {
+        return ERR_DEVICE;
+    }
+    if (hipStreamSynchronize(st) != hipSuccess) return ERR_DEVICE;
+    return 0;
+}
+
+int qk_engine::copy_and_launch(uint32_t rows)
 {
     if (hipMemcpyAsync(d_ids, h_ids, rows * sizeof(uint32_t), hipMemcpyHostToDevice, st) != hipSuccess)
         return ERR_DEVICE;
-    if (graph_ok && rows <= graphs.size() && graphs[rows - 1]) {
-        if (hipGraphLaunch(graphs[rows - 1], st) != hipSuccess) return ERR_DEVICE;
-    } else if (launch_rows(rows, nullptr) != QKK_OK) {
-        return ERR_DEVICE;
-    }
+    if (launch_rows(rows, nullptr) != QKK_OK) return ERR_DEVICE;
     if (hipMemcpyAsync(h_tok, d_tok, rows * sizeof(uint32_t), hipMemcpyDeviceToHost, st) != hipSuccess)
         return ERR_DEVICE;
-    if (hipStreamSynchronize(st) != hipSuccess) return ERR_DEVICE;
     return 0;
 }
 
@@ -320,9 +328,9 @@ bool qk_engine::open(const char* path, const qk_config& cfg, char* err, size_t e
         hipGraph_t graph = nullptr;
         if (hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal) != hipSuccess)
             return bad("qk_open: graph capture failed");
-        const int rc = launch_rows(z, nullptr);
+        const int rc = copy_and_launch(z);
         const hipError_t ec = hipStreamEndCapture(st, &graph);
-        if (rc != QKK_OK || ec != hipSuccess || !graph) {
+        if (rc != 0 || ec != hipSuccess || !graph) {
             if (graph) (void)hipGraphDestroy(graph);
             return bad("qk_open: graph capture failed");
         }
