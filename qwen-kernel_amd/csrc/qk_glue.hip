@@ -24,13 +24,15 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(const float* a, const 
     __shared__ float s_red[4];
     const size_t base = (size_t)blockIdx.x * n;
     const uint32_t quads = n / 4;
-    float4 v[VPT];
+    float4 v[VPT], g[VPT]; // the norm weights travel with the row: one round trip, not two
     float ss = 0.f;
 #pragma unroll
     for (int j = 0; j < VPT; j++) {
         const uint32_t q = threadIdx.x + 256u * j;
         float4 t = float4{0.f, 0.f, 0.f, 0.f};
+        g[j] = t;
         if (q < quads) {
+            g[j] = *(const float4*)(w + 4 * (size_t)q);
             t = *(const float4*)(a + base + 4 * (size_t)q);
             if (NIN >= 2) {
                 const float4 u = *(const float4*)(b + base + 4 * (size_t)q);
@@ -53,11 +55,9 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(const float* a, const 
 #pragma unroll
     for (int j = 0; j < VPT; j++) {
         const uint32_t q = threadIdx.x + 256u * j;
-        if (q < quads) {
-            const float4 g = *(const float4*)(w + 4 * (size_t)q);
-            *(float4*)(xn + base + 4 * (size_t)q) =
-                float4{v[j].x * scale * g.x, v[j].y * scale * g.y, v[j].z * scale * g.z, v[j].w * scale * g.w};
-        }
+        if (q < quads)
+            *(float4*)(xn + base + 4 * (size_t)q) = float4{v[j].x * scale * g[j].x, v[j].y * scale * g[j].y,
+                                                           v[j].z * scale * g[j].z, v[j].w * scale * g[j].w};
     }
 }
 

@@ -239,8 +239,10 @@ __global__ __launch_bounds__(256) void moe_fold_norm_kernel(MoeWs ws, const qkk_
     __shared__ float s_red[4];
     const uint32_t t = blockIdx.x;
     const float g = sel[t].w_shared;
-    float4 v[2];
+    float4 v[2], gw[2]; // the norm weights are fetched with the row, not after the reduction
     float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < 2; j++) gw[j] = *(const float4*)(w + 4 * (threadIdx.x + 256u * j));
 #pragma unroll
     for (int j = 0; j < 2; j++) {
         const uint32_t o = 4 * (threadIdx.x + 256u * j);
@@ -260,9 +262,8 @@ __global__ __launch_bounds__(256) void moe_fold_norm_kernel(MoeWs ws, const qkk_
 #pragma unroll
     for (int j = 0; j < 2; j++) {
         const uint32_t o = 4 * (threadIdx.x + 256u * j);
-        const float4 gw = *(const float4*)(w + o);
-        *(float4*)(Xn + (size_t)t * d.H + o) =
-            float4{v[j].x * scale * gw.x, v[j].y * scale * gw.y, v[j].z * scale * gw.z, v[j].w * scale * gw.w};
+        *(float4*)(Xn + (size_t)t * d.H + o) = float4{v[j].x * scale * gw[j].x, v[j].y * scale * gw[j].y,
+                                                      v[j].z * scale * gw[j].z, v[j].w * scale * gw[j].w};
     }
 }
 
