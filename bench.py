@@ -130,9 +130,10 @@ def moe_workload(qk, n_slots, down_type, ring, steps, warmup, seed=1234):
                 gateup_bytes=gu_bytes, ring=ring, ring_bytes=ring * L.active_bytes(L.n_expert))
 
 
-def moe_tail_workload(qk, n_slots, down_type, ring, steps, warmup, seed=1234):
+def moe_tail_workload(qk, n_slots, down_type, ring, steps, warmup, seed=1234, layer_row=False):
     """The step with the layer tail behind it (qkk_moe_decode_tail): residual add and the next
-    layer's RMS norm.  Same ring and inputs as moe_workload; returns microseconds per step."""
+    layer's RMS norm.  Same ring and inputs as moe_workload; returns microseconds per step.
+    layer_row: the one-row block with the norm in front instead (qkk_moe_layer_row, in place on R)."""
     import torch
     dev = "cuda:0"
     layers = [qk.synth.device_layer(seed + 16 * i, down_type=down_type, device=dev) for i in range(ring)]
@@ -144,6 +145,10 @@ def moe_tail_workload(qk, n_slots, down_type, ring, steps, warmup, seed=1234):
     S, Xn = torch.empty_like(X), torch.empty_like(X)
     sel = torch.zeros((ring, n_slots, 160), dtype=torch.uint8, device=dev)
     ws = torch.zeros(qk.moe_workspace_bytes(layers[0], n_slots), dtype=torch.uint8, device=dev)
+    if layer_row:
+        _, ev, _ = run_ring([(lambda i=i: qk.moe_layer_row(layers[i], R[i], W[i], ws, sel=sel[i])) for i in range(ring)],
+                            steps, warmup)
+        return ev * 1e3
     _, ev, _ = run_ring([(lambda i=i: qk.moe_decode_tail(layers[i], X[i], R[i], W[i], ws, S=S[i], Xn=Xn[i], sel=sel[i]))
                          for i in range(ring)], steps, warmup)
     return ev * 1e3
@@ -427,6 +432,7 @@ def main():
             # layer glue (add + RMS norm alone, and behind the step in one call)
             ex["add_rmsnorm_2048"] = dict(us_1_row=norm_workload(qk, 1, 640, 64), us_16_rows=norm_workload(qk, 16, 640, 64))
             ex["moe_decode_tail_bs1"] = dict(us=moe_tail_workload(qk, 1, qk.IQ4_XS, 8, 400, 40))
+            ex["moe_layer_row_bs1"] = dict(us=moe_tail_workload(qk, 1, qk.IQ4_XS, 8, 400, 40, layer_row=True))
             torch.cuda.empty_cache()
             ex["moe_decode_tail_bs16_q6k_down"] = dict(us=moe_tail_workload(qk, 16, qk.Q6_K, 4, 200, 20))
             log(f"[bench] glue: {ex['add_rmsnorm_2048']} tail bs1 {ex['moe_decode_tail_bs1']} "

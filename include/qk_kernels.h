@@ -132,6 +132,18 @@ int qkk_moe_decode_tail(const qkk_moe_layer *L_host, const float *X, const float
                         const float *w_next, float eps, float *S, float *Xn, qkk_sel *sel,
                         void *workspace, size_t workspace_bytes, uint32_t n_slots, void *stream);
 
+/* One whole MoE block of a layer for ONE activation row, norm in front and residual behind
+ * (reference src/main.cpp:4376-4402: the norm half of add_rmsnorm.comp, the MoE stages, the sum of
+ * add_rms3.comp), in place on the residual row S:
+ *   xn = S * w_norm / sqrt(mean(S^2) + eps);   S <- S + (routed + shared contribution of xn)
+ * No launch is spent on the norm or the add: every wave of the router and gate/up launches holds the
+ * whole row, so it sums the squares itself, runs its dot products on S * w_norm and scales the
+ * results (the factor is common to a row's sum); the down launch adds the residual to its outputs.
+ * Three launches.  sel, workspace as for qkk_moe_decode with n_slots = 1.  For several rows use
+ * qkk_moe_decode_tail. */
+int qkk_moe_layer_row(const qkk_moe_layer *L_host, float *S, const float *w_norm, float eps, qkk_sel *sel,
+                      void *workspace, size_t workspace_bytes, void *stream);
+
 /* The same step cut at its launch boundaries, for per-stage timing (the reference times its
  * MoE stages separately under QK_STEP_PROF, src/main.cpp:4173-4185, 4591-4632).  `stages` is
  * a mask of QKK_STAGE_*; a stage reads what the earlier stages of a previous call left in

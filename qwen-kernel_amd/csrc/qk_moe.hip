@@ -71,6 +71,93 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     }
 }
 
+// The same launch with the RMS norm in front: x is the un-normalised residual row; the workgroup
+// forms x * nw once, in LDS, and sums the squares (a wave that fetched x and nw for itself made the
+// launch 1.7 us longer: three 8 KB rows per wave through the L1 instead of two); the dot products
+// run on x * nw and their sums are scaled by 1/sqrt(mean(x^2) + eps), which is common to a row's
+// terms.  The task's weights are requested first, so they are in flight while x arrives.
+template <int NCH>
+__global__ __launch_bounds__(256) void moe_route_norm_kernel(const float* __restrict__ gate_inp,
+                                                        const float* __restrict__ gate_inp_shexp,
+                                                        const uint8_t* __restrict__ gate_shexp,
+                                                        const uint8_t* __restrict__ up_shexp,
+                                                        const float* __restrict__ x, MoeWs ws, MoeDims d,
+                                                        const float* __restrict__ nw, float eps)
+{
+    constexpr int P = NCH / 8; // 2048-weight passes per Q8_0 row
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t n_dense = d.E + 1, n_tasks = n_dense + d.F;
+    const uint32_t q8_row = d.H / 32 * Q8_0_BYTES;
+    const uint32_t t = blockIdx.x * 4 + wave;
+
+    // the task's weights first: they are in flight while x arrives
+    const bool dense = t < n_dense, shared = !dense && t < n_tasks;
+    float4 w[NCH];
+    LaneW<QKK_Q8_0> wg[P], wu[P];
+    if (dense) {
+        const float4* row = (const float4*)(t < d.E ? gate_inp + (size_t)t * d.H : gate_inp_shexp);
+#pragma unroll
+        for (int i = 0; i < NCH; i++) w[i] = row[lane + 64 * i];
+    } else if (shared) {
+        const uint32_t r = t - n_dense;
+#pragma unroll
+        for (int p = 0; p < P; p++) {
+            wg[p].load(gate_shexp + (size_t)r * q8_row + (size_t)p * 64 * Q8_0_BYTES, lane);
+            wu[p].load(up_shexp + (size_t)r * q8_row + (size_t)p * 64 * Q8_0_BYTES, lane);
+        }
+    }
+
+    __shared__ __attribute__((aligned(16))) float s_x[256 * NCH];
+    __shared__ float s_red[4];
+    float scale = 1.f;
+    const float* xrow = x;
+    {
+        float4 xv[NCH / 4], nv[NCH / 4];
+#pragma unroll
+        for (int i = 0; i < NCH / 4; i++) xv[i] = ((const float4*)x)[threadIdx.x + 256 * i];
+#pragma unroll
+        for (int i = 0; i < NCH / 4; i++) nv[i] = ((const float4*)nw)[threadIdx.x + 256 * i];
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < NCH / 4; i++) {
+            ss += (xv[i].x * xv[i].x + xv[i].y * xv[i].y) + (xv[i].z * xv[i].z + xv[i].w * xv[i].w);
+            ((float4*)s_x)[threadIdx.x + 256 * i] =
+                float4{xv[i].x * nv[i].x, xv[i].y * nv[i].y, xv[i].z * nv[i].z, xv[i].w * nv[i].w};
+        }
+        scale = 1.f / sqrtf(block_sum4(ss, s_red) / (float)d.H + eps); // its barrier also publishes s_x
+        xrow = s_x;
+    }
+
+    if (dense) {
+        const float4* xv = (const float4*)xrow;
+        float4 xx[NCH];
+#pragma unroll
+        for (int i = 0; i < NCH; i++) xx[i] = xv[lane + 64 * i];
+        float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            a0 += w[i].x * xx[i].x + w[i].y * xx[i].y;
+            a1 += w[i].z * xx[i].z + w[i].w * xx[i].w;
+        }
+        const float s = wave_sum(a0 + a1) * scale;
+        if (lane == 0) ws.logits[t] = s;
+    } else if (shared) {
+        const uint32_t r = t - n_dense;
+        XSlice xs[P];
+#pragma unroll
+        for (int p = 0; p < P; p++) load_xslice<QKK_Q8_0>(xs[p], xrow + p * 2048, lane);
+        float g = 0.f, u = 0.f;
+#pragma unroll
+        for (int p = 0; p < P; p++) {
+            g += wg[p].dot(xs[p], nullptr, nullptr, lane);
+            u += wu[p].dot(xs[p], nullptr, nullptr, lane);
+        }
+        g = wave_sum(g) * scale;
+        u = wave_sum(u) * scale;
+        if (lane == 0) ws.h[(size_t)d.k * d.F + r] = (g / (1.f + expf(-g))) * u;
+    }
+}
+
 // ---- launch 2: select + routed gate/up + SiLU --------------------------------------------
 // Every workgroup picks the top-n_used experts itself from the E logits of launch 1 (one wave,
 // ~1.7 us) instead of waiting for a selector launch: the logits, the activation slice and the
@@ -163,16 +250,126 @@ __global__ __launch_bounds__(256) void moe_gateup_kernel(const uint8_t* __restri
     }
 }
 
+// Launch 2 with the RMS norm in front, as moe_route_norm_kernel: x * nw through LDS, sums scaled.
+template <int TYPE, int PASSES, int RIF>
+__global__ __launch_bounds__(256) void moe_gateup_norm_kernel(const uint8_t* __restrict__ gate_exps,
+                                                         const uint8_t* __restrict__ up_exps,
+                                                         const float* __restrict__ x, MoeWs ws,
+                                                         qkk_sel* __restrict__ sel, MoeDims d,
+                                                         const float* __restrict__ nw, float eps)
+{
+    __shared__ Iq3HalfTables tab;
+    __shared__ float s_log[QKK_MAX_EXPERTS + 8];
+    __shared__ qkk_sel s_sel;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t row_bytes = (uint32_t)qkk_row_bytes_dev<TYPE>(d.H);
+    const uint32_t pass_bytes = row_bytes / PASSES;
+
+    // round trip 1: codebook word, logits (wave 0), activation slice
+    const uint32_t grid_word = g_iq3xxs_grid[threadIdx.x];
+    float lv[QKK_MAX_EXPERTS / 64 + 1];
+    if (wave == 0) {
+#pragma unroll
+        for (int i = 0; i <= (int)(QKK_MAX_EXPERTS / 64); i++)
+            lv[i] = (uint32_t)(lane + 64 * i) <= d.E ? ws.logits[lane + 64 * i] : 0.f;
+    }
+    XSliceH xs[PASSES];
+    __shared__ __attribute__((aligned(16))) float s_x[2048 * PASSES];
+    __shared__ float s_red[4];
+    float scale = 1.f;
+    { // the workgroup forms x * nw once, in LDS, and sums the squares
+        float4 xv[2 * PASSES], nv[2 * PASSES];
+#pragma unroll
+        for (int i = 0; i < 2 * PASSES; i++) xv[i] = ((const float4*)x)[threadIdx.x + 256 * i];
+#pragma unroll
+        for (int i = 0; i < 2 * PASSES; i++) nv[i] = ((const float4*)nw)[threadIdx.x + 256 * i];
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < 2 * PASSES; i++) {
+            ss += (xv[i].x * xv[i].x + xv[i].y * xv[i].y) + (xv[i].z * xv[i].z + xv[i].w * xv[i].w);
+            ((float4*)s_x)[threadIdx.x + 256 * i] =
+                float4{xv[i].x * nv[i].x, xv[i].y * nv[i].y, xv[i].z * nv[i].z, xv[i].w * nv[i].w};
+        }
+        scale = 1.f / sqrtf(block_sum4(ss, s_red) / (float)(2048 * PASSES) + eps); // its barrier publishes s_x
+    }
+#pragma unroll
+    for (int p = 0; p < PASSES; p++) {
+        XSlice f;
+        load_xslice<TYPE>(f, s_x + p * 2048, lane);
+        split_xslice(xs[p], f);
+    }
+
+    fill_iq3_half_entry(tab, threadIdx.x, grid_word);
+    if (wave == 0) {
+#pragma unroll
+        for (int i = 0; i <= (int)(QKK_MAX_EXPERTS / 64); i++)
+            if ((uint32_t)(lane + 64 * i) <= d.E) s_log[lane + 64 * i] = lv[i];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        select_wave(s_log, d.E, d.k, &s_sel);
+        if (lane == 0) s_sel.w_shared = 1.f / (1.f + expf(-s_log[d.E]));
+    }
+    __syncthreads();
+    if (blockIdx.x == 0 && threadIdx.x < 33) {
+        if (threadIdx.x < 16) {
+            if (threadIdx.x < d.k) {
+                sel->ids[threadIdx.x] = s_sel.ids[threadIdx.x];
+                sel->w[threadIdx.x] = s_sel.w[threadIdx.x];
+            }
+        } else if (threadIdx.x == 32) {
+            sel->w_shared = s_sel.w_shared;
+        }
+    }
+
+    const uint32_t groups = (d.F + RIF - 1) / RIF; // row groups per pick
+    for (uint32_t t = blockIdx.x * 4 + wave; t < d.k * groups; t += gridDim.x * 4) {
+        const uint32_t s = t / groups, r0 = (t % groups) * RIF;
+        const uint32_t e = min(s_sel.ids[s], d.E - 1);
+        const uint8_t* gbase = gate_exps + ((size_t)e * d.F) * row_bytes;
+        const uint8_t* ubase = up_exps + ((size_t)e * d.F) * row_bytes;
+        LaneW<TYPE> wg[RIF][PASSES], wu[RIF][PASSES];
+#pragma unroll
+        for (int i = 0; i < RIF; i++) {
+            const uint32_t r = min(r0 + i, d.F - 1);
+#pragma unroll
+            for (int p = 0; p < PASSES; p++) {
+                wg[i][p].load(gbase + (size_t)r * row_bytes + (size_t)p * pass_bytes, lane);
+                wu[i][p].load(ubase + (size_t)r * row_bytes + (size_t)p * pass_bytes, lane);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < RIF; i++) {
+            float g = 0.f, u = 0.f;
+#pragma unroll
+            for (int p = 0; p < PASSES; p++) {
+                g += wg[i][p].dot_h(xs[p], &tab);
+                u += wu[i][p].dot_h(xs[p], &tab);
+            }
+            g = wave_sum(g) * scale;
+            u = wave_sum(u) * scale;
+            if (lane == 0 && r0 + i < d.F) ws.h[(size_t)s * d.F + r0 + i] = (g / (1.f + expf(-g))) * u;
+        }
+    }
+}
+
 // ---- launch 3: routed down + shared down + combine ---------------------------------------
 // Wave task = RIF consecutive outputs o.  F = 32*LPR: LPR lanes cover one down row, so
 // 64/LPR picks are processed side by side; the shared Q8_0 row rides on lane group 0.
 // Round trip 1 fetches everything that does not depend on the picks (router record, h slices,
 // shared rows, codebook); round trip 2 the picked experts' rows.
-template <int TYPE, int LPR, int ROUNDS, int RIF>
+template <bool ON>
+struct ResidArg {
+    const float* p;
+};
+template <>
+struct ResidArg<false> {};
+
+// RESID: y = resid + step (the residual row may be y: an element is read and written by the same lane).
+template <int TYPE, int LPR, int ROUNDS, int RIF, bool RESID>
 __global__ __launch_bounds__(256) void moe_down_kernel(const uint8_t* __restrict__ down_exps,
                                                        const uint8_t* __restrict__ down_shexp,
                                                        MoeWs ws, const qkk_sel* __restrict__ sel,
-                                                       float* __restrict__ y, MoeDims d)
+                                                       float* y, MoeDims d, ResidArg<RESID> ra)
 {
     extern __shared__ __attribute__((aligned(16))) float s_h[]; // [(k+1)][F]: the gated activations of every pick
     __shared__ IqTables tab;
@@ -196,6 +393,12 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const uint8_t* __restrict
         wt[q] = sel->w[sc];
     }
     float wsh = sel->w_shared;
+    float res[RIF];
+#pragma unroll
+    for (int i = 0; i < RIF; i++) {
+        if constexpr (RESID) res[i] = ra.p[min(o0 + i, d.H - 1)];
+        else res[i] = 0.f;
+    }
     const uint32_t h_quads = (d.k + 1) * d.F / 4;
     constexpr int HQ = 8; // quads per thread in flight: covers (16 + 1) * 1024 / 4 / 256 = 17 in three rounds
     const float4* hg = (const float4*)ws.h;
@@ -245,6 +448,7 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const uint8_t* __restrict
 #pragma unroll
         for (int q = 0; q < ROUNDS; q++) acc += wt[q] * w[i][q].dot(hs[q], hsum[q], &tab, lir);
         acc = wave_sum(acc);
+        if constexpr (RESID) acc += res[i];
         if (lane == 0 && o0 + i < d.H) y[o0 + i] = acc;
     }
 }
@@ -285,15 +489,24 @@ static int check_layer(const qkk_moe_layer* L, const char* who)
 
 template <int TYPE, int LPR, int ROUNDS, int RIF>
 static void launch_down2(const qkk_moe_layer* L, const MoeWs& ws, const qkk_sel* sel, float* Y,
-                         const MoeDims& d, uint32_t n_slots, hipStream_t st)
+                         const MoeDims& d, const float* resid, hipStream_t st)
 {
     const uint32_t waves = (d.H + RIF - 1) / RIF;
     const uint32_t lds = (d.k + 1) * d.F * 4; // h in LDS (at most 17 * 1024 floats = 68 KB)
-    static bool raised = ((void)hipFuncSetAttribute((const void*)moe_down_kernel<TYPE, LPR, ROUNDS, RIF>,
+    static bool raised = ((void)hipFuncSetAttribute((const void*)moe_down_kernel<TYPE, LPR, ROUNDS, RIF, false>,
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, 17 * 1024 * 4),
+                          (void)hipFuncSetAttribute((const void*)moe_down_kernel<TYPE, LPR, ROUNDS, RIF, true>,
                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 17 * 1024 * 4), true);
     (void)raised;
-    hipLaunchKernelGGL((moe_down_kernel<TYPE, LPR, ROUNDS, RIF>), dim3((waves + 3) / 4), dim3(256), lds, st,
-                       (const uint8_t*)L->down_exps, (const uint8_t*)L->down_shexp, ws, sel, Y, d);
+    const dim3 grid((waves + 3) / 4), block(256);
+    if (resid)
+        hipLaunchKernelGGL((moe_down_kernel<TYPE, LPR, ROUNDS, RIF, true>), grid, block, lds, st,
+                           (const uint8_t*)L->down_exps, (const uint8_t*)L->down_shexp, ws, sel, Y, d,
+                           ResidArg<true>{resid});
+    else
+        hipLaunchKernelGGL((moe_down_kernel<TYPE, LPR, ROUNDS, RIF, false>), grid, block, lds, st,
+                           (const uint8_t*)L->down_exps, (const uint8_t*)L->down_shexp, ws, sel, Y, d,
+                           ResidArg<false>{});
 }
 
 // Picks processed side by side = 64/LPR; ROUNDS covers n_used with the fewest passes and
@@ -302,22 +515,63 @@ static void launch_down2(const qkk_moe_layer* L, const MoeWs& ws, const qkk_sel*
 // four outputs per wave, which leaves half the CUs without work.
 template <int TYPE, int LPR>
 static void launch_down(const qkk_moe_layer* L, const MoeWs& ws, const qkk_sel* sel, float* Y,
-                        const MoeDims& d, uint32_t n_slots, hipStream_t st)
+                        const MoeDims& d, const float* resid, hipStream_t st)
 {
     const uint32_t need = (d.k + 64 / LPR - 1) / (64 / LPR);
-    if (need <= 1) launch_down2<TYPE, LPR, 1, 4>(L, ws, sel, Y, d, n_slots, st);
-    else if (need <= 2) launch_down2<TYPE, LPR, 2, 2>(L, ws, sel, Y, d, n_slots, st); // 256 workgroups at n_embd 2048
-    else if (need <= 4) launch_down2<TYPE, LPR, 4, 2>(L, ws, sel, Y, d, n_slots, st);
-    else launch_down2<TYPE, LPR, 8, 1>(L, ws, sel, Y, d, n_slots, st);
+    if (need <= 1) launch_down2<TYPE, LPR, 1, 4>(L, ws, sel, Y, d, resid, st);
+    else if (need <= 2) launch_down2<TYPE, LPR, 2, 2>(L, ws, sel, Y, d, resid, st); // 256 workgroups at n_embd 2048
+    else if (need <= 4) launch_down2<TYPE, LPR, 4, 2>(L, ws, sel, Y, d, resid, st);
+    else launch_down2<TYPE, LPR, 8, 1>(L, ws, sel, Y, d, resid, st);
 }
 
 template <int TYPE>
 static void launch_down(const qkk_moe_layer* L, const MoeWs& ws, const qkk_sel* sel, float* Y,
-                        const MoeDims& d, uint32_t n_slots, hipStream_t st)
+                        const MoeDims& d, const float* resid, hipStream_t st)
 {
-    if (d.F == 512) launch_down<TYPE, 16>(L, ws, sel, Y, d, n_slots, st);
-    else if (d.F == 256) launch_down<TYPE, 8>(L, ws, sel, Y, d, n_slots, st);
-    else launch_down<TYPE, 32>(L, ws, sel, Y, d, n_slots, st);
+    if (d.F == 512) launch_down<TYPE, 16>(L, ws, sel, Y, d, resid, st);
+    else if (d.F == 256) launch_down<TYPE, 8>(L, ws, sel, Y, d, resid, st);
+    else launch_down<TYPE, 32>(L, ws, sel, Y, d, resid, st);
+}
+
+// One row with the RMS norm in front (weights w) and the residual behind: see qkk_moe_layer_row.
+struct MoeNorm {
+    const float* w;
+    float eps;
+};
+
+// Launches 1 and 2; norm given: the variants with the RMS norm in front.
+static void launch_route_gateup(const qkk_moe_layer* L, const float* X, const MoeWs& ws, qkk_sel* sel, const MoeDims& d,
+                                uint32_t stages, const MoeNorm* norm, hipStream_t st)
+{
+    const uint8_t *gs = (const uint8_t*)L->gate_shexp, *us = (const uint8_t*)L->up_shexp;
+    const uint8_t *ge = (const uint8_t*)L->gate_exps, *ue = (const uint8_t*)L->up_exps;
+    if (stages & QKK_STAGE_ROUTE) {
+        const dim3 grid((d.E + 1 + d.F + 3) / 4), block(256);
+        if (d.H == 2048 && !norm)
+            hipLaunchKernelGGL(moe_route_kernel<8>, grid, block, 0, st, L->gate_inp, L->gate_inp_shexp, gs, us, X, ws, d);
+        else if (!norm)
+            hipLaunchKernelGGL(moe_route_kernel<16>, grid, block, 0, st, L->gate_inp, L->gate_inp_shexp, gs, us, X, ws, d);
+        else if (d.H == 2048)
+            hipLaunchKernelGGL(moe_route_norm_kernel<8>, grid, block, 0, st, L->gate_inp, L->gate_inp_shexp, gs, us, X, ws,
+                               d, norm->w, norm->eps);
+        else
+            hipLaunchKernelGGL(moe_route_norm_kernel<16>, grid, block, 0, st, L->gate_inp, L->gate_inp_shexp, gs, us, X, ws,
+                               d, norm->w, norm->eps);
+    }
+    if (stages & QKK_STAGE_GATEUP) {
+        constexpr int GU_RIF = 4;
+        const dim3 g1((d.k * ((d.F + GU_RIF - 1) / GU_RIF) + 3) / 4), g2((d.k * ((d.F + 1) / 2) + 3) / 4), block(256);
+        if (d.H == 2048 && !norm)
+            hipLaunchKernelGGL((moe_gateup_kernel<QKK_IQ3_XXS, 1, GU_RIF>), g1, block, 0, st, ge, ue, X, ws, sel, d);
+        else if (!norm)
+            hipLaunchKernelGGL((moe_gateup_kernel<QKK_IQ3_XXS, 2, 2>), g2, block, 0, st, ge, ue, X, ws, sel, d);
+        else if (d.H == 2048)
+            hipLaunchKernelGGL((moe_gateup_norm_kernel<QKK_IQ3_XXS, 1, GU_RIF>), g1, block, 0, st, ge, ue, X, ws, sel, d,
+                               norm->w, norm->eps);
+        else
+            hipLaunchKernelGGL((moe_gateup_norm_kernel<QKK_IQ3_XXS, 2, 2>), g2, block, 0, st, ge, ue, X, ws, sel, d,
+                               norm->w, norm->eps);
+    }
 }
 
 extern "C" {
@@ -331,7 +585,7 @@ size_t qkk_moe_workspace_bytes(const qkk_moe_layer* L, uint32_t n_slots)
 
 static int moe_decode_impl(const char* who, const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* sel,
                            void* workspace, size_t workspace_bytes, uint32_t n_slots, uint32_t stages,
-                           void* stream, const MoeTail* tail = nullptr)
+                           void* stream, const MoeTail* tail = nullptr, const MoeNorm* norm = nullptr)
 {
     if (int rc = check_layer(L, who)) return rc;
     if (!X || !Y || !sel || !workspace) return fail(QKK_EINVAL, "%s: null pointer", who);
@@ -346,32 +600,11 @@ static int moe_decode_impl(const char* who, const qkk_moe_layer* L, const float*
     if (n_slots >= 2) return moe_grouped_launch(L, X, Y, sel, workspace, n_slots, stages, st, tail);
     const MoeWs ws = ws_carve(workspace, d, n_slots);
 
-    if (stages & QKK_STAGE_ROUTE) {
-        const uint32_t t1 = d.E + 1 + d.F;
-        if (d.H == 2048)
-            hipLaunchKernelGGL(moe_route_kernel<8>, dim3((t1 + 3) / 4), dim3(256), 0, st, L->gate_inp,
-                               L->gate_inp_shexp, (const uint8_t*)L->gate_shexp, (const uint8_t*)L->up_shexp,
-                               X, ws, d);
-        else
-            hipLaunchKernelGGL(moe_route_kernel<16>, dim3((t1 + 3) / 4), dim3(256), 0, st, L->gate_inp,
-                               L->gate_inp_shexp, (const uint8_t*)L->gate_shexp, (const uint8_t*)L->up_shexp,
-                               X, ws, d);
-    }
-    if (stages & QKK_STAGE_GATEUP) {
-        constexpr int GU_RIF = 4;
-        const uint32_t t2 = d.k * ((d.F + GU_RIF - 1) / GU_RIF);
-        if (d.H == 2048)
-            hipLaunchKernelGGL((moe_gateup_kernel<QKK_IQ3_XXS, 1, GU_RIF>), dim3((t2 + 3) / 4),
-                               dim3(256), 0, st, (const uint8_t*)L->gate_exps, (const uint8_t*)L->up_exps, X,
-                               ws, sel, d);
-        else
-            hipLaunchKernelGGL((moe_gateup_kernel<QKK_IQ3_XXS, 2, 2>),
-                               dim3((d.k * ((d.F + 1) / 2) + 3) / 4), dim3(256), 0, st,
-                               (const uint8_t*)L->gate_exps, (const uint8_t*)L->up_exps, X, ws, sel, d);
-    }
+    launch_route_gateup(L, X, ws, sel, d, stages, norm, st);
     if (stages & QKK_STAGE_DOWN) {
-        if (L->down_type == QKK_IQ4_XS) launch_down<QKK_IQ4_XS>(L, ws, sel, Y, d, n_slots, st);
-        else launch_down<QKK_Q6_K>(L, ws, sel, Y, d, n_slots, st);
+        const float* resid = norm ? X : nullptr; // norm in front: the input row is the residual, Y may be X
+        if (L->down_type == QKK_IQ4_XS) launch_down<QKK_IQ4_XS>(L, ws, sel, Y, d, resid, st);
+        else launch_down<QKK_Q6_K>(L, ws, sel, Y, d, resid, st);
         // one row: the step's output went to tail->Xn (see qkk_moe_decode_tail); add and norm in place
         if (tail) launch_add_rmsnorm(tail->resid, Y, tail->w_next, tail->S, tail->Xn, d.H, 1, tail->eps, st);
     }
@@ -399,6 +632,17 @@ int qkk_moe_decode_tail(const qkk_moe_layer* L, const float* X, const float* res
     // the step writes its output row(s) to Xn when it has to materialise them (one row)
     return moe_decode_impl("qkk_moe_decode_tail", L, X, Xn, sel, workspace, workspace_bytes, n_slots, QKK_STAGE_ALL, stream,
                            &tail);
+}
+
+int qkk_moe_layer_row(const qkk_moe_layer* L, float* S, const float* w_norm, float eps, qkk_sel* sel, void* workspace,
+                      size_t workspace_bytes, void* stream)
+{
+    if (!w_norm) return fail(QKK_EINVAL, "qkk_moe_layer_row: null pointer");
+    if (!aligned16(w_norm)) return fail(QKK_EINVAL, "qkk_moe_layer_row: w_norm must be 16-byte aligned");
+    if (!(eps >= 0.f)) return fail(QKK_EINVAL, "qkk_moe_layer_row: eps must be non-negative");
+    const MoeNorm norm{w_norm, eps};
+    return moe_decode_impl("qkk_moe_layer_row", L, S, S, sel, workspace, workspace_bytes, 1, QKK_STAGE_ALL, stream,
+                           nullptr, &norm);
 }
 
 int qkk_moe_decode_stages(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* sel, void* workspace,

@@ -45,9 +45,14 @@ def world(qk, dev, tmp_path_factory):
     def step(ids, want_logits=False):   # one device step over len(ids) rows, as the engine chains it
         t = torch.tensor(ids, dtype=torch.int32, device=dev)
         x = qk.embed(model.embd_type, embd, VOCAB, H, t, len(ids))
-        xn = qk.rmsnorm(x, pnorm[0])
-        for l, L in enumerate(layers):
-            x, xn, _ = qk.moe_decode_tail(L, xn, x, pnorm[l + 1] if l + 1 < len(layers) else onorm, ws, S=x)
+        if len(ids) == 1:   # one row: the norm rides inside each layer's launches
+            for l, L in enumerate(layers):
+                qk.moe_layer_row(L, x, pnorm[l], ws)
+            xn = qk.rmsnorm(x, onorm)
+        else:
+            xn = qk.rmsnorm(x, pnorm[0])
+            for l, L in enumerate(layers):
+                x, xn, _ = qk.moe_decode_tail(L, xn, x, pnorm[l + 1] if l + 1 < len(layers) else onorm, ws, S=x)
         tok, logits = qk.head_argmax(head, xn, VOCAB, H, hws, want_logits=want_logits)
         torch.cuda.synchronize()
         return (tok.cpu().tolist(), logits.cpu().numpy()) if want_logits else tok.cpu().tolist()

@@ -311,6 +311,50 @@ def test_moe_decode_tail(qk, orc, dev, layer_iq4, n):
         qk.moe_decode_tail(layer, Xd, Rd, Wd, ws, Xn=Xd)
 
 
+@pytest.mark.parametrize("which", ["iq4", "q6k"])
+def test_moe_layer_row(qk, orc, dev, layer_iq4, layer_q6k, which):
+    """One row's whole MoE block in place -- norm inside the router and gate/up launches, residual
+    added by the down launch -- against the oracle's norm, step and sum
+    (reference src/main.cpp:4376-4402)."""
+    import torch
+    hl = layer_iq4 if which == "iq4" else layer_q6k
+    print(f"[case] moe layer row, down {which}", flush=True)
+    layer = hl.to_device(dev)
+    ws = torch.zeros(qk.moe_workspace_bytes(layer, 1), dtype=torch.uint8, device=dev)
+    rng = np.random.default_rng(17)
+    w = rng.uniform(0.5, 1.5, 2048).astype(np.float32)
+    Wd = torch.from_numpy(w).to(dev)
+    done = 0
+    for trial in range(40):
+        # a residual row far from unit scale: the norm, not the input, must bring it to O(1)
+        s0 = (rng.standard_normal(2048) * rng.choice([0.03, 1.0, 40.0])).astype(np.float32)
+        xn = orc.add_rms(s0, w, 1e-6)
+        r = orc.moe_ref(hl, xn)
+        lw = np.log(np.array(sorted(r["sel"].w[:8], reverse=True)))
+        if r["sel"].gap <= 2e-3 or np.min(-np.diff(lw)) <= 2e-3:
+            continue
+        Sd = torch.from_numpy(s0).to(dev).reshape(1, 2048)
+        S, sel = qk.moe_layer_row(layer, Sd, Wd, ws)
+        torch.cuda.synchronize()
+        assert S.data_ptr() == Sd.data_ptr()
+        ids, wts, wsh = sel_fields(sel)
+        assert list(ids[0, :8]) == list(r["sel"].ids[:8])
+        assert np.max(np.abs(wts[0, :8] - np.array(r["sel"].w[:8]))) <= 1e-4
+        got = S.cpu().numpy()[0]
+        assert np.max(np.abs((got - s0) - r["y"])) <= TOL * np.max(np.abs(r["y"])) + 2e-7 * np.max(np.abs(s0))
+        # the same bits as the plain step on the normalised row plus the residual, up to the
+        # place where the scale is applied (after the dot products instead of before)
+        Y, _ = qk.moe_decode(layer, torch.from_numpy(xn).to(dev).reshape(1, 2048), ws)
+        torch.cuda.synchronize()
+        assert orc.rel_maxabs_err(got - s0, Y.cpu().numpy()[0]) <= 1e-4
+        done += 1
+        if done == 4:
+            break
+    assert done == 4
+    with pytest.raises(qk.QkError):
+        qk.moe_layer_row(layer, Sd, None, ws)
+
+
 def test_group_pairs_matches_oracle(qk, orc, dev):
     import torch
     print("[case] group pairs", flush=True)
