@@ -353,6 +353,15 @@ def main():
                               higher_is_better=True, data="synthetic", dtype="f32",
                               config=dict(workload="engine_decode", **r["config"]), detail=r)), flush=True)
         return
+    if a.workload in ("head_bs1", "head_bs16"):   # the LM head alone (for counter runs on its kernel)
+        b = 1 if a.workload == "head_bs1" else 16
+        h = head_workload(qk, 151936, 2048, b, min(a.steps, 40), min(a.warmup, 8))
+        gb = h["bytes_step"] / (h["ms_event"] * 1e-3) / 1e9
+        print(json.dumps(dict(metric="lm_head_argmax_hbm_gbps", value=gb, unit="GB/s", n_gpus=1, steps=h["steps"],
+                              ms_per_step=h["ms_event"], higher_is_better=True, data="synthetic", dtype="f32",
+                              config=dict(workload=a.workload, vocab=151936, n_embd=2048, weights="Q6_K", rows=b),
+                              bytes_per_step=h["bytes_step"], frac_of_hbm_peak=gb / HBM_PEAK_GBPS)), flush=True)
+        return
     if a.workload == "moe_decode_bs1":
         m = moe_workload(qk, 1, qk.IQ4_XS, a.ring, steps, a.warmup)
     elif a.workload == "moe_decode_bs16":
