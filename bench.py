@@ -133,7 +133,7 @@ def moe_workload(qk, n_slots, down_type, ring, steps, warmup, seed=1234):
 def moe_tail_workload(qk, n_slots, down_type, ring, steps, warmup, seed=1234, layer_row=False):
     """The step with the layer tail behind it (qkk_moe_decode_tail): residual add and the next
     layer's RMS norm.  Same ring and inputs as moe_workload; returns microseconds per step.
-    layer_row: the one-row block with the norm in front instead (qkk_moe_layer_row, in place on R)."""
+    layer_row: the one-row block with the norm in front instead (qkk_moe_layer_rows, in place on R)."""
     import torch
     dev = "cuda:0"
     layers = [qk.synth.device_layer(seed + 16 * i, down_type=down_type, device=dev) for i in range(ring)]
@@ -146,7 +146,7 @@ def moe_tail_workload(qk, n_slots, down_type, ring, steps, warmup, seed=1234, la
     sel = torch.zeros((ring, n_slots, 160), dtype=torch.uint8, device=dev)
     ws = torch.zeros(qk.moe_workspace_bytes(layers[0], n_slots), dtype=torch.uint8, device=dev)
     if layer_row:
-        _, ev, _ = run_ring([(lambda i=i: qk.moe_layer_row(layers[i], R[i], W[i], ws, sel=sel[i])) for i in range(ring)],
+        _, ev, _ = run_ring([(lambda i=i: qk.moe_layer_rows(layers[i], R[i], W[i], ws, sel=sel[i])) for i in range(ring)],
                             steps, warmup)
         return ev * 1e3
     _, ev, _ = run_ring([(lambda i=i: qk.moe_decode_tail(layers[i], X[i], R[i], W[i], ws, S=S[i], Xn=Xn[i], sel=sel[i]))

@@ -116,8 +116,8 @@ size_t qkk_moe_workspace_bytes(const qkk_moe_layer *L_host, uint32_t n_slots);
  *                                  time.  A workspace that breaks this gives wrong results,
  *                                  never an access outside the tensors: the kernels clamp
  *                                  every index they take from it.
- * With n_slots >= 2 every picked expert's weights are read once per 16 rows that picked it
- * (matrix-core path); that path needs n_embd = 2048 and returns QKK_ESHAPE otherwise. */
+ * With n_slots > QKK_ROWWISE_MAX every picked expert's weights are read once per 16 rows that picked
+ * it (matrix-core path); that path needs n_embd = 2048 and returns QKK_ESHAPE otherwise. */
 int qkk_moe_decode(const qkk_moe_layer *L_host, const float *X, float *Y, qkk_sel *sel,
                    void *workspace, size_t workspace_bytes, uint32_t n_slots, void *stream);
 
@@ -132,17 +132,22 @@ int qkk_moe_decode_tail(const qkk_moe_layer *L_host, const float *X, const float
                         const float *w_next, float eps, float *S, float *Xn, qkk_sel *sel,
                         void *workspace, size_t workspace_bytes, uint32_t n_slots, void *stream);
 
-/* One whole MoE block of a layer for ONE activation row, norm in front and residual behind
- * (reference src/main.cpp:4376-4402: the norm half of add_rmsnorm.comp, the MoE stages, the sum of
- * add_rms3.comp), in place on the residual row S:
+/* Rows up to which qkk_moe_decode / qkk_moe_decode_tail run every row through the one-row launches
+ * (a few rows hardly ever pick the same expert, so there is little to share, and a row's result is
+ * then bit for bit what it is alone); more rows take the expert-major path. */
+#define QKK_ROWWISE_MAX 10u
+
+/* One whole MoE block of a layer for n_slots <= QKK_ROWWISE_MAX activation rows, norm in front and
+ * residual behind (reference src/main.cpp:4376-4402: the norm half of add_rmsnorm.comp, the MoE
+ * stages, the sum of add_rms3.comp), in place on the residual rows S [n_slots][n_embd]:
  *   xn = S * w_norm / sqrt(mean(S^2) + eps);   S <- S + (routed + shared contribution of xn)
- * No launch is spent on the norm or the add: every wave of the router and gate/up launches holds the
- * whole row, so it sums the squares itself, runs its dot products on S * w_norm and scales the
- * results (the factor is common to a row's sum); the down launch adds the residual to its outputs.
- * Three launches.  sel, workspace as for qkk_moe_decode with n_slots = 1.  For several rows use
+ * No launch is spent on the norm or the add: a dot product against xn is 1/rms(S) times the dot
+ * product against S * w_norm, so the router and gate/up launches form S * w_norm once per workgroup
+ * while summing the squares and scale their sums; the down launch adds the residual to its outputs.
+ * Three launches.  sel, workspace as for qkk_moe_decode.  More rows: QKK_ESHAPE, use
  * qkk_moe_decode_tail. */
-int qkk_moe_layer_row(const qkk_moe_layer *L_host, float *S, const float *w_norm, float eps, qkk_sel *sel,
-                      void *workspace, size_t workspace_bytes, void *stream);
+int qkk_moe_layer_rows(const qkk_moe_layer *L_host, float *S, const float *w_norm, float eps, qkk_sel *sel,
+                       void *workspace, size_t workspace_bytes, uint32_t n_slots, void *stream);
 
 /* The same step cut at its launch boundaries, for per-stage timing (the reference times its
  * MoE stages separately under QK_STEP_PROF, src/main.cpp:4173-4185, 4591-4632).  `stages` is

@@ -10,7 +10,7 @@ from .capi import (  # noqa: F401
     F32, F16, Q8_0, Q6_K, IQ3_XXS, IQ4_XS, QkError, QkSel, MoeLayer, lib, lib_path, row_bytes,
     dequant, gemv, moe_decode, moe_workspace_bytes, head_argmax, head_workspace_bytes, argmax,
     moe_group_pairs, gemm_q8_0, moe_prefill, moe_prefill_workspace_bytes, device_info,
-    rmsnorm, add_rmsnorm, add_rms3, vec_add, embed, moe_decode_tail, moe_layer_row,
+    rmsnorm, add_rmsnorm, add_rms3, vec_add, embed, moe_decode_tail, moe_layer_rows, ROWWISE_MAX,
 )
 from . import synth  # noqa: F401
 from . import gguf  # noqa: F401

@@ -140,14 +140,15 @@ int qk_engine::launch_rows(uint32_t rows, float** final_rows)
 {
     if (rows < 1 || rows > MAX_ROWS) return QKK_ESHAPE;
     if (int rc = qkk_embed(embd_type, d_embd, embd_rows, N_EMBD, d_ids, MAX_ROWS, 0, 1, d_x, rows, st)) return rc;
-    if (rows == 1) {
-        // one row: each layer's norm runs inside its MoE launches and the residual is added by the
-        // last of them -- three launches per layer, then the output norm and the head
+    if (rows <= QKK_ROWWISE_MAX) {
+        // few rows: each layer's norm runs inside its MoE launches and the residual is added by the
+        // last of them -- three launches per layer, then the output norm and the head.  Every row
+        // goes through the one-row kernels, so a slot's tokens do not depend on its company.
         for (const EngineLayer& L : layers)
-            if (int rc = qkk_moe_layer_row(&L.moe, d_x, L.post_norm, eps, d_sel, d_ws, ws_bytes, st)) return rc;
-        if (int rc = qkk_rmsnorm(d_x, d_onorm, d_xn[0], N_EMBD, 1, eps, st)) return rc;
+            if (int rc = qkk_moe_layer_rows(&L.moe, d_x, L.post_norm, eps, d_sel, d_ws, ws_bytes, rows, st)) return rc;
+        if (int rc = qkk_rmsnorm(d_x, d_onorm, d_xn[0], N_EMBD, rows, eps, st)) return rc;
         if (final_rows) *final_rows = d_xn[0];
-        return qkk_head_argmax(d_head, d_xn[0], d_tok, nullptr, vocab, N_EMBD, 1, d_hws, hws_bytes, st);
+        return qkk_head_argmax(d_head, d_xn[0], d_tok, nullptr, vocab, N_EMBD, rows, d_hws, hws_bytes, st);
     }
     if (int rc = qkk_rmsnorm(d_x, layers[0].post_norm, d_xn[0], N_EMBD, rows, eps, st)) return rc;
     int cur = 0;

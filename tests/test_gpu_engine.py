@@ -45,9 +45,9 @@ def world(qk, dev, tmp_path_factory):
     def step(ids, want_logits=False):   # one device step over len(ids) rows, as the engine chains it
         t = torch.tensor(ids, dtype=torch.int32, device=dev)
         x = qk.embed(model.embd_type, embd, VOCAB, H, t, len(ids))
-        if len(ids) == 1:   # one row: the norm rides inside each layer's launches
+        if len(ids) <= qk.ROWWISE_MAX:   # few rows: the norm rides inside each layer's launches
             for l, L in enumerate(layers):
-                qk.moe_layer_row(L, x, pnorm[l], ws)
+                qk.moe_layer_rows(L, x, pnorm[l], ws)
             xn = qk.rmsnorm(x, onorm)
         else:
             xn = qk.rmsnorm(x, pnorm[0])
@@ -58,22 +58,29 @@ def world(qk, dev, tmp_path_factory):
         return (tok.cpu().tolist(), logits.cpu().numpy()) if want_logits else tok.cpu().tolist()
 
     print("[engine] next-token maps", flush=True)
-    nxt1 = [step([t])[0] for t in range(VOCAB)]                      # the one-row kernels
-    nxtn = sum((step(list(range(t, t + 16))) for t in range(0, VOCAB, 16)), [])   # the several-row kernels
+    nxt1 = [step([t])[0] for t in range(VOCAB)]                      # one row: one-row kernels, one-row head
+    nxtf = sum((step(list(range(t, t + 8))) for t in range(0, VOCAB, 8)), [])     # few rows: one-row MoE kernels, several-row head
+    nxtn = sum((step(list(range(t, t + 16))) for t in range(0, VOCAB, 16)), [])   # many rows: expert-major MoE, several-row head
     # the end-of-sequence id goes into the file's metadata: take one that a stream reaches as its
     # 4th sample (the next-token maps do not depend on it)
     t0 = next(t for t in range(VOCAB) if len(set(walk(lambda u, z: nxt1[u], t, 4) + [t])) == 5)
     model.eos = walk(lambda u, z: nxt1[u], t0, 4)[3]
     path = model.write(str(tmp_path_factory.mktemp("engine") / "stack.gguf"))
-    return dict(model=model, path=path, nxt1=nxt1, nxtn=nxtn, step=step, eos=model.eos, eos_prompt=t0,
-                nxt=lambda t, z: nxt1[t] if z == 1 else nxtn[t])
+    return dict(model=model, path=path, nxt1=nxt1, nxtf=nxtf, nxtn=nxtn, step=step, eos=model.eos, eos_prompt=t0,
+                nxt=lambda t, z: nxt1[t] if z == 1 else nxtf[t] if z <= qk.ROWWISE_MAX else nxtn[t])
 
 
 def test_next_token_maps(world, orc):
     nxt1, nxtn, model = world["nxt1"], world["nxtn"], world["model"]
     assert len(set(nxt1)) > VOCAB // 8            # a real map, not a constant
-    differ = sum(a != b for a, b in zip(nxt1, nxtn))
-    assert differ <= VOCAB // 50, differ          # two kernel families, same tolerance: near-ties only
+    nxtf = world["nxtf"]
+    for other in (nxtf, nxtn):
+        differ = sum(a != b for a, b in zip(nxt1, other))
+        assert differ <= VOCAB // 50, differ      # other kernel families, same tolerance: near-ties only
+    # few rows: the rows' company and position do not matter
+    few = np.random.default_rng(2).permutation(VOCAB)[:15].tolist()
+    for i in range(0, 15, 5):
+        assert world["step"](few[i:i + 5]) == [nxtf[t] for t in few[i:i + 5]]
     # rows do not influence each other: another grouping of the same tokens gives the same ids
     perm = np.random.default_rng(1).permutation(VOCAB)[:48].tolist()
     for i in range(0, 48, 12):
@@ -152,6 +159,15 @@ def test_slots_staggered_against_the_state_machine(qk, world, monkeypatch):
         assert eng.step_chunk() == (0, {s: [] for s in range(6)}, 0)
 
 
+def test_twelve_slots_take_the_expert_major_path(qk, world):
+    nxt, EOS = world["nxt"], world["eos"]
+    with qk.engine.Engine(world["path"], n_slots=12, n_ctx=64, chunk=3) as eng:
+        ref = OE.SlotMachine(nxt, VOCAB, EOS, 12, 64, 3)
+        script = {0: [("start", s, [20 + 7 * s], 5 + s % 3, 0) for s in range(12)]}
+        drive(eng, ref, script, 5)
+        assert ref.depths[0] == 12 and not any(sl["active"] for sl in ref.slots)
+
+
 def test_serial_prefill_and_eager_launches_give_the_same_streams(qk, world, monkeypatch):
     """QK_NO_BATCH consumes every prompt token in a serial step; QK_NO_GRAPH launches the step's
     kernels one by one instead of replaying the captured graph.  Neither changes a token."""
@@ -186,7 +202,7 @@ def test_stage_run_and_topk(qk, world):
         assert eng.stage_run(0, [1] * 10, 60)[0] == -1          # beyond n_ctx
         toks = [int(t) for t in np.random.default_rng(3).integers(0, VOCAB, 40)]
         rc, ids = eng.stage_run(1, toks, 8)                     # 16 + 16 + 8 rows
-        assert rc == 0 and ids == [nxtn[t] for t in toks]
+        assert rc == 0 and ids == [nxtn[t] for t in toks[:32]] + [world["nxtf"][t] for t in toks[32:]]
         rc, top_ids, top_vals = eng.stage_topk(5)
         assert rc == 0 and len(set(top_ids)) == 5
         assert all(a >= b for a, b in zip(top_vals, top_vals[1:]))

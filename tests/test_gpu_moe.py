@@ -197,15 +197,25 @@ def test_moe_argument_errors(qk, dev, layer_iq4):
     assert e.value.code == -5
 
 
-def test_moe_several_rows_need_n_embd_2048(qk, dev):
-    """One row works at n_embd = 4096; several rows are refused with a shape error, not run wrong."""
+def test_moe_n_embd_4096_rows(qk, orc, dev):
+    """n_embd = 4096: up to ROWWISE_MAX rows run (each through the one-row launches); more rows need
+    the expert-major path, which is built for n_embd = 2048, and are refused with a shape error."""
     import torch
     hl = qk.synth.HostLayer(seed=55, n_embd=4096, n_ff=256, n_expert=4, n_used=2)
     layer = hl.to_device(dev)
-    X = torch.zeros((3, 4096), device=dev)
+    X = np.random.default_rng(3).standard_normal((3, 4096)).astype(np.float32)
     ws = torch.zeros(qk.moe_workspace_bytes(layer, 3), dtype=torch.uint8, device=dev)
+    Y, sel = qk.moe_decode(layer, torch.from_numpy(X).to(dev), ws)
+    torch.cuda.synchronize()
+    ids, _, _ = sel_fields(sel)
+    for t in range(3):
+        r = orc.moe_ref(hl, X[t])
+        assert sorted(ids[t, :2]) == sorted(r["sel"].ids[:2])
+        assert orc.rel_maxabs_err(Y.cpu().numpy()[t], r["y"]) <= TOL
+    X5 = torch.zeros((qk.ROWWISE_MAX + 1, 4096), device=dev)
+    ws5 = torch.zeros(qk.moe_workspace_bytes(layer, qk.ROWWISE_MAX + 1), dtype=torch.uint8, device=dev)
     with pytest.raises(qk.QkError) as e:
-        qk.moe_decode(layer, X, ws)
+        qk.moe_decode(layer, X5, ws5)
     assert e.value.code == -2 and "2048" in str(e.value)
 
 
@@ -312,7 +322,7 @@ def test_moe_decode_tail(qk, orc, dev, layer_iq4, n):
 
 
 @pytest.mark.parametrize("which", ["iq4", "q6k"])
-def test_moe_layer_row(qk, orc, dev, layer_iq4, layer_q6k, which):
+def test_moe_layer_rows_one_row(qk, orc, dev, layer_iq4, layer_q6k, which):
     """One row's whole MoE block in place -- norm inside the router and gate/up launches, residual
     added by the down launch -- against the oracle's norm, step and sum
     (reference src/main.cpp:4376-4402)."""
@@ -334,7 +344,7 @@ def test_moe_layer_row(qk, orc, dev, layer_iq4, layer_q6k, which):
         if r["sel"].gap <= 2e-3 or np.min(-np.diff(lw)) <= 2e-3:
             continue
         Sd = torch.from_numpy(s0).to(dev).reshape(1, 2048)
-        S, sel = qk.moe_layer_row(layer, Sd, Wd, ws)
+        S, sel = qk.moe_layer_rows(layer, Sd, Wd, ws)
         torch.cuda.synchronize()
         assert S.data_ptr() == Sd.data_ptr()
         ids, wts, wsh = sel_fields(sel)
@@ -352,7 +362,40 @@ def test_moe_layer_row(qk, orc, dev, layer_iq4, layer_q6k, which):
             break
     assert done == 4
     with pytest.raises(qk.QkError):
-        qk.moe_layer_row(layer, Sd, None, ws)
+        qk.moe_layer_rows(layer, Sd, None, ws)
+
+
+def test_rows_up_to_the_rowwise_limit_do_not_depend_on_company(qk, dev, layer_iq4):
+    """Up to ROWWISE_MAX rows every row runs the one-row launches: the same row gives the same bits
+    alone, among other rows and at another position; one row more takes the expert-major path and
+    agrees to the tolerance.  The same for the block with the norm in front."""
+    import torch
+    layer = layer_iq4.to_device(dev)
+    nmax = qk.ROWWISE_MAX
+    g = torch.Generator(device=dev)
+    g.manual_seed(5)
+    X = torch.randn((nmax + 1, 2048), device=dev, generator=g)
+    W = torch.rand(2048, device=dev, generator=g) + 0.5
+    ws = torch.zeros(qk.moe_workspace_bytes(layer, nmax + 1), dtype=torch.uint8, device=dev)
+    alone = torch.cat([qk.moe_decode(layer, X[i:i + 1].contiguous(), ws)[0] for i in range(nmax + 1)])
+    Y, sel = qk.moe_decode(layer, X[:nmax].contiguous(), ws)
+    assert torch.equal(Y, alone[:nmax])
+    perm = torch.tensor([3, 0, 2], device=dev)
+    Yp, _ = qk.moe_decode(layer, X[perm].contiguous(), ws)
+    assert torch.equal(Yp, alone[perm])
+    Yg, selg = qk.moe_decode(layer, X.contiguous(), ws)         # one row more: expert-major path
+    torch.cuda.synchronize()
+    scale = float(alone.abs().max())
+    assert float((Yg - alone).abs().max()) <= TOL * scale
+    assert np.array_equal(sel_fields(selg)[0][:nmax, :8], sel_fields(sel)[0][:, :8])
+    # the block with the norm in front
+    one = torch.cat([qk.moe_layer_rows(layer, X[i:i + 1].clone(), W, ws)[0] for i in range(nmax)])
+    S, _ = qk.moe_layer_rows(layer, X[:nmax].clone(), W, ws)
+    torch.cuda.synchronize()
+    assert torch.equal(S, one)
+    with pytest.raises(qk.QkError) as e:
+        qk.moe_layer_rows(layer, X.clone(), W, ws)
+    assert e.value.code == -2
 
 
 def test_group_pairs_matches_oracle(qk, orc, dev):
