@@ -348,7 +348,7 @@ def main():
         del src, dst
     steps = max(a.ring, a.steps // a.ring * a.ring)
     if a.workload == "engine_decode":   # the engine ABI alone (for kernel traces of its graph replays)
-        r = engine_workload(qk, 8, (1, 16), 8, 2)
+        r = engine_workload(qk, 8, (1, 4, 16), 8, 2)
         print(json.dumps(dict(metric="engine_decode_tok_per_s", value=r["slots_16"]["tok_per_s"], unit="tok/s", n_gpus=1,
                               higher_is_better=True, data="synthetic", dtype="f32",
                               config=dict(workload="engine_decode", **r["config"]), detail=r)), flush=True)
@@ -438,6 +438,13 @@ def main():
                                                   stage_us={k: v * 1e3 for k, v in m16["stage_ms"].items()})
             log(f"[bench] moe bs16: {ex['moe_decode_bs16_q6k_down']}")
             torch.cuda.empty_cache()
+            # a few concurrent slots: every row through the one-row launches (grid.y = row)
+            ex["moe_decode_few_rows_q6k_down_us"] = {}
+            for nr in (2, 4, 8):
+                mf = moe_workload(qk, nr, qk.Q6_K, 8, 400, 40)
+                ex["moe_decode_few_rows_q6k_down_us"][f"rows_{nr}"] = mf["ms_event"] * 1e3
+                torch.cuda.empty_cache()
+            log(f"[bench] moe few rows: {ex['moe_decode_few_rows_q6k_down_us']}")
             # layer glue (add + RMS norm alone, and behind the step in one call)
             ex["add_rmsnorm_2048"] = dict(us_1_row=norm_workload(qk, 1, 640, 64), us_16_rows=norm_workload(qk, 16, 640, 64))
             ex["moe_decode_tail_bs1"] = dict(us=moe_tail_workload(qk, 1, qk.IQ4_XS, 8, 400, 40))
@@ -461,7 +468,7 @@ def main():
                                                 tflops=pm["flops"] / (pm["ms_event"] * 1e-3) / 1e12)
             log(f"[bench] prefill moe: {ex['prefill_moe_128_tokens']}")
             torch.cuda.empty_cache()
-            ex["engine_decode_8_layers"] = engine_workload(qk, 8, (1, 16), 8, 2)
+            ex["engine_decode_8_layers"] = engine_workload(qk, 8, (1, 4, 16), 8, 2)
             log(f"[bench] engine: {ex['engine_decode_8_layers']}")
         out["extras"] = ex
 
