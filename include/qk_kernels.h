@@ -126,8 +126,9 @@ int qkk_moe_decode(const qkk_moe_layer *L_host, const float *X, float *Y, qkk_se
  *   S[r]  = resid[r] + (routed + shared contribution of row r)    the next layer's residual input
  *   Xn[r] = S[r] * w_next / sqrt(mean(S[r]^2) + eps)              normalised with the NEXT layer's weight
  * X, sel, workspace, n_slots as for qkk_moe_decode.  resid may be S (in place); Xn must be a buffer
- * of its own.  With several rows the tail runs inside the launch that sums the experts' slots, so
- * the step's output is never written on its own; with one row it costs one more small launch. */
+ * of its own.  Above QKK_ROWWISE_MAX rows the tail runs inside the launch that sums the experts'
+ * slots, so the step's output is never written on its own; up to that many rows it costs one more
+ * small launch (qkk_moe_layer_rows spends none). */
 int qkk_moe_decode_tail(const qkk_moe_layer *L_host, const float *X, const float *resid,
                         const float *w_next, float eps, float *S, float *Xn, qkk_sel *sel,
                         void *workspace, size_t workspace_bytes, uint32_t n_slots, void *stream);
