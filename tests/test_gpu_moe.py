@@ -398,6 +398,24 @@ def test_rows_up_to_the_rowwise_limit_do_not_depend_on_company(qk, dev, layer_iq
     assert e.value.code == -2
 
 
+def test_one_workspace_serves_changing_row_counts(qk, dev, layer_q6k):
+    """An engine keeps one workspace and its step's row count changes from call to call (both
+    paths, whose workspace areas lie at offsets that depend on the row count): every call must give
+    the bits it gives on a freshly cleared workspace."""
+    import torch
+    layer = layer_q6k.to_device(dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(11)
+    X = torch.randn((16, 2048), device=dev, generator=g)
+    shared = torch.zeros(qk.moe_workspace_bytes(layer, 16), dtype=torch.uint8, device=dev)
+    for n in (16, 11, 3, 12, 1, 10, 16, 2, 13):
+        fresh = torch.zeros(qk.moe_workspace_bytes(layer, n), dtype=torch.uint8, device=dev)
+        want, wsel = qk.moe_decode(layer, X[:n].contiguous(), fresh)
+        got, gsel = qk.moe_decode(layer, X[:n].contiguous(), shared)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want) and torch.equal(gsel, wsel), n
+
+
 def test_group_pairs_matches_oracle(qk, orc, dev):
     import torch
     print("[case] group pairs", flush=True)
