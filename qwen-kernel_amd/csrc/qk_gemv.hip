@@ -387,7 +387,9 @@ using namespace qk;
 namespace qk {
 bool coop_gemm_launch(int type, const uint8_t* W, const float* X, float* Y, uint32_t M, uint32_t K, uint32_t N,
                       hipStream_t st);
-constexpr uint32_t COOP_MIN_BATCH = 3;
+// rows from which the weights are read once for all rows on the matrix cores; K = 4096 takes two
+// passes there (13 us at 2048 x 4096 whatever the batch), so one more row stays on one pass per row
+constexpr uint32_t COOP_MIN_BATCH = 3, COOP_MIN_BATCH_K4096 = 4;
 } // namespace qk
 
 extern "C" {
@@ -502,7 +504,7 @@ int qkk_gemv(int type, const void* W, const float* X, float* Y, uint32_t M, uint
     hipStream_t st = as_stream(stream);
     // several rows: read the weights once for all of them on the matrix cores (needs Y aligned
     // like any output of that path); one row, or a shape that path does not cover: one pass per row
-    if (batch >= COOP_MIN_BATCH && aligned16(Y) && coop_gemm_launch(type, (const uint8_t*)W, X, Y, M, K, batch, st))
+    if (batch >= (K >= 4096 ? COOP_MIN_BATCH_K4096 : COOP_MIN_BATCH) && aligned16(Y) && coop_gemm_launch(type, (const uint8_t*)W, X, Y, M, K, batch, st))
         return check_launch("qkk_gemv");
     switch (type) {
     case QKK_Q8_0: return dispatch_q<QKK_Q8_0>(W, X, Y, M, K, batch, st);
