@@ -168,6 +168,30 @@ def test_twelve_slots_take_the_expert_major_path(qk, world):
         assert ref.depths[0] == 12 and not any(sl["active"] for sl in ref.slots)
 
 
+@pytest.mark.parametrize("seed", [1, 2])
+def test_random_request_traffic(qk, world, seed):
+    """Sixteen slots, requests arriving, finishing and being cancelled at random for a few hundred
+    chunks: every return of the engine against the restated state machine."""
+    import random
+    nxt, EOS = world["nxt"], world["eos"]
+    rnd = random.Random(seed)
+    with qk.engine.Engine(world["path"], n_slots=16, n_ctx=96, chunk=4) as eng:
+        ref = OE.SlotMachine(nxt, VOCAB, EOS, 16, 96, 4)
+        script = {}
+        for call in range(120):
+            ops = []
+            for _ in range(rnd.choice([0, 0, 1, 1, 2, 5])):
+                slot = rnd.randrange(16)
+                if rnd.random() < 0.15:
+                    ops.append(("cancel", slot))
+                else:
+                    prompt = [rnd.randrange(VOCAB) for _ in range(rnd.choice([1, 2, 5, 18, 40]))]
+                    ops.append(("start", slot, prompt, rnd.choice([1, 4, 9, 30, 60]), rnd.choice([0, 0, 17])))
+            script[call] = ops
+        drive(eng, ref, script, 150)
+        assert len(set(ref.depths)) >= 8 and max(ref.depths) > qk.ROWWISE_MAX and min(ref.depths) <= 4
+
+
 def test_serial_prefill_and_eager_launches_give_the_same_streams(qk, world, monkeypatch):
     """QK_NO_BATCH consumes every prompt token in a serial step; QK_NO_GRAPH launches the step's
     kernels one by one instead of replaying the captured graph.  Neither changes a token."""
