@@ -225,6 +225,34 @@ int qkk_vec_add(const float *a, const float *b, float *out, uint64_t n, void *st
 int qkk_embed(int type, const void *W, uint32_t n_vocab, uint32_t kdim, const uint32_t *ids,
               uint32_t n_ids, uint32_t idx, uint32_t per_req, float *x, uint32_t rows, void *stream);
 
+/* ---- full-attention mixer, decode step ---------------------------------------------------------
+ * (reference shaders/fa_prep_srv.comp:26-76, fa_attn_srv.comp:27-95 and its split / grouped forms
+ * fa_attn_srv_split_gqa.comp, fa_attn_srv_reduce.comp; host src/main.cpp:4246-4300; CPU mirror
+ * src/main.cpp:2138-2201.)  Head size dh = 256; hQ query heads on hKV KV heads, hQ/hKV <= 8.
+ *   qfull    [slots][hQ][2*dh]   per head dh query values, then dh output-gate pre-activations
+ *   kin, vin [slots][hKV][dh]
+ *   caches   [slots][hKV][tmax][dh] fp32
+ *   rope     [tmax][n_rot/2][2] (cos, sin) on the device; qkk_rope_table fills a host array the
+ *            way the reference does (src/main.cpp:2011-2020, float powf / cosf / sinf)
+ *   slot_pos [slots] device words: position of the slot's new token (clamped to tmax - 1)
+ * qkk_attn_prep: per head RMS norm with q_norm_w / k_norm_w, the first n_rot dims rotated by the
+ *   position's angles (pairs j, j + n_rot/2); queries to qhat [slots][hQ][dh], keys and values into
+ *   the caches at slot_pos.
+ * qkk_attn_decode: att[slot][h] = softmax(qhat[h] . K[0..pos] / sqrt(dh)) V[0..pos] * sigmoid(gate),
+ *   K/V of KV head h / (hQ/hKV).  Every cache row is read once for the hQ/hKV heads that share it;
+ *   positions are cut into 64 ranges that run in parallel and are folded in range order.  The
+ *   launch shape depends on tmax only, so a captured graph stays valid as positions advance.
+ *   workspace: qkk_attn_workspace_bytes(), 256-byte aligned, no initialisation needed. */
+int qkk_rope_table(float *rope_host, uint32_t tmax, uint32_t n_rot, float freq_base);
+int qkk_attn_prep(const float *qfull, const float *kin, const float *vin, const float *q_norm_w,
+                  const float *k_norm_w, const float *rope, const uint32_t *slot_pos, float *qhat,
+                  float *k_cache, float *v_cache, uint32_t n_slots, uint32_t hQ, uint32_t hKV, uint32_t dh,
+                  uint32_t n_rot, uint32_t tmax, float eps, void *stream);
+size_t qkk_attn_workspace_bytes(uint32_t n_slots, uint32_t hQ, uint32_t dh);
+int qkk_attn_decode(const float *qhat, const float *k_cache, const float *v_cache, const float *qfull,
+                    const uint32_t *slot_pos, float *att, void *workspace, size_t workspace_bytes,
+                    uint32_t n_slots, uint32_t hQ, uint32_t hKV, uint32_t dh, uint32_t tmax, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -71,6 +71,11 @@ def lib():
         L.qkk_add_rms3.argtypes = [vp, vp, vp, vp, vp, vp, u32, u32, f32, vp]
         L.qkk_vec_add.argtypes = [vp, vp, vp, u64, vp]
         L.qkk_embed.argtypes = [C.c_int, vp, u32, u32, vp, u32, u32, u32, vp, u32, vp]
+        L.qkk_rope_table.argtypes = [vp, u32, u32, f32]
+        L.qkk_attn_prep.argtypes = [vp] * 10 + [u32] * 6 + [f32, vp]
+        L.qkk_attn_workspace_bytes.restype = sz
+        L.qkk_attn_workspace_bytes.argtypes = [u32, u32, u32]
+        L.qkk_attn_decode.argtypes = [vp] * 7 + [sz] + [u32] * 5 + [vp]
         _lib = L
     return _lib
 
@@ -302,3 +307,43 @@ def embed(type_, W, n_vocab, kdim, ids, rows, idx=0, per_req=1, out=None):
     _check(lib().qkk_embed(type_, _ptr(W), n_vocab, kdim, _ptr(ids), ids.numel(), idx, per_req, _ptr(out), rows,
                            _stream()))
     return out
+
+
+def rope_table(tmax, n_rot, freq_base=1e7):
+    """[tmax][n_rot/2][2] (cos, sin) as a float32 numpy array, computed by the library on the host."""
+    import numpy as np
+    out = np.empty((tmax, n_rot // 2, 2), dtype=np.float32)
+    _check(lib().qkk_rope_table(out.ctypes.data_as(C.c_void_p), tmax, n_rot, freq_base))
+    return out
+
+
+def attn_prep(qfull, kin, vin, q_norm_w, k_norm_w, rope, slot_pos, k_cache, v_cache, n_rot, eps=1e-6, qhat=None):
+    """Head norm + RoPE + cache write for the slots' new tokens.  qfull [slots][hQ][2*dh],
+    kin / vin [slots][hKV][dh], caches [slots][hKV][tmax][dh].  Returns qhat [slots][hQ][dh]."""
+    import torch
+    n, hQ, dh2 = qfull.shape
+    hKV, tmax, dh = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
+    if qhat is None:
+        qhat = torch.empty((n, hQ, dh), dtype=torch.float32, device=qfull.device)
+    _check(lib().qkk_attn_prep(_ptr(qfull), _ptr(kin), _ptr(vin), _ptr(q_norm_w), _ptr(k_norm_w), _ptr(rope),
+                               _ptr(slot_pos), _ptr(qhat), _ptr(k_cache), _ptr(v_cache), n, hQ, hKV, dh, n_rot, tmax,
+                               eps, _stream()))
+    return qhat
+
+
+def attn_workspace_bytes(n_slots, hQ, dh=256):
+    return lib().qkk_attn_workspace_bytes(n_slots, hQ, dh)
+
+
+def attn_decode(qhat, k_cache, v_cache, qfull, slot_pos, workspace, att=None):
+    """Attention of the slots' new tokens over positions 0..slot_pos with the output gate.
+    Returns att [slots][hQ][dh]."""
+    import torch
+    n, hQ, dh = qhat.shape
+    hKV, tmax = k_cache.shape[1], k_cache.shape[2]
+    if att is None:
+        att = torch.empty_like(qhat)
+    _check(lib().qkk_attn_decode(_ptr(qhat), _ptr(k_cache), _ptr(v_cache), _ptr(qfull), _ptr(slot_pos), _ptr(att),
+                                 _ptr(workspace), workspace.numel() * workspace.element_size(), n, hQ, hKV, dh, tmax,
+                                 _stream()))
+    return att
