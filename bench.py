@@ -246,6 +246,40 @@ def prefill_moe_workload(qk, n_tokens, steps, warmup, seed=4242):
     return dict(ms_event=ev, distinct_experts=u, bytes_step=L.active_bytes(u) + n_tokens * 2 * H * 4, flops=flops)
 
 
+def attn_workload(qk, n_slots, ctx, steps, warmup, tmax=4096, seed=5):
+    """The full-attention decode step (prep + attention) of n_slots slots at position ctx - 1: the
+    reference's head shape (16 query heads of 256 on 2 KV heads, 64 rotated dims), fp32 caches of
+    tmax positions.  A ring of distinct cache sets (> 1 GB in all) stands for the attention layers
+    of a model, so no step finds its keys in a cache.  Bytes: the K and V rows of the ctx positions."""
+    import numpy as np
+    import torch
+    dev = "cuda:0"
+    hQ, hKV, dh, n_rot = 16, 2, 256, 64
+    per_set = 2 * n_slots * hKV * tmax * dh * 4
+    ring = max(2, min(64, (1 << 30) // per_set + 1))
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    kc = [torch.randn((n_slots, hKV, tmax, dh), device=dev, generator=g) for _ in range(ring)]
+    vc = [torch.randn((n_slots, hKV, tmax, dh), device=dev, generator=g) for _ in range(ring)]
+    qfull = torch.randn((ring, n_slots, hQ, 2 * dh), device=dev, generator=g)
+    kin = torch.randn((ring, n_slots, hKV, dh), device=dev, generator=g)
+    vin = torch.randn((ring, n_slots, hKV, dh), device=dev, generator=g)
+    w = torch.ones(dh, device=dev)
+    rope = torch.from_numpy(qk.rope_table(tmax, n_rot)).to(dev)
+    pos = torch.full((n_slots,), ctx - 1, dtype=torch.int32, device=dev)
+    qhat = torch.empty((ring, n_slots, hQ, dh), device=dev)
+    att = torch.empty((ring, n_slots, hQ, dh), device=dev)
+    ws = torch.empty(qk.attn_workspace_bytes(n_slots, hQ), dtype=torch.uint8, device=dev)
+
+    def step(i):
+        def f():
+            qk.attn_prep(qfull[i], kin[i], vin[i], w, w, rope, pos, kc[i], vc[i], n_rot, qhat=qhat[i])
+            qk.attn_decode(qhat[i], kc[i], vc[i], qfull[i], pos, ws, att=att[i])
+        return f
+    wall, ev, n = run_ring([step(i) for i in range(ring)], steps // ring * ring, warmup)
+    return dict(ms_event=ev, steps=n, ring=ring, bytes_step=2 * n_slots * hKV * ctx * dh * 4)
+
+
 def engine_workload(qk, n_layer, slots_list, chunks, warm_chunks, seed=31):
     """Tokens per second through the engine ABI (qk_open / qk_slot_start / qk_step_chunk) on a
     synthetic MoE-only model file at the full layer shape and vocabulary: host wall clock over
@@ -352,6 +386,16 @@ def main():
         print(json.dumps(dict(metric="engine_decode_tok_per_s", value=r["slots_16"]["tok_per_s"], unit="tok/s", n_gpus=1,
                               higher_is_better=True, data="synthetic", dtype="f32",
                               config=dict(workload="engine_decode", **r["config"]), detail=r)), flush=True)
+        return
+    if a.workload in ("attn_bs1", "attn_bs16"):   # the attention decode step alone
+        b = 1 if a.workload == "attn_bs1" else 16
+        at = attn_workload(qk, b, 4096, min(a.steps, 400), min(a.warmup, 40))
+        gb = at["bytes_step"] / (at["ms_event"] * 1e-3) / 1e9
+        print(json.dumps(dict(metric="attn_decode_hbm_gbps", value=gb, unit="GB/s", n_gpus=1, steps=at["steps"],
+                              ms_per_step=at["ms_event"], higher_is_better=True, data="synthetic", dtype="f32",
+                              config=dict(workload=a.workload, slots=b, positions=4096, heads="16 x 256 on 2 KV heads",
+                                          ring=at["ring"]),
+                              bytes_per_step=at["bytes_step"], frac_of_hbm_peak=gb / HBM_PEAK_GBPS)), flush=True)
         return
     if a.workload in ("head_bs1", "head_bs16"):   # the LM head alone (for counter runs on its kernel)
         b = 1 if a.workload == "head_bs1" else 16
@@ -468,6 +512,13 @@ def main():
                                                 tflops=pm["flops"] / (pm["ms_event"] * 1e-3) / 1e12)
             log(f"[bench] prefill moe: {ex['prefill_moe_128_tokens']}")
             torch.cuda.empty_cache()
+            for b in (1, 16):   # the full-attention mixer's decode step at 4096 cached positions
+                at = attn_workload(qk, b, 4096, 200, 20)
+                gb = at["bytes_step"] / (at["ms_event"] * 1e-3) / 1e9
+                ex[f"attn_decode_ctx4096_bs{b}"] = dict(us=at["ms_event"] * 1e3, gbps=gb, frac=gb / HBM_PEAK_GBPS,
+                                                        ring=at["ring"])
+                torch.cuda.empty_cache()
+            log(f"[bench] attention: {ex['attn_decode_ctx4096_bs1']} {ex['attn_decode_ctx4096_bs16']}")
             ex["engine_decode_8_layers"] = engine_workload(qk, 8, (1, 4, 16), 8, 2)
             log(f"[bench] engine: {ex['engine_decode_8_layers']}")
         out["extras"] = ex

@@ -13,19 +13,23 @@
 //
 // Attention is bound by reading the cache: 2 * hKV * n * dh * 4 bytes per slot.  The G = hQ/hKV
 // query heads that share a KV head are handled by ONE workgroup, so every K and V row is read once
-// for all of them, and the positions are cut into ATT_CHUNKS ranges that run in parallel (two KV
-// heads alone would leave 254 CUs idle); a second launch folds the ranges' (max, sum, accumulator)
-// triples in range order.  Which ranges hold keys is decided on the device from slot_pos, so the
-// launch shape depends on tmax only and a captured graph stays valid as the sequences grow.
+// for all of them, and the positions are cut into ranges that run in parallel (two KV heads alone
+// would leave 254 CUs idle; the host picks 8..128 ranges so that about a thousand workgroups
+// result); a second launch folds the ranges' (max, sum, accumulator) triples in range order.  Which
+// ranges hold keys is decided on the device from slot_pos, so the launch shape depends on the slot
+// count and tmax only and a captured graph stays valid as the sequences grow.
 #include "qk_device.h"
 #include "qk_host.h"
+#include "qk_mfma.h"
 
 #include <math.h>
+
+#include <algorithm>
 
 namespace qk {
 
 constexpr uint32_t ATT_DH = 256;    // head size = workgroup size
-constexpr uint32_t ATT_CHUNKS = 64; // position ranges per (slot, KV head)
+constexpr uint32_t ATT_MAX_RANGES = 128; // position ranges per (slot, KV head), at most
 constexpr uint32_t ATT_TILE = 64;   // positions scored per pass
 constexpr uint32_t ATT_GMAX = 8;    // query heads per KV head
 constexpr float ATT_FLOOR = -3.4e38f;
@@ -75,52 +79,111 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const float* __restrict_
 // Partial results of one position range: per query head the running maximum, the sum of
 // exp(score - maximum) and the exp-weighted sum of the value rows.
 struct AttnWs {
-    float* acc; // [slots][hQ][ATT_CHUNKS][dh]
-    float* ml;  // [slots][hQ][ATT_CHUNKS][2]
+    float* acc; // [slots][hQ][n_ranges][dh]
+    float* ml;  // [slots][hQ][n_ranges][2]
 };
 
-// grid (ATT_CHUNKS, hKV, slots), 256 threads.  G query heads of one KV head over one position range.
+// Eight floats as hi + lo halves (x = hi + lo to ~2^-22 of x): hi truncates x, lo rounds the exact rest.
+struct HalfSplit {
+    half8 hi, lo;
+};
+__device__ __forceinline__ HalfSplit split8(float4 a, float4 b)
+{
+    const float x[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    uint32_t h[4], l[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const auto hp = __builtin_amdgcn_cvt_pkrtz(x[2 * i], x[2 * i + 1]);
+        const auto lp = __builtin_amdgcn_cvt_pkrtz(x[2 * i] - (float)hp[0], x[2 * i + 1] - (float)hp[1]);
+        h[i] = __builtin_bit_cast(uint32_t, hp);
+        l[i] = __builtin_bit_cast(uint32_t, lp);
+    }
+    HalfSplit r;
+    r.hi = __builtin_bit_cast(half8, uint4{h[0], h[1], h[2], h[3]});
+    r.lo = __builtin_bit_cast(half8, uint4{l[0], l[1], l[2], l[3]});
+    return r;
+}
+
+// grid (n_ranges, hKV, slots), 256 threads.  The G query heads of one KV head over one position
+// range, a tile of ATT_TILE positions at a time; wave w owns the tile's positions 16w .. 16w+15 and
+// requests their K and V rows (32 pieces of 16 bytes per lane) before any arithmetic, so a tile
+// costs one memory round trip.
+//   scores  on the matrix cores: D[head][position] += Q[head][32 dims] . K[position][32 dims]
+//           (v_mfma_f32_16x16x32_f16, heads padded to 16 with zeros), both operands split into
+//           hi + lo halves and three products kept (hi.hi, hi.lo, lo.hi), so a score is exact to
+//           ~2^-22 of its terms.  A K row's 256 dims are read by four lanes in pieces of 32 bytes,
+//           full cache lines per wave instruction.  (Per-lane partial dot products folded across
+//           the wave took ten times the vector instructions: one cross-lane sum per head and row.)
+//   softmax running maximum and sum per head over the tile, in LDS.
+//   values  a lane keeps 4 dims of every head's accumulator and adds its wave's 16 rows; the four
+//           waves' accumulators are added through LDS at the end, in wave order.
 __global__ __launch_bounds__(256) void attn_range_kernel(const float* __restrict__ qhat, const float* __restrict__ kc,
                                                          const float* __restrict__ vc,
                                                          const uint32_t* __restrict__ slot_pos, AttnWs ws, uint32_t hQ,
                                                          uint32_t hKV, uint32_t G, uint32_t tmax)
 {
+    constexpr uint32_t RPW = ATT_TILE / 4; // rows per wave and tile (16: one MFMA column block)
+    constexpr uint32_t KB = ATT_DH / 32;   // 32-dim blocks of a row
+    __shared__ __attribute__((aligned(16))) half8 s_qh[KB][64], s_ql[KB][64]; // Q as the A operand, per lane
     __shared__ __attribute__((aligned(16))) float s_sc[ATT_GMAX][ATT_TILE];
     __shared__ float s_corr[ATT_GMAX], s_m[ATT_GMAX], s_l[ATT_GMAX];
-    const uint32_t c = blockIdx.x, kv = blockIdx.y, rq = blockIdx.z, t = threadIdx.x;
-    const uint32_t lane = t & 63u, wave = t >> 6;
+    __shared__ __attribute__((aligned(16))) float s_acc[3][ATT_GMAX][ATT_DH]; // waves 1..3 hand theirs to wave 0
+    const uint32_t n_ranges = gridDim.x, c = blockIdx.x, kv = blockIdx.y, rq = blockIdx.z, t = threadIdx.x;
+    const uint32_t lane = t & 63u, wave = t >> 6, col = lane & 15u, quad = lane >> 4;
     const uint32_t n = slot_position(slot_pos, rq, tmax) + 1u;
-    const uint32_t per = (tmax + ATT_CHUNKS - 1) / ATT_CHUNKS;
+    const uint32_t per = (tmax + n_ranges - 1) / n_ranges;
     const uint32_t p_begin = c * per, p_end = min(n, p_begin + per);
     if (p_begin >= n) return; // the whole workgroup: this range holds no key yet
 
-    // the lane's four dims of every query head, in registers for all tiles
-    float4 q[ATT_GMAX];
+    // Q operand: lane feeds A[head = col][dims 32*kb + 8*quad .. +7]; wave w prepares blocks 2w, 2w+1
 #pragma unroll
-    for (uint32_t h = 0; h < ATT_GMAX; h++)
-        q[h] = h < G ? ((const float4*)(qhat + ((size_t)rq * hQ + kv * G + h) * ATT_DH))[lane] : float4{0.f, 0.f, 0.f, 0.f};
+    for (uint32_t i = 0; i < 2; i++) {
+        const uint32_t kb = 2 * wave + i;
+        float4 a = float4{0.f, 0.f, 0.f, 0.f}, b = a;
+        if (col < G) {
+            const float4* qrow = (const float4*)(qhat + ((size_t)rq * hQ + kv * G + col) * ATT_DH);
+            a = qrow[kb * 8 + 2 * quad];
+            b = qrow[kb * 8 + 2 * quad + 1];
+        }
+        const HalfSplit sp = split8(a, b);
+        s_qh[kb][lane] = sp.hi;
+        s_ql[kb][lane] = sp.lo;
+    }
     if (t < ATT_GMAX) { s_m[t] = ATT_FLOOR; s_l[t] = 0.f; }
     const float qs = 1.f / sqrtf((float)ATT_DH);
-    const float* kbase = kc + ((size_t)rq * hKV + kv) * tmax * ATT_DH;
-    const float* vbase = vc + ((size_t)rq * hKV + kv) * tmax * ATT_DH;
-    float acc[ATT_GMAX];
+    const float4* kbase = (const float4*)(kc + ((size_t)rq * hKV + kv) * tmax * ATT_DH);
+    const float4* vbase = (const float4*)(vc + ((size_t)rq * hKV + kv) * tmax * ATT_DH);
+    float4 acc[ATT_GMAX];
 #pragma unroll
-    for (uint32_t h = 0; h < ATT_GMAX; h++) acc[h] = 0.f;
+    for (uint32_t h = 0; h < ATT_GMAX; h++) acc[h] = float4{0.f, 0.f, 0.f, 0.f};
     __syncthreads();
 
     for (uint32_t p0 = p_begin; p0 < p_end; p0 += ATT_TILE) {
         const uint32_t ts = min(ATT_TILE, p_end - p0);
-        // scores: a wave takes every fourth position of the tile; one coalesced 1 KB row per position
-        for (uint32_t i = wave; i < ts; i += 4) {
-            const float4 k4 = ((const float4*)(kbase + (size_t)(p0 + i) * ATT_DH))[lane];
+        // rows beyond the tile repeat its last row (their scores are masked, their weights zero)
+        const size_t krow = p0 + min(RPW * wave + col, ts - 1);
+        float4 ka[KB], kb4[KB], v4[RPW];
 #pragma unroll
-            for (uint32_t h = 0; h < ATT_GMAX; h++) {
-                if (h < G) { // uniform
-                    const float d = wave_sum((q[h].x * k4.x + q[h].y * k4.y) + (q[h].z * k4.z + q[h].w * k4.w));
-                    if (lane == 0) s_sc[h][i] = d * qs;
-                }
-            }
+        for (uint32_t kb = 0; kb < KB; kb++) {
+            ka[kb] = kbase[krow * (ATT_DH / 4) + kb * 8 + 2 * quad];
+            kb4[kb] = kbase[krow * (ATT_DH / 4) + kb * 8 + 2 * quad + 1];
         }
+#pragma unroll
+        for (uint32_t i = 0; i < RPW; i++)
+            v4[i] = vbase[(size_t)(p0 + min(RPW * wave + i, ts - 1)) * (ATT_DH / 4) + lane];
+        float4v sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (uint32_t kb = 0; kb < KB; kb++) {
+            const HalfSplit k = split8(ka[kb], kb4[kb]);
+            const half8 qh = s_qh[kb][lane], ql = s_ql[kb][lane];
+            sc = mfma16x32(qh, k.hi, sc);
+            sc = mfma16x32(qh, k.lo, sc);
+            sc = mfma16x32(ql, k.hi, sc);
+        }
+        // D[4*quad + e][col]: head 4*quad + e, position 16*wave + col
+#pragma unroll
+        for (uint32_t e = 0; e < 4; e++)
+            if (4 * quad + e < G) s_sc[4 * quad + e][RPW * wave + col] = sc[e] * qs;
         __syncthreads();
         // running maximum and sum per head: wave w folds heads w, w + 4 (lane = position of the tile)
         for (uint32_t h = wave; h < G; h += 4) {
@@ -138,45 +201,96 @@ __global__ __launch_bounds__(256) void attn_range_kernel(const float* __restrict
             }
         }
         __syncthreads();
-        // weighted value rows: thread t owns dim t of every head's accumulator
 #pragma unroll
-        for (uint32_t h = 0; h < ATT_GMAX; h++) acc[h] *= h < G ? s_corr[h] : 0.f;
-        for (uint32_t j = 0; j < ts; j++) {
-            const float vv = vbase[(size_t)(p0 + j) * ATT_DH + t];
+        for (uint32_t h = 0; h < ATT_GMAX; h++) {
+            if (h < G) { // uniform
+                const float corr = s_corr[h];
+                float4 a = float4{acc[h].x * corr, acc[h].y * corr, acc[h].z * corr, acc[h].w * corr};
 #pragma unroll
-            for (uint32_t h = 0; h < ATT_GMAX; h++)
-                if (h < G) acc[h] += s_sc[h][j] * vv;
+                for (uint32_t i = 0; i < RPW; i += 4) { // the weights of positions beyond the tile are zero
+                    const float4 w = *(const float4*)&s_sc[h][RPW * wave + i];
+                    a.x += w.x * v4[i].x + w.y * v4[i + 1].x + w.z * v4[i + 2].x + w.w * v4[i + 3].x;
+                    a.y += w.x * v4[i].y + w.y * v4[i + 1].y + w.z * v4[i + 2].y + w.w * v4[i + 3].y;
+                    a.z += w.x * v4[i].z + w.y * v4[i + 1].z + w.z * v4[i + 2].z + w.w * v4[i + 3].z;
+                    a.w += w.x * v4[i].w + w.y * v4[i + 1].w + w.z * v4[i + 2].w + w.w * v4[i + 3].w;
+                }
+                acc[h] = a;
+            }
         }
         __syncthreads(); // the next tile overwrites the scores
     }
-    for (uint32_t h = 0; h < G; h++) {
-        const size_t slot = ((size_t)rq * hQ + kv * G + h) * ATT_CHUNKS + c;
-        ws.acc[slot * ATT_DH + t] = acc[h];
-        if (t == 0) { ws.ml[2 * slot] = s_m[h]; ws.ml[2 * slot + 1] = s_l[h]; }
+    // the four waves' accumulators, added in wave order
+    if (wave > 0) {
+#pragma unroll
+        for (uint32_t h = 0; h < ATT_GMAX; h++)
+            if (h < G) ((float4*)s_acc[wave - 1][h])[lane] = acc[h];
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+        for (uint32_t h = 0; h < ATT_GMAX; h++) {
+            if (h < G) {
+                float4 a = acc[h];
+                for (uint32_t w = 0; w < 3; w++) {
+                    const float4 b = ((const float4*)s_acc[w][h])[lane];
+                    a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+                }
+                const size_t slot = ((size_t)rq * hQ + kv * G + h) * n_ranges + c;
+                ((float4*)(ws.acc + slot * ATT_DH))[lane] = a;
+                if (lane == 0) { ws.ml[2 * slot] = s_m[h]; ws.ml[2 * slot + 1] = s_l[h]; }
+            }
+        }
     }
 }
 
 // grid (hQ, slots), 256 threads: folds the ranges of one query head in range order, divides by the
-// sum and applies the output gate sigmoid(qfull[head][dh + t]).
+// sum and applies the output gate sigmoid(qfull[head][dh + t]).  Wave w adds the ranges w, w+4, ...
+// (a lane 4 dims, eight ranges requested at a time); the waves' sums are added in wave order.
 __global__ __launch_bounds__(256) void attn_fold_kernel(AttnWs ws, const float* __restrict__ qfull,
                                                         const uint32_t* __restrict__ slot_pos, float* __restrict__ att,
-                                                        uint32_t hQ, uint32_t tmax)
+                                                        uint32_t hQ, uint32_t tmax, uint32_t n_ranges_all)
 {
-    const uint32_t h = blockIdx.x, rq = blockIdx.y, t = threadIdx.x;
+    __shared__ float s_f[ATT_MAX_RANGES], s_lf[ATT_MAX_RANGES];
+    __shared__ __attribute__((aligned(16))) float s_o[4][ATT_DH];
+    const uint32_t h = blockIdx.x, rq = blockIdx.y, t = threadIdx.x, lane = t & 63u, wave = t >> 6;
     const uint32_t n = slot_position(slot_pos, rq, tmax) + 1u;
-    const uint32_t per = (tmax + ATT_CHUNKS - 1) / ATT_CHUNKS;
-    const uint32_t n_ranges = min(ATT_CHUNKS, (n + per - 1) / per);
-    const size_t base = ((size_t)rq * hQ + h) * ATT_CHUNKS;
-    float m = ATT_FLOOR;
-    for (uint32_t c = 0; c < n_ranges; c++) m = fmaxf(m, ws.ml[2 * (base + c)]);
-    float l = 0.f, o = 0.f;
-    for (uint32_t c = 0; c < n_ranges; c++) {
-        const float f = expf(ws.ml[2 * (base + c)] - m);
-        l += ws.ml[2 * (base + c) + 1] * f;
-        o += ws.acc[(base + c) * ATT_DH + t] * f;
-    }
+    const uint32_t per = (tmax + n_ranges_all - 1) / n_ranges_all;
+    const uint32_t n_ranges = min(n_ranges_all, (n + per - 1) / per); // the ranges that hold keys
+    const size_t base = ((size_t)rq * hQ + h) * n_ranges_all;
     const float g = qfull[((size_t)rq * hQ + h) * 2 * ATT_DH + ATT_DH + t];
-    att[((size_t)rq * hQ + h) * ATT_DH + t] = (o / l) * (1.f / (1.f + expf(-g)));
+    float my_m = ATT_FLOOR, my_l = 0.f;
+    if (t < n_ranges) { my_m = ws.ml[2 * (base + t)]; my_l = ws.ml[2 * (base + t) + 1]; }
+    if (t < ATT_MAX_RANGES) s_f[t] = my_m;
+    __syncthreads();
+    float m = ATT_FLOOR;
+    for (uint32_t c = 0; c < n_ranges; c++) m = fmaxf(m, s_f[c]);
+    __syncthreads();
+    if (t < n_ranges) {
+        const float f = expf(my_m - m);
+        s_f[t] = f;
+        s_lf[t] = my_l * f;
+    }
+    __syncthreads();
+    float l = 0.f;
+    for (uint32_t c = 0; c < n_ranges; c++) l += s_lf[c];
+    float4 o = float4{0.f, 0.f, 0.f, 0.f};
+    for (uint32_t c0 = wave; c0 < n_ranges; c0 += 32) {
+        float4 a[8];
+#pragma unroll
+        for (uint32_t i = 0; i < 8; i++) {
+            const uint32_t c = min(c0 + 4 * i, n_ranges - 1);
+            a[i] = ((const float4*)(ws.acc + (base + c) * ATT_DH))[lane];
+        }
+#pragma unroll
+        for (uint32_t i = 0; i < 8; i++) {
+            const float f = c0 + 4 * i < n_ranges ? s_f[c0 + 4 * i] : 0.f;
+            o.x += a[i].x * f; o.y += a[i].y * f; o.z += a[i].z * f; o.w += a[i].w * f;
+        }
+    }
+    ((float4*)s_o[wave])[lane] = o;
+    __syncthreads();
+    const float tot = ((s_o[0][t] + s_o[1][t]) + s_o[2][t]) + s_o[3][t];
+    att[((size_t)rq * hQ + h) * ATT_DH + t] = (tot / l) * (1.f / (1.f + expf(-g)));
 }
 
 static int check_shape(const char* who, uint32_t n_slots, uint32_t hQ, uint32_t hKV, uint32_t dh, uint32_t tmax)
@@ -229,7 +343,7 @@ int qkk_attn_prep(const float* qfull, const float* kin, const float* vin, const 
 size_t qkk_attn_workspace_bytes(uint32_t n_slots, uint32_t hQ, uint32_t dh)
 {
     if (!n_slots || !hQ || !dh) return 0;
-    return (size_t)n_slots * hQ * ATT_CHUNKS * ((size_t)dh + 2) * sizeof(float) + 256;
+    return (size_t)n_slots * hQ * ATT_MAX_RANGES * ((size_t)dh + 2) * sizeof(float) + 256;
 }
 
 int qkk_attn_decode(const float* qhat, const float* k_cache, const float* v_cache, const float* qfull,
@@ -239,19 +353,22 @@ int qkk_attn_decode(const float* qhat, const float* k_cache, const float* v_cach
     if (!qhat || !k_cache || !v_cache || !qfull || !slot_pos || !att || !workspace)
         return fail(QKK_EINVAL, "qkk_attn_decode: null pointer");
     if (int rc = check_shape("qkk_attn_decode", n_slots, hQ, hKV, dh, tmax)) return rc;
-    if (!aligned16(qhat) || !aligned16(k_cache) || (reinterpret_cast<uintptr_t>(workspace) & 255u))
-        return fail(QKK_EINVAL, "qkk_attn_decode: qhat and k_cache must be 16-byte, workspace 256-byte aligned");
+    if (!aligned16(qhat) || !aligned16(k_cache) || !aligned16(v_cache) || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+        return fail(QKK_EINVAL, "qkk_attn_decode: qhat and the caches must be 16-byte, workspace 256-byte aligned");
     if (workspace_bytes < qkk_attn_workspace_bytes(n_slots, hQ, dh))
         return fail(QKK_EWORKSPACE, "qkk_attn_decode: workspace %zu < %zu bytes", workspace_bytes,
                     qkk_attn_workspace_bytes(n_slots, hQ, dh));
     if (int rc = require_device()) return rc;
     hipStream_t st = as_stream(stream);
+    // about a thousand workgroups (four per CU) over the (slot, KV head) pairs, 8..128 ranges each
+    const uint32_t n_ranges = std::min(ATT_MAX_RANGES, std::max(8u, persistent_blocks() / (n_slots * hKV)));
     AttnWs ws;
     ws.acc = (float*)workspace;
-    ws.ml = ws.acc + (size_t)n_slots * hQ * ATT_CHUNKS * ATT_DH;
-    hipLaunchKernelGGL(attn_range_kernel, dim3(ATT_CHUNKS, hKV, n_slots), dim3(256), 0, st, qhat, k_cache, v_cache,
+    ws.ml = ws.acc + (size_t)n_slots * hQ * n_ranges * ATT_DH;
+    hipLaunchKernelGGL(attn_range_kernel, dim3(n_ranges, hKV, n_slots), dim3(256), 0, st, qhat, k_cache, v_cache,
                        slot_pos, ws, hQ, hKV, hQ / hKV, tmax);
-    hipLaunchKernelGGL(attn_fold_kernel, dim3(hQ, n_slots), dim3(256), 0, st, ws, qfull, slot_pos, att, hQ, tmax);
+    hipLaunchKernelGGL(attn_fold_kernel, dim3(hQ, n_slots), dim3(256), 0, st, ws, qfull, slot_pos, att, hQ, tmax,
+                       n_ranges);
     return check_launch("qkk_attn_decode");
 }
 
