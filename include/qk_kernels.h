@@ -240,7 +240,7 @@ int qkk_embed(int type, const void *W, uint32_t n_vocab, uint32_t kdim, const ui
  *   the caches at slot_pos.
  * qkk_attn_decode: att[slot][h] = softmax(qhat[h] . K[0..pos] / sqrt(dh)) V[0..pos] * sigmoid(gate),
  *   K/V of KV head h / (hQ/hKV).  Every cache row is read once for the hQ/hKV heads that share it;
- *   positions are cut into 8..128 ranges that run in parallel and are folded in range order.  The
+ *   positions are cut into 8..64 ranges that run in parallel and are folded in range order.  The
  *   launch shape depends on the slot count and tmax only, so a captured graph stays valid as
  *   positions advance.
  *   workspace: qkk_attn_workspace_bytes(), 256-byte aligned, no initialisation needed. */

@@ -14,7 +14,7 @@
 // Attention is bound by reading the cache: 2 * hKV * n * dh * 4 bytes per slot.  The G = hQ/hKV
 // query heads that share a KV head are handled by ONE workgroup, so every K and V row is read once
 // for all of them, and the positions are cut into ranges that run in parallel (two KV heads alone
-// would leave 254 CUs idle; the host picks 8..128 ranges so that about a thousand workgroups
+// would leave 254 CUs idle; the host picks 8..64 ranges so that about two workgroups per CU
 // result); a second launch folds the ranges' (max, sum, accumulator) triples in range order.  Which
 // ranges hold keys is decided on the device from slot_pos, so the launch shape depends on the slot
 // count and tmax only and a captured graph stays valid as the sequences grow.
@@ -29,7 +29,7 @@
 namespace qk {
 
 constexpr uint32_t ATT_DH = 256;    // head size = workgroup size
-constexpr uint32_t ATT_MAX_RANGES = 128; // position ranges per (slot, KV head), at most
+constexpr uint32_t ATT_MAX_RANGES = 64; // position ranges per (slot, KV head), at most
 constexpr uint32_t ATT_TILE = 64;   // positions scored per pass
 constexpr uint32_t ATT_GMAX = 8;    // query heads per KV head
 constexpr float ATT_FLOOR = -3.4e38f;
@@ -360,8 +360,10 @@ int qkk_attn_decode(const float* qhat, const float* k_cache, const float* v_cach
                     qkk_attn_workspace_bytes(n_slots, hQ, dh));
     if (int rc = require_device()) return rc;
     hipStream_t st = as_stream(stream);
-    // about a thousand workgroups (four per CU) over the (slot, KV head) pairs, 8..128 ranges each
-    const uint32_t n_ranges = std::min(ATT_MAX_RANGES, std::max(8u, persistent_blocks() / (n_slots * hKV)));
+    // two workgroups per CU over the (slot, KV head) pairs, 8..64 ranges each: 16 slots x 4096 positions
+    // measured 4.5 TB/s with 16 ranges, 4.2 with 32, 3.1 with 128 (the partial results are traffic too);
+    // one slot 0.98 TB/s with 64 ranges, 0.80 with 32
+    const uint32_t n_ranges = std::min(ATT_MAX_RANGES, std::max(8u, persistent_blocks() / 2 / (n_slots * hKV)));
     AttnWs ws;
     ws.acc = (float*)workspace;
     ws.ml = ws.acc + (size_t)n_slots * hQ * n_ranges * ATT_DH;
