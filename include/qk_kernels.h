@@ -254,6 +254,33 @@ int qkk_attn_decode(const float *qhat, const float *k_cache, const float *v_cach
                     const uint32_t *slot_pos, float *att, void *workspace, size_t workspace_bytes,
                     uint32_t n_slots, uint32_t hQ, uint32_t hKV, uint32_t dh, uint32_t tmax, void *stream);
 
+/* ---- gated-DeltaNet mixer, decode step ----------------------------------------------------------
+ * (reference shaders/dn_ab.comp:20-50, dn_convn.comp:20-54, dn_step_gate.comp:26-81 = dn_step.comp
+ * + dn_gate.comp; host src/main.cpp:4200-4244; CPU mirror src/main.cpp:1704-1768.)  State size
+ * dS = 128; hK query/key heads, hV value heads; channels = (2*hK + hV) * dS, q heads first, then k,
+ * then v.
+ * qkk_dn_ab    gb[slot][h]      = a_vec[h] * softplus(alpha_w[h] . x[slot] + dt_bias[h])   (log decay)
+ *              gb[slot][hV + h] = sigmoid(beta_w[h] . x[slot])                             (write strength)
+ *              alpha_w, beta_w F32 [hV][n_embd]; n_embd 2048 or 4096.
+ * qkk_dn_conv  out[slot][ch] = silu(st0*ker[ch][0] + st1*ker[ch][1] + st2*ker[ch][2] + qkv[slot][ch]*ker[ch][3]),
+ *              conv_state [slots][channels][3] shifted (oldest first); the heads below qk_channels
+ *              are then scaled by 1 / max(|head|, eps).
+ * qkk_dn_step  per value head h, with kh = h / kdiv (kdiv = 0: h % hK, the reference's two pairings,
+ *              src/main.cpp:3092-3094), decay = exp(gb[h]), beta = gb[hV + h]:
+ *                sk_j = decay * sum_i S[j][i] k_i;  d_j = beta * (v_j - sk_j);
+ *                S[j][i] <- S[j][i] * decay + k_i * d_j;  o_j = sum_i S[j][i] q_i / sqrt(dS);
+ *                att[slot][h][j] = o_j / sqrt(mean_j o_j^2 + eps) * norm_w[j] * silu(z[slot][h][j])
+ *              state [slots][hV][dS][dS] fp32, COLUMN-major per head: element (row j, column i) at
+ *              [i][j] (a wave then reads consecutive floats; the reference keeps it row-major).
+ *              Bound by the state: dS*dS*4 bytes read and written per head. */
+int qkk_dn_ab(const float *x, const float *alpha_w, const float *beta_w, const float *dt_bias,
+              const float *a_vec, float *gb, uint32_t n_embd, uint32_t hV, uint32_t n_slots, void *stream);
+int qkk_dn_conv(float *conv_state, const float *qkv, const float *ker, float *out, uint32_t channels,
+                uint32_t d_state, uint32_t qk_channels, float eps, uint32_t n_slots, void *stream);
+int qkk_dn_step(const float *conv, const float *gb, float *state, const float *norm_w, const float *z,
+                float *att, uint32_t d_state, uint32_t hK, uint32_t hV, uint32_t kdiv, float eps,
+                uint32_t n_slots, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

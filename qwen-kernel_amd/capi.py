@@ -71,6 +71,9 @@ def lib():
         L.qkk_add_rms3.argtypes = [vp, vp, vp, vp, vp, vp, u32, u32, f32, vp]
         L.qkk_vec_add.argtypes = [vp, vp, vp, u64, vp]
         L.qkk_embed.argtypes = [C.c_int, vp, u32, u32, vp, u32, u32, u32, vp, u32, vp]
+        L.qkk_dn_ab.argtypes = [vp] * 6 + [u32] * 3 + [vp]
+        L.qkk_dn_conv.argtypes = [vp] * 4 + [u32] * 3 + [f32, u32, vp]
+        L.qkk_dn_step.argtypes = [vp] * 6 + [u32] * 4 + [f32, u32, vp]
         L.qkk_rope_table.argtypes = [vp, u32, u32, f32]
         L.qkk_attn_prep.argtypes = [vp] * 10 + [u32] * 6 + [f32, vp]
         L.qkk_attn_workspace_bytes.restype = sz
@@ -346,4 +349,39 @@ def attn_decode(qhat, k_cache, v_cache, qfull, slot_pos, workspace, att=None):
     _check(lib().qkk_attn_decode(_ptr(qhat), _ptr(k_cache), _ptr(v_cache), _ptr(qfull), _ptr(slot_pos), _ptr(att),
                                  _ptr(workspace), workspace.numel() * workspace.element_size(), n, hQ, hKV, dh, tmax,
                                  _stream()))
+    return att
+
+
+def dn_ab(x, alpha_w, beta_w, dt_bias, a_vec, gb=None):
+    """DeltaNet log decay and write strength: gb [slots][2*hV] (g first, then beta)."""
+    import torch
+    n, hV = x.shape[0], alpha_w.shape[0]
+    if gb is None:
+        gb = torch.empty((n, 2 * hV), dtype=torch.float32, device=x.device)
+    _check(lib().qkk_dn_ab(_ptr(x), _ptr(alpha_w), _ptr(beta_w), _ptr(dt_bias), _ptr(a_vec), _ptr(gb), x.shape[1], hV, n,
+                           _stream()))
+    return gb
+
+
+def dn_conv(conv_state, qkv, ker, qk_channels, d_state=128, eps=1e-6, out=None):
+    """Depthwise conv(4) + SiLU + window shift, q/k heads scaled to unit length.  conv_state
+    [slots][channels][3] is updated in place; returns out [slots][channels]."""
+    import torch
+    n, channels = qkv.shape
+    if out is None:
+        out = torch.empty_like(qkv)
+    _check(lib().qkk_dn_conv(_ptr(conv_state), _ptr(qkv), _ptr(ker), _ptr(out), channels, d_state, qk_channels, eps, n,
+                             _stream()))
+    return out
+
+
+def dn_step(conv, gb, state, norm_w, z, hK, hV, kdiv=0, d_state=128, eps=1e-6, att=None):
+    """Gated delta-rule update of state [slots][hV][dS][dS] (column-major per head, in place) and the
+    gated, normalised output att [slots][hV*dS]."""
+    import torch
+    n = conv.shape[0]
+    if att is None:
+        att = torch.empty((n, hV * d_state), dtype=torch.float32, device=conv.device)
+    _check(lib().qkk_dn_step(_ptr(conv), _ptr(gb), _ptr(state), _ptr(norm_w), _ptr(z), _ptr(att), d_state, hK, hV, kdiv,
+                             eps, n, _stream()))
     return att

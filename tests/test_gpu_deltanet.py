@@ -1,0 +1,108 @@
+"""The gated-DeltaNet decode step on the GPU (qkk_dn_ab, qkk_dn_conv, qkk_dn_step) against the
+restated CPU mirror in oracle/qk_oracle_deltanet.py, through the C ABI.  Tolerance 1e-3 relative
+max-abs as for the other fp32 kernels; the conv window is a copy and must be bit-exact."""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "oracle"))
+import qk_oracle_deltanet as OD  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+DS, HK, HV, NE = 128, 16, 32, 2048      # the reference's shape (src/main.cpp:3085)
+CH, QK = (2 * HK + HV) * DS, 2 * HK * DS
+F = np.float32
+TOL = 1e-3
+
+
+def rel(got, want):
+    return float(np.max(np.abs(got.astype(np.float64) - want)) / max(np.max(np.abs(want)), 1e-30))
+
+
+def rand(shape, seed, scale=1.0):
+    return (np.random.default_rng(seed).standard_normal(shape) * scale).astype(F)
+
+
+class Weights:
+    def __init__(self, seed, hk=HK, hv=HV, ne=NE):
+        self.hk, self.hv, self.ch, self.qk = hk, hv, (2 * hk + hv) * DS, 2 * hk * DS
+        self.alpha_w, self.beta_w = rand((hv, ne), seed, 0.03), rand((hv, ne), seed + 1, 0.03)
+        self.dt_bias, self.a_vec = rand(hv, seed + 2), -np.abs(rand(hv, seed + 3)) - F(0.05)
+        self.ker = rand((self.ch, 4), seed + 4, 0.5)
+        self.norm_w = (1 + 0.1 * rand(DS, seed + 5)).astype(F)
+
+
+def run_tokens(qk, dev, w, n_slots, n_tok, seed, kdiv=0, ne=NE):
+    """n_tok decode steps of n_slots independent slots on the GPU and in the oracle; returns the
+    worst relative errors per quantity and the final states."""
+    import torch
+    up = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    rng = np.random.default_rng(seed)
+    st = rng.standard_normal((n_slots, w.ch, 3)).astype(F)
+    S = (rng.standard_normal((n_slots, w.hv, DS, DS)) * 0.1).astype(F)          # row-major (row j, column i)
+    std, Sd = up(st), up(np.ascontiguousarray(S.transpose(0, 1, 3, 2)))          # device: column-major per head
+    wd = {k: up(getattr(w, k)) for k in ("alpha_w", "beta_w", "dt_bias", "a_vec", "ker", "norm_w")}
+    worst = dict(gb=0.0, conv=0.0, att=0.0)
+    for t in range(n_tok):
+        x = rng.standard_normal((n_slots, ne)).astype(F)
+        qkv = rng.standard_normal((n_slots, w.ch)).astype(F)
+        z = rng.standard_normal((n_slots, w.hv * DS)).astype(F)
+        gb = qk.dn_ab(up(x), wd["alpha_w"], wd["beta_w"], wd["dt_bias"], wd["a_vec"])
+        conv = qk.dn_conv(std, up(qkv), wd["ker"], w.qk)
+        att = qk.dn_step(conv, gb, Sd, wd["norm_w"], up(z), w.hk, w.hv, kdiv=kdiv)
+        torch.cuda.synchronize()
+        gb, conv, att = gb.cpu().numpy(), conv.cpu().numpy(), att.cpu().numpy()
+        for s in range(n_slots):
+            g, b = OD.ab(x[s], w.alpha_w, w.beta_w, w.dt_bias, w.a_vec)
+            c = OD.conv(st[s], qkv[s], w.ker, DS, w.qk)
+            a = OD.step(c, g, b, S[s], w.norm_w, z[s], w.hk, w.hv, kdiv=kdiv)
+            worst["gb"] = max(worst["gb"], rel(gb[s], np.concatenate([g, b])))
+            worst["conv"] = max(worst["conv"], rel(conv[s], c))
+            worst["att"] = max(worst["att"], rel(att[s], a))
+    return worst, std.cpu().numpy(), Sd.cpu().numpy().transpose(0, 1, 3, 2), st, S
+
+
+@pytest.mark.parametrize("n_slots,n_tok,kdiv", [(1, 6, 0), (3, 4, 2), (16, 2, 0)])
+def test_deltanet_steps_match_the_cpu_mirror(qk, dev, n_slots, n_tok, kdiv):
+    print(f"[case] deltanet slots={n_slots} tokens={n_tok} kdiv={kdiv}", flush=True)
+    worst, st_gpu, S_gpu, st, S = run_tokens(qk, dev, Weights(7), n_slots, n_tok, seed=n_slots + 10 * kdiv, kdiv=kdiv)
+    assert worst["gb"] <= 1e-5 and worst["conv"] <= 1e-5 and worst["att"] <= TOL, worst
+    assert np.array_equal(st_gpu, st)            # the conv window holds copies of the inputs
+    assert rel(S_gpu, S) <= TOL                  # the states after all tokens
+
+
+def test_deltanet_other_shapes(qk, dev):
+    """Fewer heads (1 key head for 2 value heads, both pairings) and n_embd = 4096."""
+    print("[case] deltanet other shapes", flush=True)
+    for hk, hv, kdiv, ne in ((1, 2, 0, 2048), (1, 2, 2, 2048), (4, 8, 2, 4096), (3, 3, 0, 2048)):
+        worst, st_gpu, S_gpu, st, S = run_tokens(qk, dev, Weights(9, hk, hv, ne), 2, 3, seed=hk + hv, kdiv=kdiv, ne=ne)
+        assert worst["gb"] <= 1e-5 and worst["conv"] <= 1e-5 and worst["att"] <= TOL, (hk, hv, kdiv, worst)
+        assert np.array_equal(st_gpu, st) and rel(S_gpu, S) <= TOL
+
+
+def test_deltanet_long_run_stays_on_the_oracle(qk, dev):
+    """Sixty tokens on one slot: the recurrent state does not drift away from the mirror."""
+    print("[case] deltanet sixty tokens", flush=True)
+    worst, _, S_gpu, _, S = run_tokens(qk, dev, Weights(11, 2, 4), 1, 60, seed=5)
+    assert worst["att"] <= TOL and rel(S_gpu, S) <= TOL, worst
+
+
+def test_deltanet_argument_checks(qk, dev):
+    import torch
+    z = lambda *s: torch.zeros(s, device=dev)
+    with pytest.raises(qk.QkError) as e:      # n_embd
+        qk.dn_ab(z(1, 1024), z(HV, 1024), z(HV, 1024), z(HV), z(HV))
+    assert e.value.code == -2
+    with pytest.raises(qk.QkError) as e:      # channels not whole heads
+        qk.dn_conv(z(1, 200, 3), z(1, 200), z(200, 4), 128)
+    assert e.value.code == -2
+    with pytest.raises(qk.QkError) as e:      # state size
+        qk.dn_step(z(1, CH), z(1, 2 * HV), z(1, HV, 64, 64), z(64), z(1, HV * 64), HK, HV, d_state=64)
+    assert e.value.code == -2
+    with pytest.raises(qk.QkError) as e:      # pairing beyond the key heads
+        qk.dn_step(z(1, (2 * 2 + 8) * DS), z(1, 16), z(1, 8, DS, DS), z(DS), z(1, 8 * DS), 2, 8, kdiv=2)
+    assert e.value.code == -2
