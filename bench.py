@@ -280,6 +280,43 @@ def attn_workload(qk, n_slots, ctx, steps, warmup, tmax=4096, seed=5):
     return dict(ms_event=ev, steps=n, ring=ring, bytes_step=2 * n_slots * hKV * ctx * dh * 4)
 
 
+def deltanet_workload(qk, n_slots, steps, warmup, seed=6):
+    """The gated-DeltaNet decode step (decay/beta dots, conv, state update + gated norm) of n_slots
+    slots at the reference's shape (32 value heads on 16 key heads, state 128 x 128 per head).  A
+    ring of distinct state sets (> 1 GB in all) stands for the DeltaNet layers of a model.  Bytes:
+    the states, read and written (2 * 32 * 128 * 128 * 4 B each way per slot)."""
+    import torch
+    dev = "cuda:0"
+    hK, hV, dS, ne = 16, 32, 128, 2048
+    ch, qkc = (2 * hK + hV) * dS, 2 * hK * dS
+    per_set = n_slots * hV * dS * dS * 4
+    ring = max(2, min(128, (1 << 30) // per_set + 1))
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    S = [torch.randn((n_slots, hV, dS, dS), device=dev, generator=g) * 0.1 for _ in range(ring)]
+    st = [torch.randn((n_slots, ch, 3), device=dev, generator=g) for _ in range(ring)]
+    x = torch.randn((ring, n_slots, ne), device=dev, generator=g)
+    qkv = torch.randn((ring, n_slots, ch), device=dev, generator=g)
+    z = torch.randn((ring, n_slots, hV * dS), device=dev, generator=g)
+    aw, bw = (torch.randn((hV, ne), device=dev, generator=g) * 0.03 for _ in range(2))
+    dt = torch.randn(hV, device=dev, generator=g)
+    av = -torch.rand(hV, device=dev, generator=g) - 0.05
+    ker = torch.randn((ch, 4), device=dev, generator=g) * 0.5
+    nw = torch.ones(dS, device=dev)
+    gb = torch.empty((ring, n_slots, 2 * hV), device=dev)
+    conv = torch.empty((ring, n_slots, ch), device=dev)
+    att = torch.empty((ring, n_slots, hV * dS), device=dev)
+
+    def step(i):
+        def f():
+            qk.dn_ab(x[i], aw, bw, dt, av, gb=gb[i])
+            qk.dn_conv(st[i], qkv[i], ker, qkc, out=conv[i])
+            qk.dn_step(conv[i], gb[i], S[i], nw, z[i], hK, hV, att=att[i])
+        return f
+    wall, ev, n = run_ring([step(i) for i in range(ring)], max(ring, steps // ring * ring), warmup)
+    return dict(ms_event=ev, steps=n, ring=ring, bytes_step=2 * n_slots * hV * dS * dS * 4)
+
+
 def engine_workload(qk, n_layer, slots_list, chunks, warm_chunks, seed=31):
     """Tokens per second through the engine ABI (qk_open / qk_slot_start / qk_step_chunk) on a
     synthetic MoE-only model file at the full layer shape and vocabulary: host wall clock over
@@ -386,6 +423,16 @@ def main():
         print(json.dumps(dict(metric="engine_decode_tok_per_s", value=r["slots_16"]["tok_per_s"], unit="tok/s", n_gpus=1,
                               higher_is_better=True, data="synthetic", dtype="f32",
                               config=dict(workload="engine_decode", **r["config"]), detail=r)), flush=True)
+        return
+    if a.workload in ("deltanet_bs1", "deltanet_bs16"):   # the gated-DeltaNet decode step alone
+        b = 1 if a.workload == "deltanet_bs1" else 16
+        dn = deltanet_workload(qk, b, min(a.steps, 512), min(a.warmup, 64))
+        gb = dn["bytes_step"] / (dn["ms_event"] * 1e-3) / 1e9
+        print(json.dumps(dict(metric="deltanet_decode_hbm_gbps", value=gb, unit="GB/s", n_gpus=1, steps=dn["steps"],
+                              ms_per_step=dn["ms_event"], higher_is_better=True, data="synthetic", dtype="f32",
+                              config=dict(workload=a.workload, slots=b, heads="32 value heads on 16 key heads, state 128 x 128",
+                                          ring=dn["ring"]),
+                              bytes_per_step=dn["bytes_step"], frac_of_hbm_peak=gb / HBM_PEAK_GBPS)), flush=True)
         return
     if a.workload in ("attn_bs1", "attn_bs16"):   # the attention decode step alone
         b = 1 if a.workload == "attn_bs1" else 16
@@ -519,6 +566,12 @@ def main():
                                                         ring=at["ring"])
                 torch.cuda.empty_cache()
             log(f"[bench] attention: {ex['attn_decode_ctx4096_bs1']} {ex['attn_decode_ctx4096_bs16']}")
+            for b in (1, 16):   # the gated-DeltaNet mixer's decode step
+                dn = deltanet_workload(qk, b, 256, 32)
+                gb = dn["bytes_step"] / (dn["ms_event"] * 1e-3) / 1e9
+                ex[f"deltanet_decode_bs{b}"] = dict(us=dn["ms_event"] * 1e3, gbps=gb, frac=gb / HBM_PEAK_GBPS, ring=dn["ring"])
+                torch.cuda.empty_cache()
+            log(f"[bench] deltanet: {ex['deltanet_decode_bs1']} {ex['deltanet_decode_bs16']}")
             ex["engine_decode_8_layers"] = engine_workload(qk, 8, (1, 4, 16), 8, 2)
             log(f"[bench] engine: {ex['engine_decode_8_layers']}")
         out["extras"] = ex
