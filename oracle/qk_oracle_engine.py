@@ -25,7 +25,14 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 
 
 class SlotMachine:
+    """nxt: a function (token, dispatch depth) -> next token for a model without memory, or an object
+    with reset(slot) and feed(slot, token, position, depth) -> next token for one with per-slot state
+    (the positions [0, done) that qk_slot_start prefills are fed at the start, reference
+    src/main.cpp:5470-5500; a step feeds prompt[cursor] at position cursor or the last sample at
+    pos, :4563-4573)."""
+
     def __init__(self, nxt, vocab, eos, n_slots, n_ctx, chunk, max_b=128, no_batch=False):
+        self.model = nxt if hasattr(nxt, "feed") else None
         self.nxt, self.vocab, self.eos = nxt, vocab, eos
         self.n_slots, self.n_ctx, self.chunk, self.max_b, self.no_batch = n_slots, n_ctx, chunk, max_b, no_batch
         self.slots = [dict(active=False) for _ in range(n_slots)]
@@ -52,6 +59,10 @@ class SlotMachine:
             if snap_at:
                 batch_to(snap_at)
             batch_to(target)
+        if self.model:
+            self.model.reset(slot)
+            for p in range(done):
+                self.model.feed(slot, prompt[p], p, 1)
         self.slots[slot] = dict(active=True, prompt=list(prompt), cursor=done, pos=done, last=0, gen=0, max_gen=max_gen)
         return 0
 
@@ -67,17 +78,17 @@ class SlotMachine:
         if not active_at_entry:
             return 0, out, 0
         for _ in range(self.chunk):
-            n_act, max_z, need, fed = 0, 0, False, {}
+            n_act, max_z, need, fed, at = 0, 0, False, {}, {}
             for s, sl in enumerate(self.slots):
                 if not sl["active"]:
                     continue
                 n_act += 1
                 max_z = s + 1
                 if sl["cursor"] < len(sl["prompt"]):
-                    fed[s] = sl["prompt"][sl["cursor"]]
+                    fed[s], at[s] = sl["prompt"][sl["cursor"]], sl["cursor"]
                     need = True
                 else:
-                    fed[s] = sl["last"]
+                    fed[s], at[s] = sl["last"], sl["pos"]
                     if len(out[s]) < self.chunk:
                         need = True
             if not n_act or not need:
@@ -86,7 +97,7 @@ class SlotMachine:
             for s, sl in enumerate(self.slots):
                 if not sl["active"]:
                     continue
-                sampled = self.nxt(fed[s], max_z)
+                sampled = self.model.feed(s, fed[s], at[s], max_z) if self.model else self.nxt(fed[s], max_z)
                 prefilling = sl["cursor"] < len(sl["prompt"])
                 if prefilling and sl["cursor"] + 1 < len(sl["prompt"]):
                     sl["cursor"] += 1
@@ -172,3 +183,58 @@ class Stub:
         rc = self.L.qk_step_chunk(self.h, self._tok, self._cnt, C.byref(self._fin))
         out = {s: [self._tok[s * self.chunk + i] for i in range(self._cnt[s])] for s in range(self.n_slots)}
         return rc, out, self._fin.value
+
+
+class FullModelOracle:
+    """The decode step of a whole model (mixer + MoE block per layer) with per-slot state, from the
+    oracle's pieces, following the reference's recorded step (src/main.cpp:4194-4419): an object with
+    the fields of qwen-kernel_amd's engine.FullModel.  feed() returns the greedy next token and
+    records the top-2 logit gap and the largest logit of the step in .last_margin."""
+
+    def __init__(self, model, n_slots, n_ctx, kdiv=0, eps=1e-6):
+        import qk_oracle_attn as OA
+        import qk_oracle_deltanet as OD
+        self.OA, self.OD, self.m, self.n_ctx, self.kdiv, self.eps = OA, OD, model, n_ctx, kdiv, eps
+        self.rope = OA.rope_table(n_ctx, model.FA["n_rot"])
+        self.state = [None] * n_slots
+        self.last_margin = None
+        for s in range(n_slots):
+            self.reset(s)
+
+    def reset(self, slot):
+        d, a = self.m.DN, self.m.FA
+        st = []
+        for mix in self.m.mix:
+            if mix["kind"] == "R":
+                st.append([np.zeros((d["ch"], 3), np.float32), np.zeros((d["hv"], d["ds"], d["ds"]), np.float32)])
+            else:
+                st.append([np.zeros((a["hkv"], self.n_ctx, a["dh"]), np.float32), np.zeros((a["hkv"], self.n_ctx, a["dh"]), np.float32)])
+        self.state[slot] = st
+
+    def feed(self, slot, token, pos, depth=1):
+        m, d, a, eps, H = self.m, self.m.DN, self.m.FA, self.eps, 2048
+        x = O.embed(m.embd_type, m.embd, m.vocab, H, np.array([token], dtype=np.uint32), 0, 1, 1)[0]
+        for l, mix in enumerate(m.mix):
+            st = self.state[slot][l]
+            xn = O.add_rms(x, m.attn_norm[l], eps)
+            if mix["kind"] == "R":
+                qkv = O.gemv(O.Q8_0, mix["qkv"], xn, d["ch"], H)
+                z = O.gemv(O.Q8_0, mix["gate"], xn, d["d_in"], H)
+                g, b = self.OD.ab(xn, mix["alpha"], mix["beta"], mix["dt"], mix["a"])
+                c = self.OD.conv(st[0], qkv, mix["ker"], d["ds"], 2 * d["hk"] * d["ds"], eps)
+                att = self.OD.step(c, g, b, st[1], mix["norm"], z, d["hk"], d["hv"], kdiv=self.kdiv, eps=eps)
+                mixed = O.gemv(O.Q8_0, mix["out"], att, H, d["d_in"])
+            else:
+                qfull = O.gemv(O.Q8_0, mix["q"], xn, a["hq"] * 2 * a["dh"], H).reshape(a["hq"], 2 * a["dh"])
+                kin = O.gemv(O.Q8_0, mix["k"], xn, a["hkv"] * a["dh"], H).reshape(a["hkv"], a["dh"])
+                vin = O.gemv(O.Q8_0, mix["v"], xn, a["hkv"] * a["dh"], H).reshape(a["hkv"], a["dh"])
+                qhat = self.OA.prep(qfull, kin, vin, mix["qn"], mix["kn"], self.rope, pos, st[0], st[1], a["n_rot"], eps)
+                att = self.OA.attend(qhat, st[0], st[1], qfull, pos).reshape(-1)
+                mixed = O.gemv(O.Q8_0, mix["out"], att, H, a["hq"] * a["dh"])
+            y = (x + mixed).astype(np.float32)
+            xn2 = O.add_rms(y, m.post_norm[l], eps)
+            x = (y + O.moe_ref(m.layers[l], xn2)["y"]).astype(np.float32)
+        logits = O.gemv(O.Q6_K, m.head, O.add_rms(x, m.out_norm, eps), m.vocab, H)
+        srt = np.sort(logits.astype(np.float64))
+        self.last_margin = (float(srt[-1] - srt[-2]), float(np.abs(logits).max()))
+        return O.argmax(logits)

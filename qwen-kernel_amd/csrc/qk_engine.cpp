@@ -34,9 +34,29 @@ constexpr uint32_t MAX_ROWS = QKK_MAX_SLOTS; // rows one device step carries
 constexpr uint32_t N_STATE = 3;             // snapshot entries (reference default, stub/qk_stub.c:98)
 constexpr int ERR_DEVICE = -6;              // a launch, copy or synchronisation failed
 
+// The mixers' shapes are fixed, as in the reference engine (src/main.cpp:3085-3090).
+constexpr uint32_t DN_CH = 8192, DN_IN = 4096, DN_HV = 32, DN_DS = 128, DN_HK = 16; // gated DeltaNet
+constexpr uint32_t FA_DH = 256, FA_HQ = 16, FA_HKV = 2, FA_ROT = 64;                // full attention
+constexpr float FA_FREQ_BASE = 1e7f;                                                // src/main.cpp:1872
+
+struct Dense { // a Q8_0 / IQ4_XS projection [M][K]
+    const void* w = nullptr;
+    int type = 0;
+    uint32_t M = 0, K = 0;
+};
+
 struct EngineLayer {
+    enum Kind { MOE_ONLY, RECURRENT, ATTENTION };
+    Kind kind = MOE_ONLY;
     qkk_moe_layer moe;
-    const float* post_norm; // blk.l.post_attention_norm.weight
+    const float* post_norm = nullptr; // blk.l.post_attention_norm.weight
+    const float* attn_norm = nullptr; // blk.l.attn_norm.weight (layers with a mixer)
+    Dense p1, p2, p3, out;            // recurrent: attn_qkv, attn_gate, -, ssm_out; attention: attn_q, attn_k, attn_v, attn_output
+    const float *alpha_w = nullptr, *beta_w = nullptr, *dt_bias = nullptr, *a_vec = nullptr, *ker = nullptr,
+                *ssm_norm = nullptr;                  // recurrent
+    const float *q_norm = nullptr, *k_norm = nullptr; // attention
+    float *st1 = nullptr, *st2 = nullptr; // per-slot state: recurrent conv window + delta-rule state; attention K + V cache
+    size_t ps1 = 0, ps2 = 0;              // floats per slot of st1 / st2
 };
 
 } // namespace
@@ -72,6 +92,17 @@ struct qk_engine {
     uint32_t* h_tok = nullptr; // pinned, [MAX_ROWS]
     std::vector<hipGraphExec_t> graphs; // [depth - 1], empty when graphs are switched off
     uint32_t last_run_rows = 0;
+    // whole-model files (layers with mixers)
+    bool full_model = false;
+    uint32_t dn_kdiv = 0;        // 0: value head h reads key head h % hK; else h / dn_kdiv (src/main.cpp:3092-3094)
+    uint32_t* d_pos = nullptr;   // [MAX_ROWS] position of the token fed this step
+    uint32_t* h_pos = nullptr;   // pinned
+    float* d_rope = nullptr;     // [n_ctx][FA_ROT/2][2]
+    float *d_big = nullptr, *d_mid = nullptr, *d_kin = nullptr, *d_vin = nullptr, *d_gb = nullptr, *d_conv = nullptr,
+          *d_qhat = nullptr, *d_att = nullptr, *d_mix = nullptr; // per-step rows of the mixers
+    void* d_aws = nullptr;       // attention workspace
+    size_t aws_bytes = 0;
+    std::vector<std::vector<float*>> snaps; // [N_STATE][2 * layer]: one slot's state stripes
 
     // host side (reference src/main.cpp:3153-3175, Slot)
     struct Slot {
@@ -86,6 +117,11 @@ struct qk_engine {
     bool upload(const qkg_tensor& t, const void** out, char* err, size_t err_len);
     void* dev_alloc(size_t bytes, bool zero);
     int launch_rows(uint32_t rows, float** final_rows);
+    int launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool want_head);
+    int feed_one(uint32_t slot, uint32_t tok, uint32_t pos, bool want_head);
+    int reset_slot(uint32_t slot);
+    bool load_mixers(qkg_file* g, char* err, size_t err_len);
+    int copy_state(uint32_t slot, uint32_t idx, bool save, uint32_t n_tok);
     int run_rows(uint32_t rows, bool graph_ok);
     int copy_and_launch(uint32_t rows);
     int step_chunk(uint32_t* out_tok, uint32_t* out_cnt, uint32_t* out_fin);
@@ -109,6 +145,7 @@ qk_engine::~qk_engine()
     for (void* p : dev_allocs) (void)hipFree(p);
     if (h_ids) (void)hipHostFree(h_ids);
     if (h_tok) (void)hipHostFree(h_tok);
+    if (h_pos) (void)hipHostFree(h_pos);
     if (st) (void)hipStreamDestroy(st);
 }
 
@@ -163,6 +200,86 @@ int qk_engine::launch_rows(uint32_t rows, float** final_rows)
     return qkk_head_argmax(d_head, d_xn[cur], d_tok, nullptr, vocab, N_EMBD, rows, d_hws, hws_bytes, st);
 }
 
+static int dense(const Dense& d, const float* x, float* y, uint32_t rows, hipStream_t st)
+{
+    return qkk_gemv(d.type, d.w, x, y, d.M, d.K, rows, st);
+}
+
+// The launches of one step of a whole model over the slots [s0, s0 + rows): d_ids / d_pos -> d_tok
+// (reference src/main.cpp:4194-4419).  Every per-slot buffer is indexed from s0, so a single slot
+// can be stepped alone (batch prefill of a starting request, qk_stage_run) while the others rest.
+int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool want_head)
+{
+    if (rows < 1 || s0 + rows > MAX_ROWS) return QKK_ESHAPE;
+    float* x = d_x + (size_t)s0 * N_EMBD;
+    const uint32_t* pos = d_pos + s0;
+    if (int rc = qkk_embed(embd_type, d_embd, embd_rows, N_EMBD, d_ids, MAX_ROWS, s0, 1, x, rows, st)) return rc;
+    if (int rc = qkk_rmsnorm(x, layers[0].attn_norm, d_xn[0], N_EMBD, rows, eps, st)) return rc;
+    int cur = 0;
+    for (size_t l = 0; l < layers.size(); l++) {
+        const EngineLayer& L = layers[l];
+        float* xn = d_xn[cur];
+        if (L.kind == EngineLayer::RECURRENT) {
+            if (int rc = dense(L.p1, xn, d_big, rows, st)) return rc;
+            if (int rc = dense(L.p2, xn, d_mid, rows, st)) return rc;
+            if (int rc = qkk_dn_ab(xn, L.alpha_w, L.beta_w, L.dt_bias, L.a_vec, d_gb, N_EMBD, DN_HV, rows, st)) return rc;
+            if (int rc = qkk_dn_conv(L.st1 + s0 * L.ps1, d_big, L.ker, d_conv, DN_CH, DN_DS, 2 * DN_HK * DN_DS, eps, rows, st))
+                return rc;
+            if (int rc = qkk_dn_step(d_conv, d_gb, L.st2 + s0 * L.ps2, L.ssm_norm, d_mid, d_att, DN_DS, DN_HK, DN_HV, dn_kdiv,
+                                     eps, rows, st))
+                return rc;
+        } else {
+            if (int rc = dense(L.p1, xn, d_big, rows, st)) return rc;
+            if (int rc = dense(L.p2, xn, d_kin, rows, st)) return rc;
+            if (int rc = dense(L.p3, xn, d_vin, rows, st)) return rc;
+            if (int rc = qkk_attn_prep(d_big, d_kin, d_vin, L.q_norm, L.k_norm, d_rope, pos, d_qhat, L.st1 + s0 * L.ps1,
+                                       L.st2 + s0 * L.ps2, rows, FA_HQ, FA_HKV, FA_DH, FA_ROT, n_ctx, eps, st))
+                return rc;
+            if (int rc = qkk_attn_decode(d_qhat, L.st1 + s0 * L.ps1, L.st2 + s0 * L.ps2, d_big, pos, d_att, d_aws, aws_bytes,
+                                         rows, FA_HQ, FA_HKV, FA_DH, n_ctx, st))
+                return rc;
+        }
+        if (int rc = dense(L.out, d_att, d_mix, rows, st)) return rc;
+        // y = x + mixer, normalised for the MoE block; then x = y + MoE, normalised for the next layer
+        if (int rc = qkk_add_rmsnorm(x, d_mix, L.post_norm, x, xn, N_EMBD, rows, eps, st)) return rc;
+        const float* w_next = l + 1 < layers.size() ? layers[l + 1].attn_norm : d_onorm;
+        if (int rc = qkk_moe_decode_tail(&L.moe, xn, x, w_next, eps, x, d_xn[cur ^ 1], d_sel, d_ws, ws_bytes, rows, st))
+            return rc;
+        cur ^= 1;
+    }
+    if (final_rows) *final_rows = d_xn[cur];
+    if (!want_head) return QKK_OK;
+    return qkk_head_argmax(d_head, d_xn[cur], d_tok + s0, nullptr, vocab, N_EMBD, rows, d_hws, hws_bytes, st);
+}
+
+// Clears a slot's recurrent state (reference resetSlot, src/main.cpp:3416-3433); the KV rows of an
+// attention layer are overwritten as the positions are fed.
+int qk_engine::reset_slot(uint32_t slot)
+{
+    for (const EngineLayer& L : layers)
+        if (L.kind == EngineLayer::RECURRENT &&
+            (hipMemsetAsync(L.st1 + slot * L.ps1, 0, L.ps1 * sizeof(float), st) != hipSuccess ||
+             hipMemsetAsync(L.st2 + slot * L.ps2, 0, L.ps2 * sizeof(float), st) != hipSuccess))
+            return ERR_DEVICE;
+    return hipStreamSynchronize(st) == hipSuccess ? 0 : ERR_DEVICE;
+}
+
+// One token of one slot, alone, eagerly (the other slots' states are not touched).
+int qk_engine::feed_one(uint32_t slot, uint32_t tok, uint32_t pos, bool want_head)
+{
+    h_ids[slot] = tok;
+    h_pos[slot] = pos;
+    if (hipMemcpyAsync(d_ids + slot, h_ids + slot, 4, hipMemcpyHostToDevice, st) != hipSuccess ||
+        hipMemcpyAsync(d_pos + slot, h_pos + slot, 4, hipMemcpyHostToDevice, st) != hipSuccess)
+        return ERR_DEVICE;
+    float* fin = nullptr;
+    if (launch_full(1, slot, &fin, want_head) != QKK_OK) return ERR_DEVICE;
+    if (want_head && (hipMemcpyAsync(h_tok + slot, d_tok + slot, 4, hipMemcpyDeviceToHost, st) != hipSuccess ||
+                      hipMemcpyAsync(d_last, fin, N_EMBD * sizeof(float), hipMemcpyDeviceToDevice, st) != hipSuccess))
+        return ERR_DEVICE;
+    return hipStreamSynchronize(st) == hipSuccess ? 0 : ERR_DEVICE;
+}
+
 // One device step: h_ids[0..rows) in, h_tok[0..rows) out, host blocked until it is done.  A
 // captured step holds the two copies as well, so a replay is one launch and one wait.
 int qk_engine::run_rows(uint32_t rows, bool graph_ok)
@@ -180,10 +297,120 @@ int qk_engine::copy_and_launch(uint32_t rows)
 {
     if (hipMemcpyAsync(d_ids, h_ids, rows * sizeof(uint32_t), hipMemcpyHostToDevice, st) != hipSuccess)
         return ERR_DEVICE;
-    if (launch_rows(rows, nullptr) != QKK_OK) return ERR_DEVICE;
+    if (full_model) {
+        if (hipMemcpyAsync(d_pos, h_pos, rows * sizeof(uint32_t), hipMemcpyHostToDevice, st) != hipSuccess)
+            return ERR_DEVICE;
+        if (launch_full(rows, 0, nullptr, true) != QKK_OK) return ERR_DEVICE;
+    } else if (launch_rows(rows, nullptr) != QKK_OK) {
+        return ERR_DEVICE;
+    }
     if (hipMemcpyAsync(h_tok, d_tok, rows * sizeof(uint32_t), hipMemcpyDeviceToHost, st) != hipSuccess)
         return ERR_DEVICE;
     return 0;
+}
+
+// The mixers of a whole-model file (reference src/main.cpp:3916-4010): tensors, per-slot state
+// stripes, the step's scratch rows, the RoPE table.  Shapes are the reference's fixed ones.
+bool qk_engine::load_mixers(qkg_file* g, char* err, size_t err_len)
+{
+    auto bad = [&](const char* m) { return set_err(err, err_len, m); };
+    auto find = [&](uint32_t l, const char* suffix, qkg_tensor* t) {
+        char name[96];
+        snprintf(name, sizeof name, "blk.%u.%s", l, suffix);
+        return qkg_find(g, name, t) == 0;
+    };
+    auto f32 = [&](uint32_t l, const char* suffix, uint64_t n_elems, const float** out) {
+        qkg_tensor t;
+        const void* p = nullptr;
+        if (!find(l, suffix, &t) || t.type != QKK_F32 || t.nbytes != n_elems * 4) return false;
+        if (!upload(t, &p, err, err_len)) return false;
+        *out = (const float*)p;
+        return true;
+    };
+    auto proj = [&](uint32_t l, const char* suffix, uint32_t K, uint32_t M, Dense* d) {
+        qkg_tensor t;
+        if (!find(l, suffix, &t) || (t.type != QKK_Q8_0 && t.type != QKK_IQ4_XS) || t.ne[0] != K || t.ne[1] != M || !t.nbytes)
+            return false;
+        d->type = (int)t.type; d->M = M; d->K = K;
+        return upload(t, &d->w, err, err_len);
+    };
+    for (uint32_t l = 0; l < n_layer; l++) {
+        EngineLayer& L = layers[l];
+        if (!f32(l, "attn_norm.weight", N_EMBD, &L.attn_norm)) return bad("qk_open: missing/unexpected attn_norm tensor");
+        if (L.kind == EngineLayer::RECURRENT) {
+            if (!proj(l, "attn_qkv.weight", N_EMBD, DN_CH, &L.p1) || !proj(l, "attn_gate.weight", N_EMBD, DN_IN, &L.p2) ||
+                !proj(l, "ssm_out.weight", DN_IN, N_EMBD, &L.out))
+                return bad("qk_open: gated-DeltaNet projections missing or of an unsupported type / shape");
+            if (!f32(l, "ssm_alpha.weight", (uint64_t)DN_HV * N_EMBD, &L.alpha_w) ||
+                !f32(l, "ssm_beta.weight", (uint64_t)DN_HV * N_EMBD, &L.beta_w))
+                return bad("qk_open: missing ssm_alpha/ssm_beta (the fused ssm_ba form is not supported)");
+            if (!f32(l, "ssm_dt.bias", DN_HV, &L.dt_bias) || !f32(l, "ssm_a", DN_HV, &L.a_vec) ||
+                !(f32(l, "ssm_conv1d.weight", (uint64_t)DN_CH * 4, &L.ker) || f32(l, "ssm_conv1d", (uint64_t)DN_CH * 4, &L.ker)) ||
+                !f32(l, "ssm_norm.weight", DN_DS, &L.ssm_norm))
+                return bad("qk_open: gated-DeltaNet tensors missing or of an unexpected shape");
+            L.ps1 = (size_t)DN_CH * 3;
+            L.ps2 = (size_t)DN_HV * DN_DS * DN_DS;
+        } else {
+            if (!proj(l, "attn_q.weight", N_EMBD, FA_HQ * 2 * FA_DH, &L.p1) || !proj(l, "attn_k.weight", N_EMBD, FA_HKV * FA_DH, &L.p2) ||
+                !proj(l, "attn_v.weight", N_EMBD, FA_HKV * FA_DH, &L.p3) || !proj(l, "attn_output.weight", FA_HQ * FA_DH, N_EMBD, &L.out))
+                return bad("qk_open: attention projections missing or of an unsupported type / shape");
+            if (!f32(l, "attn_q_norm.weight", FA_DH, &L.q_norm) || !f32(l, "attn_k_norm.weight", FA_DH, &L.k_norm))
+                return bad("qk_open: attention norm tensors missing or of an unexpected shape");
+            L.ps1 = L.ps2 = (size_t)FA_HKV * n_ctx * FA_DH;
+        }
+        L.st1 = (float*)dev_alloc(MAX_ROWS * L.ps1 * sizeof(float), true);
+        L.st2 = (float*)dev_alloc(MAX_ROWS * L.ps2 * sizeof(float), true);
+        if (!L.st1 || !L.st2) return bad("qk_open: device memory exhausted (per-slot state)");
+    }
+    auto rows_of = [&](size_t n) { return (float*)dev_alloc(MAX_ROWS * n * sizeof(float), true); };
+    d_big = rows_of(DN_CH); d_mid = rows_of(DN_IN); d_kin = rows_of(FA_HKV * FA_DH); d_vin = rows_of(FA_HKV * FA_DH);
+    d_gb = rows_of(2 * DN_HV); d_conv = rows_of(DN_CH); d_qhat = rows_of(FA_HQ * FA_DH); d_att = rows_of(DN_IN);
+    d_mix = rows_of(N_EMBD);
+    d_pos = (uint32_t*)dev_alloc(MAX_ROWS * 4, true);
+    aws_bytes = qkk_attn_workspace_bytes(MAX_ROWS, FA_HQ, FA_DH);
+    d_aws = dev_alloc(aws_bytes, true);
+    d_rope = (float*)dev_alloc((size_t)n_ctx * FA_ROT * sizeof(float), false);
+    if (!d_big || !d_mid || !d_kin || !d_vin || !d_gb || !d_conv || !d_qhat || !d_att || !d_mix || !d_pos || !d_aws || !d_rope)
+        return bad("qk_open: device memory exhausted");
+    std::vector<float> rope((size_t)n_ctx * FA_ROT);
+    if (qkk_rope_table(rope.data(), n_ctx, FA_ROT, FA_FREQ_BASE) != QKK_OK ||
+        hipMemcpy(d_rope, rope.data(), rope.size() * sizeof(float), hipMemcpyHostToDevice) != hipSuccess)
+        return bad("qk_open: upload failed");
+    // snapshot entries: one slot's state stripes each (reference src/main.cpp:3435-3487, copyStripes)
+    snaps.assign(N_STATE, std::vector<float*>(2 * n_layer, nullptr));
+    for (auto& sn : snaps)
+        for (uint32_t l = 0; l < n_layer; l++) {
+            sn[2 * l] = (float*)dev_alloc(layers[l].ps1 * sizeof(float), true);
+            sn[2 * l + 1] = (float*)dev_alloc(layers[l].ps2 * sizeof(float), true);
+            if (!sn[2 * l] || !sn[2 * l + 1]) return bad("qk_open: device memory exhausted (snapshots)");
+        }
+    return true;
+}
+
+// Saves a slot's state stripes into snapshot idx, or loads them back.  Of an attention layer's caches
+// only the first n_tok positions travel (all of them when n_tok is 0 or beyond n_ctx).
+int qk_engine::copy_state(uint32_t slot, uint32_t idx, bool save, uint32_t n_tok)
+{
+    const uint32_t keep = n_tok == 0 || n_tok > n_ctx ? n_ctx : n_tok;
+    for (uint32_t l = 0; l < n_layer; l++) {
+        const EngineLayer& L = layers[l];
+        float* live[2] = {L.st1 + slot * L.ps1, L.st2 + slot * L.ps2};
+        for (int k = 0; k < 2; k++) {
+            float* snap = snaps[idx][2 * l + k];
+            if (L.kind == EngineLayer::ATTENTION) { // [hKV][n_ctx][dh]: the first `keep` rows of every KV head
+                for (uint32_t h = 0; h < FA_HKV; h++) {
+                    const size_t off = (size_t)h * n_ctx * FA_DH, n = (size_t)keep * FA_DH * sizeof(float);
+                    if (hipMemcpyAsync(save ? snap + off : live[k] + off, save ? live[k] + off : snap + off, n,
+                                       hipMemcpyDeviceToDevice, st) != hipSuccess)
+                        return ERR_DEVICE;
+                }
+            } else if (hipMemcpyAsync(save ? snap : live[k], save ? live[k] : snap, (k ? L.ps2 : L.ps1) * sizeof(float),
+                                      hipMemcpyDeviceToDevice, st) != hipSuccess) {
+                return ERR_DEVICE;
+            }
+        }
+    }
+    return hipStreamSynchronize(st) == hipSuccess ? 0 : ERR_DEVICE;
 }
 
 bool qk_engine::open(const char* path, const qk_config& cfg, char* err, size_t err_len)
@@ -242,18 +469,26 @@ bool qk_engine::open(const char* path, const qk_config& cfg, char* err, size_t e
     embd_rows = (uint32_t)t_embd.ne[1];
     vocab = (uint32_t)t_head.ne[1];
 
-    // the layers: MoE tensor sets (reference src/main.cpp:3611-3622, 1265-1311) and no mixer
+    // the layers: MoE tensor sets (reference src/main.cpp:3611-3622, 1265-1311); with mixers (a
+    // whole-model file: "ssm_a" marks a gated-DeltaNet layer, src/main.cpp:3919) or without any
     std::vector<qkg_moe_tensors> mt(n_layer);
     std::vector<qkg_tensor> pn(n_layer);
+    std::vector<EngineLayer::Kind> kinds(n_layer, EngineLayer::MOE_ONLY);
+    dn_kdiv = arch == "qwen3next" ? DN_HV / DN_HK : 0; // reference src/main.cpp:3588
     for (uint32_t l = 0; l < n_layer; l++) {
         char name[96];
-        for (const char* mixer : {"attn_qkv.weight", "attn_q.weight", "attn_output.weight", "ssm_out.weight"}) {
-            snprintf(name, sizeof name, "blk.%u.%s", l, mixer);
-            qkg_tensor tmp;
-            if (qkg_find(g, name, &tmp) == 0)
-                return bad("qk_open: this libqk.so implements the quantized decode hot path only (see qk_kernels.h); "
-                           "the attention / gated-DeltaNet mixers this file's layers need are not part of it");
-        }
+        qkg_tensor tmp;
+        snprintf(name, sizeof name, "blk.%u.ssm_a", l);
+        if (qkg_find(g, name, &tmp) == 0) kinds[l] = EngineLayer::RECURRENT;
+        snprintf(name, sizeof name, "blk.%u.attn_q.weight", l);
+        if (kinds[l] == EngineLayer::MOE_ONLY && qkg_find(g, name, &tmp) == 0) kinds[l] = EngineLayer::ATTENTION;
+        if (kinds[l] == EngineLayer::MOE_ONLY)
+            for (const char* mixer : {"attn_qkv.weight", "attn_output.weight", "ssm_out.weight"}) {
+                snprintf(name, sizeof name, "blk.%u.%s", l, mixer);
+                if (qkg_find(g, name, &tmp) == 0) return bad("qk_open: a layer has mixer tensors but neither ssm_a nor attn_q");
+            }
+        if ((kinds[l] == EngineLayer::MOE_ONLY) != (kinds[0] == EngineLayer::MOE_ONLY))
+            return bad("qk_open: layers with and without mixers in one file");
         if (qkg_moe_layer(g, l, &mt[l]) != 0) {
             if (err && err_len) snprintf(err, err_len, "qk_open: %s", qkk_last_error());
             return false;
@@ -285,7 +520,9 @@ bool qk_engine::open(const char* path, const qk_config& cfg, char* err, size_t e
         return false;
     d_onorm = (const float*)p;
     layers.resize(n_layer);
+    full_model = kinds[0] != EngineLayer::MOE_ONLY;
     for (uint32_t l = 0; l < n_layer; l++) {
+        layers[l].kind = kinds[l];
         qkk_moe_layer& m = layers[l].moe;
         m.n_embd = mt[l].n_embd; m.n_ff = mt[l].n_ff; m.n_expert = mt[l].n_expert; m.n_used = mt[l].n_used;
         m.gu_type = mt[l].gu_type; m.down_type = mt[l].down_type;
@@ -318,10 +555,13 @@ bool qk_engine::open(const char* path, const qk_config& cfg, char* err, size_t e
     if (!d_ids || !d_tok || !d_x || !d_xn[0] || !d_xn[1] || !d_last || !d_logits || !d_sel || !d_ws || !d_hws)
         return bad("qk_open: device memory exhausted");
     if (hipHostMalloc((void**)&h_ids, MAX_ROWS * 4, hipHostMallocDefault) != hipSuccess ||
-        hipHostMalloc((void**)&h_tok, MAX_ROWS * 4, hipHostMallocDefault) != hipSuccess)
+        hipHostMalloc((void**)&h_tok, MAX_ROWS * 4, hipHostMallocDefault) != hipSuccess ||
+        hipHostMalloc((void**)&h_pos, MAX_ROWS * 4, hipHostMallocDefault) != hipSuccess)
         return bad("qk_open: cannot allocate pinned memory");
     memset(h_ids, 0, MAX_ROWS * 4);
     memset(h_tok, 0, MAX_ROWS * 4);
+    memset(h_pos, 0, MAX_ROWS * 4);
+    if (full_model && !load_mixers(g, err, err_len)) return false;
     if (hipDeviceSynchronize() != hipSuccess) return bad("qk_open: upload failed"); // fills and uploads are complete
 
     // One graph per dispatch depth z = highest active slot + 1 (the reference records one
@@ -348,6 +588,9 @@ bool qk_engine::open(const char* path, const qk_config& cfg, char* err, size_t e
         (void)hipGraphDestroy(graph);
         if (ei != hipSuccess) { graphs[z - 1] = nullptr; return bad("qk_open: graph instantiation failed"); }
     }
+    if (full_model) // the warm-up steps above fed token 0 to every slot
+        for (uint32_t sl = 0; sl < n_slots; sl++)
+            if (reset_slot(sl) != 0) return bad("qk_open: device step failed");
     slots.assign(n_slots, Slot{});
     return true;
 }
@@ -372,14 +615,16 @@ int qk_engine::step_chunk(uint32_t* out_tok, uint32_t* out_cnt, uint32_t* out_fi
         bool need = false;             // someone still owes prefill progress or emitted tokens
         for (uint32_t s = 0; s < n_slots; s++) {
             Slot& sl = slots[s];
-            if (!sl.active) { h_ids[s] = 0; continue; }
+            if (!sl.active) { h_ids[s] = 0; h_pos[s] = 0; continue; } // stepped with token 0 at position 0, like the reference
             n_act++;
             max_z = s + 1;
             if (sl.cursor < sl.prompt.size()) { // prefill: feed prompt[cursor] at position cursor
                 h_ids[s] = sl.prompt[sl.cursor];
+                h_pos[s] = sl.cursor;
                 need = true;
-            } else { // decode: feed the last sampled token
+            } else { // decode: feed the last sampled token at position pos
                 h_ids[s] = sl.last;
+                h_pos[s] = sl.pos;
                 if (out_cnt[s] < chunk) need = true;
             }
         }
@@ -423,6 +668,15 @@ int qk_engine::stage_run(uint32_t slot, const uint32_t* toks, const float* hidde
     if (!ids_out) return -3;
     for (uint32_t i = 0; i < n; i++)
         if (toks[i] >= vocab) return -1;
+    if (full_model) { // positions base .. base+n-1 of this slot, one after the other (the state is sequential)
+        if (base == 0 && reset_slot(slot) != 0) return ERR_DEVICE; // base 0 starts from empty (reference src/main.cpp:4668-4675)
+        for (uint32_t i = 0; i < n; i++) {
+            if (int rc = feed_one(slot, toks[i], base + i, true)) return rc;
+            ids_out[i] = h_tok[slot];
+        }
+        last_run_rows = n; // feed_one left the final position's normalised row in d_last
+        return 0;
+    }
     for (uint32_t off = 0; off < n; off += MAX_ROWS) {
         const uint32_t rows = std::min(MAX_ROWS, n - off);
         memcpy(h_ids, toks + off, rows * sizeof(uint32_t));
@@ -504,9 +758,9 @@ int qk_slot_start(qk_engine* e, uint32_t slot, const uint32_t* prompt, uint32_t 
     // Positions [0, n_prompt - 1) are batch-prefilled in chunks of max_b while 16 or more
     // remain, first up to the caller's history boundary, then up to the last prompt token; what
     // is left is consumed one token per serial step, and the last prompt token's step yields
-    // the first generated token.  With no per-position state a prefilled position writes
-    // nothing, so only the bookkeeping is left of the batch prefill; no cached prefix ever
-    // matches for the same reason (start = 0).
+    // the first generated token.  In a MoE-only model a prefilled position writes nothing (no
+    // per-position state), so only the bookkeeping is left of the batch prefill.  The prefix
+    // cache is not part of this library: start = 0.
     const uint32_t start = 0, target = n_prompt - 1;
     uint32_t done = start;
     auto batch_to = [&](uint32_t limit) {
@@ -516,6 +770,14 @@ int qk_slot_start(qk_engine* e, uint32_t slot, const uint32_t* prompt, uint32_t 
     if (!getenv("QK_NO_BATCH")) {
         if (snap_at) batch_to(snap_at);
         batch_to(target);
+    }
+    if (e->full_model) {
+        // a fresh request: clear the previous occupant's recurrent state, then the prefilled
+        // positions, one token at a time on this slot alone (no batched-prefill kernels for the
+        // mixers here; the last prompt token is left to the serial step as in the reference)
+        if (e->reset_slot(slot) != 0) return -6;
+        for (uint32_t p = 0; p < done; p++)
+            if (e->feed_one(slot, prompt[p], p, false) != 0) return -6;
     }
     s.cursor = done; s.pos = done;
     s.active = true;
@@ -552,15 +814,17 @@ int qk_stage_topk(qk_engine* e, uint32_t k, uint32_t* ids, float* vals)
     return e->stage_topk(k, ids, vals);
 }
 
-// No per-position state to save: the calls validate their bounds (reference src/main.cpp:5428-5445).
+// reference src/main.cpp:5428-5445.  A MoE-only model has no per-position state: bounds only.
 uint32_t qk_state_n(const qk_engine* e) { return e ? N_STATE : 0; }
-int qk_state_save(qk_engine* e, uint32_t slot, uint32_t idx, uint32_t)
+int qk_state_save(qk_engine* e, uint32_t slot, uint32_t idx, uint32_t n_tok)
 {
-    return (!e || slot >= e->n_slots || idx >= N_STATE) ? -1 : 0;
+    if (!e || slot >= e->n_slots || idx >= N_STATE) return -1;
+    return e->full_model ? e->copy_state(slot, idx, true, n_tok) : 0;
 }
-int qk_state_load(qk_engine* e, uint32_t slot, uint32_t idx, uint32_t)
+int qk_state_load(qk_engine* e, uint32_t slot, uint32_t idx, uint32_t n_tok)
 {
-    return (!e || slot >= e->n_slots || idx >= N_STATE) ? -1 : 0;
+    if (!e || slot >= e->n_slots || idx >= N_STATE) return -1;
+    return e->full_model ? e->copy_state(slot, idx, false, n_tok) : 0;
 }
 
 } // extern "C"

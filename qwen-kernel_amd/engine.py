@@ -153,3 +153,77 @@ class StackModel:
     def write(self, path):
         gguf.write(path, self.kvs(), self.tensors())
         return path
+
+
+class FullModel:
+    """Synthetic whole model on the host: every layer a mixer (gated DeltaNet "R" or full attention
+    "A", the reference's fixed head shapes) followed by a MoE block; the tensors of a file qk_open
+    accepts, under the reference's names (reference src/main.cpp:3916-4010)."""
+
+    DN = dict(ch=8192, d_in=4096, hv=32, ds=128, hk=16)
+    FA = dict(dh=256, hq=16, hkv=2, n_rot=64)
+
+    def __init__(self, seed, kinds="RRRA", vocab=512, n_expert=8, n_ff=256, n_used=4, eos=1000, bos=11, arch="qwen35moe"):
+        H = 2048
+        rng = np.random.default_rng(seed)
+        f = lambda *shape, scale=1.0: (rng.standard_normal(shape) * scale).astype(np.float32)
+        near1 = lambda n: (1.0 + 0.1 * rng.standard_normal(n)).astype(np.float32)
+        q8 = lambda rows, k, s, sc: synth.tensor_host(capi.Q8_0, rows, k, s, sc)
+        self.arch, self.vocab, self.eos, self.bos, self.n_used, self.kinds = arch, vocab, eos, bos, n_used, kinds
+        self.embd_type = capi.Q6_K
+        self.embd = synth.tensor_host(capi.Q6_K, vocab, H, seed + 101, 1e-3)      # rows of rms ~1
+        self.head = synth.tensor_host(capi.Q6_K, vocab, H, seed + 102)
+        self.out_norm = near1(H)
+        self.layers, self.post_norm, self.attn_norm, self.mix = [], [], [], []
+        for l, kind in enumerate(kinds):
+            s0 = seed + 1000 * (l + 1)
+            # block scales chosen so that residual, mixer output and MoE output are all of order one
+            self.layers.append(synth.HostLayer(s0, H, n_ff, n_expert, n_used, capi.IQ4_XS if l % 2 == 0 else capi.Q6_K,
+                                               d_scale=1.5e-4))
+            self.post_norm.append(near1(H))
+            self.attn_norm.append(near1(H))
+            if kind == "R":
+                d = self.DN
+                self.mix.append(dict(kind="R", qkv=q8(d["ch"], H, s0 + 11, 4e-4), gate=q8(d["d_in"], H, s0 + 12, 4e-4),
+                                     out=q8(H, d["d_in"], s0 + 13, 3e-4), alpha=f(d["hv"], H, scale=0.03),
+                                     beta=f(d["hv"], H, scale=0.03), dt=f(d["hv"]),
+                                     a=(-np.abs(rng.standard_normal(d["hv"])) - 0.05).astype(np.float32),
+                                     ker=f(d["ch"], 4, scale=0.5), norm=near1(d["ds"])))
+            elif kind == "A":
+                a = self.FA
+                self.mix.append(dict(kind="A", q=q8(a["hq"] * 2 * a["dh"], H, s0 + 21, 4e-4), k=q8(a["hkv"] * a["dh"], H, s0 + 22, 4e-4),
+                                     v=q8(a["hkv"] * a["dh"], H, s0 + 23, 4e-4), out=q8(H, a["hq"] * a["dh"], s0 + 24, 3e-4),
+                                     qn=near1(a["dh"]), kn=near1(a["dh"])))
+            else:
+                raise ValueError(kind)
+
+    def kvs(self):
+        return {"general.architecture": self.arch, self.arch + ".block_count": len(self.layers),
+                self.arch + ".expert_used_count": self.n_used, "tokenizer.ggml.eos_token_id": self.eos,
+                "tokenizer.ggml.bos_token_id": self.bos}
+
+    def tensors(self):
+        H, d, a = 2048, self.DN, self.FA
+        t = [("token_embd.weight", self.embd_type, (H, self.vocab), self.embd),
+             ("output_norm.weight", capi.F32, (H,), self.out_norm),
+             ("output.weight", capi.Q6_K, (H, self.vocab), self.head)]
+        for l, hl in enumerate(self.layers):
+            p, m = f"blk.{l}.", self.mix[l]
+            t += gguf.layer_tensors(hl, l)
+            t += [(p + "post_attention_norm.weight", capi.F32, (H,), self.post_norm[l]),
+                  (p + "attn_norm.weight", capi.F32, (H,), self.attn_norm[l])]
+            if m["kind"] == "R":
+                t += [(p + "attn_qkv.weight", capi.Q8_0, (H, d["ch"]), m["qkv"]), (p + "attn_gate.weight", capi.Q8_0, (H, d["d_in"]), m["gate"]),
+                      (p + "ssm_out.weight", capi.Q8_0, (d["d_in"], H), m["out"]), (p + "ssm_alpha.weight", capi.F32, (H, d["hv"]), m["alpha"]),
+                      (p + "ssm_beta.weight", capi.F32, (H, d["hv"]), m["beta"]), (p + "ssm_dt.bias", capi.F32, (d["hv"],), m["dt"]),
+                      (p + "ssm_a", capi.F32, (d["hv"],), m["a"]), (p + "ssm_conv1d.weight", capi.F32, (4, d["ch"]), m["ker"]),
+                      (p + "ssm_norm.weight", capi.F32, (d["ds"],), m["norm"])]
+            else:
+                t += [(p + "attn_q.weight", capi.Q8_0, (H, a["hq"] * 2 * a["dh"]), m["q"]), (p + "attn_k.weight", capi.Q8_0, (H, a["hkv"] * a["dh"]), m["k"]),
+                      (p + "attn_v.weight", capi.Q8_0, (H, a["hkv"] * a["dh"]), m["v"]), (p + "attn_output.weight", capi.Q8_0, (a["hq"] * a["dh"], H), m["out"]),
+                      (p + "attn_q_norm.weight", capi.F32, (a["dh"],), m["qn"]), (p + "attn_k_norm.weight", capi.F32, (a["dh"],), m["kn"])]
+        return t
+
+    def write(self, path):
+        gguf.write(path, self.kvs(), self.tensors())
+        return path

@@ -174,10 +174,12 @@ def test_open_rejects_what_the_reference_rejects(qk, tiny, tmp_path, monkeypatch
     assert not ok and "ffn_up_exps" in msg
     assert variant(drop=("blk.1.post_attention_norm.weight",)) == \
         (False, "qk_open: missing/unexpected post_attention_norm tensor")
-    # a layer with a mixer is a whole-model file: refused, with the reason
-    for mixer in ("blk.0.attn_q.weight", "blk.1.attn_qkv.weight", "blk.1.ssm_out.weight"):
-        ok, msg = variant(add=[(mixer, qk.F32, (2048, 4), np.zeros(8192, np.float32))])
-        assert not ok and "mixers" in msg
+    # mixer tensors on some layers only, or without the tensor that tells the kind of mixer
+    stray = lambda name: variant(add=[(name, qk.F32, (2048, 4), np.zeros(8192, np.float32))])
+    assert stray("blk.0.attn_q.weight") == (False, "qk_open: layers with and without mixers in one file")
+    assert stray("blk.1.ssm_a") == (False, "qk_open: layers with and without mixers in one file")
+    for name in ("blk.1.attn_qkv.weight", "blk.0.ssm_out.weight"):
+        assert stray(name) == (False, "qk_open: a layer has mixer tensors but neither ssm_a nor attn_q")
     monkeypatch.setenv("QK_LAYERS", "2:1")
     assert variant() == (False, "qk_open: bad QK_LAYERS (want a:b with 0 <= a < b <= 2)")
     monkeypatch.setenv("QK_LAYERS", "1:2")

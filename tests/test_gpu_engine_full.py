@@ -1,0 +1,126 @@
+"""qk_open on a synthetic whole-model GGUF (gated-DeltaNet and full-attention layers, each followed
+by a MoE block): the engine's token streams against the restated state machine driving the CPU
+oracle of the whole model (oracle/qk_oracle_engine.py FullModelOracle: the reference's recorded step,
+src/main.cpp:4194-4419, from the oracles of its parts).  Greedy tokens are compared exactly: the
+kernels agree with the oracle to 1e-3, so a step whose two best logits lie closer than that could
+legitimately differ; the seeds used here have no such step among those that decide a token (the
+narrowest gap seen is printed)."""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "oracle"))
+import qk_oracle_engine as OE  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+VOCAB = 384
+
+
+class Checked:
+    """The oracle model behind the state machine, recording the narrowest margin it saw."""
+
+    def __init__(self, model, n_slots, n_ctx):
+        self.o = OE.FullModelOracle(model, n_slots, n_ctx)
+        self.narrowest = np.inf
+
+    def reset(self, slot):
+        self.o.reset(slot)
+
+    def feed(self, slot, token, pos, depth):
+        t = self.o.feed(slot, token, pos, depth)
+        gap, top = self.o.last_margin
+        self.narrowest = min(self.narrowest, gap / top)
+        return t
+
+
+@pytest.fixture(scope="module")
+def full(qk, dev, tmp_path_factory):
+    model = qk.engine.FullModel(17, kinds="RRAR", vocab=VOCAB, eos=VOCAB + 5)
+    path = model.write(str(tmp_path_factory.mktemp("full") / "model.gguf"))
+    return model, path
+
+
+def drive(eng, ref, script, n_calls):
+    for call in range(n_calls):
+        for op in script.get(call, []):
+            if op[0] == "start":
+                _, slot, prompt, max_gen, snap = op
+                assert eng.slot_start(slot, prompt, max_gen, snap) == ref.slot_start(slot, prompt, max_gen, snap), op
+            else:
+                eng.slot_cancel(op[1])
+                ref.slot_cancel(op[1])
+        got, want = eng.step_chunk(), ref.step_chunk()
+        assert got == want, (call, got, want)
+
+
+def test_whole_model_streams(qk, full):
+    """Three slots with different prompt lengths (serial prefill, a prefilled prompt, a one-token
+    prompt), a slot reused after it finished, one cancelled: the recurrent state and the KV rows of a
+    slot belong to it alone and are cleared when the next request takes the slot."""
+    model, path = full
+    print("[case] whole model, three slots", flush=True)
+    rng = np.random.default_rng(4)
+    P = lambda n: [int(t) for t in rng.integers(0, VOCAB, n)]
+    with qk.engine.Engine(path, n_slots=3, n_ctx=96, chunk=3) as eng:
+        assert (eng.vocab, eng.n_layer, eng.eos) == (VOCAB, 4, VOCAB + 5)
+        chk = Checked(model, 3, 96)
+        ref = OE.SlotMachine(chk, VOCAB, VOCAB + 5, 3, 96, 3)
+        script = {0: [("start", 1, P(5), 7, 0)],
+                  1: [("start", 0, P(20), 5, 0), ("start", 2, P(1), 9, 0)],   # 20 tokens: 19 prefilled at the start
+                  3: [("cancel", 2)],
+                  4: [("start", 2, P(3), 4, 0)],                               # slot 2 again, fresh state
+                  6: [("start", 1, P(2), 3, 0)]}                               # slot 1 again after it finished
+        drive(eng, ref, script, 10)
+        assert not any(sl["active"] for sl in ref.slots)
+        print(f"[info] narrowest top-2 gap / largest logit over all steps fed: {chk.narrowest:.2e}", flush=True)
+
+
+def test_whole_model_eager_launches_and_serial_prefill(qk, full, monkeypatch):
+    """QK_NO_GRAPH launches the kernels one by one; QK_NO_BATCH feeds every prompt token in a serial
+    step instead of at the start: the same streams."""
+    model, path = full
+    print("[case] whole model, eager / serial prefill", flush=True)
+    prompt = [int(t) for t in np.random.default_rng(6).integers(0, VOCAB, 18)]
+    streams = []
+    for env in ({}, {"QK_NO_GRAPH": "1"}, {"QK_NO_BATCH": "1"}):
+        for k in ("QK_NO_GRAPH", "QK_NO_BATCH"):
+            monkeypatch.delenv(k, raising=False)
+        for k, v in env.items():
+            monkeypatch.setenv(k, v)
+        with qk.engine.Engine(path, n_slots=2, n_ctx=64, chunk=8) as eng:
+            assert eng.slot_start(1, prompt, 6) == 0
+            got = []
+            for _ in range(4):
+                rc, out, fin = eng.step_chunk()
+                got += out[1]
+            streams.append(got)
+    assert len(streams[0]) == 6 and streams[0] == streams[1] == streams[2]
+
+
+def test_whole_model_stage_run_and_snapshots(qk, full):
+    """qk_stage_run feeds a slot's positions in order; a snapshot taken after a prefix brings the slot
+    back to it (qk_state_save / qk_state_load), so the continuation repeats."""
+    model, path = full
+    print("[case] whole model, stage run and snapshots", flush=True)
+    toks = [int(t) for t in np.random.default_rng(9).integers(0, VOCAB, 9)]
+    with qk.engine.Engine(path, n_slots=2, n_ctx=64, chunk=2) as eng:
+        o = OE.FullModelOracle(model, 1, 64)
+        want = [o.feed(0, t, p) for p, t in enumerate(toks)]
+        rc, ids = eng.stage_run(1, toks[:6], 0)
+        assert rc == 0 and ids == want[:6]
+        assert eng.state_save(1, 2, 6) == 0
+        rc, tail = eng.stage_run(1, toks[6:], 6)
+        assert rc == 0 and tail == want[6:]
+        rc, top_ids, top_vals = eng.stage_topk(3)
+        assert rc == 0 and top_ids[0] == tail[-1] and top_vals[0] >= top_vals[1] >= top_vals[2]
+        # other tokens move the state on; loading the snapshot restores the prefix's state
+        rc, other = eng.stage_run(1, [7, 8, 9], 6)
+        assert rc == 0
+        assert eng.state_load(1, 2, 6) == 0
+        rc, again = eng.stage_run(1, toks[6:], 6)
+        assert rc == 0 and again == tail
+        assert eng.state_save(1, 3, 0) == -1 and eng.state_load(2, 0, 0) == -1
