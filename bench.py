@@ -317,22 +317,27 @@ def deltanet_workload(qk, n_slots, steps, warmup, seed=6):
     return dict(ms_event=ev, steps=n, ring=ring, bytes_step=2 * n_slots * hV * dS * dS * 4)
 
 
-def engine_workload(qk, n_layer, slots_list, chunks, warm_chunks, seed=31):
+def engine_workload(qk, n_layer, slots_list, chunks, warm_chunks, seed=31, kinds=None):
     """Tokens per second through the engine ABI (qk_open / qk_slot_start / qk_step_chunk) on a
-    synthetic MoE-only model file at the full layer shape and vocabulary: host wall clock over
-    whole chunks, host synchronisation after every step included.  Two distinct layers' weights
-    alternate through the file; each layer has its own copy in device memory."""
+    synthetic model file at the full layer shape and vocabulary: host wall clock over whole chunks,
+    host synchronisation after every step included.  kinds = None: MoE-only layers; else one letter
+    per layer, "R" gated DeltaNet or "A" full attention in front of each MoE block (a whole model).
+    Two distinct layers' MoE weights alternate through the file; each layer has its own copy in
+    device memory."""
     import shutil
     import tempfile
-    import time
-    model = qk.engine.StackModel(seed, n_layer=2, vocab=151936, n_expert=256, n_ff=512, n_used=8,
-                                 down_types=[qk.IQ4_XS, qk.Q6_K], eos=151935)
-    model.layers = [model.layers[l % 2] for l in range(n_layer)]
-    model.post_norm = [model.post_norm[l % 2] for l in range(n_layer)]
+    if kinds is None:
+        model = qk.engine.StackModel(seed, n_layer=2, vocab=151936, n_expert=256, n_ff=512, n_used=8,
+                                     down_types=[qk.IQ4_XS, qk.Q6_K], eos=151935)
+        model.layers = [model.layers[l % 2] for l in range(n_layer)]
+        model.post_norm = [model.post_norm[l % 2] for l in range(n_layer)]
+    else:
+        model = qk.engine.FullModel(seed, kinds=kinds, vocab=151936, n_expert=256, n_ff=512, n_used=8, eos=151935,
+                                    distinct_moe=2)
     tmp = tempfile.mkdtemp(prefix="qk_bench_")
     res = {}
     try:
-        path = model.write(os.path.join(tmp, "stack.gguf"))
+        path = model.write(os.path.join(tmp, "model.gguf"))
         del model
         for n_slots in slots_list:
             t0 = time.perf_counter()
@@ -357,7 +362,7 @@ def engine_workload(qk, n_layer, slots_list, chunks, warm_chunks, seed=31):
                                            open_s=t_open)
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
-    res["config"] = dict(n_layer=n_layer, vocab=151936, chunk=32,
+    res["config"] = dict(n_layer=n_layer, vocab=151936, chunk=32, mixers=kinds or "none",
                          layer="256 experts, IQ3_XXS gate/up, IQ4_XS / Q6_K down alternating, Q8_0 shared")
     return res
 
@@ -392,6 +397,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", default="moe_decode_bs1")
     ap.add_argument("--ring", type=int, default=40)
+    ap.add_argument("--layers", type=int, default=8,
+                    help="layers of the synthetic model of the engine workloads (40 = the reference model's depth, a 16 GB file)")
     ap.add_argument("--extras", dest="extras", action="store_true", default=True)
     ap.add_argument("--no-extras", dest="extras", action="store_false")
     ap.add_argument("--copy-probe", action="store_true",
@@ -418,6 +425,12 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     steps = max(a.ring, a.steps // a.ring * a.ring)
+    if a.workload == "engine_whole_model":   # the engine ABI on a whole model (mixers + MoE blocks)
+        r = engine_workload(qk, a.layers, (1, 16), 8, 2, kinds=("RRRA" * ((a.layers + 3) // 4))[:a.layers])
+        print(json.dumps(dict(metric="engine_decode_tok_per_s", value=r["slots_16"]["tok_per_s"], unit="tok/s", n_gpus=1,
+                              higher_is_better=True, data="synthetic", dtype="f32",
+                              config=dict(workload="engine_whole_model", **r["config"]), detail=r)), flush=True)
+        return
     if a.workload == "engine_decode":   # the engine ABI alone (for kernel traces of its graph replays)
         r = engine_workload(qk, 8, (1, 4, 16), 8, 2)
         print(json.dumps(dict(metric="engine_decode_tok_per_s", value=r["slots_16"]["tok_per_s"], unit="tok/s", n_gpus=1,
@@ -574,6 +587,9 @@ def main():
             log(f"[bench] deltanet: {ex['deltanet_decode_bs1']} {ex['deltanet_decode_bs16']}")
             ex["engine_decode_8_layers"] = engine_workload(qk, 8, (1, 4, 16), 8, 2)
             log(f"[bench] engine: {ex['engine_decode_8_layers']}")
+            # a whole model: three gated-DeltaNet layers and one full-attention layer, twice (positions 1..320)
+            ex["engine_decode_whole_model_8_layers"] = engine_workload(qk, 8, (1, 16), 8, 2, kinds="RRRARRRA")
+            log(f"[bench] engine, whole model: {ex['engine_decode_whole_model_8_layers']}")
         out["extras"] = ex
 
     if a.cpu:

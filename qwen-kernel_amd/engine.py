@@ -163,7 +163,8 @@ class FullModel:
     DN = dict(ch=8192, d_in=4096, hv=32, ds=128, hk=16)
     FA = dict(dh=256, hq=16, hkv=2, n_rot=64)
 
-    def __init__(self, seed, kinds="RRRA", vocab=512, n_expert=8, n_ff=256, n_used=4, eos=1000, bos=11, arch="qwen35moe"):
+    def __init__(self, seed, kinds="RRRA", vocab=512, n_expert=8, n_ff=256, n_used=4, eos=1000, bos=11, arch="qwen35moe",
+                 distinct_moe=None):
         H = 2048
         rng = np.random.default_rng(seed)
         f = lambda *shape, scale=1.0: (rng.standard_normal(shape) * scale).astype(np.float32)
@@ -178,8 +179,11 @@ class FullModel:
         for l, kind in enumerate(kinds):
             s0 = seed + 1000 * (l + 1)
             # block scales chosen so that residual, mixer output and MoE output are all of order one
-            self.layers.append(synth.HostLayer(s0, H, n_ff, n_expert, n_used, capi.IQ4_XS if l % 2 == 0 else capi.Q6_K,
-                                               d_scale=1.5e-4))
+            if distinct_moe and l >= distinct_moe:   # large files: reuse the first layers' MoE weights (own copy in the file)
+                self.layers.append(self.layers[l % distinct_moe])
+            else:
+                self.layers.append(synth.HostLayer(s0, H, n_ff, n_expert, n_used, capi.IQ4_XS if l % 2 == 0 else capi.Q6_K,
+                                                   d_scale=1.5e-4))
             self.post_norm.append(near1(H))
             self.attn_norm.append(near1(H))
             if kind == "R":
