@@ -7,16 +7,21 @@
  * Threading: every function is called from one engine thread; nothing is thread-safe;
  * qk_step_chunk blocks that thread for one chunk of device steps.
  *
- * What qk_open() runs: a GGUF whose layers are MoE blocks only (token embedding, per layer
- * post_attention_norm + the eight MoE tensors, output_norm, Q6_K head) -- the reference's decode
- * step with every mixer output zero.  A file whose layers carry attention or gated-DeltaNet
- * mixer tensors is refused with a message saying that the mixers are not part of this library.
- * On the file it accepts, every entry point behaves as the reference's: argument checks and
- * return codes, the serial-step state machine of qk_step_chunk (one captured hipGraph per
- * dispatch depth), greedy sampling, EOS / max_gen / n_ctx endings.  Such a model keeps no
- * per-position state, so snapshots validate their bounds only, as in the reference's stub
- * engine (reference stub/qk_stub.c:95-106).  QK_LAYERS pipeline stages are refused: one GPU runs
- * every layer.  A device failure inside qk_step_chunk / qk_stage_run / qk_stage_topk returns -6.
+ * What qk_open() runs:
+ *   - a whole-model GGUF of the reference's family: token embedding, per layer attn_norm + a mixer
+ *     (gated DeltaNet where "ssm_a" is present, else full attention) + post_attention_norm + the
+ *     eight MoE tensors, output_norm, Q6_K head; head shapes as in the reference engine (DeltaNet
+ *     32 value / 16 key heads of 128, attention 16 x 256 query heads on 2 KV heads, n_embd 2048);
+ *     dense projections Q8_0 or IQ4_XS; ssm_alpha / ssm_beta as separate F32 tensors (the fused
+ *     ssm_ba form is refused);
+ *   - a GGUF whose layers are MoE blocks only (no mixer tensors at all).
+ * Every entry point behaves as the reference's: argument checks and return codes, the serial-step
+ * state machine of qk_step_chunk (one captured hipGraph per dispatch depth), greedy sampling,
+ * EOS / max_gen / n_ctx endings, qk_stage_run / qk_stage_topk on the unsplit engine, state
+ * snapshots (three entries).  Not part of this library: batched prefill kernels for the mixers
+ * (qk_slot_start feeds the positions the reference batch-prefills one token at a time, on the
+ * starting slot alone), the prefix cache, speculative decoding, QK_LAYERS pipeline stages (refused:
+ * one GPU runs every layer).  A device failure inside a call returns -6.
  * Environment, as in the reference: QK_MAXB (batch-prefill chunk, 16..1024, default 128),
  * QK_NO_BATCH (serial prefill of the whole prompt); and QK_NO_GRAPH (launch the step's kernels
  * one by one instead of replaying the graph).

@@ -3,18 +3,20 @@
 // over the kernels of this library, one hipGraph per dispatch depth in place of the
 // reference's pre-recorded command buffers (reference src/main.cpp:4186-4422).
 //
-// What the engine can run.  The reference model alternates a mixer (attention or gated
-// DeltaNet) with a MoE block in every layer.  The mixers are not part of this library, so
-// qk_open() refuses a file whose layers carry mixer tensors; it runs a file whose layers are
-// MoE blocks only:
-//   x      = embed(token)                                    token_embd.weight (Q6_K / Q8_0)
-//   layer: xn = rmsnorm(x, blk.l.post_attention_norm);  x = x + MoE_l(xn)
-//   token' = argmax(output.weight . rmsnorm(x, output_norm)) Q6_K head, ties to the lower id
-// -- the reference's decode step (src/main.cpp:4194-4405) with every mixer output taken as
-// zero.  Such a model keeps no per-position state, so a slot's device state is empty:
-// snapshots validate their bounds only and a batch-prefilled position has nothing to write.
+// What the engine can run.  The reference model alternates a mixer (full attention or gated
+// DeltaNet) with a MoE block in every layer.  qk_open() takes
+//   - a whole-model file: per layer  xn = rmsnorm(x, attn_norm); y = x + mixer(xn);
+//     x = y + MoE(rmsnorm(y, post_attention_norm))  -- the reference's decode step
+//     (src/main.cpp:4194-4405) from this library's operators; per-slot state stripes (conv window
+//     and delta-rule state, or K / V cache) live in the engine;
+//   - a file whose layers are MoE blocks only: the same step with every mixer output zero; such a
+//     model keeps no per-position state.
+//   token' = argmax(output.weight . rmsnorm(x, output_norm)), Q6_K head, ties to the lower id.
 // Everything the host sees -- argument checks, return codes, which step emits which token,
-// EOS / max_gen / n_ctx endings, the finished mask -- follows the reference line by line.
+// EOS / max_gen / n_ctx endings, the finished mask -- follows the reference line by line.  The
+// positions the reference batch-prefills at qk_slot_start are fed here one token at a time on the
+// starting slot alone (no batched-prefill kernels for the mixers); prefix cache and speculative
+// decoding are not part of this library.
 #include <stdlib.h>
 #include <string.h>
 
