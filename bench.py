@@ -358,8 +358,20 @@ def engine_workload(qk, n_layer, slots_list, chunks, warm_chunks, seed=31, kinds
                 t0 = time.perf_counter()
                 toks = run(chunks)
                 dt = time.perf_counter() - t0
+                pre = {}
+                if kinds is not None and n_slots == slots_list[0]:
+                    # prompt positions per second: qk_stage_run over 512 positions of one slot, twice
+                    # (the first pass warms the prefill path's launch set-up)
+                    ptoks = [(7 * i + 3) % 151000 for i in range(512)]
+                    for _ in range(2):
+                        tp = time.perf_counter()
+                        rcp, _ids = eng.stage_run(0, ptoks, 0)
+                        tp = time.perf_counter() - tp
+                        if rcp != 0:
+                            sys.exit(f"bench.py: qk_stage_run returned {rcp}")
+                    pre = dict(prefill_tok_per_s=len(ptoks) / tp, prefill_positions=len(ptoks))
             res[f"slots_{n_slots}"] = dict(tok_per_s=toks / dt, us_per_step=dt / (chunks * 32) * 1e6, tokens=toks,
-                                           open_s=t_open)
+                                           open_s=t_open, **pre)
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
     res["config"] = dict(n_layer=n_layer, vocab=151936, chunk=32, mixers=kinds or "none",

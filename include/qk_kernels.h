@@ -281,6 +281,31 @@ int qkk_dn_step(const float *conv, const float *gb, float *state, const float *n
                 float *att, uint32_t d_state, uint32_t hK, uint32_t hV, uint32_t kdiv, float eps,
                 uint32_t n_slots, void *stream);
 
+/* ---- the mixers over consecutive positions of ONE slot (prompt prefill) ---------------------------
+ * (reference shaders/fa_prep_batch.comp, fa_attn_batch.comp, dn_conv_batch.comp, dn_step_batch.comp
+ * + dn_gate_batch.comp; host src/main.cpp:3953-4090.)  Rows are positions base, base+1, ... of one
+ * slot; conv_state, state and the caches are that slot's alone.  Results per position are those of
+ * the decode-step entry points called position by position.
+ * qkk_attn_prep_seq  row t is written into the caches at positions[t] (distinct, ascending).
+ * qkk_attn_seq       row t attends to the cache rows 0..positions[t]: causal over the rows of this
+ *                    call and everything the cache held before.  Every row scans the cache for
+ *                    itself (served from the L2 / last-level cache, but not a query-blocked scan as
+ *                    the reference's). workspace: qkk_attn_workspace_bytes(n_pos, hQ, dh).
+ * qkk_dn_conv_seq / qkk_dn_step_seq  the input window / the state stay in registers over all
+ *                    positions and are written back once; one launch each. */
+int qkk_attn_prep_seq(const float *qfull, const float *kin, const float *vin, const float *q_norm_w,
+                      const float *k_norm_w, const float *rope, const uint32_t *positions, float *qhat,
+                      float *k_cache, float *v_cache, uint32_t n_pos, uint32_t hQ, uint32_t hKV,
+                      uint32_t dh, uint32_t n_rot, uint32_t tmax, float eps, void *stream);
+int qkk_attn_seq(const float *qhat, const float *k_cache, const float *v_cache, const float *qfull,
+                 const uint32_t *positions, float *att, void *workspace, size_t workspace_bytes,
+                 uint32_t n_pos, uint32_t hQ, uint32_t hKV, uint32_t dh, uint32_t tmax, void *stream);
+int qkk_dn_conv_seq(float *conv_state, const float *qkv, const float *ker, float *out, uint32_t channels,
+                    uint32_t d_state, uint32_t qk_channels, float eps, uint32_t n_pos, void *stream);
+int qkk_dn_step_seq(const float *conv, const float *gb, float *state, const float *norm_w, const float *z,
+                    float *att, uint32_t d_state, uint32_t hK, uint32_t hV, uint32_t kdiv, float eps,
+                    uint32_t n_pos, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

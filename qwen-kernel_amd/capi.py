@@ -74,11 +74,15 @@ def lib():
         L.qkk_dn_ab.argtypes = [vp] * 6 + [u32] * 3 + [vp]
         L.qkk_dn_conv.argtypes = [vp] * 4 + [u32] * 3 + [f32, u32, vp]
         L.qkk_dn_step.argtypes = [vp] * 6 + [u32] * 4 + [f32, u32, vp]
+        L.qkk_dn_conv_seq.argtypes = L.qkk_dn_conv.argtypes
+        L.qkk_dn_step_seq.argtypes = L.qkk_dn_step.argtypes
         L.qkk_rope_table.argtypes = [vp, u32, u32, f32]
         L.qkk_attn_prep.argtypes = [vp] * 10 + [u32] * 6 + [f32, vp]
         L.qkk_attn_workspace_bytes.restype = sz
         L.qkk_attn_workspace_bytes.argtypes = [u32, u32, u32]
         L.qkk_attn_decode.argtypes = [vp] * 7 + [sz] + [u32] * 5 + [vp]
+        L.qkk_attn_prep_seq.argtypes = L.qkk_attn_prep.argtypes
+        L.qkk_attn_seq.argtypes = L.qkk_attn_decode.argtypes
         _lib = L
     return _lib
 
@@ -320,17 +324,20 @@ def rope_table(tmax, n_rot, freq_base=1e7):
     return out
 
 
-def attn_prep(qfull, kin, vin, q_norm_w, k_norm_w, rope, slot_pos, k_cache, v_cache, n_rot, eps=1e-6, qhat=None):
+def attn_prep(qfull, kin, vin, q_norm_w, k_norm_w, rope, slot_pos, k_cache, v_cache, n_rot, eps=1e-6, qhat=None, seq=False):
     """Head norm + RoPE + cache write for the slots' new tokens.  qfull [slots][hQ][2*dh],
-    kin / vin [slots][hKV][dh], caches [slots][hKV][tmax][dh].  Returns qhat [slots][hQ][dh]."""
+    kin / vin [slots][hKV][dh], caches [slots][hKV][tmax][dh].  Returns qhat [slots][hQ][dh].
+    seq: the rows are positions slot_pos[t] of ONE slot, caches [1][hKV][tmax][dh]."""
     import torch
     n, hQ, dh2 = qfull.shape
     hKV, tmax, dh = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
     if qhat is None:
         qhat = torch.empty((n, hQ, dh), dtype=torch.float32, device=qfull.device)
-    _check(lib().qkk_attn_prep(_ptr(qfull), _ptr(kin), _ptr(vin), _ptr(q_norm_w), _ptr(k_norm_w), _ptr(rope),
-                               _ptr(slot_pos), _ptr(qhat), _ptr(k_cache), _ptr(v_cache), n, hQ, hKV, dh, n_rot, tmax,
-                               eps, _stream()))
+    if k_cache.shape[0] != (1 if seq else n) or v_cache.shape != k_cache.shape:
+        raise ValueError("attn_prep: caches do not match the rows")
+    fn = lib().qkk_attn_prep_seq if seq else lib().qkk_attn_prep
+    _check(fn(_ptr(qfull), _ptr(kin), _ptr(vin), _ptr(q_norm_w), _ptr(k_norm_w), _ptr(rope), _ptr(slot_pos), _ptr(qhat),
+              _ptr(k_cache), _ptr(v_cache), n, hQ, hKV, dh, n_rot, tmax, eps, _stream()))
     return qhat
 
 
@@ -338,17 +345,20 @@ def attn_workspace_bytes(n_slots, hQ, dh=256):
     return lib().qkk_attn_workspace_bytes(n_slots, hQ, dh)
 
 
-def attn_decode(qhat, k_cache, v_cache, qfull, slot_pos, workspace, att=None):
+def attn_decode(qhat, k_cache, v_cache, qfull, slot_pos, workspace, att=None, seq=False):
     """Attention of the slots' new tokens over positions 0..slot_pos with the output gate.
-    Returns att [slots][hQ][dh]."""
+    Returns att [slots][hQ][dh].  seq: the rows are positions of ONE slot (caches [1][hKV][tmax][dh]),
+    row t attends to cache rows 0..slot_pos[t]."""
     import torch
     n, hQ, dh = qhat.shape
     hKV, tmax = k_cache.shape[1], k_cache.shape[2]
     if att is None:
         att = torch.empty_like(qhat)
-    _check(lib().qkk_attn_decode(_ptr(qhat), _ptr(k_cache), _ptr(v_cache), _ptr(qfull), _ptr(slot_pos), _ptr(att),
-                                 _ptr(workspace), workspace.numel() * workspace.element_size(), n, hQ, hKV, dh, tmax,
-                                 _stream()))
+    if k_cache.shape[0] != (1 if seq else n) or v_cache.shape != k_cache.shape:
+        raise ValueError("attn_decode: caches do not match the rows")
+    fn = lib().qkk_attn_seq if seq else lib().qkk_attn_decode
+    _check(fn(_ptr(qhat), _ptr(k_cache), _ptr(v_cache), _ptr(qfull), _ptr(slot_pos), _ptr(att), _ptr(workspace),
+              workspace.numel() * workspace.element_size(), n, hQ, hKV, dh, tmax, _stream()))
     return att
 
 
@@ -363,25 +373,31 @@ def dn_ab(x, alpha_w, beta_w, dt_bias, a_vec, gb=None):
     return gb
 
 
-def dn_conv(conv_state, qkv, ker, qk_channels, d_state=128, eps=1e-6, out=None):
+def dn_conv(conv_state, qkv, ker, qk_channels, d_state=128, eps=1e-6, out=None, seq=False):
     """Depthwise conv(4) + SiLU + window shift, q/k heads scaled to unit length.  conv_state
-    [slots][channels][3] is updated in place; returns out [slots][channels]."""
+    [slots][channels][3] is updated in place; returns out [slots][channels].  seq: the rows are
+    consecutive positions of ONE slot, conv_state [1][channels][3]."""
     import torch
     n, channels = qkv.shape
     if out is None:
         out = torch.empty_like(qkv)
-    _check(lib().qkk_dn_conv(_ptr(conv_state), _ptr(qkv), _ptr(ker), _ptr(out), channels, d_state, qk_channels, eps, n,
-                             _stream()))
+    if conv_state.numel() != (1 if seq else n) * channels * 3:
+        raise ValueError("dn_conv: conv_state does not match the rows")
+    fn = lib().qkk_dn_conv_seq if seq else lib().qkk_dn_conv
+    _check(fn(_ptr(conv_state), _ptr(qkv), _ptr(ker), _ptr(out), channels, d_state, qk_channels, eps, n, _stream()))
     return out
 
 
-def dn_step(conv, gb, state, norm_w, z, hK, hV, kdiv=0, d_state=128, eps=1e-6, att=None):
+def dn_step(conv, gb, state, norm_w, z, hK, hV, kdiv=0, d_state=128, eps=1e-6, att=None, seq=False):
     """Gated delta-rule update of state [slots][hV][dS][dS] (column-major per head, in place) and the
-    gated, normalised output att [slots][hV*dS]."""
+    gated, normalised output att [slots][hV*dS].  seq: the rows are consecutive positions of ONE
+    slot, state [1][hV][dS][dS]."""
     import torch
     n = conv.shape[0]
     if att is None:
         att = torch.empty((n, hV * d_state), dtype=torch.float32, device=conv.device)
-    _check(lib().qkk_dn_step(_ptr(conv), _ptr(gb), _ptr(state), _ptr(norm_w), _ptr(z), _ptr(att), d_state, hK, hV, kdiv,
-                             eps, n, _stream()))
+    if state.numel() != (1 if seq else n) * hV * d_state * d_state:
+        raise ValueError("dn_step: state does not match the rows")
+    fn = lib().qkk_dn_step_seq if seq else lib().qkk_dn_step
+    _check(fn(_ptr(conv), _ptr(gb), _ptr(state), _ptr(norm_w), _ptr(z), _ptr(att), d_state, hK, hV, kdiv, eps, n, _stream()))
     return att

@@ -45,15 +45,17 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const float* __restrict_
                                                         const float* __restrict__ kn, const float* __restrict__ rope,
                                                         const uint32_t* __restrict__ slot_pos, float* __restrict__ qhat,
                                                         float* __restrict__ kc, float* __restrict__ vc, uint32_t hQ,
-                                                        uint32_t hKV, uint32_t n_rot, uint32_t tmax, float eps)
+                                                        uint32_t hKV, uint32_t n_rot, uint32_t tmax, float eps,
+                                                        uint32_t own)
 {
     __shared__ float s_v[ATT_DH];
     __shared__ float s_red[4];
     const uint32_t w = blockIdx.x, rq = blockIdx.y, t = threadIdx.x;
     const uint32_t pos = slot_position(slot_pos, rq, tmax);
+    const size_t cq = (size_t)rq * own; // the cache row rq writes: its own, or the one all rows share
     if (w >= hQ + hKV) { // value head: copied into the cache
         const uint32_t h = w - hQ - hKV;
-        vc[(((size_t)rq * hKV + h) * tmax + pos) * ATT_DH + t] = vin[((size_t)rq * hKV + h) * ATT_DH + t];
+        vc[((cq * hKV + h) * tmax + pos) * ATT_DH + t] = vin[((size_t)rq * hKV + h) * ATT_DH + t];
         return;
     }
     const bool is_q = w < hQ;
@@ -73,7 +75,7 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const float* __restrict_
         out = t < half ? x0 * c - x1 * s : x0 * s + x1 * c;
     }
     if (is_q) qhat[((size_t)rq * hQ + h) * ATT_DH + t] = out;
-    else kc[(((size_t)rq * hKV + h) * tmax + pos) * ATT_DH + t] = out;
+    else kc[((cq * hKV + h) * tmax + pos) * ATT_DH + t] = out;
 }
 
 // Partial results of one position range: per query head the running maximum, the sum of
@@ -120,7 +122,7 @@ __device__ __forceinline__ HalfSplit split8(float4 a, float4 b)
 __global__ __launch_bounds__(256) void attn_range_kernel(const float* __restrict__ qhat, const float* __restrict__ kc,
                                                          const float* __restrict__ vc,
                                                          const uint32_t* __restrict__ slot_pos, AttnWs ws, uint32_t hQ,
-                                                         uint32_t hKV, uint32_t G, uint32_t tmax)
+                                                         uint32_t hKV, uint32_t G, uint32_t tmax, uint32_t own)
 {
     constexpr uint32_t RPW = ATT_TILE / 4; // rows per wave and tile (16: one MFMA column block)
     constexpr uint32_t KB = ATT_DH / 32;   // 32-dim blocks of a row
@@ -151,8 +153,8 @@ __global__ __launch_bounds__(256) void attn_range_kernel(const float* __restrict
     }
     if (t < ATT_GMAX) { s_m[t] = ATT_FLOOR; s_l[t] = 0.f; }
     const float qs = 1.f / sqrtf((float)ATT_DH);
-    const float4* kbase = (const float4*)(kc + ((size_t)rq * hKV + kv) * tmax * ATT_DH);
-    const float4* vbase = (const float4*)(vc + ((size_t)rq * hKV + kv) * tmax * ATT_DH);
+    const float4* kbase = (const float4*)(kc + ((size_t)rq * own * hKV + kv) * tmax * ATT_DH);
+    const float4* vbase = (const float4*)(vc + ((size_t)rq * own * hKV + kv) * tmax * ATT_DH);
     float4 acc[ATT_GMAX];
 #pragma unroll
     for (uint32_t h = 0; h < ATT_GMAX; h++) acc[h] = float4{0.f, 0.f, 0.f, 0.f};
@@ -324,20 +326,40 @@ int qkk_rope_table(float* rope_host, uint32_t tmax, uint32_t n_rot, float freq_b
     return QKK_OK;
 }
 
+// rows of their own caches (own = 1: decode, one row per slot) or of one cache (own = 0: consecutive
+// positions of one slot)
+static int attn_prep_impl(const char* who, const float* qfull, const float* kin, const float* vin, const float* q_norm_w,
+                          const float* k_norm_w, const float* rope, const uint32_t* slot_pos, float* qhat, float* k_cache,
+                          float* v_cache, uint32_t rows, uint32_t hQ, uint32_t hKV, uint32_t dh, uint32_t n_rot,
+                          uint32_t tmax, float eps, uint32_t own, void* stream)
+{
+    if (!qfull || !kin || !vin || !q_norm_w || !k_norm_w || !rope || !slot_pos || !qhat || !k_cache || !v_cache)
+        return fail(QKK_EINVAL, "%s: null pointer", who);
+    if (int rc = check_shape(who, rows, hQ, hKV, dh, tmax)) return rc;
+    if (n_rot < 2 || n_rot % 2 || n_rot > dh) return fail(QKK_ESHAPE, "%s: n_rot %u must be even, 2..%u", who, n_rot, dh);
+    if (!(eps >= 0.f)) return fail(QKK_EINVAL, "%s: eps must be non-negative", who);
+    if (int rc = require_device()) return rc;
+    hipLaunchKernelGGL(attn_prep_kernel, dim3(hQ + 2 * hKV, rows), dim3(256), 0, as_stream(stream), qfull, kin, vin,
+                       q_norm_w, k_norm_w, rope, slot_pos, qhat, k_cache, v_cache, hQ, hKV, n_rot, tmax, eps, own);
+    return check_launch(who);
+}
+
 int qkk_attn_prep(const float* qfull, const float* kin, const float* vin, const float* q_norm_w, const float* k_norm_w,
                   const float* rope, const uint32_t* slot_pos, float* qhat, float* k_cache, float* v_cache,
                   uint32_t n_slots, uint32_t hQ, uint32_t hKV, uint32_t dh, uint32_t n_rot, uint32_t tmax, float eps,
                   void* stream)
 {
-    if (!qfull || !kin || !vin || !q_norm_w || !k_norm_w || !rope || !slot_pos || !qhat || !k_cache || !v_cache)
-        return fail(QKK_EINVAL, "qkk_attn_prep: null pointer");
-    if (int rc = check_shape("qkk_attn_prep", n_slots, hQ, hKV, dh, tmax)) return rc;
-    if (n_rot < 2 || n_rot % 2 || n_rot > dh) return fail(QKK_ESHAPE, "qkk_attn_prep: n_rot %u must be even, 2..%u", n_rot, dh);
-    if (!(eps >= 0.f)) return fail(QKK_EINVAL, "qkk_attn_prep: eps must be non-negative");
-    if (int rc = require_device()) return rc;
-    hipLaunchKernelGGL(attn_prep_kernel, dim3(hQ + 2 * hKV, n_slots), dim3(256), 0, as_stream(stream), qfull, kin, vin,
-                       q_norm_w, k_norm_w, rope, slot_pos, qhat, k_cache, v_cache, hQ, hKV, n_rot, tmax, eps);
-    return check_launch("qkk_attn_prep");
+    return attn_prep_impl("qkk_attn_prep", qfull, kin, vin, q_norm_w, k_norm_w, rope, slot_pos, qhat, k_cache, v_cache,
+                          n_slots, hQ, hKV, dh, n_rot, tmax, eps, 1, stream);
+}
+
+int qkk_attn_prep_seq(const float* qfull, const float* kin, const float* vin, const float* q_norm_w, const float* k_norm_w,
+                      const float* rope, const uint32_t* positions, float* qhat, float* k_cache, float* v_cache,
+                      uint32_t n_pos, uint32_t hQ, uint32_t hKV, uint32_t dh, uint32_t n_rot, uint32_t tmax, float eps,
+                      void* stream)
+{
+    return attn_prep_impl("qkk_attn_prep_seq", qfull, kin, vin, q_norm_w, k_norm_w, rope, positions, qhat, k_cache, v_cache,
+                          n_pos, hQ, hKV, dh, n_rot, tmax, eps, 0, stream);
 }
 
 size_t qkk_attn_workspace_bytes(uint32_t n_slots, uint32_t hQ, uint32_t dh)
@@ -346,32 +368,47 @@ size_t qkk_attn_workspace_bytes(uint32_t n_slots, uint32_t hQ, uint32_t dh)
     return (size_t)n_slots * hQ * ATT_MAX_RANGES * ((size_t)dh + 2) * sizeof(float) + 256;
 }
 
+static int attn_decode_impl(const char* who, const float* qhat, const float* k_cache, const float* v_cache,
+                            const float* qfull, const uint32_t* slot_pos, float* att, void* workspace,
+                            size_t workspace_bytes, uint32_t rows, uint32_t hQ, uint32_t hKV, uint32_t dh, uint32_t tmax,
+                            uint32_t own, void* stream)
+{
+    if (!qhat || !k_cache || !v_cache || !qfull || !slot_pos || !att || !workspace) return fail(QKK_EINVAL, "%s: null pointer", who);
+    if (int rc = check_shape(who, rows, hQ, hKV, dh, tmax)) return rc;
+    if (!aligned16(qhat) || !aligned16(k_cache) || !aligned16(v_cache) || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+        return fail(QKK_EINVAL, "%s: qhat and the caches must be 16-byte, workspace 256-byte aligned", who);
+    if (workspace_bytes < qkk_attn_workspace_bytes(rows, hQ, dh))
+        return fail(QKK_EWORKSPACE, "%s: workspace %zu < %zu bytes", who, workspace_bytes,
+                    qkk_attn_workspace_bytes(rows, hQ, dh));
+    if (int rc = require_device()) return rc;
+    hipStream_t st = as_stream(stream);
+    // two workgroups per CU over the (row, KV head) pairs, 8..64 ranges each: 16 slots x 4096 positions
+    // measured 4.5 TB/s with 16 ranges, 4.2 with 32, 3.1 with 128 (the partial results are traffic too);
+    // one slot 0.98 TB/s with 64 ranges, 0.80 with 32
+    const uint32_t n_ranges = std::min(ATT_MAX_RANGES, std::max(8u, persistent_blocks() / 2 / (rows * hKV)));
+    AttnWs ws;
+    ws.acc = (float*)workspace;
+    ws.ml = ws.acc + (size_t)rows * hQ * n_ranges * ATT_DH;
+    hipLaunchKernelGGL(attn_range_kernel, dim3(n_ranges, hKV, rows), dim3(256), 0, st, qhat, k_cache, v_cache, slot_pos, ws,
+                       hQ, hKV, hQ / hKV, tmax, own);
+    hipLaunchKernelGGL(attn_fold_kernel, dim3(hQ, rows), dim3(256), 0, st, ws, qfull, slot_pos, att, hQ, tmax, n_ranges);
+    return check_launch(who);
+}
+
 int qkk_attn_decode(const float* qhat, const float* k_cache, const float* v_cache, const float* qfull,
                     const uint32_t* slot_pos, float* att, void* workspace, size_t workspace_bytes, uint32_t n_slots,
                     uint32_t hQ, uint32_t hKV, uint32_t dh, uint32_t tmax, void* stream)
 {
-    if (!qhat || !k_cache || !v_cache || !qfull || !slot_pos || !att || !workspace)
-        return fail(QKK_EINVAL, "qkk_attn_decode: null pointer");
-    if (int rc = check_shape("qkk_attn_decode", n_slots, hQ, hKV, dh, tmax)) return rc;
-    if (!aligned16(qhat) || !aligned16(k_cache) || !aligned16(v_cache) || (reinterpret_cast<uintptr_t>(workspace) & 255u))
-        return fail(QKK_EINVAL, "qkk_attn_decode: qhat and the caches must be 16-byte, workspace 256-byte aligned");
-    if (workspace_bytes < qkk_attn_workspace_bytes(n_slots, hQ, dh))
-        return fail(QKK_EWORKSPACE, "qkk_attn_decode: workspace %zu < %zu bytes", workspace_bytes,
-                    qkk_attn_workspace_bytes(n_slots, hQ, dh));
-    if (int rc = require_device()) return rc;
-    hipStream_t st = as_stream(stream);
-    // two workgroups per CU over the (slot, KV head) pairs, 8..64 ranges each: 16 slots x 4096 positions
-    // measured 4.5 TB/s with 16 ranges, 4.2 with 32, 3.1 with 128 (the partial results are traffic too);
-    // one slot 0.98 TB/s with 64 ranges, 0.80 with 32
-    const uint32_t n_ranges = std::min(ATT_MAX_RANGES, std::max(8u, persistent_blocks() / 2 / (n_slots * hKV)));
-    AttnWs ws;
-    ws.acc = (float*)workspace;
-    ws.ml = ws.acc + (size_t)n_slots * hQ * n_ranges * ATT_DH;
-    hipLaunchKernelGGL(attn_range_kernel, dim3(n_ranges, hKV, n_slots), dim3(256), 0, st, qhat, k_cache, v_cache,
-                       slot_pos, ws, hQ, hKV, hQ / hKV, tmax);
-    hipLaunchKernelGGL(attn_fold_kernel, dim3(hQ, n_slots), dim3(256), 0, st, ws, qfull, slot_pos, att, hQ, tmax,
-                       n_ranges);
-    return check_launch("qkk_attn_decode");
+    return attn_decode_impl("qkk_attn_decode", qhat, k_cache, v_cache, qfull, slot_pos, att, workspace, workspace_bytes,
+                            n_slots, hQ, hKV, dh, tmax, 1, stream);
+}
+
+int qkk_attn_seq(const float* qhat, const float* k_cache, const float* v_cache, const float* qfull,
+                 const uint32_t* positions, float* att, void* workspace, size_t workspace_bytes, uint32_t n_pos, uint32_t hQ,
+                 uint32_t hKV, uint32_t dh, uint32_t tmax, void* stream)
+{
+    return attn_decode_impl("qkk_attn_seq", qhat, k_cache, v_cache, qfull, positions, att, workspace, workspace_bytes, n_pos,
+                            hQ, hKV, dh, tmax, 0, stream);
 }
 
 } // extern "C"

@@ -118,6 +118,88 @@ __global__ __launch_bounds__(128) void dn_step_kernel(const float* __restrict__ 
     att[((size_t)rq * hV + h) * DN_DS + j] = oj * scale * nw * (zv / (1.f + expf(-zv)));
 }
 
+// The same two steps over n_pos consecutive positions of ONE slot in one launch each (reference
+// shaders/dn_conv_batch.comp, dn_step_batch.comp + dn_gate_batch.comp): rows t of qkv / conv / gb /
+// z / att are positions, the window and the state stay in registers from one position to the next
+// and are written back once.  Per position the arithmetic is that of the one-position kernels; the
+// next position's inputs are requested before the current one is worked on.  Shared arrays are
+// double-buffered by the position's parity, so one barrier per use suffices.
+
+// grid (channels / dS), 128 threads.
+__global__ __launch_bounds__(128) void dn_conv_seq_kernel(float* __restrict__ st, const float* __restrict__ qkv,
+                                                          const float* __restrict__ ker, float* __restrict__ out,
+                                                          uint32_t channels, uint32_t qk_channels, float eps, uint32_t n_pos)
+{
+    __shared__ float s_red[2][2];
+    const uint32_t ch = blockIdx.x * DN_DS + threadIdx.x;
+    float* s = st + (size_t)ch * 3;
+    float s0 = s[0], s1 = s[1], s2 = s[2];
+    const float4 k = ((const float4*)ker)[ch];
+    const bool unit = blockIdx.x * DN_DS < qk_channels; // a q or k head (uniform)
+    float nxt = qkv[ch];
+    for (uint32_t t = 0; t < n_pos; t++) {
+        const float xin = nxt;
+        if (t + 1 < n_pos) nxt = qkv[(size_t)(t + 1) * channels + ch];
+        const float c = s0 * k.x + s1 * k.y + s2 * k.z + xin * k.w;
+        float v = c / (1.f + expf(-c));
+        s0 = s1; s1 = s2; s2 = xin;
+        if (unit) v *= 1.f / fmaxf(sqrtf(block_sum2(v * v, s_red[t & 1u])), eps);
+        out[(size_t)t * channels + ch] = v;
+    }
+    s[0] = s0; s[1] = s1; s[2] = s2;
+}
+
+// grid (hV), 128 threads: thread j = row j of the head's state, held in registers over all positions.
+__global__ __launch_bounds__(128) void dn_step_seq_kernel(const float* __restrict__ conv, const float* __restrict__ gb,
+                                                          float* __restrict__ state, const float* __restrict__ norm_w,
+                                                          const float* __restrict__ z, float* __restrict__ att, uint32_t hK,
+                                                          uint32_t hV, uint32_t kdiv, float eps, uint32_t n_pos)
+{
+    __shared__ float s_q[2][DN_DS], s_k[2][DN_DS];
+    __shared__ float s_red[2][2];
+    const uint32_t h = blockIdx.x, j = threadIdx.x;
+    const uint32_t kh = kdiv ? min(h / kdiv, hK - 1) : h % hK;
+    const size_t cstride = (size_t)(2 * hK + hV) * DN_DS;
+    float* S = state + (size_t)h * DN_DS * DN_DS;
+    float s[DN_DS];
+#pragma unroll
+    for (uint32_t i = 0; i < DN_DS; i++) s[i] = S[(size_t)i * DN_DS + j];
+    const float nw = norm_w[j], q_scale = 1.f / sqrtf((float)DN_DS);
+    float nq = conv[(size_t)kh * DN_DS + j], nk = conv[(size_t)(hK + kh) * DN_DS + j];
+    float nv = conv[(size_t)(2 * hK + h) * DN_DS + j], ng = gb[h], nb = gb[hV + h], nz = z[(size_t)h * DN_DS + j];
+    for (uint32_t t = 0; t < n_pos; t++) {
+        const uint32_t b = t & 1u;
+        s_q[b][j] = nq * q_scale;
+        s_k[b][j] = nk;
+        const float vj = nv, decay = expf(ng), beta = nb, zv = nz;
+        if (t + 1 < n_pos) {
+            const float* cv = conv + (size_t)(t + 1) * cstride;
+            nq = cv[(size_t)kh * DN_DS + j];
+            nk = cv[(size_t)(hK + kh) * DN_DS + j];
+            nv = cv[(size_t)(2 * hK + h) * DN_DS + j];
+            ng = gb[(size_t)(t + 1) * 2 * hV + h];
+            nb = gb[(size_t)(t + 1) * 2 * hV + hV + h];
+            nz = z[((size_t)(t + 1) * hV + h) * DN_DS + j];
+        }
+        __syncthreads();
+        float sk = 0.f;
+#pragma unroll
+        for (uint32_t i = 0; i < DN_DS; i++) sk += s[i] * s_k[b][i];
+        const float dj = beta * (vj - sk * decay);
+        float oj = 0.f;
+#pragma unroll
+        for (uint32_t i = 0; i < DN_DS; i++) {
+            const float sn = s[i] * decay + s_k[b][i] * dj;
+            s[i] = sn;
+            oj += sn * s_q[b][i];
+        }
+        const float scale = 1.f / sqrtf(block_sum2(oj * oj, s_red[b]) / (float)DN_DS + eps);
+        att[((size_t)t * hV + h) * DN_DS + j] = oj * scale * nw * (zv / (1.f + expf(-zv)));
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < DN_DS; i++) S[(size_t)i * DN_DS + j] = s[i];
+}
+
 static int check_slots(const char* who, uint32_t n_slots)
 {
     if (n_slots < 1 || n_slots > 65535) return fail(QKK_ESHAPE, "%s: %u slots outside 1..65535", who, n_slots);
@@ -163,6 +245,39 @@ int qkk_dn_conv(float* conv_state, const float* qkv, const float* ker, float* ou
     hipLaunchKernelGGL(dn_conv_kernel, dim3(channels / DN_DS, n_slots), dim3(DN_DS), 0, as_stream(stream), conv_state, qkv,
                        ker, out, channels, qk_channels, eps);
     return check_launch("qkk_dn_conv");
+}
+
+int qkk_dn_conv_seq(float* conv_state, const float* qkv, const float* ker, float* out, uint32_t channels, uint32_t d_state,
+                    uint32_t qk_channels, float eps, uint32_t n_pos, void* stream)
+{
+    if (!conv_state || !qkv || !ker || !out) return fail(QKK_EINVAL, "qkk_dn_conv_seq: null pointer");
+    if (n_pos < 1 || n_pos > (1u << 20)) return fail(QKK_ESHAPE, "qkk_dn_conv_seq: %u positions outside 1..2^20", n_pos);
+    if (d_state != DN_DS) return fail(QKK_ESHAPE, "qkk_dn_conv_seq: state size %u not supported (128)", d_state);
+    if (channels < DN_DS || channels % DN_DS || qk_channels % DN_DS || qk_channels > channels || channels > (1u << 24))
+        return fail(QKK_ESHAPE, "qkk_dn_conv_seq: %u channels (%u of q and k) must be whole heads of %u", channels,
+                    qk_channels, DN_DS);
+    if (!aligned16(ker)) return fail(QKK_EINVAL, "qkk_dn_conv_seq: ker must be 16-byte aligned");
+    if (!(eps >= 0.f)) return fail(QKK_EINVAL, "qkk_dn_conv_seq: eps must be non-negative");
+    if (int rc = require_device()) return rc;
+    hipLaunchKernelGGL(dn_conv_seq_kernel, dim3(channels / DN_DS), dim3(DN_DS), 0, as_stream(stream), conv_state, qkv, ker,
+                       out, channels, qk_channels, eps, n_pos);
+    return check_launch("qkk_dn_conv_seq");
+}
+
+int qkk_dn_step_seq(const float* conv, const float* gb, float* state, const float* norm_w, const float* z, float* att,
+                    uint32_t d_state, uint32_t hK, uint32_t hV, uint32_t kdiv, float eps, uint32_t n_pos, void* stream)
+{
+    if (!conv || !gb || !state || !norm_w || !z || !att) return fail(QKK_EINVAL, "qkk_dn_step_seq: null pointer");
+    if (n_pos < 1 || n_pos > (1u << 20)) return fail(QKK_ESHAPE, "qkk_dn_step_seq: %u positions outside 1..2^20", n_pos);
+    if (d_state != DN_DS) return fail(QKK_ESHAPE, "qkk_dn_step_seq: state size %u not supported (128)", d_state);
+    if (hK < 1 || hV < 1 || hV > 65535 || hK > 65535) return fail(QKK_ESHAPE, "qkk_dn_step_seq: head counts out of range");
+    if (kdiv ? (hV + kdiv - 1) / kdiv > hK : false)
+        return fail(QKK_ESHAPE, "qkk_dn_step_seq: %u value heads / %u exceed %u key heads", hV, kdiv, hK);
+    if (!(eps >= 0.f)) return fail(QKK_EINVAL, "qkk_dn_step_seq: eps must be non-negative");
+    if (int rc = require_device()) return rc;
+    hipLaunchKernelGGL(dn_step_seq_kernel, dim3(hV), dim3(DN_DS), 0, as_stream(stream), conv, gb, state, norm_w, z, att, hK,
+                       hV, kdiv, eps, n_pos);
+    return check_launch("qkk_dn_step_seq");
 }
 
 int qkk_dn_step(const float* conv, const float* gb, float* state, const float* norm_w, const float* z, float* att,

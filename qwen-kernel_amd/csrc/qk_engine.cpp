@@ -33,6 +33,7 @@ namespace {
 
 constexpr uint32_t N_EMBD = 2048;           // reference src/main.cpp:3086 (compile-time there too)
 constexpr uint32_t MAX_ROWS = QKK_MAX_SLOTS; // rows one device step carries
+constexpr uint32_t PF_ROWS = 128;            // positions of one slot a prefill pass carries (whole-model files)
 constexpr uint32_t N_STATE = 3;             // snapshot entries (reference default, stub/qk_stub.c:98)
 constexpr int ERR_DEVICE = -6;              // a launch, copy or synchronisation failed
 
@@ -99,6 +100,8 @@ struct qk_engine {
     uint32_t dn_kdiv = 0;        // 0: value head h reads key head h % hK; else h / dn_kdiv (src/main.cpp:3092-3094)
     uint32_t* d_pos = nullptr;   // [MAX_ROWS] position of the token fed this step
     uint32_t* h_pos = nullptr;   // pinned
+    uint32_t cap = MAX_ROWS;     // rows the step's buffers hold (PF_ROWS for whole-model files)
+    uint32_t *d_pf = nullptr, *h_pf = nullptr; // [3][PF_ROWS] ids, positions, sampled ids of a prefill pass (device / pinned)
     float* d_rope = nullptr;     // [n_ctx][FA_ROT/2][2]
     float *d_big = nullptr, *d_mid = nullptr, *d_kin = nullptr, *d_vin = nullptr, *d_gb = nullptr, *d_conv = nullptr,
           *d_qhat = nullptr, *d_att = nullptr, *d_mix = nullptr; // per-step rows of the mixers
@@ -119,8 +122,8 @@ struct qk_engine {
     bool upload(const qkg_tensor& t, const void** out, char* err, size_t err_len);
     void* dev_alloc(size_t bytes, bool zero);
     int launch_rows(uint32_t rows, float** final_rows);
-    int launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool want_head);
-    int feed_one(uint32_t slot, uint32_t tok, uint32_t pos, bool want_head);
+    int launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool want_head, bool seq);
+    int prefill(uint32_t slot, const uint32_t* toks, uint32_t n, uint32_t base, uint32_t* ids_out);
     int reset_slot(uint32_t slot);
     bool load_mixers(qkg_file* g, char* err, size_t err_len);
     int copy_state(uint32_t slot, uint32_t idx, bool save, uint32_t n_tok);
@@ -148,6 +151,7 @@ qk_engine::~qk_engine()
     if (h_ids) (void)hipHostFree(h_ids);
     if (h_tok) (void)hipHostFree(h_tok);
     if (h_pos) (void)hipHostFree(h_pos);
+    if (h_pf) (void)hipHostFree(h_pf);
     if (st) (void)hipStreamDestroy(st);
 }
 
@@ -207,39 +211,62 @@ static int dense(const Dense& d, const float* x, float* y, uint32_t rows, hipStr
     return qkk_gemv(d.type, d.w, x, y, d.M, d.K, rows, st);
 }
 
-// The launches of one step of a whole model over the slots [s0, s0 + rows): d_ids / d_pos -> d_tok
-// (reference src/main.cpp:4194-4419).  Every per-slot buffer is indexed from s0, so a single slot
-// can be stepped alone (batch prefill of a starting request, qk_stage_run) while the others rest.
-int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool want_head)
+// The launches of one pass of a whole model (reference src/main.cpp:4194-4419).
+//   seq = false: one decode step over the slots [s0, s0 + rows): d_ids / d_pos -> d_tok.  Every
+//                per-slot buffer is indexed from s0, so slots can be stepped apart from the others.
+//   seq = true:  `rows` consecutive positions of slot s0 (ids, positions, sampled ids in d_pf): the
+//                projections, norms and MoE blocks take all rows at once -- every weight is read once
+//                for the pass -- and the mixers run their sequence forms (one launch per kernel:
+//                the conv window and the recurrent state stay in registers over the positions,
+//                attention is causal over the rows).
+int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool want_head, bool seq)
 {
-    if (rows < 1 || s0 + rows > MAX_ROWS) return QKK_ESHAPE;
-    float* x = d_x + (size_t)s0 * N_EMBD;
-    const uint32_t* pos = d_pos + s0;
-    if (int rc = qkk_embed(embd_type, d_embd, embd_rows, N_EMBD, d_ids, MAX_ROWS, s0, 1, x, rows, st)) return rc;
+    if (rows < 1 || s0 >= MAX_ROWS || (seq ? rows > PF_ROWS : s0 + rows > MAX_ROWS)) return QKK_ESHAPE;
+    float* x = d_x;
+    const uint32_t* ids = seq ? d_pf : d_ids;
+    const uint32_t* pos = seq ? d_pf + PF_ROWS : d_pos + s0;
+    uint32_t* tok = seq ? d_pf + 2 * PF_ROWS : d_tok + s0;
+    if (int rc = qkk_embed(embd_type, d_embd, embd_rows, N_EMBD, ids, seq ? PF_ROWS : MAX_ROWS, seq ? 0 : s0, 1, x, rows, st))
+        return rc;
     if (int rc = qkk_rmsnorm(x, layers[0].attn_norm, d_xn[0], N_EMBD, rows, eps, st)) return rc;
     int cur = 0;
     for (size_t l = 0; l < layers.size(); l++) {
         const EngineLayer& L = layers[l];
         float* xn = d_xn[cur];
+        float *s1 = L.st1 + s0 * L.ps1, *s2 = L.st2 + s0 * L.ps2;
         if (L.kind == EngineLayer::RECURRENT) {
             if (int rc = dense(L.p1, xn, d_big, rows, st)) return rc;
             if (int rc = dense(L.p2, xn, d_mid, rows, st)) return rc;
             if (int rc = qkk_dn_ab(xn, L.alpha_w, L.beta_w, L.dt_bias, L.a_vec, d_gb, N_EMBD, DN_HV, rows, st)) return rc;
-            if (int rc = qkk_dn_conv(L.st1 + s0 * L.ps1, d_big, L.ker, d_conv, DN_CH, DN_DS, 2 * DN_HK * DN_DS, eps, rows, st))
-                return rc;
-            if (int rc = qkk_dn_step(d_conv, d_gb, L.st2 + s0 * L.ps2, L.ssm_norm, d_mid, d_att, DN_DS, DN_HK, DN_HV, dn_kdiv,
-                                     eps, rows, st))
-                return rc;
+            if (seq) {
+                if (int rc = qkk_dn_conv_seq(s1, d_big, L.ker, d_conv, DN_CH, DN_DS, 2 * DN_HK * DN_DS, eps, rows, st)) return rc;
+                if (int rc = qkk_dn_step_seq(d_conv, d_gb, s2, L.ssm_norm, d_mid, d_att, DN_DS, DN_HK, DN_HV, dn_kdiv, eps, rows,
+                                             st))
+                    return rc;
+            } else {
+                if (int rc = qkk_dn_conv(s1, d_big, L.ker, d_conv, DN_CH, DN_DS, 2 * DN_HK * DN_DS, eps, rows, st)) return rc;
+                if (int rc = qkk_dn_step(d_conv, d_gb, s2, L.ssm_norm, d_mid, d_att, DN_DS, DN_HK, DN_HV, dn_kdiv, eps, rows, st))
+                    return rc;
+            }
         } else {
             if (int rc = dense(L.p1, xn, d_big, rows, st)) return rc;
             if (int rc = dense(L.p2, xn, d_kin, rows, st)) return rc;
             if (int rc = dense(L.p3, xn, d_vin, rows, st)) return rc;
-            if (int rc = qkk_attn_prep(d_big, d_kin, d_vin, L.q_norm, L.k_norm, d_rope, pos, d_qhat, L.st1 + s0 * L.ps1,
-                                       L.st2 + s0 * L.ps2, rows, FA_HQ, FA_HKV, FA_DH, FA_ROT, n_ctx, eps, st))
-                return rc;
-            if (int rc = qkk_attn_decode(d_qhat, L.st1 + s0 * L.ps1, L.st2 + s0 * L.ps2, d_big, pos, d_att, d_aws, aws_bytes,
-                                         rows, FA_HQ, FA_HKV, FA_DH, n_ctx, st))
-                return rc;
+            if (seq) {
+                if (int rc = qkk_attn_prep_seq(d_big, d_kin, d_vin, L.q_norm, L.k_norm, d_rope, pos, d_qhat, s1, s2, rows, FA_HQ,
+                                               FA_HKV, FA_DH, FA_ROT, n_ctx, eps, st))
+                    return rc;
+                if (int rc = qkk_attn_seq(d_qhat, s1, s2, d_big, pos, d_att, d_aws, aws_bytes, rows, FA_HQ, FA_HKV, FA_DH, n_ctx,
+                                          st))
+                    return rc;
+            } else {
+                if (int rc = qkk_attn_prep(d_big, d_kin, d_vin, L.q_norm, L.k_norm, d_rope, pos, d_qhat, s1, s2, rows, FA_HQ,
+                                           FA_HKV, FA_DH, FA_ROT, n_ctx, eps, st))
+                    return rc;
+                if (int rc = qkk_attn_decode(d_qhat, s1, s2, d_big, pos, d_att, d_aws, aws_bytes, rows, FA_HQ, FA_HKV, FA_DH,
+                                             n_ctx, st))
+                    return rc;
+            }
         }
         if (int rc = dense(L.out, d_att, d_mix, rows, st)) return rc;
         // y = x + mixer, normalised for the MoE block; then x = y + MoE, normalised for the next layer
@@ -251,7 +278,37 @@ int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool 
     }
     if (final_rows) *final_rows = d_xn[cur];
     if (!want_head) return QKK_OK;
-    return qkk_head_argmax(d_head, d_xn[cur], d_tok + s0, nullptr, vocab, N_EMBD, rows, d_hws, hws_bytes, st);
+    for (uint32_t r0 = 0; r0 < rows; r0 += MAX_ROWS) // the head takes sixteen rows at a time
+        if (int rc = qkk_head_argmax(d_head, d_xn[cur] + (size_t)r0 * N_EMBD, tok + r0, nullptr, vocab, N_EMBD,
+                                     std::min(MAX_ROWS, rows - r0), d_hws, hws_bytes, st))
+            return rc;
+    return QKK_OK;
+}
+
+// Positions base .. base+n-1 of one slot, alone (the other slots' states are not touched), in
+// passes of PF_ROWS.  ids_out (optional): the greedy id after every position; the last position's
+// normalised row is kept for qk_stage_topk.
+int qk_engine::prefill(uint32_t slot, const uint32_t* toks, uint32_t n, uint32_t base, uint32_t* ids_out)
+{
+    for (uint32_t off = 0; off < n; off += PF_ROWS) {
+        const uint32_t rows = std::min(PF_ROWS, n - off);
+        for (uint32_t t = 0; t < rows; t++) {
+            h_pf[t] = toks[off + t];
+            h_pf[PF_ROWS + t] = base + off + t;
+        }
+        if (hipMemcpyAsync(d_pf, h_pf, 2 * PF_ROWS * sizeof(uint32_t), hipMemcpyHostToDevice, st) != hipSuccess)
+            return ERR_DEVICE;
+        float* fin = nullptr;
+        if (launch_full(rows, slot, &fin, ids_out != nullptr, true) != QKK_OK) return ERR_DEVICE;
+        if (ids_out && (hipMemcpyAsync(h_pf + 2 * PF_ROWS, d_pf + 2 * PF_ROWS, rows * sizeof(uint32_t), hipMemcpyDeviceToHost,
+                                       st) != hipSuccess ||
+                        hipMemcpyAsync(d_last, fin + (size_t)(rows - 1) * N_EMBD, N_EMBD * sizeof(float),
+                                       hipMemcpyDeviceToDevice, st) != hipSuccess))
+            return ERR_DEVICE;
+        if (hipStreamSynchronize(st) != hipSuccess) return ERR_DEVICE;
+        if (ids_out) memcpy(ids_out + off, h_pf + 2 * PF_ROWS, rows * sizeof(uint32_t));
+    }
+    return 0;
 }
 
 // Clears a slot's recurrent state (reference resetSlot, src/main.cpp:3416-3433); the KV rows of an
@@ -263,22 +320,6 @@ int qk_engine::reset_slot(uint32_t slot)
             (hipMemsetAsync(L.st1 + slot * L.ps1, 0, L.ps1 * sizeof(float), st) != hipSuccess ||
              hipMemsetAsync(L.st2 + slot * L.ps2, 0, L.ps2 * sizeof(float), st) != hipSuccess))
             return ERR_DEVICE;
-    return hipStreamSynchronize(st) == hipSuccess ? 0 : ERR_DEVICE;
-}
-
-// One token of one slot, alone, eagerly (the other slots' states are not touched).
-int qk_engine::feed_one(uint32_t slot, uint32_t tok, uint32_t pos, bool want_head)
-{
-    h_ids[slot] = tok;
-    h_pos[slot] = pos;
-    if (hipMemcpyAsync(d_ids + slot, h_ids + slot, 4, hipMemcpyHostToDevice, st) != hipSuccess ||
-        hipMemcpyAsync(d_pos + slot, h_pos + slot, 4, hipMemcpyHostToDevice, st) != hipSuccess)
-        return ERR_DEVICE;
-    float* fin = nullptr;
-    if (launch_full(1, slot, &fin, want_head) != QKK_OK) return ERR_DEVICE;
-    if (want_head && (hipMemcpyAsync(h_tok + slot, d_tok + slot, 4, hipMemcpyDeviceToHost, st) != hipSuccess ||
-                      hipMemcpyAsync(d_last, fin, N_EMBD * sizeof(float), hipMemcpyDeviceToDevice, st) != hipSuccess))
-        return ERR_DEVICE;
     return hipStreamSynchronize(st) == hipSuccess ? 0 : ERR_DEVICE;
 }
 
@@ -302,7 +343,7 @@ int qk_engine::copy_and_launch(uint32_t rows)
     if (full_model) {
         if (hipMemcpyAsync(d_pos, h_pos, rows * sizeof(uint32_t), hipMemcpyHostToDevice, st) != hipSuccess)
             return ERR_DEVICE;
-        if (launch_full(rows, 0, nullptr, true) != QKK_OK) return ERR_DEVICE;
+        if (launch_full(rows, 0, nullptr, true, false) != QKK_OK) return ERR_DEVICE;
     } else if (launch_rows(rows, nullptr) != QKK_OK) {
         return ERR_DEVICE;
     }
@@ -364,12 +405,16 @@ bool qk_engine::load_mixers(qkg_file* g, char* err, size_t err_len)
         L.st2 = (float*)dev_alloc(MAX_ROWS * L.ps2 * sizeof(float), true);
         if (!L.st1 || !L.st2) return bad("qk_open: device memory exhausted (per-slot state)");
     }
-    auto rows_of = [&](size_t n) { return (float*)dev_alloc(MAX_ROWS * n * sizeof(float), true); };
+    auto rows_of = [&](size_t n) { return (float*)dev_alloc(cap * n * sizeof(float), true); };
     d_big = rows_of(DN_CH); d_mid = rows_of(DN_IN); d_kin = rows_of(FA_HKV * FA_DH); d_vin = rows_of(FA_HKV * FA_DH);
     d_gb = rows_of(2 * DN_HV); d_conv = rows_of(DN_CH); d_qhat = rows_of(FA_HQ * FA_DH); d_att = rows_of(DN_IN);
     d_mix = rows_of(N_EMBD);
     d_pos = (uint32_t*)dev_alloc(MAX_ROWS * 4, true);
-    aws_bytes = qkk_attn_workspace_bytes(MAX_ROWS, FA_HQ, FA_DH);
+    d_pf = (uint32_t*)dev_alloc(3 * PF_ROWS * 4, true);
+    if (!d_pf || hipHostMalloc((void**)&h_pf, 3 * PF_ROWS * 4, hipHostMallocDefault) != hipSuccess)
+        return bad("qk_open: cannot allocate the prefill buffers");
+    memset(h_pf, 0, 3 * PF_ROWS * 4);
+    aws_bytes = qkk_attn_workspace_bytes(cap, FA_HQ, FA_DH);
     d_aws = dev_alloc(aws_bytes, true);
     d_rope = (float*)dev_alloc((size_t)n_ctx * FA_ROT * sizeof(float), false);
     if (!d_big || !d_mid || !d_kin || !d_vin || !d_gb || !d_conv || !d_qhat || !d_att || !d_mix || !d_pos || !d_aws || !d_rope)
@@ -540,10 +585,11 @@ bool qk_engine::open(const char* path, const qk_config& cfg, char* err, size_t e
         layers[l].post_norm = (const float*)p;
     }
 
-    for (const EngineLayer& L : layers) ws_bytes = std::max(ws_bytes, qkk_moe_workspace_bytes(&L.moe, MAX_ROWS));
+    cap = full_model ? PF_ROWS : MAX_ROWS;
+    for (const EngineLayer& L : layers) ws_bytes = std::max(ws_bytes, qkk_moe_workspace_bytes(&L.moe, cap));
     hws_bytes = qkk_head_workspace_bytes(vocab, MAX_ROWS);
     if (!ws_bytes || !hws_bytes) return bad("qk_open: expert shape unsupported by the kernels");
-    const size_t row_b = (size_t)MAX_ROWS * N_EMBD * sizeof(float);
+    const size_t row_b = (size_t)cap * N_EMBD * sizeof(float);
     d_ids = (uint32_t*)dev_alloc(MAX_ROWS * 4, true);
     d_tok = (uint32_t*)dev_alloc(MAX_ROWS * 4, true);
     d_x = (float*)dev_alloc(row_b, true);
@@ -551,7 +597,7 @@ bool qk_engine::open(const char* path, const qk_config& cfg, char* err, size_t e
     d_xn[1] = (float*)dev_alloc(row_b, true);
     d_last = (float*)dev_alloc(N_EMBD * sizeof(float), true);
     d_logits = (float*)dev_alloc((size_t)vocab * sizeof(float), true);
-    d_sel = (qkk_sel*)dev_alloc(MAX_ROWS * sizeof(qkk_sel), true);
+    d_sel = (qkk_sel*)dev_alloc(cap * sizeof(qkk_sel), true);
     d_ws = dev_alloc(ws_bytes, true);   // the kernels' workspaces start zero-filled
     d_hws = dev_alloc(hws_bytes, true);
     if (!d_ids || !d_tok || !d_x || !d_xn[0] || !d_xn[1] || !d_last || !d_logits || !d_sel || !d_ws || !d_hws)
@@ -672,11 +718,8 @@ int qk_engine::stage_run(uint32_t slot, const uint32_t* toks, const float* hidde
         if (toks[i] >= vocab) return -1;
     if (full_model) { // positions base .. base+n-1 of this slot, one after the other (the state is sequential)
         if (base == 0 && reset_slot(slot) != 0) return ERR_DEVICE; // base 0 starts from empty (reference src/main.cpp:4668-4675)
-        for (uint32_t i = 0; i < n; i++) {
-            if (int rc = feed_one(slot, toks[i], base + i, true)) return rc;
-            ids_out[i] = h_tok[slot];
-        }
-        last_run_rows = n; // feed_one left the final position's normalised row in d_last
+        if (int rc = prefill(slot, toks, n, base, ids_out)) return rc;
+        last_run_rows = n; // the final position's normalised row is in d_last
         return 0;
     }
     for (uint32_t off = 0; off < n; off += MAX_ROWS) {
@@ -775,11 +818,10 @@ int qk_slot_start(qk_engine* e, uint32_t slot, const uint32_t* prompt, uint32_t 
     }
     if (e->full_model) {
         // a fresh request: clear the previous occupant's recurrent state, then the prefilled
-        // positions, one token at a time on this slot alone (no batched-prefill kernels for the
-        // mixers here; the last prompt token is left to the serial step as in the reference)
+        // positions on this slot alone (the last prompt token is left to the serial step as in the
+        // reference)
         if (e->reset_slot(slot) != 0) return -6;
-        for (uint32_t p = 0; p < done; p++)
-            if (e->feed_one(slot, prompt[p], p, false) != 0) return -6;
+        if (done && e->prefill(slot, prompt, done, 0, nullptr) != 0) return -6;
     }
     s.cursor = done; s.pos = done;
     s.active = true;

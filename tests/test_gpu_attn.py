@@ -132,3 +132,56 @@ def test_attention_argument_checks(qk, dev):
     qk.attn_prep(z(1, HQ, 2 * DH) + 1, z(1, HKV, DH) + 1, z(1, HKV, DH) + 3, z(DH) + 1, z(DH) + 1, rope, big, kc, vc, NROT)
     torch.cuda.synchronize()
     assert float(vc[0, 0, 63, 0]) == 3.0 and float(vc[0, :, :63].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("tmax,base,n_pos", [(96, 0, 1), (96, 0, 70), (300, 150, 128), (4096, 3000, 40)])
+def test_attention_sequence_forms_equal_the_steps(qk, dev, tmax, base, n_pos):
+    """qkk_attn_prep_seq / qkk_attn_seq over n_pos consecutive positions of one slot whose cache
+    already holds `base` rows: row t sees the cache rows 0..base+t.  Against the decode-step entry
+    points called position by position (the same kernels; the number of position ranges depends on
+    the row count, so the sums are folded in another order) and, for the shorter cases, the CPU
+    mirror."""
+    import torch
+    print(f"[case] attention sequence tmax={tmax} base={base} n_pos={n_pos}", flush=True)
+    rng = np.random.default_rng(tmax + n_pos)
+    rope = OA.rope_table(tmax, NROT)
+    kc, vc = np.zeros((HKV, tmax, DH), np.float32), np.zeros((HKV, tmax, DH), np.float32)
+    kc[:, :base], vc[:, :base] = rng.standard_normal((HKV, base, DH)), rng.standard_normal((HKV, base, DH))
+    qn, kn = (1 + 0.2 * rng.standard_normal(DH)).astype(np.float32), (1 + 0.2 * rng.standard_normal(DH)).astype(np.float32)
+    qfull = rng.standard_normal((n_pos, HQ, 2 * DH)).astype(np.float32)
+    kin, vin = rng.standard_normal((n_pos, HKV, DH)).astype(np.float32), rng.standard_normal((n_pos, HKV, DH)).astype(np.float32)
+    up = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    roped, qnd, knd = up(rope), up(qn), up(kn)
+    qfd, kind, vind = up(qfull), up(kin), up(vin)
+    pos = torch.arange(base, base + n_pos, dtype=torch.int32, device=dev)
+    # position by position
+    k1, v1 = up(kc[None]), up(vc[None])
+    ws1 = torch.empty(qk.attn_workspace_bytes(1, HQ), dtype=torch.uint8, device=dev)
+    att1 = []
+    for t in range(n_pos):
+        qh = qk.attn_prep(qfd[t:t + 1], kind[t:t + 1], vind[t:t + 1], qnd, knd, roped, pos[t:t + 1], k1, v1, NROT)
+        att1.append(qk.attn_decode(qh, k1, v1, qfd[t:t + 1], pos[t:t + 1], ws1))
+    att1 = torch.cat(att1).cpu().numpy()
+    # one launch per kernel
+    k2, v2 = up(kc[None]), up(vc[None])
+    ws2 = torch.empty(qk.attn_workspace_bytes(n_pos, HQ), dtype=torch.uint8, device=dev)
+    qh2 = qk.attn_prep(qfd, kind, vind, qnd, knd, roped, pos, k2, v2, NROT, seq=True)
+    att2 = qk.attn_decode(qh2, k2, v2, qfd, pos, ws2, seq=True).cpu().numpy()
+    assert np.array_equal(k1.cpu().numpy(), k2.cpu().numpy()) and np.array_equal(v1.cpu().numpy(), v2.cpu().numpy())
+    assert rel(att2, att1) <= 1e-5, rel(att2, att1)   # the range count differs with the row count: not bitwise
+    if n_pos <= 70:
+        for t in range(n_pos):
+            want = OA.attend(OA.prep(qfull[t], kin[t], vin[t], qn, kn, rope, base + t, kc, vc, NROT), kc, vc, qfull[t], base + t)
+            assert rel(att2[t], want) <= TOL, t
+
+
+def test_attention_sequence_argument_checks(qk, dev):
+    import torch
+    z = lambda *s: torch.zeros(s, device=dev)
+    pos = torch.zeros(4, dtype=torch.int32, device=dev)
+    ws = torch.empty(qk.attn_workspace_bytes(1, HQ), dtype=torch.uint8, device=dev)
+    with pytest.raises(ValueError):        # four rows of a sequence share one cache
+        qk.attn_decode(z(4, HQ, DH), z(4, HKV, 64, DH), z(4, HKV, 64, DH), z(4, HQ, 2 * DH), pos, ws, seq=True)
+    with pytest.raises(qk.QkError) as e:   # a workspace for one row
+        qk.attn_decode(z(4, HQ, DH), z(1, HKV, 64, DH), z(1, HKV, 64, DH), z(4, HQ, 2 * DH), pos, ws, seq=True)
+    assert e.value.code == -5

@@ -106,3 +106,56 @@ def test_deltanet_argument_checks(qk, dev):
     with pytest.raises(qk.QkError) as e:      # pairing beyond the key heads
         qk.dn_step(z(1, (2 * 2 + 8) * DS), z(1, 16), z(1, 8, DS, DS), z(DS), z(1, 8 * DS), 2, 8, kdiv=2)
     assert e.value.code == -2
+
+
+@pytest.mark.parametrize("n_pos,kdiv", [(1, 0), (2, 0), (37, 2), (128, 0)])
+def test_deltanet_sequence_forms_equal_the_steps(qk, dev, n_pos, kdiv):
+    """qkk_dn_conv_seq / qkk_dn_step_seq over n_pos consecutive positions of one slot (a state of
+    earlier positions already in place): the outputs and the final window / state of n_pos calls of
+    the one-position kernels, and the CPU mirror's within tolerance."""
+    import torch
+    print(f"[case] deltanet sequence n_pos={n_pos} kdiv={kdiv}", flush=True)
+    w = Weights(23)
+    up = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    rng = np.random.default_rng(n_pos)
+    st = rng.standard_normal((1, w.ch, 3)).astype(F)
+    S = (rng.standard_normal((1, w.hv, DS, DS)) * 0.1).astype(F)
+    qkv = rng.standard_normal((n_pos, w.ch)).astype(F)
+    z = rng.standard_normal((n_pos, w.hv * DS)).astype(F)
+    gb = np.concatenate([-np.abs(rng.standard_normal((n_pos, w.hv))) * 0.3, rng.random((n_pos, w.hv))], axis=1).astype(F)
+    ker, nw = up(w.ker), up(w.norm_w)
+    # position by position
+    st1, S1 = up(st), up(np.ascontiguousarray(S.transpose(0, 1, 3, 2)))
+    conv1, att1 = [], []
+    for t in range(n_pos):
+        c = qk.dn_conv(st1, up(qkv[t:t + 1]), ker, w.qk)
+        conv1.append(c)
+        att1.append(qk.dn_step(c, up(gb[t:t + 1]), S1, nw, up(z[t:t + 1]), w.hk, w.hv, kdiv=kdiv))
+    # all positions in one launch each
+    st2, S2 = up(st), up(np.ascontiguousarray(S.transpose(0, 1, 3, 2)))
+    conv2 = qk.dn_conv(st2, up(qkv), ker, w.qk, seq=True)
+    att2 = qk.dn_step(conv2, up(gb), S2, nw, up(z), w.hk, w.hv, kdiv=kdiv, seq=True)
+    torch.cuda.synchronize()
+    conv1, att1 = torch.cat(conv1).cpu().numpy(), torch.cat(att1).cpu().numpy()
+    conv2, att2 = conv2.cpu().numpy(), att2.cpu().numpy()
+    assert np.array_equal(st1.cpu().numpy(), st2.cpu().numpy())
+    assert rel(conv2, conv1) <= 1e-6 and rel(att2, att1) <= 1e-5, (rel(conv2, conv1), rel(att2, att1))
+    assert rel(S2.cpu().numpy(), S1.cpu().numpy()) <= 1e-5
+    print(f"[info] sequence vs steps: conv {rel(conv2, conv1):.1e} att {rel(att2, att1):.1e}", flush=True)
+    if n_pos <= 37:   # and the CPU mirror
+        so, So = st[0].copy(), S[0].copy()
+        for t in range(n_pos):
+            c = OD.conv(so, qkv[t], w.ker, DS, w.qk)
+            a = OD.step(c, gb[t, :w.hv], gb[t, w.hv:], So, w.norm_w, z[t], w.hk, w.hv, kdiv=kdiv)
+            assert rel(conv2[t], c) <= 1e-5 and rel(att2[t], a) <= TOL, t
+        assert rel(S2.cpu().numpy()[0].transpose(0, 2, 1), So) <= TOL
+
+
+def test_deltanet_sequence_argument_checks(qk, dev):
+    import torch
+    w = Weights(3)
+    z = lambda *s: torch.zeros(s, dtype=torch.float32, device=dev)
+    with pytest.raises(ValueError):   # a state of two slots is not a sequence's
+        qk.dn_step(z(4, w.ch), z(4, 2 * w.hv), z(2, w.hv, DS, DS), z(DS), z(4, w.hv * DS), w.hk, w.hv, seq=True)
+    with pytest.raises(qk.QkError):
+        qk.dn_step(z(4, w.ch), z(4, 2 * w.hv), z(1, w.hv, 64, 64), z(64), z(4, w.hv * 64), w.hk, w.hv, d_state=64, seq=True)

@@ -124,3 +124,24 @@ def test_whole_model_stage_run_and_snapshots(qk, full):
         rc, again = eng.stage_run(1, toks[6:], 6)
         assert rc == 0 and again == tail
         assert eng.state_save(1, 3, 0) == -1 and eng.state_load(2, 0, 0) == -1
+
+
+def test_whole_model_long_prompt_and_long_stage_run(qk, full):
+    """A prompt longer than one prefill pass (128 positions go through the projections and the MoE
+    blocks together, the mixers position by position), then the rest, then the serial steps: the
+    same stream as the oracle fed one token at a time.  qk_stage_run over 40 positions returns the
+    oracle's id after every one of them."""
+    model, path = full
+    print("[case] whole model, 150-token prompt and a 40-position stage run", flush=True)
+    rng = np.random.default_rng(21)
+    prompt = [int(t) for t in rng.integers(0, VOCAB, 150)]
+    with qk.engine.Engine(path, n_slots=2, n_ctx=192, chunk=4) as eng:
+        chk = Checked(model, 2, 192)
+        ref = OE.SlotMachine(chk, VOCAB, VOCAB + 5, 2, 192, 4)
+        drive(eng, ref, {0: [("start", 1, prompt, 6, 0)], 1: [("start", 0, prompt[:40], 3, 0)]}, 3)
+        assert not any(sl["active"] for sl in ref.slots)
+        print(f"[info] narrowest top-2 gap / largest logit: {chk.narrowest:.2e}", flush=True)
+        o = OE.FullModelOracle(model, 1, 192)
+        want = [o.feed(0, t, p) for p, t in enumerate(prompt[:40])]
+        rc, ids = eng.stage_run(0, prompt[:40], 0)
+        assert rc == 0 and ids == want
