@@ -317,11 +317,12 @@ def deltanet_workload(qk, n_slots, steps, warmup, seed=6):
     return dict(ms_event=ev, steps=n, ring=ring, bytes_step=2 * n_slots * hV * dS * dS * 4)
 
 
-def engine_workload(qk, n_layer, slots_list, chunks, warm_chunks, seed=31, kinds=None):
+def engine_workload(qk, n_layer, slots_list, chunks, warm_chunks, seed=31, kinds=None, prefill_only=0):
     """Tokens per second through the engine ABI (qk_open / qk_slot_start / qk_step_chunk) on a
     synthetic model file at the full layer shape and vocabulary: host wall clock over whole chunks,
     host synchronisation after every step included.  kinds = None: MoE-only layers; else one letter
     per layer, "R" gated DeltaNet or "A" full attention in front of each MoE block (a whole model).
+    prefill_only = P: no decode steps, P positions through qk_stage_run four times instead.
     Two distinct layers' MoE weights alternate through the file; each layer has its own copy in
     device memory."""
     import shutil
@@ -354,23 +355,24 @@ def engine_workload(qk, n_layer, slots_list, chunks, warm_chunks, seed=31, kinds
                             sys.exit(f"bench.py: qk_step_chunk returned {rc}")
                         toks += sum(len(v) for v in out.values())
                     return toks
-                run(warm_chunks)
+                if not prefill_only:
+                    run(warm_chunks)
                 t0 = time.perf_counter()
-                toks = run(chunks)
+                toks = 0 if prefill_only else run(chunks)
                 dt = time.perf_counter() - t0
                 pre = {}
                 if kinds is not None and n_slots == slots_list[0]:
                     # prompt positions per second: qk_stage_run over 512 positions of one slot, twice
                     # (the first pass warms the prefill path's launch set-up)
-                    ptoks = [(7 * i + 3) % 151000 for i in range(512)]
-                    for _ in range(2):
+                    ptoks = [(7 * i + 3) % 151000 for i in range(prefill_only or 512)]
+                    for _ in range(4 if prefill_only else 2):
                         tp = time.perf_counter()
                         rcp, _ids = eng.stage_run(0, ptoks, 0)
                         tp = time.perf_counter() - tp
                         if rcp != 0:
                             sys.exit(f"bench.py: qk_stage_run returned {rcp}")
                     pre = dict(prefill_tok_per_s=len(ptoks) / tp, prefill_positions=len(ptoks))
-            res[f"slots_{n_slots}"] = dict(tok_per_s=toks / dt, us_per_step=dt / (chunks * 32) * 1e6, tokens=toks,
+            res[f"slots_{n_slots}"] = dict(tok_per_s=toks / dt, us_per_step=dt / (max(chunks, 1) * 32) * 1e6, tokens=toks,
                                            open_s=t_open, **pre)
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
@@ -442,6 +444,12 @@ def main():
         print(json.dumps(dict(metric="engine_decode_tok_per_s", value=r["slots_16"]["tok_per_s"], unit="tok/s", n_gpus=1,
                               higher_is_better=True, data="synthetic", dtype="f32",
                               config=dict(workload="engine_whole_model", **r["config"]), detail=r)), flush=True)
+        return
+    if a.workload == "engine_prefill":   # prompt positions through qk_stage_run on a whole model
+        r = engine_workload(qk, a.layers, (1,), 0, 0, kinds=("RRRA" * ((a.layers + 3) // 4))[:a.layers], prefill_only=1024)
+        print(json.dumps(dict(metric="engine_prefill_tok_per_s", value=r["slots_1"]["prefill_tok_per_s"], unit="tok/s",
+                              n_gpus=1, higher_is_better=True, data="synthetic", dtype="f32",
+                              config=dict(workload="engine_prefill", positions=1024, **r["config"]), detail=r)), flush=True)
         return
     if a.workload == "engine_decode":   # the engine ABI alone (for kernel traces of its graph replays)
         r = engine_workload(qk, 8, (1, 4, 16), 8, 2)

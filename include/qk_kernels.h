@@ -291,8 +291,12 @@ int qkk_dn_step(const float *conv, const float *gb, float *state, const float *n
  *                    call and everything the cache held before.  Every row scans the cache for
  *                    itself (served from the L2 / last-level cache, but not a query-blocked scan as
  *                    the reference's). workspace: qkk_attn_workspace_bytes(n_pos, hQ, dh).
- * qkk_dn_conv_seq / qkk_dn_step_seq  the input window / the state stay in registers over all
- *                    positions and are written back once; one launch each. */
+ * qkk_dn_conv_seq    the conv is a 4-tap filter over the inputs, so all positions run in parallel
+ *                    (bit-identical to the steps); the window is moved on by a second small launch.
+ * qkk_dn_step_seq    the state is read once, kept in registers over all positions (16 rows of a head
+ *                    per workgroup, 8 lanes per row) and written once; q, k, v and the gates are
+ *                    staged through LDS 16 positions at a time; the head norm and output gate run
+ *                    as a second launch over (head, position).  conv 16-byte aligned, n_pos <= 65535. */
 int qkk_attn_prep_seq(const float *qfull, const float *kin, const float *vin, const float *q_norm_w,
                       const float *k_norm_w, const float *rope, const uint32_t *positions, float *qhat,
                       float *k_cache, float *v_cache, uint32_t n_pos, uint32_t hQ, uint32_t hKV,

@@ -118,86 +118,181 @@ __global__ __launch_bounds__(128) void dn_step_kernel(const float* __restrict__ 
     att[((size_t)rq * hV + h) * DN_DS + j] = oj * scale * nw * (zv / (1.f + expf(-zv)));
 }
 
-// The same two steps over n_pos consecutive positions of ONE slot in one launch each (reference
+// The same two steps over n_pos consecutive positions of ONE slot (reference
 // shaders/dn_conv_batch.comp, dn_step_batch.comp + dn_gate_batch.comp): rows t of qkv / conv / gb /
-// z / att are positions, the window and the state stay in registers from one position to the next
-// and are written back once.  Per position the arithmetic is that of the one-position kernels; the
-// next position's inputs are requested before the current one is worked on.  Shared arrays are
-// double-buffered by the position's parity, so one barrier per use suffices.
+// z / att are positions; the window and the state are read once and written once.
 
-// grid (channels / dS), 128 threads.
-__global__ __launch_bounds__(128) void dn_conv_seq_kernel(float* __restrict__ st, const float* __restrict__ qkv,
+// The conv is a 4-tap filter over the inputs, not a recurrence: position t needs the inputs t-3..t,
+// the first three positions taking the missing ones from the window.  grid (channels / dS, positions),
+// 128 threads; the window itself is moved on by dn_window_seq_kernel afterwards.
+__global__ __launch_bounds__(128) void dn_conv_seq_kernel(const float* __restrict__ st, const float* __restrict__ qkv,
                                                           const float* __restrict__ ker, float* __restrict__ out,
-                                                          uint32_t channels, uint32_t qk_channels, float eps, uint32_t n_pos)
+                                                          uint32_t channels, uint32_t qk_channels, float eps)
 {
-    __shared__ float s_red[2][2];
-    const uint32_t ch = blockIdx.x * DN_DS + threadIdx.x;
-    float* s = st + (size_t)ch * 3;
-    float s0 = s[0], s1 = s[1], s2 = s[2];
+    __shared__ float s_red[2];
+    const uint32_t ch = blockIdx.x * DN_DS + threadIdx.x, t = blockIdx.y;
+    auto input = [&](int u) { return u >= 0 ? qkv[(size_t)u * channels + ch] : st[(size_t)ch * 3 + (3 + u)]; };
+    const float s0 = input((int)t - 3), s1 = input((int)t - 2), s2 = input((int)t - 1), xin = input((int)t);
     const float4 k = ((const float4*)ker)[ch];
-    const bool unit = blockIdx.x * DN_DS < qk_channels; // a q or k head (uniform)
-    float nxt = qkv[ch];
-    for (uint32_t t = 0; t < n_pos; t++) {
-        const float xin = nxt;
-        if (t + 1 < n_pos) nxt = qkv[(size_t)(t + 1) * channels + ch];
-        const float c = s0 * k.x + s1 * k.y + s2 * k.z + xin * k.w;
-        float v = c / (1.f + expf(-c));
-        s0 = s1; s1 = s2; s2 = xin;
-        if (unit) v *= 1.f / fmaxf(sqrtf(block_sum2(v * v, s_red[t & 1u])), eps);
-        out[(size_t)t * channels + ch] = v;
-    }
-    s[0] = s0; s[1] = s1; s[2] = s2;
+    const float c = s0 * k.x + s1 * k.y + s2 * k.z + xin * k.w;
+    float v = c / (1.f + expf(-c));
+    if (blockIdx.x * DN_DS < qk_channels) // a q or k head (uniform): unit length
+        v *= 1.f / fmaxf(sqrtf(block_sum2(v * v, s_red)), eps);
+    out[(size_t)t * channels + ch] = v;
 }
 
-// grid (hV), 128 threads: thread j = row j of the head's state, held in registers over all positions.
-__global__ __launch_bounds__(128) void dn_step_seq_kernel(const float* __restrict__ conv, const float* __restrict__ gb,
-                                                          float* __restrict__ state, const float* __restrict__ norm_w,
-                                                          const float* __restrict__ z, float* __restrict__ att, uint32_t hK,
-                                                          uint32_t hV, uint32_t kdiv, float eps, uint32_t n_pos)
+// grid (channels / dS), 128 threads: the window after n_pos positions = the last three inputs.
+__global__ __launch_bounds__(128) void dn_window_seq_kernel(float* __restrict__ st, const float* __restrict__ qkv,
+                                                            uint32_t channels, uint32_t n_pos)
 {
-    __shared__ float s_q[2][DN_DS], s_k[2][DN_DS];
-    __shared__ float s_red[2][2];
-    const uint32_t h = blockIdx.x, j = threadIdx.x;
+    const uint32_t ch = blockIdx.x * DN_DS + threadIdx.x;
+    float* s = st + (size_t)ch * 3;
+    auto input = [&](int u) { return u >= 0 ? qkv[(size_t)u * channels + ch] : s[3 + u]; };
+    const float a = input((int)n_pos - 3), b = input((int)n_pos - 2), c = input((int)n_pos - 1);
+    s[0] = a; s[1] = b; s[2] = c;
+}
+
+// The delta rule over the positions is one serial chain per state row, and a head has only dS rows:
+// a workgroup per head would leave most of the chip idle and spend ~3 dS multiply-adds per thread
+// and position.  So a head is cut into SEQ_RB-row blocks (hV * dS / SEQ_RB workgroups) and every row
+// into SEQ_NQ parts of its columns: thread (row r, part c) keeps dS/SEQ_NQ state values and the two
+// sums over columns are finished across the SEQ_NQ neighbouring lanes.  q, k, v and the gates of
+// SEQ_CH positions at a time are staged in LDS (double-buffered; the next chunk's global loads are
+// in flight while the current one is worked on), one barrier per chunk.  The head-wide norm and the
+// output gate need all rows of a head and run as a second kernel over (head, position).
+constexpr uint32_t SEQ_NQ = 8;               // lanes per state row
+constexpr uint32_t SEQ_RB = 128 / SEQ_NQ;    // state rows per workgroup of 128 threads
+constexpr uint32_t SEQ_CH = 16;              // positions per staged chunk
+constexpr uint32_t SEQ_QS = DN_DS / SEQ_NQ;  // columns per part
+constexpr uint32_t SEQ_PAD = SEQ_QS + 4;     // part stride in LDS: the parts' float4 reads hit distinct banks
+constexpr uint32_t SEQ_TOTAL = SEQ_CH * (2 * DN_DS + SEQ_RB) / 4; // float4 loads per chunk
+constexpr uint32_t SEQ_ITEMS = (SEQ_TOTAL + 127) / 128;           // per thread
+static_assert(2 * SEQ_CH <= 128 && (SEQ_NQ == 4 || SEQ_NQ == 8), "chunk staging");
+
+struct SeqChunk {
+    float q[SEQ_CH][SEQ_NQ * SEQ_PAD];
+    float k[SEQ_CH][SEQ_NQ * SEQ_PAD];
+    float v[SEQ_CH][SEQ_RB];
+    float g[SEQ_CH][2]; // decay = exp(log decay), write strength
+};
+
+// grid (hV * dS / SEQ_RB), 128 threads.  att receives the raw o_j; dn_gate_seq_kernel finishes it.
+__global__ __launch_bounds__(128) void dn_step_seq_kernel(const float* __restrict__ conv, const float* __restrict__ gb,
+                                                          float* __restrict__ state, float* __restrict__ att, uint32_t hK,
+                                                          uint32_t hV, uint32_t kdiv, uint32_t n_pos)
+{
+    __shared__ __attribute__((aligned(16))) SeqChunk s_c[2];
+    constexpr uint32_t BPH = DN_DS / SEQ_RB, PER_POS = (2 * DN_DS + SEQ_RB) / 4;
+    const uint32_t h = blockIdx.x / BPH, rb = blockIdx.x % BPH, tid = threadIdx.x;
+    const uint32_t r = tid / SEQ_NQ, c = tid % SEQ_NQ, row = rb * SEQ_RB + r;
     const uint32_t kh = kdiv ? min(h / kdiv, hK - 1) : h % hK;
     const size_t cstride = (size_t)(2 * hK + hV) * DN_DS;
-    float* S = state + (size_t)h * DN_DS * DN_DS;
-    float s[DN_DS];
+    const float q_scale = 1.f / sqrtf((float)DN_DS);
+    float* S = state + (size_t)h * DN_DS * DN_DS; // column-major: (row, column i) at [i][row]
+    float s[SEQ_QS];
 #pragma unroll
-    for (uint32_t i = 0; i < DN_DS; i++) s[i] = S[(size_t)i * DN_DS + j];
-    const float nw = norm_w[j], q_scale = 1.f / sqrtf((float)DN_DS);
-    float nq = conv[(size_t)kh * DN_DS + j], nk = conv[(size_t)(hK + kh) * DN_DS + j];
-    float nv = conv[(size_t)(2 * hK + h) * DN_DS + j], ng = gb[h], nb = gb[hV + h], nz = z[(size_t)h * DN_DS + j];
-    for (uint32_t t = 0; t < n_pos; t++) {
-        const uint32_t b = t & 1u;
-        s_q[b][j] = nq * q_scale;
-        s_k[b][j] = nk;
-        const float vj = nv, decay = expf(ng), beta = nb, zv = nz;
-        if (t + 1 < n_pos) {
-            const float* cv = conv + (size_t)(t + 1) * cstride;
-            nq = cv[(size_t)kh * DN_DS + j];
-            nk = cv[(size_t)(hK + kh) * DN_DS + j];
-            nv = cv[(size_t)(2 * hK + h) * DN_DS + j];
-            ng = gb[(size_t)(t + 1) * 2 * hV + h];
-            nb = gb[(size_t)(t + 1) * 2 * hV + hV + h];
-            nz = z[((size_t)(t + 1) * hV + h) * DN_DS + j];
+    for (uint32_t i = 0; i < SEQ_QS; i++) s[i] = S[(size_t)(c * SEQ_QS + i) * DN_DS + row];
+
+    float4 pre[SEQ_ITEMS];
+    float pre_g = 0.f;
+    // item x of a chunk: position x / PER_POS; word w = x % PER_POS: float4 w of q, w - 32 of k, w - 64 of the block's v
+    auto fetch = [&](uint32_t t0) {
+#pragma unroll
+        for (uint32_t it = 0; it < SEQ_ITEMS; it++) {
+            const uint32_t x = min(tid + 128 * it, SEQ_TOTAL - 1), p = x / PER_POS, w = x % PER_POS;
+            const uint32_t t = min(t0 + p, n_pos - 1); // positions beyond the end repeat the last one, unused
+            const float* cv = conv + (size_t)t * cstride;
+            const float* src = w < DN_DS / 4       ? cv + (size_t)kh * DN_DS + 4 * w
+                               : w < 2 * DN_DS / 4 ? cv + (size_t)(hK + kh) * DN_DS + 4 * (w - DN_DS / 4)
+                                                   : cv + (size_t)(2 * hK + h) * DN_DS + rb * SEQ_RB + 4 * (w - 2 * DN_DS / 4);
+            pre[it] = *(const float4*)src;
         }
+        if (tid < 2 * SEQ_CH) {
+            const uint32_t t = min(t0 + (tid >> 1), n_pos - 1);
+            pre_g = gb[(size_t)t * 2 * hV + (tid & 1u) * hV + h];
+        }
+    };
+    auto stage = [&](uint32_t b) {
+#pragma unroll
+        for (uint32_t it = 0; it < SEQ_ITEMS; it++) {
+            const uint32_t x = tid + 128 * it, p = x / PER_POS, w = x % PER_POS;
+            float4 v = pre[it];
+            if (x >= SEQ_TOTAL) {
+            } else if (w < DN_DS / 4) {
+                v.x *= q_scale; v.y *= q_scale; v.z *= q_scale; v.w *= q_scale;
+                *(float4*)&s_c[b].q[p][(4 * w / SEQ_QS) * SEQ_PAD + 4 * w % SEQ_QS] = v;
+            } else if (w < 2 * DN_DS / 4) {
+                const uint32_t e = 4 * (w - DN_DS / 4);
+                *(float4*)&s_c[b].k[p][(e / SEQ_QS) * SEQ_PAD + e % SEQ_QS] = v;
+            } else {
+                *(float4*)&s_c[b].v[p][4 * (w - 2 * DN_DS / 4)] = v;
+            }
+        }
+        if (tid < 2 * SEQ_CH) s_c[b].g[tid >> 1][tid & 1u] = (tid & 1u) ? pre_g : expf(pre_g);
+    };
+
+    fetch(0);
+    stage(0);
+    __syncthreads();
+    for (uint32_t t0 = 0; t0 < n_pos; t0 += SEQ_CH) {
+        const uint32_t b = (t0 / SEQ_CH) & 1u;
+        const bool more = t0 + SEQ_CH < n_pos;
+        if (more) fetch(t0 + SEQ_CH);
+        const uint32_t np = min(SEQ_CH, n_pos - t0);
+        auto position = [&](uint32_t p) {
+            const float4* k4 = (const float4*)&s_c[b].k[p][c * SEQ_PAD];
+            const float4* q4 = (const float4*)&s_c[b].q[p][c * SEQ_PAD];
+            const float decay = s_c[b].g[p][0], beta = s_c[b].g[p][1], vj = s_c[b].v[p][r];
+            float4 kk[SEQ_QS / 4];
+            float4 ps = float4{0.f, 0.f, 0.f, 0.f}; // four independent sums: the chain of multiply-adds is the critical path
+#pragma unroll
+            for (uint32_t i = 0; i < SEQ_QS / 4; i++) {
+                kk[i] = k4[i];
+                ps.x += s[4 * i] * kk[i].x; ps.y += s[4 * i + 1] * kk[i].y;
+                ps.z += s[4 * i + 2] * kk[i].z; ps.w += s[4 * i + 3] * kk[i].w;
+            }
+            float sk = (ps.x + ps.y) + (ps.z + ps.w);
+            sk += dpp_f<DPP_XOR1>(sk);
+            sk += dpp_f<DPP_XOR2>(sk);
+            if (SEQ_NQ == 8) sk += dpp_f<DPP_HALF_MIRROR>(sk);
+            const float dj = beta * (vj - sk * decay);
+            float4 po = float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (uint32_t i = 0; i < SEQ_QS / 4; i++) {
+                const float4 qq = q4[i];
+                const float a0 = s[4 * i] * decay + kk[i].x * dj, a1 = s[4 * i + 1] * decay + kk[i].y * dj;
+                const float a2 = s[4 * i + 2] * decay + kk[i].z * dj, a3 = s[4 * i + 3] * decay + kk[i].w * dj;
+                s[4 * i] = a0; s[4 * i + 1] = a1; s[4 * i + 2] = a2; s[4 * i + 3] = a3;
+                po.x += a0 * qq.x; po.y += a1 * qq.y; po.z += a2 * qq.z; po.w += a3 * qq.w;
+            }
+            float oj = (po.x + po.y) + (po.z + po.w);
+            oj += dpp_f<DPP_XOR1>(oj);
+            oj += dpp_f<DPP_XOR2>(oj);
+            if (SEQ_NQ == 8) oj += dpp_f<DPP_HALF_MIRROR>(oj);
+            if (c == 0) att[((size_t)(t0 + p) * hV + h) * DN_DS + row] = oj;
+        };
+        if (np == SEQ_CH) { // whole chunk: unrolled, so that the next position's LDS reads can start early
+#pragma unroll 4
+            for (uint32_t p = 0; p < SEQ_CH; p++) position(p);
+        } else {
+            for (uint32_t p = 0; p < np; p++) position(p);
+        }
+        if (more) stage(b ^ 1u);
         __syncthreads();
-        float sk = 0.f;
-#pragma unroll
-        for (uint32_t i = 0; i < DN_DS; i++) sk += s[i] * s_k[b][i];
-        const float dj = beta * (vj - sk * decay);
-        float oj = 0.f;
-#pragma unroll
-        for (uint32_t i = 0; i < DN_DS; i++) {
-            const float sn = s[i] * decay + s_k[b][i] * dj;
-            s[i] = sn;
-            oj += sn * s_q[b][i];
-        }
-        const float scale = 1.f / sqrtf(block_sum2(oj * oj, s_red[b]) / (float)DN_DS + eps);
-        att[((size_t)t * hV + h) * DN_DS + j] = oj * scale * nw * (zv / (1.f + expf(-zv)));
     }
 #pragma unroll
-    for (uint32_t i = 0; i < DN_DS; i++) S[(size_t)i * DN_DS + j] = s[i];
+    for (uint32_t i = 0; i < SEQ_QS; i++) S[(size_t)(c * SEQ_QS + i) * DN_DS + row] = s[i];
+}
+
+// grid (hV, positions), 128 threads: att <- att / rms(att over the head) * norm_w * silu(z), in place.
+__global__ __launch_bounds__(128) void dn_gate_seq_kernel(float* __restrict__ att, const float* __restrict__ norm_w,
+                                                          const float* __restrict__ z, uint32_t hV, float eps)
+{
+    __shared__ float s_red[2];
+    const size_t at = ((size_t)blockIdx.y * hV + blockIdx.x) * DN_DS + threadIdx.x;
+    const float oj = att[at], zv = z[at], nw = norm_w[threadIdx.x];
+    const float scale = 1.f / sqrtf(block_sum2(oj * oj, s_red) / (float)DN_DS + eps);
+    att[at] = oj * scale * nw * (zv / (1.f + expf(-zv)));
 }
 
 static int check_slots(const char* who, uint32_t n_slots)
@@ -259,8 +354,11 @@ int qkk_dn_conv_seq(float* conv_state, const float* qkv, const float* ker, float
     if (!aligned16(ker)) return fail(QKK_EINVAL, "qkk_dn_conv_seq: ker must be 16-byte aligned");
     if (!(eps >= 0.f)) return fail(QKK_EINVAL, "qkk_dn_conv_seq: eps must be non-negative");
     if (int rc = require_device()) return rc;
-    hipLaunchKernelGGL(dn_conv_seq_kernel, dim3(channels / DN_DS), dim3(DN_DS), 0, as_stream(stream), conv_state, qkv, ker,
-                       out, channels, qk_channels, eps, n_pos);
+    if (n_pos > 65535) return fail(QKK_ESHAPE, "qkk_dn_conv_seq: %u positions above 65535", n_pos);
+    hipLaunchKernelGGL(dn_conv_seq_kernel, dim3(channels / DN_DS, n_pos), dim3(DN_DS), 0, as_stream(stream), conv_state, qkv,
+                       ker, out, channels, qk_channels, eps);
+    hipLaunchKernelGGL(dn_window_seq_kernel, dim3(channels / DN_DS), dim3(DN_DS), 0, as_stream(stream), conv_state, qkv,
+                       channels, n_pos);
     return check_launch("qkk_dn_conv_seq");
 }
 
@@ -275,8 +373,11 @@ int qkk_dn_step_seq(const float* conv, const float* gb, float* state, const floa
         return fail(QKK_ESHAPE, "qkk_dn_step_seq: %u value heads / %u exceed %u key heads", hV, kdiv, hK);
     if (!(eps >= 0.f)) return fail(QKK_EINVAL, "qkk_dn_step_seq: eps must be non-negative");
     if (int rc = require_device()) return rc;
-    hipLaunchKernelGGL(dn_step_seq_kernel, dim3(hV), dim3(DN_DS), 0, as_stream(stream), conv, gb, state, norm_w, z, att, hK,
-                       hV, kdiv, eps, n_pos);
+    if (!aligned16(conv) || n_pos > 65535)
+        return fail(QKK_EINVAL, "qkk_dn_step_seq: conv must be 16-byte aligned and n_pos at most 65535");
+    hipLaunchKernelGGL(dn_step_seq_kernel, dim3(hV * (DN_DS / SEQ_RB)), dim3(128), 0, as_stream(stream), conv, gb, state, att,
+                       hK, hV, kdiv, n_pos);
+    hipLaunchKernelGGL(dn_gate_seq_kernel, dim3(hV, n_pos), dim3(DN_DS), 0, as_stream(stream), att, norm_w, z, hV, eps);
     return check_launch("qkk_dn_step_seq");
 }
 
