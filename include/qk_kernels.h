@@ -150,6 +150,15 @@ int qkk_moe_decode_tail(const qkk_moe_layer *L_host, const float *X, const float
 int qkk_moe_layer_rows(const qkk_moe_layer *L_host, float *S, const float *w_norm, float eps, qkk_sel *sel,
                        void *workspace, size_t workspace_bytes, uint32_t n_slots, void *stream);
 
+/* The same with a mixer's output on top of the residual (reference src/main.cpp:4376-4402 with the
+ * add half of add_rmsnorm.comp too):  T <- S + mix;  S <- T + (contribution of norm(T)).
+ * The first launch adds while it loads (and stores T [n_slots][n_embd], a buffer of its own, for the
+ * other two), so the add + norm launch between mixer and MoE block is not needed.  Results are bit
+ * for bit those of qkk_moe_layer_rows on rows added beforehand. */
+int qkk_moe_layer_rows_add(const qkk_moe_layer *L_host, float *S, const float *mix, float *T,
+                           const float *w_norm, float eps, qkk_sel *sel, void *workspace,
+                           size_t workspace_bytes, uint32_t n_slots, void *stream);
+
 /* The same step cut at its launch boundaries, for per-stage timing (the reference times its
  * MoE stages separately under QK_STEP_PROF, src/main.cpp:4173-4185, 4591-4632).  `stages` is
  * a mask of QKK_STAGE_*; a stage reads what the earlier stages of a previous call left in

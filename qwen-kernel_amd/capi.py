@@ -60,6 +60,7 @@ def lib():
         L.qkk_moe_decode_stages.argtypes = [vp, vp, vp, vp, vp, sz, u32, u32, vp]
         L.qkk_moe_decode_tail.argtypes = [vp, vp, vp, vp, C.c_float, vp, vp, vp, vp, sz, u32, vp]
         L.qkk_moe_layer_rows.argtypes = [vp, vp, vp, C.c_float, vp, vp, sz, u32, vp]
+        L.qkk_moe_layer_rows_add.argtypes = [vp, vp, vp, vp, vp, C.c_float, vp, vp, sz, u32, vp]
         L.qkk_moe_group_pairs.argtypes = [vp, u32, u32, u32, vp, vp, vp]
         L.qkk_head_argmax.argtypes = [vp, vp, vp, vp, u32, u32, u32, vp, sz, vp]
         L.qkk_argmax.argtypes = [vp, vp, u32, u32, vp]
@@ -196,15 +197,25 @@ def moe_decode_tail(layer, X, resid, w_next, workspace, eps=1e-6, S=None, Xn=Non
 ROWWISE_MAX = 10   # QKK_ROWWISE_MAX
 
 
-def moe_layer_rows(layer, S, w_norm, workspace, eps=1e-6, sel=None):
+def moe_layer_rows(layer, S, w_norm, workspace, eps=1e-6, sel=None, mix=None, T=None):
     """The MoE block of a layer for up to ROWWISE_MAX rows, in place: S <- S + step(rmsnorm(S) * w_norm).
+    With mix (a mixer's output rows): T <- S + mix, S <- T + step(rmsnorm(T) * w_norm).
     Returns (S, sel)."""
     import torch
     n = S.shape[0]
     if sel is None:
         sel = torch.zeros((n, 160), dtype=torch.uint8, device=S.device)
-    _check(lib().qkk_moe_layer_rows(C.byref(layer.c), _ptr(S), _ptr(w_norm), eps, _ptr(sel), _ptr(workspace),
-                                    workspace.numel() * workspace.element_size(), n, _stream()))
+    nbytes = workspace.numel() * workspace.element_size()
+    if mix is None:
+        _check(lib().qkk_moe_layer_rows(C.byref(layer.c), _ptr(S), _ptr(w_norm), eps, _ptr(sel), _ptr(workspace), nbytes, n,
+                                        _stream()))
+    else:
+        if T is None:
+            T = torch.empty_like(S)
+        if mix.shape != S.shape or T.shape != S.shape:
+            raise ValueError("moe_layer_rows: mix and T must have the shape of S")
+        _check(lib().qkk_moe_layer_rows_add(C.byref(layer.c), _ptr(S), _ptr(mix), _ptr(T), _ptr(w_norm), eps, _ptr(sel),
+                                            _ptr(workspace), nbytes, n, _stream()))
     return S, sel
 
 

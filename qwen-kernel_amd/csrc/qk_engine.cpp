@@ -269,11 +269,19 @@ int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool 
             }
         }
         if (int rc = dense(L.out, d_att, d_mix, rows, st)) return rc;
-        // y = x + mixer, normalised for the MoE block; then x = y + MoE, normalised for the next layer
-        if (int rc = qkk_add_rmsnorm(x, d_mix, L.post_norm, x, xn, N_EMBD, rows, eps, st)) return rc;
         const float* w_next = l + 1 < layers.size() ? layers[l + 1].attn_norm : d_onorm;
-        if (int rc = qkk_moe_decode_tail(&L.moe, xn, x, w_next, eps, x, d_xn[cur ^ 1], d_sel, d_ws, ws_bytes, rows, st))
-            return rc;
+        if (rows <= QKK_ROWWISE_MAX) {
+            // x <- (x + mixer) + MoE(norm(x + mixer)) in three launches (xn, read by now, takes the sum), then
+            // the next layer's norm
+            if (int rc = qkk_moe_layer_rows_add(&L.moe, x, d_mix, xn, L.post_norm, eps, d_sel, d_ws, ws_bytes, rows, st))
+                return rc;
+            if (int rc = qkk_rmsnorm(x, w_next, d_xn[cur ^ 1], N_EMBD, rows, eps, st)) return rc;
+        } else {
+            // y = x + mixer, normalised for the MoE block; then x = y + MoE, normalised for the next layer
+            if (int rc = qkk_add_rmsnorm(x, d_mix, L.post_norm, x, xn, N_EMBD, rows, eps, st)) return rc;
+            if (int rc = qkk_moe_decode_tail(&L.moe, xn, x, w_next, eps, x, d_xn[cur ^ 1], d_sel, d_ws, ws_bytes, rows, st))
+                return rc;
+        }
         cur ^= 1;
     }
     if (final_rows) *final_rows = d_xn[cur];

@@ -84,14 +84,28 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
 // launch 1.7 us longer: three 8 KB rows per wave through the L1 instead of two); the dot products
 // run on x * nw and their sums are scaled by 1/sqrt(mean(x^2) + eps), which is common to a row's
 // terms.  The task's weights are requested first, so they are in flight while x arrives.
-template <int NCH, bool ROWS>
+// ADD: the row is x + mix (a mixer's output on top of the residual); the first workgroup of the row
+// also stores the sum to `sum`, a buffer of its own, for the launches behind this one.
+template <bool ON>
+struct AddArg {
+    const float* mix;
+    float* sum;
+};
+template <>
+struct AddArg<false> {};
+
+template <int NCH, bool ROWS, bool ADD = false>
 __global__ __launch_bounds__(256) void moe_route_norm_kernel(const float* __restrict__ gate_inp,
                                                         const float* __restrict__ gate_inp_shexp,
                                                         const uint8_t* __restrict__ gate_shexp,
                                                         const uint8_t* __restrict__ up_shexp,
                                                         const float* __restrict__ x, MoeWs ws, MoeDims d,
-                                                        const float* __restrict__ nw, float eps)
+                                                        const float* __restrict__ nw, float eps, AddArg<ADD> aa)
 {
+    if constexpr (ROWS && ADD) {
+        aa.mix += (size_t)blockIdx.y * d.H;
+        aa.sum += (size_t)blockIdx.y * d.H;
+    }
     if constexpr (ROWS) {
         x += (size_t)blockIdx.y * d.H;
         ws.logits += (size_t)blockIdx.y * lstride(d.E);
@@ -130,6 +144,14 @@ __global__ __launch_bounds__(256) void moe_route_norm_kernel(const float* __rest
         for (int i = 0; i < NCH / 4; i++) xv[i] = ((const float4*)x)[threadIdx.x + 256 * i];
 #pragma unroll
         for (int i = 0; i < NCH / 4; i++) nv[i] = ((const float4*)nw)[threadIdx.x + 256 * i];
+        if constexpr (ADD) {
+#pragma unroll
+            for (int i = 0; i < NCH / 4; i++) {
+                const float4 m = ((const float4*)aa.mix)[threadIdx.x + 256 * i];
+                xv[i] = float4{xv[i].x + m.x, xv[i].y + m.y, xv[i].z + m.z, xv[i].w + m.w};
+                if (blockIdx.x == 0) ((float4*)aa.sum)[threadIdx.x + 256 * i] = xv[i];
+            }
+        }
         float ss = 0.f;
 #pragma unroll
         for (int i = 0; i < NCH / 4; i++) {
@@ -579,6 +601,8 @@ constexpr uint32_t ROWWISE_MAX = QKK_ROWWISE_MAX; // rows up to which each row r
 struct MoeNorm {
     const float* w;
     float eps;
+    const float* mix = nullptr; // the row is X + mix ...
+    float* sum = nullptr;       // ... which launch 1 stores here for launches 2 and 3
 };
 
 // Launches 1 and 2 for `rows` activation rows (grid.y); norm given (one row only): the variants with
@@ -594,8 +618,17 @@ static void launch_route_gateup(const qkk_moe_layer* L, const float* X, const Mo
         const dim3 grid((d.E + 1 + d.F + 3) / 4, rows);
 #define QK_ROUTE(K) hipLaunchKernelGGL(K, grid, block, 0, st, L->gate_inp, L->gate_inp_shexp, gs, us, X, ws, d)
 #define QK_ROUTE_NORM(K) \
-    hipLaunchKernelGGL(K, grid, block, 0, st, L->gate_inp, L->gate_inp_shexp, gs, us, X, ws, d, norm->w, norm->eps)
-        if (norm && rows > 1) {
+    hipLaunchKernelGGL(K, grid, block, 0, st, L->gate_inp, L->gate_inp_shexp, gs, us, X, ws, d, norm->w, norm->eps, \
+                       AddArg<false>{})
+#define QK_ROUTE_ADD(K) \
+    hipLaunchKernelGGL(K, grid, block, 0, st, L->gate_inp, L->gate_inp_shexp, gs, us, X, ws, d, norm->w, norm->eps, \
+                       AddArg<true>{norm->mix, norm->sum})
+        if (norm && norm->mix) {
+            if (!wide && rows > 1) QK_ROUTE_ADD((moe_route_norm_kernel<8, true, true>));
+            else if (!wide) QK_ROUTE_ADD((moe_route_norm_kernel<8, false, true>));
+            else if (rows > 1) QK_ROUTE_ADD((moe_route_norm_kernel<16, true, true>));
+            else QK_ROUTE_ADD((moe_route_norm_kernel<16, false, true>));
+        } else if (norm && rows > 1) {
             if (!wide) QK_ROUTE_NORM((moe_route_norm_kernel<8, true>));
             else QK_ROUTE_NORM((moe_route_norm_kernel<16, true>));
         } else if (norm) {
@@ -610,7 +643,9 @@ static void launch_route_gateup(const qkk_moe_layer* L, const float* X, const Mo
         }
 #undef QK_ROUTE
 #undef QK_ROUTE_NORM
+#undef QK_ROUTE_ADD
     }
+    if (norm && norm->mix) X = norm->sum; // launch 2 reads the sum launch 1 stored
     if (stages & QKK_STAGE_GATEUP) {
         constexpr int GU_RIF = 4;
         const dim3 grid(wide ? (d.k * ((d.F + 1) / 2) + 3) / 4 : (d.k * ((d.F + GU_RIF - 1) / GU_RIF) + 3) / 4, rows);
@@ -669,7 +704,8 @@ static int moe_decode_impl(const char* who, const qkk_moe_layer* L, const float*
 
     launch_route_gateup(L, X, ws, sel, d, stages, norm, n_slots, st);
     if (stages & QKK_STAGE_DOWN) {
-        const float* resid = norm ? X : nullptr; // norm in front: the input row is the residual, Y may be X
+        // norm in front: the input row (with the mixer's output, if any) is the residual; Y may be X
+        const float* resid = norm ? (norm->mix ? norm->sum : X) : nullptr;
         if (L->down_type == QKK_IQ4_XS) launch_down<QKK_IQ4_XS>(L, ws, sel, Y, d, resid, n_slots, st);
         else launch_down<QKK_Q6_K>(L, ws, sel, Y, d, resid, n_slots, st);
         // the step's output went to tail->Xn (see qkk_moe_decode_tail); add and norm in place
@@ -710,6 +746,19 @@ int qkk_moe_layer_rows(const qkk_moe_layer* L, float* S, const float* w_norm, fl
     const MoeNorm norm{w_norm, eps};
     return moe_decode_impl("qkk_moe_layer_rows", L, S, S, sel, workspace, workspace_bytes, n_slots, QKK_STAGE_ALL, stream,
                            nullptr, &norm);
+}
+
+int qkk_moe_layer_rows_add(const qkk_moe_layer* L, float* S, const float* mix, float* T, const float* w_norm, float eps,
+                           qkk_sel* sel, void* workspace, size_t workspace_bytes, uint32_t n_slots, void* stream)
+{
+    if (!w_norm || !mix || !T) return fail(QKK_EINVAL, "qkk_moe_layer_rows_add: null pointer");
+    if (!aligned16(w_norm) || !aligned16(mix) || !aligned16(T))
+        return fail(QKK_EINVAL, "qkk_moe_layer_rows_add: w_norm, mix and T must be 16-byte aligned");
+    if (T == S || T == mix) return fail(QKK_EINVAL, "qkk_moe_layer_rows_add: T must be a buffer of its own");
+    if (!(eps >= 0.f)) return fail(QKK_EINVAL, "qkk_moe_layer_rows_add: eps must be non-negative");
+    const MoeNorm norm{w_norm, eps, mix, T};
+    return moe_decode_impl("qkk_moe_layer_rows_add", L, S, S, sel, workspace, workspace_bytes, n_slots, QKK_STAGE_ALL,
+                           stream, nullptr, &norm);
 }
 
 int qkk_moe_decode_stages(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* sel, void* workspace,

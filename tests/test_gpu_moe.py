@@ -365,6 +365,35 @@ def test_moe_layer_rows_one_row(qk, orc, dev, layer_iq4, layer_q6k, which):
         qk.moe_layer_rows(layer, Sd, None, ws)
 
 
+@pytest.mark.parametrize("rows", [1, 3, 10])
+def test_moe_layer_rows_with_a_mixer_output_on_top(qk, dev, layer_iq4, layer_q6k, rows):
+    """qkk_moe_layer_rows_add: the first launch adds the mixer's rows to the residual while it loads
+    and stores the sum for the other two.  Bit for bit qkk_moe_layer_rows on rows added beforehand
+    (which the oracle pins above); T holds the sum."""
+    import torch
+    print(f"[case] moe layer rows + mixer output, rows={rows}", flush=True)
+    for hl in (layer_iq4, layer_q6k):
+        layer = hl.to_device(dev)
+        ws = torch.zeros(qk.moe_workspace_bytes(layer, rows), dtype=torch.uint8, device=dev)
+        g = torch.Generator(device="cpu").manual_seed(rows)
+        S0 = (torch.randn(rows, 2048, generator=g) * 3).to(dev)
+        mix = torch.randn(rows, 2048, generator=g).to(dev)
+        W = (0.5 + torch.rand(2048, generator=g)).to(dev)
+        want, sel_w = qk.moe_layer_rows(layer, (S0 + mix).clone(), W, ws)
+        want, sel_w = want.clone(), sel_w.clone()
+        S, T = S0.clone(), torch.full_like(S0, float("nan"))
+        got, sel = qk.moe_layer_rows(layer, S, W, ws, mix=mix, T=T)
+        torch.cuda.synchronize()
+        assert torch.equal(T, S0 + mix)
+        assert torch.equal(got, want) and torch.equal(sel, sel_w)
+    with pytest.raises(qk.QkError):   # T must be a buffer of its own
+        qk.moe_layer_rows(layer, S, W, ws, mix=mix, T=S)
+    with pytest.raises(qk.QkError):   # more rows than the row-wise launches take
+        big = torch.zeros(11, 2048, device=dev)
+        qk.moe_layer_rows(layer, big, W, torch.zeros(qk.moe_workspace_bytes(layer, 11), dtype=torch.uint8, device=dev),
+                          mix=big.clone(), T=big.clone())
+
+
 def test_rows_up_to_the_rowwise_limit_do_not_depend_on_company(qk, dev, layer_iq4):
     """Up to ROWWISE_MAX rows every row runs the one-row launches: the same row gives the same bits
     alone, among other rows and at another position; one row more takes the expert-major path and
