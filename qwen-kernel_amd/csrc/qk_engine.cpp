@@ -21,8 +21,10 @@
 #include <string.h>
 
 #include <algorithm>
+#include <initializer_list>
 #include <new>
 #include <string>
+#include <utility>
 #include <vector>
 
 #include "../../include/qk.h"
@@ -55,6 +57,7 @@ struct EngineLayer {
     const float* post_norm = nullptr; // blk.l.post_attention_norm.weight
     const float* attn_norm = nullptr; // blk.l.attn_norm.weight (layers with a mixer)
     Dense p1, p2, p3, out;            // recurrent: attn_qkv, attn_gate, -, ssm_out; attention: attn_q, attn_k, attn_v, attn_output
+    Dense cat;                        // p1, p2 (, p3) as one matrix when they share a type and lie back to back (else w = null)
     const float *alpha_w = nullptr, *beta_w = nullptr, *dt_bias = nullptr, *a_vec = nullptr, *ker = nullptr,
                 *ssm_norm = nullptr;                  // recurrent
     const float *q_norm = nullptr, *k_norm = nullptr; // attention
@@ -234,9 +237,16 @@ int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool 
         const EngineLayer& L = layers[l];
         float* xn = d_xn[cur];
         float *s1 = L.st1 + s0 * L.ps1, *s2 = L.st2 + s0 * L.ps2;
+        // one row: the input projections as one product into d_big, their outputs back to back
+        const bool one = rows == 1 && L.cat.w;
+        if (one)
+            if (int rc = dense(L.cat, xn, d_big, 1, st)) return rc;
         if (L.kind == EngineLayer::RECURRENT) {
-            if (int rc = dense(L.p1, xn, d_big, rows, st)) return rc;
-            if (int rc = dense(L.p2, xn, d_mid, rows, st)) return rc;
+            float* d_mid = one ? d_big + DN_CH : this->d_mid;
+            if (!one) {
+                if (int rc = dense(L.p1, xn, d_big, rows, st)) return rc;
+                if (int rc = dense(L.p2, xn, d_mid, rows, st)) return rc;
+            }
             if (int rc = qkk_dn_ab(xn, L.alpha_w, L.beta_w, L.dt_bias, L.a_vec, d_gb, N_EMBD, DN_HV, rows, st)) return rc;
             if (seq) {
                 if (int rc = qkk_dn_conv_seq(s1, d_big, L.ker, d_conv, DN_CH, DN_DS, 2 * DN_HK * DN_DS, eps, rows, st)) return rc;
@@ -249,9 +259,13 @@ int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool 
                     return rc;
             }
         } else {
-            if (int rc = dense(L.p1, xn, d_big, rows, st)) return rc;
-            if (int rc = dense(L.p2, xn, d_kin, rows, st)) return rc;
-            if (int rc = dense(L.p3, xn, d_vin, rows, st)) return rc;
+            float* d_kin = one ? d_big + FA_HQ * 2 * FA_DH : this->d_kin;
+            float* d_vin = one ? d_kin + FA_HKV * FA_DH : this->d_vin;
+            if (!one) {
+                if (int rc = dense(L.p1, xn, d_big, rows, st)) return rc;
+                if (int rc = dense(L.p2, xn, d_kin, rows, st)) return rc;
+                if (int rc = dense(L.p3, xn, d_vin, rows, st)) return rc;
+            }
             if (seq) {
                 if (int rc = qkk_attn_prep_seq(d_big, d_kin, d_vin, L.q_norm, L.k_norm, d_rope, pos, d_qhat, s1, s2, rows, FA_HQ,
                                                FA_HKV, FA_DH, FA_ROT, n_ctx, eps, st))
@@ -385,11 +399,47 @@ bool qk_engine::load_mixers(qkg_file* g, char* err, size_t err_len)
         d->type = (int)t.type; d->M = M; d->K = K;
         return upload(t, &d->w, err, err_len);
     };
+    // The projections that read the same normalised row, uploaded back to back: one row's step
+    // runs them as ONE matrix-vector product (their outputs then lie back to back too).
+    auto proj_in = [&](uint32_t l, EngineLayer& L, std::initializer_list<std::pair<const char*, uint32_t>> parts) {
+        Dense* ds[3] = {&L.p1, &L.p2, &L.p3};
+        qkg_tensor ts[3];
+        size_t total = 0, n = 0;
+        bool same = true;
+        for (const auto& pr : parts) {
+            qkg_tensor& t = ts[n];
+            if (!find(l, pr.first, &t) || (t.type != QKK_Q8_0 && t.type != QKK_IQ4_XS) || t.ne[0] != N_EMBD ||
+                t.ne[1] != pr.second || !t.nbytes)
+                return false;
+            ds[n]->type = (int)t.type; ds[n]->M = pr.second; ds[n]->K = N_EMBD;
+            same = same && t.type == ts[0].type && t.nbytes % 16 == 0;
+            total += t.nbytes;
+            n++;
+        }
+        if (!same) {
+            for (size_t i = 0; i < n; i++)
+                if (!upload(ts[i], &ds[i]->w, err, err_len)) return false;
+            return true;
+        }
+        uint8_t* base = (uint8_t*)dev_alloc(total, false);
+        if (!base) return set_err(err, err_len, "qk_open: device memory exhausted");
+        size_t at = 0;
+        for (size_t i = 0; i < n; i++) {
+            if (hipMemcpy(base + at, ts[i].data, ts[i].nbytes, hipMemcpyHostToDevice) != hipSuccess)
+                return set_err(err, err_len, "qk_open: upload failed");
+            ds[i]->w = base + at;
+            at += ts[i].nbytes;
+            L.cat.M += ds[i]->M;
+        }
+        if (hipMemset(base + total, 0, 256) != hipSuccess) return set_err(err, err_len, "qk_open: upload failed");
+        L.cat.w = base; L.cat.type = ds[0]->type; L.cat.K = N_EMBD;
+        return true;
+    };
     for (uint32_t l = 0; l < n_layer; l++) {
         EngineLayer& L = layers[l];
         if (!f32(l, "attn_norm.weight", N_EMBD, &L.attn_norm)) return bad("qk_open: missing/unexpected attn_norm tensor");
         if (L.kind == EngineLayer::RECURRENT) {
-            if (!proj(l, "attn_qkv.weight", N_EMBD, DN_CH, &L.p1) || !proj(l, "attn_gate.weight", N_EMBD, DN_IN, &L.p2) ||
+            if (!proj_in(l, L, {{"attn_qkv.weight", DN_CH}, {"attn_gate.weight", DN_IN}}) ||
                 !proj(l, "ssm_out.weight", DN_IN, N_EMBD, &L.out))
                 return bad("qk_open: gated-DeltaNet projections missing or of an unsupported type / shape");
             if (!f32(l, "ssm_alpha.weight", (uint64_t)DN_HV * N_EMBD, &L.alpha_w) ||
@@ -402,8 +452,8 @@ bool qk_engine::load_mixers(qkg_file* g, char* err, size_t err_len)
             L.ps1 = (size_t)DN_CH * 3;
             L.ps2 = (size_t)DN_HV * DN_DS * DN_DS;
         } else {
-            if (!proj(l, "attn_q.weight", N_EMBD, FA_HQ * 2 * FA_DH, &L.p1) || !proj(l, "attn_k.weight", N_EMBD, FA_HKV * FA_DH, &L.p2) ||
-                !proj(l, "attn_v.weight", N_EMBD, FA_HKV * FA_DH, &L.p3) || !proj(l, "attn_output.weight", FA_HQ * FA_DH, N_EMBD, &L.out))
+            if (!proj_in(l, L, {{"attn_q.weight", FA_HQ * 2 * FA_DH}, {"attn_k.weight", FA_HKV * FA_DH}, {"attn_v.weight", FA_HKV * FA_DH}}) ||
+                !proj(l, "attn_output.weight", FA_HQ * FA_DH, N_EMBD, &L.out))
                 return bad("qk_open: attention projections missing or of an unsupported type / shape");
             if (!f32(l, "attn_q_norm.weight", FA_DH, &L.q_norm) || !f32(l, "attn_k_norm.weight", FA_DH, &L.k_norm))
                 return bad("qk_open: attention norm tensors missing or of an unexpected shape");
