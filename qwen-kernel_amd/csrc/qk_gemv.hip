@@ -361,7 +361,11 @@ static int dispatch_q(const void* W, const float* X, float* Y, uint32_t M, uint3
     constexpr uint32_t MINK = TYPE == QKK_Q8_0 ? 32 : 256;
     // rows per wave: four where the matrix has rows enough to give every CU several waves that way,
     // fewer for short matrices (512 rows: 3.1-3.4 us with one row per wave against 4.6-5.2 us with four)
-    if (K == 2048 && M >= 8192 && TYPE == QKK_Q8_0) launch_q<TYPE, 64, 1, 8>(W, X, Y, M, K, batch, rb, st); // 7.5 -> 6.9 us
+    // a layer's input projections as one matrix (12288 = qkv + gate, 9216 = q + k + v rows): M / 1024 rows
+    // per wave make 256 workgroups, one per CU, where eight leave half the CUs with a second one
+    if (K == 2048 && M == 12288 && TYPE == QKK_Q8_0) launch_q<TYPE, 64, 1, 12>(W, X, Y, M, K, batch, rb, st);
+    else if (K == 2048 && M == 9216 && TYPE == QKK_Q8_0) launch_q<TYPE, 64, 1, 9>(W, X, Y, M, K, batch, rb, st);
+    else if (K == 2048 && M >= 8192 && TYPE == QKK_Q8_0) launch_q<TYPE, 64, 1, 8>(W, X, Y, M, K, batch, rb, st); // 7.5 -> 6.9 us
     else if (K == 2048 && M >= 2048) launch_q<TYPE, 64, 1, 4>(W, X, Y, M, K, batch, rb, st);
     else if (K == 2048 && M >= 1024) launch_q<TYPE, 64, 1, 2>(W, X, Y, M, K, batch, rb, st);
     else if (K == 2048) launch_q<TYPE, 64, 1, 1>(W, X, Y, M, K, batch, rb, st);

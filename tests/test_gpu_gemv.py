@@ -43,11 +43,12 @@ def test_gemv_quantised_several_rows(qk, orc, dev, name, M, K, batch):
     run_case(qk, orc, dev, name, M, K, batch, seed=77)
 
 
-@pytest.mark.parametrize("M,K", [(8192, 2048), (4096, 2048), (2048, 4096), (512, 2048)])
+@pytest.mark.parametrize("M,K", [(8192, 2048), (4096, 2048), (2048, 4096), (512, 2048), (12288, 2048), (9216, 2048)])
 @pytest.mark.parametrize("batch", [1, 16])
 def test_gemv_q8_0_engine_shapes(qk, orc, dev, M, K, batch):
     """The dense projections of a decode step at the shapes the reference dispatches them
-    (src/main.cpp:4310-4335, 4195-4196), for one slot and for sixteen."""
+    (src/main.cpp:4310-4335, 4195-4196), for one slot and for sixteen; 12288 and 9216 rows are a
+    layer's input projections back to back, as the engine runs them for one slot."""
     run_case(qk, orc, dev, "q8_0", M, K, batch, seed=5)
 
 
