@@ -411,6 +411,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", default="moe_decode_bs1")
     ap.add_argument("--ring", type=int, default=40)
+    ap.add_argument("--prefill-rows", dest="maxb", type=int, default=0,
+                    help="engine workloads: positions per prefill pass (sets QK_PREFILL_ROWS, 16..1024; default the engine's 1024)")
     ap.add_argument("--layers", type=int, default=8,
                     help="layers of the synthetic model of the engine workloads (40 = the reference model's depth, a 16 GB file)")
     ap.add_argument("--extras", dest="extras", action="store_true", default=True)
@@ -445,11 +447,14 @@ def main():
                               higher_is_better=True, data="synthetic", dtype="f32",
                               config=dict(workload="engine_whole_model", **r["config"]), detail=r)), flush=True)
         return
+    if a.maxb:
+        os.environ["QK_PREFILL_ROWS"] = str(a.maxb)
     if a.workload == "engine_prefill":   # prompt positions through qk_stage_run on a whole model
         r = engine_workload(qk, a.layers, (1,), 0, 0, kinds=("RRRA" * ((a.layers + 3) // 4))[:a.layers], prefill_only=1024)
         print(json.dumps(dict(metric="engine_prefill_tok_per_s", value=r["slots_1"]["prefill_tok_per_s"], unit="tok/s",
                               n_gpus=1, higher_is_better=True, data="synthetic", dtype="f32",
-                              config=dict(workload="engine_prefill", positions=1024, **r["config"]), detail=r)), flush=True)
+                              config=dict(workload="engine_prefill", positions=1024, positions_per_pass=a.maxb or 1024,
+                                          **r["config"]), detail=r)), flush=True)
         return
     if a.workload == "engine_decode":   # the engine ABI alone (for kernel traces of its graph replays)
         r = engine_workload(qk, 8, (1, 4, 16), 8, 2)

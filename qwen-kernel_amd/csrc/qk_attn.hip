@@ -362,10 +362,14 @@ int qkk_attn_prep_seq(const float* qfull, const float* kin, const float* vin, co
                           n_pos, hQ, hKV, dh, n_rot, tmax, eps, 0, stream);
 }
 
+// Position ranges a launch over `rows` rows uses at most: the more rows, the fewer ranges are needed
+// to fill the chip (two workgroups per CU over rows x KV heads; 512 CUs assumed for the bound).
+static uint32_t max_ranges(uint32_t rows) { return std::min(ATT_MAX_RANGES, std::max(8u, 512u / rows)); }
+
 size_t qkk_attn_workspace_bytes(uint32_t n_slots, uint32_t hQ, uint32_t dh)
 {
     if (!n_slots || !hQ || !dh) return 0;
-    return (size_t)n_slots * hQ * ATT_MAX_RANGES * ((size_t)dh + 2) * sizeof(float) + 256;
+    return (size_t)n_slots * hQ * max_ranges(n_slots) * ((size_t)dh + 2) * sizeof(float) + 256;
 }
 
 static int attn_decode_impl(const char* who, const float* qhat, const float* k_cache, const float* v_cache,
@@ -385,7 +389,7 @@ static int attn_decode_impl(const char* who, const float* qhat, const float* k_c
     // two workgroups per CU over the (row, KV head) pairs, 8..64 ranges each: 16 slots x 4096 positions
     // measured 4.5 TB/s with 16 ranges, 4.2 with 32, 3.1 with 128 (the partial results are traffic too);
     // one slot 0.98 TB/s with 64 ranges, 0.80 with 32
-    const uint32_t n_ranges = std::min(ATT_MAX_RANGES, std::max(8u, persistent_blocks() / 2 / (rows * hKV)));
+    const uint32_t n_ranges = std::min(max_ranges(rows), std::max(8u, persistent_blocks() / 2 / (rows * hKV)));
     AttnWs ws;
     ws.acc = (float*)workspace;
     ws.ml = ws.acc + (size_t)rows * hQ * n_ranges * ATT_DH;

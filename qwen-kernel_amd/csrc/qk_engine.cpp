@@ -35,7 +35,6 @@ namespace {
 
 constexpr uint32_t N_EMBD = 2048;           // reference src/main.cpp:3086 (compile-time there too)
 constexpr uint32_t MAX_ROWS = QKK_MAX_SLOTS; // rows one device step carries
-constexpr uint32_t PF_ROWS = 128;            // positions of one slot a prefill pass carries (whole-model files)
 constexpr uint32_t N_STATE = 3;             // snapshot entries (reference default, stub/qk_stub.c:98)
 constexpr int ERR_DEVICE = -6;              // a launch, copy or synchronisation failed
 
@@ -103,8 +102,9 @@ struct qk_engine {
     uint32_t dn_kdiv = 0;        // 0: value head h reads key head h % hK; else h / dn_kdiv (src/main.cpp:3092-3094)
     uint32_t* d_pos = nullptr;   // [MAX_ROWS] position of the token fed this step
     uint32_t* h_pos = nullptr;   // pinned
-    uint32_t cap = MAX_ROWS;     // rows the step's buffers hold (PF_ROWS for whole-model files)
-    uint32_t *d_pf = nullptr, *h_pf = nullptr; // [3][PF_ROWS] ids, positions, sampled ids of a prefill pass (device / pinned)
+    uint32_t pf_rows = 1024;     // positions of one slot a prefill pass carries (whole-model files; QK_PREFILL_ROWS)
+    uint32_t cap = MAX_ROWS;     // rows the step's buffers hold (pf_rows for whole-model files)
+    uint32_t *d_pf = nullptr, *h_pf = nullptr; // [3][pf_rows] ids, positions, sampled ids of a prefill pass (device / pinned)
     float* d_rope = nullptr;     // [n_ctx][FA_ROT/2][2]
     float *d_big = nullptr, *d_mid = nullptr, *d_kin = nullptr, *d_vin = nullptr, *d_gb = nullptr, *d_conv = nullptr,
           *d_qhat = nullptr, *d_att = nullptr, *d_mix = nullptr; // per-step rows of the mixers
@@ -224,12 +224,12 @@ static int dense(const Dense& d, const float* x, float* y, uint32_t rows, hipStr
 //                attention is causal over the rows).
 int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool want_head, bool seq)
 {
-    if (rows < 1 || s0 >= MAX_ROWS || (seq ? rows > PF_ROWS : s0 + rows > MAX_ROWS)) return QKK_ESHAPE;
+    if (rows < 1 || s0 >= MAX_ROWS || (seq ? rows > pf_rows : s0 + rows > MAX_ROWS)) return QKK_ESHAPE;
     float* x = d_x;
     const uint32_t* ids = seq ? d_pf : d_ids;
-    const uint32_t* pos = seq ? d_pf + PF_ROWS : d_pos + s0;
-    uint32_t* tok = seq ? d_pf + 2 * PF_ROWS : d_tok + s0;
-    if (int rc = qkk_embed(embd_type, d_embd, embd_rows, N_EMBD, ids, seq ? PF_ROWS : MAX_ROWS, seq ? 0 : s0, 1, x, rows, st))
+    const uint32_t* pos = seq ? d_pf + pf_rows : d_pos + s0;
+    uint32_t* tok = seq ? d_pf + 2 * pf_rows : d_tok + s0;
+    if (int rc = qkk_embed(embd_type, d_embd, embd_rows, N_EMBD, ids, seq ? pf_rows : MAX_ROWS, seq ? 0 : s0, 1, x, rows, st))
         return rc;
     if (int rc = qkk_rmsnorm(x, layers[0].attn_norm, d_xn[0], N_EMBD, rows, eps, st)) return rc;
     int cur = 0;
@@ -308,27 +308,27 @@ int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool 
 }
 
 // Positions base .. base+n-1 of one slot, alone (the other slots' states are not touched), in
-// passes of PF_ROWS.  ids_out (optional): the greedy id after every position; the last position's
+// passes of pf_rows.  ids_out (optional): the greedy id after every position; the last position's
 // normalised row is kept for qk_stage_topk.
 int qk_engine::prefill(uint32_t slot, const uint32_t* toks, uint32_t n, uint32_t base, uint32_t* ids_out)
 {
-    for (uint32_t off = 0; off < n; off += PF_ROWS) {
-        const uint32_t rows = std::min(PF_ROWS, n - off);
+    for (uint32_t off = 0; off < n; off += pf_rows) {
+        const uint32_t rows = std::min(pf_rows, n - off);
         for (uint32_t t = 0; t < rows; t++) {
             h_pf[t] = toks[off + t];
-            h_pf[PF_ROWS + t] = base + off + t;
+            h_pf[pf_rows + t] = base + off + t;
         }
-        if (hipMemcpyAsync(d_pf, h_pf, 2 * PF_ROWS * sizeof(uint32_t), hipMemcpyHostToDevice, st) != hipSuccess)
+        if (hipMemcpyAsync(d_pf, h_pf, 2 * pf_rows * sizeof(uint32_t), hipMemcpyHostToDevice, st) != hipSuccess)
             return ERR_DEVICE;
         float* fin = nullptr;
         if (launch_full(rows, slot, &fin, ids_out != nullptr, true) != QKK_OK) return ERR_DEVICE;
-        if (ids_out && (hipMemcpyAsync(h_pf + 2 * PF_ROWS, d_pf + 2 * PF_ROWS, rows * sizeof(uint32_t), hipMemcpyDeviceToHost,
+        if (ids_out && (hipMemcpyAsync(h_pf + 2 * pf_rows, d_pf + 2 * pf_rows, rows * sizeof(uint32_t), hipMemcpyDeviceToHost,
                                        st) != hipSuccess ||
                         hipMemcpyAsync(d_last, fin + (size_t)(rows - 1) * N_EMBD, N_EMBD * sizeof(float),
                                        hipMemcpyDeviceToDevice, st) != hipSuccess))
             return ERR_DEVICE;
         if (hipStreamSynchronize(st) != hipSuccess) return ERR_DEVICE;
-        if (ids_out) memcpy(ids_out + off, h_pf + 2 * PF_ROWS, rows * sizeof(uint32_t));
+        if (ids_out) memcpy(ids_out + off, h_pf + 2 * pf_rows, rows * sizeof(uint32_t));
     }
     return 0;
 }
@@ -468,10 +468,10 @@ bool qk_engine::load_mixers(qkg_file* g, char* err, size_t err_len)
     d_gb = rows_of(2 * DN_HV); d_conv = rows_of(DN_CH); d_qhat = rows_of(FA_HQ * FA_DH); d_att = rows_of(DN_IN);
     d_mix = rows_of(N_EMBD);
     d_pos = (uint32_t*)dev_alloc(MAX_ROWS * 4, true);
-    d_pf = (uint32_t*)dev_alloc(3 * PF_ROWS * 4, true);
-    if (!d_pf || hipHostMalloc((void**)&h_pf, 3 * PF_ROWS * 4, hipHostMallocDefault) != hipSuccess)
+    d_pf = (uint32_t*)dev_alloc(3 * pf_rows * 4, true);
+    if (!d_pf || hipHostMalloc((void**)&h_pf, 3 * pf_rows * 4, hipHostMallocDefault) != hipSuccess)
         return bad("qk_open: cannot allocate the prefill buffers");
-    memset(h_pf, 0, 3 * PF_ROWS * 4);
+    memset(h_pf, 0, 3 * pf_rows * 4);
     aws_bytes = qkk_attn_workspace_bytes(cap, FA_HQ, FA_DH);
     d_aws = dev_alloc(aws_bytes, true);
     d_rope = (float*)dev_alloc((size_t)n_ctx * FA_ROT * sizeof(float), false);
@@ -552,6 +552,14 @@ bool qk_engine::open(const char* path, const qk_config& cfg, char* err, size_t e
             return false;
         }
         if (split()) return bad("qk_open: QK_LAYERS pipeline stages are not part of this library (one GPU runs every layer)");
+    }
+    // Rows of one prefill pass.  Independent of QK_MAXB, which decides only WHICH positions are
+    // prefilled at qk_slot_start (the reference's bookkeeping): more rows per pass read the weights
+    // less often (40 layers: 6.7 k positions/s at 128, 8.7 k at 256, 11.3 k at 512, 12.7 k at 1024).
+    if (const char* pr = getenv("QK_PREFILL_ROWS")) {
+        const long x = atol(pr);
+        if (x >= 16 && x <= 1024) pf_rows = (uint32_t)x;
+        else fprintf(stderr, "QK_PREFILL_ROWS=%s out of range [16,1024]; using %u\n", pr, pf_rows);
     }
     if (const char* mb = getenv("QK_MAXB")) { // reference src/main.cpp:3834-3838
         const long x = atol(mb);
@@ -643,7 +651,7 @@ bool qk_engine::open(const char* path, const qk_config& cfg, char* err, size_t e
         layers[l].post_norm = (const float*)p;
     }
 
-    cap = full_model ? PF_ROWS : MAX_ROWS;
+    cap = full_model ? pf_rows : MAX_ROWS;
     for (const EngineLayer& L : layers) ws_bytes = std::max(ws_bytes, qkk_moe_workspace_bytes(&L.moe, cap));
     hws_bytes = qkk_head_workspace_bytes(vocab, MAX_ROWS);
     if (!ws_bytes || !hws_bytes) return bad("qk_open: expert shape unsupported by the kernels");

@@ -81,13 +81,15 @@ def test_whole_model_streams(qk, full):
 
 def test_whole_model_eager_launches_and_serial_prefill(qk, full, monkeypatch):
     """QK_NO_GRAPH launches the kernels one by one; QK_NO_BATCH feeds every prompt token in a serial
-    step instead of at the start: the same streams."""
+    step instead of at the start; QK_MAXB moves the border between prefilled and serially fed positions,
+    QK_PREFILL_ROWS sets the rows per prefill pass: the same streams."""
     model, path = full
     print("[case] whole model, eager / serial prefill", flush=True)
     prompt = [int(t) for t in np.random.default_rng(6).integers(0, VOCAB, 18)]
     streams = []
-    for env in ({}, {"QK_NO_GRAPH": "1"}, {"QK_NO_BATCH": "1"}):
-        for k in ("QK_NO_GRAPH", "QK_NO_BATCH"):
+    for env in ({}, {"QK_NO_GRAPH": "1"}, {"QK_NO_BATCH": "1"}, {"QK_MAXB": "16"},
+                {"QK_PREFILL_ROWS": "16"}):   # QK_MAXB 16: 16 positions prefilled, one serial step more; rows 16: two passes
+        for k in ("QK_NO_GRAPH", "QK_NO_BATCH", "QK_MAXB", "QK_PREFILL_ROWS"):
             monkeypatch.delenv(k, raising=False)
         for k, v in env.items():
             monkeypatch.setenv(k, v)
@@ -98,7 +100,7 @@ def test_whole_model_eager_launches_and_serial_prefill(qk, full, monkeypatch):
                 rc, out, fin = eng.step_chunk()
                 got += out[1]
             streams.append(got)
-    assert len(streams[0]) == 6 and streams[0] == streams[1] == streams[2]
+    assert len(streams[0]) == 6 and all(st == streams[0] for st in streams)
 
 
 def test_whole_model_stage_run_and_snapshots(qk, full):
@@ -126,12 +128,13 @@ def test_whole_model_stage_run_and_snapshots(qk, full):
         assert eng.state_save(1, 3, 0) == -1 and eng.state_load(2, 0, 0) == -1
 
 
-def test_whole_model_long_prompt_and_long_stage_run(qk, full):
-    """A prompt longer than one prefill pass (128 positions go through the projections and the MoE
-    blocks together, the mixers position by position), then the rest, then the serial steps: the
-    same stream as the oracle fed one token at a time.  qk_stage_run over 40 positions returns the
-    oracle's id after every one of them."""
+def test_whole_model_long_prompt_and_long_stage_run(qk, full, monkeypatch):
+    """A prompt longer than one prefill pass (64 positions here go through the projections and the
+    MoE blocks together, the mixers through their sequence kernels), then two more passes, then the
+    serial steps: the same stream as the oracle fed one token at a time.  qk_stage_run over 40
+    positions returns the oracle's id after every one of them."""
     model, path = full
+    monkeypatch.setenv("QK_PREFILL_ROWS", "64")
     print("[case] whole model, 150-token prompt and a 40-position stage run", flush=True)
     rng = np.random.default_rng(21)
     prompt = [int(t) for t in rng.integers(0, VOCAB, 150)]
