@@ -19,13 +19,13 @@
  * state machine of qk_step_chunk (one captured hipGraph per dispatch depth), greedy sampling,
  * EOS / max_gen / n_ctx endings, qk_stage_run / qk_stage_topk on the unsplit engine, state
  * snapshots (three entries).  qk_slot_start prefills the positions the reference batch-prefills,
- * and qk_stage_run feeds its positions, in passes of up to QK_PREFILL_ROWS rows on the slot alone.  Not part of
- * this library: the prefix cache, speculative decoding, QK_LAYERS pipeline stages (refused: one
- * GPU runs every layer).  A device failure inside a call returns -6.
+ * and qk_stage_run feeds its positions, in passes of up to QK_PREFILL_ROWS rows on the slot
+ * alone.  Not part of this library: the prefix cache, speculative decoding, QK_LAYERS pipeline
+ * stages (refused: one GPU runs every layer).  A device failure inside a call returns -6.
  * Environment, as in the reference: QK_MAXB (batch-prefill chunk, 16..1024, default 128),
- * QK_NO_BATCH (serial prefill of the whole prompt); and QK_PREFILL_ROWS (rows of one prefill pass,
- * 16..1024, default 1024: how the prefilled positions are cut, not which are prefilled), QK_NO_GRAPH (launch the step's kernels
- * one by one instead of replaying the graph).
+ * QK_NO_BATCH (serial prefill of the whole prompt); and QK_PREFILL_ROWS (rows of one prefill
+ * pass, 16..1024, default 1024: how the prefilled positions are cut, not which are prefilled),
+ * QK_NO_GRAPH (launch the step's kernels one by one instead of replaying the graph).
  */
 #ifndef QK_H
 #define QK_H
