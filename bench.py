@@ -372,6 +372,17 @@ def engine_workload(qk, n_layer, slots_list, chunks, warm_chunks, seed=31, kinds
                         if rcp != 0:
                             sys.exit(f"bench.py: qk_stage_run returned {rcp}")
                     pre = dict(prefill_tok_per_s=len(ptoks) / tp, prefill_positions=len(ptoks))
+                    # the serving path: qk_slot_start prefills all but the last prompt token (no LM head there)
+                    for s in range(n_slots):
+                        eng.slot_cancel(s)
+                    for _ in range(2):
+                        tp = time.perf_counter()
+                        rcs = eng.slot_start(0, ptoks + [5], 8)
+                        tp = time.perf_counter() - tp
+                        eng.slot_cancel(0)
+                        if rcs != 0:
+                            sys.exit(f"bench.py: qk_slot_start returned {rcs}")
+                    pre["slot_start_prefill_tok_per_s"] = len(ptoks) / tp
             res[f"slots_{n_slots}"] = dict(tok_per_s=toks / dt, us_per_step=dt / (max(chunks, 1) * 32) * 1e6, tokens=toks,
                                            open_s=t_open, **pre)
     finally:
