@@ -302,8 +302,8 @@ int qkk_dn_step(const float *conv, const float *gb, float *state, const float *n
  *                    the reference's). workspace: qkk_attn_workspace_bytes(n_pos, hQ, dh).
  * qkk_dn_conv_seq    the conv is a 4-tap filter over the inputs, so all positions run in parallel
  *                    (bit-identical to the steps); the window is moved on by a second small launch.
- * qkk_dn_step_seq    the state is read once, kept in registers over all positions (16 rows of a head
- *                    per workgroup, 8 lanes per row) and written once; q, k, v and the gates are
+ * qkk_dn_step_seq    the state is read once, kept in registers over all positions (8 rows of a head
+ *                    per workgroup, 16 lanes per row) and written once; q, k, v and the gates are
  *                    staged through LDS 16 positions at a time; the head norm and output gate run
  *                    as a second launch over (head, position).  conv 16-byte aligned, n_pos <= 65535. */
 int qkk_attn_prep_seq(const float *qfull, const float *kin, const float *vin, const float *q_norm_w,

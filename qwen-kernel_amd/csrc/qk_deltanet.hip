@@ -189,14 +189,14 @@ __global__ __launch_bounds__(128) void dn_window_seq_kernel(float* __restrict__ 
 // SEQ_CH positions at a time are staged in LDS (double-buffered; the next chunk's global loads are
 // in flight while the current one is worked on), one barrier per chunk.  The head-wide norm and the
 // output gate need all rows of a head and run as a second kernel over (head, position).
-constexpr uint32_t SEQ_NQ = 8;               // lanes per state row
+constexpr uint32_t SEQ_NQ = 16;              // lanes per state row
 constexpr uint32_t SEQ_RB = 128 / SEQ_NQ;    // state rows per workgroup of 128 threads
 constexpr uint32_t SEQ_CH = 16;              // positions per staged chunk
 constexpr uint32_t SEQ_QS = DN_DS / SEQ_NQ;  // columns per part
 constexpr uint32_t SEQ_PAD = SEQ_QS + 4;     // part stride in LDS: the parts' float4 reads hit distinct banks
 constexpr uint32_t SEQ_TOTAL = SEQ_CH * (2 * DN_DS + SEQ_RB) / 4; // float4 loads per chunk
 constexpr uint32_t SEQ_ITEMS = (SEQ_TOTAL + 127) / 128;           // per thread
-static_assert(2 * SEQ_CH <= 128 && (SEQ_NQ == 4 || SEQ_NQ == 8), "chunk staging");
+static_assert(2 * SEQ_CH <= 128 && (SEQ_NQ == 4 || SEQ_NQ == 8 || SEQ_NQ == 16), "chunk staging");
 
 struct SeqChunk {
     float q[SEQ_CH][SEQ_NQ * SEQ_PAD];
@@ -283,7 +283,8 @@ __global__ __launch_bounds__(128) void dn_step_seq_kernel(const float* __restric
             float sk = (ps.x + ps.y) + (ps.z + ps.w);
             sk += dpp_f<DPP_XOR1>(sk);
             sk += dpp_f<DPP_XOR2>(sk);
-            if (SEQ_NQ == 8) sk += dpp_f<DPP_HALF_MIRROR>(sk);
+            if (SEQ_NQ >= 8) sk += dpp_f<DPP_HALF_MIRROR>(sk);
+            if (SEQ_NQ >= 16) sk += dpp_f<DPP_MIRROR>(sk);
             const float dj = beta * (vj - sk * decay);
             float4 po = float4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -297,7 +298,8 @@ __global__ __launch_bounds__(128) void dn_step_seq_kernel(const float* __restric
             float oj = (po.x + po.y) + (po.z + po.w);
             oj += dpp_f<DPP_XOR1>(oj);
             oj += dpp_f<DPP_XOR2>(oj);
-            if (SEQ_NQ == 8) oj += dpp_f<DPP_HALF_MIRROR>(oj);
+            if (SEQ_NQ >= 8) oj += dpp_f<DPP_HALF_MIRROR>(oj);
+            if (SEQ_NQ >= 16) oj += dpp_f<DPP_MIRROR>(oj);
             if (c == 0) att[((size_t)(t0 + p) * hV + h) * DN_DS + row] = oj;
         };
         if (np == SEQ_CH) { // whole chunk: unrolled, so that the next position's LDS reads can start early
