@@ -245,6 +245,147 @@ __global__ __launch_bounds__(256) void attn_range_kernel(const float* __restrict
     }
 }
 
+// The same scan for TWO consecutive rows of a sequence (positions p, p + 1 of one slot) per
+// workgroup: the second row's heads take the MFMA rows 8..15 that one row leaves empty, every cache
+// row loaded serves both, and the later keys are masked per row.  grid (n_ranges, hKV, ceil(rows/2)).
+__global__ __launch_bounds__(256) void attn_range_pair_kernel(const float* __restrict__ qhat, const float* __restrict__ kc,
+                                                         const float* __restrict__ vc,
+                                                         const uint32_t* __restrict__ slot_pos, AttnWs ws, uint32_t hQ,
+                                                         uint32_t hKV, uint32_t G, uint32_t tmax, uint32_t rows)
+{
+    constexpr uint32_t RPW = ATT_TILE / 4; // rows per wave and tile (16: one MFMA column block)
+    constexpr uint32_t KB = ATT_DH / 32;   // 32-dim blocks of a row
+    constexpr uint32_t NH = 2 * ATT_GMAX;  // (row of the pair, head) = MFMA row 8 * row + head
+    __shared__ __attribute__((aligned(16))) half8 s_qh[KB][64], s_ql[KB][64]; // Q as the A operand, per lane
+    __shared__ __attribute__((aligned(16))) float s_sc[NH][ATT_TILE];
+    __shared__ float s_corr[NH], s_m[NH], s_l[NH];
+    __shared__ __attribute__((aligned(16))) float s_acc[3][ATT_GMAX][ATT_DH]; // waves 1..3 hand theirs to wave 0
+    const uint32_t n_ranges = gridDim.x, c = blockIdx.x, kv = blockIdx.y, r0 = 2 * blockIdx.z, t = threadIdx.x;
+    const bool two = r0 + 1 < rows; // the last pair of an odd row count has one row
+    const uint32_t lane = t & 63u, wave = t >> 6, col = lane & 15u, quad = lane >> 4;
+    const uint32_t n0 = slot_position(slot_pos, r0, tmax) + 1u;
+    const uint32_t n1 = two ? slot_position(slot_pos, r0 + 1, tmax) + 1u : 0u;
+    const uint32_t n = max(n0, n1);
+    const uint32_t per = (tmax + n_ranges - 1) / n_ranges;
+    const uint32_t p_begin = c * per, p_end = min(n, p_begin + per);
+    if (p_begin >= n) return; // the whole workgroup: this range holds no key yet
+
+    // Q operand: lane feeds A[head = col][dims 32*kb + 8*quad .. +7]; wave w prepares blocks 2w, 2w+1
+#pragma unroll
+    for (uint32_t i = 0; i < 2; i++) {
+        const uint32_t kb = 2 * wave + i;
+        float4 a = float4{0.f, 0.f, 0.f, 0.f}, b = a;
+        const uint32_t qr = col >> 3, qhd = col & 7u;
+        if (qhd < G && (qr == 0 || two)) {
+            const float4* qrow = (const float4*)(qhat + ((size_t)(r0 + qr) * hQ + kv * G + qhd) * ATT_DH);
+            a = qrow[kb * 8 + 2 * quad];
+            b = qrow[kb * 8 + 2 * quad + 1];
+        }
+        const HalfSplit sp = split8(a, b);
+        s_qh[kb][lane] = sp.hi;
+        s_ql[kb][lane] = sp.lo;
+    }
+    if (t < NH) { s_m[t] = ATT_FLOOR; s_l[t] = 0.f; }
+    const float qs = 1.f / sqrtf((float)ATT_DH);
+    const float4* kbase = (const float4*)(kc + (size_t)kv * tmax * ATT_DH); // one slot's caches
+    const float4* vbase = (const float4*)(vc + (size_t)kv * tmax * ATT_DH);
+    float4 acc[NH];
+#pragma unroll
+    for (uint32_t h = 0; h < NH; h++) acc[h] = float4{0.f, 0.f, 0.f, 0.f};
+    __syncthreads();
+
+    for (uint32_t p0 = p_begin; p0 < p_end; p0 += ATT_TILE) {
+        const uint32_t ts = min(ATT_TILE, p_end - p0);
+        // rows beyond the tile repeat its last row (their scores are masked, their weights zero)
+        const size_t krow = p0 + min(RPW * wave + col, ts - 1);
+        float4 ka[KB], kb4[KB], v4[RPW];
+#pragma unroll
+        for (uint32_t kb = 0; kb < KB; kb++) {
+            ka[kb] = kbase[krow * (ATT_DH / 4) + kb * 8 + 2 * quad];
+            kb4[kb] = kbase[krow * (ATT_DH / 4) + kb * 8 + 2 * quad + 1];
+        }
+#pragma unroll
+        for (uint32_t i = 0; i < RPW; i++)
+            v4[i] = vbase[(size_t)(p0 + min(RPW * wave + i, ts - 1)) * (ATT_DH / 4) + lane];
+        float4v sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (uint32_t kb = 0; kb < KB; kb++) {
+            const HalfSplit k = split8(ka[kb], kb4[kb]);
+            const half8 qh = s_qh[kb][lane], ql = s_ql[kb][lane];
+            sc = mfma16x32(qh, k.hi, sc);
+            sc = mfma16x32(qh, k.lo, sc);
+            sc = mfma16x32(ql, k.hi, sc);
+        }
+        // D[4*quad + e][col]: head 4*quad + e, position 16*wave + col
+#pragma unroll
+        for (uint32_t e = 0; e < 4; e++)
+            if (((4 * quad + e) & 7u) < G) s_sc[4 * quad + e][RPW * wave + col] = sc[e] * qs;
+        __syncthreads();
+        // running maximum and sum per head: wave w folds heads w, w + 4 (lane = position of the tile)
+        for (uint32_t h = wave; h < NH; h += 4) {
+            if ((h & 7u) >= G || (h >= ATT_GMAX && !two)) continue; // the whole wave
+            const bool live = lane < ts && p0 + lane < (h < ATT_GMAX ? n0 : n1); // a row sees the keys up to its own position
+            const float v = live ? s_sc[h][lane] : ATT_FLOOR;
+            const float old_m = s_m[h];
+            const float new_m = fmaxf(old_m, wave_max(v));
+            const float e = live ? expf(v - new_m) : 0.f;
+            const float tl = wave_sum(e);
+            s_sc[h][lane] = e;
+            if (lane == 0) {
+                const float corr = expf(old_m - new_m);
+                s_corr[h] = corr;
+                s_m[h] = new_m;
+                s_l[h] = s_l[h] * corr + tl;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (uint32_t h = 0; h < NH; h++) {
+            if ((h & 7u) < G && (h < ATT_GMAX || two)) { // uniform
+                const float corr = s_corr[h];
+                float4 a = float4{acc[h].x * corr, acc[h].y * corr, acc[h].z * corr, acc[h].w * corr};
+#pragma unroll
+                for (uint32_t i = 0; i < RPW; i += 4) { // the weights of positions beyond the tile are zero
+                    const float4 w = *(const float4*)&s_sc[h][RPW * wave + i];
+                    a.x += w.x * v4[i].x + w.y * v4[i + 1].x + w.z * v4[i + 2].x + w.w * v4[i + 3].x;
+                    a.y += w.x * v4[i].y + w.y * v4[i + 1].y + w.z * v4[i + 2].y + w.w * v4[i + 3].y;
+                    a.z += w.x * v4[i].z + w.y * v4[i + 1].z + w.z * v4[i + 2].z + w.w * v4[i + 3].z;
+                    a.w += w.x * v4[i].w + w.y * v4[i + 1].w + w.z * v4[i + 2].w + w.w * v4[i + 3].w;
+                }
+                acc[h] = a;
+            }
+        }
+        __syncthreads(); // the next tile overwrites the scores
+    }
+    // the four waves' accumulators, added in wave order; one row of the pair at a time through s_acc
+#pragma unroll
+    for (uint32_t half = 0; half < 2; half++) {
+        if (half == 1 && !two) break; // the whole workgroup
+        if (wave > 0) {
+#pragma unroll
+            for (uint32_t h = 0; h < ATT_GMAX; h++)
+                if (h < G) ((float4*)s_acc[wave - 1][h])[lane] = acc[half * ATT_GMAX + h];
+        }
+        __syncthreads();
+        if (wave == 0) {
+#pragma unroll
+            for (uint32_t h = 0; h < ATT_GMAX; h++) {
+                if (h < G) {
+                    float4 a = acc[half * ATT_GMAX + h];
+                    for (uint32_t w = 0; w < 3; w++) {
+                        const float4 b = ((const float4*)s_acc[w][h])[lane];
+                        a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+                    }
+                    const size_t slot = ((size_t)(r0 + half) * hQ + kv * G + h) * n_ranges + c;
+                    ((float4*)(ws.acc + slot * ATT_DH))[lane] = a;
+                    if (lane == 0) { ws.ml[2 * slot] = s_m[half * ATT_GMAX + h]; ws.ml[2 * slot + 1] = s_l[half * ATT_GMAX + h]; }
+                }
+            }
+        }
+        __syncthreads(); // s_acc is reused by the second row
+    }
+}
+
 // grid (hQ, slots), 256 threads: folds the ranges of one query head in range order, divides by the
 // sum and applies the output gate sigmoid(qfull[head][dh + t]).  Wave w adds the ranges w, w+4, ...
 // (a lane 4 dims, eight ranges requested at a time); the waves' sums are added in wave order.
@@ -393,8 +534,12 @@ static int attn_decode_impl(const char* who, const float* qhat, const float* k_c
     AttnWs ws;
     ws.acc = (float*)workspace;
     ws.ml = ws.acc + (size_t)rows * hQ * n_ranges * ATT_DH;
-    hipLaunchKernelGGL(attn_range_kernel, dim3(n_ranges, hKV, rows), dim3(256), 0, st, qhat, k_cache, v_cache, slot_pos, ws,
-                       hQ, hKV, hQ / hKV, tmax, own);
+    if (own == 0 && rows >= 2)
+        hipLaunchKernelGGL(attn_range_pair_kernel, dim3(n_ranges, hKV, (rows + 1) / 2), dim3(256), 0, st, qhat, k_cache,
+                           v_cache, slot_pos, ws, hQ, hKV, hQ / hKV, tmax, rows);
+    else
+        hipLaunchKernelGGL(attn_range_kernel, dim3(n_ranges, hKV, rows), dim3(256), 0, st, qhat, k_cache, v_cache, slot_pos,
+                           ws, hQ, hKV, hQ / hKV, tmax, own);
     hipLaunchKernelGGL(attn_fold_kernel, dim3(hQ, rows), dim3(256), 0, st, ws, qfull, slot_pos, att, hQ, tmax, n_ranges);
     return check_launch(who);
 }
