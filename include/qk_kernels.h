@@ -286,6 +286,12 @@ int qkk_dn_ab(const float *x, const float *alpha_w, const float *beta_w, const f
               const float *a_vec, float *gb, uint32_t n_embd, uint32_t hV, uint32_t n_slots, void *stream);
 int qkk_dn_conv(float *conv_state, const float *qkv, const float *ker, float *out, uint32_t channels,
                 uint32_t d_state, uint32_t qk_channels, float eps, uint32_t n_slots, void *stream);
+/* qkk_dn_ab and qkk_dn_conv in one launch (neither reads what the other writes; the same results
+ * bit for bit): for decode steps, where two launches of a few microseconds are mostly launch ramp. */
+int qkk_dn_ab_conv(const float *x, const float *alpha_w, const float *beta_w, const float *dt_bias,
+                   const float *a_vec, float *gb, uint32_t n_embd, uint32_t hV, float *conv_state,
+                   const float *qkv, const float *ker, float *out, uint32_t channels, uint32_t d_state,
+                   uint32_t qk_channels, float eps, uint32_t n_slots, void *stream);
 int qkk_dn_step(const float *conv, const float *gb, float *state, const float *norm_w, const float *z,
                 float *att, uint32_t d_state, uint32_t hK, uint32_t hV, uint32_t kdiv, float eps,
                 uint32_t n_slots, void *stream);

@@ -11,7 +11,7 @@ from .capi import (  # noqa: F401
     dequant, gemv, moe_decode, moe_workspace_bytes, head_argmax, head_workspace_bytes, argmax,
     moe_group_pairs, gemm_q8_0, moe_prefill, moe_prefill_workspace_bytes, device_info,
     rmsnorm, add_rmsnorm, add_rms3, vec_add, embed, moe_decode_tail, moe_layer_rows, ROWWISE_MAX,
-    rope_table, attn_prep, attn_workspace_bytes, attn_decode, dn_ab, dn_conv, dn_step,
+    rope_table, attn_prep, attn_workspace_bytes, attn_decode, dn_ab, dn_conv, dn_step, dn_ab_conv,
 )
 from . import synth  # noqa: F401
 from . import gguf  # noqa: F401

@@ -76,6 +76,7 @@ def lib():
         L.qkk_dn_conv.argtypes = [vp] * 4 + [u32] * 3 + [f32, u32, vp]
         L.qkk_dn_step.argtypes = [vp] * 6 + [u32] * 4 + [f32, u32, vp]
         L.qkk_dn_conv_seq.argtypes = L.qkk_dn_conv.argtypes
+        L.qkk_dn_ab_conv.argtypes = [vp] * 6 + [u32, u32] + [vp] * 4 + [u32] * 3 + [f32, u32, vp]
         L.qkk_dn_step_seq.argtypes = L.qkk_dn_step.argtypes
         L.qkk_rope_table.argtypes = [vp, u32, u32, f32]
         L.qkk_attn_prep.argtypes = [vp] * 10 + [u32] * 6 + [f32, vp]
@@ -382,6 +383,21 @@ def dn_ab(x, alpha_w, beta_w, dt_bias, a_vec, gb=None):
     _check(lib().qkk_dn_ab(_ptr(x), _ptr(alpha_w), _ptr(beta_w), _ptr(dt_bias), _ptr(a_vec), _ptr(gb), x.shape[1], hV, n,
                            _stream()))
     return gb
+
+
+def dn_ab_conv(x, alpha_w, beta_w, dt_bias, a_vec, conv_state, qkv, ker, qk_channels, d_state=128, eps=1e-6):
+    """dn_ab and dn_conv in one launch.  Returns (gb [slots][2*hV], out [slots][channels]); conv_state is
+    updated in place."""
+    import torch
+    n, hV, channels = x.shape[0], alpha_w.shape[0], qkv.shape[1]
+    if qkv.shape[0] != n or conv_state.numel() != n * channels * 3:
+        raise ValueError("dn_ab_conv: shapes do not match the rows")
+    gb = torch.empty((n, 2 * hV), dtype=torch.float32, device=x.device)
+    out = torch.empty_like(qkv)
+    _check(lib().qkk_dn_ab_conv(_ptr(x), _ptr(alpha_w), _ptr(beta_w), _ptr(dt_bias), _ptr(a_vec), _ptr(gb), x.shape[1], hV,
+                                _ptr(conv_state), _ptr(qkv), _ptr(ker), _ptr(out), channels, d_state, qk_channels, eps, n,
+                                _stream()))
+    return gb, out
 
 
 def dn_conv(conv_state, qkv, ker, qk_channels, d_state=128, eps=1e-6, out=None, seq=False):

@@ -80,6 +80,58 @@ __global__ __launch_bounds__(128) void dn_conv_kernel(float* __restrict__ st, co
     out[(size_t)rq * channels + ch] = v;
 }
 
+// dn_ab and dn_conv in one launch for a decode step (neither needs the other's result; two launches
+// of 3-5 us each are mostly launch ramp): grid (channels / dS + hV, slots), 128 threads.  Workgroups
+// below channels / dS run the conv of one head exactly as dn_conv_kernel; the others form two outputs
+// of dn_ab each (one per wave: g of head b and beta of head b), exactly as dn_ab_kernel.
+template <int NCH>
+__global__ __launch_bounds__(128) void dn_ab_conv_kernel(float* __restrict__ st, const float* __restrict__ qkv,
+                                                         const float* __restrict__ ker, float* __restrict__ out,
+                                                         uint32_t channels, uint32_t qk_channels, float eps,
+                                                         const float* __restrict__ x, const float* __restrict__ alpha_w,
+                                                         const float* __restrict__ beta_w, const float* __restrict__ dt_bias,
+                                                         const float* __restrict__ a_vec, float* __restrict__ gb, uint32_t hV)
+{
+    __shared__ float s_red[2];
+    const uint32_t rq = blockIdx.y, conv_blocks = channels / DN_DS;
+    if (blockIdx.x < conv_blocks) { // uniform per workgroup
+        const uint32_t ch = blockIdx.x * DN_DS + threadIdx.x;
+        float* s = st + ((size_t)rq * channels + ch) * 3;
+        const float s0 = s[0], s1 = s[1], s2 = s[2], xin = qkv[(size_t)rq * channels + ch];
+        const float4 k = ((const float4*)ker)[ch];
+        const float c = s0 * k.x + s1 * k.y + s2 * k.z + xin * k.w;
+        float v = c / (1.f + expf(-c));
+        s[0] = s1; s[1] = s2; s[2] = xin;
+        if (blockIdx.x * DN_DS < qk_channels) v *= 1.f / fmaxf(sqrtf(block_sum2(v * v, s_red)), eps);
+        out[(size_t)rq * channels + ch] = v;
+        return;
+    }
+    const uint32_t lane = threadIdx.x & 63u, h = blockIdx.x - conv_blocks;
+    const bool is_beta = threadIdx.x >= 64; // wave 0: g, wave 1: beta
+    const float4* row = (const float4*)((is_beta ? beta_w : alpha_w) + (size_t)h * 256 * NCH);
+    const float4* xv = (const float4*)(x + (size_t)rq * 256 * NCH);
+    float4 a[NCH], b[NCH];
+#pragma unroll
+    for (int i = 0; i < NCH; i++) a[i] = row[lane + 64 * i];
+#pragma unroll
+    for (int i = 0; i < NCH; i++) b[i] = xv[lane + 64 * i];
+    float p0 = 0.f, p1 = 0.f;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        p0 += a[i].x * b[i].x + a[i].y * b[i].y;
+        p1 += a[i].z * b[i].z + a[i].w * b[i].w;
+    }
+    const float d = wave_sum(p0 + p1);
+    if (lane == 0) {
+        if (is_beta) {
+            gb[(size_t)rq * 2 * hV + hV + h] = 1.f / (1.f + expf(-d));
+        } else {
+            const float v = d + dt_bias[h];
+            gb[(size_t)rq * 2 * hV + h] = a_vec[h] * (v > 20.f ? v : log1pf(expf(v)));
+        }
+    }
+}
+
 // The step: grid (hV, slots), 128 * DN_PARTS threads.  A row's columns are cut into DN_PARTS parts:
 // thread (row j = t % 128, part c = t / 128) keeps dS / DN_PARTS state values -- one round of loads --
 // and the two sums over columns are finished through LDS (a wave holds one part of 64 consecutive
@@ -371,6 +423,34 @@ int qkk_dn_conv(float* conv_state, const float* qkv, const float* ker, float* ou
     hipLaunchKernelGGL(dn_conv_kernel, dim3(channels / DN_DS, n_slots), dim3(DN_DS), 0, as_stream(stream), conv_state, qkv,
                        ker, out, channels, qk_channels, eps);
     return check_launch("qkk_dn_conv");
+}
+
+int qkk_dn_ab_conv(const float* x, const float* alpha_w, const float* beta_w, const float* dt_bias, const float* a_vec,
+                   float* gb, uint32_t n_embd, uint32_t hV, float* conv_state, const float* qkv, const float* ker, float* out,
+                   uint32_t channels, uint32_t d_state, uint32_t qk_channels, float eps, uint32_t n_slots, void* stream)
+{
+    if (!x || !alpha_w || !beta_w || !dt_bias || !a_vec || !gb || !conv_state || !qkv || !ker || !out)
+        return fail(QKK_EINVAL, "qkk_dn_ab_conv: null pointer");
+    if (int rc = check_slots("qkk_dn_ab_conv", n_slots)) return rc;
+    if (n_embd != 2048 && n_embd != 4096)
+        return fail(QKK_ESHAPE, "qkk_dn_ab_conv: n_embd %u not supported (2048 or 4096)", n_embd);
+    if (hV < 1 || hV > 4096) return fail(QKK_ESHAPE, "qkk_dn_ab_conv: %u heads outside 1..4096", hV);
+    if (d_state != DN_DS) return fail(QKK_ESHAPE, "qkk_dn_ab_conv: state size %u not supported (128)", d_state);
+    if (channels < DN_DS || channels % DN_DS || qk_channels % DN_DS || qk_channels > channels || channels > (1u << 24))
+        return fail(QKK_ESHAPE, "qkk_dn_ab_conv: %u channels (%u of q and k) must be whole heads of %u", channels,
+                    qk_channels, DN_DS);
+    if (!aligned16(x) || !aligned16(alpha_w) || !aligned16(beta_w) || !aligned16(ker))
+        return fail(QKK_EINVAL, "qkk_dn_ab_conv: x, the weight rows and ker must be 16-byte aligned");
+    if (!(eps >= 0.f)) return fail(QKK_EINVAL, "qkk_dn_ab_conv: eps must be non-negative");
+    if (int rc = require_device()) return rc;
+    const dim3 grid(channels / DN_DS + hV, n_slots), block(DN_DS);
+    if (n_embd == 2048)
+        hipLaunchKernelGGL(dn_ab_conv_kernel<8>, grid, block, 0, as_stream(stream), conv_state, qkv, ker, out, channels,
+                           qk_channels, eps, x, alpha_w, beta_w, dt_bias, a_vec, gb, hV);
+    else
+        hipLaunchKernelGGL(dn_ab_conv_kernel<16>, grid, block, 0, as_stream(stream), conv_state, qkv, ker, out, channels,
+                           qk_channels, eps, x, alpha_w, beta_w, dt_bias, a_vec, gb, hV);
+    return check_launch("qkk_dn_ab_conv");
 }
 
 int qkk_dn_conv_seq(float* conv_state, const float* qkv, const float* ker, float* out, uint32_t channels, uint32_t d_state,

@@ -247,14 +247,17 @@ int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool 
                 if (int rc = dense(L.p1, xn, d_big, rows, st)) return rc;
                 if (int rc = dense(L.p2, xn, d_mid, rows, st)) return rc;
             }
-            if (int rc = qkk_dn_ab(xn, L.alpha_w, L.beta_w, L.dt_bias, L.a_vec, d_gb, N_EMBD, DN_HV, rows, st)) return rc;
             if (seq) {
+                if (int rc = qkk_dn_ab(xn, L.alpha_w, L.beta_w, L.dt_bias, L.a_vec, d_gb, N_EMBD, DN_HV, rows, st)) return rc;
                 if (int rc = qkk_dn_conv_seq(s1, d_big, L.ker, d_conv, DN_CH, DN_DS, 2 * DN_HK * DN_DS, eps, rows, st)) return rc;
                 if (int rc = qkk_dn_step_seq(d_conv, d_gb, s2, L.ssm_norm, d_mid, d_att, DN_DS, DN_HK, DN_HV, dn_kdiv, eps, rows,
                                              st))
                     return rc;
             } else {
-                if (int rc = qkk_dn_conv(s1, d_big, L.ker, d_conv, DN_CH, DN_DS, 2 * DN_HK * DN_DS, eps, rows, st)) return rc;
+                // decay / write strength and the conv in one launch
+                if (int rc = qkk_dn_ab_conv(xn, L.alpha_w, L.beta_w, L.dt_bias, L.a_vec, d_gb, N_EMBD, DN_HV, s1, d_big, L.ker,
+                                            d_conv, DN_CH, DN_DS, 2 * DN_HK * DN_DS, eps, rows, st))
+                    return rc;
                 if (int rc = qkk_dn_step(d_conv, d_gb, s2, L.ssm_norm, d_mid, d_att, DN_DS, DN_HK, DN_HV, dn_kdiv, eps, rows, st))
                     return rc;
             }

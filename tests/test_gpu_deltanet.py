@@ -52,7 +52,11 @@ def run_tokens(qk, dev, w, n_slots, n_tok, seed, kdiv=0, ne=NE):
         qkv = rng.standard_normal((n_slots, w.ch)).astype(F)
         z = rng.standard_normal((n_slots, w.hv * DS)).astype(F)
         gb = qk.dn_ab(up(x), wd["alpha_w"], wd["beta_w"], wd["dt_bias"], wd["a_vec"])
+        st_before = std.clone()
         conv = qk.dn_conv(std, up(qkv), wd["ker"], w.qk)
+        # the two in one launch: the same bits, the same window
+        gb2, conv2 = qk.dn_ab_conv(up(x), wd["alpha_w"], wd["beta_w"], wd["dt_bias"], wd["a_vec"], st_before, up(qkv), wd["ker"], w.qk)
+        assert torch.equal(gb2, gb) and torch.equal(conv2, conv) and torch.equal(st_before, std)
         att = qk.dn_step(conv, gb, Sd, wd["norm_w"], up(z), w.hk, w.hv, kdiv=kdiv)
         torch.cuda.synchronize()
         gb, conv, att = gb.cpu().numpy(), conv.cpu().numpy(), att.cpu().numpy()
