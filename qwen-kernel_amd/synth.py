@@ -83,7 +83,8 @@ def blocks_device(type_, n_blocks, seed, device="cuda", d_scale=1e-3):
 
 
 class HostLayer:
-    """One synthetic MoE layer on the host (numpy), the reference model's shapes by default (2048 wide, 256 experts of 512, 8 used)."""
+    """One synthetic MoE layer on the host (numpy), the reference model's shapes by default
+    (2048 wide, 256 experts of 512, 8 used)."""
 
     def __init__(self, seed, n_embd=2048, n_ff=512, n_expert=256, n_used=8, down_type=IQ4_XS, gu_type=IQ3_XXS,
                  d_scale=1e-3):
