@@ -134,7 +134,7 @@ def test_attention_argument_checks(qk, dev):
     assert float(vc[0, 0, 63, 0]) == 3.0 and float(vc[0, :, :63].abs().max()) == 0.0
 
 
-@pytest.mark.parametrize("tmax,base,n_pos", [(96, 0, 1), (96, 0, 70), (96, 5, 33), (300, 150, 128), (4096, 3000, 40)])
+@pytest.mark.parametrize("tmax,base,n_pos", [(96, 0, 1), (96, 0, 70), (96, 5, 33), (300, 150, 128), (4096, 3000, 40), (4096, 3050, 1023)])
 def test_attention_sequence_forms_equal_the_steps(qk, dev, tmax, base, n_pos):
     """qkk_attn_prep_seq / qkk_attn_seq over n_pos consecutive positions of one slot whose cache
     already holds `base` rows: row t sees the cache rows 0..base+t.  Against the decode-step entry
