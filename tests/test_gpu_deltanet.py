@@ -112,7 +112,7 @@ def test_deltanet_argument_checks(qk, dev):
     assert e.value.code == -2
 
 
-@pytest.mark.parametrize("n_pos,kdiv", [(1, 0), (2, 0), (16, 0), (17, 2), (37, 2), (128, 0)])
+@pytest.mark.parametrize("n_pos,kdiv", [(1, 0), (2, 0), (16, 0), (17, 2), (37, 2), (128, 0), (1000, 2)])
 def test_deltanet_sequence_forms_equal_the_steps(qk, dev, n_pos, kdiv):
     """qkk_dn_conv_seq / qkk_dn_step_seq over n_pos consecutive positions of one slot (a state of
     earlier positions already in place): the outputs and the final window / state of n_pos calls of
