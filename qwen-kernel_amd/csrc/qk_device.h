@@ -43,9 +43,10 @@ __host__ __device__ constexpr size_t qkk_row_bytes_dev(uint64_t k)
 // A release fence at device scope writes back the whole L2 of the XCD (buffer_wbl2); issued
 // once per workgroup by a thousand workgroups it costs tens of microseconds.  Values another
 // workgroup of the same launch will read are therefore stored with device-scope atomic stores
-// (written through to memory), the arrival is counted with a relaxed device-scope atomic after
-// the stores have completed, and only the single workgroup that reads them executes an acquire
-// fence (cache invalidate).
+// (written through to memory); every lane that published waits for its own stores to be
+// acknowledged (publish_wait) before the workgroup's barrier, the arrival is then counted with a
+// relaxed device-scope atomic, and only the single workgroup that reads the values executes an
+// acquire fence (cache invalidate).
 __device__ __forceinline__ void publish(float* p, float v)
 {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -54,12 +55,21 @@ __device__ __forceinline__ void publish(uint32_t* p, uint32_t v)
 {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// Called by ONE thread after a __syncthreads() that follows the workgroup's publish() calls.
-// Returns true for the workgroup that arrives last; that one may then read what the others
-// published.
+// Waits until every vector-memory operation of this wave, the publish() stores among them, has been
+// acknowledged: s_waitcnt vmcnt(0) (expcnt and lgkmcnt fields left at their maxima).  A workgroup-scope
+// release fence does not do this -- it only drains the LDS/scalar counter -- so without the wait the
+// arrival below could be counted while a published value is still on its way to another L2 channel.
+__device__ __forceinline__ void publish_wait()
+{
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    asm volatile("" ::: "memory");
+}
+// Called by ONE thread after a __syncthreads() that follows the workgroup's publish() +
+// publish_wait() calls (the caller's own stores are waited for here as well).  Returns true for the
+// workgroup that arrives last; that one may then read what the others published.
 __device__ __forceinline__ bool arrive_last(uint32_t* counter, uint32_t n_workgroups)
 {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); // the stores above have completed
+    publish_wait();
     const bool last =
         __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == n_workgroups - 1;
     if (last) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");

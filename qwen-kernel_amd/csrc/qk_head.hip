@@ -239,6 +239,7 @@ __global__ __launch_bounds__(CT) void head_q6k_coop_kernel(const uint8_t* __rest
             }
         publish(&ws.cand_v[(size_t)tid * gridDim.x + blockIdx.x], v);
         publish(&ws.cand_i[(size_t)tid * gridDim.x + blockIdx.x], i);
+        publish_wait(); // acknowledged before the barrier and the arrival count
     }
     __syncthreads();
     if (tid == 0) s_last = arrive_last(&ws.counter[0], gridDim.x) ? 1u : 0u;

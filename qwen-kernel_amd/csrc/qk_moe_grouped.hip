@@ -55,6 +55,7 @@ __device__ static void select_tokens(const MoeWs& ws, qkk_sel* __restrict__ sel,
         }
         __builtin_amdgcn_wave_barrier();
     }
+    if (publish_ids) publish_wait(); // acknowledged before the caller's barrier and arrival count
 }
 
 // ---- grouping of the N*k (token, pick) pairs by expert, by one workgroup of NW waves ----------
@@ -155,6 +156,7 @@ __global__ __launch_bounds__(512) void moe_route_multi_kernel(const float* __res
     }
     if (!select_here) return;
 
+    publish_wait(); // every wave's logits are acknowledged before the arrival is counted
     __syncthreads();
     if (threadIdx.x == 0) s_last = arrive_last(&ws.counter[0], gridDim.x) ? 1u : 0u;
     __syncthreads();
