@@ -121,6 +121,21 @@ size_t qkk_moe_workspace_bytes(const qkk_moe_layer *L_host, uint32_t n_slots);
 int qkk_moe_decode(const qkk_moe_layer *L_host, const float *X, float *Y, qkk_sel *sel,
                    void *workspace, size_t workspace_bytes, uint32_t n_slots, void *stream);
 
+/* qkk_moe_decode without a workspace argument, for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  The workspace is a device array of QKK_MOE_STATIC_BYTES inside the
+ * library (one copy per device, held until the process ends); the entry point calls no hipMalloc,
+ * hipFree or other allocating routine.  Same kernels, same results bit for bit as qkk_moe_decode.
+ *   n_slots <= QKK_MOE_STATIC_MAX_SLOTS; a layer shape whose workspace exceeds the array is refused
+ *   with QKK_EWORKSPACE (n_embd 2048, n_ff 512, 256 experts, 8 picks, 16 rows need 1.5 MB).
+ * Every call on a device shares that device's array: calls that overlap in time on one device race,
+ * whatever their streams.  The array's address is resolved on the first call on a device (or by
+ * qkk_device_info); make that call outside a stream capture. */
+#define QKK_MOE_STATIC_MAX_SLOTS 16u
+#define QKK_MOE_STATIC_BYTES (2u << 20)
+int qkk_moe_decode_static(const qkk_moe_layer *L_host, const float *X, float *Y, qkk_sel *sel,
+                          uint32_t n_slots, void *stream);
+
 /* The step followed by the layer tail (reference src/main.cpp:4379-4402 with add_rms3.comp:24-41,
  * for several rows add_rms3_grouped.comp:22-50):
  *   S[r]  = resid[r] + (routed + shared contribution of row r)    the next layer's residual input

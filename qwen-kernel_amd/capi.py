@@ -57,6 +57,7 @@ def lib():
         L.qkk_dequant.argtypes = [C.c_int, vp, vp, u64, vp]
         L.qkk_gemv.argtypes = [C.c_int, vp, vp, vp, u32, u32, u32, vp]
         L.qkk_moe_decode.argtypes = [vp, vp, vp, vp, vp, sz, u32, vp]
+        L.qkk_moe_decode_static.argtypes = [vp, vp, vp, vp, u32, vp]
         L.qkk_moe_decode_stages.argtypes = [vp, vp, vp, vp, vp, sz, u32, u32, vp]
         L.qkk_moe_decode_tail.argtypes = [vp, vp, vp, vp, C.c_float, vp, vp, vp, vp, sz, u32, vp]
         L.qkk_moe_layer_rows.argtypes = [vp, vp, vp, C.c_float, vp, vp, sz, u32, vp]
@@ -177,6 +178,17 @@ def moe_decode(layer, X, workspace, Y=None, sel=None, stages=None):
     else:
         _check(lib().qkk_moe_decode_stages(C.byref(layer.c), _ptr(X), _ptr(Y), _ptr(sel), _ptr(workspace), wsb,
                                            n, stages, _stream()))
+    return Y, sel
+
+
+MOE_STATIC_MAX_SLOTS = 16        # QKK_MOE_STATIC_MAX_SLOTS
+MOE_STATIC_BYTES = 2 << 20       # QKK_MOE_STATIC_BYTES
+
+
+def moe_decode_static(layer, X, Y, sel):
+    """qkk_moe_decode on the library's own static workspace: allocates nothing, so the caller
+    passes every output (Y [n_slots, n_embd] fp32, sel uint8 [n_slots, 160])."""
+    _check(lib().qkk_moe_decode_static(C.byref(layer.c), _ptr(X), _ptr(Y), _ptr(sel), X.shape[0], _stream()))
     return Y, sel
 
 

@@ -394,6 +394,7 @@ bool coop_gemm_launch(int type, const uint8_t* W, const float* X, float* Y, uint
 // rows from which the weights are read once for all rows on the matrix cores; K = 4096 takes two
 // passes there (13 us at 2048 x 4096 whatever the batch), so one more row stays on one pass per row
 constexpr uint32_t COOP_MIN_BATCH = 3, COOP_MIN_BATCH_K4096 = 4;
+void* moe_static_scratch();
 } // namespace qk
 
 extern "C" {
@@ -416,6 +417,7 @@ int qkk_device_info(char* arch_host, size_t arch_len, uint32_t* n_cu_host)
             if (arch_host && arch_len) snprintf(arch_host, arch_len, "%s", p.gcnArchName);
             if (n_cu_host) *n_cu_host = (uint32_t)p.multiProcessorCount;
         }
+        (void)moe_static_scratch(); // set-up for qkk_moe_decode_static on the current device
     }
     return n;
 }

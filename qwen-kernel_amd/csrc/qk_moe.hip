@@ -13,6 +13,8 @@
 // dropped.)  Several rows go through the expert-major path in qk_moe_grouped.hip.
 #include "qk_moe_common.h"
 
+#include <mutex>
+
 namespace qk {
 
 // ---- launch 1: router logits + shared gate/up ---------------------------------------------
@@ -669,6 +671,49 @@ static void launch_route_gateup(const qkk_moe_layer* L, const float* X, const Mo
     }
 }
 
+// ---- the step for callers that cannot allocate ---------------------------------------------------
+// The workspace of qkk_moe_decode as a file-scope device array: each device the library runs on holds
+// its own copy, at its own address, until the process ends.  In host code the array's name is only a
+// stand-in for that address; it is resolved once per device (with that device current) and every
+// launch takes the resolved pointer.
+static __device__ __align__(256) unsigned char scratch[QKK_MOE_STATIC_BYTES];
+
+namespace qk {
+constexpr int MAX_DEVICES = 64;
+static void* g_scratch_ptr[MAX_DEVICES]; // resolved device address of `scratch`, per device
+static std::mutex g_scratch_mu;
+
+// Address of the current device's copy of the array, or nullptr with the error recorded.
+void* moe_static_scratch()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+        (void)hipGetLastError();
+        fail(QKK_EDEVICE, "qkk_moe_decode_static: no current HIP device below %d", MAX_DEVICES);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            (void)hipGetLastError();
+            fail(QKK_EDEVICE, "qkk_moe_decode_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    return g_scratch_ptr[dev];
+}
+
+// Clears the arrival counters at the head of the workspace (a fill kernel, not a memset node: the
+// caller may be capturing a graph).
+__global__ void moe_static_clear_kernel(uint32_t* counters)
+{
+    counters[threadIdx.x] = 0u;
+}
+} // namespace qk
+
 extern "C" {
 
 size_t qkk_moe_workspace_bytes(const qkk_moe_layer* L, uint32_t n_slots)
@@ -719,6 +764,27 @@ int qkk_moe_decode(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* se
 {
     return moe_decode_impl("qkk_moe_decode", L, X, Y, sel, workspace, workspace_bytes, n_slots, QKK_STAGE_ALL,
                            stream);
+}
+
+int qkk_moe_decode_static(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* sel, uint32_t n_slots,
+                          void* stream)
+{
+    const char* who = "qkk_moe_decode_static";
+    if (int rc = check_layer(L, who)) return rc;
+    if (n_slots < 1 || n_slots > QKK_MOE_STATIC_MAX_SLOTS)
+        return fail(QKK_ESHAPE, "%s: %u rows outside 1..%u", who, n_slots, QKK_MOE_STATIC_MAX_SLOTS);
+    const MoeDims d{L->n_embd, L->n_ff, L->n_expert, L->n_used};
+    if (ws_bytes(d, n_slots) > QKK_MOE_STATIC_BYTES)
+        return fail(QKK_EWORKSPACE, "%s: this layer shape with %u rows needs %zu bytes of workspace, the static array holds %u",
+                    who, n_slots, ws_bytes(d, n_slots), QKK_MOE_STATIC_BYTES);
+    if (int rc = require_device()) return rc;
+    void* ws = moe_static_scratch();
+    if (!ws) return QKK_EDEVICE;
+    // The array keeps what the last call left.  Logits, h, pair lists and contributions are written
+    // before they are read; the arrival counters of the expert-major path must start at zero.
+    if (n_slots > ROWWISE_MAX)
+        hipLaunchKernelGGL(moe_static_clear_kernel, dim3(1), dim3(64), 0, as_stream(stream), (uint32_t*)ws);
+    return moe_decode_impl(who, L, X, Y, sel, ws, QKK_MOE_STATIC_BYTES, n_slots, QKK_STAGE_ALL, stream);
 }
 
 int qkk_moe_decode_tail(const qkk_moe_layer* L, const float* X, const float* resid, const float* w_next, float eps,
