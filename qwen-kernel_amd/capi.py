@@ -34,6 +34,66 @@ def lib_path():
 _lib = None
 
 
+def _signatures():
+    """name -> (restype or None for int, argtypes) of every entry point the wrappers call."""
+    vp, u32, u64, sz, f32, i32 = C.c_void_p, C.c_uint32, C.c_uint64, C.c_size_t, C.c_float, C.c_int
+    dn_conv = [vp] * 4 + [u32] * 3 + [f32, u32, vp]
+    dn_step = [vp] * 6 + [u32] * 4 + [f32, u32, vp]
+    attn_prep = [vp] * 10 + [u32] * 6 + [f32, vp]
+    attn_decode = [vp] * 7 + [sz] + [u32] * 5 + [vp]
+    return {
+        "qkk_last_error": (C.c_char_p, []),
+        "qkk_row_bytes": (sz, [i32, u64]),
+        "qkk_moe_workspace_bytes": (sz, [vp, u32]),
+        "qkk_moe_prefill_workspace_bytes": (sz, [vp, u32]),
+        "qkk_head_workspace_bytes": (sz, [u32, u32]),
+        "qkk_attn_workspace_bytes": (sz, [u32, u32, u32]),
+        "qkk_device_info": (None, [C.c_char_p, sz, C.POINTER(u32)]),
+        "qkk_dequant": (None, [i32, vp, vp, u64, vp]),
+        "qkk_gemv": (None, [i32, vp, vp, vp, u32, u32, u32, vp]),
+        "qkk_moe_decode": (None, [vp, vp, vp, vp, vp, sz, u32, vp]),
+        "qkk_moe_decode_static": (None, [vp, vp, vp, vp, u32, vp]),
+        "qkk_moe_decode_stages": (None, [vp, vp, vp, vp, vp, sz, u32, u32, vp]),
+        "qkk_moe_decode_tail": (None, [vp, vp, vp, vp, f32, vp, vp, vp, vp, sz, u32, vp]),
+        "qkk_moe_layer_rows": (None, [vp, vp, vp, f32, vp, vp, sz, u32, vp]),
+        "qkk_moe_layer_rows_add": (None, [vp, vp, vp, vp, vp, f32, vp, vp, sz, u32, vp]),
+        "qkk_moe_group_pairs": (None, [vp, u32, u32, u32, vp, vp, vp]),
+        "qkk_head_argmax": (None, [vp, vp, vp, vp, u32, u32, u32, vp, sz, vp]),
+        "qkk_argmax": (None, [vp, vp, u32, u32, vp]),
+        "qkk_gemm_q8_0": (None, [vp, vp, vp, u32, u32, u32, vp]),
+        "qkk_moe_prefill": (None, [vp, vp, vp, vp, vp, sz, u32, vp]),
+        "qkk_rmsnorm": (None, [vp, vp, vp, u32, u32, f32, vp]),
+        "qkk_add_rmsnorm": (None, [vp, vp, vp, vp, vp, u32, u32, f32, vp]),
+        "qkk_add_rms3": (None, [vp, vp, vp, vp, vp, vp, u32, u32, f32, vp]),
+        "qkk_vec_add": (None, [vp, vp, vp, u64, vp]),
+        "qkk_embed": (None, [i32, vp, u32, u32, vp, u32, u32, u32, vp, u32, vp]),
+        "qkk_dn_ab": (None, [vp] * 6 + [u32] * 3 + [vp]),
+        "qkk_dn_conv": (None, dn_conv),
+        "qkk_dn_conv_seq": (None, dn_conv),
+        "qkk_dn_step": (None, dn_step),
+        "qkk_dn_step_seq": (None, dn_step),
+        "qkk_dn_ab_conv": (None, [vp] * 6 + [u32, u32] + [vp] * 4 + [u32] * 3 + [f32, u32, vp]),
+        "qkk_rope_table": (None, [vp, u32, u32, f32]),
+        "qkk_attn_prep": (None, attn_prep),
+        "qkk_attn_prep_seq": (None, attn_prep),
+        "qkk_attn_decode": (None, attn_decode),
+        "qkk_attn_seq": (None, attn_decode),
+    }
+
+
+def bind(L, partial=False):
+    """Declares the C signatures on a loaded library.  partial: skip entry points the library does not
+    export (the tests' host-side build of some kernels)."""
+    for name, (restype, argtypes) in _signatures().items():
+        if partial and not hasattr(L, name):
+            continue
+        f = getattr(L, name)
+        f.argtypes = argtypes
+        if restype is not None:
+            f.restype = restype
+    return L
+
+
 def lib():
     """Loads libqk.so from the package directory; raises if it has not been built."""
     global _lib
@@ -42,51 +102,7 @@ def lib():
         if not os.path.exists(p):
             raise QkError(-4, f"{p} is missing: build it with `make -C qwen-kernel_amd` "
                               "(or __graft_entry__.build()); there is no fallback path")
-        L = C.CDLL(p)
-        L.qkk_last_error.restype = C.c_char_p
-        L.qkk_row_bytes.restype = C.c_size_t
-        L.qkk_row_bytes.argtypes = [C.c_int, C.c_uint64]
-        L.qkk_moe_workspace_bytes.restype = C.c_size_t
-        L.qkk_moe_workspace_bytes.argtypes = [C.c_void_p, C.c_uint32]
-        L.qkk_moe_prefill_workspace_bytes.restype = C.c_size_t
-        L.qkk_moe_prefill_workspace_bytes.argtypes = [C.c_void_p, C.c_uint32]
-        L.qkk_head_workspace_bytes.restype = C.c_size_t
-        L.qkk_head_workspace_bytes.argtypes = [C.c_uint32, C.c_uint32]
-        L.qkk_device_info.argtypes = [C.c_char_p, C.c_size_t, C.POINTER(C.c_uint32)]
-        vp, u32, u64, sz = C.c_void_p, C.c_uint32, C.c_uint64, C.c_size_t
-        L.qkk_dequant.argtypes = [C.c_int, vp, vp, u64, vp]
-        L.qkk_gemv.argtypes = [C.c_int, vp, vp, vp, u32, u32, u32, vp]
-        L.qkk_moe_decode.argtypes = [vp, vp, vp, vp, vp, sz, u32, vp]
-        L.qkk_moe_decode_static.argtypes = [vp, vp, vp, vp, u32, vp]
-        L.qkk_moe_decode_stages.argtypes = [vp, vp, vp, vp, vp, sz, u32, u32, vp]
-        L.qkk_moe_decode_tail.argtypes = [vp, vp, vp, vp, C.c_float, vp, vp, vp, vp, sz, u32, vp]
-        L.qkk_moe_layer_rows.argtypes = [vp, vp, vp, C.c_float, vp, vp, sz, u32, vp]
-        L.qkk_moe_layer_rows_add.argtypes = [vp, vp, vp, vp, vp, C.c_float, vp, vp, sz, u32, vp]
-        L.qkk_moe_group_pairs.argtypes = [vp, u32, u32, u32, vp, vp, vp]
-        L.qkk_head_argmax.argtypes = [vp, vp, vp, vp, u32, u32, u32, vp, sz, vp]
-        L.qkk_argmax.argtypes = [vp, vp, u32, u32, vp]
-        L.qkk_gemm_q8_0.argtypes = [vp, vp, vp, u32, u32, u32, vp]
-        L.qkk_moe_prefill.argtypes = [vp, vp, vp, vp, vp, sz, u32, vp]
-        f32 = C.c_float
-        L.qkk_rmsnorm.argtypes = [vp, vp, vp, u32, u32, f32, vp]
-        L.qkk_add_rmsnorm.argtypes = [vp, vp, vp, vp, vp, u32, u32, f32, vp]
-        L.qkk_add_rms3.argtypes = [vp, vp, vp, vp, vp, vp, u32, u32, f32, vp]
-        L.qkk_vec_add.argtypes = [vp, vp, vp, u64, vp]
-        L.qkk_embed.argtypes = [C.c_int, vp, u32, u32, vp, u32, u32, u32, vp, u32, vp]
-        L.qkk_dn_ab.argtypes = [vp] * 6 + [u32] * 3 + [vp]
-        L.qkk_dn_conv.argtypes = [vp] * 4 + [u32] * 3 + [f32, u32, vp]
-        L.qkk_dn_step.argtypes = [vp] * 6 + [u32] * 4 + [f32, u32, vp]
-        L.qkk_dn_conv_seq.argtypes = L.qkk_dn_conv.argtypes
-        L.qkk_dn_ab_conv.argtypes = [vp] * 6 + [u32, u32] + [vp] * 4 + [u32] * 3 + [f32, u32, vp]
-        L.qkk_dn_step_seq.argtypes = L.qkk_dn_step.argtypes
-        L.qkk_rope_table.argtypes = [vp, u32, u32, f32]
-        L.qkk_attn_prep.argtypes = [vp] * 10 + [u32] * 6 + [f32, vp]
-        L.qkk_attn_workspace_bytes.restype = sz
-        L.qkk_attn_workspace_bytes.argtypes = [u32, u32, u32]
-        L.qkk_attn_decode.argtypes = [vp] * 7 + [sz] + [u32] * 5 + [vp]
-        L.qkk_attn_prep_seq.argtypes = L.qkk_attn_prep.argtypes
-        L.qkk_attn_seq.argtypes = L.qkk_attn_decode.argtypes
-        _lib = L
+        _lib = bind(C.CDLL(p))
     return _lib
 
 

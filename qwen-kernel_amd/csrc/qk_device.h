@@ -10,6 +10,17 @@ namespace qk {
 
 constexpr int WAVE = 64;
 
+// Two hooks that let a host-side build of these kernels (the tests' bounds and logic check; it
+// defines both before this header is read) supply what only the device has:
+// the dynamic LDS of a launch, declared at the top of a kernel, and the register constraint of the
+// empty asm statements that pin values.
+#ifndef QK_DYN_LDS
+#define QK_DYN_LDS(type, name) extern __shared__ __attribute__((aligned(16))) type name[]
+#endif
+#ifndef QK_REG
+#define QK_REG(x) "+v"(x)
+#endif
+
 // ---- loads -----------------------------------------------------------------------
 // GGUF blocks are 2-byte (Q8_0, Q6_K, IQ3_XXS) or 8-byte (IQ4_XS) aligned.  gfx950
 // global loads accept any byte alignment, so a block field is fetched with the widest
@@ -266,6 +277,28 @@ __device__ __forceinline__ void split_xslice(XSliceH& h, const XSlice& xs)
     }
 }
 
+// IQ4_XS codebook by byte: the weights j and j + 16 of a 32-weight sub-block share byte j, so entry b
+// holds (kv[b & 15], kv[b >> 4]) as two halves (the codebook values are integers below 128: exact).
+static __device__ const int8_t g_iq4nl[16] = {QK_IQ4NL_VALUES};
+struct Iq4PairTable {
+    uint32_t pair[256];
+};
+__device__ __forceinline__ void fill_iq4_pair_entry(Iq4PairTable& t, uint32_t i) // thread i < 256 fills entry i
+{
+    const qk_half2 v = {(_Float16)(float)g_iq4nl[i & 15u], (_Float16)(float)g_iq4nl[i >> 4]};
+    t.pair[i] = __builtin_bit_cast(uint32_t, v);
+}
+// The activations paired the same way: pair j = (x[j], x[j + 16]), as hi + lo halves.
+__device__ __forceinline__ void split_xslice_iq4(XSliceH& h, const XSlice& xs)
+{
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+        const _Float16 a = (_Float16)xs.v[j], b = (_Float16)xs.v[j + 16];
+        h.hi[j] = qk_half2{a, b};
+        h.lo[j] = qk_half2{(_Float16)(xs.v[j] - (float)a), (_Float16)(xs.v[j + 16] - (float)b)};
+    }
+}
+
 // Bytes of weights one lane fetches per pass, held in registers between the load and the
 // arithmetic so several rows can be in flight.
 template <int TYPE>
@@ -280,7 +313,7 @@ struct LaneW<8> { // Q8_0
     __device__ __forceinline__ void touch()
     {
 #pragma unroll
-        for (int i = 0; i < 8; i++) asm volatile("" : "+v"(q[i]));
+        for (int i = 0; i < 8; i++) asm volatile("" : QK_REG(q[i]));
     }
     __device__ __forceinline__ void load(const uint8_t* row, int lane_in_row)
     {
@@ -309,7 +342,7 @@ struct LaneW<14> { // Q6_K
     uint16_t d;
     __device__ __forceinline__ void touch()
     {
-        asm volatile("" : "+v"(qa.x), "+v"(qa.y), "+v"(qb.x), "+v"(qb.y), "+v"(qh.x), "+v"(qh.y));
+        asm volatile("" : QK_REG(qa.x), QK_REG(qa.y), QK_REG(qb.x), QK_REG(qb.y), QK_REG(qh.x), QK_REG(qh.y));
     }
     __device__ __forceinline__ void load(const uint8_t* row, int lane_in_row)
     {
@@ -354,7 +387,7 @@ template <>
 struct LaneW<23> { // IQ4_XS
     uint4 q;
     uint2 hdr; // d | scales_h<<16, scales_l[4]
-    __device__ __forceinline__ void touch() { asm volatile("" : "+v"(q.x), "+v"(q.y), "+v"(q.z), "+v"(q.w)); }
+    __device__ __forceinline__ void touch() { asm volatile("" : QK_REG(q.x), QK_REG(q.y), QK_REG(q.z), QK_REG(q.w)); }
     __device__ __forceinline__ void load(const uint8_t* row, int lane_in_row)
     {
         const int b = lane_in_row >> 3, ib = lane_in_row & 7;
@@ -381,6 +414,28 @@ struct LaneW<23> { // IQ4_XS
         }
         return h2f((uint16_t)hdr.x) * (float)ls * s;
     }
+    // The same product on packed halves: one LDS lookup per byte gives both of its weights, each
+    // v_dot2_f32_f16 takes them against a pair of activations (hi, then lo).  The sixteen lookups are
+    // issued before the first product so that their latencies overlap.
+    __device__ __forceinline__ float dot_h(const XSliceH& xh, const Iq4PairTable* tab, int lane_in_row) const
+    {
+        const int ib = lane_in_row & 7;
+        const uint32_t sh = hdr.x >> 16;
+        const int ls = (int)(((hdr.y >> (4 * ib)) & 0xFu) | (((sh >> (2 * ib)) & 3u) << 4)) - 32;
+        const uint32_t qq[4] = {q.x, q.y, q.z, q.w};
+        uint32_t w[16];
+#pragma unroll
+        for (int k = 0; k < 16; k++) w[k] = tab->pair[(qq[k >> 2] >> (8 * (k & 3))) & 0xFFu];
+        __builtin_amdgcn_sched_barrier(0);
+        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            const qk_half2 wk = __builtin_bit_cast(qk_half2, w[k]);
+            s0 = __builtin_amdgcn_fdot2(wk, xh.hi[k], s0, false);
+            s1 = __builtin_amdgcn_fdot2(wk, xh.lo[k], s1, false);
+        }
+        return h2f((uint16_t)hdr.x) * (float)ls * (s0 + s1);
+    }
 };
 
 template <>
@@ -388,7 +443,7 @@ struct LaneW<18> { // IQ3_XXS
     uint2 g;      // 8 grid indices
     uint32_t aux; // 4 x 7-bit sign selectors + 4-bit scale
     uint16_t d;
-    __device__ __forceinline__ void touch() { asm volatile("" : "+v"(g.x), "+v"(g.y), "+v"(aux)); }
+    __device__ __forceinline__ void touch() { asm volatile("" : QK_REG(g.x), QK_REG(g.y), QK_REG(aux)); }
     __device__ __forceinline__ void load(const uint8_t* row, int lane_in_row)
     {
         const int b = lane_in_row >> 3, ib = lane_in_row & 7;
@@ -422,19 +477,28 @@ struct LaneW<18> { // IQ3_XXS
         return h2f(d) * (0.5f + (float)(aux >> 28)) * 0.5f * s;
     }
     // The same product on packed halves: signed magnitudes come out of two LDS lookups and two
-    // XORs per four weights, each v_dot2_f32_f16 takes two weights (products exact, fp32 sums).
+    // XORs per four weights, each v_dot2_f32_f16 takes two weights (products exact, fp32 sums).  All
+    // twelve lookups are issued before the first product, so that their latencies overlap (one at a
+    // time, as the compiler had scheduled them, a lone lookup's latency was paid twelve times).
     __device__ __forceinline__ float dot_h(const XSliceH& xh, const Iq3HalfTables* tab) const
     {
+        uint2 m[8];
+        uint4 sg[4];
+#pragma unroll
+        for (int l = 0; l < 4; l++) {
+            sg[l] = tab->sign[(aux >> (7 * l)) & 127u];
+            const uint32_t gw = l < 2 ? g.x : g.y;
+#pragma unroll
+            for (int hh = 0; hh < 2; hh++) m[l * 2 + hh] = tab->grid[(gw >> (16 * (l & 1) + 8 * hh)) & 0xFFu];
+        }
+        __builtin_amdgcn_sched_barrier(0);
         float s0 = 0.f, s1 = 0.f;
 #pragma unroll
         for (int l = 0; l < 4; l++) {
-            const uint4 sm = tab->sign[(aux >> (7 * l)) & 127u];
-            const uint32_t gw = l < 2 ? g.x : g.y;
 #pragma unroll
             for (int hh = 0; hh < 2; hh++) {
-                const uint2 m = tab->grid[(gw >> (16 * (l & 1) + 8 * hh)) & 0xFFu];
-                const qk_half2 w01 = __builtin_bit_cast(qk_half2, m.x ^ (hh ? sm.z : sm.x));
-                const qk_half2 w23 = __builtin_bit_cast(qk_half2, m.y ^ (hh ? sm.w : sm.y));
+                const qk_half2 w01 = __builtin_bit_cast(qk_half2, m[l * 2 + hh].x ^ (hh ? sg[l].z : sg[l].x));
+                const qk_half2 w23 = __builtin_bit_cast(qk_half2, m[l * 2 + hh].y ^ (hh ? sg[l].w : sg[l].y));
                 const int q = l * 4 + hh * 2;
                 s0 = __builtin_amdgcn_fdot2(w01, xh.hi[q], s0, false);
                 s1 = __builtin_amdgcn_fdot2(w23, xh.hi[q + 1], s1, false);

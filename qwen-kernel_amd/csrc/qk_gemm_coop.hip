@@ -26,7 +26,7 @@ __global__ __launch_bounds__(CT) void gemm_coop_kernel(const uint8_t* __restrict
 {
     using Geo = GemmGeo<TYPE, KS, NA>;
     constexpr uint32_t KPART = 256 * KS, K = KPART * KP, RB = Geo::RB, RBF = RB * KP, BT = Geo::BT;
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    QK_DYN_LDS(uint8_t, smem);
     __shared__ MfmaTables tab;
     const int tid = threadIdx.x;
     fill_mfma_tables_for<TYPE>(tab, tid, CT); // in place before the stream's first barrier

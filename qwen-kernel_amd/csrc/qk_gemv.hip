@@ -6,6 +6,7 @@
 // flight, and reduces on DPP.  Rows shorter than 2048 share a wave (64/LPR rows per pass).
 #include "qk_device.h"
 #include "qk_host.h"
+#include "qk_stream.h"
 
 #include <stdarg.h>
 
@@ -157,102 +158,114 @@ __global__ __launch_bounds__(256) void dequant_f16_kernel(const uint16_t* __rest
 }
 
 // ---- quantised GEMV ---------------------------------------------------------------------
-// LPR   lanes per row (8..64): a row of K = 32*LPR*PASSES weights.
-// PASSES how many 32*LPR slices a row has; x slices for all passes stay in registers.
-// RIF   rows in flight per lane group: loads of RIF rows are issued before any arithmetic.
-// DEEP  true: two register sets, the next chunk's loads in flight during the arithmetic of the
-//       current one (large matrices); false: one chunk at a time (a wave has one or two chunks).
-template <int TYPE, int LPR, int PASSES, int RIF, bool DEEP>
-__global__ __launch_bounds__(256) void gemv_q_kernel(const uint8_t* __restrict__ W,
-                                                     const float* __restrict__ X,
-                                                     float* __restrict__ Y, uint32_t M, uint32_t K,
-                                                     uint32_t row_bytes)
+// K = 32 * LPR * PASSES.  LPR lanes (8..64) cover 32*LPR weights of a row, so 64/LPR rows lie side
+// by side in a wave; PASSES (1, 2, 4) slices of 2048 weights make up longer rows (LPR = 64 then),
+// the activation slices of all passes stay in registers.
+// The rows are streamed (qk_stream.h): a wave takes chunks of RPC * 64/LPR consecutive rows -- one
+// contiguous byte range, a multiple of 16 bytes for every format -- as 16-byte pieces through its own
+// LDS area, the next chunk's loads in flight during the arithmetic of the current one.  A matrix of a
+// few thousand chunks gets one chunk per wave, so that all of it is requested the moment the launch
+// starts (a launch of this size is latency, not bandwidth); a larger one a persistent grid.  The rows
+// behind the last full chunk are fetched per lane (the exact bytes: a partial chunk would end in a
+// partial piece behind the tensor).  IQ3_XXS and IQ4_XS run their products on packed halves
+// (LaneW::dot_h: LDS lookups that return signed half pairs, v_dot2_f32_f16 against the activations
+// split into hi + lo halves); Q8_0 and Q6_K convert their integers (LaneW::dot).
+template <int TYPE>
+struct GemvShape {
+    static constexpr bool HALF = TYPE == QKK_IQ3_XXS || TYPE == QKK_IQ4_XS;
+    // rows of 2048 weights per chunk: about 3-4 KB in flight per wave
+    static constexpr int RPC2048 = (TYPE == QKK_Q8_0 || TYPE == QKK_Q6_K) ? 2 : 4;
+};
+
+template <int TYPE, int LPR, int PASSES, int RPC>
+__global__ __launch_bounds__(256) void gemv_stream_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X,
+                                                          float* __restrict__ Y, uint32_t M)
 {
-    __shared__ IqTables tab;
-    constexpr bool TABLES = TYPE == QKK_IQ3_XXS || TYPE == QKK_IQ4_XS;
-    // the codebook word travels with the first round trip (activations, first rows) and goes to LDS
-    // after those loads are issued: a fill and a barrier up front would be a round trip of their own
-    uint32_t grid_word = 0;
-    if constexpr (TABLES) grid_word = g_iq3xxs_grid[threadIdx.x];
-    constexpr int GROUPS = WAVE / LPR; // rows a wave works on side by side
+    constexpr int GROUPS = WAVE / LPR;
+    constexpr uint32_t K = 32u * LPR * PASSES;
+    constexpr uint32_t RB = (uint32_t)qkk_row_bytes_dev<TYPE>(K), PB = RB / PASSES;
+    constexpr uint32_t CH = RPC * GROUPS, CB = CH * RB, NPC = CB / 16;
+    constexpr int NP = (NPC + 63) / 64;
+    constexpr bool HALF = GemvShape<TYPE>::HALF;
+    static_assert(CB % 16 == 0, "a chunk of rows must be whole 16-byte pieces");
+    static_assert(PASSES == 1 || LPR == 64, "several passes need whole waves per row");
+    __shared__ __attribute__((aligned(16))) uint8_t s_stage[4][WaveStage<NP>::AREA + 16];
+    __shared__ IqTables tab;        // Q8_0 / Q6_K take no table; the unused ones cost no LDS
+    __shared__ Iq3HalfTables tab3;
+    __shared__ Iq4PairTable tab4;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lir = lane % LPR, grp = lane / LPR;
     const float* x = X + (size_t)blockIdx.y * K;
     float* y = Y + (size_t)blockIdx.y * M;
+    const uint32_t n_full = M / CH, stride = gridDim.x * 4;
+    uint32_t c = blockIdx.x * 4 + wave;
 
-    XSlice xs[PASSES];
+    // round trip 1: the first chunk, the activations, the codebook
+    WaveStage<NP> st;
+    if (c < n_full) st.fetch(W + (size_t)c * CB, NPC, lane);
+    uint32_t grid_word = 0;
+    if constexpr (TYPE == QKK_IQ3_XXS) grid_word = g_iq3xxs_grid[threadIdx.x];
+    XSlice xs[HALF ? 1 : PASSES];
+    XSliceH xh[HALF ? PASSES : 1];
     float xsum[PASSES][4];
 #pragma unroll
     for (int p = 0; p < PASSES; p++) {
-        load_xslice<TYPE>(xs[p], x + p * 32 * LPR, lir);
+        XSlice f;
+        load_xslice<TYPE>(f, x + p * 32 * LPR, lir);
+        if constexpr (TYPE == QKK_IQ4_XS) split_xslice_iq4(xh[p], f);
+        else if constexpr (HALF) split_xslice(xh[p], f);
+        else {
+            xs[p] = f;
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            float s = 0.f;
+            for (int q = 0; q < 4; q++) {
+                float t = 0.f;
 #pragma unroll
-            for (int i = 0; i < 8; i++) s += xs[p].v[c * 8 + i];
-            xsum[p][c] = s;
+                for (int i = 0; i < 8; i++) t += f.v[q * 8 + i];
+                xsum[p][q] = t;
+            }
         }
     }
-    const uint32_t pass_bytes = row_bytes / PASSES;
+    if constexpr (TYPE == QKK_IQ3_XXS) fill_iq3_half_entry(tab3, threadIdx.x, grid_word);
+    if constexpr (TYPE == QKK_IQ4_XS) fill_iq4_pair_entry(tab4, threadIdx.x);
+    if constexpr (HALF) __syncthreads();
 
-    // chunks of GROUPS*RIF rows are dealt round-robin to the waves of the (persistent) grid;
-    // the loads of a wave's next chunk are issued before the arithmetic of the current one
-    // (two register sets, loop unrolled by two, no branch around the loads: chunks past the
-    // end re-read the last row and their results are dropped)
-    constexpr uint32_t CHUNK = GROUPS * RIF;
-    const uint32_t stride = gridDim.x * 4 * CHUNK;
-    LaneW<TYPE> w[DEEP ? 2 : 1][RIF][PASSES];
-    auto fetch = [&](int set, uint32_t r0) {
+    auto dot_row = [&](const LaneW<TYPE> (&w)[PASSES]) {
+        float acc = 0.f;
 #pragma unroll
-        for (int i = 0; i < RIF; i++) {
-            const uint32_t r = min(r0 + i * GROUPS + grp, M - 1);
-#pragma unroll
-            for (int p = 0; p < PASSES; p++)
-                w[set][i][p].load(W + (size_t)r * row_bytes + (size_t)p * pass_bytes, lir);
+        for (int p = 0; p < PASSES; p++) {
+            if constexpr (TYPE == QKK_IQ3_XXS) acc += w[p].dot_h(xh[p], &tab3);
+            else if constexpr (TYPE == QKK_IQ4_XS) acc += w[p].dot_h(xh[p], &tab4, lir);
+            else acc += w[p].dot(xs[p], xsum[p], &tab, lir);
         }
+        return lanes_sum<LPR>(acc);
     };
-    auto reduce = [&](int set, uint32_t r0) {
+
+    uint8_t* area = s_stage[wave];
+    vmem_drain(); // the activations have arrived: no wait for them inside the loop, behind the next chunk's loads
+    for (; c < n_full; c += stride) {
+        st.commit(area, lane);
+        const uint32_t cn = c + stride;
+        if (cn < n_full) st.fetch(W + (size_t)cn * CB, NPC, lane);
 #pragma unroll
-        for (int i = 0; i < RIF; i++) {
-            float acc = 0.f;
+        for (int r = 0; r < RPC; r++) {
+            const uint32_t in_chunk = r * GROUPS + grp;
+            LaneW<TYPE> w[PASSES];
 #pragma unroll
-            for (int p = 0; p < PASSES; p++) acc += w[set][i][p].dot(xs[p], xsum[p], &tab, lir);
-            acc = lanes_sum<LPR>(acc);
-            const uint32_t r = r0 + i * GROUPS + grp;
-            if (lir == 0 && r < M) y[r] = acc;
+            for (int p = 0; p < PASSES; p++) lane_load_lds<TYPE>(w[p], area, in_chunk * RB + p * PB, lir);
+            const float acc = dot_row(w);
+            if (lir == 0) y[c * CH + in_chunk] = acc;
         }
-    };
-    uint32_t r0 = (blockIdx.x * 4 + wave) * CHUNK;
-    if constexpr (TABLES || DEEP) fetch(0, r0); // rows past the end re-read the last row
-    if constexpr (TABLES) {
-        tab.grid[threadIdx.x] = grid_word;
-        if (threadIdx.x < 16) {
-            constexpr int8_t kv[16] = {QK_IQ4NL_VALUES};
-            float v = 0.f;
-#pragma unroll
-            for (int i = 0; i < 16; i++) v = (int)threadIdx.x == i ? (float)kv[i] : v;
-            tab.iq4[threadIdx.x] = v;
-        }
-        __syncthreads();
     }
-    if constexpr (DEEP) {
-        for (; r0 < M; r0 += 2 * stride) {
-            fetch(1, r0 + stride);
-            reduce(0, r0);
-            fetch(0, r0 + 2 * stride);
-            reduce(1, r0 + stride);
-        }
-    } else if constexpr (TABLES) { // the first chunk is already on its way
-        while (r0 < M) {
-            reduce(0, r0);
-            r0 += stride;
-            if (r0 < M) fetch(0, r0); // wave-uniform
-        }
-    } else {
-        for (; r0 < M; r0 += stride) {
-            fetch(0, r0);
-            reduce(0, r0);
-        }
+    // the rows behind the last full chunk, 64/LPR at a time, each lane fetching its own fields
+    const uint32_t tail0 = n_full * CH, tail_groups = (M - tail0 + GROUPS - 1) / GROUPS;
+    for (uint32_t t = blockIdx.x * 4 + wave; t < tail_groups; t += stride) {
+        const uint32_t row = tail0 + t * GROUPS + grp;
+        const uint8_t* rp = W + (size_t)min(row, M - 1) * RB; // lanes past the end re-read the last row
+        LaneW<TYPE> w[PASSES];
+#pragma unroll
+        for (int p = 0; p < PASSES; p++) w[p].load(rp + (size_t)p * PB, lir);
+        const float acc = dot_row(w);
+        if (lir == 0 && row < M) y[row] = acc;
     }
 }
 
@@ -338,19 +351,21 @@ __global__ __launch_bounds__(256) void gemv_dense_kernel(const T* __restrict__ W
 
 // ---- launchers ----------------------------------------------------------------------------
 
-template <int TYPE, int LPR, int PASSES, int RIF>
-static void launch_q(const void* W, const float* X, float* Y, uint32_t M, uint32_t K, uint32_t batch,
-                     uint32_t row_bytes, hipStream_t st)
+template <int TYPE, int LPR, int PASSES>
+static void launch_q(const void* W, const float* X, float* Y, uint32_t M, uint32_t batch, hipStream_t st)
 {
-    constexpr uint32_t CHUNK = WAVE / LPR * RIF;
-    const uint32_t waves = (M + CHUNK - 1) / CHUNK;
-    const dim3 grid(std::min((waves + 3) / 4, persistent_blocks()), batch);
-    if (waves > 4 * grid.x * 4) // at least four chunks per wave: worth the second register set
-        hipLaunchKernelGGL((gemv_q_kernel<TYPE, LPR, PASSES, RIF, true>), grid, dim3(256), 0, st,
-                           (const uint8_t*)W, X, Y, M, K, row_bytes);
-    else
-        hipLaunchKernelGGL((gemv_q_kernel<TYPE, LPR, PASSES, RIF, false>), grid, dim3(256), 0, st,
-                           (const uint8_t*)W, X, Y, M, K, row_bytes);
+    constexpr int RPC = GemvShape<TYPE>::RPC2048 / PASSES > 0 ? GemvShape<TYPE>::RPC2048 / PASSES : 1;
+    constexpr uint32_t CH = RPC * (WAVE / LPR);
+    constexpr uint32_t RB = (uint32_t)qkk_row_bytes_dev<TYPE>(32u * LPR * PASSES);
+    constexpr uint32_t NP = (CH * RB / 16 + 63) / 64;
+    // workgroups a CU holds (LDS: the four waves' areas + tables; 160 KB per CU) and the depth of the persistent grid
+    constexpr uint32_t WG_LDS = 4 * (NP * 1024 + 16) + 4096, RESIDENT = std::min<uint32_t>(8, 160 * 1024 / WG_LDS);
+    constexpr uint32_t DEPTH = TYPE == QKK_Q8_0 ? std::min<uint32_t>(4, RESIDENT) : RESIDENT;
+    const uint32_t cus = persistent_blocks() / 4;
+    const uint32_t chunks = M / CH, tail_groups = (M - chunks * CH + WAVE / LPR - 1) / (WAVE / LPR);
+    const uint32_t want = (std::max(chunks, tail_groups) + 3) / 4; // one chunk per wave
+    const uint32_t blocks = std::max(1u, want <= cus * RESIDENT ? want : cus * DEPTH);
+    hipLaunchKernelGGL((gemv_stream_kernel<TYPE, LPR, PASSES, RPC>), dim3(blocks, batch), dim3(256), 0, st, (const uint8_t*)W, X, Y, M);
 }
 
 template <int TYPE>
@@ -358,25 +373,13 @@ static int dispatch_q(const void* W, const float* X, float* Y, uint32_t M, uint3
                       hipStream_t st)
 {
     const uint32_t rb = (uint32_t)qkk_row_bytes(TYPE, K);
-    constexpr uint32_t MINK = TYPE == QKK_Q8_0 ? 32 : 256;
-    // rows per wave: four where the matrix has rows enough to give every CU several waves that way,
-    // fewer for short matrices (512 rows: 3.1-3.4 us with one row per wave against 4.6-5.2 us with four)
-    // a layer's input projections as one matrix (12288 = qkv + gate, 9216 = q + k + v rows): M / 1024 rows
-    // per wave make 256 workgroups, one per CU, where eight leave half the CUs with a second one
-    if (K == 2048 && M == 12288 && TYPE == QKK_Q8_0) launch_q<TYPE, 64, 1, 12>(W, X, Y, M, K, batch, rb, st);
-    else if (K == 2048 && M == 9216 && TYPE == QKK_Q8_0) launch_q<TYPE, 64, 1, 9>(W, X, Y, M, K, batch, rb, st);
-    else if (K == 2048 && M >= 8192 && TYPE == QKK_Q8_0) launch_q<TYPE, 64, 1, 8>(W, X, Y, M, K, batch, rb, st); // 7.5 -> 6.9 us
-    else if (K == 2048 && M >= 2048) launch_q<TYPE, 64, 1, 4>(W, X, Y, M, K, batch, rb, st);
-    else if (K == 2048 && M >= 1024) launch_q<TYPE, 64, 1, 2>(W, X, Y, M, K, batch, rb, st);
-    else if (K == 2048) launch_q<TYPE, 64, 1, 1>(W, X, Y, M, K, batch, rb, st);
-    else if (K == 4096 && M >= 1024) launch_q<TYPE, 64, 2, 2>(W, X, Y, M, K, batch, rb, st);
-    else if (K == 4096) launch_q<TYPE, 64, 2, 1>(W, X, Y, M, K, batch, rb, st);
-    else if (K == 8192) launch_q<TYPE, 64, 4, 1>(W, X, Y, M, K, batch, rb, st);
-    else if (K == 1024) launch_q<TYPE, 32, 1, 4>(W, X, Y, M, K, batch, rb, st);
-    else if (K == 512) launch_q<TYPE, 16, 1, 4>(W, X, Y, M, K, batch, rb, st);
-    else if (K == 256) launch_q<TYPE, 8, 1, 4>(W, X, Y, M, K, batch, rb, st);
+    if (K == 2048) launch_q<TYPE, 64, 1>(W, X, Y, M, batch, st);
+    else if (K == 4096) launch_q<TYPE, 64, 2>(W, X, Y, M, batch, st);
+    else if (K == 8192) launch_q<TYPE, 64, 4>(W, X, Y, M, batch, st);
+    else if (K == 1024) launch_q<TYPE, 32, 1>(W, X, Y, M, batch, st);
+    else if (K == 512) launch_q<TYPE, 16, 1>(W, X, Y, M, batch, st);
+    else if (K == 256) launch_q<TYPE, 8, 1>(W, X, Y, M, batch, st);
     else {
-        (void)MINK;
         const uint32_t blocks = (uint32_t)std::min<uint64_t>(((uint64_t)M + 3) / 4, 4096);
         hipLaunchKernelGGL((gemv_q_generic_kernel<TYPE>), dim3(blocks, batch), dim3(256), 0, st,
                            (const uint8_t*)W, X, Y, M, K, rb);

@@ -195,7 +195,7 @@ __global__ __launch_bounds__(CT) void head_q6k_coop_kernel(const uint8_t* __rest
 {
     constexpr uint32_t K = 2048, ROW = HeadGeo::RB, BT = HeadGeo::BT;
     static_assert(BT * 256 <= CT, "one output per thread and batch");
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    QK_DYN_LDS(uint8_t, smem);
     __shared__ MfmaTables tab;
     __shared__ uint32_t s_last;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;

@@ -6,86 +6,28 @@
 //               IQ3_XXS gate and up rows of the picks, SiLU gating -> h; writes the router record.
 //   3. down:    routed down rows (IQ4_XS or Q6_K) weighted by the router, shared down row
 //               (Q8_0) weighted by the sigmoid gate, summed into y.
-// On this device a dependent memory access costs 2-3 us when the line is cold (each step
-// touches a different layer's weights) while a kernel boundary costs well under 1 us, so each
-// launch is arranged as two round trips at most and nothing synchronises inside a kernel.
-// (A single-launch form with device-wide barriers was measured at ~5 us per barrier and
-// dropped.)  Several rows go through the expert-major path in qk_moe_grouped.hip.
+// Inside a HIP graph a launch costs about 1.7 us whatever it does and a cold read of a few MB adds
+// about 1 us, while a device-wide barrier inside a kernel measured 5 us: so the step is three
+// launches, each arranged as at most two dependent round trips to memory.  Block rows are streamed
+// as 16-byte pieces through a wave-private LDS area (qk_stream.h): with per-lane loads of the
+// misaligned block fields the address unit of the CU, not memory, set the pace (the picked experts'
+// 6.4 MB took 4.5 us to arrive).  Several rows go through the expert-major path in
+// qk_moe_grouped.hip.
 #include "qk_moe_common.h"
+#include "qk_stream.h"
 
 #include <mutex>
 
 namespace qk {
 
-// ---- launch 1: router logits + shared gate/up ---------------------------------------------
-// One wave per task, no loop: tasks [0, E] are F32 rows (row E = the shared gate row), tasks
-// after that are shared-expert gate/up row pairs.  Every load of a task is issued before its
-// arithmetic, so a task costs one memory round trip.  H = 256*NCH.
-// ROWS: blockIdx.y is the activation row (slot); every row runs the one-row launch on its own part
-// of x and of the workspace -- for a few rows, which hardly ever pick the same expert, this beats
-// the expert-major path, and a row's result does not depend on its company.
-template <int NCH, bool ROWS>
-__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ gate_inp,
-                                                        const float* __restrict__ gate_inp_shexp,
-                                                        const uint8_t* __restrict__ gate_shexp,
-                                                        const uint8_t* __restrict__ up_shexp,
-                                                        const float* __restrict__ x, MoeWs ws, MoeDims d)
-{
-    if constexpr (ROWS) {
-        x += (size_t)blockIdx.y * d.H;
-        ws.logits += (size_t)blockIdx.y * lstride(d.E);
-        ws.h += (size_t)blockIdx.y * (d.k + 1) * d.F;
-    }
-    constexpr int P = NCH / 8; // 2048-weight passes per Q8_0 row
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t n_dense = d.E + 1, n_tasks = n_dense + d.F;
-    const uint32_t q8_row = d.H / 32 * Q8_0_BYTES;
-    const uint32_t t = blockIdx.x * 4 + wave;
+template <bool ON>
+struct NormArg {
+    const float* w; // RMS-norm weights of the row
+    float eps;
+};
+template <>
+struct NormArg<false> {};
 
-    if (t < n_dense) {
-        const float4* row = (const float4*)(t < d.E ? gate_inp + (size_t)t * d.H : gate_inp_shexp);
-        const float4* xv = (const float4*)x;
-        float4 w[NCH], xx[NCH];
-#pragma unroll
-        for (int i = 0; i < NCH; i++) w[i] = row[lane + 64 * i];
-#pragma unroll
-        for (int i = 0; i < NCH; i++) xx[i] = xv[lane + 64 * i];
-        float a0 = 0.f, a1 = 0.f;
-#pragma unroll
-        for (int i = 0; i < NCH; i++) {
-            a0 += w[i].x * xx[i].x + w[i].y * xx[i].y;
-            a1 += w[i].z * xx[i].z + w[i].w * xx[i].w;
-        }
-        const float s = wave_sum(a0 + a1);
-        if (lane == 0) ws.logits[t] = s;
-    } else if (t < n_tasks) {
-        const uint32_t r = t - n_dense;
-        LaneW<QKK_Q8_0> wg[P], wu[P];
-        XSlice xs[P];
-#pragma unroll
-        for (int p = 0; p < P; p++) {
-            wg[p].load(gate_shexp + (size_t)r * q8_row + (size_t)p * 64 * Q8_0_BYTES, lane);
-            wu[p].load(up_shexp + (size_t)r * q8_row + (size_t)p * 64 * Q8_0_BYTES, lane);
-        }
-#pragma unroll
-        for (int p = 0; p < P; p++) load_xslice<QKK_Q8_0>(xs[p], x + p * 2048, lane);
-        float g = 0.f, u = 0.f;
-#pragma unroll
-        for (int p = 0; p < P; p++) {
-            g += wg[p].dot(xs[p], nullptr, nullptr, lane);
-            u += wu[p].dot(xs[p], nullptr, nullptr, lane);
-        }
-        g = wave_sum(g);
-        u = wave_sum(u);
-        if (lane == 0) ws.h[(size_t)d.k * d.F + r] = (g / (1.f + expf(-g))) * u;
-    }
-}
-
-// The same launch with the RMS norm in front: x is the un-normalised residual row; the workgroup
-// forms x * nw once, in LDS, and sums the squares (a wave that fetched x and nw for itself made the
-// launch 1.7 us longer: three 8 KB rows per wave through the L1 instead of two); the dot products
-// run on x * nw and their sums are scaled by 1/sqrt(mean(x^2) + eps), which is common to a row's
-// terms.  The task's weights are requested first, so they are in flight while x arrives.
 // ADD: the row is x + mix (a mixer's output on top of the residual); the first workgroup of the row
 // also stores the sum to `sum`, a buffer of its own, for the launches behind this one.
 template <bool ON>
@@ -96,72 +38,121 @@ struct AddArg {
 template <>
 struct AddArg<false> {};
 
-template <int NCH, bool ROWS, bool ADD = false>
-__global__ __launch_bounds__(256) void moe_route_norm_kernel(const float* __restrict__ gate_inp,
+// Sum over a workgroup of NW waves in wave order; every thread returns the same bits.
+template <int NW>
+__device__ __forceinline__ float block_sum_waves(float v, float* s_red)
+{
+    const float w = wave_sum(v);
+    if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = w;
+    __syncthreads();
+    float t = s_red[0];
+#pragma unroll
+    for (int i = 1; i < NW; i++) t += s_red[i];
+    return t;
+}
+
+// The workgroup (NT threads) forms x * nw once, in LDS, and returns 1/sqrt(mean(x^2) + eps): a dot
+// product against the normalised row is that factor times the dot product against x * nw, so the
+// callers run on x * nw and scale their sums.  (A wave that fetched x and nw for itself made the
+// launch 1.7 us longer: three 8 KB rows per wave through the L1 instead of two.)  ADD as above.
+// The barrier inside the block sum also publishes s_x.
+template <int NT, int NQ /* float4s of the row */, bool ADD>
+__device__ __forceinline__ float stage_normed_row(const float* __restrict__ x, const float* __restrict__ nw, float eps,
+                                                  float* s_x, float* s_red, const AddArg<ADD>& aa, bool store_sum)
+{
+    constexpr int NV = (NQ + NT - 1) / NT;
+    float4 xv[NV], nv[NV];
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const uint32_t q = min(threadIdx.x + NT * i, (uint32_t)NQ - 1);
+        xv[i] = ((const float4*)x)[q];
+        nv[i] = ((const float4*)nw)[q];
+    }
+    if constexpr (ADD) {
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const uint32_t q = min(threadIdx.x + NT * i, (uint32_t)NQ - 1);
+            const float4 m = ((const float4*)aa.mix)[q];
+            xv[i] = float4{xv[i].x + m.x, xv[i].y + m.y, xv[i].z + m.z, xv[i].w + m.w};
+            if (store_sum && threadIdx.x + NT * i < NQ) ((float4*)aa.sum)[q] = xv[i];
+        }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        if (threadIdx.x + NT * i < NQ) {
+            ss += (xv[i].x * xv[i].x + xv[i].y * xv[i].y) + (xv[i].z * xv[i].z + xv[i].w * xv[i].w);
+            ((float4*)s_x)[threadIdx.x + NT * i] =
+                float4{xv[i].x * nv[i].x, xv[i].y * nv[i].y, xv[i].z * nv[i].z, xv[i].w * nv[i].w};
+        }
+    }
+    return 1.f / sqrtf(block_sum_waves<NT / 64>(ss, s_red) / (float)(4 * NQ) + eps);
+}
+
+// ---- launch 1: router logits + shared gate/up ---------------------------------------------
+// One wave per task, no loop: tasks [0, E] are F32 rows (row E = the shared gate row), tasks after
+// that are shared-expert gate/up row pairs (Q8_0, both rows staged through LDS).  Every load of a
+// task is issued before its arithmetic, so a task costs one memory round trip.  Three waves per
+// workgroup: E + 1 + F = 769 tasks make 257 workgroups, three tasks on every CU (four waves per
+// workgroup made 193 and left a quarter of the CUs idle).  H = 256*NCH.
+// ROWS: blockIdx.y is the activation row (slot); every row runs the one-row launch on its own part
+// of x and of the workspace -- for a few rows, which hardly ever pick the same expert, this beats
+// the expert-major path, and a row's result does not depend on its company.
+// MODE 0: x is the (normalised) activation row.  MODE 1: x is the un-normalised residual row, the
+// RMS norm with weights na.w runs in front (stage_normed_row).  MODE 2: the row is x + mix.
+constexpr int ROUTE_WAVES = 3;
+
+template <int NCH, bool ROWS, int MODE>
+__global__ __launch_bounds__(64 * ROUTE_WAVES) void moe_route_kernel(const float* __restrict__ gate_inp,
                                                         const float* __restrict__ gate_inp_shexp,
                                                         const uint8_t* __restrict__ gate_shexp,
                                                         const uint8_t* __restrict__ up_shexp,
                                                         const float* __restrict__ x, MoeWs ws, MoeDims d,
-                                                        const float* __restrict__ nw, float eps, AddArg<ADD> aa)
+                                                        NormArg<MODE != 0> na, AddArg<MODE == 2> aa)
 {
-    if constexpr (ROWS && ADD) {
-        aa.mix += (size_t)blockIdx.y * d.H;
-        aa.sum += (size_t)blockIdx.y * d.H;
+    if constexpr (MODE == 2) {
+        if constexpr (ROWS) {
+            aa.mix += (size_t)blockIdx.y * d.H;
+            aa.sum += (size_t)blockIdx.y * d.H;
+        }
     }
     if constexpr (ROWS) {
         x += (size_t)blockIdx.y * d.H;
         ws.logits += (size_t)blockIdx.y * lstride(d.E);
         ws.h += (size_t)blockIdx.y * (d.k + 1) * d.F;
     }
-    constexpr int P = NCH / 8; // 2048-weight passes per Q8_0 row
+    constexpr int P = NCH / 8;                          // 2048-weight passes per Q8_0 row
+    constexpr uint32_t Q8ROW = 64 * P * Q8_0_BYTES;     // bytes of one shared-expert row
+    constexpr uint32_t NPIECE = 2 * Q8ROW / 16;         // the gate row, then the up row
+    constexpr int NP = (NPIECE + 63) / 64;
+    __shared__ __attribute__((aligned(16))) uint8_t s_stage[ROUTE_WAVES][WaveStage<NP>::AREA + 16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t n_dense = d.E + 1, n_tasks = n_dense + d.F;
-    const uint32_t q8_row = d.H / 32 * Q8_0_BYTES;
-    const uint32_t t = blockIdx.x * 4 + wave;
+    const uint32_t t = blockIdx.x * ROUTE_WAVES + wave;
 
     // the task's weights first: they are in flight while x arrives
     const bool dense = t < n_dense, shared = !dense && t < n_tasks;
     float4 w[NCH];
-    LaneW<QKK_Q8_0> wg[P], wu[P];
+    WaveStage<NP> st;
     if (dense) {
         const float4* row = (const float4*)(t < d.E ? gate_inp + (size_t)t * d.H : gate_inp_shexp);
 #pragma unroll
         for (int i = 0; i < NCH; i++) w[i] = row[lane + 64 * i];
     } else if (shared) {
-        const uint32_t r = t - n_dense;
-#pragma unroll
-        for (int p = 0; p < P; p++) {
-            wg[p].load(gate_shexp + (size_t)r * q8_row + (size_t)p * 64 * Q8_0_BYTES, lane);
-            wu[p].load(up_shexp + (size_t)r * q8_row + (size_t)p * 64 * Q8_0_BYTES, lane);
-        }
+        const uint8_t* g = gate_shexp + (size_t)(t - n_dense) * Q8ROW;
+        const uint8_t* u = up_shexp + (size_t)(t - n_dense) * Q8ROW;
+        st.fetch_at([&](uint32_t i) {
+            const uint32_t c = min(i, NPIECE - 1);
+            return c < NPIECE / 2 ? g + 16 * c : u + 16 * (c - NPIECE / 2);
+        }, lane);
     }
 
-    __shared__ __attribute__((aligned(16))) float s_x[256 * NCH];
-    __shared__ float s_red[4];
     float scale = 1.f;
     const float* xrow = x;
-    {
-        float4 xv[NCH / 4], nv[NCH / 4];
-#pragma unroll
-        for (int i = 0; i < NCH / 4; i++) xv[i] = ((const float4*)x)[threadIdx.x + 256 * i];
-#pragma unroll
-        for (int i = 0; i < NCH / 4; i++) nv[i] = ((const float4*)nw)[threadIdx.x + 256 * i];
-        if constexpr (ADD) {
-#pragma unroll
-            for (int i = 0; i < NCH / 4; i++) {
-                const float4 m = ((const float4*)aa.mix)[threadIdx.x + 256 * i];
-                xv[i] = float4{xv[i].x + m.x, xv[i].y + m.y, xv[i].z + m.z, xv[i].w + m.w};
-                if (blockIdx.x == 0) ((float4*)aa.sum)[threadIdx.x + 256 * i] = xv[i];
-            }
-        }
-        float ss = 0.f;
-#pragma unroll
-        for (int i = 0; i < NCH / 4; i++) {
-            ss += (xv[i].x * xv[i].x + xv[i].y * xv[i].y) + (xv[i].z * xv[i].z + xv[i].w * xv[i].w);
-            ((float4*)s_x)[threadIdx.x + 256 * i] =
-                float4{xv[i].x * nv[i].x, xv[i].y * nv[i].y, xv[i].z * nv[i].z, xv[i].w * nv[i].w};
-        }
-        scale = 1.f / sqrtf(block_sum4(ss, s_red) / (float)d.H + eps); // its barrier also publishes s_x
+    if constexpr (MODE != 0) {
+        __shared__ __attribute__((aligned(16))) float s_x[256 * NCH];
+        __shared__ float s_red[ROUTE_WAVES];
+        scale = stage_normed_row<64 * ROUTE_WAVES, 64 * NCH, MODE == 2>(x, na.w, na.eps, s_x, s_red, aa, blockIdx.x == 0);
         xrow = s_x;
     }
 
@@ -179,37 +170,40 @@ __global__ __launch_bounds__(256) void moe_route_norm_kernel(const float* __rest
         const float s = wave_sum(a0 + a1) * scale;
         if (lane == 0) ws.logits[t] = s;
     } else if (shared) {
-        const uint32_t r = t - n_dense;
         XSlice xs[P];
 #pragma unroll
         for (int p = 0; p < P; p++) load_xslice<QKK_Q8_0>(xs[p], xrow + p * 2048, lane);
+        uint8_t* area = s_stage[wave];
+        st.commit(area, lane);
         float g = 0.f, u = 0.f;
 #pragma unroll
         for (int p = 0; p < P; p++) {
-            g += wg[p].dot(xs[p], nullptr, nullptr, lane);
-            u += wu[p].dot(xs[p], nullptr, nullptr, lane);
+            LaneW<QKK_Q8_0> wg, wu;
+            lane_load_lds<QKK_Q8_0>(wg, area, p * 64 * Q8_0_BYTES, lane);
+            lane_load_lds<QKK_Q8_0>(wu, area, Q8ROW + p * 64 * Q8_0_BYTES, lane);
+            g += wg.dot(xs[p], nullptr, nullptr, lane);
+            u += wu.dot(xs[p], nullptr, nullptr, lane);
         }
         g = wave_sum(g) * scale;
         u = wave_sum(u) * scale;
-        if (lane == 0) ws.h[(size_t)d.k * d.F + r] = (g / (1.f + expf(-g))) * u;
+        if (lane == 0) ws.h[(size_t)d.k * d.F + (t - n_dense)] = (g / (1.f + expf(-g))) * u;
     }
 }
 
 // ---- launch 2: select + routed gate/up + SiLU --------------------------------------------
-// Every workgroup picks the top-n_used experts itself from the E logits of launch 1 (one wave,
-// ~1.7 us) instead of waiting for a selector launch: the logits, the activation slice and the
-// codebook are fetched in one round trip, the picked rows in a second.  Workgroup 0 also
-// writes the router record.  Wave task = (pick s, RIF consecutive FFN rows); gate and up rows
-// of one FFN row are fetched together.  IQ3_XXS rows of H = 2048*PASSES weights.  A workgroup's
-// time line, measured with the device clock: round trip 1 about 1.5 us, selection 1.7 us, second
-// round trip and first row 1.9 us, the other rows 2.6 us (arrival of the picked experts' 6.4 MB,
-// not arithmetic: the product on packed halves -- two LDS lookups and two XORs per four weights,
-// v_dot2_f32_f16 against the activations split into hi + lo halves -- cut the launch by 0.2 us).
-template <int TYPE, int PASSES, int RIF, bool ROWS>
+// Every workgroup picks the top-n_used experts itself from the E logits of launch 1 (one wave)
+// instead of waiting for a selector launch: the logits, the activation slice and the codebook are
+// fetched in one round trip, the picked rows in a second.  Workgroup 0 also writes the router
+// record.  Wave task = (pick s, RPW consecutive FFN rows): the gate rows are one contiguous range of
+// the expert, the up rows another; both are requested as 16-byte pieces right after the selection
+// and go through the wave's LDS area one after the other.  IQ3_XXS rows of H = 2048*PASSES weights;
+// the product runs on packed halves (two LDS lookups and two XORs per four weights, v_dot2_f32_f16
+// against the activations split into hi + lo halves).  NORM: the RMS norm in front, as in launch 1.
+template <int PASSES, int RPW, bool ROWS, bool NORM>
 __global__ __launch_bounds__(256) void moe_gateup_kernel(const uint8_t* __restrict__ gate_exps,
                                                          const uint8_t* __restrict__ up_exps,
                                                          const float* __restrict__ x, MoeWs ws,
-                                                         qkk_sel* __restrict__ sel, MoeDims d)
+                                                         qkk_sel* __restrict__ sel, MoeDims d, NormArg<NORM> na)
 {
     if constexpr (ROWS) { // blockIdx.y = activation row, as in launch 1
         x += (size_t)blockIdx.y * d.H;
@@ -217,12 +211,15 @@ __global__ __launch_bounds__(256) void moe_gateup_kernel(const uint8_t* __restri
         ws.h += (size_t)blockIdx.y * (d.k + 1) * d.F;
         sel += blockIdx.y;
     }
+    constexpr uint32_t RB = 8 * PASSES * IQ3_XXS_BYTES; // bytes of a row
+    constexpr uint32_t NPIECE = RPW * RB / 16;
+    constexpr int NP = (NPIECE + 63) / 64;
+    static_assert((RPW * RB) % 16 == 0, "a wave's rows must be whole 16-byte pieces");
     __shared__ Iq3HalfTables tab;
     __shared__ float s_log[QKK_MAX_EXPERTS + 8];
     __shared__ qkk_sel s_sel;
+    __shared__ __attribute__((aligned(16))) uint8_t s_stage[4][WaveStage<NP>::AREA + 16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t row_bytes = (uint32_t)qkk_row_bytes_dev<TYPE>(d.H);
-    const uint32_t pass_bytes = row_bytes / PASSES;
 
     // round trip 1: codebook word, logits (wave 0), activation slice
     const uint32_t grid_word = g_iq3xxs_grid[threadIdx.x];
@@ -233,119 +230,24 @@ __global__ __launch_bounds__(256) void moe_gateup_kernel(const uint8_t* __restri
             lv[i] = (uint32_t)(lane + 64 * i) <= d.E ? ws.logits[lane + 64 * i] : 0.f;
     }
     XSliceH xs[PASSES];
-#pragma unroll
-    for (int p = 0; p < PASSES; p++) {
-        XSlice f;
-        load_xslice<TYPE>(f, x + p * 2048, lane);
-        split_xslice(xs[p], f);
-    }
-
-    fill_iq3_half_entry(tab, threadIdx.x, grid_word);
-    if (wave == 0) {
-#pragma unroll
-        for (int i = 0; i <= (int)(QKK_MAX_EXPERTS / 64); i++)
-            if ((uint32_t)(lane + 64 * i) <= d.E) s_log[lane + 64 * i] = lv[i];
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        select_wave(s_log, d.E, d.k, &s_sel);
-        if (lane == 0) s_sel.w_shared = 1.f / (1.f + expf(-s_log[d.E]));
-    }
-    __syncthreads();
-    if (blockIdx.x == 0 && threadIdx.x < 33) {
-        if (threadIdx.x < 16) {
-            if (threadIdx.x < d.k) {
-                sel->ids[threadIdx.x] = s_sel.ids[threadIdx.x];
-                sel->w[threadIdx.x] = s_sel.w[threadIdx.x];
-            }
-        } else if (threadIdx.x == 32) {
-            sel->w_shared = s_sel.w_shared;
-        }
-    }
-
-    const uint32_t groups = (d.F + RIF - 1) / RIF; // row groups per pick
-    for (uint32_t t = blockIdx.x * 4 + wave; t < d.k * groups; t += gridDim.x * 4) {
-        const uint32_t s = t / groups, r0 = (t % groups) * RIF;
-        const uint32_t e = min(s_sel.ids[s], d.E - 1);
-        const uint8_t* gbase = gate_exps + ((size_t)e * d.F) * row_bytes;
-        const uint8_t* ubase = up_exps + ((size_t)e * d.F) * row_bytes;
-        LaneW<TYPE> wg[RIF][PASSES], wu[RIF][PASSES];
-#pragma unroll
-        for (int i = 0; i < RIF; i++) {
-            const uint32_t r = min(r0 + i, d.F - 1);
-#pragma unroll
-            for (int p = 0; p < PASSES; p++) {
-                wg[i][p].load(gbase + (size_t)r * row_bytes + (size_t)p * pass_bytes, lane);
-                wu[i][p].load(ubase + (size_t)r * row_bytes + (size_t)p * pass_bytes, lane);
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < RIF; i++) {
-            float g = 0.f, u = 0.f;
-#pragma unroll
-            for (int p = 0; p < PASSES; p++) {
-                g += wg[i][p].dot_h(xs[p], &tab);
-                u += wu[i][p].dot_h(xs[p], &tab);
-            }
-            g = wave_sum(g);
-            u = wave_sum(u);
-            if (lane == 0 && r0 + i < d.F) ws.h[(size_t)s * d.F + r0 + i] = (g / (1.f + expf(-g))) * u;
-        }
-    }
-}
-
-// Launch 2 with the RMS norm in front, as moe_route_norm_kernel: x * nw through LDS, sums scaled.
-template <int TYPE, int PASSES, int RIF, bool ROWS>
-__global__ __launch_bounds__(256) void moe_gateup_norm_kernel(const uint8_t* __restrict__ gate_exps,
-                                                         const uint8_t* __restrict__ up_exps,
-                                                         const float* __restrict__ x, MoeWs ws,
-                                                         qkk_sel* __restrict__ sel, MoeDims d,
-                                                         const float* __restrict__ nw, float eps)
-{
-    if constexpr (ROWS) {
-        x += (size_t)blockIdx.y * d.H;
-        ws.logits += (size_t)blockIdx.y * lstride(d.E);
-        ws.h += (size_t)blockIdx.y * (d.k + 1) * d.F;
-        sel += blockIdx.y;
-    }
-    __shared__ Iq3HalfTables tab;
-    __shared__ float s_log[QKK_MAX_EXPERTS + 8];
-    __shared__ qkk_sel s_sel;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t row_bytes = (uint32_t)qkk_row_bytes_dev<TYPE>(d.H);
-    const uint32_t pass_bytes = row_bytes / PASSES;
-
-    // round trip 1: codebook word, logits (wave 0), activation slice
-    const uint32_t grid_word = g_iq3xxs_grid[threadIdx.x];
-    float lv[QKK_MAX_EXPERTS / 64 + 1];
-    if (wave == 0) {
-#pragma unroll
-        for (int i = 0; i <= (int)(QKK_MAX_EXPERTS / 64); i++)
-            lv[i] = (uint32_t)(lane + 64 * i) <= d.E ? ws.logits[lane + 64 * i] : 0.f;
-    }
-    XSliceH xs[PASSES];
-    __shared__ __attribute__((aligned(16))) float s_x[2048 * PASSES];
-    __shared__ float s_red[4];
     float scale = 1.f;
-    { // the workgroup forms x * nw once, in LDS, and sums the squares
-        float4 xv[2 * PASSES], nv[2 * PASSES];
+    if constexpr (NORM) {
+        __shared__ __attribute__((aligned(16))) float s_x[2048 * PASSES];
+        __shared__ float s_red[4];
+        scale = stage_normed_row<256, 512 * PASSES, false>(x, na.w, na.eps, s_x, s_red, AddArg<false>{}, false);
 #pragma unroll
-        for (int i = 0; i < 2 * PASSES; i++) xv[i] = ((const float4*)x)[threadIdx.x + 256 * i];
-#pragma unroll
-        for (int i = 0; i < 2 * PASSES; i++) nv[i] = ((const float4*)nw)[threadIdx.x + 256 * i];
-        float ss = 0.f;
-#pragma unroll
-        for (int i = 0; i < 2 * PASSES; i++) {
-            ss += (xv[i].x * xv[i].x + xv[i].y * xv[i].y) + (xv[i].z * xv[i].z + xv[i].w * xv[i].w);
-            ((float4*)s_x)[threadIdx.x + 256 * i] =
-                float4{xv[i].x * nv[i].x, xv[i].y * nv[i].y, xv[i].z * nv[i].z, xv[i].w * nv[i].w};
+        for (int p = 0; p < PASSES; p++) {
+            XSlice f;
+            load_xslice<QKK_IQ3_XXS>(f, s_x + p * 2048, lane);
+            split_xslice(xs[p], f);
         }
-        scale = 1.f / sqrtf(block_sum4(ss, s_red) / (float)(2048 * PASSES) + eps); // its barrier publishes s_x
-    }
+    } else {
 #pragma unroll
-    for (int p = 0; p < PASSES; p++) {
-        XSlice f;
-        load_xslice<TYPE>(f, s_x + p * 2048, lane);
-        split_xslice(xs[p], f);
+        for (int p = 0; p < PASSES; p++) {
+            XSlice f;
+            load_xslice<QKK_IQ3_XXS>(f, x + p * 2048, lane);
+            split_xslice(xs[p], f);
+        }
     }
 
     fill_iq3_half_entry(tab, threadIdx.x, grid_word);
@@ -370,48 +272,79 @@ __global__ __launch_bounds__(256) void moe_gateup_norm_kernel(const uint8_t* __r
         }
     }
 
-    const uint32_t groups = (d.F + RIF - 1) / RIF; // row groups per pick
+    // round trip 2: the picked rows
+    const uint32_t groups = d.F / RPW; // row groups per pick (the launcher checks F % RPW == 0)
+    uint8_t* area = s_stage[wave];
     for (uint32_t t = blockIdx.x * 4 + wave; t < d.k * groups; t += gridDim.x * 4) {
-        const uint32_t s = t / groups, r0 = (t % groups) * RIF;
+        const uint32_t s = t / groups, r0 = (t % groups) * RPW;
         const uint32_t e = min(s_sel.ids[s], d.E - 1);
-        const uint8_t* gbase = gate_exps + ((size_t)e * d.F) * row_bytes;
-        const uint8_t* ubase = up_exps + ((size_t)e * d.F) * row_bytes;
-        LaneW<TYPE> wg[RIF][PASSES], wu[RIF][PASSES];
+        WaveStage<NP> sg, su;
+        sg.fetch(gate_exps + ((size_t)e * d.F + r0) * RB, NPIECE, lane);
+        su.fetch(up_exps + ((size_t)e * d.F + r0) * RB, NPIECE, lane);
+        float g[RPW], u[RPW];
+        sg.commit(area, lane);
 #pragma unroll
-        for (int i = 0; i < RIF; i++) {
-            const uint32_t r = min(r0 + i, d.F - 1);
+        for (int i = 0; i < RPW; i++) {
+            float a = 0.f;
 #pragma unroll
             for (int p = 0; p < PASSES; p++) {
-                wg[i][p].load(gbase + (size_t)r * row_bytes + (size_t)p * pass_bytes, lane);
-                wu[i][p].load(ubase + (size_t)r * row_bytes + (size_t)p * pass_bytes, lane);
+                LaneW<QKK_IQ3_XXS> w;
+                lane_load_lds<QKK_IQ3_XXS>(w, area, i * RB + p * 8 * IQ3_XXS_BYTES, lane);
+                a += w.dot_h(xs[p], &tab);
             }
+            g[i] = wave_sum(a) * scale;
         }
+        su.commit(area, lane); // LDS operations of a wave run in order: the reads above are done
 #pragma unroll
-        for (int i = 0; i < RIF; i++) {
-            float g = 0.f, u = 0.f;
+        for (int i = 0; i < RPW; i++) {
+            float a = 0.f;
 #pragma unroll
             for (int p = 0; p < PASSES; p++) {
-                g += wg[i][p].dot_h(xs[p], &tab);
-                u += wu[i][p].dot_h(xs[p], &tab);
+                LaneW<QKK_IQ3_XXS> w;
+                lane_load_lds<QKK_IQ3_XXS>(w, area, i * RB + p * 8 * IQ3_XXS_BYTES, lane);
+                a += w.dot_h(xs[p], &tab);
             }
-            g = wave_sum(g) * scale;
-            u = wave_sum(u) * scale;
-            if (lane == 0 && r0 + i < d.F) ws.h[(size_t)s * d.F + r0 + i] = (g / (1.f + expf(-g))) * u;
+            u[i] = wave_sum(a) * scale;
+        }
+        if (lane == 0) {
+#pragma unroll
+            for (int i = 0; i < RPW; i++) ws.h[(size_t)s * d.F + r0 + i] = (g[i] / (1.f + expf(-g[i]))) * u[i];
         }
     }
 }
 
 // ---- launch 3: routed down + shared down + combine ---------------------------------------
-// Wave task = RIF consecutive outputs o.  F = 32*LPR: LPR lanes cover one down row, so
-// 64/LPR picks are processed side by side; the shared Q8_0 row rides on lane group 0.
-// Round trip 1 fetches everything that does not depend on the picks (router record, h slices,
-// shared rows, codebook); round trip 2 the picked experts' rows.
+// Wave task = RIF consecutive outputs o.  F = 32*LPR: LPR lanes cover one down row, so 64/LPR picks
+// are processed side by side, in ROUNDS rounds; the shared Q8_0 row rides on lane group 0.
+// Round trip 1 fetches everything that does not depend on the picks (router record, h, shared rows,
+// codebook); round trip 2 the picked experts' rows: for every pick the RIF rows are one contiguous
+// run of its expert, fetched as 16-byte pieces (all picks' runs in one set of loads) into the wave's
+// LDS area.  Every wave needs all of h: fetched once per workgroup and shared through LDS.
 template <bool ON>
 struct ResidArg {
     const float* p;
 };
 template <>
 struct ResidArg<false> {};
+
+// LDS of the down launch, carved from one dynamic allocation.
+template <int TYPE, int LPR, int ROUNDS, int RIF>
+struct DownShape {
+    static constexpr int GROUPS = WAVE / LPR, PICKS = ROUNDS * GROUPS;
+    static constexpr uint32_t F = 32 * LPR;
+    static constexpr uint32_t RB = (uint32_t)qkk_row_bytes_dev<TYPE>(F), RUN = RIF * RB;
+    // a run starts at a multiple of RUN bytes inside its expert (whose size is a multiple of 16)
+    static constexpr uint32_t NRUN = RUN % 16 == 0 ? RUN / 16 : (RUN + 14 + 15) / 16; // pieces per pick, from the 16-byte boundary below
+    static_assert(RUN % 2 == 0 && (TYPE != QKK_IQ4_XS || RUN % 8 == 0), "runs start on 2-byte (IQ4_XS: 8-byte) boundaries");
+    static constexpr int NP = (PICKS * NRUN + 63) / 64;
+    static constexpr uint32_t Q8ROW = F / 32 * Q8_0_BYTES, SRUN = RIF * Q8ROW;
+    static_assert(SRUN % 16 == 0, "shared rows must be whole 16-byte pieces");
+    static constexpr int NPS = (SRUN / 16 + 63) / 64;
+    static constexpr uint32_t WAVE_LDS = WaveStage<NP>::AREA + WaveStage<NPS>::AREA + 32;
+    // whether the IQ4_XS product runs on packed halves (its activation slices take 32 registers per round)
+    static constexpr bool HALF = TYPE == QKK_IQ4_XS && ROUNDS <= 2;
+    static size_t lds_bytes(uint32_t k) { return (size_t)(k + 1) * F * 4 + 4 * WAVE_LDS; }
+};
 
 // RESID: y = resid + step (the residual row may be y: an element is read and written by the same lane).
 template <int TYPE, int LPR, int ROUNDS, int RIF, bool RESID, bool ROWS>
@@ -420,38 +353,41 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const uint8_t* __restrict
                                                        MoeWs ws, const qkk_sel* __restrict__ sel,
                                                        float* y, MoeDims d, ResidArg<RESID> ra)
 {
+    using S = DownShape<TYPE, LPR, ROUNDS, RIF>;
     if constexpr (ROWS) { // blockIdx.y = activation row, as in launch 1
         ws.h += (size_t)blockIdx.y * (d.k + 1) * d.F;
         sel += blockIdx.y;
         y += (size_t)blockIdx.y * d.H;
         if constexpr (RESID) ra.p += (size_t)blockIdx.y * d.H;
     }
-    extern __shared__ __attribute__((aligned(16))) float s_h[]; // [(k+1)][F]: the gated activations of every pick
+    QK_DYN_LDS(uint8_t, s_dyn);
+    float* s_h = (float*)s_dyn; // [(k+1)][F]: the gated activations of every pick
     __shared__ IqTables tab;
-    constexpr int GROUPS = WAVE / LPR;
+    __shared__ Iq4PairTable tab4;
+    __shared__ uint32_t s_eid[QKK_MAX_USED];
+    __shared__ float s_wt[QKK_MAX_USED + 1];
+    constexpr int GROUPS = S::GROUPS;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lir = lane % LPR, grp = lane / LPR;
-    const uint32_t row_bytes = (uint32_t)qkk_row_bytes_dev<TYPE>(d.F);
-    const uint32_t q8_row = d.F / 32 * Q8_0_BYTES;
-    const uint32_t o0 = (blockIdx.x * 4 + wave) * RIF; // the grid covers every output once
+    uint8_t* area = s_dyn + (size_t)(d.k + 1) * d.F * 4 + (size_t)wave * S::WAVE_LDS;
+    uint8_t* sarea = area + WaveStage<S::NP>::AREA + 16;
+    const uint32_t o0 = min((blockIdx.x * 4 + wave) * RIF, d.H - RIF); // the grid covers every output once (H % RIF == 0)
+    const bool live = (blockIdx.x * 4 + wave) * RIF < d.H;
 
-    // round trip 1: everything that does not depend on the picks.  Every wave needs all of h (each
-    // lane group one pick's row per round): fetched once per workgroup and shared through LDS --
-    // a thousand waves each reading the same 18 KB made this round trip twice as long as the next.
-    uint32_t eid[ROUNDS];
-    float wt[ROUNDS];
-#pragma unroll
-    for (int q = 0; q < ROUNDS; q++) {
-        const uint32_t s = q * GROUPS + grp;
-        const uint32_t sc = s < d.k ? s : 0;
-        eid[q] = sel->ids[sc];
-        wt[q] = sel->w[sc];
+    // round trip 1: everything that does not depend on the picks
+    uint32_t my_eid = 0;
+    float my_wt = 0.f;
+    if (threadIdx.x < QKK_MAX_USED) {
+        const uint32_t sc = threadIdx.x < d.k ? threadIdx.x : 0;
+        my_eid = sel->ids[sc];
+        my_wt = threadIdx.x < d.k ? sel->w[sc] : 0.f;
+    } else if (threadIdx.x == QKK_MAX_USED) {
+        my_wt = sel->w_shared;
     }
-    float wsh = sel->w_shared;
     float res[RIF];
 #pragma unroll
     for (int i = 0; i < RIF; i++) {
-        if constexpr (RESID) res[i] = ra.p[min(o0 + i, d.H - 1)];
+        if constexpr (RESID) res[i] = ra.p[o0 + i];
         else res[i] = 0.f;
     }
     const uint32_t h_quads = (d.k + 1) * d.F / 4;
@@ -460,51 +396,106 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const uint8_t* __restrict
     float4 hq[HQ];
 #pragma unroll
     for (int i = 0; i < HQ; i++) hq[i] = hg[min(threadIdx.x + 256u * i, h_quads - 1)];
-    LaneW<QKK_Q8_0> wq[RIF];
+    WaveStage<S::NPS> ss;
+    ss.fetch(down_shexp + (size_t)o0 * S::Q8ROW, S::SRUN / 16, lane);
+    if constexpr (S::HALF) fill_iq4_pair_entry(tab4, threadIdx.x);
+    else fill_iq_tables(tab, g_iq3xxs_grid, threadIdx.x, 256);
 #pragma unroll
-    for (int i = 0; i < RIF; i++) wq[i].load(down_shexp + (size_t)min(o0 + i, d.H - 1) * q8_row, lir);
-    fill_iq_tables(tab, g_iq3xxs_grid, threadIdx.x, 256);
+    for (int i = 0; i < HQ; i++) // keeps the loads of h above this line, all in flight at once: sunk into the guarded stores below, they ran one after the other
+        asm volatile("" : QK_REG(hq[i].x), QK_REG(hq[i].y), QK_REG(hq[i].z), QK_REG(hq[i].w));
+    if (threadIdx.x < QKK_MAX_USED) s_eid[threadIdx.x] = min(my_eid, d.E - 1);
+    if (threadIdx.x <= QKK_MAX_USED) s_wt[threadIdx.x] = my_wt;
 #pragma unroll
     for (int i = 0; i < HQ; i++)
         if (threadIdx.x + 256u * i < h_quads) ((float4*)s_h)[threadIdx.x + 256u * i] = hq[i];
     for (uint32_t q4 = threadIdx.x + 256u * HQ; q4 < h_quads; q4 += 256u) ((float4*)s_h)[q4] = hg[q4]; // wide layers only
+    ss.commit(sarea, lane);
+    __syncthreads(); // the picks, h and the codebook in LDS
 
-    // round trip 2
-    LaneW<TYPE> w[RIF][ROUNDS];
-#pragma unroll
-    for (int q = 0; q < ROUNDS; q++) {
-        const uint8_t* base = down_exps + (size_t)min(eid[q], d.E - 1) * d.H * row_bytes;
-        if (q * GROUPS + grp >= (int)d.k) wt[q] = 0.f;
-#pragma unroll
-        for (int i = 0; i < RIF; i++) w[i][q].load(base + (size_t)min(o0 + i, d.H - 1) * row_bytes, lir);
+    // round trip 2: the picks' runs
+    const uint32_t A = ((size_t)o0 * S::RB) & 15u; // where a run starts behind its 16-byte boundary
+    WaveStage<S::NP> st;
+    {
+        const uint8_t* base = down_exps + (size_t)o0 * S::RB - A;
+        const size_t expert_bytes = (size_t)d.H * S::RB;
+        // NRUN is the largest piece count over the possible start offsets A; pieces behind the run's
+        // last byte are not needed and may lie behind the end of the tensor: re-read the last one
+        const uint32_t last = (A + S::RUN - 1) / 16;
+        st.fetch_at([&](uint32_t i) {
+            const uint32_t c = min(i, (uint32_t)(S::PICKS * S::NRUN) - 1), pick = c / S::NRUN, idx = min(c % S::NRUN, last);
+            return base + (size_t)s_eid[min(pick, d.k - 1)] * expert_bytes + 16 * idx;
+        }, lane);
     }
-    if (grp != 0) wsh = 0.f;
-    __syncthreads(); // h and the codebook in LDS
-    XSlice hs[ROUNDS], hsh;
+    // while they travel: this lane's slices of h and its weights
+    float wt[ROUNDS];
 #pragma unroll
     for (int q = 0; q < ROUNDS; q++) {
         const uint32_t s = q * GROUPS + grp;
-        load_xslice<TYPE>(hs[q], s_h + (size_t)(s < d.k ? s : 0) * d.F, lir);
+        wt[q] = s < d.k ? s_wt[s] : 0.f;
     }
+    const float wsh = grp == 0 ? s_wt[QKK_MAX_USED] : 0.f;
+    XSlice hsh;
     load_xslice<QKK_Q8_0>(hsh, s_h + (size_t)d.k * d.F, lir);
-    float hsum[ROUNDS][4];
-#pragma unroll
-    for (int q = 0; q < ROUNDS; q++)
-#pragma unroll
-        for (int c = 0; c < 4; c++) {
-            float a = 0.f;
-#pragma unroll
-            for (int i = 0; i < 8; i++) a += hs[q].v[c * 8 + i];
-            hsum[q][c] = a;
-        }
+    float shared_part[RIF];
 #pragma unroll
     for (int i = 0; i < RIF; i++) {
-        float acc = wsh * wq[i].dot(hsh, nullptr, nullptr, lir);
+        LaneW<QKK_Q8_0> wq;
+        lane_load_lds<QKK_Q8_0>(wq, sarea, i * S::Q8ROW, lir);
+        shared_part[i] = wsh * wq.dot(hsh, nullptr, nullptr, lir);
+    }
+    float acc[RIF];
+    if constexpr (S::HALF) {
+        XSliceH hs[ROUNDS];
 #pragma unroll
-        for (int q = 0; q < ROUNDS; q++) acc += wt[q] * w[i][q].dot(hs[q], hsum[q], &tab, lir);
-        acc = wave_sum(acc);
-        if constexpr (RESID) acc += res[i];
-        if (lane == 0 && o0 + i < d.H) y[o0 + i] = acc;
+        for (int q = 0; q < ROUNDS; q++) {
+            const uint32_t s = q * GROUPS + grp;
+            XSlice f;
+            load_xslice<TYPE>(f, s_h + (size_t)(s < d.k ? s : 0) * d.F, lir);
+            split_xslice_iq4(hs[q], f);
+        }
+        st.commit(area, lane);
+#pragma unroll
+        for (int i = 0; i < RIF; i++) {
+            acc[i] = shared_part[i];
+#pragma unroll
+            for (int q = 0; q < ROUNDS; q++) {
+                LaneW<TYPE> w;
+                lane_load_lds<TYPE>(w, area, (q * GROUPS + grp) * S::NRUN * 16 + A + i * S::RB, lir);
+                acc[i] += wt[q] * w.dot_h(hs[q], &tab4, lir);
+            }
+        }
+    } else {
+        XSlice hs[ROUNDS];
+        float hsum[ROUNDS][4];
+#pragma unroll
+        for (int q = 0; q < ROUNDS; q++) {
+            const uint32_t s = q * GROUPS + grp;
+            load_xslice<TYPE>(hs[q], s_h + (size_t)(s < d.k ? s : 0) * d.F, lir);
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                float a = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; i++) a += hs[q].v[c * 8 + i];
+                hsum[q][c] = a;
+            }
+        }
+        st.commit(area, lane);
+#pragma unroll
+        for (int i = 0; i < RIF; i++) {
+            acc[i] = shared_part[i];
+#pragma unroll
+            for (int q = 0; q < ROUNDS; q++) {
+                LaneW<TYPE> w;
+                lane_load_lds<TYPE>(w, area, (q * GROUPS + grp) * S::NRUN * 16 + A + i * S::RB, lir);
+                acc[i] += wt[q] * w.dot(hs[q], hsum[q], &tab, lir);
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < RIF; i++) {
+        float a = wave_sum(acc[i]);
+        if constexpr (RESID) a += res[i];
+        if (lane == 0 && live) y[o0 + i] = a;
     }
 }
 
@@ -546,14 +537,16 @@ template <int TYPE, int LPR, int ROUNDS, int RIF>
 static void launch_down2(const qkk_moe_layer* L, const MoeWs& ws, const qkk_sel* sel, float* Y,
                          const MoeDims& d, const float* resid, uint32_t rows, hipStream_t st)
 {
+    using S = DownShape<TYPE, LPR, ROUNDS, RIF>;
     const uint32_t waves = (d.H + RIF - 1) / RIF;
-    const uint32_t lds = (d.k + 1) * d.F * 4; // h in LDS (at most 17 * 1024 floats = 68 KB)
+    const uint32_t lds = (uint32_t)S::lds_bytes(d.k); // h [(k+1)][F] + the waves' staging areas
     static bool raised = [] {
+        const int most = (int)S::lds_bytes(QKK_MAX_USED);
         for (const void* f : {(const void*)moe_down_kernel<TYPE, LPR, ROUNDS, RIF, false, false>,
                               (const void*)moe_down_kernel<TYPE, LPR, ROUNDS, RIF, true, false>,
                               (const void*)moe_down_kernel<TYPE, LPR, ROUNDS, RIF, false, true>,
                               (const void*)moe_down_kernel<TYPE, LPR, ROUNDS, RIF, true, true>})
-            (void)hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 17 * 1024 * 4);
+            (void)hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, most);
         return true;
     }();
     (void)raised;
@@ -607,67 +600,53 @@ struct MoeNorm {
     float* sum = nullptr;       // ... which launch 1 stores here for launches 2 and 3
 };
 
-// Launches 1 and 2 for `rows` activation rows (grid.y); norm given (one row only): the variants with
-// the RMS norm in front.
+// Launches 1 and 2 for `rows` activation rows (grid.y); norm given: the variants with the RMS norm
+// in front.
 static void launch_route_gateup(const qkk_moe_layer* L, const float* X, const MoeWs& ws, qkk_sel* sel, const MoeDims& d,
                                 uint32_t stages, const MoeNorm* norm, uint32_t rows, hipStream_t st)
 {
     const uint8_t *gs = (const uint8_t*)L->gate_shexp, *us = (const uint8_t*)L->up_shexp;
     const uint8_t *ge = (const uint8_t*)L->gate_exps, *ue = (const uint8_t*)L->up_exps;
     const bool wide = d.H != 2048; // n_embd 4096
-    const dim3 block(256);
     if (stages & QKK_STAGE_ROUTE) {
-        const dim3 grid((d.E + 1 + d.F + 3) / 4, rows);
-#define QK_ROUTE(K) hipLaunchKernelGGL(K, grid, block, 0, st, L->gate_inp, L->gate_inp_shexp, gs, us, X, ws, d)
-#define QK_ROUTE_NORM(K) \
-    hipLaunchKernelGGL(K, grid, block, 0, st, L->gate_inp, L->gate_inp_shexp, gs, us, X, ws, d, norm->w, norm->eps, \
-                       AddArg<false>{})
-#define QK_ROUTE_ADD(K) \
-    hipLaunchKernelGGL(K, grid, block, 0, st, L->gate_inp, L->gate_inp_shexp, gs, us, X, ws, d, norm->w, norm->eps, \
-                       AddArg<true>{norm->mix, norm->sum})
-        if (norm && norm->mix) {
-            if (!wide && rows > 1) QK_ROUTE_ADD((moe_route_norm_kernel<8, true, true>));
-            else if (!wide) QK_ROUTE_ADD((moe_route_norm_kernel<8, false, true>));
-            else if (rows > 1) QK_ROUTE_ADD((moe_route_norm_kernel<16, true, true>));
-            else QK_ROUTE_ADD((moe_route_norm_kernel<16, false, true>));
-        } else if (norm && rows > 1) {
-            if (!wide) QK_ROUTE_NORM((moe_route_norm_kernel<8, true>));
-            else QK_ROUTE_NORM((moe_route_norm_kernel<16, true>));
-        } else if (norm) {
-            if (!wide) QK_ROUTE_NORM((moe_route_norm_kernel<8, false>));
-            else QK_ROUTE_NORM((moe_route_norm_kernel<16, false>));
-        } else if (rows > 1) {
-            if (!wide) QK_ROUTE((moe_route_kernel<8, true>));
-            else QK_ROUTE((moe_route_kernel<16, true>));
-        } else {
-            if (!wide) QK_ROUTE((moe_route_kernel<8, false>));
-            else QK_ROUTE((moe_route_kernel<16, false>));
-        }
+        const dim3 grid((d.E + 1 + d.F + ROUTE_WAVES - 1) / ROUTE_WAVES, rows), block(64 * ROUTE_WAVES);
+#define QK_ROUTE(NCH, ROWS) \
+    do { \
+        if (norm && norm->mix) \
+            hipLaunchKernelGGL((moe_route_kernel<NCH, ROWS, 2>), grid, block, 0, st, L->gate_inp, L->gate_inp_shexp, gs, us, X, \
+                               ws, d, NormArg<true>{norm->w, norm->eps}, AddArg<true>{norm->mix, norm->sum}); \
+        else if (norm) \
+            hipLaunchKernelGGL((moe_route_kernel<NCH, ROWS, 1>), grid, block, 0, st, L->gate_inp, L->gate_inp_shexp, gs, us, X, \
+                               ws, d, NormArg<true>{norm->w, norm->eps}, AddArg<false>{}); \
+        else \
+            hipLaunchKernelGGL((moe_route_kernel<NCH, ROWS, 0>), grid, block, 0, st, L->gate_inp, L->gate_inp_shexp, gs, us, X, \
+                               ws, d, NormArg<false>{}, AddArg<false>{}); \
+    } while (0)
+        if (!wide && rows > 1) QK_ROUTE(8, true);
+        else if (!wide) QK_ROUTE(8, false);
+        else if (rows > 1) QK_ROUTE(16, true);
+        else QK_ROUTE(16, false);
 #undef QK_ROUTE
-#undef QK_ROUTE_NORM
-#undef QK_ROUTE_ADD
     }
     if (norm && norm->mix) X = norm->sum; // launch 2 reads the sum launch 1 stored
     if (stages & QKK_STAGE_GATEUP) {
-        constexpr int GU_RIF = 4;
-        const dim3 grid(wide ? (d.k * ((d.F + 1) / 2) + 3) / 4 : (d.k * ((d.F + GU_RIF - 1) / GU_RIF) + 3) / 4, rows);
-#define QK_GATEUP(K) hipLaunchKernelGGL(K, grid, block, 0, st, ge, ue, X, ws, sel, d)
-#define QK_GATEUP_NORM(K) hipLaunchKernelGGL(K, grid, block, 0, st, ge, ue, X, ws, sel, d, norm->w, norm->eps)
-        if (norm && rows > 1) {
-            if (!wide) QK_GATEUP_NORM((moe_gateup_norm_kernel<QKK_IQ3_XXS, 1, GU_RIF, true>));
-            else QK_GATEUP_NORM((moe_gateup_norm_kernel<QKK_IQ3_XXS, 2, 2, true>));
-        } else if (norm) {
-            if (!wide) QK_GATEUP_NORM((moe_gateup_norm_kernel<QKK_IQ3_XXS, 1, GU_RIF, false>));
-            else QK_GATEUP_NORM((moe_gateup_norm_kernel<QKK_IQ3_XXS, 2, 2, false>));
-        } else if (rows > 1) {
-            if (!wide) QK_GATEUP((moe_gateup_kernel<QKK_IQ3_XXS, 1, GU_RIF, true>));
-            else QK_GATEUP((moe_gateup_kernel<QKK_IQ3_XXS, 2, 2, true>));
-        } else {
-            if (!wide) QK_GATEUP((moe_gateup_kernel<QKK_IQ3_XXS, 1, GU_RIF, false>));
-            else QK_GATEUP((moe_gateup_kernel<QKK_IQ3_XXS, 2, 2, false>));
-        }
+        // FFN rows per wave: four at n_embd 2048, two at 4096 (the same bytes); n_ff is a multiple of both
+        const uint32_t rpw = wide ? 2 : 4;
+        const dim3 grid((d.k * (d.F / rpw) + 3) / 4, rows), block(256);
+#define QK_GATEUP(PASSES, RPW, ROWS) \
+    do { \
+        if (norm) \
+            hipLaunchKernelGGL((moe_gateup_kernel<PASSES, RPW, ROWS, true>), grid, block, 0, st, ge, ue, X, ws, sel, d, \
+                               NormArg<true>{norm->w, norm->eps}); \
+        else \
+            hipLaunchKernelGGL((moe_gateup_kernel<PASSES, RPW, ROWS, false>), grid, block, 0, st, ge, ue, X, ws, sel, d, \
+                               NormArg<false>{}); \
+    } while (0)
+        if (!wide && rows > 1) QK_GATEUP(1, 4, true);
+        else if (!wide) QK_GATEUP(1, 4, false);
+        else if (rows > 1) QK_GATEUP(2, 2, true);
+        else QK_GATEUP(2, 2, false);
 #undef QK_GATEUP
-#undef QK_GATEUP_NORM
     }
 }
 

@@ -183,7 +183,7 @@ __global__ __launch_bounds__(512) void moe_logits_tiled_kernel(const float* __re
                                                                const float* __restrict__ X, MoeWs ws, MoeDims d,
                                                                uint32_t N)
 {
-    extern __shared__ __attribute__((aligned(16))) float s_x[]; // [16][2048]
+    QK_DYN_LDS(float, s_x); // [16][2048]
     constexpr int NCH = 8;                                      // n_embd = 2048: eight float4 per lane
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t n_rows = RIDE ? d.E : d.E + 1; // rows dealt out in groups of eight

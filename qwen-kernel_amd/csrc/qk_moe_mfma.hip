@@ -115,7 +115,7 @@ __global__ __launch_bounds__(CT, SHARED ? 2 : 4) void moe_gateup_mfma_kernel(con
 {
     using Geo = GuGeo<SHARED>;
     constexpr int TYPE = SHARED ? QKK_Q8_0 : QKK_IQ3_XXS;
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    QK_DYN_LDS(uint8_t, smem);
     __shared__ MfmaTables tab;
     __shared__ uint32_t s_tok[16], s_slot[16];
     const int tid = threadIdx.x;
@@ -161,7 +161,7 @@ __global__ __launch_bounds__(CT) void moe_down_mfma_kernel(const uint8_t* __rest
 {
     using Geo = DnGeo<TYPE, FB>;
     constexpr int TG = TYPE == QKK_IQ4_XS ? 2 : 1;
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    QK_DYN_LDS(uint8_t, smem);
     __shared__ MfmaTables tab;
     __shared__ uint32_t s_tok[16], s_slot[16];
     __shared__ float s_wt[16];
@@ -293,7 +293,7 @@ __global__ __launch_bounds__(CT) void moe_gateup_fused_kernel(const uint8_t* __r
                                                              const float* __restrict__ X, MoeWs ws, MoeDims d,
                                                              uint32_t N)
 {
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    QK_DYN_LDS(uint8_t, smem);
     __shared__ MfmaTables tab;
     __shared__ uint32_t s_tok[16], s_slot[16];
     const int tid = threadIdx.x;
@@ -367,7 +367,7 @@ __global__ __launch_bounds__(CT) void moe_down_fused_kernel(const uint8_t* __res
                                                            const qkk_sel* __restrict__ sel, MoeDims d, uint32_t N)
 {
     using Geo = DnGeoF<TYPE_DN, FB>;
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    QK_DYN_LDS(uint8_t, smem);
     __shared__ MfmaTables tab;
     __shared__ uint32_t s_tok[16], s_slot[16];
     __shared__ float s_wt[16];

@@ -5,6 +5,7 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 
 import __graft_entry__ as entry  # noqa: E402
 
@@ -24,8 +25,28 @@ def orc():
 
 
 @pytest.fixture(scope="session")
-def dev():
+def dev(qk):
     import torch
+    if os.environ.get("QK_EMU") == "1":
+        # The GPU tests against the host-side build of the kernels (tests/emu): tensors live in host
+        # memory, the wrappers call libqk_emu.so.  For checking kernel logic where no GPU is at hand;
+        # entry points that build leaves out fail with a status, not silently.
+        import emu_util
+        qk.capi._lib = emu_util.emu_lib(qk)
+        qk.capi._stream = lambda: None
+        torch.cuda.synchronize = lambda *a, **k: None
+        plain_zeros = torch.zeros
+
+        def zeros(*a, **k):   # workspaces must be 256-byte aligned; host allocations are 64-byte aligned
+            t = plain_zeros(*a, **k)
+            if t.dtype == torch.uint8 and t.dim() == 1 and t.data_ptr() % 256:
+                big = plain_zeros(t.numel() + 256, dtype=torch.uint8)
+                off = (-big.data_ptr()) % 256
+                return big[off:off + t.numel()]
+            return t
+        torch.zeros = zeros
+        print("[emu] kernels run in the host-side build", flush=True)
+        return "cpu"
     if not torch.cuda.is_available():
         pytest.skip("no HIP device")
     print(f"[gpu] {torch.cuda.get_device_name(0)}", flush=True)

@@ -1,0 +1,321 @@
+// Runtime of the host-side kernel build (see include/hip/hip_runtime.h).  TEST INFRASTRUCTURE ONLY.
+//
+// Every GPU thread of a workgroup is a fiber (its own stack, switched in user space) on ONE OS
+// thread; a scheduler runs the fibers round robin and a fiber leaves the CPU only at a barrier that
+// is not complete yet.  Workgroups of a launch run on a few OS threads side by side (`__shared__`
+// is thread-local storage).  A launch in which every live fiber waits and nothing can run is
+// reported as a deadlock, with the barrier kinds, instead of hanging.  The dynamic LDS of a
+// workgroup ends at an inaccessible page.
+#include <hip/hip_runtime.h>
+
+#include <stdlib.h>
+#include <sys/mman.h>
+#include <unistd.h>
+
+#include <atomic>
+#include <mutex>
+#include <thread>
+#include <vector>
+
+// void emu_ctx_switch(void** save_sp, void* load_sp): saves the callee-saved registers on the current
+// stack, leaves the stack pointer in *save_sp and continues on the stack load_sp (System V x86-64).
+asm(R"(
+.text
+.globl emu_ctx_switch
+.type emu_ctx_switch,@function
+emu_ctx_switch:
+    pushq %rbp
+    pushq %rbx
+    pushq %r12
+    pushq %r13
+    pushq %r14
+    pushq %r15
+    movq %rsp, (%rdi)
+    movq %rsi, %rsp
+    popq %r15
+    popq %r14
+    popq %r13
+    popq %r12
+    popq %rbx
+    popq %rbp
+    ret
+.size emu_ctx_switch,.-emu_ctx_switch
+)");
+extern "C" void emu_ctx_switch(void** save_sp, void* load_sp);
+
+namespace emu {
+
+Idx g_block_dim, g_grid_dim;
+
+namespace {
+constexpr int MAX_WAVES = 16;
+constexpr size_t STACK_BYTES = 512 * 1024;
+
+struct Fiber {
+    void* sp = nullptr;
+    uint8_t* stack = nullptr; // mapping of STACK_BYTES + one guard page below
+    Idx tid{};
+    bool done = false;
+    int wait_kind = 0; // 0 runnable, 1 wave barrier, 2 block barrier
+    uint64_t wait_gen = 0;
+};
+
+// n bytes that END at an inaccessible page: an access behind the buffer faults at once.
+struct GuardBuf {
+    uint8_t* map = nullptr;
+    size_t map_bytes = 0;
+    uint8_t* p = nullptr;
+    explicit GuardBuf(size_t n, size_t align = 16)
+    {
+        const size_t page = (size_t)sysconf(_SC_PAGESIZE);
+        const size_t body = (n + page - 1) / page * page;
+        map_bytes = body + page;
+        map = (uint8_t*)mmap(nullptr, map_bytes, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS, -1, 0);
+        if (map == MAP_FAILED) abort();
+        mprotect(map + body, page, PROT_NONE);
+        p = map + body - (n + align - 1) / align * align; // aligned; for sizes that are multiples of `align` the end is exact
+    }
+    ~GuardBuf() { munmap(map, map_bytes); }
+    GuardBuf(const GuardBuf&) = delete;
+};
+
+struct Workgroup {
+    std::vector<Fiber> f;
+    int n = 0;
+    void* main_sp = nullptr;
+    Fiber* cur = nullptr;
+    Idx block{};
+    const std::function<void()>* body = nullptr;
+    uint64_t block_gen = 0, wave_gen[MAX_WAVES] = {};
+    int block_arrived = 0, block_expected = 0, wave_arrived[MAX_WAVES] = {}, wave_expected[MAX_WAVES] = {};
+    uint64_t xbuf[MAX_WAVES][64];
+    _Float16 mfma_a[MAX_WAVES][64][8], mfma_b[MAX_WAVES][64][8];
+    GuardBuf* dyn = nullptr;
+    ~Workgroup()
+    {
+        for (auto& x : f)
+            if (x.stack) munmap(x.stack, STACK_BYTES + 4096);
+        delete dyn;
+    }
+};
+thread_local Workgroup* t_wg = nullptr;
+
+void yield_to_scheduler()
+{
+    Workgroup& g = *t_wg;
+    emu_ctx_switch(&g.cur->sp, g.main_sp);
+}
+
+void fiber_entry()
+{
+    Workgroup& g = *t_wg;
+    Fiber* me = g.cur;
+    (*g.body)();
+    // a thread that has left the kernel takes no further part in its barriers
+    me->done = true;
+    const int w = me->tid.x >> 6;
+    if (--g.wave_expected[w] > 0 && g.wave_arrived[w] >= g.wave_expected[w]) {
+        g.wave_arrived[w] = 0;
+        g.wave_gen[w]++;
+    }
+    if (--g.block_expected > 0 && g.block_arrived >= g.block_expected) {
+        g.block_arrived = 0;
+        g.block_gen++;
+    }
+    yield_to_scheduler();
+    abort(); // never resumed
+}
+
+void prepare_fiber(Fiber& fb, uint32_t tid)
+{
+    if (!fb.stack) {
+        fb.stack = (uint8_t*)mmap(nullptr, STACK_BYTES + 4096, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
+        if (fb.stack == MAP_FAILED) abort();
+        mprotect(fb.stack, 4096, PROT_NONE);
+    }
+    uint64_t* top = (uint64_t*)(fb.stack + 4096 + STACK_BYTES); // 16-byte aligned
+    top[-1] = 0;                                                // what fiber_entry would return to
+    top[-2] = (uint64_t)(void*)&fiber_entry;
+    for (int i = 3; i <= 8; i++) top[-i] = 0; // rbp, rbx, r12..r15
+    fb.sp = top - 8;
+    fb.tid = Idx{tid, 0, 0};
+    fb.done = false;
+    fb.wait_kind = 0;
+}
+
+void run_workgroup(Workgroup& g, Idx block, int n, size_t lds, const std::function<void()>& body)
+{
+    t_wg = &g;
+    g.block = block;
+    g.body = &body;
+    g.n = n;
+    if ((int)g.f.size() < n) g.f.resize(n);
+    for (int t = 0; t < n; t++) prepare_fiber(g.f[t], (uint32_t)t);
+    g.block_arrived = 0;
+    g.block_expected = n;
+    for (int w = 0; w < n / 64; w++) {
+        g.wave_arrived[w] = 0;
+        g.wave_expected[w] = 64;
+    }
+    delete g.dyn;
+    g.dyn = new GuardBuf(lds ? lds : 16);
+    int live = n;
+    while (live > 0) {
+        bool ran = false;
+        for (int t = 0; t < n; t++) {
+            Fiber& fb = g.f[t];
+            if (fb.done) continue;
+            if (fb.wait_kind == 1 && g.wave_gen[t >> 6] == fb.wait_gen) continue;
+            if (fb.wait_kind == 2 && g.block_gen == fb.wait_gen) continue;
+            fb.wait_kind = 0;
+            g.cur = &fb;
+            emu_ctx_switch(&g.main_sp, fb.sp);
+            ran = true;
+            if (fb.done) live--;
+        }
+        if (!ran) {
+            int at_wave = 0, at_block = 0;
+            for (int t = 0; t < n; t++)
+                if (!g.f[t].done) (g.f[t].wait_kind == 1 ? at_wave : at_block)++;
+            fprintf(stderr, "emu: deadlock in workgroup (%u,%u,%u): %d threads wait at a wave barrier or cross-lane operation, "
+                            "%d at __syncthreads(), none can run\n", block.x, block.y, block.z, at_wave, at_block);
+            abort();
+        }
+    }
+    t_wg = nullptr;
+}
+
+std::mutex g_launch_mu; // one launch at a time
+} // namespace
+
+const Idx& cur_thread() { return t_wg->cur->tid; }
+const Idx& cur_block() { return t_wg->block; }
+void* dyn_lds() { return t_wg->dyn->p; }
+
+void block_barrier()
+{
+    Workgroup& g = *t_wg;
+    if (++g.block_arrived >= g.block_expected) {
+        g.block_arrived = 0;
+        g.block_gen++;
+        return;
+    }
+    g.cur->wait_kind = 2;
+    g.cur->wait_gen = g.block_gen;
+    yield_to_scheduler();
+}
+void wave_barrier()
+{
+    Workgroup& g = *t_wg;
+    const int w = g.cur->tid.x >> 6;
+    if (++g.wave_arrived[w] >= g.wave_expected[w]) {
+        g.wave_arrived[w] = 0;
+        g.wave_gen[w]++;
+        return;
+    }
+    g.cur->wait_kind = 1;
+    g.cur->wait_gen = g.wave_gen[w];
+    yield_to_scheduler();
+}
+const uint64_t* exchange(uint64_t v)
+{
+    Workgroup& g = *t_wg;
+    const uint32_t t = g.cur->tid.x;
+    g.xbuf[t >> 6][t & 63u] = v;
+    wave_barrier();
+    return t_wg->xbuf[t >> 6];
+}
+void exchange_done() { wave_barrier(); }
+
+void run(dim3 grid, dim3 block, size_t lds, const std::function<void()>& body)
+{
+    std::lock_guard<std::mutex> launch(g_launch_mu);
+    const int n = (int)(block.x * block.y * block.z);
+    if (n <= 0 || n > 64 * MAX_WAVES || (n % 64) != 0 || block.y != 1 || block.z != 1) {
+        fprintf(stderr, "emu: workgroup of %ux%ux%u threads not modelled (multiples of 64 up to %d)\n", block.x, block.y, block.z, 64 * MAX_WAVES);
+        abort();
+    }
+    g_block_dim = Idx{block.x, block.y, block.z};
+    g_grid_dim = Idx{grid.x, grid.y, grid.z};
+    const uint64_t total = (uint64_t)grid.x * grid.y * grid.z;
+    std::atomic<uint64_t> next{0};
+    auto worker = [&] {
+        Workgroup g;
+        for (;;) {
+            const uint64_t b = next.fetch_add(1);
+            if (b >= total) break;
+            const Idx bi{(uint32_t)(b % grid.x), (uint32_t)(b / grid.x % grid.y), (uint32_t)(b / ((uint64_t)grid.x * grid.y))};
+            run_workgroup(g, bi, n, lds, body);
+        }
+    };
+    static const unsigned hw = [] {
+        const char* e = getenv("QK_EMU_THREADS");
+        const unsigned v = e ? (unsigned)atoi(e) : std::thread::hardware_concurrency();
+        return v ? v : 1u;
+    }();
+    const unsigned nt = (unsigned)std::min<uint64_t>(hw, total);
+    std::vector<std::thread> threads;
+    for (unsigned i = 1; i < nt; i++) threads.emplace_back(worker);
+    worker();
+    for (auto& th : threads) th.join();
+}
+
+} // namespace emu
+
+emu_float4 emu_mfma_16x16x32_f16(emu_half8 a, emu_half8 b, emu_float4 c)
+{
+    using namespace emu;
+    Workgroup& g = *t_wg;
+    const uint32_t t = g.cur->tid.x, w = t >> 6, lane = t & 63u;
+    for (int i = 0; i < 8; i++) {
+        g.mfma_a[w][lane][i] = a[i];
+        g.mfma_b[w][lane][i] = b[i];
+    }
+    wave_barrier();
+    const uint32_t col = lane & 15u, rq = lane >> 4;
+    emu_float4 d = c;
+    for (int i = 0; i < 4; i++) {
+        const uint32_t row = 4 * rq + i;
+        float s = 0.f;
+        for (uint32_t kq = 0; kq < 4; kq++)
+            for (int j = 0; j < 8; j++) s += (float)g.mfma_a[w][row + 16 * kq][j] * (float)g.mfma_b[w][col + 16 * kq][j];
+        d[i] += s;
+    }
+    wave_barrier();
+    return d;
+}
+
+// Device allocations of the library itself (the engine's tensors): guarded like the tests' buffers.
+static std::mutex g_alloc_mu;
+static std::vector<std::pair<void*, emu::GuardBuf*>> g_allocs;
+hipError_t hipMalloc(void** p, size_t n)
+{
+    auto* g = new emu::GuardBuf(n ? n : 16);
+    std::lock_guard<std::mutex> l(g_alloc_mu);
+    g_allocs.emplace_back(g->p, g);
+    *p = g->p;
+    return hipSuccess;
+}
+hipError_t hipFree(void* p)
+{
+    if (!p) return hipSuccess;
+    std::lock_guard<std::mutex> l(g_alloc_mu);
+    for (size_t i = 0; i < g_allocs.size(); i++)
+        if (g_allocs[i].first == p) {
+            delete g_allocs[i].second;
+            g_allocs.erase(g_allocs.begin() + i);
+            return hipSuccess;
+        }
+    return hipErrorInvalidValue;
+}
+
+// C entry points for the tests: buffers that end at a guard page.
+extern "C" {
+void* emu_guard_alloc(size_t n, size_t align, void** handle)
+{
+    auto* g = new emu::GuardBuf(n ? n : 16, align < 16 ? 16 : align);
+    *handle = g;
+    return g->p;
+}
+void emu_guard_free(void* handle) { delete (emu::GuardBuf*)handle; }
+}

@@ -1,0 +1,150 @@
+"""The HIP kernels in a host-side build (tests/emu: the kernel sources compiled as C++, one fiber per
+GPU thread) on tensors that END AT AN INACCESSIBLE PAGE, against the oracle.  What this pins without
+a GPU: every index the kernels form stays inside its tensor -- a device allocation can end at a
+mapping boundary exactly like these buffers, and a read behind it is a memory fault there -- and the
+kernels' logic (selection, staging through LDS, reductions, tails of ragged shapes) gives the
+oracle's numbers.  What it cannot pin: timing, the compiler's code for the device, hardware
+behaviour of the cross-lane instructions (modelled after the ISA manual).  The shapes are chosen so
+that the LAST row, the LAST expert and ragged tails are touched."""
+import numpy as np
+import pytest
+
+import emu_util
+
+
+@pytest.fixture(scope="module")
+def emu(qk):
+    with emu_util.emulated(qk) as pool:
+        yield pool
+
+
+QUANT = ["q8_0", "q6_k", "iq4_xs", "iq3_xxs"]
+
+
+def type_id(qk, name):
+    return {"q8_0": qk.Q8_0, "q6_k": qk.Q6_K, "iq4_xs": qk.IQ4_XS, "iq3_xxs": qk.IQ3_XXS}[name]
+
+
+@pytest.mark.parametrize("name", QUANT)
+@pytest.mark.parametrize("K,M", [(2048, 1), (2048, 9), (2048, 67), (4096, 5), (8192, 3), (1024, 11), (512, 23), (256, 70),
+                                 (768, 6)])
+def test_gemv_inside_its_tensors(qk, orc, emu, name, K, M):
+    """Ragged row counts: full chunks go through the staged 16-byte pieces, the rest through per-lane
+    loads; the last row ends at the guard page."""
+    t = type_id(qk, name)
+    if qk.row_bytes(t, K) == 0:
+        pytest.skip("K is not a block multiple of this format")
+    W = qk.synth.tensor_host(t, M, K, seed=K + M)
+    x = np.random.default_rng(M).standard_normal(K).astype(np.float32)
+    pad = (-W.nbytes) % 16   # the kernels want 16-byte aligned tensors; the end stays exact for whole pieces
+    Wd = emu.tensor(W.reshape(-1))
+    Xd, Yd = emu.tensor(x.reshape(1, K)), emu.zeros((1, M), np.float32)
+    qk.gemv(t, Wd, Xd, M, K, out=Yd)
+    want = orc.gemv(t, W, x, M, K)
+    assert orc.rel_maxabs_err(Yd.numpy()[0], want) <= 1e-3, (name, K, M, pad)
+
+
+def moe_case(qk, orc, emu, hl, x, norm_w=None, mix=None):
+    """One call of the step (or of the block with the norm in front) on guarded tensors; returns what
+    the kernels gave and the oracle's reference per row."""
+    n = x.shape[0]
+    layer = emu_util.layer_in_pool(qk, emu, hl)
+    ws = emu.workspace(qk.moe_workspace_bytes(layer, n))
+    sel = emu.zeros((n, 160), np.uint8)
+    if norm_w is None:
+        Y = emu.zeros((n, hl.n_embd), np.float32)
+        qk.moe_decode(layer, emu.tensor(x), ws, Y=Y, sel=sel)
+        got, inp = Y.numpy(), x
+    else:
+        S = emu.tensor(x)
+        W = emu.tensor(norm_w)
+        if mix is None:
+            qk.moe_layer_rows(layer, S, W, ws, sel=sel)
+            base = x
+        else:
+            T = emu.zeros(x.shape, np.float32)
+            qk.moe_layer_rows(layer, S, W, ws, sel=sel, mix=emu.tensor(mix), T=T)
+            base = x + mix
+            assert np.array_equal(T.numpy(), base)
+        inp = np.stack([orc.add_rms(base[r], norm_w, 1e-6) for r in range(n)])
+        got = S.numpy() - base
+    ids = sel.numpy().view(np.uint32).reshape(-1, 40)[:, :hl.n_used]
+    for r in range(n):
+        ref = orc.moe_ref(hl, inp[r])
+        if ref["sel"].gap > 2e-3:
+            assert sorted(ids[r]) == sorted(ref["sel"].ids[:hl.n_used]), r
+            scale = np.max(np.abs(ref["y"]))
+            assert np.max(np.abs(got[r] - ref["y"])) <= 1e-3 * scale + 4e-7 * np.max(np.abs(inp[r])) * (norm_w is not None), r
+    return ids
+
+
+def rows_that_pick_the_last_expert(hl, n, seed, scale=None):
+    rng = np.random.default_rng(seed)
+    gi = hl.gate_inp.astype(np.float64)
+    rows = []
+    while len(rows) < n:
+        x = rng.standard_normal(hl.n_embd).astype(np.float32)
+        top = np.argsort(-(gi @ (x.astype(np.float64) * (1.0 if scale is None else scale))))[:hl.n_used]
+        if hl.n_expert - 1 in top:
+            rows.append(x)
+    return np.stack(rows)
+
+
+@pytest.mark.parametrize("down", ["iq4_xs", "q6_k"])
+@pytest.mark.parametrize("E,k,F,H,n", [(8, 2, 256, 2048, 1), (8, 2, 512, 2048, 3), (16, 16, 256, 2048, 1), (6, 3, 1024, 2048, 2),
+                                       (4, 2, 256, 4096, 2), (20, 10, 512, 2048, 1)])
+def test_moe_step_inside_its_tensors(qk, orc, emu, down, E, k, F, H, n):
+    """The three one-row launches with the LAST expert among the picks: its last rows end at the guard
+    page (a Q6_K run of rows is not a whole number of 16-byte pieces -- the staging must not fetch the
+    piece behind it)."""
+    hl = qk.synth.HostLayer(seed=E + k + F, n_embd=H, n_ff=F, n_expert=E, n_used=k, down_type=type_id(qk, down))
+    x = rows_that_pick_the_last_expert(hl, n, seed=F + n)
+    ids = moe_case(qk, orc, emu, hl, x)
+    assert all(E - 1 in row for row in ids)
+
+
+@pytest.mark.parametrize("down", ["iq4_xs", "q6_k"])
+def test_moe_block_with_norm_inside_its_tensors(qk, orc, emu, down):
+    """The block with the RMS norm in front and the residual behind, alone and with a mixer's rows
+    added on the way, 1 and 3 rows."""
+    hl = qk.synth.HostLayer(seed=91, n_ff=256, n_expert=8, n_used=2, down_type=type_id(qk, down))
+    rng = np.random.default_rng(3)
+    w = rng.uniform(0.5, 1.5, 2048).astype(np.float32)
+    for n in (1, 3):
+        x = (rows_that_pick_the_last_expert(hl, n, seed=n, scale=w.astype(np.float64)) * np.float32(7.0)).astype(np.float32)
+        moe_case(qk, orc, emu, hl, x, norm_w=w)
+        mix = rng.standard_normal(x.shape).astype(np.float32)
+        moe_case(qk, orc, emu, hl, x, norm_w=w, mix=mix)
+
+
+def test_moe_static_workspace_in_the_host_build(qk, orc, emu):
+    """qkk_moe_decode_static against qkk_moe_decode, both through the host-side build: same bits."""
+    hl = qk.synth.HostLayer(seed=12, n_ff=256, n_expert=8, n_used=2)
+    layer = emu_util.layer_in_pool(qk, emu, hl)
+    rng = np.random.default_rng(0)
+    for n in (3, 1):
+        x = rng.standard_normal((n, 2048)).astype(np.float32)
+        ws = emu.workspace(qk.moe_workspace_bytes(layer, n))
+        Y0, sel0 = emu.zeros((n, 2048), np.float32), emu.zeros((n, 160), np.uint8)
+        Y1, sel1 = emu.zeros((n, 2048), np.float32), emu.zeros((n, 160), np.uint8)
+        X = emu.tensor(x)
+        qk.moe_decode(layer, X, ws, Y=Y0, sel=sel0)
+        qk.moe_decode_static(layer, X, Y1, sel1)
+        assert np.array_equal(Y0.numpy().view(np.uint32), Y1.numpy().view(np.uint32))
+        assert np.array_equal(sel0.numpy(), sel1.numpy())
+
+
+@pytest.mark.parametrize("V,batch", [(37, 1), (1000, 1), (300, 3)])
+def test_head_inside_its_tensors(qk, orc, emu, V, batch):
+    """LM head + argmax on a small vocabulary whose last row ends at the guard page."""
+    K = 2048
+    W = qk.synth.tensor_host(qk.Q6_K, V, K, seed=V)
+    x = np.random.default_rng(V).standard_normal((batch, K)).astype(np.float32)
+    ws = emu.workspace(qk.head_workspace_bytes(V, batch))
+    tok, logits = qk.head_argmax(emu.tensor(W.reshape(-1)), emu.tensor(x), V, K, ws, want_logits=True)
+    for b in range(batch):
+        want = orc.gemv(qk.Q6_K, W, x[b], V, K)
+        assert orc.rel_maxabs_err(logits.numpy()[b], want) <= 1e-3
+        top2 = np.sort(want)[-2:]
+        if top2[1] - top2[0] > 2e-3 * abs(top2[1]):
+            assert int(tok.numpy()[b]) == int(np.argmax(want))
