@@ -24,11 +24,11 @@ sys.path.insert(0, ROOT)
 import __graft_entry__ as entry  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what
-# the same counters read for a plain 256 MiB copy (see profiles/); None where no counter run
-# of that kernel has been recorded.
-TRAFFIC = {"moe_gateup_kernel": 6722776,          # profiles/moe_decode_bs1_hbm_traffic.txt
-           "moe_gateup_fused_kernel": 85845150}   # profiles/moe_decode_bs16_hbm_traffic.txt (103 distinct experts)
+MIN_REPLAYS = 10   # graph replays timed at least, whatever --steps says (steps timed = replays x ring, reported)
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by what the same
+# counters read for a plain 256 MiB copy (profiles/); None where no counter run of the CURRENT kernel
+# has been recorded (a figure of an earlier version of a kernel is not carried over).
+TRAFFIC = {"moe_gateup_fused_kernel": 85845150}   # profiles/moe_decode_bs16_hbm_traffic.txt (103 distinct experts)
 
 
 def log(*a):
@@ -77,7 +77,7 @@ def run_ring(launches, steps, warmup):
     (ms_per_step wall, ms_per_step by events)."""
     import torch
     g = Graphed(launches)
-    reps = max(1, steps // g.n)
+    reps = max(MIN_REPLAYS, steps // g.n)   # never a single replay: a driver's small --steps still times ten
     for _ in range(max(1, warmup // g.n)):
         g.replay()
     torch.cuda.synchronize()
@@ -166,11 +166,11 @@ def norm_workload(qk, rows, steps, warmup):
     return ev * 1e3
 
 
-def gemv_workload(qk, type_, M, K, batch, steps, warmup, seed=99):
+def gemv_workload(qk, type_, M, K, batch, steps, warmup, seed=99, ring=None):
     import torch
     dev = "cuda:0"
     rb = qk.row_bytes(type_, K)
-    ring = max(2, int(320e6 // (M * rb)) + 1)
+    ring = ring or max(2, int(320e6 // (M * rb)) + 1)
     be = qk.capi.BLOCK[type_][0]
     if type_ == qk.F16:
         Ws = [(torch.randn(M * K, device=dev) * 0.05).to(torch.float16) for _ in range(ring)]
@@ -392,27 +392,103 @@ def engine_workload(qk, n_layer, slots_list, chunks, warm_chunks, seed=31, kinds
     return res
 
 
-def cpu_baseline(qk, orc, budget_s=12.0):
-    """The oracle's scalar fused-MoE step (the reference's moeCpuRef restated) on one host
-    core, on the same layer shape, a fresh activation row per step."""
+def host_threads():
+    """Threads of the all-cores CPU runs: the cores this process may use, at most 16 (a one-GPU box's share)."""
+    try:
+        n = len(os.sched_getaffinity(0))
+    except AttributeError:
+        n = os.cpu_count() or 1
+    return max(1, min(16, n))
+
+
+def _timed(fn, reps):
+    fn()
+    ts = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    return ts[len(ts) // 2]
+
+
+def cpu_baseline(qk, orc):
+    """The reference's scalar CPU path restated (oracle: dequantise a row, dot in double,
+    src/main.cpp:673-679; moeCpuRef, src/main.cpp:1316-1387) timed on this host: one thread, as the
+    reference runs it, and all host threads (rows or tokens split), per BASELINE config, on bounded
+    samples of each workload.  `value` is the headline config (one fused MoE decode step, bs=1)."""
     import numpy as np
-    hl = qk.synth.HostLayer(seed=4321)
+    nt = host_threads()
+    per = {}
     rng = np.random.default_rng(5)
-    xs = rng.standard_normal((64, 2048)).astype(np.float32)
-    orc.moe_ref(hl, xs[0])  # touch
-    t0 = time.perf_counter()
-    n = 0
-    while True:
-        orc.moe_ref(hl, xs[(n + 1) % 64])
-        n += 1
-        if time.perf_counter() - t0 > budget_s or n >= 400:
-            break
-    dt = (time.perf_counter() - t0) / n
+
+    def entry_(us1, usN, nbytes, sample):
+        return dict(us_1_thread=us1, us_all_threads=usN, threads=nt, gbps_1_thread=nbytes / us1 / 1e3,
+                    gbps_all_threads=nbytes / usN / 1e3, bytes=nbytes, sample=sample)
+
+    # C1: one GEMV 8192 x 2048 per format (a quarter of the rows timed, scaled: rows are independent)
+    M, K, part = 8192, 2048, 2048
+    x = rng.standard_normal(K).astype(np.float32)
+    for name, t in (("q8_0", orc.Q8_0), ("q6_k", orc.Q6_K), ("iq4_xs", orc.IQ4_XS), ("iq3_xxs", orc.IQ3_XXS)):
+        W = qk.synth.tensor_host(t, part, K, seed=42)
+        t1 = _timed(lambda: orc.gemv(t, W, x, part, K), 3) * (M / part)
+        tn = _timed(lambda: orc.gemv(t, W, x, part, K, threads=nt), 5) * (M / part)
+        per[f"C1_gemv_{name}_8192x2048"] = entry_(t1 * 1e6, tn * 1e6, M * orc.row_bytes(t, K) + (K + M) * 4,
+                                                  f"{part} of {M} rows timed, scaled")
+    # C2: the fused MoE decode step, one row
+    hl = qk.synth.HostLayer(seed=4321)
+    xs = rng.standard_normal((16, 2048)).astype(np.float32)
+    it = [0]
+
+    def step1():
+        it[0] += 1
+        orc.moe_ref(hl, xs[it[0] % 16])
+
+    def stepn():
+        it[0] += 1
+        orc.moe_ref_threads(hl, xs[it[0] % 16][None, :], nt)
+    t1, tn = _timed(step1, 5), _timed(stepn, 9)
     layer_bytes = 256 * 2048 * 4 + 2048 * 4 + 8 * (2 * 512 * 784 + 2048 * 272) + 2 * 512 * 2176 + 2048 * 544
-    return dict(value=layer_bytes / dt / 1e9, unit="GB/s", cores=1, kind="port",
-                sample=f"{n} fused MoE decode steps (bs=1, one synthetic layer, fresh x per step), "
-                       f"{dt * 1e6:.0f} us/step, oracle moe_ref single-threaded",
-                us_per_step=dt * 1e6)
+    per["C2_moe_decode_bs1"] = entry_(t1 * 1e6, tn * 1e6, layer_bytes, "whole steps, a fresh activation row per step")
+    c2 = per["C2_moe_decode_bs1"]
+    # C3: the same step for 16 slots, Q6_K down (tokens split over the threads; one thread: 2 slots timed, scaled)
+    hl6 = qk.synth.HostLayer(seed=4322, down_type=qk.Q6_K)
+    t1 = _timed(lambda: orc.moe_ref_threads(hl6, xs[:2], 1), 1) * 8
+    tn = _timed(lambda: orc.moe_ref_threads(hl6, xs, nt), 3)
+    per["C3_moe_decode_bs16_q6k_down"] = entry_(t1 * 1e6, tn * 1e6, 0, "16 slots; one thread: 2 slots timed, scaled; "
+                                                "the CPU path re-reads the weights per slot, so no byte rate is given")
+    for k_ in ("gbps_1_thread", "gbps_all_threads"):
+        per["C3_moe_decode_bs16_q6k_down"][k_] = None
+    # C4: the LM head (Q6_K, 151,936 x 2048) + argmax: 1/16 of the vocabulary timed, scaled
+    V, Vs = 151936, 9496
+    Wh = qk.synth.tensor_host(qk.Q6_K, Vs, K, seed=77)
+    t1 = _timed(lambda: orc.argmax(orc.gemv(orc.Q6_K, Wh, x, Vs, K)), 2) * (V / Vs)
+    tn = _timed(lambda: orc.argmax(orc.gemv(orc.Q6_K, Wh, x, Vs, K, threads=nt)), 3) * (V / Vs)
+    per["C4_lm_head_q6k_151936_bs1"] = entry_(t1 * 1e6, tn * 1e6, V * orc.row_bytes(orc.Q6_K, K) + K * 4,
+                                              f"{Vs} of {V} rows timed, scaled")
+    # C5a: the Q8_0 GEMM 8192 x 2048 x 128 tokens (1/8 of the weight rows timed, scaled)
+    Wg = qk.synth.tensor_host(qk.Q8_0, 1024, K, seed=55)
+    Xg = rng.standard_normal((128, K)).astype(np.float32)
+    t1 = _timed(lambda: orc.gemm_q8_0(Wg, Xg, 1024, K), 1) * 8
+    tn = _timed(lambda: orc.gemm_q8_0(Wg, Xg, 1024, K, threads=nt), 3) * 8
+    per["C5a_gemm_q8_0_8192x2048x128"] = dict(entry_(t1 * 1e6, tn * 1e6, 8192 * 2176 + 128 * (K + 8192) * 4,
+                                                     "1024 of 8192 weight rows timed, scaled"),
+                                              gflops_1_thread=2.0 * 8192 * K * 128 / t1 / 1e9,
+                                              gflops_all_threads=2.0 * 8192 * K * 128 / tn / 1e9)
+    # C5b: the MoE block for 128 tokens (tokens split; one thread: 2 tokens timed, scaled)
+    X128 = rng.standard_normal((128, 2048)).astype(np.float32)
+    t1 = _timed(lambda: orc.moe_ref_threads(hl, X128[:2], 1), 1) * 64
+    tn = _timed(lambda: orc.moe_ref_threads(hl, X128[:4 * nt], nt), 1) * (128 / (4 * nt))
+    per["C5b_moe_prefill_128_tokens"] = dict(us_1_thread=t1 * 1e6, us_all_threads=tn * 1e6, threads=nt,
+                                             tok_per_s_1_thread=128 / t1, tok_per_s_all_threads=128 / tn,
+                                             sample=f"one thread: 2 tokens timed, scaled; all threads: {4 * nt} tokens timed, scaled")
+    return dict(value=c2["gbps_all_threads"], unit="GB/s", cores=nt, kind="port",
+                sample=f"fused MoE decode step (bs=1, one synthetic layer, a fresh activation row per step), oracle moeCpuRef "
+                       f"restatement with its row loops split over {nt} host threads: {c2['us_all_threads']:.0f} us/step "
+                       f"({c2['us_1_thread']:.0f} us/step on one thread, as the reference runs it)",
+                us_per_step=c2["us_all_threads"],
+                one_thread=dict(value=c2["gbps_1_thread"], unit="GB/s", cores=1, us_per_step=c2["us_1_thread"]),
+                host_cpus=os.cpu_count(), per_config=per)
 
 
 def main():
@@ -531,8 +607,10 @@ def main():
                config=dict(workload=a.workload, n_embd=2048, n_ff=512, n_expert=256, n_used=8,
                            gate_up="IQ3_XXS", down="Q6_K" if a.workload.endswith("bs16") else "IQ4_XS",
                            shared="Q8_0", slots={"moe_decode_bs1": 1, "moe_decode_bs16": 16}.get(a.workload, 128),
-                           ring_layers=m["ring"],
-                           ring_bytes=m["ring_bytes"], timing="hipGraph replay of the ring"),
+                           ring_layers=m["ring"], ring_bytes=m["ring_bytes"],
+                           steps_timed=m["steps"], graph_replays_timed=m["steps"] // m["ring"],
+                           timing=f"hipGraph replays of the ring (one launch set per layer of the ring), at least "
+                                  f"{MIN_REPLAYS} replays whatever --steps asks"),
                us_per_step=m["ms_wall"] * 1e3, us_per_step_events=m["ms_event"] * 1e3,
                bytes_per_step=m["bytes_step"], frac_of_hbm_peak=gbps / HBM_PEAK_GBPS,
                distinct_experts_per_step=m["distinct_experts"],
@@ -555,6 +633,16 @@ def main():
                                                          frac=g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9 / HBM_PEAK_GBPS)
                 log(f"[bench] gemv {name} bs16: {ex[f'gemv_{name}_8192x2048_bs16']}")
                 torch.cuda.empty_cache()
+        # the same kernels at a sustained size: one tensor of >= 256 MiB per launch (K = 2048), two tensors
+        # alternating, so neither launch latency nor the caches carry the figure
+        for name, t in (("q8_0", qk.Q8_0), ("q6_k", qk.Q6_K), ("iq4_xs", qk.IQ4_XS), ("iq3_xxs", qk.IQ3_XXS)):
+            Ms = -(-(256 << 20) // qk.row_bytes(t, 2048) // 64) * 64
+            g = gemv_workload(qk, t, Ms, 2048, 1, 40, 4, ring=2)
+            gb = g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9
+            ex[f"gemv_{name}_sustained_256MiB"] = dict(rows=Ms, us=g["ms_event"] * 1e3, gbps=gb, frac=gb / HBM_PEAK_GBPS,
+                                                       steps_timed=g["steps"])
+            log(f"[bench] gemv {name} sustained: {ex[f'gemv_{name}_sustained_256MiB']}")
+            torch.cuda.empty_cache()
         # the other dense projections of a decode step at the reference's shapes (src/main.cpp:4310-4335)
         for M, K in ((4096, 2048), (2048, 4096), (512, 2048)):
             for b in (1, 16):
@@ -571,6 +659,13 @@ def main():
             log(f"[bench] head bs{b}: {ex[f'head_q6k_151936_bs{b}']}")
             torch.cuda.empty_cache()
         if a.workload == "moe_decode_bs1":
+            # the same step on ONE layer replayed: its 16 MB stay in the caches, so this is the step without
+            # HBM in the way (launch, selection and dependency chain) beside the ring's figure above
+            mh = moe_workload(qk, 1, qk.IQ4_XS, 1, 400, 40)
+            ex["moe_decode_bs1_cache_hot"] = dict(us=mh["ms_event"] * 1e3, steps_timed=mh["steps"],
+                                                  stage_us={k: v * 1e3 for k, v in mh["stage_ms"].items()})
+            log(f"[bench] moe bs1, one layer replayed: {ex['moe_decode_bs1_cache_hot']}")
+            torch.cuda.empty_cache()
             m16 = moe_workload(qk, 16, qk.Q6_K, 4, 200, 20)
             ex["moe_decode_bs16_q6k_down"] = dict(us=m16["ms_event"] * 1e3, distinct_experts=m16["distinct_experts"],
                                                   gbps=m16["bytes_step"] / (m16["ms_event"] * 1e-3) / 1e9,

@@ -107,6 +107,14 @@ int qko_group_pairs(const qko_sel *sel, uint32_t n_tokens, uint32_t n_expert, ui
 /* Y[n][m] = sum_k X[n][k] * dequant_q8_0(W[m])[k] in double (src/main.cpp:5561-5570). */
 int qko_gemm_q8_0(const void *W, const float *X, float *Y, uint32_t M, uint32_t K, uint32_t N);
 
+/* The same row loops on n_threads host threads (qk_oracle_mt.c): bit for bit the results of the
+ * single-threaded functions above; for the benchmark's all-cores CPU baseline. */
+int qko_gemv_mt(int type, const void *W, const float *x, float *y, uint32_t M, uint32_t K, uint32_t batch,
+                uint32_t n_threads);
+int qko_gemm_q8_0_mt(const void *W, const float *X, float *Y, uint32_t M, uint32_t K, uint32_t N, uint32_t n_threads);
+int qko_moe_ref_mt(const qko_moe_layer *L, const float *x, float *y, uint32_t n_threads);
+int qko_moe_ref_tokens_mt(const qko_moe_layer *L, const float *X, float *Y, uint32_t n_tokens, uint32_t n_threads);
+
 /* Scale-aware acceptance metric of the CLI self checks (src/main.cpp:548-565):
  * max over i of |got-ref| / max(|ref|, max(1e-3, 1e-3*rms(ref))). */
 double qko_max_rel_err(const float *got, const float *ref, size_t n);

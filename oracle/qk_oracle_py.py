@@ -55,6 +55,10 @@ def lib():
         L.qko_moe_ref.argtypes = [vp, vp, vp, vp, vp, vp]
         L.qko_group_pairs.argtypes = [vp, u32, u32, u32, vp, vp]
         L.qko_gemm_q8_0.argtypes = [vp, vp, vp, u32, u32, u32]
+        L.qko_gemv_mt.argtypes = [C.c_int, vp, vp, vp, u32, u32, u32, u32]
+        L.qko_gemm_q8_0_mt.argtypes = [vp, vp, vp, u32, u32, u32, u32]
+        L.qko_moe_ref_mt.argtypes = [vp, vp, vp, u32]
+        L.qko_moe_ref_tokens_mt.argtypes = [vp, vp, vp, u32, u32]
         L.qko_max_rel_err.restype = C.c_double
         L.qko_max_rel_err.argtypes = [vp, vp, C.c_size_t]
         L.qko_max_err_over_rms.restype = C.c_double
@@ -112,12 +116,16 @@ def dequant(type_, raw, n_elems, use_ref=False):
     return out
 
 
-def gemv(type_, W, x, M, K):
+def gemv(type_, W, x, M, K, threads=1):
+    """threads > 1: the rows split over host threads (bit for bit the same result)."""
     W = np.ascontiguousarray(W).reshape(-1)
     x = np.ascontiguousarray(x, dtype=np.float32)
     batch = 1 if x.ndim == 1 else x.shape[0]
     y = np.empty((batch, M), dtype=np.float32)
-    rc = lib().qko_gemv(type_, _p(W), _p(x), _p(y), M, K, batch)
+    if threads > 1:
+        rc = lib().qko_gemv_mt(type_, _p(W), _p(x), _p(y), M, K, batch, threads)
+    else:
+        rc = lib().qko_gemv(type_, _p(W), _p(x), _p(y), M, K, batch)
     if rc:
         raise ValueError(f"gemv rc={rc}")
     return y if x.ndim == 2 else y[0]
@@ -194,6 +202,22 @@ def moe_ref(h, x, want_h=False, want_logits=False):
     return dict(y=y, sel=sel, h=hbuf, logits=lbuf)
 
 
+def moe_ref_threads(h, X, threads):
+    """y of the fused step for the rows of X on `threads` host threads: one row -> the row loops of
+    the step are split; several rows -> the rows are (each a single-threaded step).  Bit for bit
+    moe_ref()["y"]."""
+    L = make_layer(h)
+    X = np.ascontiguousarray(X, dtype=np.float32).reshape(-1, h.n_embd)
+    Y = np.empty_like(X)
+    if X.shape[0] == 1:
+        rc = lib().qko_moe_ref_mt(C.byref(L), _p(X), _p(Y), threads)
+    else:
+        rc = lib().qko_moe_ref_tokens_mt(C.byref(L), _p(X), _p(Y), X.shape[0], threads)
+    if rc:
+        raise ValueError(f"moe_ref_mt rc={rc}")
+    return Y
+
+
 def group_pairs(sel_bytes, n_tokens, n_expert, n_used):
     """sel_bytes: uint8 [n_tokens, 160] of Sel records."""
     sel_bytes = np.ascontiguousarray(sel_bytes)
@@ -205,11 +229,14 @@ def group_pairs(sel_bytes, n_tokens, n_expert, n_used):
     return offsets, pairs
 
 
-def gemm_q8_0(W, X, M, K):
+def gemm_q8_0(W, X, M, K, threads=1):
     W = np.ascontiguousarray(W).reshape(-1)
     X = np.ascontiguousarray(X, dtype=np.float32)
     Y = np.empty((X.shape[0], M), dtype=np.float32)
-    rc = lib().qko_gemm_q8_0(_p(W), _p(X), _p(Y), M, K, X.shape[0])
+    if threads > 1:
+        rc = lib().qko_gemm_q8_0_mt(_p(W), _p(X), _p(Y), M, K, X.shape[0], threads)
+    else:
+        rc = lib().qko_gemm_q8_0(_p(W), _p(X), _p(Y), M, K, X.shape[0])
     if rc:
         raise ValueError(f"gemm rc={rc}")
     return Y

@@ -8,6 +8,7 @@
 #include "qk_coop.h"
 #include "qk_device.h"
 #include "qk_host.h"
+#include "qk_stream.h"
 
 #include <algorithm>
 
@@ -50,70 +51,77 @@ __device__ static uint32_t fold_candidates(const volatile float* cv, const volat
     return s_i[0] == 0xFFFFFFFFu ? 0u : s_i[0];
 }
 
-template <int PASSES, int RIF>
+// One activation row: the Q6_K rows are streamed as in the GEMV (qk_stream.h: chunks of RPC rows as
+// 16-byte pieces through the wave's LDS area, the next chunk in flight during the arithmetic), and a
+// wave keeps the best (logit, id) of its rows, which ascend, so a strict '>' keeps the lowest id.
+// The vocabulary's rows behind the last full chunk are fetched per lane.
+template <int PASSES, int RPC>
 __global__ __launch_bounds__(256) void head_q6k_kernel(const uint8_t* __restrict__ W,
                                                        const float* __restrict__ X,
                                                        float* __restrict__ logits_out,
-                                                       uint32_t* __restrict__ tok, HeadWs ws, uint32_t V,
-                                                       uint32_t K, uint32_t row_bytes)
+                                                       uint32_t* __restrict__ tok, HeadWs ws, uint32_t V)
 {
+    constexpr uint32_t K = 2048u * PASSES, RB = (uint32_t)qkk_row_bytes_dev<QKK_Q6_K>(K), PB = RB / PASSES;
+    constexpr uint32_t CB = RPC * RB, NPC = CB / 16;
+    constexpr int NP = (NPC + 63) / 64;
+    static_assert(CB % 16 == 0, "a chunk of rows must be whole 16-byte pieces");
+    __shared__ __attribute__((aligned(16))) uint8_t s_stage[4][WaveStage<NP>::AREA + 16];
     __shared__ float s_v[256];
     __shared__ uint32_t s_i[256];
     __shared__ uint32_t s_last;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t b = blockIdx.y;
     const float* x = X + (size_t)b * K;
+    const uint32_t n_full = V / RPC, stride = gridDim.x * 4;
+    uint32_t c = blockIdx.x * 4 + wave;
 
+    WaveStage<NP> st;
+    if (c < n_full) st.fetch(W + (size_t)c * CB, NPC, lane);
     XSlice xs[PASSES];
     float xsum[PASSES][4];
 #pragma unroll
     for (int p = 0; p < PASSES; p++) {
         load_xslice<QKK_Q6_K>(xs[p], x + p * 2048, lane);
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            float s = 0.f;
+        for (int q = 0; q < 4; q++) {
+            float t = 0.f;
 #pragma unroll
-            for (int i = 0; i < 8; i++) s += xs[p].v[c * 8 + i];
-            xsum[p][c] = s;
+            for (int i = 0; i < 8; i++) t += xs[p].v[q * 8 + i];
+            xsum[p][q] = t;
         }
     }
-    const uint32_t pass_bytes = row_bytes / PASSES;
     float bv = ARG_FLOOR;
     uint32_t bi = 0xFFFFFFFFu;
-    // chunks of RIF rows dealt round-robin to the waves; a wave's rows ascend.  The next
-    // chunk's loads are issued before the arithmetic of the current one.
-    const uint32_t stride = gridDim.x * 4 * RIF;
-    LaneW<QKK_Q6_K> w[2][RIF][PASSES];
-    auto fetch = [&](int set, uint32_t r0) {
+    auto take = [&](const LaneW<QKK_Q6_K> (&w)[PASSES], uint32_t r) {
+        float acc = 0.f;
 #pragma unroll
-        for (int i = 0; i < RIF; i++) {
-            const uint32_t r = min(r0 + i, V - 1);
-#pragma unroll
-            for (int p = 0; p < PASSES; p++)
-                w[set][i][p].load(W + (size_t)r * row_bytes + (size_t)p * pass_bytes, lane);
+        for (int p = 0; p < PASSES; p++) acc += w[p].dot(xs[p], xsum[p], nullptr, lane);
+        acc = wave_sum(acc);
+        if (r < V) {
+            if (logits_out && lane == 0) logits_out[(size_t)b * V + r] = acc;
+            if (acc > bv) { bv = acc; bi = r; }
         }
     };
-    auto reduce = [&](int set, uint32_t r0) {
+    uint8_t* area = s_stage[wave];
+    vmem_drain(); // the activations are here: no wait for them inside the loop, behind the next chunk's loads
+    for (; c < n_full; c += stride) {
+        st.commit(area, lane);
+        const uint32_t cn = c + stride;
+        if (cn < n_full) st.fetch(W + (size_t)cn * CB, NPC, lane);
 #pragma unroll
-        for (int i = 0; i < RIF; i++) {
-            float acc = 0.f;
+        for (int r = 0; r < RPC; r++) {
+            LaneW<QKK_Q6_K> w[PASSES];
 #pragma unroll
-            for (int p = 0; p < PASSES; p++) acc += w[set][i][p].dot(xs[p], xsum[p], nullptr, lane);
-            acc = wave_sum(acc);
-            const uint32_t r = r0 + i;
-            if (r < V) {
-                if (logits_out && lane == 0) logits_out[(size_t)b * V + r] = acc;
-                if (acc > bv) { bv = acc; bi = r; } // rows ascend: strict '>' keeps the lowest id
-            }
+            for (int p = 0; p < PASSES; p++) lane_load_lds<QKK_Q6_K>(w[p], area, r * RB + p * PB, lane);
+            take(w, c * RPC + r);
         }
-    };
-    uint32_t r0 = (blockIdx.x * 4 + wave) * RIF;
-    fetch(0, r0);
-    for (; r0 < V; r0 += 2 * stride) {
-        fetch(1, r0 + stride);
-        reduce(0, r0);
-        fetch(0, r0 + 2 * stride);
-        reduce(1, r0 + stride);
+    }
+    // rows behind the last full chunk (they are the highest ids: still ascending for the wave that takes them last)
+    for (uint32_t r = n_full * RPC + blockIdx.x * 4 + wave; r < V; r += stride) {
+        LaneW<QKK_Q6_K> w[PASSES];
+#pragma unroll
+        for (int p = 0; p < PASSES; p++) w[p].load(W + (size_t)r * RB + (size_t)p * PB, lane);
+        take(w, r);
     }
 
     // fold the four waves of the block
@@ -270,15 +278,15 @@ __global__ __launch_bounds__(CT) void head_q6k_coop_kernel(const uint8_t* __rest
     }
 }
 
-// Persistent grid of the one-row kernel.  Measured on the 151,936-row head (two rows in flight per
-// wave, double-buffered): 256 workgroups 65.0 us, 512: 60.0, 768: 62.4, 1024: 63.2, and grids that
-// are not a multiple of the CU count lose 5 us more; four rows in flight (133 VGPRs) 68.3 us.
-static uint32_t head_blocks(uint32_t V, uint32_t rif)
+// Grid of the one-row kernel: one chunk per wave for a small vocabulary, else a persistent grid eight
+// workgroups deep per CU (16 KB of LDS each), the depth at which the same streaming loop read Q6_K
+// fastest as a plain GEMV.
+constexpr uint32_t HEAD_RPC = 2, HEAD_DEPTH = 8;
+static uint32_t head_blocks(uint32_t V, uint32_t rpc)
 {
-    const uint32_t waves = (V + rif - 1) / rif;
-    return std::min((waves + 3) / 4, persistent_blocks() / 2);
+    const uint32_t waves = std::max(V / rpc, V % rpc);
+    return std::max(1u, std::min((waves + 3) / 4, persistent_blocks() / 4 * HEAD_DEPTH));
 }
-constexpr uint32_t HEAD_RIF = 2;
 
 } // namespace qk
 
@@ -323,19 +331,17 @@ int qkk_head_argmax(const void* W, const float* X, uint32_t* tok, float* logits,
                            logits, tok, ws, V, batch);
         return check_launch("qkk_head_argmax");
     }
-    const uint32_t rif = K == 2048 ? HEAD_RIF : 2;
-    const uint32_t blocks = head_blocks(V, rif);
+    const uint32_t blocks = head_blocks(V, K == 2048 ? HEAD_RPC : 1);
     HeadWs ws;
     ws.counter = (uint32_t*)workspace;
     ws.cand_v = (float*)((uint8_t*)workspace + 256);
     ws.cand_i = (uint32_t*)(ws.cand_v + (size_t)batch * blocks);
-    const uint32_t rb = (uint32_t)qkk_row_bytes(QKK_Q6_K, K);
     if (K == 2048)
-        hipLaunchKernelGGL((head_q6k_kernel<1, HEAD_RIF>), dim3(blocks, batch), dim3(256), 0, st, (const uint8_t*)W,
-                           X, logits, tok, ws, V, K, rb);
+        hipLaunchKernelGGL((head_q6k_kernel<1, HEAD_RPC>), dim3(blocks, batch), dim3(256), 0, st, (const uint8_t*)W,
+                           X, logits, tok, ws, V);
     else
-        hipLaunchKernelGGL((head_q6k_kernel<2, 2>), dim3(blocks, batch), dim3(256), 0, st, (const uint8_t*)W, X,
-                           logits, tok, ws, V, K, rb);
+        hipLaunchKernelGGL((head_q6k_kernel<2, 1>), dim3(blocks, batch), dim3(256), 0, st, (const uint8_t*)W, X,
+                           logits, tok, ws, V);
     return check_launch("qkk_head_argmax");
 }
 

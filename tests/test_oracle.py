@@ -408,3 +408,27 @@ def test_embed_is_dequant_of_the_chosen_rows(orc, qk):
             assert np.array_equal(got[r].view(np.uint32), want.view(np.uint32))
     with pytest.raises(ValueError):
         orc.embed(qk.Q8_0, W, V, K, np.array([V], dtype=np.uint32), 0, 1, 1)
+
+
+def test_threaded_row_loops_give_the_single_thread_bits(qk, orc):
+    """The all-cores CPU baseline of the benchmark runs the oracle's row loops on several host
+    threads; every output element is still computed by one thread with the same scalar code, so
+    the results are the single-threaded ones bit for bit (ragged splits included)."""
+    rng = np.random.default_rng(21)
+    for t, name in ((orc.Q8_0, "q8_0"), (orc.Q6_K, "q6_k"), (orc.IQ4_XS, "iq4_xs"), (orc.IQ3_XXS, "iq3_xxs")):
+        W = qk.synth.tensor_host(t, 37, 512, seed=3)
+        x = rng.standard_normal((3, 512)).astype(np.float32)
+        for nt in (2, 5, 64):
+            assert np.array_equal(orc.gemv(t, W, x, 37, 512, threads=nt).view(np.uint32),
+                                  orc.gemv(t, W, x, 37, 512).view(np.uint32)), (name, nt)
+            assert np.array_equal(orc.gemv(t, W, x[0], 37, 512, threads=nt).view(np.uint32),
+                                  orc.gemv(t, W, x[0], 37, 512).view(np.uint32)), (name, nt)
+    W = qk.synth.tensor_host(orc.Q8_0, 19, 256, seed=4)
+    X = rng.standard_normal((5, 256)).astype(np.float32)
+    assert np.array_equal(orc.gemm_q8_0(W, X, 19, 256, threads=3).view(np.uint32), orc.gemm_q8_0(W, X, 19, 256).view(np.uint32))
+    for down in (orc.IQ4_XS, orc.Q6_K):
+        hl = qk.synth.HostLayer(seed=8, n_ff=256, n_expert=8, n_used=3, down_type=down)
+        X = rng.standard_normal((4, 2048)).astype(np.float32)
+        want = np.stack([orc.moe_ref(hl, X[r])["y"] for r in range(4)])
+        assert np.array_equal(orc.moe_ref_threads(hl, X, 3).view(np.uint32), want.view(np.uint32))
+        assert np.array_equal(orc.moe_ref_threads(hl, X[:1], 7).view(np.uint32), want[:1].view(np.uint32))
