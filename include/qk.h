@@ -12,8 +12,8 @@
  *     (gated DeltaNet where "ssm_a" is present, else full attention) + post_attention_norm + the
  *     eight MoE tensors, output_norm, Q6_K head; head shapes as in the reference engine (DeltaNet
  *     32 value / 16 key heads of 128, attention 16 x 256 query heads on 2 KV heads, n_embd 2048);
- *     dense projections Q8_0 or IQ4_XS; ssm_alpha / ssm_beta as separate F32 tensors (the fused
- *     ssm_ba form is refused);
+ *     dense projections Q8_0 or IQ4_XS; ssm_alpha / ssm_beta as separate F32 tensors, or fused as
+ *     ssm_ba (F32, Q8_0 or IQ4_XS; reference src/main.cpp:3931-3948): split on the device at open);
  *   - a GGUF whose layers are MoE blocks only (no mixer tensors at all).
  * Every entry point behaves as the reference's: argument checks and return codes, the serial-step
  * state machine of qk_step_chunk (one captured hipGraph per dispatch depth), greedy sampling,

@@ -98,6 +98,14 @@ int qkk_dequant(int type, const void *W, float *out, uint64_t n_elems, void *str
 int qkk_gemv(int type, const void *W, const float *X, float *Y, uint32_t M, uint32_t K,
              uint32_t batch, void *stream);
 
+/* The same product with the RMS norm of the activation row in front and no launch of its own:
+ * Y[b][m] = W[m] . (X[b] * w_norm / sqrt(mean(X[b]^2) + eps)).  Stands for rmsnorm.comp followed by the
+ * gemv_*.comp dispatches that read the normalised row (reference src/main.cpp:4307-4335: attn_norm, then
+ * the mixer's input projections).  Quantised block formats, K = 2048, batch <= 16 (one pass over the
+ * weights per row). */
+int qkk_gemv_norm(int type, const void *W, const float *X, const float *w_norm, float eps, float *Y,
+                  uint32_t M, uint32_t K, uint32_t batch, void *stream);
+
 /* Workspace for qkk_moe_decode with up to n_slots slots. */
 size_t qkk_moe_workspace_bytes(const qkk_moe_layer *L_host, uint32_t n_slots);
 
@@ -120,6 +128,15 @@ size_t qkk_moe_workspace_bytes(const qkk_moe_layer *L_host, uint32_t n_slots);
  * it (matrix-core path); that path needs n_embd = 2048 and returns QKK_ESHAPE otherwise. */
 int qkk_moe_decode(const qkk_moe_layer *L_host, const float *X, float *Y, qkk_sel *sel,
                    void *workspace, size_t workspace_bytes, uint32_t n_slots, void *stream);
+
+/* Waits for `stream` and says whether a routing launch since the last such call found a workspace whose
+ * header was not zero -- never cleared, or cleared on another stream that had not finished: with more
+ * than QKK_ROWWISE_MAX rows the step then counts its workgroups' arrivals from garbage, and its results
+ * are invalid (inside the tensors, but wrong).  QKK_OK, or QKK_EINVAL once per occurrence (the flag is
+ * per device and cleared by the call that reports it).  The reference's dispatches need no such state
+ * (a command buffer's barriers order them); this is the check for this library's one-time zero-fill
+ * contract.  Synchronises: for set-up code, tests and debug builds, not for a serving loop. */
+int qkk_moe_workspace_status(void *stream);
 
 /* qkk_moe_decode without a workspace argument, for callers that cannot allocate device memory (code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
@@ -199,6 +216,13 @@ size_t qkk_head_workspace_bytes(uint32_t V, uint32_t batch);
 int qkk_head_argmax(const void *W, const float *X, uint32_t *tok, float *logits, uint32_t V,
                     uint32_t K, uint32_t batch, void *workspace, size_t workspace_bytes,
                     void *stream);
+
+/* The same for ONE row with the output norm in front and no launch of its own: tok[0] = argmax_m
+ * W[m] . (X * w_norm / sqrt(mean(X^2) + eps)) (reference src/main.cpp:4406-4419: rmsnorm.comp with
+ * output_norm, then the head's GEMV and the argmax pair).  K = 2048. */
+int qkk_head_argmax_norm(const void *W, const float *X, const float *w_norm, float eps, uint32_t *tok,
+                         float *logits, uint32_t V, uint32_t K, void *workspace,
+                         size_t workspace_bytes, void *stream);
 
 /* Two-pass argmax over fp32 rows (reference shaders/argmax1.comp:17-40, argmax2.comp:16-30):
  * tok[b] = first index of the maximum of logits[b][0..n). */
@@ -307,6 +331,14 @@ int qkk_dn_ab_conv(const float *x, const float *alpha_w, const float *beta_w, co
                    const float *a_vec, float *gb, uint32_t n_embd, uint32_t hV, float *conv_state,
                    const float *qkv, const float *ker, float *out, uint32_t channels, uint32_t d_state,
                    uint32_t qk_channels, float eps, uint32_t n_slots, void *stream);
+/* qkk_dn_ab_conv with x the residual row: the RMS norm in front of the mixer (weights w_norm, norm_eps)
+ * is applied to x on the way into the alpha / beta dot products (n_embd 2048), so a one-row decode step
+ * needs no norm launch (the projections that feed qkv take the norm the same way: qkk_gemv_norm). */
+int qkk_dn_ab_conv_norm(const float *x, const float *w_norm, float norm_eps, const float *alpha_w,
+                        const float *beta_w, const float *dt_bias, const float *a_vec, float *gb,
+                        uint32_t n_embd, uint32_t hV, float *conv_state, const float *qkv, const float *ker,
+                        float *out, uint32_t channels, uint32_t d_state, uint32_t qk_channels, float eps,
+                        uint32_t n_slots, void *stream);
 int qkk_dn_step(const float *conv, const float *gb, float *state, const float *norm_w, const float *z,
                 float *att, uint32_t d_state, uint32_t hK, uint32_t hV, uint32_t kdiv, float eps,
                 uint32_t n_slots, void *stream);

@@ -121,16 +121,18 @@ class SlotMachine:
         return active_at_entry, out, fin
 
 
-def stack_next(model, token, eps=1e-6, want_margin=False):
+def stack_next(model, token, eps=1e-6, want_margin=False, threads=1):
     """Next greedy token of a MoE-only model (an object with embd, embd_type, vocab, layers,
-    post_norm, out_norm, head, as qwen-kernel_amd's engine.StackModel) after `token`."""
+    post_norm, out_norm, head, as qwen-kernel_amd's engine.StackModel) after `token`.  `threads`
+    splits the row loops of the step over host threads (the same bits)."""
     H = 2048
     x = O.embed(model.embd_type, model.embd, model.vocab, H, np.array([token], dtype=np.uint32), 0, 1, 1)[0]
     for l, hl in enumerate(model.layers):
         xn = O.add_rms(x, model.post_norm[l], eps)
-        x = (x + O.moe_ref(hl, xn)["y"]).astype(np.float32)
+        y = O.moe_ref(hl, xn)["y"] if threads <= 1 else O.moe_ref_threads(hl, xn[None, :], threads)[0]
+        x = (x + y).astype(np.float32)
     xn = O.add_rms(x, model.out_norm, eps)
-    logits = O.gemv(O.Q6_K, model.head, xn, model.vocab, H)
+    logits = O.gemv(O.Q6_K, model.head, xn, model.vocab, H, threads=threads)
     best = O.argmax(logits)
     if want_margin:
         srt = np.sort(logits.astype(np.float64))

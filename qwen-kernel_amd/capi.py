@@ -51,14 +51,17 @@ def _signatures():
         "qkk_device_info": (None, [C.c_char_p, sz, C.POINTER(u32)]),
         "qkk_dequant": (None, [i32, vp, vp, u64, vp]),
         "qkk_gemv": (None, [i32, vp, vp, vp, u32, u32, u32, vp]),
+        "qkk_gemv_norm": (None, [i32, vp, vp, vp, f32, vp, u32, u32, u32, vp]),
         "qkk_moe_decode": (None, [vp, vp, vp, vp, vp, sz, u32, vp]),
         "qkk_moe_decode_static": (None, [vp, vp, vp, vp, u32, vp]),
+        "qkk_moe_workspace_status": (None, [vp]),
         "qkk_moe_decode_stages": (None, [vp, vp, vp, vp, vp, sz, u32, u32, vp]),
         "qkk_moe_decode_tail": (None, [vp, vp, vp, vp, f32, vp, vp, vp, vp, sz, u32, vp]),
         "qkk_moe_layer_rows": (None, [vp, vp, vp, f32, vp, vp, sz, u32, vp]),
         "qkk_moe_layer_rows_add": (None, [vp, vp, vp, vp, vp, f32, vp, vp, sz, u32, vp]),
         "qkk_moe_group_pairs": (None, [vp, u32, u32, u32, vp, vp, vp]),
         "qkk_head_argmax": (None, [vp, vp, vp, vp, u32, u32, u32, vp, sz, vp]),
+        "qkk_head_argmax_norm": (None, [vp, vp, vp, f32, vp, vp, u32, u32, vp, sz, vp]),
         "qkk_argmax": (None, [vp, vp, u32, u32, vp]),
         "qkk_gemm_q8_0": (None, [vp, vp, vp, u32, u32, u32, vp]),
         "qkk_moe_prefill": (None, [vp, vp, vp, vp, vp, sz, u32, vp]),
@@ -73,6 +76,7 @@ def _signatures():
         "qkk_dn_step": (None, dn_step),
         "qkk_dn_step_seq": (None, dn_step),
         "qkk_dn_ab_conv": (None, [vp] * 6 + [u32, u32] + [vp] * 4 + [u32] * 3 + [f32, u32, vp]),
+        "qkk_dn_ab_conv_norm": (None, [vp, vp, f32] + [vp] * 5 + [u32, u32] + [vp] * 4 + [u32] * 3 + [f32, u32, vp]),
         "qkk_rope_table": (None, [vp, u32, u32, f32]),
         "qkk_attn_prep": (None, attn_prep),
         "qkk_attn_prep_seq": (None, attn_prep),
@@ -150,6 +154,16 @@ def gemv(type_, W, X, M, K, out=None):
     return out if X.dim() == 2 else out[0]
 
 
+def gemv_norm(type_, W, X, w_norm, M, K, eps=1e-6, out=None):
+    """Y[b][m] = W[m] . rmsnorm(X[b]) * w_norm, the norm applied inside the launch."""
+    import torch
+    batch = 1 if X.dim() == 1 else X.shape[0]
+    if out is None:
+        out = torch.empty((batch, M), dtype=torch.float32, device=X.device)
+    _check(lib().qkk_gemv_norm(type_, _ptr(W), _ptr(X), _ptr(w_norm), eps, _ptr(out), M, K, batch, _stream()))
+    return out if X.dim() == 2 else out[0]
+
+
 class MoeLayer:
     """Device tensors of one MoE layer plus the C struct that names them."""
 
@@ -199,6 +213,12 @@ def moe_decode(layer, X, workspace, Y=None, sel=None, stages=None):
 
 MOE_STATIC_MAX_SLOTS = 16        # QKK_MOE_STATIC_MAX_SLOTS
 MOE_STATIC_BYTES = 2 << 20       # QKK_MOE_STATIC_BYTES
+
+
+def moe_workspace_status():
+    """Waits for the current stream; raises QkError (QKK_EINVAL) if a routing launch since the last such
+    call found a workspace header that was not zero."""
+    _check(lib().qkk_moe_workspace_status(_stream()))
 
 
 def moe_decode_static(layer, X, Y, sel):
@@ -283,6 +303,16 @@ def head_argmax(W, X, V, K, workspace, want_logits=False):
     logits = torch.empty((batch, V), dtype=torch.float32, device=X.device) if want_logits else None
     _check(lib().qkk_head_argmax(_ptr(W), _ptr(X), _ptr(tok), _ptr(logits), V, K, batch, _ptr(workspace),
                                  workspace.numel() * workspace.element_size(), _stream()))
+    return tok, logits
+
+
+def head_argmax_norm(W, X, w_norm, V, K, workspace, eps=1e-6, want_logits=False):
+    """The head for ONE row X [1, K] with the output norm (weights w_norm) applied inside the launch."""
+    import torch
+    tok = torch.empty(1, dtype=torch.int32, device=X.device)
+    logits = torch.empty((1, V), dtype=torch.float32, device=X.device) if want_logits else None
+    _check(lib().qkk_head_argmax_norm(_ptr(W), _ptr(X), _ptr(w_norm), eps, _ptr(tok), _ptr(logits), V, K, _ptr(workspace),
+                                      workspace.numel() * workspace.element_size(), _stream()))
     return tok, logits
 
 
@@ -413,15 +443,21 @@ def dn_ab(x, alpha_w, beta_w, dt_bias, a_vec, gb=None):
     return gb
 
 
-def dn_ab_conv(x, alpha_w, beta_w, dt_bias, a_vec, conv_state, qkv, ker, qk_channels, d_state=128, eps=1e-6):
+def dn_ab_conv(x, alpha_w, beta_w, dt_bias, a_vec, conv_state, qkv, ker, qk_channels, d_state=128, eps=1e-6,
+               w_norm=None, norm_eps=1e-6):
     """dn_ab and dn_conv in one launch.  Returns (gb [slots][2*hV], out [slots][channels]); conv_state is
-    updated in place."""
+    updated in place.  w_norm: x is the residual row, its RMS norm is applied inside the launch."""
     import torch
     n, hV, channels = x.shape[0], alpha_w.shape[0], qkv.shape[1]
     if qkv.shape[0] != n or conv_state.numel() != n * channels * 3:
         raise ValueError("dn_ab_conv: shapes do not match the rows")
     gb = torch.empty((n, 2 * hV), dtype=torch.float32, device=x.device)
     out = torch.empty_like(qkv)
+    if w_norm is not None:
+        _check(lib().qkk_dn_ab_conv_norm(_ptr(x), _ptr(w_norm), norm_eps, _ptr(alpha_w), _ptr(beta_w), _ptr(dt_bias),
+                                         _ptr(a_vec), _ptr(gb), x.shape[1], hV, _ptr(conv_state), _ptr(qkv), _ptr(ker),
+                                         _ptr(out), channels, d_state, qk_channels, eps, n, _stream()))
+        return gb, out
     _check(lib().qkk_dn_ab_conv(_ptr(x), _ptr(alpha_w), _ptr(beta_w), _ptr(dt_bias), _ptr(a_vec), _ptr(gb), x.shape[1], hV,
                                 _ptr(conv_state), _ptr(qkv), _ptr(ker), _ptr(out), channels, d_state, qk_channels, eps, n,
                                 _stream()))

@@ -84,13 +84,16 @@ __global__ __launch_bounds__(128) void dn_conv_kernel(float* __restrict__ st, co
 // of 3-5 us each are mostly launch ramp): grid (channels / dS + hV, slots), 128 threads.  Workgroups
 // below channels / dS run the conv of one head exactly as dn_conv_kernel; the others form two outputs
 // of dn_ab each (one per wave: g of head b and beta of head b), exactly as dn_ab_kernel.
-template <int NCH>
+// NORM: x is the residual row and its RMS norm (weights nw) is applied on the way in -- a wave holds
+// the whole row, so the mean square is one cross-lane sum and the two dot products are scaled by it.
+template <int NCH, bool NORM = false>
 __global__ __launch_bounds__(128) void dn_ab_conv_kernel(float* __restrict__ st, const float* __restrict__ qkv,
                                                          const float* __restrict__ ker, float* __restrict__ out,
                                                          uint32_t channels, uint32_t qk_channels, float eps,
                                                          const float* __restrict__ x, const float* __restrict__ alpha_w,
                                                          const float* __restrict__ beta_w, const float* __restrict__ dt_bias,
-                                                         const float* __restrict__ a_vec, float* __restrict__ gb, uint32_t hV)
+                                                         const float* __restrict__ a_vec, float* __restrict__ gb, uint32_t hV,
+                                                         const float* __restrict__ nw, float norm_eps)
 {
     __shared__ float s_red[2];
     const uint32_t rq = blockIdx.y, conv_blocks = channels / DN_DS;
@@ -115,13 +118,24 @@ __global__ __launch_bounds__(128) void dn_ab_conv_kernel(float* __restrict__ st,
     for (int i = 0; i < NCH; i++) a[i] = row[lane + 64 * i];
 #pragma unroll
     for (int i = 0; i < NCH; i++) b[i] = xv[lane + 64 * i];
+    float scale = 1.f;
+    if constexpr (NORM) {
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const float4 g = ((const float4*)nw)[lane + 64 * i];
+            ss += (b[i].x * b[i].x + b[i].y * b[i].y) + (b[i].z * b[i].z + b[i].w * b[i].w);
+            b[i] = float4{b[i].x * g.x, b[i].y * g.y, b[i].z * g.z, b[i].w * g.w};
+        }
+        scale = 1.f / sqrtf(wave_sum(ss) / (float)(256 * NCH) + norm_eps);
+    }
     float p0 = 0.f, p1 = 0.f;
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
         p0 += a[i].x * b[i].x + a[i].y * b[i].y;
         p1 += a[i].z * b[i].z + a[i].w * b[i].w;
     }
-    const float d = wave_sum(p0 + p1);
+    const float d = wave_sum(p0 + p1) * scale;
     if (lane == 0) {
         if (is_beta) {
             gb[(size_t)rq * 2 * hV + hV + h] = 1.f / (1.f + expf(-d));
@@ -425,9 +439,10 @@ int qkk_dn_conv(float* conv_state, const float* qkv, const float* ker, float* ou
     return check_launch("qkk_dn_conv");
 }
 
-int qkk_dn_ab_conv(const float* x, const float* alpha_w, const float* beta_w, const float* dt_bias, const float* a_vec,
-                   float* gb, uint32_t n_embd, uint32_t hV, float* conv_state, const float* qkv, const float* ker, float* out,
-                   uint32_t channels, uint32_t d_state, uint32_t qk_channels, float eps, uint32_t n_slots, void* stream)
+static int dn_ab_conv_impl(const float* x, const float* w_norm, float norm_eps, const float* alpha_w, const float* beta_w,
+                           const float* dt_bias, const float* a_vec, float* gb, uint32_t n_embd, uint32_t hV,
+                           float* conv_state, const float* qkv, const float* ker, float* out, uint32_t channels,
+                           uint32_t d_state, uint32_t qk_channels, float eps, uint32_t n_slots, void* stream)
 {
     if (!x || !alpha_w || !beta_w || !dt_bias || !a_vec || !gb || !conv_state || !qkv || !ker || !out)
         return fail(QKK_EINVAL, "qkk_dn_ab_conv: null pointer");
@@ -444,13 +459,36 @@ int qkk_dn_ab_conv(const float* x, const float* alpha_w, const float* beta_w, co
     if (!(eps >= 0.f)) return fail(QKK_EINVAL, "qkk_dn_ab_conv: eps must be non-negative");
     if (int rc = require_device()) return rc;
     const dim3 grid(channels / DN_DS + hV, n_slots), block(DN_DS);
-    if (n_embd == 2048)
+    if (w_norm) {
+        if (n_embd != 2048) return fail(QKK_ESHAPE, "qkk_dn_ab_conv_norm: n_embd %u not supported (2048)", n_embd);
+        hipLaunchKernelGGL((dn_ab_conv_kernel<8, true>), grid, block, 0, as_stream(stream), conv_state, qkv, ker, out, channels,
+                           qk_channels, eps, x, alpha_w, beta_w, dt_bias, a_vec, gb, hV, w_norm, norm_eps);
+    } else if (n_embd == 2048)
         hipLaunchKernelGGL(dn_ab_conv_kernel<8>, grid, block, 0, as_stream(stream), conv_state, qkv, ker, out, channels,
-                           qk_channels, eps, x, alpha_w, beta_w, dt_bias, a_vec, gb, hV);
+                           qk_channels, eps, x, alpha_w, beta_w, dt_bias, a_vec, gb, hV, (const float*)nullptr, 0.f);
     else
         hipLaunchKernelGGL(dn_ab_conv_kernel<16>, grid, block, 0, as_stream(stream), conv_state, qkv, ker, out, channels,
-                           qk_channels, eps, x, alpha_w, beta_w, dt_bias, a_vec, gb, hV);
+                           qk_channels, eps, x, alpha_w, beta_w, dt_bias, a_vec, gb, hV, (const float*)nullptr, 0.f);
     return check_launch("qkk_dn_ab_conv");
+}
+
+int qkk_dn_ab_conv(const float* x, const float* alpha_w, const float* beta_w, const float* dt_bias, const float* a_vec,
+                   float* gb, uint32_t n_embd, uint32_t hV, float* conv_state, const float* qkv, const float* ker, float* out,
+                   uint32_t channels, uint32_t d_state, uint32_t qk_channels, float eps, uint32_t n_slots, void* stream)
+{
+    return dn_ab_conv_impl(x, nullptr, 0.f, alpha_w, beta_w, dt_bias, a_vec, gb, n_embd, hV, conv_state, qkv, ker, out,
+                           channels, d_state, qk_channels, eps, n_slots, stream);
+}
+
+int qkk_dn_ab_conv_norm(const float* x, const float* w_norm, float norm_eps, const float* alpha_w, const float* beta_w,
+                        const float* dt_bias, const float* a_vec, float* gb, uint32_t n_embd, uint32_t hV,
+                        float* conv_state, const float* qkv, const float* ker, float* out, uint32_t channels,
+                        uint32_t d_state, uint32_t qk_channels, float eps, uint32_t n_slots, void* stream)
+{
+    if (!w_norm || !aligned16(w_norm)) return fail(QKK_EINVAL, "qkk_dn_ab_conv_norm: w_norm must be a 16-byte aligned pointer");
+    if (!(norm_eps >= 0.f)) return fail(QKK_EINVAL, "qkk_dn_ab_conv_norm: norm_eps must be non-negative");
+    return dn_ab_conv_impl(x, w_norm, norm_eps, alpha_w, beta_w, dt_bias, a_vec, gb, n_embd, hV, conv_state, qkv, ker, out,
+                           channels, d_state, qk_channels, eps, n_slots, stream);
 }
 
 int qkk_dn_conv_seq(float* conv_state, const float* qkv, const float* ker, float* out, uint32_t channels, uint32_t d_state,

@@ -104,6 +104,7 @@ struct qk_engine {
     uint32_t* h_pos = nullptr;   // pinned
     uint32_t pf_rows = 1024;     // positions of one slot a prefill pass carries (whole-model files; QK_PREFILL_ROWS)
     uint32_t cap = MAX_ROWS;     // rows the step's buffers hold (pf_rows for whole-model files)
+    bool cat_everywhere = false; // every layer's input projections lie back to back (one product per layer)
     uint32_t *d_pf = nullptr, *h_pf = nullptr; // [3][pf_rows] ids, positions, sampled ids of a prefill pass (device / pinned)
     float* d_rope = nullptr;     // [n_ctx][FA_ROT/2][2]
     float *d_big = nullptr, *d_mid = nullptr, *d_kin = nullptr, *d_vin = nullptr, *d_gb = nullptr, *d_conv = nullptr,
@@ -224,14 +225,21 @@ static int dense(const Dense& d, const float* x, float* y, uint32_t rows, hipStr
 //                attention is causal over the rows).
 int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool want_head, bool seq)
 {
-    if (rows < 1 || s0 >= MAX_ROWS || (seq ? rows > pf_rows : s0 + rows > MAX_ROWS)) return QKK_ESHAPE;
+    // the state stripes hold n_slots slots: no pass reaches behind them
+    if (rows < 1 || s0 >= n_slots || (seq ? rows > pf_rows : s0 + rows > n_slots)) return QKK_ESHAPE;
     float* x = d_x;
     const uint32_t* ids = seq ? d_pf : d_ids;
     const uint32_t* pos = seq ? d_pf + pf_rows : d_pos + s0;
     uint32_t* tok = seq ? d_pf + 2 * pf_rows : d_tok + s0;
     if (int rc = qkk_embed(embd_type, d_embd, embd_rows, N_EMBD, ids, seq ? pf_rows : MAX_ROWS, seq ? 0 : s0, 1, x, rows, st))
         return rc;
-    if (int rc = qkk_rmsnorm(x, layers[0].attn_norm, d_xn[0], N_EMBD, rows, eps, st)) return rc;
+    // One row of a decode step (no caller wants the normalised rows): no norm launches at all.  The
+    // consumers of a normalised row -- the input projections, the decay / write-strength products, the
+    // head -- take the residual row and the norm's weights and normalise on the way in; the MoE
+    // launches have done so all along.
+    const bool fuse = rows == 1 && !seq && !final_rows && cat_everywhere && !getenv("QK_NO_FUSED_NORM");
+    if (!fuse)
+        if (int rc = qkk_rmsnorm(x, layers[0].attn_norm, d_xn[0], N_EMBD, rows, eps, st)) return rc;
     int cur = 0;
     for (size_t l = 0; l < layers.size(); l++) {
         const EngineLayer& L = layers[l];
@@ -239,7 +247,9 @@ int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool 
         float *s1 = L.st1 + s0 * L.ps1, *s2 = L.st2 + s0 * L.ps2;
         // one row: the input projections as one product into d_big, their outputs back to back
         const bool one = rows == 1 && L.cat.w;
-        if (one)
+        if (fuse) {
+            if (int rc = qkk_gemv_norm(L.cat.type, L.cat.w, x, L.attn_norm, eps, d_big, L.cat.M, L.cat.K, 1, st)) return rc;
+        } else if (one)
             if (int rc = dense(L.cat, xn, d_big, 1, st)) return rc;
         if (L.kind == EngineLayer::RECURRENT) {
             float* d_mid = one ? d_big + DN_CH : this->d_mid;
@@ -255,8 +265,11 @@ int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool 
                     return rc;
             } else {
                 // decay / write strength and the conv in one launch
-                if (int rc = qkk_dn_ab_conv(xn, L.alpha_w, L.beta_w, L.dt_bias, L.a_vec, d_gb, N_EMBD, DN_HV, s1, d_big, L.ker,
-                                            d_conv, DN_CH, DN_DS, 2 * DN_HK * DN_DS, eps, rows, st))
+                if (int rc = fuse ? qkk_dn_ab_conv_norm(x, L.attn_norm, eps, L.alpha_w, L.beta_w, L.dt_bias, L.a_vec, d_gb, N_EMBD,
+                                                        DN_HV, s1, d_big, L.ker, d_conv, DN_CH, DN_DS, 2 * DN_HK * DN_DS, eps, rows,
+                                                        st)
+                                  : qkk_dn_ab_conv(xn, L.alpha_w, L.beta_w, L.dt_bias, L.a_vec, d_gb, N_EMBD, DN_HV, s1, d_big,
+                                                   L.ker, d_conv, DN_CH, DN_DS, 2 * DN_HK * DN_DS, eps, rows, st))
                     return rc;
                 if (int rc = qkk_dn_step(d_conv, d_gb, s2, L.ssm_norm, d_mid, d_att, DN_DS, DN_HK, DN_HV, dn_kdiv, eps, rows, st))
                     return rc;
@@ -292,7 +305,8 @@ int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool 
             // the next layer's norm
             if (int rc = qkk_moe_layer_rows_add(&L.moe, x, d_mix, xn, L.post_norm, eps, d_sel, d_ws, ws_bytes, rows, st))
                 return rc;
-            if (int rc = qkk_rmsnorm(x, w_next, d_xn[cur ^ 1], N_EMBD, rows, eps, st)) return rc;
+            if (!fuse)
+                if (int rc = qkk_rmsnorm(x, w_next, d_xn[cur ^ 1], N_EMBD, rows, eps, st)) return rc;
         } else {
             // y = x + mixer, normalised for the MoE block; then x = y + MoE, normalised for the next layer
             if (int rc = qkk_add_rmsnorm(x, d_mix, L.post_norm, x, xn, N_EMBD, rows, eps, st)) return rc;
@@ -303,6 +317,7 @@ int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool 
     }
     if (final_rows) *final_rows = d_xn[cur];
     if (!want_head) return QKK_OK;
+    if (fuse) return qkk_head_argmax_norm(d_head, x, d_onorm, eps, tok, nullptr, vocab, N_EMBD, d_hws, hws_bytes, st);
     for (uint32_t r0 = 0; r0 < rows; r0 += MAX_ROWS) // the head takes sixteen rows at a time
         if (int rc = qkk_head_argmax(d_head, d_xn[cur] + (size_t)r0 * N_EMBD, tok + r0, nullptr, vocab, N_EMBD,
                                      std::min(MAX_ROWS, rows - r0), d_hws, hws_bytes, st))
@@ -438,6 +453,41 @@ bool qk_engine::load_mixers(qkg_file* g, char* err, size_t err_len)
         L.cat.w = base; L.cat.type = ds[0]->type; L.cat.K = N_EMBD;
         return true;
     };
+    // qwen3next files hold alpha and beta as ONE tensor ssm_ba [n_embd, 2 * hV] (F32, Q8_0 or IQ4_XS),
+    // interleaved per key-head group g: rows 4g, 4g+1 are beta of the value heads 2g, 2g+1, rows 4g+2,
+    // 4g+3 their alpha (reference src/main.cpp:3931-3948, which dequantises on the host).  Here the
+    // tensor is uploaded as it is, dequantised on the device by the bit-exact kernel and its rows copied
+    // apart into the split layout the decay / write-strength kernel reads.
+    auto fused_ba = [&](uint32_t l, const float** alpha, const float** beta) {
+        qkg_tensor t;
+        if (!find(l, "ssm_ba.weight", &t) || t.ne[0] != N_EMBD || t.ne[1] != 2 * DN_HV || !t.nbytes)
+            return set_err(err, err_len, "qk_open: missing ssm_alpha/ssm_beta/ssm_ba");
+        if (t.type != QKK_F32 && t.type != QKK_Q8_0 && t.type != QKK_IQ4_XS)
+            return set_err(err, err_len, "qk_open: ssm_ba type unsupported");
+        const uint64_t n_el = 2ull * DN_HV * N_EMBD;
+        const void* raw = nullptr;
+        if (!upload(t, &raw, err, err_len)) return false;
+        const float* rows = (const float*)raw;
+        if (t.type != QKK_F32) {
+            float* deq = (float*)dev_alloc(n_el * sizeof(float), false);
+            if (!deq) return set_err(err, err_len, "qk_open: device memory exhausted");
+            if (qkk_dequant((int)t.type, raw, deq, n_el, st) != QKK_OK)
+                return set_err(err, err_len, "qk_open: ssm_ba dequantisation failed");
+            rows = deq;
+        }
+        float* al = (float*)dev_alloc((size_t)DN_HV * N_EMBD * sizeof(float), false);
+        float* be = (float*)dev_alloc((size_t)DN_HV * N_EMBD * sizeof(float), false);
+        if (!al || !be) return set_err(err, err_len, "qk_open: device memory exhausted");
+        for (uint32_t r = 0; r < 2 * DN_HV; r++) {
+            const uint32_t grp = r >> 2, sub = r & 3;
+            float* dst = (sub < 2 ? be : al) + ((size_t)grp * 2 + (sub & 1)) * N_EMBD;
+            if (hipMemcpyAsync(dst, rows + (size_t)r * N_EMBD, N_EMBD * sizeof(float), hipMemcpyDeviceToDevice, st) != hipSuccess)
+                return set_err(err, err_len, "qk_open: upload failed");
+        }
+        if (hipStreamSynchronize(st) != hipSuccess) return set_err(err, err_len, "qk_open: upload failed");
+        *alpha = al; *beta = be;
+        return true;
+    };
     for (uint32_t l = 0; l < n_layer; l++) {
         EngineLayer& L = layers[l];
         if (!f32(l, "attn_norm.weight", N_EMBD, &L.attn_norm)) return bad("qk_open: missing/unexpected attn_norm tensor");
@@ -445,9 +495,14 @@ bool qk_engine::load_mixers(qkg_file* g, char* err, size_t err_len)
             if (!proj_in(l, L, {{"attn_qkv.weight", DN_CH}, {"attn_gate.weight", DN_IN}}) ||
                 !proj(l, "ssm_out.weight", DN_IN, N_EMBD, &L.out))
                 return bad("qk_open: gated-DeltaNet projections missing or of an unsupported type / shape");
-            if (!f32(l, "ssm_alpha.weight", (uint64_t)DN_HV * N_EMBD, &L.alpha_w) ||
-                !f32(l, "ssm_beta.weight", (uint64_t)DN_HV * N_EMBD, &L.beta_w))
-                return bad("qk_open: missing ssm_alpha/ssm_beta (the fused ssm_ba form is not supported)");
+            qkg_tensor t_al;
+            if (find(l, "ssm_alpha.weight", &t_al)) {
+                if (!f32(l, "ssm_alpha.weight", (uint64_t)DN_HV * N_EMBD, &L.alpha_w) ||
+                    !f32(l, "ssm_beta.weight", (uint64_t)DN_HV * N_EMBD, &L.beta_w))
+                    return bad("qk_open: ssm_alpha/ssm_beta missing or of an unexpected shape");
+            } else if (!fused_ba(l, &L.alpha_w, &L.beta_w)) {
+                return false;
+            }
             if (!f32(l, "ssm_dt.bias", DN_HV, &L.dt_bias) || !f32(l, "ssm_a", DN_HV, &L.a_vec) ||
                 !(f32(l, "ssm_conv1d.weight", (uint64_t)DN_CH * 4, &L.ker) || f32(l, "ssm_conv1d", (uint64_t)DN_CH * 4, &L.ker)) ||
                 !f32(l, "ssm_norm.weight", DN_DS, &L.ssm_norm))
@@ -462,8 +517,8 @@ bool qk_engine::load_mixers(qkg_file* g, char* err, size_t err_len)
                 return bad("qk_open: attention norm tensors missing or of an unexpected shape");
             L.ps1 = L.ps2 = (size_t)FA_HKV * n_ctx * FA_DH;
         }
-        L.st1 = (float*)dev_alloc(MAX_ROWS * L.ps1 * sizeof(float), true);
-        L.st2 = (float*)dev_alloc(MAX_ROWS * L.ps2 * sizeof(float), true);
+        L.st1 = (float*)dev_alloc(n_slots * L.ps1 * sizeof(float), true);   // one stripe per configured slot
+        L.st2 = (float*)dev_alloc(n_slots * L.ps2 * sizeof(float), true);
         if (!L.st1 || !L.st2) return bad("qk_open: device memory exhausted (per-slot state)");
     }
     auto rows_of = [&](size_t n) { return (float*)dev_alloc(cap * n * sizeof(float), true); };
@@ -620,14 +675,31 @@ bool qk_engine::open(const char* path, const qk_config& cfg, char* err, size_t e
 
     // ---- device ----
     if (qk::require_device() != QKK_OK) return bad("qk_open: no HIP device: libqk.so has no CPU path");
-    uint64_t need = t_embd.nbytes + t_head.nbytes + (64u << 20);
-    for (uint32_t l = 0; l < n_layer; l++)
-        for (const qkg_tensor* t : {&mt[l].gate_inp, &mt[l].gate_inp_shexp, &mt[l].gate_exps, &mt[l].up_exps,
-                                    &mt[l].down_exps, &mt[l].gate_shexp, &mt[l].up_shexp, &mt[l].down_shexp})
-            need += t->nbytes + 512;
+    // Everything the open will hold on the device, before the first upload: the tensors of the file
+    // (every one is uploaded at most once), per-slot state and the snapshot entries of the mixers, the
+    // rows of a pass and the workspaces (a generous 64 KiB per row) -- a configuration that cannot fit
+    // is refused here and not after gigabytes have been uploaded.
+    uint64_t need = 64u << 20;
+    for (uint64_t i = 0; i < qkg_n_tensors(g); i++) {
+        qkg_tensor t;
+        if (qkg_tensor_at(g, i, &t) == 0) need += t.nbytes + 512;
+    }
+    const bool with_mixers = kinds[0] != EngineLayer::MOE_ONLY;
+    for (uint32_t l = 0; l < n_layer && with_mixers; l++) {
+        const uint64_t per_slot = kinds[l] == EngineLayer::RECURRENT
+                                      ? (uint64_t)DN_CH * 3 + (uint64_t)DN_HV * DN_DS * DN_DS
+                                      : 2ull * FA_HKV * n_ctx * FA_DH;
+        need += (n_slots + N_STATE) * per_slot * sizeof(float);
+    }
+    need += (uint64_t)(with_mixers ? pf_rows : MAX_ROWS) * (64u << 10) * sizeof(float) + (uint64_t)vocab * 80;
     size_t free_b = 0, total_b = 0;
     if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) return bad("qk_open: cannot query device memory");
-    if (need > free_b) return bad("qk_open: the model does not fit this device's free memory");
+    if (need > free_b) {
+        if (err && err_len)
+            snprintf(err, err_len, "qk_open: the model, %u slot(s) of state at n_ctx %u and the snapshots need about %.1f GB, "
+                     "the device has %.1f GB free", n_slots, n_ctx, need / 1e9, free_b / 1e9);
+        return false;
+    }
     if (hipStreamCreateWithFlags(&st, hipStreamNonBlocking) != hipSuccess) return bad("qk_open: cannot create a stream");
 
     const void* p = nullptr;
@@ -679,6 +751,8 @@ bool qk_engine::open(const char* path, const qk_config& cfg, char* err, size_t e
     memset(h_tok, 0, MAX_ROWS * 4);
     memset(h_pos, 0, MAX_ROWS * 4);
     if (full_model && !load_mixers(g, err, err_len)) return false;
+    cat_everywhere = full_model;
+    for (const EngineLayer& L : layers) cat_everywhere = cat_everywhere && L.cat.w != nullptr;
     if (hipDeviceSynchronize() != hipSuccess) return bad("qk_open: upload failed"); // fills and uploads are complete
 
     // One graph per dispatch depth z = highest active slot + 1 (the reference records one

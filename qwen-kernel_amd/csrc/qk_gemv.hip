@@ -177,9 +177,13 @@ struct GemvShape {
     static constexpr int RPC2048 = (TYPE == QKK_Q8_0 || TYPE == QKK_Q6_K) ? 2 : 4;
 };
 
-template <int TYPE, int LPR, int PASSES, int RPC>
+// NORM: the activation row is RMS-normalised on the way in, y = W . (x * nw / sqrt(mean(x^2) + eps)): the
+// lanes that share a weight row hold all of x between them, so the mean square is one cross-lane sum and
+// the dot products run on x * nw and are scaled at the end -- the norm costs no launch of its own.
+template <int TYPE, int LPR, int PASSES, int RPC, bool NORM = false>
 __global__ __launch_bounds__(256) void gemv_stream_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X,
-                                                          float* __restrict__ Y, uint32_t M)
+                                                          float* __restrict__ Y, uint32_t M,
+                                                          const float* __restrict__ nw, float eps)
 {
     constexpr int GROUPS = WAVE / LPR;
     constexpr uint32_t K = 32u * LPR * PASSES;
@@ -208,10 +212,20 @@ __global__ __launch_bounds__(256) void gemv_stream_kernel(const uint8_t* __restr
     XSlice xs[HALF ? 1 : PASSES];
     XSliceH xh[HALF ? PASSES : 1];
     float xsum[PASSES][4];
+    float ss = 0.f;
 #pragma unroll
     for (int p = 0; p < PASSES; p++) {
         XSlice f;
         load_xslice<TYPE>(f, x + p * 32 * LPR, lir);
+        if constexpr (NORM) {
+            XSlice g;
+            load_xslice<TYPE>(g, nw + p * 32 * LPR, lir);
+#pragma unroll
+            for (int i = 0; i < 32; i++) {
+                ss += f.v[i] * f.v[i];
+                f.v[i] *= g.v[i];
+            }
+        }
         if constexpr (TYPE == QKK_IQ4_XS) split_xslice_iq4(xh[p], f);
         else if constexpr (HALF) split_xslice(xh[p], f);
         else {
@@ -228,6 +242,8 @@ __global__ __launch_bounds__(256) void gemv_stream_kernel(const uint8_t* __restr
     if constexpr (TYPE == QKK_IQ3_XXS) fill_iq3_half_entry(tab3, threadIdx.x, grid_word);
     if constexpr (TYPE == QKK_IQ4_XS) fill_iq4_pair_entry(tab4, threadIdx.x);
     if constexpr (HALF) __syncthreads();
+    float out_scale = 1.f;
+    if constexpr (NORM) out_scale = 1.f / sqrtf(lanes_sum<LPR>(ss) / (float)K + eps);
 
     auto dot_row = [&](const LaneW<TYPE> (&w)[PASSES]) {
         float acc = 0.f;
@@ -237,7 +253,7 @@ __global__ __launch_bounds__(256) void gemv_stream_kernel(const uint8_t* __restr
             else if constexpr (TYPE == QKK_IQ4_XS) acc += w[p].dot_h(xh[p], &tab4, lir);
             else acc += w[p].dot(xs[p], xsum[p], &tab, lir);
         }
-        return lanes_sum<LPR>(acc);
+        return lanes_sum<LPR>(acc) * out_scale;
     };
 
     uint8_t* area = s_stage[wave];
@@ -351,8 +367,9 @@ __global__ __launch_bounds__(256) void gemv_dense_kernel(const T* __restrict__ W
 
 // ---- launchers ----------------------------------------------------------------------------
 
-template <int TYPE, int LPR, int PASSES>
-static void launch_q(const void* W, const float* X, float* Y, uint32_t M, uint32_t batch, hipStream_t st)
+template <int TYPE, int LPR, int PASSES, bool NORM = false>
+static void launch_q(const void* W, const float* X, float* Y, uint32_t M, uint32_t batch, hipStream_t st,
+                     const float* nw = nullptr, float eps = 0.f)
 {
     constexpr int RPC = GemvShape<TYPE>::RPC2048 / PASSES > 0 ? GemvShape<TYPE>::RPC2048 / PASSES : 1;
     constexpr uint32_t CH = RPC * (WAVE / LPR);
@@ -365,7 +382,8 @@ static void launch_q(const void* W, const float* X, float* Y, uint32_t M, uint32
     const uint32_t chunks = M / CH, tail_groups = (M - chunks * CH + WAVE / LPR - 1) / (WAVE / LPR);
     const uint32_t want = (std::max(chunks, tail_groups) + 3) / 4; // one chunk per wave
     const uint32_t blocks = std::max(1u, want <= cus * RESIDENT ? want : cus * DEPTH);
-    hipLaunchKernelGGL((gemv_stream_kernel<TYPE, LPR, PASSES, RPC>), dim3(blocks, batch), dim3(256), 0, st, (const uint8_t*)W, X, Y, M);
+    hipLaunchKernelGGL((gemv_stream_kernel<TYPE, LPR, PASSES, RPC, NORM>), dim3(blocks, batch), dim3(256), 0, st,
+                       (const uint8_t*)W, X, Y, M, nw, eps);
 }
 
 template <int TYPE>
@@ -533,6 +551,28 @@ int qkk_gemv(int type, const void* W, const float* X, float* Y, uint32_t M, uint
     }
     default: return fail(QKK_ETYPE, "qkk_gemv: unsupported tensor type %d", type);
     }
+}
+
+int qkk_gemv_norm(int type, const void* W, const float* X, const float* w_norm, float eps, float* Y, uint32_t M,
+                  uint32_t K, uint32_t batch, void* stream)
+{
+    if (!W || !X || !Y || !w_norm) return fail(QKK_EINVAL, "qkk_gemv_norm: null pointer");
+    if (M == 0 || batch == 0) return fail(QKK_EINVAL, "qkk_gemv_norm: M and batch must be positive");
+    if (batch > 16) return fail(QKK_ESHAPE, "qkk_gemv_norm: batch %u exceeds 16 (one pass over the weights per row)", batch);
+    if (K != 2048) return fail(QKK_ESHAPE, "qkk_gemv_norm: K=%u not supported (2048)", K);
+    if (!aligned16(W) || !aligned16(X) || !aligned16(w_norm))
+        return fail(QKK_EINVAL, "qkk_gemv_norm: W, X and w_norm must be 16-byte aligned");
+    if (!(eps >= 0.f)) return fail(QKK_EINVAL, "qkk_gemv_norm: eps must be non-negative");
+    if (int rc = require_device()) return rc;
+    hipStream_t st = as_stream(stream);
+    switch (type) {
+    case QKK_Q8_0: launch_q<QKK_Q8_0, 64, 1, true>(W, X, Y, M, batch, st, w_norm, eps); break;
+    case QKK_Q6_K: launch_q<QKK_Q6_K, 64, 1, true>(W, X, Y, M, batch, st, w_norm, eps); break;
+    case QKK_IQ4_XS: launch_q<QKK_IQ4_XS, 64, 1, true>(W, X, Y, M, batch, st, w_norm, eps); break;
+    case QKK_IQ3_XXS: launch_q<QKK_IQ3_XXS, 64, 1, true>(W, X, Y, M, batch, st, w_norm, eps); break;
+    default: return fail(QKK_ETYPE, "qkk_gemv_norm: tensor type %d is not a quantised block format", type);
+    }
+    return check_launch("qkk_gemv_norm");
 }
 
 } // extern "C"

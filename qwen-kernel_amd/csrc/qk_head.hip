@@ -55,11 +55,15 @@ __device__ static uint32_t fold_candidates(const volatile float* cv, const volat
 // 16-byte pieces through the wave's LDS area, the next chunk in flight during the arithmetic), and a
 // wave keeps the best (logit, id) of its rows, which ascend, so a strict '>' keeps the lowest id.
 // The vocabulary's rows behind the last full chunk are fetched per lane.
-template <int PASSES, int RPC>
+// NORM: the activation row is RMS-normalised with the weights nw on the way in (the output norm in
+// front of the head): a wave holds all of x, so the mean square is one cross-lane sum; the dot products
+// run on x * nw and the logits are scaled at the end.
+template <int PASSES, int RPC, bool NORM = false>
 __global__ __launch_bounds__(256) void head_q6k_kernel(const uint8_t* __restrict__ W,
                                                        const float* __restrict__ X,
                                                        float* __restrict__ logits_out,
-                                                       uint32_t* __restrict__ tok, HeadWs ws, uint32_t V)
+                                                       uint32_t* __restrict__ tok, HeadWs ws, uint32_t V,
+                                                       const float* __restrict__ nw, float eps)
 {
     constexpr uint32_t K = 2048u * PASSES, RB = (uint32_t)qkk_row_bytes_dev<QKK_Q6_K>(K), PB = RB / PASSES;
     constexpr uint32_t CB = RPC * RB, NPC = CB / 16;
@@ -79,9 +83,19 @@ __global__ __launch_bounds__(256) void head_q6k_kernel(const uint8_t* __restrict
     if (c < n_full) st.fetch(W + (size_t)c * CB, NPC, lane);
     XSlice xs[PASSES];
     float xsum[PASSES][4];
+    float ss = 0.f;
 #pragma unroll
     for (int p = 0; p < PASSES; p++) {
         load_xslice<QKK_Q6_K>(xs[p], x + p * 2048, lane);
+        if constexpr (NORM) {
+            XSlice g;
+            load_xslice<QKK_Q6_K>(g, nw + p * 2048, lane);
+#pragma unroll
+            for (int i = 0; i < 32; i++) {
+                ss += xs[p].v[i] * xs[p].v[i];
+                xs[p].v[i] *= g.v[i];
+            }
+        }
 #pragma unroll
         for (int q = 0; q < 4; q++) {
             float t = 0.f;
@@ -90,13 +104,15 @@ __global__ __launch_bounds__(256) void head_q6k_kernel(const uint8_t* __restrict
             xsum[p][q] = t;
         }
     }
+    float out_scale = 1.f;
+    if constexpr (NORM) out_scale = 1.f / sqrtf(wave_sum(ss) / (float)K + eps);
     float bv = ARG_FLOOR;
     uint32_t bi = 0xFFFFFFFFu;
     auto take = [&](const LaneW<QKK_Q6_K> (&w)[PASSES], uint32_t r) {
         float acc = 0.f;
 #pragma unroll
         for (int p = 0; p < PASSES; p++) acc += w[p].dot(xs[p], xsum[p], nullptr, lane);
-        acc = wave_sum(acc);
+        acc = wave_sum(acc) * out_scale;
         if (r < V) {
             if (logits_out && lane == 0) logits_out[(size_t)b * V + r] = acc;
             if (acc > bv) { bv = acc; bi = r; }
@@ -301,8 +317,9 @@ size_t qkk_head_workspace_bytes(uint32_t V, uint32_t batch)
     return 256 + (size_t)batch * blocks * 8;
 }
 
-int qkk_head_argmax(const void* W, const float* X, uint32_t* tok, float* logits, uint32_t V, uint32_t K,
-                    uint32_t batch, void* workspace, size_t workspace_bytes, void* stream)
+static int head_argmax_impl(const void* W, const float* X, uint32_t* tok, float* logits, uint32_t V, uint32_t K,
+                            uint32_t batch, void* workspace, size_t workspace_bytes, void* stream,
+                            const float* w_norm, float eps)
 {
     if (!W || !X || !tok || !workspace) return fail(QKK_EINVAL, "qkk_head_argmax: null pointer");
     if (V == 0 || batch == 0) return fail(QKK_EINVAL, "qkk_head_argmax: V and batch must be positive");
@@ -315,6 +332,8 @@ int qkk_head_argmax(const void* W, const float* X, uint32_t* tok, float* logits,
                     qkk_head_workspace_bytes(V, batch));
     if (int rc = require_device()) return rc;
     hipStream_t st = as_stream(stream);
+    if (w_norm && (batch != 1 || K != 2048))
+        return fail(QKK_ESHAPE, "qkk_head_argmax_norm: one row of 2048 (got %u rows of %u)", batch, K);
     if (batch >= 2 && batch <= 16 && K == 2048) {
         HeadWs ws;
         const uint32_t blocks = persistent_blocks() / 4; // one workgroup per CU (LDS)
@@ -336,13 +355,30 @@ int qkk_head_argmax(const void* W, const float* X, uint32_t* tok, float* logits,
     ws.counter = (uint32_t*)workspace;
     ws.cand_v = (float*)((uint8_t*)workspace + 256);
     ws.cand_i = (uint32_t*)(ws.cand_v + (size_t)batch * blocks);
-    if (K == 2048)
+    if (w_norm)
+        hipLaunchKernelGGL((head_q6k_kernel<1, HEAD_RPC, true>), dim3(blocks, batch), dim3(256), 0, st, (const uint8_t*)W,
+                           X, logits, tok, ws, V, w_norm, eps);
+    else if (K == 2048)
         hipLaunchKernelGGL((head_q6k_kernel<1, HEAD_RPC>), dim3(blocks, batch), dim3(256), 0, st, (const uint8_t*)W,
-                           X, logits, tok, ws, V);
+                           X, logits, tok, ws, V, (const float*)nullptr, 0.f);
     else
         hipLaunchKernelGGL((head_q6k_kernel<2, 1>), dim3(blocks, batch), dim3(256), 0, st, (const uint8_t*)W, X,
-                           logits, tok, ws, V);
+                           logits, tok, ws, V, (const float*)nullptr, 0.f);
     return check_launch("qkk_head_argmax");
+}
+
+int qkk_head_argmax(const void* W, const float* X, uint32_t* tok, float* logits, uint32_t V, uint32_t K,
+                    uint32_t batch, void* workspace, size_t workspace_bytes, void* stream)
+{
+    return head_argmax_impl(W, X, tok, logits, V, K, batch, workspace, workspace_bytes, stream, nullptr, 0.f);
+}
+
+int qkk_head_argmax_norm(const void* W, const float* X, const float* w_norm, float eps, uint32_t* tok, float* logits,
+                         uint32_t V, uint32_t K, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!w_norm || !aligned16(w_norm)) return fail(QKK_EINVAL, "qkk_head_argmax_norm: w_norm must be a 16-byte aligned pointer");
+    if (!(eps >= 0.f)) return fail(QKK_EINVAL, "qkk_head_argmax_norm: eps must be non-negative");
+    return head_argmax_impl(W, X, tok, logits, V, K, 1, workspace, workspace_bytes, stream, w_norm, eps);
 }
 
 int qkk_argmax(const float* logits, uint32_t* tok, uint32_t n, uint32_t batch, void* stream)

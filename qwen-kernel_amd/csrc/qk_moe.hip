@@ -504,6 +504,7 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const uint8_t* __restrict
 namespace qk {
 int moe_grouped_launch(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* sel, void* workspace,
                        uint32_t N, uint32_t stages, hipStream_t st, const MoeTail* tail);
+int moe_ws_alarm_take(bool* was_set);
 void launch_add_rmsnorm(const float* a, const float* b, const float* w, float* y, float* xn, uint32_t n, uint32_t rows,
                         float eps, hipStream_t st);
 }
@@ -743,6 +744,21 @@ int qkk_moe_decode(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* se
 {
     return moe_decode_impl("qkk_moe_decode", L, X, Y, sel, workspace, workspace_bytes, n_slots, QKK_STAGE_ALL,
                            stream);
+}
+
+int qkk_moe_workspace_status(void* stream)
+{
+    if (int rc = require_device()) return rc;
+    if (hipStreamSynchronize(as_stream(stream)) != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(QKK_EDEVICE, "qkk_moe_workspace_status: the stream failed");
+    }
+    bool dirty = false;
+    if (int rc = moe_ws_alarm_take(&dirty)) return rc;
+    if (dirty)
+        return fail(QKK_EINVAL, "qkk_moe_workspace_status: a call with more than %u rows ran on a workspace whose header "
+                    "was not zero (never cleared, or the clear had not completed): its results are invalid", ROWWISE_MAX);
+    return QKK_OK;
 }
 
 int qkk_moe_decode_static(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel* sel, uint32_t n_slots,

@@ -10,11 +10,27 @@
 // and groups in its last workgroup), gate/up, down, fold.
 #include "qk_moe_common.h"
 
+#include <map>
+#include <mutex>
+#include <utility>
 #include <algorithm>
 
 namespace qk {
 
 constexpr uint32_t SELECT_INLINE_MAX = 32; // up to this many tokens the route launch also selects
+
+// The caller clears a workspace once; the arrival counter (word 0 of its 256-byte header) then returns to
+// zero after every step, and no kernel ever writes the 63 words behind it.  Anything but zero there means
+// the header was never cleared (or the clear, issued on another stream, has not completed): the counter
+// cannot be trusted either, no workgroup may find itself last, and the step's numbers are wrong.  The
+// routing launches look at those words and raise this flag (per device, sticky until
+// qkk_moe_workspace_status reads it) so that the mistake is an error and not only wrong numbers.
+static __device__ uint32_t g_ws_alarm;
+__device__ __forceinline__ void check_ws_header(const MoeWs& ws, int lane)
+{
+    const uint32_t v = lane < 63 ? ws.counter[1 + lane] : 0u;
+    if (__builtin_amdgcn_ballot_w64(v != 0u) != 0 && lane == 0) g_ws_alarm = 1u;
+}
 
 // ---- selection: one wave takes the tokens first, first+stride, ... TPW (1 or 2) at a time ---------
 // (logits written by other workgroups: the caller's acquire fence, or a kernel boundary, precedes)
@@ -130,6 +146,7 @@ __global__ __launch_bounds__(512) void moe_route_multi_kernel(const float* __res
     const uint32_t task = blockIdx.x * NW + wave;
     const uint32_t t = task % n_rows, t0 = (task / n_rows) * TG;
     const uint32_t LS = lstride(d.E);
+    if (select_here && blockIdx.x == 0 && wave == 0) check_ws_header(ws, lane);
 
     if (t0 < N) {
         const float4* row = (const float4*)(t < d.E ? gate_inp + (size_t)t * d.H : gate_inp_shexp);
@@ -193,6 +210,7 @@ __global__ __launch_bounds__(512) void moe_logits_tiled_kernel(const float* __re
     const uint32_t nt = min(LOGITS_TILE_TOKENS, N - t0);
     const uint32_t LS = lstride(d.E);
     const bool extra = RIDE && wave == 0 && rg == tt % rgroups; // this wave also takes the shared-gate row
+    if (blockIdx.x == 0 && wave == 0) check_ws_header(ws, lane); // the selection launch behind this one counts arrivals
 
     const float4* xs = (const float4*)(X + (size_t)t0 * 2048); // nt consecutive rows: one contiguous range
     float4 xv[LOGITS_TILE_TOKENS];
@@ -266,26 +284,47 @@ constexpr uint32_t FUSED_MAX_ROWS = 32; // up to here the shared expert rides in
 
 // The shared expert's chain runs on a side stream of the library, forked from and joined back into
 // the caller's stream with events (capturable: under stream capture the side stream joins the
-// caller's graph).  One per device, created on first use, default priority.
+// caller's graph).  One side stream and one event pair PER CALLER STREAM and device, created under a
+// lock on first use and kept until the process ends, default priority: two engines, or two host
+// threads on streams of their own, never re-record each other's events.
 struct SideStream {
     hipStream_t stream = nullptr;
     hipEvent_t fork = nullptr, join = nullptr;
 };
-static SideStream* side_stream()
+static SideStream* side_stream(hipStream_t caller)
 {
-    static SideStream per_device[64];
+    static std::mutex lock;
+    static std::map<std::pair<int, hipStream_t>, SideStream> made;
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
-    SideStream& s = per_device[dev];
-    if (!s.stream) {
-        if (hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking) != hipSuccess ||
-            hipEventCreateWithFlags(&s.fork, hipEventDisableTiming) != hipSuccess ||
-            hipEventCreateWithFlags(&s.join, hipEventDisableTiming) != hipSuccess) {
-            s.stream = nullptr;
-            return nullptr;
-        }
+    if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+    std::lock_guard<std::mutex> hold(lock);
+    auto it = made.find({dev, caller});
+    if (it != made.end()) return &it->second;   // std::map: the address of an entry stays put
+    SideStream s;
+    if (hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking) != hipSuccess) return nullptr;
+    if (hipEventCreateWithFlags(&s.fork, hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&s.join, hipEventDisableTiming) != hipSuccess) {
+        if (s.fork) (void)hipEventDestroy(s.fork);
+        (void)hipStreamDestroy(s.stream);
+        return nullptr;
     }
-    return &s;
+    return &(made[{dev, caller}] = s);
+}
+
+// Reads (and clears) the current device's flag; the caller has synchronised the stream it asks about.
+int moe_ws_alarm_take(bool* was_set)
+{
+    uint32_t* flag = nullptr;
+    uint32_t v = 0;
+    const uint32_t zero = 0;
+    if (hipGetSymbolAddress((void**)&flag, HIP_SYMBOL(g_ws_alarm)) != hipSuccess || !flag ||
+        hipMemcpy(&v, flag, sizeof v, hipMemcpyDeviceToHost) != hipSuccess ||
+        (v && hipMemcpy(flag, &zero, sizeof zero, hipMemcpyHostToDevice) != hipSuccess)) {
+        (void)hipGetLastError();
+        return fail(QKK_EDEVICE, "moe: cannot read the workspace flag");
+    }
+    *was_set = v != 0;
+    return QKK_OK;
 }
 
 // Host entry of the path for N >= 2 rows (arguments already validated).
@@ -299,7 +338,7 @@ int moe_grouped_launch(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel
     const uint32_t experts_stages = stages & (QKK_STAGE_GATEUP | QKK_STAGE_DOWN);
     const bool split = N > FUSED_MAX_ROWS;
     // fork: the shared expert needs only X (and its own h), so it starts right away
-    SideStream* side = experts_stages && split ? side_stream() : nullptr;
+    SideStream* side = experts_stages && split ? side_stream(st) : nullptr;
     if (experts_stages && split) {
         if (side && hipEventRecord(side->fork, st) == hipSuccess && hipStreamWaitEvent(side->stream, side->fork, 0) == hipSuccess)
             moe_mfma_launch_shared(L, X, sel, ws, d, N, stages, side->stream);

@@ -135,6 +135,27 @@ class StackModel:
                        for l in range(n_layer)]
         self.post_norm = [(1.0 + 0.1 * rng.standard_normal(H)).astype(np.float32) for _ in range(n_layer)]
 
+    @staticmethod
+    def interleave_ba(alpha, beta):
+        """[hV, H] alpha and beta -> the fused [2 hV, H] rows: per key-head group g the rows 4g, 4g+1 are
+        beta of the value heads 2g, 2g+1 and 4g+2, 4g+3 their alpha."""
+        hv = alpha.shape[0]
+        ba = np.empty((2 * hv,) + alpha.shape[1:], dtype=alpha.dtype)
+        for r in range(2 * hv):
+            grp, sub = r >> 2, r & 3
+            ba[r] = (beta if sub < 2 else alpha)[grp * 2 + (sub & 1)]
+        return ba
+
+    @staticmethod
+    def split_ba(rows):
+        """The inverse of interleave_ba: fused rows -> (alpha, beta)."""
+        hv = rows.shape[0] // 2
+        alpha, beta = np.empty((hv,) + rows.shape[1:], rows.dtype), np.empty((hv,) + rows.shape[1:], rows.dtype)
+        for r in range(2 * hv):
+            grp, sub = r >> 2, r & 3
+            (beta if sub < 2 else alpha)[grp * 2 + (sub & 1)] = rows[r]
+        return alpha, beta
+
     def kvs(self):
         return {"general.architecture": self.arch, self.arch + ".block_count": len(self.layers),
                 self.arch + ".expert_used_count": self.n_used, "tokenizer.ggml.eos_token_id": self.eos,
@@ -164,8 +185,13 @@ class FullModel:
     FA = dict(dh=256, hq=16, hkv=2, n_rot=64)
 
     def __init__(self, seed, kinds="RRRA", vocab=512, n_expert=8, n_ff=256, n_used=4, eos=1000, bos=11, arch="qwen35moe",
-                 distinct_moe=None):
+                 distinct_moe=None, fused_ba=None):
+        """fused_ba: None writes ssm_alpha / ssm_beta as two F32 tensors; capi.F32 writes the same numbers
+        as one interleaved ssm_ba tensor (the qwen3next form, reference src/main.cpp:3931-3948); capi.Q8_0 /
+        capi.IQ4_XS write a quantised ssm_ba of its own -- alpha and beta of such a model are the
+        dequantised rows, which whoever needs them on the host computes (mix[l]["alpha"] is None)."""
         H = 2048
+        self.fused_ba = fused_ba
         rng = np.random.default_rng(seed)
         f = lambda *shape, scale=1.0: (rng.standard_normal(shape) * scale).astype(np.float32)
         near1 = lambda n: (1.0 + 0.1 * rng.standard_normal(n)).astype(np.float32)
@@ -193,6 +219,12 @@ class FullModel:
                                      beta=f(d["hv"], H, scale=0.03), dt=f(d["hv"]),
                                      a=(-np.abs(rng.standard_normal(d["hv"])) - 0.05).astype(np.float32),
                                      ker=f(d["ch"], 4, scale=0.5), norm=near1(d["ds"])))
+                m = self.mix[-1]
+                if fused_ba == capi.F32:
+                    m["ba"] = self.interleave_ba(m["alpha"], m["beta"])
+                elif fused_ba is not None:
+                    m["ba"] = synth.tensor_host(fused_ba, 2 * d["hv"], H, s0 + 14, 4e-4 if fused_ba == capi.Q8_0 else 2.4e-5)   # rows of std ~0.03, like the split tensors
+                    m["alpha"] = m["beta"] = None
             elif kind == "A":
                 a = self.FA
                 self.mix.append(dict(kind="A", q=q8(a["hq"] * 2 * a["dh"], H, s0 + 21, 4e-4), k=q8(a["hkv"] * a["dh"], H, s0 + 22, 4e-4),
@@ -200,6 +232,27 @@ class FullModel:
                                      qn=near1(a["dh"]), kn=near1(a["dh"])))
             else:
                 raise ValueError(kind)
+
+    @staticmethod
+    def interleave_ba(alpha, beta):
+        """[hV, H] alpha and beta -> the fused [2 hV, H] rows: per key-head group g the rows 4g, 4g+1 are
+        beta of the value heads 2g, 2g+1 and 4g+2, 4g+3 their alpha."""
+        hv = alpha.shape[0]
+        ba = np.empty((2 * hv,) + alpha.shape[1:], dtype=alpha.dtype)
+        for r in range(2 * hv):
+            grp, sub = r >> 2, r & 3
+            ba[r] = (beta if sub < 2 else alpha)[grp * 2 + (sub & 1)]
+        return ba
+
+    @staticmethod
+    def split_ba(rows):
+        """The inverse of interleave_ba: fused rows -> (alpha, beta)."""
+        hv = rows.shape[0] // 2
+        alpha, beta = np.empty((hv,) + rows.shape[1:], rows.dtype), np.empty((hv,) + rows.shape[1:], rows.dtype)
+        for r in range(2 * hv):
+            grp, sub = r >> 2, r & 3
+            (beta if sub < 2 else alpha)[grp * 2 + (sub & 1)] = rows[r]
+        return alpha, beta
 
     def kvs(self):
         return {"general.architecture": self.arch, self.arch + ".block_count": len(self.layers),
@@ -218,10 +271,14 @@ class FullModel:
                   (p + "attn_norm.weight", capi.F32, (H,), self.attn_norm[l])]
             if m["kind"] == "R":
                 t += [(p + "attn_qkv.weight", capi.Q8_0, (H, d["ch"]), m["qkv"]), (p + "attn_gate.weight", capi.Q8_0, (H, d["d_in"]), m["gate"]),
-                      (p + "ssm_out.weight", capi.Q8_0, (d["d_in"], H), m["out"]), (p + "ssm_alpha.weight", capi.F32, (H, d["hv"]), m["alpha"]),
-                      (p + "ssm_beta.weight", capi.F32, (H, d["hv"]), m["beta"]), (p + "ssm_dt.bias", capi.F32, (d["hv"],), m["dt"]),
+                      (p + "ssm_out.weight", capi.Q8_0, (d["d_in"], H), m["out"]), (p + "ssm_dt.bias", capi.F32, (d["hv"],), m["dt"]),
                       (p + "ssm_a", capi.F32, (d["hv"],), m["a"]), (p + "ssm_conv1d.weight", capi.F32, (4, d["ch"]), m["ker"]),
                       (p + "ssm_norm.weight", capi.F32, (d["ds"],), m["norm"])]
+                if "ba" in m:
+                    t += [(p + "ssm_ba.weight", self.fused_ba, (H, 2 * d["hv"]), m["ba"])]
+                else:
+                    t += [(p + "ssm_alpha.weight", capi.F32, (H, d["hv"]), m["alpha"]),
+                          (p + "ssm_beta.weight", capi.F32, (H, d["hv"]), m["beta"])]
             else:
                 t += [(p + "attn_q.weight", capi.Q8_0, (H, a["hq"] * 2 * a["dh"]), m["q"]), (p + "attn_k.weight", capi.Q8_0, (H, a["hkv"] * a["dh"]), m["k"]),
                       (p + "attn_v.weight", capi.Q8_0, (H, a["hkv"] * a["dh"]), m["v"]), (p + "attn_output.weight", capi.Q8_0, (a["hq"] * a["dh"], H), m["out"]),

@@ -260,6 +260,29 @@ void run(dim3 grid, dim3 block, size_t lds, const std::function<void()>& body)
     for (auto& th : threads) th.join();
 }
 
+// ---- stream capture ---------------------------------------------------------------------------
+static thread_local Graph* t_capture = nullptr;
+
+void submit(std::function<void()> op)
+{
+    if (t_capture) t_capture->ops.push_back(std::move(op));
+    else op();
+}
+
+bool capture_begin()
+{
+    if (t_capture) return false;
+    t_capture = new Graph;
+    return true;
+}
+
+Graph* capture_end()
+{
+    Graph* g = t_capture;
+    t_capture = nullptr;
+    return g;
+}
+
 } // namespace emu
 
 emu_float4 emu_mfma_16x16x32_f16(emu_half8 a, emu_half8 b, emu_float4 c)

@@ -18,6 +18,7 @@
 #include <string.h>
 
 #include <functional>
+#include <vector>
 #include <type_traits>
 
 #define __global__
@@ -65,6 +66,13 @@ void wave_barrier();
 const uint64_t* exchange(uint64_t v);
 void exchange_done();
 void run(dim3 grid, dim3 block, size_t lds, const std::function<void()>& body);
+// Stream capture: between hipStreamBeginCapture and hipStreamEndCapture (per host thread) launches,
+// copies and fills are recorded instead of run; a graph is the recorded list, a launch of it runs
+// the list in order.  submit() runs `op` now, or records it while the calling thread captures.
+void submit(std::function<void()> op);
+bool capture_begin();
+struct Graph { std::vector<std::function<void()>> ops; };
+Graph* capture_end();
 } // namespace emu
 
 #define threadIdx emu::cur_thread()
@@ -75,7 +83,7 @@ void run(dim3 grid, dim3 block, size_t lds, const std::function<void()>& body);
 template <class K, class... A>
 static inline void emu_launch(K kernel, dim3 grid, dim3 block, size_t lds, hipStream_t, A... args)
 {
-    emu::run(grid, block, lds, [=]() { kernel(args...); });
+    emu::submit([=]() { emu::run(grid, block, lds, [=]() { kernel(args...); }); });
 }
 #define hipLaunchKernelGGL(kernel, grid, block, lds, stream, ...) emu_launch(kernel, grid, block, lds, stream, __VA_ARGS__)
 #define HIP_SYMBOL(x) ((const void*)&(x))
@@ -88,7 +96,7 @@ static inline const char* hipGetErrorString(hipError_t) { return "host build"; }
 static inline hipError_t hipDeviceGetAttribute(int* v, hipDeviceAttribute_t, int) { *v = 4; return hipSuccess; } // a small "device": 4 CUs
 static inline hipError_t hipFuncSetAttribute(const void*, hipFuncAttribute, int) { return hipSuccess; }
 static inline hipError_t hipGetDeviceProperties(hipDeviceProp_t* p, int) { snprintf(p->gcnArchName, 64, "host"); p->multiProcessorCount = 4; return hipSuccess; }
-static inline hipError_t hipMemcpyAsync(void* d, const void* s, size_t n, hipMemcpyKind, hipStream_t) { memmove(d, s, n); return hipSuccess; }
+static inline hipError_t hipMemcpyAsync(void* d, const void* s, size_t n, hipMemcpyKind, hipStream_t) { emu::submit([=]() { memmove(d, s, n); }); return hipSuccess; }
 static inline hipError_t hipGetSymbolAddress(void** p, const void* sym) { *p = (void*)sym; return hipSuccess; }
 hipError_t hipMalloc(void** p, size_t n);   // ends at a guard page
 hipError_t hipFree(void* p);
@@ -98,21 +106,28 @@ template <class T> static inline hipError_t hipHostMalloc(T** p, size_t n, unsig
 static inline hipError_t hipHostFree(void* p) { free(p); return hipSuccess; }
 static inline hipError_t hipMemcpy(void* d, const void* s, size_t n, hipMemcpyKind) { memmove(d, s, n); return hipSuccess; }
 static inline hipError_t hipMemset(void* d, int v, size_t n) { memset(d, v, n); return hipSuccess; }
-static inline hipError_t hipMemsetAsync(void* d, int v, size_t n, hipStream_t = nullptr) { memset(d, v, n); return hipSuccess; }
+static inline hipError_t hipMemsetAsync(void* d, int v, size_t n, hipStream_t = nullptr) { emu::submit([=]() { memset(d, v, n); }); return hipSuccess; }
 static inline hipError_t hipMemGetInfo(size_t* f, size_t* t) { *f = (size_t)64 << 30; *t = (size_t)64 << 30; return hipSuccess; }
 static inline hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
 static inline hipError_t hipDeviceSynchronize() { return hipSuccess; }
 static inline hipError_t hipStreamDestroy(hipStream_t) { return hipSuccess; }
 static inline hipError_t hipEventDestroy(hipEvent_t) { return hipSuccess; }
 template <class K> static inline hipError_t hipOccupancyMaxActiveBlocksPerMultiprocessor(int* n, K, int, size_t) { *n = 2; return hipSuccess; }
-// no graphs in the host build: launches run at once, so a capture cannot be replayed; the engine is
-// opened with QK_NO_GRAPH=1
-static inline hipError_t hipStreamBeginCapture(hipStream_t, hipStreamCaptureMode) { return hipErrorUnknown; }
-static inline hipError_t hipStreamEndCapture(hipStream_t, hipGraph_t* g) { *g = nullptr; return hipErrorUnknown; }
-static inline hipError_t hipGraphInstantiate(hipGraphExec_t* e, hipGraph_t, void*, void*, size_t) { *e = nullptr; return hipErrorUnknown; }
-static inline hipError_t hipGraphLaunch(hipGraphExec_t, hipStream_t) { return hipErrorUnknown; }
-static inline hipError_t hipGraphDestroy(hipGraph_t) { return hipSuccess; }
-static inline hipError_t hipGraphExecDestroy(hipGraphExec_t) { return hipSuccess; }
+static inline hipError_t hipStreamBeginCapture(hipStream_t, hipStreamCaptureMode) { return emu::capture_begin() ? hipSuccess : hipErrorUnknown; }
+static inline hipError_t hipStreamEndCapture(hipStream_t, hipGraph_t* g) { *g = (hipGraph_t)emu::capture_end(); return *g ? hipSuccess : hipErrorUnknown; }
+static inline hipError_t hipGraphInstantiate(hipGraphExec_t* e, hipGraph_t g, void*, void*, size_t)
+{
+    *e = g ? (hipGraphExec_t) new emu::Graph(*(emu::Graph*)g) : nullptr;
+    return *e ? hipSuccess : hipErrorInvalidValue;
+}
+static inline hipError_t hipGraphLaunch(hipGraphExec_t e, hipStream_t)
+{
+    if (!e) return hipErrorInvalidValue;
+    for (const auto& op : ((emu::Graph*)e)->ops) emu::submit(op);
+    return hipSuccess;
+}
+static inline hipError_t hipGraphDestroy(hipGraph_t g) { delete (emu::Graph*)g; return hipSuccess; }
+static inline hipError_t hipGraphExecDestroy(hipGraphExec_t e) { delete (emu::Graph*)e; return hipSuccess; }
 static inline hipError_t hipStreamCreateWithFlags(hipStream_t* s, unsigned) { *s = nullptr; return hipSuccess; }
 static inline hipError_t hipEventCreateWithFlags(hipEvent_t* e, unsigned) { *e = nullptr; return hipSuccess; }
 static inline hipError_t hipEventRecord(hipEvent_t, hipStream_t) { return hipSuccess; }

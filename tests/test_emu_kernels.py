@@ -148,3 +148,32 @@ def test_head_inside_its_tensors(qk, orc, emu, V, batch):
         top2 = np.sort(want)[-2:]
         if top2[1] - top2[0] > 2e-3 * abs(top2[1]):
             assert int(tok.numpy()[b]) == int(np.argmax(want))
+
+
+@pytest.mark.parametrize("name", QUANT)
+@pytest.mark.parametrize("M,batch", [(37, 1), (9, 2)])
+def test_gemv_norm_inside_its_tensors(qk, orc, emu, name, M, batch):
+    """The GEMV with the RMS norm in front (no launch of its own) against the oracle's norm + GEMV."""
+    t, K = type_id(qk, name), 2048
+    W = qk.synth.tensor_host(t, M, K, seed=M)
+    rng = np.random.default_rng(M + batch)
+    x = (rng.standard_normal((batch, K)) * 3.0).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, K).astype(np.float32)
+    Yd = emu.zeros((batch, M), np.float32)
+    qk.gemv_norm(t, emu.tensor(W.reshape(-1)), emu.tensor(x), emu.tensor(w), M, K, out=Yd)
+    want = orc.gemv(t, W, np.stack([orc.add_rms(x[b], w, 1e-6) for b in range(batch)]), M, K)
+    assert orc.rel_maxabs_err(Yd.numpy(), want) <= 1e-3
+
+
+def test_head_norm_inside_its_tensors(qk, orc, emu):
+    """The LM head with the output norm in front against the oracle's norm + GEMV + argmax."""
+    V, K = 301, 2048
+    W = qk.synth.tensor_host(qk.Q6_K, V, K, seed=V)
+    rng = np.random.default_rng(V)
+    x = (rng.standard_normal((1, K)) * 2.0).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, K).astype(np.float32)
+    ws = emu.workspace(qk.head_workspace_bytes(V, 1))
+    tok, logits = qk.head_argmax_norm(emu.tensor(W.reshape(-1)), emu.tensor(x), emu.tensor(w), V, K, ws, want_logits=True)
+    want = orc.gemv(qk.Q6_K, W, orc.add_rms(x[0], w, 1e-6), V, K)
+    assert orc.rel_maxabs_err(logits.numpy()[0], want) <= 1e-3
+    assert int(tok.numpy()[0]) == int(np.argmax(want))

@@ -173,3 +173,27 @@ def test_moe_layer_checks(qk, small_layer, tmp_path):
     with pytest.raises(qk.QkError) as e:                  # top-k above the selector's 16
         load(base, dict(KVS, **{"qwen3next.expert_used_count": 17}))
     assert e.value.code == -2
+
+
+def test_fused_ssm_ba_rows(qk, tmp_path):
+    """The fused decay / write-strength tensor of qwen3next files (reference src/main.cpp:3936-3948):
+    per key-head group g the rows 4g, 4g+1 are beta of the value heads 2g, 2g+1 and the rows 4g+2, 4g+3
+    their alpha.  The synthetic writer interleaves by that rule, split_ba undoes it, and a whole-model
+    file written with the fused form holds ssm_ba [n_embd, 64] in place of the two split tensors."""
+    FM = qk.engine.FullModel
+    hv = 32
+    alpha = np.arange(hv, dtype=np.float32)[:, None] + np.zeros((1, 4), np.float32)          # row h holds h
+    beta = 100 + np.arange(hv, dtype=np.float32)[:, None] + np.zeros((1, 4), np.float32)     # row h holds 100 + h
+    ba = FM.interleave_ba(alpha, beta)
+    assert ba[:8, 0].tolist() == [100, 101, 0, 1, 102, 103, 2, 3]
+    assert ba[60:, 0].tolist() == [130, 131, 30, 31]
+    a2, b2 = FM.split_ba(ba)
+    assert np.array_equal(a2, alpha) and np.array_equal(b2, beta)
+    for type_, nbytes in ((qk.F32, 64 * 2048 * 4), (qk.Q8_0, 64 * 2176)):
+        model = FM(3, kinds="R", vocab=64, fused_ba=type_)
+        path = model.write(str(tmp_path / f"fused_{type_}.gguf"))
+        with qk.gguf.File(path) as f:
+            names = f.names()
+            assert "blk.0.ssm_alpha.weight" not in names and "blk.0.ssm_beta.weight" not in names
+            t = f.find("blk.0.ssm_ba.weight")
+            assert (t.type, tuple(t.ne[:2]), t.nbytes) == (type_, (2048, 64), nbytes)

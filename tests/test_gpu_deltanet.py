@@ -79,6 +79,31 @@ def test_deltanet_steps_match_the_cpu_mirror(qk, dev, n_slots, n_tok, kdiv):
     assert rel(S_gpu, S) <= TOL                  # the states after all tokens
 
 
+def test_deltanet_ab_with_the_norm_in_front(qk, orc, dev):
+    """qkk_dn_ab_conv_norm: x is the residual row; decay and write strength come out as from the norm
+    launch followed by qkk_dn_ab_conv (to rounding) and match the oracle on the oracle's normalised row;
+    the conv half is untouched (bit for bit)."""
+    import torch
+    print("[case] deltanet ab with the norm in front", flush=True)
+    w = Weights(3)
+    up = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    rng = np.random.default_rng(9)
+    for n in (1, 3):
+        x = (rng.standard_normal((n, NE)) * 4.0).astype(F)
+        nw = rng.uniform(0.5, 1.5, NE).astype(F)
+        qkv, st = rng.standard_normal((n, w.ch)).astype(F), rng.standard_normal((n, w.ch, 3)).astype(F)
+        wd = [up(getattr(w, k)) for k in ("alpha_w", "beta_w", "dt_bias", "a_vec")]
+        st1, st2 = up(st.copy()), up(st.copy())   # two buffers also where up() does not copy
+        gb, conv = qk.dn_ab_conv(up(x), *wd, st1, up(qkv), up(w.ker), w.qk, w_norm=up(nw))
+        gb0, conv0 = qk.dn_ab_conv(qk.rmsnorm(up(x), up(nw)), *wd, st2, up(qkv), up(w.ker), w.qk)
+        torch.cuda.synchronize()
+        assert torch.equal(conv, conv0) and torch.equal(st1, st2)
+        assert rel(gb.cpu().numpy(), gb0.cpu().numpy().astype(np.float64)) <= 1e-5
+        for s in range(n):
+            g, b = OD.ab(orc.add_rms(x[s], nw, 1e-6), w.alpha_w, w.beta_w, w.dt_bias, w.a_vec)
+            assert rel(gb.cpu().numpy()[s], np.concatenate([g, b])) <= TOL
+
+
 def test_deltanet_other_shapes(qk, dev):
     """Fewer heads (1 key head for 2 value heads, both pairings) and n_embd = 4096."""
     print("[case] deltanet other shapes", flush=True)

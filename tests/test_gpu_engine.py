@@ -74,9 +74,6 @@ def test_next_token_maps(world, orc):
     nxt1, nxtn, model = world["nxt1"], world["nxtn"], world["model"]
     assert len(set(nxt1)) > VOCAB // 8            # a real map, not a constant
     nxtf = world["nxtf"]
-    for other in (nxtf, nxtn):
-        differ = sum(a != b for a, b in zip(nxt1, other))
-        assert differ <= VOCAB // 50, differ      # other kernel families, same tolerance: near-ties only
     # few rows: the rows' company and position do not matter
     few = np.random.default_rng(2).permutation(VOCAB)[:15].tolist()
     for i in range(0, 15, 5):
@@ -85,14 +82,20 @@ def test_next_token_maps(world, orc):
     perm = np.random.default_rng(1).permutation(VOCAB)[:48].tolist()
     for i in range(0, 48, 12):
         assert world["step"](perm[i:i + 12]) == [nxtn[t] for t in perm[i:i + 12]]
-    # against the CPU oracle
-    checked = 0
-    for t in range(0, VOCAB, 64):
-        want, gap, top = OE.stack_next(model, t, want_margin=True)
+    # against the CPU oracle, EVERY token: all three kernel families give the oracle's id wherever its two
+    # best logits lie further apart than both sides' tolerance (1e-3 of the largest logit each); a token on
+    # which the families disagree with each other must therefore be such a near-tie
+    threads = max(1, min(16, len(os.sched_getaffinity(0))))
+    checked, ties = 0, []
+    for t in range(VOCAB):
+        want, gap, top = OE.stack_next(model, t, want_margin=True, threads=threads)
         if gap > 2e-3 * top:
-            assert nxt1[t] == want and nxtn[t] == want, (t, gap, top)
+            assert nxt1[t] == want and nxtf[t] == want and nxtn[t] == want, (t, gap, top, nxt1[t], nxtf[t], nxtn[t], want)
             checked += 1
-    assert checked >= 12
+        else:
+            ties.append(t)
+    print(f"[info] {checked} of {VOCAB} tokens decided by more than the tolerance; near-ties at {ties[:10]}", flush=True)
+    assert checked >= VOCAB - VOCAB // 50
     # every layer moves the result: without the last layer most next tokens change
     import copy
     short = copy.copy(model)

@@ -52,6 +52,30 @@ def test_gemv_q8_0_engine_shapes(qk, orc, dev, M, K, batch):
     run_case(qk, orc, dev, "q8_0", M, K, batch, seed=5)
 
 
+@pytest.mark.parametrize("name", ["q8_0", "q6_k", "iq4_xs", "iq3_xxs"])
+@pytest.mark.parametrize("M,batch", [(12288, 1), (9216, 1), (515, 2), (3, 1)])
+def test_gemv_with_the_norm_in_front(qk, orc, dev, name, M, batch):
+    """qkk_gemv_norm: y = W . rmsnorm(x) * w with the norm inside the launch, against the oracle's norm
+    (double) followed by its GEMV; 12288 and 9216 rows are a layer's input projections back to back."""
+    import torch
+    print(f"[case] gemv with norm {name} M={M} batch={batch}", flush=True)
+    K, t = 2048, TYPES[name]
+    W = qk.synth.tensor_host(t, M, K, 31)
+    rng = np.random.default_rng(M)
+    x = (rng.standard_normal((batch, K)) * 3.0).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, K).astype(np.float32)
+    up = lambda a: torch.from_numpy(a).to(dev)
+    got = qk.gemv_norm(t, up(W), up(x), up(w), M, K, eps=1e-6).cpu().numpy()
+    xn = np.stack([orc.add_rms(x[b], w, 1e-6) for b in range(batch)])
+    want = orc.gemv(t, W, xn, M, K)
+    assert orc.rel_maxabs_err(got, want) <= TOL
+    # the same numbers as the norm launch followed by the plain product, to rounding
+    two = qk.gemv(t, up(W), qk.rmsnorm(up(x), up(w)), M, K).cpu().numpy()
+    assert orc.rel_maxabs_err(got, two) <= 1e-5
+    with pytest.raises(qk.QkError):
+        qk.gemv_norm(t, up(W), up(x[:, :1024].copy()), up(w[:1024].copy()), M, 1024)
+
+
 def test_gemv_two_pass_k_is_deterministic(qk, orc, dev):
     """K = 4096 for several rows adds the second half's sum to the first's in a fixed order."""
     a = run_case(qk, orc, dev, "q6_k", 784, 4096, 9, seed=12)

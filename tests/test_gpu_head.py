@@ -44,6 +44,32 @@ def test_head_ragged(qk, orc, dev, V, K, batch):
     head_case(qk, orc, dev, V, K, batch, seed=12 + V)
 
 
+@pytest.mark.parametrize("V", [151936, 4097, 3])
+def test_head_with_the_norm_in_front(qk, orc, dev, V):
+    """qkk_head_argmax_norm: the output norm inside the head's launch, against the oracle's norm (double)
+    followed by its GEMV and argmax."""
+    import torch
+    print(f"[case] head with norm V={V}", flush=True)
+    K = 2048
+    W = qk.synth.tensor_host(qk.Q6_K, V, K, 40 + V % 7)
+    rng = np.random.default_rng(V)
+    x = (rng.standard_normal((1, K)) * 2.0).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, K).astype(np.float32)
+    ws = torch.zeros(qk.head_workspace_bytes(V, 1), dtype=torch.uint8, device=dev)
+    up = lambda a: torch.from_numpy(a).to(dev)
+    Wd, xd, wd = up(W), up(x), up(w)
+    tok, logits = qk.head_argmax_norm(Wd, xd, wd, V, K, ws, want_logits=True)
+    torch.cuda.synchronize()
+    ref = orc.gemv(orc.Q6_K, W, orc.add_rms(x[0], w, 1e-6), V, K)
+    srt = np.sort(ref)
+    if V > 1:
+        assert srt[-1] - srt[-2] > 1e-5 * abs(srt[-1]), "ambiguous fixture: pick another seed"
+    assert int(tok.cpu()[0]) == orc.argmax(ref)
+    assert orc.rel_maxabs_err(logits.cpu().numpy()[0], ref) <= 1e-3
+    tok2, _ = qk.head_argmax_norm(Wd, xd, wd, V, K, ws)      # the counters were rearmed
+    assert int(tok2.cpu()[0]) == int(tok.cpu()[0])
+
+
 def test_head_ties_pick_lowest_id(qk, dev):
     import torch
     print("[case] head ties", flush=True)

@@ -262,6 +262,33 @@ def test_moe_stale_workspace_stays_in_bounds(qk, orc, dev, layer_iq4, n):
         assert orc.rel_maxabs_err(Y[s], refs[s]["y"]) <= TOL, f"slot {s}"
 
 
+@pytest.mark.parametrize("n", [16, 40])
+def test_dirty_workspace_header_is_an_error(qk, dev, layer_iq4, n):
+    """A workspace whose header was never cleared: the routing launch of the expert-major path sees the
+    words behind the arrival counter and qkk_moe_workspace_status reports QKK_EINVAL, once; a cleared
+    workspace leaves the status clean.  Only the routing launch runs on the dirty workspace."""
+    import torch
+    print(f"[case] dirty workspace header, {n} rows", flush=True)
+    layer = layer_iq4.to_device(dev)
+    x = torch.randn((n, 2048), device=dev)
+    try:
+        qk.moe_workspace_status()                   # whatever earlier tests left is taken here
+    except qk.capi.QkError:
+        pass
+    ws = torch.zeros(qk.moe_workspace_bytes(layer, n), dtype=torch.uint8, device=dev)
+    qk.moe_decode(layer, x, ws, stages=1)
+    qk.moe_workspace_status()                       # clean: no error
+    ws[4:256] = 0x5A                                # the counter itself is zero, the 63 words behind it are not
+    qk.moe_decode(layer, x, ws, stages=1)
+    with pytest.raises(qk.capi.QkError) as e:
+        qk.moe_workspace_status()
+    assert e.value.code == -1 and "header" in str(e.value)
+    qk.moe_workspace_status()                       # reported once, then clean again
+    ws.zero_()
+    qk.moe_decode(layer, x, ws, stages=1)
+    qk.moe_workspace_status()
+
+
 def test_moe_layer_loaded_from_gguf(qk, orc, dev, tmp_path):
     """The reference's per-layer check on a model file (`qk moe <layer>`, src/main.cpp:920-1254): the
     layer's tensors come out of a GGUF file through the library's reader, the step runs on them,
