@@ -95,10 +95,15 @@ def run_ring(launches, steps, warmup):
 
 # ---- workloads -------------------------------------------------------------------------------
 
-def moe_workload(qk, n_slots, down_type, ring, steps, warmup, seed=1234):
+def moe_workload(qk, n_slots, down_type, ring, steps, warmup, seed=1234, slab=False):
+    """slab: the ring's tensors in ONE device allocation instead of one per tensor (same bytes, same
+    addresses' spread): separates what the step pays for address translation over many mappings."""
     import torch
     dev = "cuda:0"
-    layers = [qk.synth.device_layer(seed + 16 * i, down_type=down_type, device=dev) for i in range(ring)]
+    pool = qk.synth.Slab(ring * qk.synth.layer_bytes(down_type=down_type), dev) if slab else None
+    layers = [qk.synth.device_layer(seed + 16 * i, down_type=down_type, device=dev, slab=pool) for i in range(ring)]
+    if slab:
+        torch.cuda.empty_cache()   # the generators' own allocations go back to the driver
     g = torch.Generator(device=dev)
     g.manual_seed(seed)
     X = torch.randn((ring, n_slots, 2048), device=dev, generator=g)
@@ -278,6 +283,36 @@ def attn_workload(qk, n_slots, ctx, steps, warmup, tmax=4096, seed=5):
         return f
     wall, ev, n = run_ring([step(i) for i in range(ring)], steps // ring * ring, warmup)
     return dict(ms_event=ev, steps=n, ring=ring, bytes_step=2 * n_slots * hKV * ctx * dh * 4)
+
+
+def attn_prefill_workload(qk, n_pos, steps, warmup, tmax=4096, seed=8):
+    """The full-attention mixer over n_pos consecutive positions of one slot from an empty cache (prep +
+    causal attention, the prefill form): 16 query heads of 256 on 2 KV heads.  Flops: QK^T and PV over the
+    causal triangle, 2 * 2 * hQ * dh * n_pos * (n_pos + 1) / 2."""
+    import torch
+    dev = "cuda:0"
+    hQ, hKV, dh, n_rot, ring = 16, 2, 256, 64, 4
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    kc = [torch.zeros((1, hKV, tmax, dh), device=dev) for _ in range(ring)]
+    vc = [torch.zeros((1, hKV, tmax, dh), device=dev) for _ in range(ring)]
+    qfull = torch.randn((ring, n_pos, hQ, 2 * dh), device=dev, generator=g)
+    kin = torch.randn((ring, n_pos, hKV, dh), device=dev, generator=g)
+    vin = torch.randn((ring, n_pos, hKV, dh), device=dev, generator=g)
+    w = torch.ones(dh, device=dev)
+    rope = torch.from_numpy(qk.rope_table(tmax, n_rot)).to(dev)
+    pos = torch.arange(n_pos, dtype=torch.int32, device=dev)
+    qhat = torch.empty((ring, n_pos, hQ, dh), device=dev)
+    att = torch.empty((ring, n_pos, hQ, dh), device=dev)
+    ws = torch.empty(qk.attn_workspace_bytes(n_pos, hQ), dtype=torch.uint8, device=dev)
+
+    def step(i):
+        def f():
+            qk.attn_prep(qfull[i], kin[i], vin[i], w, w, rope, pos, kc[i], vc[i], n_rot, qhat=qhat[i], seq=True)
+            qk.attn_decode(qhat[i], kc[i], vc[i], qfull[i], pos, ws, att=att[i], seq=True)
+        return f
+    wall, ev, n = run_ring([step(i) for i in range(ring)], steps // ring * ring, warmup)
+    return dict(ms_event=ev, steps=n, ring=ring, flops=2.0 * 2 * hQ * dh * n_pos * (n_pos + 1) / 2)
 
 
 def deltanet_workload(qk, n_slots, steps, warmup, seed=6):
@@ -666,6 +701,13 @@ def main():
                                                   stage_us={k: v * 1e3 for k, v in mh["stage_ms"].items()})
             log(f"[bench] moe bs1, one layer replayed: {ex['moe_decode_bs1_cache_hot']}")
             torch.cuda.empty_cache()
+            # the ring's tensors carved from one allocation: what the many separate mappings cost, if anything
+            ms = moe_workload(qk, 1, qk.IQ4_XS, a.ring, min(steps, 800), a.warmup, slab=True)
+            ex["moe_decode_bs1_ring_in_one_allocation"] = dict(us=ms["ms_event"] * 1e3, steps_timed=ms["steps"],
+                                                               stage_us={k: v * 1e3 for k, v in ms["stage_ms"].items()})
+            log(f"[bench] moe bs1, ring in one allocation: {ex['moe_decode_bs1_ring_in_one_allocation']}")
+            del ms
+            torch.cuda.empty_cache()
             m16 = moe_workload(qk, 16, qk.Q6_K, 4, 200, 20)
             ex["moe_decode_bs16_q6k_down"] = dict(us=m16["ms_event"] * 1e3, distinct_experts=m16["distinct_experts"],
                                                   gbps=m16["bytes_step"] / (m16["ms_event"] * 1e-3) / 1e9,
@@ -710,6 +752,11 @@ def main():
                                                         ring=at["ring"])
                 torch.cuda.empty_cache()
             log(f"[bench] attention: {ex['attn_decode_ctx4096_bs1']} {ex['attn_decode_ctx4096_bs16']}")
+            ap = attn_prefill_workload(qk, 1024, 40, 8)   # the attention mixer over a 1,024-position prompt
+            ex["attn_prefill_1024_positions"] = dict(us=ap["ms_event"] * 1e3, tflops=ap["flops"] / (ap["ms_event"] * 1e-3) / 1e12,
+                                                     steps_timed=ap["steps"])
+            log(f"[bench] attention prefill: {ex['attn_prefill_1024_positions']}")
+            torch.cuda.empty_cache()
             for b in (1, 16):   # the gated-DeltaNet mixer's decode step
                 dn = deltanet_workload(qk, b, 256, 32)
                 gb = dn["bytes_step"] / (dn["ms_event"] * 1e-3) / 1e9

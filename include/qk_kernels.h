@@ -350,8 +350,10 @@ int qkk_dn_step(const float *conv, const float *gb, float *state, const float *n
  * the decode-step entry points called position by position.
  * qkk_attn_prep_seq  row t is written into the caches at positions[t] (distinct, ascending).
  * qkk_attn_seq       row t attends to the cache rows 0..positions[t]: causal over the rows of this
- *                    call and everything the cache held before.  Two consecutive rows share one scan
- *                    of the cache (not a scan blocked over 16 queries as the reference's). workspace: qkk_attn_workspace_bytes(n_pos, hQ, dh).
+ *                    call and everything the cache held before.  Three or more rows: a scan blocked
+ *                    over 16 rows and 4 query heads per workgroup, scores and values on the matrix
+ *                    cores (reference shaders/fa_attn_batch_coopmat.comp:58-183); two rows share one
+ *                    scan of the cache.  workspace: qkk_attn_workspace_bytes(n_pos, hQ, dh).
  * qkk_dn_conv_seq    the conv is a 4-tap filter over the inputs, so all positions run in parallel
  *                    (bit-identical to the steps); the window is moved on by a second small launch.
  * qkk_dn_step_seq    the state is read once, kept in registers over all positions (8 rows of a head

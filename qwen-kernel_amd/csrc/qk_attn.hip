@@ -23,6 +23,7 @@
 #include "qk_mfma.h"
 
 #include <math.h>
+#include <stdlib.h>
 
 #include <algorithm>
 
@@ -386,6 +387,237 @@ __global__ __launch_bounds__(256) void attn_range_pair_kernel(const float* __res
     }
 }
 
+// ---- sixteen consecutive rows of a sequence per workgroup (prompt prefill) ----------------------
+// Stands for the reference's blocked prefill attention (shaders/fa_attn_batch_coopmat.comp:58-183: 16
+// queries x 64 keys per iteration, both products on cooperative matrices).  grid (n_ranges, hKV *
+// ceil(G / 4), ceil(rows / 16)), 256 threads.  One workgroup takes SIXTEEN rows and FOUR of the G query
+// heads of one KV head over one position range, so every cached K and V row is fetched once for 64
+// query rows (the pair kernel above fetches it once per two rows of all G heads).  Wave w owns one
+// head from end to end -- scores, softmax, values -- so the running maximum, the sum and the
+// rescaling of the accumulators stay inside the wave (a query row's 16 scores of a key block lie in
+// the 16 lanes of one DPP row):
+//   K tile   64 keys as halves hi + lo in LDS, row-major (the B operand of Q.K^T reads 8 dims = 16 bytes);
+//   scores   S[query][key]: 4 key blocks x 8 steps of 32 dims x 3 products (hi.hi, hi.lo, lo.hi);
+//            Q (pre-scaled by 1/sqrt(dh), a power of two) stays in registers as hi + lo;
+//   softmax  in the MFMA output layout: lane (quad, col) holds rows 4*quad + e, key 16*kb + col;
+//   P        hi + lo halves through a wave-private LDS area into the A operand layout;
+//   V tile   in the K tile's place, TRANSPOSED ([dim][key]): the B operand of P.V reads 8 keys = 16 bytes;
+//   values   O[query][dim] += P.V: 16 dim blocks x 2 steps of 32 keys x 3 products, accumulators in
+//            registers (64), rescaled in place by exp(old max - new max).
+// Later keys are masked per row (a key is visible to row i iff it lies below pos[i] + 1), so any
+// positions work.  The (max, sum, accumulator) triples go to the same workspace as the other range
+// kernels' and attn_fold_kernel finishes the rows.
+constexpr uint32_t BLK_Q = 16;                    // rows per workgroup
+constexpr uint32_t BLK_KP = ATT_DH * 2 + 16;      // K tile row pitch in bytes (halves): 528
+constexpr uint32_t BLK_VP = ATT_TILE * 2 + 16;    // V^T tile row pitch in bytes: 144
+constexpr uint32_t BLK_PP = ATT_TILE * 2 + 16;    // P row pitch in bytes: 144
+constexpr uint32_t BLK_KV_BYTES = 2 * ATT_DH * BLK_VP;       // hi + lo of the larger tile (V^T): 73,728
+constexpr uint32_t BLK_P_BYTES = 2 * BLK_Q * BLK_PP;         // per wave: (hi, lo) x 16 rows: 4,608
+constexpr uint32_t BLK_LDS = BLK_KV_BYTES + 4 * BLK_P_BYTES; // 92,160
+static_assert(2 * ATT_TILE * BLK_KP <= BLK_KV_BYTES, "the K tile fits the V tile's area");
+
+typedef uint16_t __attribute__((may_alias)) lds_u16;
+typedef uint4 __attribute__((may_alias)) lds_u128;
+typedef uint2 __attribute__((may_alias)) lds_u64;
+
+__device__ __forceinline__ float dpp_row_max(float v) // maximum over the 16 lanes of a DPP row, in every lane
+{
+    v = fmaxf(v, dpp_f<DPP_XOR1>(v));
+    v = fmaxf(v, dpp_f<DPP_XOR2>(v));
+    v = fmaxf(v, dpp_f<DPP_HALF_MIRROR>(v));
+    return fmaxf(v, dpp_f<DPP_MIRROR>(v));
+}
+
+__global__ __launch_bounds__(256) void attn_block_kernel(const float* __restrict__ qhat, const float* __restrict__ kc,
+                                                         const float* __restrict__ vc,
+                                                         const uint32_t* __restrict__ slot_pos, AttnWs ws, uint32_t hQ,
+                                                         uint32_t hKV, uint32_t G, uint32_t tmax, uint32_t rows)
+{
+    QK_DYN_LDS(uint8_t, s_blk);
+    constexpr uint32_t KS = ATT_DH / 32; // 32-dim steps of a row
+    const uint32_t n_ranges = gridDim.x, c = blockIdx.x, r0 = BLK_Q * blockIdx.z, t = threadIdx.x;
+    const uint32_t hgroups = (G + 3) / 4, kv = blockIdx.y / hgroups, hg = blockIdx.y % hgroups;
+    const uint32_t lane = t & 63u, wave = t >> 6, col = lane & 15u, quad = lane >> 4;
+    const uint32_t nq = min(BLK_Q, rows - r0);
+    // keys visible to the rows this lane holds in the output layout (rows 4 * quad + e), and to any row
+    uint32_t n_row[4], n_max = 0;
+#pragma unroll
+    for (uint32_t e = 0; e < 4; e++) n_row[e] = 4 * quad + e < nq ? slot_position(slot_pos, r0 + 4 * quad + e, tmax) + 1u : 0u;
+    for (uint32_t i = 0; i < nq; i++) n_max = max(n_max, slot_position(slot_pos, r0 + i, tmax) + 1u);
+    const uint32_t per = (tmax + n_ranges - 1) / n_ranges;
+    const uint32_t p_begin = c * per, p_end = min(n_max, p_begin + per);
+    if (p_begin >= n_max) return; // the whole workgroup: this range holds no key of any row
+
+    uint8_t* s_kv = s_blk;                                    // K tile (hi, lo), then the V^T tile (hi, lo)
+    uint8_t* s_p = s_blk + BLK_KV_BYTES + wave * BLK_P_BYTES; // this wave's P: [hi, lo][row][key]
+    const uint32_t hq_in = 4 * hg + wave;                     // this wave's head among the G of the KV head
+    const bool has = hq_in < G;                               // uniform per wave; a wave without a head still stages tiles
+    const uint32_t head = kv * G + min(hq_in, G - 1);
+
+    // Q operand: lane feeds A[row = col][dims 32 * ks + 8 * quad .. + 7], scaled by 1/sqrt(dh)
+    half8 qh[KS], ql[KS];
+    const float qs = 1.f / sqrtf((float)ATT_DH);
+#pragma unroll
+    for (uint32_t ks = 0; ks < KS; ks++) {
+        float4 a = float4{0.f, 0.f, 0.f, 0.f}, b = a;
+        if (col < nq) {
+            const float4* qrow = (const float4*)(qhat + ((size_t)(r0 + col) * hQ + head) * ATT_DH);
+            a = qrow[ks * 8 + 2 * quad];
+            b = qrow[ks * 8 + 2 * quad + 1];
+        }
+        const HalfSplit sp = split8(float4{a.x * qs, a.y * qs, a.z * qs, a.w * qs},
+                                    float4{b.x * qs, b.y * qs, b.z * qs, b.w * qs});
+        qh[ks] = sp.hi;
+        ql[ks] = sp.lo;
+    }
+    float4v o[ATT_DH / 16];
+    float m_run[4], l_run[4];
+#pragma unroll
+    for (uint32_t db = 0; db < ATT_DH / 16; db++) o[db] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (uint32_t e = 0; e < 4; e++) { m_run[e] = ATT_FLOOR; l_run[e] = 0.f; }
+    const float4* kbase = (const float4*)(kc + (size_t)kv * tmax * ATT_DH); // one slot's caches
+    const float4* vbase = (const float4*)(vc + (size_t)kv * tmax * ATT_DH);
+
+    // staging of a tile: wave w fetches the rows 16 w .. 16 w + 15
+    //   K: one row per instruction, lane = 4 dims (a row is 64 consecutive float4)
+    //   V: lane = (key 16 w + lane % 16, dims 4 * (lane / 16 + 4 * i)), so that the transposed 2-byte stores of
+    //      16 lanes fall on consecutive keys
+    float4 stage[16];
+    auto fetch_k = [&](uint32_t p0, uint32_t ts) {
+#pragma unroll
+        for (uint32_t i = 0; i < 16; i++)
+            stage[i] = kbase[(size_t)(p0 + min(16 * wave + i, ts - 1)) * (ATT_DH / 4) + lane];
+    };
+    auto fetch_v = [&](uint32_t p0, uint32_t ts) {
+        const size_t row = p0 + min(16 * wave + col, ts - 1);
+#pragma unroll
+        for (uint32_t i = 0; i < 16; i++) stage[i] = vbase[row * (ATT_DH / 4) + quad + 4 * i];
+    };
+    auto split4 = [](float4 v, uint2& hi, uint2& lo) {
+        const auto h0 = __builtin_amdgcn_cvt_pkrtz(v.x, v.y), h1 = __builtin_amdgcn_cvt_pkrtz(v.z, v.w);
+        const auto l0 = __builtin_amdgcn_cvt_pkrtz(v.x - (float)h0[0], v.y - (float)h0[1]);
+        const auto l1 = __builtin_amdgcn_cvt_pkrtz(v.z - (float)h1[0], v.w - (float)h1[1]);
+        hi = uint2{__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1)};
+        lo = uint2{__builtin_bit_cast(uint32_t, l0), __builtin_bit_cast(uint32_t, l1)};
+    };
+
+    fetch_k(p_begin, min(ATT_TILE, p_end - p_begin));
+    for (uint32_t p0 = p_begin; p0 < p_end; p0 += ATT_TILE) {
+        const uint32_t ts = min(ATT_TILE, p_end - p0);
+        __syncthreads(); // the previous tile's V has been consumed
+        // K tile: [key][dim] halves, hi at 0, lo behind it
+#pragma unroll
+        for (uint32_t i = 0; i < 16; i++) {
+            uint2 hi, lo;
+            split4(stage[i], hi, lo);
+            const uint32_t at = (16 * wave + i) * BLK_KP + lane * 8;
+            *(lds_u64*)(s_kv + at) = hi;
+            *(lds_u64*)(s_kv + ATT_TILE * BLK_KP + at) = lo;
+        }
+        fetch_v(p0, ts); // in flight during the scores
+        __syncthreads();
+
+        if (has) {
+            float4v sc[4];
+#pragma unroll
+            for (uint32_t kb = 0; kb < 4; kb++) {
+                sc[kb] = float4v{0.f, 0.f, 0.f, 0.f};
+                const uint32_t at = (16 * kb + col) * BLK_KP + quad * 16;
+#pragma unroll
+                for (uint32_t ks = 0; ks < KS; ks++) {
+                    const half8 kh = __builtin_bit_cast(half8, *(const lds_u128*)(s_kv + at + ks * 64));
+                    const half8 kl = __builtin_bit_cast(half8, *(const lds_u128*)(s_kv + ATT_TILE * BLK_KP + at + ks * 64));
+                    sc[kb] = mfma16x32(qh[ks], kh, sc[kb]);
+                    sc[kb] = mfma16x32(qh[ks], kl, sc[kb]);
+                    sc[kb] = mfma16x32(ql[ks], kh, sc[kb]);
+                }
+            }
+            // sc[kb][e]: row 4 * quad + e, key p0 + 16 * kb + col
+#pragma unroll
+            for (uint32_t e = 0; e < 4; e++) {
+                float mx = ATT_FLOOR;
+                bool vis[4];
+#pragma unroll
+                for (uint32_t kb = 0; kb < 4; kb++) {
+                    const uint32_t key = p0 + 16 * kb + col;
+                    vis[kb] = key < p_end && key < n_row[e];
+                    if (vis[kb]) mx = fmaxf(mx, sc[kb][e]);
+                }
+                const float new_m = fmaxf(m_run[e], dpp_row_max(mx));
+                const float corr = expf(m_run[e] - new_m);
+                float sum = 0.f;
+#pragma unroll
+                for (uint32_t kb = 0; kb < 4; kb++) {
+                    const float pv = vis[kb] ? expf(sc[kb][e] - new_m) : 0.f;
+                    sum += pv;
+                    const _Float16 hi = (_Float16)pv;   // round to nearest; the rest is exact in fp32
+                    const _Float16 lo = (_Float16)(pv - (float)hi);
+                    const uint32_t at = (4 * quad + e) * BLK_PP + (16 * kb + col) * 2;
+                    *(lds_u16*)(s_p + at) = __builtin_bit_cast(uint16_t, hi);
+                    *(lds_u16*)(s_p + BLK_Q * BLK_PP + at) = __builtin_bit_cast(uint16_t, lo);
+                }
+                l_run[e] = l_run[e] * corr + group_sum<16>(sum);
+                m_run[e] = new_m;
+#pragma unroll
+                for (uint32_t db = 0; db < ATT_DH / 16; db++) o[db][e] *= corr;
+            }
+        }
+        __syncthreads(); // every wave has read the K tile
+        // V^T tile: [dim][key] halves, hi at 0, lo behind it
+#pragma unroll
+        for (uint32_t i = 0; i < 16; i++) {
+            uint2 hi, lo;
+            split4(stage[i], hi, lo);
+            const uint32_t d0 = 4 * (quad + 4 * i), at = d0 * BLK_VP + (16 * wave + col) * 2;
+            *(lds_u16*)(s_kv + at) = (uint16_t)(hi.x & 0xFFFFu);
+            *(lds_u16*)(s_kv + at + BLK_VP) = (uint16_t)(hi.x >> 16);
+            *(lds_u16*)(s_kv + at + 2 * BLK_VP) = (uint16_t)(hi.y & 0xFFFFu);
+            *(lds_u16*)(s_kv + at + 3 * BLK_VP) = (uint16_t)(hi.y >> 16);
+            *(lds_u16*)(s_kv + ATT_DH * BLK_VP + at) = (uint16_t)(lo.x & 0xFFFFu);
+            *(lds_u16*)(s_kv + ATT_DH * BLK_VP + at + BLK_VP) = (uint16_t)(lo.x >> 16);
+            *(lds_u16*)(s_kv + ATT_DH * BLK_VP + at + 2 * BLK_VP) = (uint16_t)(lo.y & 0xFFFFu);
+            *(lds_u16*)(s_kv + ATT_DH * BLK_VP + at + 3 * BLK_VP) = (uint16_t)(lo.y >> 16);
+        }
+        if (p0 + ATT_TILE < p_end) fetch_k(p0 + ATT_TILE, min(ATT_TILE, p_end - p0 - ATT_TILE)); // in flight during the values
+        __syncthreads();
+
+        // values: O[row][dim] += P[row][key] . V[key][dim]; the weights of masked keys are zero
+        if (has) {
+            half8 pa_h[2], pa_l[2];
+#pragma unroll
+            for (uint32_t ks = 0; ks < 2; ks++) { // A[row = col][keys 32 * ks + 8 * quad .. + 7]
+                const uint32_t at = col * BLK_PP + (32 * ks + 8 * quad) * 2;
+                pa_h[ks] = __builtin_bit_cast(half8, *(const lds_u128*)(s_p + at));
+                pa_l[ks] = __builtin_bit_cast(half8, *(const lds_u128*)(s_p + BLK_Q * BLK_PP + at));
+            }
+#pragma unroll
+            for (uint32_t db = 0; db < ATT_DH / 16; db++) {
+#pragma unroll
+                for (uint32_t ks = 0; ks < 2; ks++) { // B[keys 32 * ks + 8 * quad .. + 7][dim = 16 * db + col]
+                    const uint32_t at = (16 * db + col) * BLK_VP + (32 * ks + 8 * quad) * 2;
+                    const half8 vh = __builtin_bit_cast(half8, *(const lds_u128*)(s_kv + at));
+                    const half8 vl = __builtin_bit_cast(half8, *(const lds_u128*)(s_kv + ATT_DH * BLK_VP + at));
+                    o[db] = mfma16x32(pa_h[ks], vh, o[db]);
+                    o[db] = mfma16x32(pa_h[ks], vl, o[db]);
+                    o[db] = mfma16x32(pa_l[ks], vh, o[db]);
+                }
+            }
+        }
+    }
+    // the range's triples: o[db][e] is row 4 * quad + e, dim 16 * db + col
+    if (!has) return;
+#pragma unroll
+    for (uint32_t e = 0; e < 4; e++) {
+        const uint32_t i = 4 * quad + e;
+        if (i >= nq) continue;
+        const size_t slot = ((size_t)(r0 + i) * hQ + head) * n_ranges + c;
+#pragma unroll
+        for (uint32_t db = 0; db < ATT_DH / 16; db++) ws.acc[slot * ATT_DH + 16 * db + col] = o[db][e];
+        if (col == 0) { ws.ml[2 * slot] = m_run[e]; ws.ml[2 * slot + 1] = l_run[e]; }
+    }
+}
+
 // grid (hQ, slots), 256 threads: folds the ranges of one query head in range order, divides by the
 // sum and applies the output gate sigmoid(qfull[head][dh + t]).  Wave w adds the ranges w, w+4, ...
 // (a lane 4 dims, eight ranges requested at a time); the waves' sums are added in wave order.
@@ -530,11 +762,24 @@ static int attn_decode_impl(const char* who, const float* qhat, const float* k_c
     // two workgroups per CU over the (row, KV head) pairs, 8..64 ranges each: 16 slots x 4096 positions
     // measured 4.5 TB/s with 16 ranges, 4.2 with 32, 3.1 with 128 (the partial results are traffic too);
     // one slot 0.98 TB/s with 64 ranges, 0.80 with 32
-    const uint32_t n_ranges = std::min(max_ranges(rows), std::max(8u, persistent_blocks() / 2 / (rows * hKV)));
+    uint32_t n_ranges = std::min(max_ranges(rows), std::max(8u, persistent_blocks() / 2 / (rows * hKV)));
+    // three or more consecutive rows of one slot: blocks of sixteen rows (QK_ATTN_PAIR=1 keeps the pair kernel);
+    // one workgroup per CU (LDS), so about as many (block, KV head, range) triples as there are CUs
+    static const bool pair_only = getenv("QK_ATTN_PAIR") != nullptr;
+    const bool blocked = own == 0 && rows >= 3 && !pair_only;
+    const uint32_t blocks = (rows + BLK_Q - 1) / BLK_Q;
+    const uint32_t hgroups = (hQ / hKV + 3) / 4; // four query heads of a KV head per workgroup
+    if (blocked) n_ranges = std::min(max_ranges(rows), std::max(1u, persistent_blocks() / 4 / (blocks * hKV * hgroups)));
     AttnWs ws;
     ws.acc = (float*)workspace;
     ws.ml = ws.acc + (size_t)rows * hQ * n_ranges * ATT_DH;
-    if (own == 0 && rows >= 2)
+    if (blocked) {
+        static bool once = ((void)hipFuncSetAttribute((const void*)attn_block_kernel,
+                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)BLK_LDS), true);
+        (void)once;
+        hipLaunchKernelGGL(attn_block_kernel, dim3(n_ranges, hKV * hgroups, blocks), dim3(256), BLK_LDS, st, qhat, k_cache, v_cache,
+                           slot_pos, ws, hQ, hKV, hQ / hKV, tmax, rows);
+    } else if (own == 0 && rows >= 2)
         hipLaunchKernelGGL(attn_range_pair_kernel, dim3(n_ranges, hKV, (rows + 1) / 2), dim3(256), 0, st, qhat, k_cache,
                            v_cache, slot_pos, ws, hQ, hKV, hQ / hKV, tmax, rows);
     else

@@ -114,19 +114,51 @@ class HostLayer:
 
 
 def device_layer(seed, n_embd=2048, n_ff=512, n_expert=256, n_used=8, down_type=IQ4_XS, device="cuda",
-                 d_scale=1e-3):
-    """Synthetic MoE layer generated directly in device memory."""
+                 d_scale=1e-3, slab=None):
+    """Synthetic MoE layer generated directly in device memory.  slab: a Slab the tensors are carved from
+    (every layer of a ring in ONE device allocation) instead of an allocation per tensor."""
     import torch
     from .capi import MoeLayer
     g = torch.Generator(device=device)
     g.manual_seed(seed)
     H, F, E = n_embd, n_ff, n_expert
-    gi = torch.randn((E, H), device=device, generator=g) * (2.0 / H ** 0.5)
-    gis = torch.randn(H, device=device, generator=g) * (1.0 / H ** 0.5)
+    keep = (lambda x: slab.take(x)) if slab is not None else (lambda x: x)
+    gi = keep(torch.randn((E, H), device=device, generator=g) * (2.0 / H ** 0.5))
+    gis = keep(torch.randn(H, device=device, generator=g) * (1.0 / H ** 0.5))
 
     def t(type_, rows, k, s):
-        return blocks_device(type_, rows * (k // BLOCK[type_][0]), s, device, d_scale).reshape(-1)
+        return keep(blocks_device(type_, rows * (k // BLOCK[type_][0]), s, device, d_scale).reshape(-1))
 
     return MoeLayer(H, F, E, n_used, down_type, gi, gis, t(IQ3_XXS, E * F, H, seed + 1),
                     t(IQ3_XXS, E * F, H, seed + 2), t(down_type, E * H, F, seed + 3), t(Q8_0, F, H, seed + 4),
                     t(Q8_0, F, H, seed + 5), t(Q8_0, H, F, seed + 6))
+
+
+def layer_bytes(n_embd=2048, n_ff=512, n_expert=256, down_type=IQ4_XS):
+    """Bytes of one synthetic layer's tensors, each rounded up to 256."""
+    from .capi import row_bytes
+    H, F, E = n_embd, n_ff, n_expert
+    sizes = [E * H * 4, H * 4, 2 * E * F * row_bytes(IQ3_XXS, H), E * H * row_bytes(down_type, F),
+             2 * F * row_bytes(Q8_0, H), H * row_bytes(Q8_0, F)]
+    return sum((b + 255) // 256 * 256 for b in sizes) + 4 * 256
+
+
+class Slab:
+    """One device allocation that tensors are copied into back to back (256-byte aligned): a ring of
+    layers then lies in one mapping, as the tensors of a model file uploaded into one buffer would."""
+
+    def __init__(self, nbytes, device="cuda"):
+        import torch
+        self.buf = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        self.at = 0
+
+    def take(self, t):
+        import torch
+        raw = t.contiguous().view(torch.uint8).reshape(-1)
+        n = raw.numel()
+        if self.at + n > self.buf.numel():
+            raise ValueError("Slab: full")
+        view = self.buf[self.at:self.at + n]
+        view.copy_(raw)
+        self.at += (n + 255) // 256 * 256
+        return view.view(t.dtype).reshape(t.shape)

@@ -35,16 +35,16 @@ def dev(qk):
         qk.capi._lib = emu_util.emu_lib(qk)
         qk.capi._stream = lambda: None
         torch.cuda.synchronize = lambda *a, **k: None
-        plain_zeros = torch.zeros
-
-        def zeros(*a, **k):   # workspaces must be 256-byte aligned; host allocations are 64-byte aligned
-            t = plain_zeros(*a, **k)
-            if t.dtype == torch.uint8 and t.dim() == 1 and t.data_ptr() % 256:
-                big = plain_zeros(t.numel() + 256, dtype=torch.uint8)
-                off = (-big.data_ptr()) % 256
-                return big[off:off + t.numel()]
-            return t
-        torch.zeros = zeros
+        def aligned(plain):   # workspaces must be 256-byte aligned; host allocations are 64-byte aligned
+            def make(*a, **k):
+                t = plain(*a, **k)
+                if t.dtype == torch.uint8 and t.dim() == 1 and t.data_ptr() % 256:
+                    big = plain(t.numel() + 256, dtype=torch.uint8)
+                    off = (-big.data_ptr()) % 256
+                    return big[off:off + t.numel()]
+                return t
+            return make
+        torch.zeros, torch.empty = aligned(torch.zeros), aligned(torch.empty)
         print("[emu] kernels run in the host-side build", flush=True)
         return "cpu"
     if not torch.cuda.is_available():

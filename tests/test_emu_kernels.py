@@ -177,3 +177,32 @@ def test_head_norm_inside_its_tensors(qk, orc, emu):
     want = orc.gemv(qk.Q6_K, W, orc.add_rms(x[0], w, 1e-6), V, K)
     assert orc.rel_maxabs_err(logits.numpy()[0], want) <= 1e-3
     assert int(tok.numpy()[0]) == int(np.argmax(want))
+
+
+@pytest.mark.parametrize("hq,hkv,base,n_pos", [(16, 2, 0, 16), (8, 2, 45, 19), (3, 1, 60, 4)])
+def test_attention_blocks_inside_their_tensors(qk, emu, hq, hkv, base, n_pos):
+    """The sixteen-row attention kernel on caches whose LAST row is the last position fed (tmax = base +
+    n_pos) and that end at the guard page, against the CPU mirror."""
+    import os
+    import sys
+    import torch
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle"))
+    import qk_oracle_attn as OA
+    DH, NROT, tmax = 256, 64, base + n_pos
+    rng = np.random.default_rng(hq + n_pos)
+    rope = OA.rope_table(tmax, NROT)
+    kc, vc = np.zeros((hkv, tmax, DH), np.float32), np.zeros((hkv, tmax, DH), np.float32)
+    kc[:, :base], vc[:, :base] = rng.standard_normal((hkv, base, DH)), rng.standard_normal((hkv, base, DH))
+    qn, kn = (1 + 0.2 * rng.standard_normal(DH)).astype(np.float32), (1 + 0.2 * rng.standard_normal(DH)).astype(np.float32)
+    qfull = (rng.standard_normal((n_pos, hq, 2 * DH)) * 2).astype(np.float32)
+    kin, vin = rng.standard_normal((n_pos, hkv, DH)).astype(np.float32), rng.standard_normal((n_pos, hkv, DH)).astype(np.float32)
+    kd, vd, qfd = emu.tensor(kc[None]), emu.tensor(vc[None]), emu.tensor(qfull)
+    pos = emu.tensor(np.arange(base, base + n_pos, dtype=np.int32))
+    ws = emu.workspace(qk.attn_workspace_bytes(n_pos, hq))
+    qh = qk.attn_prep(qfd, emu.tensor(kin), emu.tensor(vin), emu.tensor(qn), emu.tensor(kn), emu.tensor(rope), pos, kd, vd, NROT,
+                      qhat=emu.zeros((n_pos, hq, DH), np.float32), seq=True)
+    att = qk.attn_decode(qh, kd, vd, qfd, pos, ws, att=emu.zeros((n_pos, hq, DH), np.float32), seq=True).numpy()
+    for t in range(n_pos):
+        want = OA.attend(OA.prep(qfull[t], kin[t], vin[t], qn, kn, rope, base + t, kc, vc, NROT), kc, vc, qfull[t], base + t)
+        err = float(np.max(np.abs(att[t].astype(np.float64) - want)) / np.max(np.abs(want)))
+        assert err <= 1e-3, (t, err)

@@ -150,6 +150,48 @@ def test_whole_model_long_prompt_and_long_stage_run(qk, full, monkeypatch):
         assert rc == 0 and ids == want
 
 
+def test_whole_model_stream_alone_and_among_fifteen_neighbours(qk, full):
+    """The same request on slot 0 alone (dispatch depth 1: the one-row kernels) and with fifteen busy
+    neighbours (depth 16: projections, MoE block and head on the matrix cores).  The kernel families sum
+    in different orders, so the greedy streams may part -- but only at a step whose two best logits nearly
+    tie: the streams must agree up to the first difference, and there qk_stage_topk over the common prefix
+    must show the two ids as its two best, closer together than 2e-3 of the largest logit."""
+    model, path = full
+    print("[case] whole model, one stream alone and among fifteen neighbours", flush=True)
+    rng = np.random.default_rng(77)
+    P = lambda n: [int(t) for t in rng.integers(0, VOCAB, n)]
+    prompt, n_gen = P(6), 10
+
+    def stream_of_slot_0(eng):
+        got = []
+        for _ in range(40):
+            rc, out, fin = eng.step_chunk()
+            assert rc >= 0
+            got += out[0]
+            if fin & 1:
+                return got
+        raise AssertionError("slot 0 did not finish")
+
+    with qk.engine.Engine(path, n_slots=16, n_ctx=64, chunk=4) as eng:
+        assert eng.slot_start(0, prompt, n_gen) == 0
+        alone = stream_of_slot_0(eng)
+        for s in range(1, 16):
+            assert eng.slot_start(s, P(2 + s % 5), 40) == 0
+        assert eng.slot_start(0, prompt, n_gen) == 0
+        crowd = stream_of_slot_0(eng)
+        for s in range(1, 16):
+            eng.slot_cancel(s)
+        assert len(alone) == len(crowd) == n_gen   # the end id lies outside the vocabulary: both run to max_gen
+        j = next((i for i, (a, b) in enumerate(zip(alone, crowd)) if a != b), None)
+        print(f"[info] alone {alone}\n[info] crowd {crowd}\n[info] first difference at {j}", flush=True)
+        if j is not None:
+            rc, _ = eng.stage_run(0, prompt + alone[:j], 0)
+            assert rc == 0
+            rc, top_ids, top_vals = eng.stage_topk(3)
+            assert rc == 0 and {alone[j], crowd[j]} == set(top_ids[:2]), (j, alone[j], crowd[j], top_ids, top_vals)
+            assert top_vals[0] - top_vals[1] <= 2e-3 * max(abs(v) for v in top_vals), (j, top_ids, top_vals)
+
+
 @pytest.mark.parametrize("ba", ["f32", "q8_0", "iq4_xs"])
 def test_whole_model_fused_ssm_ba(qk, orc, dev, ba, tmp_path):
     """A file that holds the decay / write-strength weights of its gated-DeltaNet layers as ONE interleaved
