@@ -24,7 +24,7 @@ sys.path.insert(0, ROOT)
 import __graft_entry__ as entry  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0
-MIN_REPLAYS = 10   # graph replays timed at least, whatever --steps says (steps timed = replays x ring, reported)
+MIN_REPLAYS = 20   # graph replays timed at least, whatever --steps says (steps timed = replays x ring, reported)
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by what the same
 # counters read for a plain 256 MiB copy (profiles/); None where no counter run of the CURRENT kernel
 # has been recorded (a figure of an earlier version of a kernel is not carried over).
@@ -74,23 +74,25 @@ class Graphed:
 
 def run_ring(launches, steps, warmup):
     """Times `steps` launches (a multiple of the ring) bracketed by synchronize.  Returns
-    (ms_per_step wall, ms_per_step by events)."""
+    (ms_per_step by the host clock over the whole region, MEDIAN ms_per_step over the graph replays by HIP
+    events on the launch stream, steps timed).  At least MIN_REPLAYS replays are timed."""
     import torch
     g = Graphed(launches)
-    reps = max(MIN_REPLAYS, steps // g.n)   # never a single replay: a driver's small --steps still times ten
+    reps = max(MIN_REPLAYS, steps // g.n)   # never a single replay: a driver's small --steps still times twenty
     for _ in range(max(1, warmup // g.n)):
         g.replay()
     torch.cuda.synchronize()
-    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
     t0 = time.perf_counter()
-    a.record()
-    for _ in range(reps):
+    marks[0].record()   # replays and events both go to torch's current stream
+    for r in range(reps):
         g.replay()
-    b.record()
+        marks[r + 1].record()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
+    per = sorted(marks[r].elapsed_time(marks[r + 1]) for r in range(reps))
     n = reps * g.n
-    return (t1 - t0) * 1e3 / n, a.elapsed_time(b) / n, n
+    return (t1 - t0) * 1e3 / n, per[reps // 2] / g.n, n
 
 
 # ---- workloads -------------------------------------------------------------------------------
@@ -645,7 +647,8 @@ def main():
                            ring_layers=m["ring"], ring_bytes=m["ring_bytes"],
                            steps_timed=m["steps"], graph_replays_timed=m["steps"] // m["ring"],
                            timing=f"hipGraph replays of the ring (one launch set per layer of the ring), at least "
-                                  f"{MIN_REPLAYS} replays whatever --steps asks"),
+                                  f"{MIN_REPLAYS} replays whatever --steps asks; value from the host clock over all of them, "
+                                  f"us_per_step_events the median replay by HIP events"),
                us_per_step=m["ms_wall"] * 1e3, us_per_step_events=m["ms_event"] * 1e3,
                bytes_per_step=m["bytes_step"], frac_of_hbm_peak=gbps / HBM_PEAK_GBPS,
                distinct_experts_per_step=m["distinct_experts"],

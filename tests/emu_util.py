@@ -14,6 +14,7 @@ EMU_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "emu")
 EMU_LIB = os.path.join(EMU_DIR, "libqk_emu.so")
 
 _emu = None
+plain_from_numpy = None   # set where torch.from_numpy is replaced by a copying one (the GPU tests' emu mode)
 
 
 def build_emu():
@@ -53,7 +54,7 @@ class GuardPool:
         raw = np.ctypeslib.as_array((C.c_uint8 * max(n, 1)).from_address(p))[:n]
         view = raw.view(arr.dtype).reshape(arr.shape)
         view[...] = arr
-        return torch.from_numpy(view)
+        return (plain_from_numpy or torch.from_numpy)(view)
 
     def zeros(self, shape, dtype, align=16):
         return self.tensor(np.zeros(shape, dtype=dtype), align)
