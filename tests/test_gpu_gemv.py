@@ -94,6 +94,32 @@ def test_gemv_dense(qk, orc, dev, name, M, K, batch):
     run_case(qk, orc, dev, name, M, K, batch)
 
 
+@pytest.mark.parametrize("name", ["q8_0", "q6_k", "iq4_xs", "iq3_xxs", "f16", "f32"])
+@pytest.mark.parametrize("batch", [1, 16])
+def test_gemv_full_size_scaling_and_linearity(qk, orc, dev, name, batch):
+    """Size-independent properties at the benchmark's shape (8192 x 2048): doubling x doubles every sum
+    -- exactly on the fp32 paths (a power of two changes no rounding; the formats that split x into two
+    halves, and the several-row matrix-core path, round the low half differently: 1e-6 there) -- and
+    W.(x1 + x2) = W.x1 + W.x2 to fp32 rounding."""
+    import torch
+    print(f"[case] gemv properties {name} batch={batch}", flush=True)
+    M, K, t = 8192, 2048, TYPES[name]
+    W = torch.from_numpy(qk.synth.tensor_host(t, M, K, 7)).to(dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(3)
+    x1, x2 = torch.randn((batch, K), device=dev, generator=g), torch.randn((batch, K), device=dev, generator=g)
+    y1, y2 = qk.gemv(t, W, x1, M, K), qk.gemv(t, W, x2, M, K)
+    y1d, y12 = qk.gemv(t, W, (2 * x1).contiguous(), M, K), qk.gemv(t, W, (x1 + x2).contiguous(), M, K)
+    torch.cuda.synchronize()
+    scale = float(y1.abs().max())
+    exact = batch == 1 and name in ("q8_0", "q6_k", "f16", "f32")
+    if exact:
+        assert torch.equal(y1d, 2 * y1)
+    else:
+        assert float((y1d - 2 * y1).abs().max()) <= 1e-6 * scale
+    assert float((y12 - (y1 + y2)).abs().max()) <= 2e-5 * scale
+
+
 def test_gemv_is_deterministic(qk, orc, dev):
     a = run_case(qk, orc, dev, "iq3_xxs", 4096, 2048, 1, seed=9)
     b = run_case(qk, orc, dev, "iq3_xxs", 4096, 2048, 1, seed=9)

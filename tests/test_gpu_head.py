@@ -70,6 +70,25 @@ def test_head_with_the_norm_in_front(qk, orc, dev, V):
     assert int(tok2.cpu()[0]) == int(tok.cpu()[0])
 
 
+def test_head_full_vocab_scaling_is_exact(qk, dev):
+    """At the full vocabulary (151,936 x 2048): doubling the activation row doubles every logit exactly
+    (a power of two changes no rounding on the fp32 path) and leaves the token unchanged; so does the
+    row given twice in a batch of one call each."""
+    import torch
+    print("[case] head properties at the full vocabulary", flush=True)
+    V, K = 151936, 2048
+    W = qk.synth.blocks_device(qk.Q6_K, V * (K // 256), 21, dev).reshape(-1)
+    g = torch.Generator(device=dev)
+    g.manual_seed(4)
+    x = torch.randn((1, K), device=dev, generator=g)
+    ws = torch.zeros(qk.head_workspace_bytes(V, 1), dtype=torch.uint8, device=dev)
+    tok, logits = qk.head_argmax(W, x, V, K, ws, want_logits=True)
+    tok2, logits2 = qk.head_argmax(W, (2 * x).contiguous(), V, K, ws, want_logits=True)
+    torch.cuda.synchronize()
+    assert torch.equal(logits2, 2 * logits) and int(tok2[0]) == int(tok[0])
+    assert int(tok[0]) == int(torch.argmax(logits[0]))
+
+
 def test_head_ties_pick_lowest_id(qk, dev):
     import torch
     print("[case] head ties", flush=True)

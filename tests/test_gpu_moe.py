@@ -454,6 +454,32 @@ def test_rows_up_to_the_rowwise_limit_do_not_depend_on_company(qk, dev, layer_iq
     assert e.value.code == -2
 
 
+@pytest.mark.parametrize("n", [16, 40])
+def test_expert_major_rows_do_not_depend_on_company(qk, dev, layer_q6k, n):
+    """The expert-major path (more than ROWWISE_MAX rows) groups the rows' picks by expert, sixteen pairs to
+    a matrix-core tile -- but a row's sums never mix with its tile companions' and the picks are folded in
+    pick order, so a row's result does not depend on which rows it is batched with or where it stands:
+    the rows permuted give the outputs permuted, and a subset of the rows (still above the limit) gives
+    the subset of the outputs, bit for bit."""
+    import torch
+    print(f"[case] expert-major rows and their company, {n} rows", flush=True)
+    layer = layer_q6k.to_device(dev)
+    g = torch.Generator(device=dev)
+    g.manual_seed(n)
+    X = torch.randn((n, 2048), device=dev, generator=g)
+    ws = torch.zeros(qk.moe_workspace_bytes(layer, n), dtype=torch.uint8, device=dev)
+    Y, sel = qk.moe_decode(layer, X, ws)
+    Y, sel = Y.clone(), sel.clone()
+    perm = torch.randperm(n, device=dev, generator=g)
+    Yp, selp = qk.moe_decode(layer, X[perm].contiguous(), ws)
+    torch.cuda.synchronize()
+    assert torch.equal(selp, sel[perm]) and torch.equal(Yp, Y[perm])
+    m = qk.ROWWISE_MAX + 1
+    Ys, sels = qk.moe_decode(layer, X[n - m:].contiguous(), ws)   # the last eleven rows alone
+    torch.cuda.synchronize()
+    assert torch.equal(sels, sel[n - m:]) and torch.equal(Ys, Y[n - m:])
+
+
 def test_one_workspace_serves_changing_row_counts(qk, dev, layer_q6k):
     """An engine keeps one workspace and its step's row count changes from call to call (both
     paths, whose workspace areas lie at offsets that depend on the row count): every call must give
