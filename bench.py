@@ -606,6 +606,21 @@ def main():
                                           ring=at["ring"]),
                               bytes_per_step=at["bytes_step"], frac_of_hbm_peak=gb / HBM_PEAK_GBPS)), flush=True)
         return
+    if a.workload == "gemv_sustained":   # every block format at a sustained size and at the 8192 x 2048 shape
+        res = {}
+        for name, t in (("q8_0", qk.Q8_0), ("q6_k", qk.Q6_K), ("iq4_xs", qk.IQ4_XS), ("iq3_xxs", qk.IQ3_XXS)):
+            Ms = -(-(256 << 20) // qk.row_bytes(t, 2048) // 64) * 64
+            for label, M, ring in ((f"gemv_{name}_sustained_256MiB", Ms, 2), (f"gemv_{name}_8192x2048", 8192, None)):
+                g = gemv_workload(qk, t, M, 2048, 1, 40 if ring else 400, 4 if ring else 40, ring=ring)
+                gb = g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9
+                res[label] = dict(us=g["ms_event"] * 1e3, gbps=gb, frac=gb / HBM_PEAK_GBPS, steps_timed=g["steps"])
+                torch.cuda.empty_cache()
+        print(json.dumps(dict(metric="gemv_hbm_gbps", value=res["gemv_q8_0_sustained_256MiB"]["gbps"], unit="GB/s", n_gpus=1,
+                              higher_is_better=True, data="synthetic", dtype="f32",
+                              config=dict(workload="gemv_sustained", K=2048, env={k: v for k, v in os.environ.items()
+                                                                                   if k.startswith("QK_")}),
+                              detail=res)), flush=True)
+        return
     if a.workload in ("head_bs1", "head_bs16"):   # the LM head alone (for counter runs on its kernel)
         b = 1 if a.workload == "head_bs1" else 16
         h = head_workload(qk, 151936, 2048, b, min(a.steps, 40), min(a.warmup, 8))

@@ -342,6 +342,16 @@ int qkk_dn_ab_conv_norm(const float *x, const float *w_norm, float norm_eps, con
 int qkk_dn_step(const float *conv, const float *gb, float *state, const float *norm_w, const float *z,
                 float *att, uint32_t d_state, uint32_t hK, uint32_t hV, uint32_t kdiv, float eps,
                 uint32_t n_slots, void *stream);
+/* The decode step of the mixer in ONE launch: qkk_dn_ab_conv (with the norm in front when w_norm is given,
+ * NULL otherwise) and qkk_dn_step, same arithmetic in the same order, same results bit for bit; conv and gb
+ * never touch memory.  A workgroup takes the two value heads of one key head (they share the q / k conv
+ * window, which is shifted once), so hV = 2 hK is required (the reference's 32 on 16; kdiv 0 or 2),
+ * n_embd 2048.  conv_state [slots][(2 hK + hV) dS][3], qkv [slots][(2 hK + hV) dS]. */
+int qkk_dn_step_fused(const float *x, const float *w_norm, float norm_eps, const float *alpha_w,
+                      const float *beta_w, const float *dt_bias, const float *a_vec, uint32_t n_embd,
+                      float *conv_state, const float *qkv, const float *ker, float *state,
+                      const float *norm_w, const float *z, float *att, uint32_t d_state, uint32_t hK,
+                      uint32_t hV, uint32_t kdiv, float eps, uint32_t n_slots, void *stream);
 
 /* ---- the mixers over consecutive positions of ONE slot (prompt prefill) ---------------------------
  * (reference shaders/fa_prep_batch.comp, fa_attn_batch.comp, dn_conv_batch.comp, dn_step_batch.comp

@@ -12,7 +12,7 @@ from .capi import (  # noqa: F401
     moe_group_pairs, gemm_q8_0, moe_prefill, moe_prefill_workspace_bytes, device_info,
     rmsnorm, add_rmsnorm, add_rms3, vec_add, embed, moe_decode_tail, moe_layer_rows, ROWWISE_MAX,
     rope_table, attn_prep, attn_workspace_bytes, attn_decode, dn_ab, dn_conv, dn_step, dn_ab_conv,
-    moe_decode_static, moe_workspace_status, gemv_norm, head_argmax_norm, MOE_STATIC_MAX_SLOTS, MOE_STATIC_BYTES,
+    moe_decode_static, moe_workspace_status, gemv_norm, head_argmax_norm, dn_step_fused, MOE_STATIC_MAX_SLOTS, MOE_STATIC_BYTES,
 )
 from . import capi  # noqa: F401
 from . import synth  # noqa: F401

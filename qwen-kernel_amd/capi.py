@@ -76,6 +76,7 @@ def _signatures():
         "qkk_dn_step": (None, dn_step),
         "qkk_dn_step_seq": (None, dn_step),
         "qkk_dn_ab_conv": (None, [vp] * 6 + [u32, u32] + [vp] * 4 + [u32] * 3 + [f32, u32, vp]),
+        "qkk_dn_step_fused": (None, [vp, vp, f32] + [vp] * 4 + [u32] + [vp] * 7 + [u32] * 4 + [f32, u32, vp]),
         "qkk_dn_ab_conv_norm": (None, [vp, vp, f32] + [vp] * 5 + [u32, u32] + [vp] * 4 + [u32] * 3 + [f32, u32, vp]),
         "qkk_rope_table": (None, [vp, u32, u32, f32]),
         "qkk_attn_prep": (None, attn_prep),
@@ -462,6 +463,19 @@ def dn_ab_conv(x, alpha_w, beta_w, dt_bias, a_vec, conv_state, qkv, ker, qk_chan
                                 _ptr(conv_state), _ptr(qkv), _ptr(ker), _ptr(out), channels, d_state, qk_channels, eps, n,
                                 _stream()))
     return gb, out
+
+
+def dn_step_fused(x, alpha_w, beta_w, dt_bias, a_vec, conv_state, qkv, ker, state, norm_w, z, hK, hV, kdiv=0, d_state=128,
+                  eps=1e-6, w_norm=None, norm_eps=1e-6):
+    """ab + conv + step of the slots' new tokens in one launch (two value heads per key head).  conv_state
+    and state are updated in place; returns att [slots][hV * dS]."""
+    import torch
+    n = x.shape[0]
+    att = torch.empty((n, hV * d_state), dtype=torch.float32, device=x.device)
+    _check(lib().qkk_dn_step_fused(_ptr(x), _ptr(w_norm), norm_eps, _ptr(alpha_w), _ptr(beta_w), _ptr(dt_bias), _ptr(a_vec),
+                                   x.shape[1], _ptr(conv_state), _ptr(qkv), _ptr(ker), _ptr(state), _ptr(norm_w), _ptr(z),
+                                   _ptr(att), d_state, hK, hV, kdiv, eps, n, _stream()))
+    return att
 
 
 def dn_conv(conv_state, qkv, ker, qk_channels, d_state=128, eps=1e-6, out=None, seq=False):

@@ -765,7 +765,7 @@ static int attn_decode_impl(const char* who, const float* qhat, const float* k_c
     uint32_t n_ranges = std::min(max_ranges(rows), std::max(8u, persistent_blocks() / 2 / (rows * hKV)));
     // three or more consecutive rows of one slot: blocks of sixteen rows (QK_ATTN_PAIR=1 keeps the pair kernel);
     // one workgroup per CU (LDS), so about as many (block, KV head, range) triples as there are CUs
-    static const bool pair_only = getenv("QK_ATTN_PAIR") != nullptr;
+    const bool pair_only = getenv("QK_ATTN_PAIR") != nullptr; // read per call: a test switches it between engines
     const bool blocked = own == 0 && rows >= 3 && !pair_only;
     const uint32_t blocks = (rows + BLK_Q - 1) / BLK_Q;
     const uint32_t hgroups = (hQ / hKV + 3) / 4; // four query heads of a KV head per workgroup

@@ -213,6 +213,150 @@ __global__ __launch_bounds__(DN_DS* DN_PARTS) void dn_step_kernel(const float* _
     }
 }
 
+// ---- the whole decode step of the mixer in ONE launch --------------------------------------------
+// ab, conv and step for the value heads of one key head per workgroup: grid (hK, slots), 1024 threads,
+// for shapes with two value heads per key head (the reference's 32 on 16).  The q / k conv window of a
+// key head is read by both of its value heads but may be shifted once only, and not before both have
+// read it -- inside one workgroup that is a barrier, across workgroups it would be a race: hence the
+// key head as the unit.  Same arithmetic in the same order as dn_ab_conv_kernel followed by
+// dn_step_kernel (the results are bit for bit theirs); what is saved is a launch and the round trip
+// of conv and gb through memory.
+//   threads    0..127 q channels, 128..255 k channels, 256..383 v of head A, 384..511 v of head B: conv +
+//              SiLU + window shift; q and k scaled to unit length (two waves each: one LDS exchange)
+//   waves 8..11 one dot product each: alpha . x and beta . x of head A and of head B
+//   then every thread (row j = t % 128, part c = t / 128) holds dS / 8 state values of BOTH heads and
+//   runs the delta rule on them with the shared q and k; the column sums of both heads share the
+//   barriers.
+// NORM as in dn_ab_conv_kernel.
+template <int NCH, bool NORM>
+__global__ __launch_bounds__(DN_DS* DN_PARTS) void dn_fused_step_kernel(
+    float* __restrict__ win, const float* __restrict__ qkv, const float* __restrict__ ker, const float* __restrict__ x,
+    const float* __restrict__ nw, float norm_eps, const float* __restrict__ alpha_w, const float* __restrict__ beta_w,
+    const float* __restrict__ dt_bias, const float* __restrict__ a_vec, float* __restrict__ state,
+    const float* __restrict__ norm_w, const float* __restrict__ z, float* __restrict__ att, uint32_t hK, uint32_t hV,
+    uint32_t kdiv, float eps)
+{
+    __shared__ float s_q[DN_DS], s_k[DN_DS], s_v[2][DN_DS];
+    __shared__ float s_part[2][2][DN_PARTS][DN_DS]; // [head][k or q sums][part][row]
+    __shared__ float s_red[2][2], s_qk[4], s_gb[4]; // q/k squares per wave; decay A, decay B, beta A, beta B
+    const uint32_t kh = blockIdx.x, rq = blockIdx.y, t = threadIdx.x, j = t % DN_DS, c = t / DN_DS, lane = t & 63u;
+    const uint32_t channels = (2 * hK + hV) * DN_DS;
+    const uint32_t hd[2] = {kdiv ? kh * kdiv : kh, kdiv ? kh * kdiv + 1 : kh + hK}; // the two value heads of key head kh
+
+    // the state of both heads: requested before anything else
+    float s[2][DN_PC];
+    float* S[2];
+#pragma unroll
+    for (int a = 0; a < 2; a++) {
+        S[a] = state + ((size_t)rq * hV + hd[a]) * DN_DS * DN_DS + (size_t)c * DN_PC * DN_DS + j;
+#pragma unroll
+        for (uint32_t i = 0; i < DN_PC; i++) s[a][i] = S[a][(size_t)i * DN_DS];
+    }
+    const float zv[2] = {z[((size_t)rq * hV + hd[0]) * DN_DS + j], z[((size_t)rq * hV + hd[1]) * DN_DS + j]};
+    const float nwj = norm_w[j];
+
+    if (c < 4) { // conv of one channel: q, k, v of head A, v of head B
+        const uint32_t ch = (c == 0 ? kh : c == 1 ? hK + kh : 2 * hK + hd[c - 2]) * DN_DS + j;
+        float* w = win + ((size_t)rq * channels + ch) * 3;
+        const float w0 = w[0], w1 = w[1], w2 = w[2], xin = qkv[(size_t)rq * channels + ch];
+        const float4 kk = ((const float4*)ker)[ch];
+        const float cv = w0 * kk.x + w1 * kk.y + w2 * kk.z + xin * kk.w;
+        const float v = cv / (1.f + expf(-cv));
+        w[0] = w1; w[1] = w2; w[2] = xin;
+        if (c < 2) { // a q or k head: its squares, wave by wave
+            const float sq = wave_sum(v * v);
+            if (lane == 0) s_qk[t >> 6] = sq;
+            (c == 0 ? s_q : s_k)[j] = v;
+        } else {
+            s_v[c - 2][j] = v;
+        }
+    } else if (c < 6) { // waves 8..11: alpha A, alpha B, beta A, beta B
+        const uint32_t wv = (t >> 6) - 8, a = wv & 1u;
+        const bool is_beta = wv >= 2;
+        const float4* row = (const float4*)((is_beta ? beta_w : alpha_w) + (size_t)hd[a] * 256 * NCH);
+        const float4* xv = (const float4*)(x + (size_t)rq * 256 * NCH);
+        float4 ra[NCH], rb[NCH];
+#pragma unroll
+        for (int i = 0; i < NCH; i++) ra[i] = row[lane + 64 * i];
+#pragma unroll
+        for (int i = 0; i < NCH; i++) rb[i] = xv[lane + 64 * i];
+        float scale = 1.f;
+        if constexpr (NORM) {
+            float ss = 0.f;
+#pragma unroll
+            for (int i = 0; i < NCH; i++) {
+                const float4 g = ((const float4*)nw)[lane + 64 * i];
+                ss += (rb[i].x * rb[i].x + rb[i].y * rb[i].y) + (rb[i].z * rb[i].z + rb[i].w * rb[i].w);
+                rb[i] = float4{rb[i].x * g.x, rb[i].y * g.y, rb[i].z * g.z, rb[i].w * g.w};
+            }
+            scale = 1.f / sqrtf(wave_sum(ss) / (float)(256 * NCH) + norm_eps);
+        }
+        float p0 = 0.f, p1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            p0 += ra[i].x * rb[i].x + ra[i].y * rb[i].y;
+            p1 += ra[i].z * rb[i].z + ra[i].w * rb[i].w;
+        }
+        const float d = wave_sum(p0 + p1) * scale;
+        if (lane == 0) {
+            if (is_beta) {
+                s_gb[2 + a] = 1.f / (1.f + expf(-d));
+            } else {
+                const float v = d + dt_bias[hd[a]];
+                s_gb[a] = expf(a_vec[hd[a]] * (v > 20.f ? v : log1pf(expf(v))));
+            }
+        }
+    }
+    __syncthreads();
+    // unit length for q and k (as block_sum2 in dn_conv_kernel: the two waves' sums in wave order), q also / sqrt(dS)
+    if (c == 0) s_q[j] = s_q[j] * (1.f / fmaxf(sqrtf(s_qk[0] + s_qk[1]), eps)) * (1.f / sqrtf((float)DN_DS));
+    if (c == 1) s_k[j] = s_k[j] * (1.f / fmaxf(sqrtf(s_qk[2] + s_qk[3]), eps));
+    __syncthreads();
+
+    float kk[DN_PC];
+#pragma unroll
+    for (uint32_t i = 0; i < DN_PC; i++) kk[i] = s_k[c * DN_PC + i];
+#pragma unroll
+    for (int a = 0; a < 2; a++) {
+        float ps = 0.f;
+#pragma unroll
+        for (uint32_t i = 0; i < DN_PC; i++) ps += s[a][i] * kk[i];
+        s_part[a][0][c][j] = ps;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int a = 0; a < 2; a++) {
+        float sk = 0.f;
+#pragma unroll
+        for (uint32_t p = 0; p < DN_PARTS; p++) sk += s_part[a][0][p][j];
+        const float decay = s_gb[a], beta = s_gb[2 + a];
+        const float dj = beta * (s_v[a][j] - sk * decay);
+        float po = 0.f;
+#pragma unroll
+        for (uint32_t i = 0; i < DN_PC; i++) {
+            const float sn = s[a][i] * decay + kk[i] * dj;
+            S[a][(size_t)i * DN_DS] = sn;
+            po += sn * s_q[c * DN_PC + i];
+        }
+        s_part[a][1][c][j] = po;
+    }
+    __syncthreads();
+    if (c < 2) { // parts 0 and 1: the 128 rows of head A and of head B
+        float oj = 0.f;
+#pragma unroll
+        for (uint32_t p = 0; p < DN_PARTS; p++) oj += s_part[c][1][p][j];
+        const float w = wave_sum(oj * oj);
+        if (lane == 0) s_red[c][(t >> 6) & 1u] = w;
+        s_part[c][0][0][j] = oj;
+    }
+    __syncthreads();
+    if (c < 2) {
+        const float oj = s_part[c][0][0][j];
+        const float scale = 1.f / sqrtf((s_red[c][0] + s_red[c][1]) / (float)DN_DS + eps);
+        att[((size_t)rq * hV + hd[c]) * DN_DS + j] = oj * scale * nwj * (zv[c] / (1.f + expf(-zv[c])));
+    }
+}
+
 // The same two steps over n_pos consecutive positions of ONE slot (reference
 // shaders/dn_conv_batch.comp, dn_step_batch.comp + dn_gate_batch.comp): rows t of qkv / conv / gb /
 // z / att are positions; the window and the state are read once and written once.
@@ -544,6 +688,34 @@ int qkk_dn_step(const float* conv, const float* gb, float* state, const float* n
     hipLaunchKernelGGL(dn_step_kernel, dim3(hV, n_slots), dim3(DN_DS * DN_PARTS), 0, as_stream(stream), conv, gb, state,
                        norm_w, z, att, hK, hV, kdiv, eps);
     return check_launch("qkk_dn_step");
+}
+
+int qkk_dn_step_fused(const float* x, const float* w_norm, float norm_eps, const float* alpha_w, const float* beta_w,
+                      const float* dt_bias, const float* a_vec, uint32_t n_embd, float* conv_state, const float* qkv,
+                      const float* ker, float* state, const float* norm_w, const float* z, float* att, uint32_t d_state,
+                      uint32_t hK, uint32_t hV, uint32_t kdiv, float eps, uint32_t n_slots, void* stream)
+{
+    const char* who = "qkk_dn_step_fused";
+    if (!x || !alpha_w || !beta_w || !dt_bias || !a_vec || !conv_state || !qkv || !ker || !state || !norm_w || !z || !att)
+        return fail(QKK_EINVAL, "%s: null pointer", who);
+    if (int rc = check_slots(who, n_slots)) return rc;
+    if (n_embd != 2048) return fail(QKK_ESHAPE, "%s: n_embd %u not supported (2048)", who, n_embd);
+    if (d_state != DN_DS) return fail(QKK_ESHAPE, "%s: state size %u not supported (128)", who, d_state);
+    if (hK < 1 || hK > 32767 || hV != 2 * hK || (kdiv != 0 && kdiv != 2))
+        return fail(QKK_ESHAPE, "%s: two value heads per key head are required (got %u on %u, kdiv %u)", who, hV, hK, kdiv);
+    if (!aligned16(x) || !aligned16(alpha_w) || !aligned16(beta_w) || !aligned16(ker) || (w_norm && !aligned16(w_norm)))
+        return fail(QKK_EINVAL, "%s: x, the weight rows, ker and w_norm must be 16-byte aligned", who);
+    if (!(eps >= 0.f) || !(norm_eps >= 0.f)) return fail(QKK_EINVAL, "%s: eps must be non-negative", who);
+    if (int rc = require_device()) return rc;
+    const dim3 grid(hK, n_slots), block(DN_DS * DN_PARTS);
+    if (w_norm)
+        hipLaunchKernelGGL((dn_fused_step_kernel<8, true>), grid, block, 0, as_stream(stream), conv_state, qkv, ker, x, w_norm,
+                           norm_eps, alpha_w, beta_w, dt_bias, a_vec, state, norm_w, z, att, hK, hV, kdiv, eps);
+    else
+        hipLaunchKernelGGL((dn_fused_step_kernel<8, false>), grid, block, 0, as_stream(stream), conv_state, qkv, ker, x,
+                           (const float*)nullptr, 0.f, alpha_w, beta_w, dt_bias, a_vec, state, norm_w, z, att, hK, hV, kdiv,
+                           eps);
+    return check_launch(who);
 }
 
 } // extern "C"

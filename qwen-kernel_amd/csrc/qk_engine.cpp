@@ -105,6 +105,7 @@ struct qk_engine {
     uint32_t pf_rows = 1024;     // positions of one slot a prefill pass carries (whole-model files; QK_PREFILL_ROWS)
     uint32_t cap = MAX_ROWS;     // rows the step's buffers hold (pf_rows for whole-model files)
     bool cat_everywhere = false; // every layer's input projections lie back to back (one product per layer)
+    bool dn_one_launch = false;  // QK_DN_FUSED=1: the gated-DeltaNet decode step as one launch (to be measured against two)
     uint32_t *d_pf = nullptr, *h_pf = nullptr; // [3][pf_rows] ids, positions, sampled ids of a prefill pass (device / pinned)
     float* d_rope = nullptr;     // [n_ctx][FA_ROT/2][2]
     float *d_big = nullptr, *d_mid = nullptr, *d_kin = nullptr, *d_vin = nullptr, *d_gb = nullptr, *d_conv = nullptr,
@@ -262,6 +263,12 @@ int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool 
                 if (int rc = qkk_dn_conv_seq(s1, d_big, L.ker, d_conv, DN_CH, DN_DS, 2 * DN_HK * DN_DS, eps, rows, st)) return rc;
                 if (int rc = qkk_dn_step_seq(d_conv, d_gb, s2, L.ssm_norm, d_mid, d_att, DN_DS, DN_HK, DN_HV, dn_kdiv, eps, rows,
                                              st))
+                    return rc;
+            } else if (dn_one_launch) {
+                // QK_DN_FUSED=1: ab, conv and step in one launch (a workgroup per key head; the same results bit for bit)
+                if (int rc = qkk_dn_step_fused(fuse ? x : xn, fuse ? L.attn_norm : nullptr, eps, L.alpha_w, L.beta_w, L.dt_bias,
+                                               L.a_vec, N_EMBD, s1, d_big, L.ker, s2, L.ssm_norm, d_mid, d_att, DN_DS, DN_HK,
+                                               DN_HV, dn_kdiv, eps, rows, st))
                     return rc;
             } else {
                 // decay / write strength and the conv in one launch
@@ -752,6 +759,7 @@ bool qk_engine::open(const char* path, const qk_config& cfg, char* err, size_t e
     memset(h_pos, 0, MAX_ROWS * 4);
     if (full_model && !load_mixers(g, err, err_len)) return false;
     cat_everywhere = full_model;
+    dn_one_launch = getenv("QK_DN_FUSED") && atoi(getenv("QK_DN_FUSED")) == 1 && DN_HV == 2 * DN_HK;
     for (const EngineLayer& L : layers) cat_everywhere = cat_everywhere && L.cat.w != nullptr;
     if (hipDeviceSynchronize() != hipSuccess) return bad("qk_open: upload failed"); // fills and uploads are complete
 

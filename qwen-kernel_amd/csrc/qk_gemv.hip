@@ -10,6 +10,8 @@
 
 #include <stdarg.h>
 
+#include <stdlib.h>
+
 #include <algorithm>
 
 namespace qk {
@@ -381,7 +383,10 @@ static void launch_q(const void* W, const float* X, float* Y, uint32_t M, uint32
     const uint32_t cus = persistent_blocks() / 4;
     const uint32_t chunks = M / CH, tail_groups = (M - chunks * CH + WAVE / LPR - 1) / (WAVE / LPR);
     const uint32_t want = (std::max(chunks, tail_groups) + 3) / 4; // one chunk per wave
-    const uint32_t blocks = std::max(1u, want <= cus * RESIDENT ? want : cus * DEPTH);
+    // QK_GEMV_DEPTH=n (1..16): workgroups per CU of the persistent grid, for sweeps on the device
+    static const uint32_t depth_env = [] { const char* e = getenv("QK_GEMV_DEPTH"); const int v = e ? atoi(e) : 0; return v >= 1 && v <= 16 ? (uint32_t)v : 0u; }();
+    const uint32_t depth = depth_env ? std::min(depth_env, RESIDENT) : DEPTH;
+    const uint32_t blocks = std::max(1u, want <= cus * RESIDENT ? want : cus * depth);
     hipLaunchKernelGGL((gemv_stream_kernel<TYPE, LPR, PASSES, RPC, NORM>), dim3(blocks, batch), dim3(256), 0, st,
                        (const uint8_t*)W, X, Y, M, nw, eps);
 }

@@ -10,6 +10,8 @@
 #include "qk_host.h"
 #include "qk_stream.h"
 
+#include <stdlib.h>
+
 #include <algorithm>
 
 namespace qk {
@@ -300,8 +302,10 @@ __global__ __launch_bounds__(CT) void head_q6k_coop_kernel(const uint8_t* __rest
 constexpr uint32_t HEAD_RPC = 2, HEAD_DEPTH = 8;
 static uint32_t head_blocks(uint32_t V, uint32_t rpc)
 {
+    // QK_HEAD_DEPTH=n (1..8): workgroups per CU, for sweeps on the device (never more than the workspace bound's 8)
+    static const uint32_t depth_env = [] { const char* e = getenv("QK_HEAD_DEPTH"); const int v = e ? atoi(e) : 0; return v >= 1 && v <= (int)HEAD_DEPTH ? (uint32_t)v : 0u; }();
     const uint32_t waves = std::max(V / rpc, V % rpc);
-    return std::max(1u, std::min((waves + 3) / 4, persistent_blocks() / 4 * HEAD_DEPTH));
+    return std::max(1u, std::min((waves + 3) / 4, persistent_blocks() / 4 * (depth_env ? depth_env : HEAD_DEPTH)));
 }
 
 } // namespace qk

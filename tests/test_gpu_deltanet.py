@@ -104,6 +104,46 @@ def test_deltanet_ab_with_the_norm_in_front(qk, orc, dev):
             assert rel(gb.cpu().numpy()[s], np.concatenate([g, b])) <= TOL
 
 
+@pytest.mark.parametrize("n_slots,kdiv,norm", [(1, 0, False), (1, 2, True), (3, 0, True), (16, 2, False)])
+def test_deltanet_one_launch_step(qk, orc, dev, n_slots, kdiv, norm):
+    """qkk_dn_step_fused (ab + conv + step of the two value heads of a key head in one workgroup) against
+    the two launches it replaces: the same arithmetic in the same order, so attention rows, conv window and
+    state come out bit for bit the same, over several tokens; the first token also against the oracle."""
+    import torch
+    print(f"[case] deltanet one-launch step slots={n_slots} kdiv={kdiv} norm={norm}", flush=True)
+    w = Weights(11)
+    up = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    rng = np.random.default_rng(n_slots + kdiv)
+    st = rng.standard_normal((n_slots, w.ch, 3)).astype(F)
+    S = (rng.standard_normal((n_slots, w.hv, DS, DS)) * 0.1).astype(F)
+    St = np.ascontiguousarray(S.transpose(0, 1, 3, 2))                     # device layout: column-major per head
+    st_a, st_b, S_a, S_b = up(st.copy()), up(st.copy()), up(St.copy()), up(St.copy())
+    wd = {k: up(getattr(w, k)) for k in ("alpha_w", "beta_w", "dt_bias", "a_vec", "ker", "norm_w")}
+    nw = rng.uniform(0.5, 1.5, NE).astype(F)
+    nwd = up(nw) if norm else None
+    for tkn in range(3):
+        x = (rng.standard_normal((n_slots, NE)) * 2.0).astype(F)
+        qkv = rng.standard_normal((n_slots, w.ch)).astype(F)
+        z = rng.standard_normal((n_slots, w.hv * DS)).astype(F)
+        xd, qd, zd = up(x), up(qkv), up(z)
+        gb, conv = qk.dn_ab_conv(xd, wd["alpha_w"], wd["beta_w"], wd["dt_bias"], wd["a_vec"], st_a, qd, wd["ker"], w.qk, w_norm=nwd)
+        att_a = qk.dn_step(conv, gb, S_a, wd["norm_w"], zd, w.hk, w.hv, kdiv=kdiv)
+        att_b = qk.dn_step_fused(xd, wd["alpha_w"], wd["beta_w"], wd["dt_bias"], wd["a_vec"], st_b, qd, wd["ker"], S_b,
+                                 wd["norm_w"], zd, w.hk, w.hv, kdiv=kdiv, w_norm=nwd)
+        torch.cuda.synchronize()
+        assert torch.equal(att_b, att_a) and torch.equal(st_b, st_a) and torch.equal(S_b, S_a), tkn
+        if tkn == 0:
+            for s_ in range(n_slots):
+                xs = orc.add_rms(x[s_], nw, 1e-6) if norm else x[s_]
+                g, b = OD.ab(xs, w.alpha_w, w.beta_w, w.dt_bias, w.a_vec)
+                c = OD.conv(st[s_].copy(), qkv[s_], w.ker, DS, w.qk)
+                a = OD.step(c, g, b, S[s_].copy(), w.norm_w, z[s_], w.hk, w.hv, kdiv=kdiv)
+                assert rel(att_b.cpu().numpy()[s_], a) <= TOL, s_
+    with pytest.raises(qk.QkError):   # three value heads per key head: not this kernel's shape
+        qk.dn_step_fused(xd, wd["alpha_w"], wd["beta_w"], wd["dt_bias"], wd["a_vec"], st_b, qd, wd["ker"], S_b, wd["norm_w"], zd,
+                         w.hk, w.hv + w.hk, kdiv=kdiv)
+
+
 def test_deltanet_other_shapes(qk, dev):
     """Fewer heads (1 key head for 2 value heads, both pairings) and n_embd = 4096."""
     print("[case] deltanet other shapes", flush=True)

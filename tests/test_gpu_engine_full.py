@@ -82,14 +82,18 @@ def test_whole_model_streams(qk, full):
 def test_whole_model_eager_launches_and_serial_prefill(qk, full, monkeypatch):
     """QK_NO_GRAPH launches the kernels one by one; QK_NO_BATCH feeds every prompt token in a serial
     step instead of at the start; QK_MAXB moves the border between prefilled and serially fed positions,
-    QK_PREFILL_ROWS sets the rows per prefill pass: the same streams."""
+    QK_PREFILL_ROWS sets the rows per prefill pass; QK_DN_FUSED, QK_NO_FUSED_NORM and QK_ATTN_PAIR choose
+    between kernel forms of the same step: the same streams."""
     model, path = full
     print("[case] whole model, eager / serial prefill", flush=True)
     prompt = [int(t) for t in np.random.default_rng(6).integers(0, VOCAB, 18)]
     streams = []
     for env in ({}, {"QK_NO_GRAPH": "1"}, {"QK_NO_BATCH": "1"}, {"QK_MAXB": "16"},
-                {"QK_PREFILL_ROWS": "16"}):   # QK_MAXB 16: 16 positions prefilled, one serial step more; rows 16: two passes
-        for k in ("QK_NO_GRAPH", "QK_NO_BATCH", "QK_MAXB", "QK_PREFILL_ROWS"):
+                {"QK_PREFILL_ROWS": "16"},    # QK_MAXB 16: 16 positions prefilled, one serial step more; rows 16: two passes
+                {"QK_DN_FUSED": "1"},         # the gated-DeltaNet step as one launch: the same bits
+                {"QK_NO_FUSED_NORM": "1"},    # the norm as launches of its own again: the same sums scaled earlier
+                {"QK_ATTN_PAIR": "1"}):       # the prompt's attention two rows at a time
+        for k in ("QK_NO_GRAPH", "QK_NO_BATCH", "QK_MAXB", "QK_PREFILL_ROWS", "QK_DN_FUSED", "QK_NO_FUSED_NORM", "QK_ATTN_PAIR"):
             monkeypatch.delenv(k, raising=False)
         for k, v in env.items():
             monkeypatch.setenv(k, v)
