@@ -367,6 +367,75 @@ __global__ __launch_bounds__(256) void gemv_dense_kernel(const T* __restrict__ W
     }
 }
 
+// The same rows for K = CPL * 64 chunks of 16 bytes exactly (K = 512 * CPL halves or 256 * CPL floats): the
+// lane's share of x -- the chunks lane, lane + 64, ... -- stays in registers for every row the wave visits
+// (re-read per row, x made up two thirds of the bytes through the L1: 8 KB of x for a 4 KB row of halves),
+// and the next row's chunks are requested before the current row's arithmetic.  Same assignment of chunks
+// to lanes and the same two partial sums as gemv_dense_kernel: the same bits.
+template <typename T, int CPL>
+__global__ __launch_bounds__(256) void gemv_dense_reg_kernel(const T* __restrict__ W, const float* __restrict__ X,
+                                                             float* __restrict__ Y, uint32_t M)
+{
+    constexpr int PER = 16 / sizeof(T);
+    constexpr uint32_t K = CPL * 64 * PER;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float* x = X + (size_t)blockIdx.y * K;
+    float* y = Y + (size_t)blockIdx.y * M;
+    const uint32_t stride = gridDim.x * 4;
+    uint32_t r = blockIdx.x * 4 + wave;
+    if (r >= M) return; // the whole wave
+    uint4 cur[CPL], nxt[CPL];
+#pragma unroll
+    for (int i = 0; i < CPL; i++) cur[i] = ((const uint4*)(W + (size_t)r * K))[lane + 64 * i];
+    float xs[CPL][PER];
+#pragma unroll
+    for (int i = 0; i < CPL; i++) {
+        const float4* xp = (const float4*)(x + (size_t)(lane + 64 * i) * PER);
+#pragma unroll
+        for (int q = 0; q < PER / 4; q++) {
+            const float4 v = xp[q];
+            xs[i][4 * q] = v.x; xs[i][4 * q + 1] = v.y; xs[i][4 * q + 2] = v.z; xs[i][4 * q + 3] = v.w;
+        }
+    }
+    for (; r < M; r += stride) {
+        const uint32_t rn = min(r + stride, M - 1); // past the end: a harmless re-read of the last row
+#pragma unroll
+        for (int i = 0; i < CPL; i++) nxt[i] = ((const uint4*)(W + (size_t)rn * K))[lane + 64 * i];
+        float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < CPL; i++) {
+            if constexpr (sizeof(T) == 2) {
+                const _Float16* h = (const _Float16*)&cur[i];
+                acc0 += (float)h[0] * xs[i][0] + (float)h[1] * xs[i][1] + (float)h[2] * xs[i][2] + (float)h[3] * xs[i][3];
+                acc1 += (float)h[4] * xs[i][4] + (float)h[5] * xs[i][5] + (float)h[6] * xs[i][6] + (float)h[7] * xs[i][7];
+            } else {
+                const float* f = (const float*)&cur[i];
+                acc0 += f[0] * xs[i][0] + f[1] * xs[i][1];
+                acc1 += f[2] * xs[i][2] + f[3] * xs[i][3];
+            }
+        }
+        const float sum = wave_sum(acc0 + acc1);
+        if (lane == 0) y[r] = sum;
+#pragma unroll
+        for (int i = 0; i < CPL; i++) cur[i] = nxt[i];
+    }
+}
+
+template <typename T>
+static bool launch_dense_reg(const void* W, const float* X, float* Y, uint32_t M, uint32_t K, uint32_t batch, hipStream_t st)
+{
+    constexpr uint32_t PER = 16 / sizeof(T);
+    if (K % (64 * PER)) return false;
+    const dim3 grid(std::min((M + 3) / 4, persistent_blocks() * 2), batch); // eight workgroups per CU: two rows in flight per wave
+    switch (K / (64 * PER)) {
+    case 1: hipLaunchKernelGGL((gemv_dense_reg_kernel<T, 1>), grid, dim3(256), 0, st, (const T*)W, X, Y, M); return true;
+    case 2: hipLaunchKernelGGL((gemv_dense_reg_kernel<T, 2>), grid, dim3(256), 0, st, (const T*)W, X, Y, M); return true;
+    case 4: hipLaunchKernelGGL((gemv_dense_reg_kernel<T, 4>), grid, dim3(256), 0, st, (const T*)W, X, Y, M); return true;
+    case 8: hipLaunchKernelGGL((gemv_dense_reg_kernel<T, 8>), grid, dim3(256), 0, st, (const T*)W, X, Y, M); return true;
+    default: return false;
+    }
+}
+
 // ---- launchers ----------------------------------------------------------------------------
 
 template <int TYPE, int LPR, int PASSES, bool NORM = false>
@@ -547,6 +616,8 @@ int qkk_gemv(int type, const void* W, const float* X, float* Y, uint32_t M, uint
     case QKK_F32: {
         const uint32_t per = type == QKK_F16 ? 8 : 4;
         if (K % per) return fail(QKK_ESHAPE, "qkk_gemv: K=%u must be a multiple of %u for dense rows", K, per);
+        if (type == QKK_F16 ? launch_dense_reg<_Float16>(W, X, Y, M, K, batch, st) : launch_dense_reg<float>(W, X, Y, M, K, batch, st))
+            return check_launch("qkk_gemv");
         const dim3 grid(std::min((M + 3) / 4, persistent_blocks()), batch);
         if (type == QKK_F16)
             hipLaunchKernelGGL(gemv_dense_kernel<_Float16>, grid, dim3(256), 0, st, (const _Float16*)W, X, Y, M, K);

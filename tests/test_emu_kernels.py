@@ -206,3 +206,17 @@ def test_attention_blocks_inside_their_tensors(qk, emu, hq, hkv, base, n_pos):
         want = OA.attend(OA.prep(qfull[t], kin[t], vin[t], qn, kn, rope, base + t, kc, vc, NROT), kc, vc, qfull[t], base + t)
         err = float(np.max(np.abs(att[t].astype(np.float64) - want)) / np.max(np.abs(want)))
         assert err <= 1e-3, (t, err)
+
+
+@pytest.mark.parametrize("name", ["f16", "f32"])
+@pytest.mark.parametrize("K,M", [(2048, 1), (2048, 9), (4096, 3), (512, 70), (768, 6)])
+def test_dense_gemv_inside_its_tensors(qk, orc, emu, name, K, M):
+    """Dense rows: K a whole number of 64 sixteen-byte chunks takes the kernel with x in registers (the row
+    after the last one is never fetched: the prefetch re-reads the last row), other K the chunk loop."""
+    t = {"f16": qk.F16, "f32": qk.F32}[name]
+    W = qk.synth.tensor_host(t, M, K, seed=K + M)
+    x = np.random.default_rng(M).standard_normal((1, K)).astype(np.float32)
+    Yd = emu.zeros((1, M), np.float32)
+    qk.gemv(t, emu.tensor(W.reshape(-1)), emu.tensor(x), M, K, out=Yd)
+    want = orc.gemv(t, W, x[0], M, K)
+    assert orc.rel_maxabs_err(Yd.numpy()[0], want) <= 1e-3
