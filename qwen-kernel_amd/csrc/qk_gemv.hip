@@ -426,7 +426,9 @@ static bool launch_dense_reg(const void* W, const float* X, float* Y, uint32_t M
 {
     constexpr uint32_t PER = 16 / sizeof(T);
     if (K % (64 * PER)) return false;
-    const dim3 grid(std::min((M + 3) / 4, persistent_blocks() * 2), batch); // eight workgroups per CU: two rows in flight per wave
+    // four workgroups per CU and at least two rows per wave where there are that many: x is fetched once per
+    // wave, so a wave that visits one row only has gained nothing over the chunk loop
+    const dim3 grid(std::max(1u, std::min((M + 7) / 8, persistent_blocks())), batch);
     switch (K / (64 * PER)) {
     case 1: hipLaunchKernelGGL((gemv_dense_reg_kernel<T, 1>), grid, dim3(256), 0, st, (const T*)W, X, Y, M); return true;
     case 2: hipLaunchKernelGGL((gemv_dense_reg_kernel<T, 2>), grid, dim3(256), 0, st, (const T*)W, X, Y, M); return true;
