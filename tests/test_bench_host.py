@@ -28,6 +28,6 @@ def test_cpu_baseline_line(qk, orc):
     assert sorted(per) == sorted(want)
     for name, e in per.items():
         assert e["us_1_thread"] > 0 and e["us_all_threads"] > 0 and e["threads"] == b["cores"] and e["sample"], name
-    assert per["C2_moe_decode_bs1"]["bytes"] == 16326656      # the survey's algorithmic bytes of the step's weights
+    assert per["C2_moe_decode_bs1"]["bytes"] == 16326656      # the weights one step touches: router, shared gate, 8 experts, shared expert
     assert per["C1_gemv_q8_0_8192x2048"]["bytes"] == 17866752
     assert per["C4_lm_head_q6k_151936_bs1"]["bytes"] == 255252480 + 8192
