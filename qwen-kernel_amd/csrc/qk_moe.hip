@@ -17,6 +17,7 @@
 #include "qk_stream.h"
 
 #include <mutex>
+#include <stdlib.h>
 
 namespace qk {
 
@@ -721,7 +722,10 @@ static int moe_decode_impl(const char* who, const qkk_moe_layer* L, const float*
     // there is little to share: each row runs the one-row launches (grid.y = row), and its result
     // is bit for bit what it is alone.  Measured: 2 rows 26 us against 40 us on the expert-major
     // path, 4 rows 37 / 50, 8 rows 62 / 71, 10 rows 76 / 78, 12 rows 87 / 86: more rows go there.
-    if (n_slots > ROWWISE_MAX) {
+    // QK_ROWWISE_MAX=n (1..64) moves the switch between the two paths for the plain step, for measurements on the
+    // device (the limit of the entry points with the norm in front stays QKK_ROWWISE_MAX)
+    static const uint32_t switch_env = [] { const char* e = getenv("QK_ROWWISE_MAX"); const int v = e ? atoi(e) : 0; return v >= 1 && v <= 64 ? (uint32_t)v : 0u; }();
+    if (n_slots > (norm || !switch_env ? ROWWISE_MAX : switch_env)) {
         if (norm) return fail(QKK_ESHAPE, "%s: %u rows exceed %u (use qkk_moe_decode_tail)", who, n_slots, ROWWISE_MAX);
         return moe_grouped_launch(L, X, Y, sel, workspace, n_slots, stages, st, tail);
     }

@@ -18,7 +18,8 @@ import qk_oracle_engine as OE  # noqa: E402
 
 pytestmark = pytest.mark.gpu
 
-H, VOCAB = 2048, 1024
+H = 2048
+VOCAB = int(os.environ.get("QK_TEST_VOCAB", "1024"))   # a smaller vocabulary (a multiple of 16, above 100) for slow runs
 
 
 def walk(nxt, start, n, depth=1):
@@ -132,7 +133,7 @@ def test_single_slot_stream(qk, world):
         assert eng.slot_start(0, [5, VOCAB], 4) == -4
         assert (eng.state_save(0, 2), eng.state_load(0, 2), eng.state_save(0, 3), eng.state_load(1, 0)) == (0, 0, -1, -1)
         start = next(t for t in range(100, VOCAB) if EOS not in walk(nxt, t, 12))
-        drive(eng, ref, {0: [("start", 0, [3, 9, 400, start], 10, 0)],
+        drive(eng, ref, {0: [("start", 0, [3, 9, min(400, VOCAB - 1), start], 10, 0)],
                          1: [("start", 0, [1], 1, 0)]},     # busy: -2 on both
               6)
         assert not ref.slots[0]["active"]
