@@ -429,6 +429,16 @@ def engine_workload(qk, n_layer, slots_list, chunks, warm_chunks, seed=31, kinds
     return res
 
 
+def guarded(ex, key, fn):
+    """Runs one extra measurement; a Python-level failure becomes an entry of the line instead of ending the run
+    (the headline figure is already measured by then)."""
+    try:
+        ex[key] = fn()
+    except Exception as e:   # noqa: BLE001 -- whatever it is, the line still goes out
+        ex[key] = dict(error=f"{type(e).__name__}: {e}")
+    log(f"[bench] {key}: {ex[key]}")
+
+
 def host_threads():
     """Threads of the all-cores CPU runs: the cores this process may use, at most 16 (a one-GPU box's share)."""
     try:
@@ -608,93 +618,13 @@ def main():
         return
     if a.workload == "gemv_sustained":   # every block format at a sustained size and at the 8192 x 2048 shape
         res = {}
-        for name, t in (("q8_0", qk.Q8_0), ("q6_k", qk.Q6_K), ("iq4_xs", qk.IQ4_XS), ("iq3_xxs", qk.IQ3_XXS)):
-            Ms = -(-(256 << 20) // qk.row_bytes(t, 2048) // 64) * 64
-            for label, M, ring in ((f"gemv_{name}_sustained_256MiB", Ms, 2), (f"gemv_{name}_8192x2048", 8192, None)):
-                g = gemv_workload(qk, t, M, 2048, 1, 40 if ring else 400, 4 if ring else 40, ring=ring)
-                gb = g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9
-                res[label] = dict(us=g["ms_event"] * 1e3, gbps=gb, frac=gb / HBM_PEAK_GBPS, steps_timed=g["steps"])
-                torch.cuda.empty_cache()
-        print(json.dumps(dict(metric="gemv_hbm_gbps", value=res["gemv_q8_0_sustained_256MiB"]["gbps"], unit="GB/s", n_gpus=1,
-                              higher_is_better=True, data="synthetic", dtype="f32",
-                              config=dict(workload="gemv_sustained", K=2048, env={k: v for k, v in os.environ.items()
-                                                                                   if k.startswith("QK_")}),
-                              detail=res)), flush=True)
-        return
-    if a.workload in ("head_bs1", "head_bs16"):   # the LM head alone (for counter runs on its kernel)
-        b = 1 if a.workload == "head_bs1" else 16
-        h = head_workload(qk, 151936, 2048, b, min(a.steps, 40), min(a.warmup, 8))
-        gb = h["bytes_step"] / (h["ms_event"] * 1e-3) / 1e9
-        print(json.dumps(dict(metric="lm_head_argmax_hbm_gbps", value=gb, unit="GB/s", n_gpus=1, steps=h["steps"],
-                              ms_per_step=h["ms_event"], higher_is_better=True, data="synthetic", dtype="f32",
-                              config=dict(workload=a.workload, vocab=151936, n_embd=2048, weights="Q6_K", rows=b),
-                              bytes_per_step=h["bytes_step"], frac_of_hbm_peak=gb / HBM_PEAK_GBPS)), flush=True)
-        return
-    if a.workload == "moe_decode_bs1":
-        m = moe_workload(qk, 1, qk.IQ4_XS, a.ring, steps, a.warmup)
-    elif a.workload == "moe_decode_bs16":
-        m = moe_workload(qk, 16, qk.Q6_K, min(a.ring, 8), steps, a.warmup)
-    elif a.workload == "moe_prefill_128":
-        m = moe_workload(qk, 128, qk.IQ4_XS, min(a.ring, 4), min(steps, 400), min(a.warmup, 40))
-    else:
-        sys.exit(f"unknown workload {a.workload}")
-    log(f"[bench] {a.workload}: {m['ms_wall'] * 1e3:.2f} us/step wall, {m['ms_event'] * 1e3:.2f} us/step events, "
-        f"stages {m['stage_ms']}")
-    gbps = m["bytes_step"] / (m["ms_wall"] * 1e-3) / 1e9
-    # dominant kernel = the routed gate/up launch (most bytes of the step); its average launch
-    # duration is measured live with HIP events on the launch stream over a replay of that
-    # stage alone on the same ring (profiles/ holds the rocprofv3 figure for the same kernel)
-    gu_ms = m["stage_ms"]["gateup"]
-    ach = m["gateup_bytes"] / (gu_ms * 1e-3) / 1e9
-    kname, kwhat = {"moe_decode_bs1": ("moe_gateup_kernel", "select + routed IQ3_XXS gate/up + SiLU"),
-                    "moe_decode_bs16": ("moe_gateup_fused_kernel", "routed IQ3_XXS + shared Q8_0 gate/up + SiLU"),
-                    "moe_prefill_128": ("moe_gateup_mfma_kernel", "routed IQ3_XXS gate/up + SiLU; the stage time also "
-                                        "covers the shared expert's launch on the side stream")}[a.workload]
-    roof = dict(bound="hbm", kernel=f"{kname} ({kwhat})", achieved=ach,
-                peak=HBM_PEAK_GBPS, unit="GB/s", frac=ach / HBM_PEAK_GBPS, traffic=TRAFFIC.get(kname),
-                bytes_per_launch=m["gateup_bytes"], us_per_launch=gu_ms * 1e3)
-    out = dict(metric="fused_moe_decode_step_hbm_gbps", value=gbps, unit="GB/s", n_gpus=1, steps=m["steps"],
-               warmup=a.warmup, ms_per_step=m["ms_wall"], higher_is_better=True, scaling="weak", vs_baseline=None,
-               dtype="f32", data="synthetic",
-               config=dict(workload=a.workload, n_embd=2048, n_ff=512, n_expert=256, n_used=8,
-                           gate_up="IQ3_XXS", down="Q6_K" if a.workload.endswith("bs16") else "IQ4_XS",
-                           shared="Q8_0", slots={"moe_decode_bs1": 1, "moe_decode_bs16": 16}.get(a.workload, 128),
-                           ring_layers=m["ring"], ring_bytes=m["ring_bytes"],
-                           steps_timed=m["steps"], graph_replays_timed=m["steps"] // m["ring"],
-                           timing=f"hipGraph replays of the ring (one launch set per layer of the ring), at least "
-                                  f"{MIN_REPLAYS} replays whatever --steps asks; value from the host clock over all of them, "
-                                  f"us_per_step_events the median replay by HIP events"),
-               us_per_step=m["ms_wall"] * 1e3, us_per_step_events=m["ms_event"] * 1e3,
-               bytes_per_step=m["bytes_step"], frac_of_hbm_peak=gbps / HBM_PEAK_GBPS,
-               distinct_experts_per_step=m["distinct_experts"],
-               three_launch_stage_us={k: v * 1e3 for k, v in m["stage_ms"].items()}, roofline=roof, device=info)
-
-    if a.extras:
-        ex = {}
-        es, ew = 400, 40
-        for name, t in (("q8_0", qk.Q8_0), ("q6_k", qk.Q6_K), ("iq4_xs", qk.IQ4_XS), ("iq3_xxs", qk.IQ3_XXS),
-                        ("f16", qk.F16)):
-            g = gemv_workload(qk, t, 8192, 2048, 1, es, ew)
-            ex[f"gemv_{name}_8192x2048"] = dict(us=g["ms_event"] * 1e3, gbps=g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9,
-                                                frac=g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9 / HBM_PEAK_GBPS)
-            log(f"[bench] gemv {name}: {ex[f'gemv_{name}_8192x2048']}")
-            torch.cuda.empty_cache()
-            if t != qk.F16:  # the same projection for 16 decode slots: weights read once
-                g = gemv_workload(qk, t, 8192, 2048, 16, es, ew)
-                ex[f"gemv_{name}_8192x2048_bs16"] = dict(us=g["ms_event"] * 1e3,
-                                                         gbps=g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9,
-                                                         frac=g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9 / HBM_PEAK_GBPS)
-                log(f"[bench] gemv {name} bs16: {ex[f'gemv_{name}_8192x2048_bs16']}")
-                torch.cuda.empty_cache()
-        # the same kernels at a sustained size: one tensor of >= 256 MiB per launch (K = 2048), two tensors
-        # alternating, so neither launch latency nor the caches carry the figure
-        for name, t in (("q8_0", qk.Q8_0), ("q6_k", qk.Q6_K), ("iq4_xs", qk.IQ4_XS), ("iq3_xxs", qk.IQ3_XXS)):
+        def sustained(t):
             Ms = -(-(256 << 20) // qk.row_bytes(t, 2048) // 64) * 64
             g = gemv_workload(qk, t, Ms, 2048, 1, 40, 4, ring=2)
             gb = g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9
-            ex[f"gemv_{name}_sustained_256MiB"] = dict(rows=Ms, us=g["ms_event"] * 1e3, gbps=gb, frac=gb / HBM_PEAK_GBPS,
-                                                       steps_timed=g["steps"])
-            log(f"[bench] gemv {name} sustained: {ex[f'gemv_{name}_sustained_256MiB']}")
+            return dict(rows=Ms, us=g["ms_event"] * 1e3, gbps=gb, frac=gb / HBM_PEAK_GBPS, steps_timed=g["steps"])
+        for name, t in (("q8_0", qk.Q8_0), ("q6_k", qk.Q6_K), ("iq4_xs", qk.IQ4_XS), ("iq3_xxs", qk.IQ3_XXS)):
+            guarded(ex, f"gemv_{name}_sustained_256MiB", lambda t=t: sustained(t))
             torch.cuda.empty_cache()
         # the other dense projections of a decode step at the reference's shapes (src/main.cpp:4310-4335)
         for M, K in ((4096, 2048), (2048, 4096), (512, 2048)):
@@ -714,17 +644,17 @@ def main():
         if a.workload == "moe_decode_bs1":
             # the same step on ONE layer replayed: its 16 MB stay in the caches, so this is the step without
             # HBM in the way (launch, selection and dependency chain) beside the ring's figure above
-            mh = moe_workload(qk, 1, qk.IQ4_XS, 1, 400, 40)
-            ex["moe_decode_bs1_cache_hot"] = dict(us=mh["ms_event"] * 1e3, steps_timed=mh["steps"],
-                                                  stage_us={k: v * 1e3 for k, v in mh["stage_ms"].items()})
-            log(f"[bench] moe bs1, one layer replayed: {ex['moe_decode_bs1_cache_hot']}")
+            def cache_hot():
+                mh = moe_workload(qk, 1, qk.IQ4_XS, 1, 400, 40)
+                return dict(us=mh["ms_event"] * 1e3, steps_timed=mh["steps"], stage_us={k: v * 1e3 for k, v in mh["stage_ms"].items()})
+            guarded(ex, "moe_decode_bs1_cache_hot", cache_hot)
             torch.cuda.empty_cache()
+
             # the ring's tensors carved from one allocation: what the many separate mappings cost, if anything
-            ms = moe_workload(qk, 1, qk.IQ4_XS, a.ring, min(steps, 800), a.warmup, slab=True)
-            ex["moe_decode_bs1_ring_in_one_allocation"] = dict(us=ms["ms_event"] * 1e3, steps_timed=ms["steps"],
-                                                               stage_us={k: v * 1e3 for k, v in ms["stage_ms"].items()})
-            log(f"[bench] moe bs1, ring in one allocation: {ex['moe_decode_bs1_ring_in_one_allocation']}")
-            del ms
+            def one_allocation():
+                ms = moe_workload(qk, 1, qk.IQ4_XS, a.ring, min(steps, 800), a.warmup, slab=True)
+                return dict(us=ms["ms_event"] * 1e3, steps_timed=ms["steps"], stage_us={k: v * 1e3 for k, v in ms["stage_ms"].items()})
+            guarded(ex, "moe_decode_bs1_ring_in_one_allocation", one_allocation)
             torch.cuda.empty_cache()
             m16 = moe_workload(qk, 16, qk.Q6_K, 4, 200, 20)
             ex["moe_decode_bs16_q6k_down"] = dict(us=m16["ms_event"] * 1e3, distinct_experts=m16["distinct_experts"],
@@ -770,10 +700,10 @@ def main():
                                                         ring=at["ring"])
                 torch.cuda.empty_cache()
             log(f"[bench] attention: {ex['attn_decode_ctx4096_bs1']} {ex['attn_decode_ctx4096_bs16']}")
-            ap = attn_prefill_workload(qk, 1024, 40, 8)   # the attention mixer over a 1,024-position prompt
-            ex["attn_prefill_1024_positions"] = dict(us=ap["ms_event"] * 1e3, tflops=ap["flops"] / (ap["ms_event"] * 1e-3) / 1e12,
-                                                     steps_timed=ap["steps"])
-            log(f"[bench] attention prefill: {ex['attn_prefill_1024_positions']}")
+            def attn_prefill():   # the attention mixer over a 1,024-position prompt
+                ap = attn_prefill_workload(qk, 1024, 40, 8)
+                return dict(us=ap["ms_event"] * 1e3, tflops=ap["flops"] / (ap["ms_event"] * 1e-3) / 1e12, steps_timed=ap["steps"])
+            guarded(ex, "attn_prefill_1024_positions", attn_prefill)
             torch.cuda.empty_cache()
             for b in (1, 16):   # the gated-DeltaNet mixer's decode step
                 dn = deltanet_workload(qk, b, 256, 32)
@@ -789,9 +719,7 @@ def main():
         out["extras"] = ex
 
     if a.cpu:
-        orc = entry.load_oracle()
-        out["cpu_baseline"] = cpu_baseline(qk, orc)
-        log(f"[bench] cpu baseline: {out['cpu_baseline']}")
+        guarded(out, "cpu_baseline", lambda: cpu_baseline(qk, entry.load_oracle()))
     print(json.dumps(out), flush=True)
 
 
