@@ -101,8 +101,8 @@ def test_next_token_maps(world, orc):
     import copy
     short = copy.copy(model)
     short.layers, short.post_norm = model.layers[:1], model.post_norm[:1]
-    changed = sum(OE.stack_next(short, t) != nxt1[t] for t in range(0, VOCAB, 64))
-    assert changed >= 8, changed
+    changed = sum(OE.stack_next(short, t) != nxt1[t] for t in range(0, VOCAB, VOCAB // 16))
+    assert changed >= 8, changed   # of sixteen samples
 
 
 def drive(eng, ref, script, n_calls):
