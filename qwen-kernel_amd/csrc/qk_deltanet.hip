@@ -243,14 +243,18 @@ __global__ __launch_bounds__(DN_DS* DN_PARTS) void dn_fused_step_kernel(
     const uint32_t channels = (2 * hK + hV) * DN_DS;
     const uint32_t hd[2] = {kdiv ? kh * kdiv : kh, kdiv ? kh * kdiv + 1 : kh + hK}; // the two value heads of key head kh
 
-    // the state of both heads: requested before anything else
+    // the state of both heads: requested before anything else -- except by the four waves that form the dot
+    // products, whose operands need the registers first (they request it when those are done)
     float s[2][DN_PC];
     float* S[2];
+    const bool dots = c == 4 || c == 5; // uniform per wave
 #pragma unroll
-    for (int a = 0; a < 2; a++) {
-        S[a] = state + ((size_t)rq * hV + hd[a]) * DN_DS * DN_DS + (size_t)c * DN_PC * DN_DS + j;
+    for (int a = 0; a < 2; a++) S[a] = state + ((size_t)rq * hV + hd[a]) * DN_DS * DN_DS + (size_t)c * DN_PC * DN_DS + j;
+    if (!dots) {
 #pragma unroll
-        for (uint32_t i = 0; i < DN_PC; i++) s[a][i] = S[a][(size_t)i * DN_DS];
+        for (int a = 0; a < 2; a++)
+#pragma unroll
+            for (uint32_t i = 0; i < DN_PC; i++) s[a][i] = S[a][(size_t)i * DN_DS];
     }
     const float zv[2] = {z[((size_t)rq * hV + hd[0]) * DN_DS + j], z[((size_t)rq * hV + hd[1]) * DN_DS + j]};
     const float nwj = norm_w[j];
@@ -306,6 +310,10 @@ __global__ __launch_bounds__(DN_DS* DN_PARTS) void dn_fused_step_kernel(
                 s_gb[a] = expf(a_vec[hd[a]] * (v > 20.f ? v : log1pf(expf(v))));
             }
         }
+#pragma unroll
+        for (int a2 = 0; a2 < 2; a2++)
+#pragma unroll
+            for (uint32_t i = 0; i < DN_PC; i++) s[a2][i] = S[a2][(size_t)i * DN_DS];
     }
     __syncthreads();
     // unit length for q and k (as block_sum2 in dn_conv_kernel: the two waves' sums in wave order), q also / sqrt(dS)
