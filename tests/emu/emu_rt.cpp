@@ -13,6 +13,7 @@
 #include <unistd.h>
 
 #include <atomic>
+#include <condition_variable>
 #include <mutex>
 #include <thread>
 #include <vector>
@@ -58,6 +59,7 @@ struct Fiber {
     bool done = false;
     int wait_kind = 0; // 0 runnable, 1 wave barrier, 2 block barrier
     uint64_t wait_gen = 0;
+    uint32_t xn = 0; // cross-lane operations done so far: the same in every lane of a wave (they run in lockstep)
 };
 
 // n bytes that END at an inaccessible page: an access behind the buffer faults at once.
@@ -88,8 +90,11 @@ struct Workgroup {
     const std::function<void()>* body = nullptr;
     uint64_t block_gen = 0, wave_gen[MAX_WAVES] = {};
     int block_arrived = 0, block_expected = 0, wave_arrived[MAX_WAVES] = {}, wave_expected[MAX_WAVES] = {};
-    uint64_t xbuf[MAX_WAVES][64];
-    _Float16 mfma_a[MAX_WAVES][64][8], mfma_b[MAX_WAVES][64][8];
+    // Two buffers in turn: operation n + 2 writes where operation n was read, and a lane reaches it only through
+    // the barrier of operation n + 1, which every lane passes after it has read n -- so one barrier per
+    // operation is enough.
+    uint64_t xbuf[MAX_WAVES][2][64];
+    float mfma_a[MAX_WAVES][2][64][8], mfma_b[MAX_WAVES][2][64][8]; // the halves, widened once by the lane that owns them
     GuardBuf* dyn = nullptr;
     ~Workgroup()
     {
@@ -141,6 +146,7 @@ void prepare_fiber(Fiber& fb, uint32_t tid)
     fb.tid = Idx{tid, 0, 0};
     fb.done = false;
     fb.wait_kind = 0;
+    fb.xn = 0;
 }
 
 void run_workgroup(Workgroup& g, Idx block, int n, size_t lds, const std::function<void()>& body)
@@ -220,12 +226,68 @@ void wave_barrier()
 const uint64_t* exchange(uint64_t v)
 {
     Workgroup& g = *t_wg;
-    const uint32_t t = g.cur->tid.x;
-    g.xbuf[t >> 6][t & 63u] = v;
+    const uint32_t t = g.cur->tid.x, par = g.cur->xn++ & 1u;
+    g.xbuf[t >> 6][par][t & 63u] = v;
     wave_barrier();
-    return t_wg->xbuf[t >> 6];
+    return t_wg->xbuf[t >> 6][par];
 }
-void exchange_done() { wave_barrier(); }
+void exchange_done() {} // the values stay valid until the wave's next operation but one
+
+// Helper threads that live as long as the process (QK_EMU_THREADS, default the host's cores, minus the caller).
+struct Pool {
+    unsigned size = 0;
+    std::mutex m;
+    std::condition_variable wake, idle;
+    uint64_t gen = 0;
+    unsigned wanted = 0, taken = 0, running = 0;
+    const std::function<void()>* job = nullptr;
+    void loop()
+    {
+        uint64_t seen = 0;
+        for (;;) {
+            const std::function<void()>* j = nullptr;
+            {
+                std::unique_lock<std::mutex> l(m);
+                wake.wait(l, [&] { return gen != seen && taken < wanted; });
+                seen = gen;
+                taken++;
+                j = job;
+            }
+            (*j)();
+            {
+                std::lock_guard<std::mutex> l(m);
+                if (--running == 0) idle.notify_all();
+            }
+        }
+    }
+    void start(const std::function<void()>& j, unsigned n)
+    {
+        std::lock_guard<std::mutex> l(m);
+        job = &j;
+        wanted = running = n;
+        taken = 0;
+        gen++;
+        wake.notify_all();
+    }
+    void wait()
+    {
+        std::unique_lock<std::mutex> l(m);
+        idle.wait(l, [&] { return running == 0; });
+        wanted = 0;
+    }
+};
+static Pool& the_pool()
+{
+    static Pool* p = [] {
+        Pool* q = new Pool; // never destroyed: its threads outlive main's statics
+        const char* e = getenv("QK_EMU_THREADS");
+        const unsigned v = e ? (unsigned)atoi(e) : std::thread::hardware_concurrency();
+        q->size = v > 1 ? v - 1 : 0;
+        for (unsigned i = 0; i < q->size; i++) std::thread([q] { q->loop(); }).detach();
+        return q;
+    }();
+    return *p;
+}
 
 void run(dim3 grid, dim3 block, size_t lds, const std::function<void()>& body)
 {
@@ -239,25 +301,23 @@ void run(dim3 grid, dim3 block, size_t lds, const std::function<void()>& body)
     g_grid_dim = Idx{grid.x, grid.y, grid.z};
     const uint64_t total = (uint64_t)grid.x * grid.y * grid.z;
     std::atomic<uint64_t> next{0};
+    // Every OS thread keeps its Workgroup (the fibers' stacks) from launch to launch: mapping a thousand stacks
+    // per launch cost more than small kernels themselves.
     auto worker = [&] {
-        Workgroup g;
+        static thread_local Workgroup* mine = new Workgroup; // lives as long as the thread
         for (;;) {
             const uint64_t b = next.fetch_add(1);
             if (b >= total) break;
             const Idx bi{(uint32_t)(b % grid.x), (uint32_t)(b / grid.x % grid.y), (uint32_t)(b / ((uint64_t)grid.x * grid.y))};
-            run_workgroup(g, bi, n, lds, body);
+            run_workgroup(*mine, bi, n, lds, body);
         }
     };
-    static const unsigned hw = [] {
-        const char* e = getenv("QK_EMU_THREADS");
-        const unsigned v = e ? (unsigned)atoi(e) : std::thread::hardware_concurrency();
-        return v ? v : 1u;
-    }();
-    const unsigned nt = (unsigned)std::min<uint64_t>(hw, total);
-    std::vector<std::thread> threads;
-    for (unsigned i = 1; i < nt; i++) threads.emplace_back(worker);
+    Pool& pool = the_pool();
+    const unsigned helpers = (unsigned)std::min<uint64_t>(pool.size, total > 1 ? total - 1 : 0);
+    const std::function<void()> job = worker; // outlives the helpers' use of it: wait() returns after the last one
+    if (helpers) pool.start(job, helpers);
     worker();
-    for (auto& th : threads) th.join();
+    if (helpers) pool.wait();
 }
 
 // ---- stream capture ---------------------------------------------------------------------------
@@ -289,10 +349,10 @@ emu_float4 emu_mfma_16x16x32_f16(emu_half8 a, emu_half8 b, emu_float4 c)
 {
     using namespace emu;
     Workgroup& g = *t_wg;
-    const uint32_t t = g.cur->tid.x, w = t >> 6, lane = t & 63u;
+    const uint32_t t = g.cur->tid.x, w = t >> 6, lane = t & 63u, par = g.cur->xn++ & 1u;
     for (int i = 0; i < 8; i++) {
-        g.mfma_a[w][lane][i] = a[i];
-        g.mfma_b[w][lane][i] = b[i];
+        g.mfma_a[w][par][lane][i] = (float)a[i];
+        g.mfma_b[w][par][lane][i] = (float)b[i];
     }
     wave_barrier();
     const uint32_t col = lane & 15u, rq = lane >> 4;
@@ -301,10 +361,9 @@ emu_float4 emu_mfma_16x16x32_f16(emu_half8 a, emu_half8 b, emu_float4 c)
         const uint32_t row = 4 * rq + i;
         float s = 0.f;
         for (uint32_t kq = 0; kq < 4; kq++)
-            for (int j = 0; j < 8; j++) s += (float)g.mfma_a[w][row + 16 * kq][j] * (float)g.mfma_b[w][col + 16 * kq][j];
+            for (int j = 0; j < 8; j++) s += g.mfma_a[w][par][row + 16 * kq][j] * g.mfma_b[w][par][col + 16 * kq][j];
         d[i] += s;
     }
-    wave_barrier();
     return d;
 }
 
