@@ -219,7 +219,7 @@ def test_serial_prefill_and_eager_launches_give_the_same_streams(qk, world, monk
                     got[s] += a[1][s]
             streams[mode] = got
     assert streams["graph"] == streams["eager"]
-    assert sum(len(v) for v in streams["graph"].values()) > 30
+    assert sum(len(v) for v in streams["graph"].values()) > 20   # the streams ran on (an end id early in a stream shortens it)
 
 
 def test_stage_run_and_topk(qk, world):
