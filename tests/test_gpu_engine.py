@@ -4,7 +4,7 @@ state machine and the stage calls, against
     engine in tests/test_engine_oracle.py), driven by the model's next-token map;
   - that map computed by the same kernels through the operator-level ABI, one launch at a time
     (bit-identical ids expected: same kernels, same inputs);
-  - the CPU oracle's model step for a sample of tokens (greedy ids equal wherever the oracle's
+  - the CPU oracle's model step for every token of the vocabulary (greedy ids equal wherever the oracle's
     top-2 logit gap exceeds 2e-3 of the largest logit, the GEMV/MoE tolerance of 1e-3 on either side)."""
 import os
 import sys
