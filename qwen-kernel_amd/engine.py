@@ -13,13 +13,9 @@ class Config(C.Structure):
     _fields_ = [("n_slots", C.c_uint32), ("n_ctx", C.c_uint32), ("chunk", C.c_uint32)]
 
 
-_bound = False
-
-
 def _lib():
-    global _bound
     L = capi.lib()
-    if not _bound:
+    if not getattr(L, "_qk_engine_bound", False):   # per library object: the tests also load a host-side build
         vp, u32 = C.c_void_p, C.c_uint32
         L.qk_open.restype = vp
         L.qk_open.argtypes = [C.c_char_p, C.POINTER(Config), C.c_char_p, C.c_size_t]
@@ -37,7 +33,7 @@ def _lib():
         L.qk_stage_topk.argtypes = [vp, u32, vp, vp]
         L.qk_state_save.argtypes = [vp, u32, u32, u32]
         L.qk_state_load.argtypes = [vp, u32, u32, u32]
-        _bound = True
+        L._qk_engine_bound = True
     return L
 
 

@@ -107,7 +107,13 @@ static inline hipError_t hipHostFree(void* p) { free(p); return hipSuccess; }
 static inline hipError_t hipMemcpy(void* d, const void* s, size_t n, hipMemcpyKind) { memmove(d, s, n); return hipSuccess; }
 static inline hipError_t hipMemset(void* d, int v, size_t n) { memset(d, v, n); return hipSuccess; }
 static inline hipError_t hipMemsetAsync(void* d, int v, size_t n, hipStream_t = nullptr) { emu::submit([=]() { memset(d, v, n); }); return hipSuccess; }
-static inline hipError_t hipMemGetInfo(size_t* f, size_t* t) { *f = (size_t)64 << 30; *t = (size_t)64 << 30; return hipSuccess; }
+static inline hipError_t hipMemGetInfo(size_t* f, size_t* t)
+{   // 64 GB free unless QK_EMU_FREE_BYTES says otherwise (for tests of the callers' checks)
+    const char* e = getenv("QK_EMU_FREE_BYTES");
+    *f = e ? (size_t)strtoull(e, nullptr, 10) : (size_t)64 << 30;
+    *t = (size_t)64 << 30;
+    return hipSuccess;
+}
 static inline hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
 static inline hipError_t hipDeviceSynchronize() { return hipSuccess; }
 static inline hipError_t hipStreamDestroy(hipStream_t) { return hipSuccess; }

@@ -220,3 +220,23 @@ def test_dense_gemv_inside_its_tensors(qk, orc, emu, name, K, M):
     qk.gemv(t, emu.tensor(W.reshape(-1)), emu.tensor(x), M, K, out=Yd)
     want = orc.gemv(t, W, x[0], M, K)
     assert orc.rel_maxabs_err(Yd.numpy()[0], want) <= 1e-3
+
+
+def test_engine_in_the_host_build_and_its_memory_check(qk, emu, tmp_path, monkeypatch):
+    """qk_open through the host-side build: a small whole-model file opens and steps; with sixteen slots of
+    4,096 positions the attention caches and their snapshots need 0.6 GB on top of the 0.5 GB of the model and
+    the rows of a pass, and a device that reports 1 GB free (QK_EMU_FREE_BYTES) refuses the configuration before
+    any tensor is uploaded, with the figures in the message; one slot of 64 positions still fits."""
+    model = qk.engine.FullModel(5, kinds="AAR", vocab=64, n_expert=8, n_ff=256, n_used=2, eos=70)
+    path = model.write(str(tmp_path / "m.gguf"))
+    with qk.engine.Engine(path, n_slots=1, n_ctx=64, chunk=2) as eng:
+        assert (eng.n_layer, eng.vocab) == (3, 64)
+        assert eng.slot_start(0, [3, 5], 3) == 0
+        rc, out, fin = eng.step_chunk()
+        assert rc == 1 and 1 <= len(out[0]) <= 2 and all(t < 64 for t in out[0])
+    monkeypatch.setenv("QK_EMU_FREE_BYTES", str(1 << 30))
+    with pytest.raises(qk.capi.QkError) as e:
+        qk.engine.Engine(path, n_slots=16, n_ctx=4096, chunk=2)
+    assert "GB" in str(e.value) and "16 slot" in str(e.value)
+    with qk.engine.Engine(path, n_slots=1, n_ctx=64, chunk=2) as eng:   # one slot of 64 positions still fits
+        assert eng.n_slots == 1
