@@ -240,3 +240,29 @@ def test_engine_in_the_host_build_and_its_memory_check(qk, emu, tmp_path, monkey
     assert "GB" in str(e.value) and "16 slot" in str(e.value)
     with qk.engine.Engine(path, n_slots=1, n_ctx=64, chunk=2) as eng:   # one slot of 64 positions still fits
         assert eng.n_slots == 1
+
+
+def test_whole_model_stream_in_the_host_build(qk, emu, tmp_path):
+    """The engine on a small whole model (one gated-DeltaNet layer, one attention layer, a MoE block each)
+    through the host-side build: two slots' greedy streams -- prompts prefilled in a pass, then serial steps
+    from a replayed graph -- equal the restated state machine driving the CPU oracle of the whole model,
+    call by call."""
+    import os
+    import sys
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle"))
+    import qk_oracle_engine as OE
+    vocab = 96
+    model = qk.engine.FullModel(9, kinds="RA", vocab=vocab, n_expert=8, n_ff=256, n_used=2, eos=vocab + 5)
+    path = model.write(str(tmp_path / "m.gguf"))
+    rng = np.random.default_rng(2)
+    prompts = {1: [int(t) for t in rng.integers(0, vocab, 7)], 0: [int(t) for t in rng.integers(0, vocab, 1)]}
+    with qk.engine.Engine(path, n_slots=2, n_ctx=64, chunk=3) as eng:
+        ref = OE.SlotMachine(OE.FullModelOracle(model, 2, 64), vocab, vocab + 5, 2, 64, 3)
+        for call in range(4):
+            if call == 0:
+                assert eng.slot_start(1, prompts[1], 5) == ref.slot_start(1, prompts[1], 5) == 0
+            if call == 1:
+                assert eng.slot_start(0, prompts[0], 4) == ref.slot_start(0, prompts[0], 4) == 0
+            got, want = eng.step_chunk(), ref.step_chunk()
+            assert got == want, (call, got, want)
+        assert not any(sl["active"] for sl in ref.slots)
