@@ -266,3 +266,85 @@ def test_whole_model_stream_in_the_host_build(qk, emu, tmp_path):
             got, want = eng.step_chunk(), ref.step_chunk()
             assert got == want, (call, got, want)
         assert not any(sl["active"] for sl in ref.slots)
+
+
+@pytest.mark.parametrize("down,n", [("iq4_xs", 16), ("q6_k", 40)])
+def test_expert_major_moe_inside_its_tensors(qk, orc, emu, down, n):
+    """The expert-major path (more than ten rows: routing with selection in the last workgroup, the
+    matrix-core gate/up and down kernels, the fold) on guarded tensors and a guarded workspace, 16 rows
+    (the fused launches) and 40 rows (the shared expert on its own launches), against the oracle."""
+    hl = qk.synth.HostLayer(seed=31 + n, n_ff=256, n_expert=8, n_used=2, down_type=type_id(qk, down))
+    x = np.random.default_rng(n).standard_normal((n, 2048)).astype(np.float32)
+    ids = moe_case(qk, orc, emu, hl, x)
+    assert ids.shape == (n, 2) and set(np.unique(ids)) <= set(range(8))
+    qk.moe_workspace_status()   # the cleared workspace raised no flag
+
+
+@pytest.mark.parametrize("M,K,N", [(48, 2048, 20), (33, 512, 9), (16, 4096, 128)])
+def test_q8_0_gemm_inside_its_tensors(qk, orc, emu, M, K, N):
+    """The prefill GEMM (cooperative matrix-core stream, weights read once for all rows) on a tensor that ends
+    at the guard page, against the oracle's double-precision product."""
+    W = qk.synth.tensor_host(qk.Q8_0, M, K, seed=M + N)
+    X = np.random.default_rng(N).standard_normal((N, K)).astype(np.float32)
+    Y = emu.zeros((N, M), np.float32)
+    qk.gemm_q8_0(emu.tensor(W.reshape(-1)), emu.tensor(X), M, K, out=Y)
+    want = orc.gemm_q8_0(W, X, M, K)
+    assert orc.rel_maxabs_err(Y.numpy(), want) <= 1e-3
+
+
+def _oracle_module(name):
+    import importlib
+    import os
+    import sys
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle"))
+    return importlib.import_module(name)
+
+
+def test_attention_decode_inside_its_tensors(qk, emu):
+    """The attention decode step (prep + position ranges + fold) for two slots whose caches end at the guard
+    page, the second slot at the cache's last position, against the CPU mirror."""
+    OA = _oracle_module("qk_oracle_attn")
+    DH, NROT, HQ, HKV, tmax, positions = 256, 64, 16, 2, 96, [5, 95]
+    rng = np.random.default_rng(1)
+    kc, vc = np.zeros((2, HKV, tmax, DH), np.float32), np.zeros((2, HKV, tmax, DH), np.float32)
+    for s, p in enumerate(positions):
+        kc[s, :, :p], vc[s, :, :p] = rng.standard_normal((HKV, p, DH)), rng.standard_normal((HKV, p, DH))
+    qfull = (rng.standard_normal((2, HQ, 2 * DH)) * 2).astype(np.float32)
+    kin, vin = rng.standard_normal((2, HKV, DH)).astype(np.float32), rng.standard_normal((2, HKV, DH)).astype(np.float32)
+    qn, kn = (1 + 0.2 * rng.standard_normal(DH)).astype(np.float32), (1 + 0.2 * rng.standard_normal(DH)).astype(np.float32)
+    rope = OA.rope_table(tmax, NROT)
+    kd, vd, qfd = emu.tensor(kc), emu.tensor(vc), emu.tensor(qfull)
+    pos = emu.tensor(np.array(positions, dtype=np.int32))
+    qh = qk.attn_prep(qfd, emu.tensor(kin), emu.tensor(vin), emu.tensor(qn), emu.tensor(kn), emu.tensor(rope), pos, kd, vd, NROT,
+                      qhat=emu.zeros((2, HQ, DH), np.float32))
+    att = qk.attn_decode(qh, kd, vd, qfd, pos, emu.workspace(qk.attn_workspace_bytes(2, HQ)),
+                         att=emu.zeros((2, HQ, DH), np.float32)).numpy()
+    for s, p in enumerate(positions):
+        want = OA.attend(OA.prep(qfull[s], kin[s], vin[s], qn, kn, rope, p, kc[s], vc[s], NROT), kc[s], vc[s], qfull[s], p)
+        assert float(np.max(np.abs(att[s] - want)) / np.max(np.abs(want))) <= 1e-3, s
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_deltanet_step_inside_its_tensors(qk, emu, fused):
+    """The gated-DeltaNet decode step for two slots -- as the two launches and as the one launch -- on guarded
+    window, state and weight tensors, against the CPU mirror."""
+    OD = _oracle_module("qk_oracle_deltanet")
+    DS, HK, HV, NE = 128, 16, 32, 2048
+    CH, QK = (2 * HK + HV) * DS, 2 * HK * DS
+    rng = np.random.default_rng(3)
+    r = lambda *shape, scale=1.0: (rng.standard_normal(shape) * scale).astype(np.float32)
+    alpha_w, beta_w, dt_bias = r(HV, NE, scale=0.03), r(HV, NE, scale=0.03), r(HV)
+    a_vec, ker, norm_w = (-np.abs(r(HV)) - 0.05).astype(np.float32), r(CH, 4, scale=0.5), (1 + 0.1 * r(DS)).astype(np.float32)
+    st, S = r(2, CH, 3), r(2, HV, DS, DS, scale=0.1)
+    x, qkv, z = r(2, NE), r(2, CH), r(2, HV * DS)
+    std, Sd = emu.tensor(st), emu.tensor(np.ascontiguousarray(S.transpose(0, 1, 3, 2)))
+    w = [emu.tensor(a) for a in (alpha_w, beta_w, dt_bias, a_vec)]
+    if fused:
+        att = qk.dn_step_fused(emu.tensor(x), *w, std, emu.tensor(qkv), emu.tensor(ker), Sd, emu.tensor(norm_w), emu.tensor(z), HK, HV)
+    else:
+        gb, conv = qk.dn_ab_conv(emu.tensor(x), *w, std, emu.tensor(qkv), emu.tensor(ker), QK)
+        att = qk.dn_step(conv, gb, Sd, emu.tensor(norm_w), emu.tensor(z), HK, HV)
+    for s in range(2):
+        g, b = OD.ab(x[s], alpha_w, beta_w, dt_bias, a_vec)
+        want = OD.step(OD.conv(st[s].copy(), qkv[s], ker, DS, QK), g, b, S[s].copy(), norm_w, z[s], HK, HV)
+        assert float(np.max(np.abs(att.numpy()[s] - want)) / np.max(np.abs(want))) <= 1e-3, s
