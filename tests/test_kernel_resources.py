@@ -58,3 +58,45 @@ def test_streaming_kernels_keep_two_waves_per_simd(usage):
     assert len(hot) >= 20, len(hot)
     low = {k: usage[k] for k in hot if usage[k]["occupancy"] < 2}
     assert not low, low
+
+
+def isa_of(path):
+    import tempfile
+    with tempfile.TemporaryDirectory() as tmp:
+        out = os.path.join(tmp, "k.s")
+        r = subprocess.run([HIPCC, "--offload-arch=gfx950", "--cuda-device-only", "-O3", "-std=c++17", "-Xclang", "-target-feature",
+                            "-Xclang", "-packed-fp32-ops", "-I" + os.path.join(ROOT, "include"), "-S", path, "-o", out],
+                           capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr[-2000:]
+        text = open(out).read()
+    funcs = {}
+    for chunk in re.split(r"\n(?=_ZN2qk\w+:)", text):
+        name = chunk.split(":", 1)[0]
+        if name.startswith("_ZN2qk"):
+            funcs[name] = chunk.split(".end_amdhsa_kernel")[0]
+    return funcs
+
+
+def test_one_row_kernels_fetch_the_weights_as_16_byte_pieces():
+    """The instruction stream of the one-row kernels at the reference's shapes: the weight bytes arrive through
+    global_load_dwordx4 (the staged 16-byte pieces, the activations, the tables' sources); in the GEMV and
+    head kernels narrower global loads remain only for the rows behind the last full chunk -- at most a third
+    as many as the wide ones (the MoE launches also fetch logits, picks and h)."""
+    if not os.path.exists(HIPCC):
+        pytest.skip("no hipcc")
+    files = [os.path.join(CSRC, f) for f in ("qk_gemv.hip", "qk_head.hip", "qk_moe.hip")]
+    with concurrent.futures.ThreadPoolExecutor(max_workers=3) as pool:
+        funcs = {}
+        for d in pool.map(isa_of, files):
+            funcs.update(d)
+    hot = [k for k in funcs if ("gemv_stream_kernelILi" in k and "ELi64ELi1E" in k) or "head_q6k_kernelILi1E" in k
+           or "moe_route_kernelILi8ELb0E" in k or "moe_gateup_kernelILi1ELi4ELb0E" in k
+           or re.search(r"moe_down_kernelILi(23|14)ELi16ELi2ELi2ELb[01]ELb0E", k)]
+    assert len(hot) >= 16, len(hot)
+    for k in hot:
+        loads = re.findall(r"\bglobal_load_(\w+)", funcs[k])
+        wide = sum(1 for l in loads if l.startswith("dwordx4"))
+        narrow = len(loads) - wide
+        assert wide >= 8, (k, wide, narrow)
+        if "gemv_stream" in k or "head_q6k" in k:   # the MoE launches also fetch logits, picks and h: scalars and short rows
+            assert narrow * 3 <= wide, (k, wide, narrow, sorted(set(loads)))
