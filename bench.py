@@ -24,6 +24,7 @@ sys.path.insert(0, ROOT)
 import __graft_entry__ as entry  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0   # dense fp16 matrix peak
 MIN_REPLAYS = 20   # graph replays timed at least, whatever --steps says (steps timed = replays x ring, reported)
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by what the same
 # counters read for a plain 256 MiB copy (profiles/); None where no counter run of the CURRENT kernel
@@ -538,6 +539,131 @@ def cpu_baseline(qk, orc):
                 host_cpus=os.cpu_count(), per_config=per)
 
 
+def qk_env():
+    """The library's environment switches that were set for this run (they change which kernels run)."""
+    return {k: v for k, v in os.environ.items() if k.startswith("QK_")}
+
+
+def rate(bytes_step, ms, **more):
+    gb = bytes_step / (ms * 1e-3) / 1e9
+    return dict(us=ms * 1e3, gbps=gb, frac=gb / HBM_PEAK_GBPS, **more)
+
+
+def gemv_entry(qk, t, M, K, batch, steps, warmup):
+    """One GEMV figure; M = None: a sustained size (one tensor of at least 256 MiB per launch, two tensors
+    alternating, so neither launch latency nor the caches carry the figure)."""
+    if M is None:
+        M = -(-(256 << 20) // qk.row_bytes(t, K) // 64) * 64
+        g = gemv_workload(qk, t, M, K, batch, steps, warmup, ring=2)
+    else:
+        g = gemv_workload(qk, t, M, K, batch, steps, warmup)
+    return rate(g["bytes_step"], g["ms_event"], rows=M, steps_timed=g["steps"])
+
+
+def gemm_entry(qk):
+    g = gemm_workload(qk, 8192, 2048, 128, 200, 20)
+    tf = g["flops"] / (g["ms_event"] * 1e-3) / 1e12
+    return dict(us=g["ms_event"] * 1e3, tflops=tf, frac_mfma_peak=tf / MFMA_F16_PEAK_TFLOPS,
+                gbps=g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9,
+                frac_hbm_peak=g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9 / HBM_PEAK_GBPS)
+
+
+def extras(qk, a, steps):
+    """The other BASELINE configs (C1 GEMVs, C3 16-slot step, C4 head, C5 prefill) and the rows beside the
+    path (glue, mixers, engine), each as an entry of its own; a failing one becomes an error entry."""
+    import torch
+    ex = {}
+    es, ew = 400, 40
+    fmts = (("q8_0", qk.Q8_0), ("q6_k", qk.Q6_K), ("iq4_xs", qk.IQ4_XS), ("iq3_xxs", qk.IQ3_XXS), ("f16", qk.F16))
+
+    def run(key, fn):
+        guarded(ex, key, fn)
+        torch.cuda.empty_cache()
+
+    for name, t in fmts:   # C1 and its four sisters, one slot and sixteen (weights read once)
+        run(f"gemv_{name}_8192x2048", lambda t=t: gemv_entry(qk, t, 8192, 2048, 1, es, ew))
+        if t != qk.F16:
+            run(f"gemv_{name}_8192x2048_bs16", lambda t=t: gemv_entry(qk, t, 8192, 2048, 16, es, ew))
+    for name, t in fmts:
+        run(f"gemv_{name}_sustained_256MiB", lambda t=t: gemv_entry(qk, t, None, 2048, 1, 40, 4))
+    for b in (1, 16):   # C4
+        def head(b=b):
+            h = head_workload(qk, 151936, 2048, b, 40, 8)
+            return rate(h["bytes_step"], h["ms_event"], steps_timed=h["steps"])
+        run(f"head_q6k_151936_bs{b}", head)
+
+    def stages(m, **more):
+        return dict(us=m["ms_event"] * 1e3, steps_timed=m["steps"], stage_us={k: v * 1e3 for k, v in m["stage_ms"].items()}, **more)
+
+    def moe16():   # C3
+        m16 = moe_workload(qk, 16, qk.Q6_K, 4, 200, 20)
+        r = rate(m16["bytes_step"], m16["ms_event"], distinct_experts=m16["distinct_experts"])
+        r["stage_us"] = {k: v * 1e3 for k, v in m16["stage_ms"].items()}
+        return r
+    run("moe_decode_bs16_q6k_down", moe16)
+    run("prefill_gemm_q8_0_8192x2048x128", lambda: gemm_entry(qk))   # C5a
+
+    def prefill_moe():   # C5b
+        pm = prefill_moe_workload(qk, 128, 20, 4)
+        tf = pm["flops"] / (pm["ms_event"] * 1e-3) / 1e12
+        return rate(pm["bytes_step"], pm["ms_event"], tok_per_s=128 / (pm["ms_event"] * 1e-3),
+                    distinct_experts=pm["distinct_experts"], tflops=tf, frac_mfma_peak=tf / MFMA_F16_PEAK_TFLOPS)
+    run("prefill_moe_128_tokens", prefill_moe)
+    # the same step on ONE layer replayed: its 16 MB stay in the caches, so this is the step without
+    # HBM in the way (launch, selection and dependency chain) beside the ring's figure
+    run("moe_decode_bs1_cache_hot", lambda: stages(moe_workload(qk, 1, qk.IQ4_XS, 1, 400, 40)))
+    # the ring's tensors carved from one allocation: what the many separate mappings cost, if anything
+    run("moe_decode_bs1_ring_in_one_allocation",
+        lambda: stages(moe_workload(qk, 1, qk.IQ4_XS, a.ring, min(steps, 800), a.warmup, slab=True)))
+    # the other dense projections of a decode step at the reference's shapes (src/main.cpp:4310-4335)
+    for M, K in ((4096, 2048), (2048, 4096), (512, 2048)):
+        for b in (1, 16):
+            run(f"gemv_q8_0_{M}x{K}" + ("_bs16" if b > 1 else ""), lambda M=M, K=K, b=b: gemv_entry(qk, qk.Q8_0, M, K, b, es, ew))
+    # a few concurrent slots: every row through the one-row launches (grid.y = row)
+    for nr in (2, 4, 8):
+        run(f"moe_decode_{nr}_rows_q6k_down", lambda nr=nr: dict(us=moe_workload(qk, nr, qk.Q6_K, 8, 400, 40)["ms_event"] * 1e3))
+    # layer glue (add + RMS norm alone, and behind the step in one call)
+    run("add_rmsnorm_2048", lambda: dict(us_1_row=norm_workload(qk, 1, 640, 64), us_16_rows=norm_workload(qk, 16, 640, 64)))
+    run("moe_decode_tail_bs1", lambda: dict(us=moe_tail_workload(qk, 1, qk.IQ4_XS, 8, 400, 40)))
+    run("moe_layer_row_bs1", lambda: dict(us=moe_tail_workload(qk, 1, qk.IQ4_XS, 8, 400, 40, layer_row=True)))
+    run("moe_decode_tail_bs16_q6k_down", lambda: dict(us=moe_tail_workload(qk, 16, qk.Q6_K, 4, 200, 20)))
+    for b in (1, 16):   # the full-attention mixer's decode step at 4096 cached positions
+        def attn(b=b):
+            at = attn_workload(qk, b, 4096, 200, 20)
+            return rate(at["bytes_step"], at["ms_event"], ring=at["ring"])
+        run(f"attn_decode_ctx4096_bs{b}", attn)
+
+    def attn_prefill():   # the attention mixer over a 1,024-position prompt
+        p = attn_prefill_workload(qk, 1024, 40, 8)
+        return dict(us=p["ms_event"] * 1e3, tflops=p["flops"] / (p["ms_event"] * 1e-3) / 1e12, steps_timed=p["steps"])
+    run("attn_prefill_1024_positions", attn_prefill)
+    for b in (1, 16):   # the gated-DeltaNet mixer's decode step
+        def dn(b=b):
+            d = deltanet_workload(qk, b, 256, 32)
+            return rate(d["bytes_step"], d["ms_event"], ring=d["ring"])
+        run(f"deltanet_decode_bs{b}", dn)
+    run("engine_decode_8_layers", lambda: engine_workload(qk, 8, (1, 4, 16), 8, 2))
+    # a whole model: three gated-DeltaNet layers and one full-attention layer, twice (positions 1..320)
+    run("engine_decode_whole_model_8_layers", lambda: engine_workload(qk, 8, (1, 16), 8, 2, kinds="RRRARRRA"))
+    return ex
+
+
+def extras_in_child(a, timeout_s=1500):
+    """Runs `--workload extras` in a child process and returns its object: the headline figure of this
+    process is already measured, and whatever happens to a side measurement -- a Python error is an
+    entry of the object, a process that dies or stalls is an error here -- the line still goes out."""
+    import subprocess
+    cmd = [sys.executable, os.path.abspath(__file__), "--workload", "extras", "--no-cpu", "--ring", str(a.ring),
+           "--steps", str(a.steps), "--warmup", str(a.warmup)]
+    try:
+        r = subprocess.run(cmd, stdout=subprocess.PIPE, text=True, timeout=timeout_s)   # its stderr is this process's
+        if r.returncode != 0:
+            return dict(error=f"the extras process ended with status {r.returncode}")
+        return json.loads(r.stdout.strip().splitlines()[-1])["extras"]
+    except Exception as e:   # noqa: BLE001
+        return dict(error=f"{type(e).__name__}: {e}")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -618,106 +744,79 @@ def main():
         return
     if a.workload == "gemv_sustained":   # every block format at a sustained size and at the 8192 x 2048 shape
         res = {}
-        def sustained(t):
-            Ms = -(-(256 << 20) // qk.row_bytes(t, 2048) // 64) * 64
-            g = gemv_workload(qk, t, Ms, 2048, 1, 40, 4, ring=2)
-            gb = g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9
-            return dict(rows=Ms, us=g["ms_event"] * 1e3, gbps=gb, frac=gb / HBM_PEAK_GBPS, steps_timed=g["steps"])
-        for name, t in (("q8_0", qk.Q8_0), ("q6_k", qk.Q6_K), ("iq4_xs", qk.IQ4_XS), ("iq3_xxs", qk.IQ3_XXS)):
-            guarded(ex, f"gemv_{name}_sustained_256MiB", lambda t=t: sustained(t))
+        for name, t in (("q8_0", qk.Q8_0), ("q6_k", qk.Q6_K), ("iq4_xs", qk.IQ4_XS), ("iq3_xxs", qk.IQ3_XXS), ("f16", qk.F16)):
+            guarded(res, f"gemv_{name}_sustained_256MiB", lambda t=t: gemv_entry(qk, t, None, 2048, 1, 40, 4))
             torch.cuda.empty_cache()
-        # the other dense projections of a decode step at the reference's shapes (src/main.cpp:4310-4335)
-        for M, K in ((4096, 2048), (2048, 4096), (512, 2048)):
-            for b in (1, 16):
-                g = gemv_workload(qk, qk.Q8_0, M, K, b, es, ew)
-                key = f"gemv_q8_0_{M}x{K}" + ("_bs16" if b > 1 else "")
-                ex[key] = dict(us=g["ms_event"] * 1e3, gbps=g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9,
-                               frac=g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9 / HBM_PEAK_GBPS)
-                log(f"[bench] {key}: {ex[key]}")
-                torch.cuda.empty_cache()
-        for b in (1, 16):
-            h = head_workload(qk, 151936, 2048, b, 40, 8)
-            ex[f"head_q6k_151936_bs{b}"] = dict(us=h["ms_event"] * 1e3, gbps=h["bytes_step"] / (h["ms_event"] * 1e-3) / 1e9,
-                                                frac=h["bytes_step"] / (h["ms_event"] * 1e-3) / 1e9 / HBM_PEAK_GBPS)
-            log(f"[bench] head bs{b}: {ex[f'head_q6k_151936_bs{b}']}")
+            guarded(res, f"gemv_{name}_8192x2048", lambda t=t: gemv_entry(qk, t, 8192, 2048, 1, 400, 40))
             torch.cuda.empty_cache()
-        if a.workload == "moe_decode_bs1":
-            # the same step on ONE layer replayed: its 16 MB stay in the caches, so this is the step without
-            # HBM in the way (launch, selection and dependency chain) beside the ring's figure above
-            def cache_hot():
-                mh = moe_workload(qk, 1, qk.IQ4_XS, 1, 400, 40)
-                return dict(us=mh["ms_event"] * 1e3, steps_timed=mh["steps"], stage_us={k: v * 1e3 for k, v in mh["stage_ms"].items()})
-            guarded(ex, "moe_decode_bs1_cache_hot", cache_hot)
-            torch.cuda.empty_cache()
+        first = res["gemv_q8_0_sustained_256MiB"]
+        print(json.dumps(dict(metric="gemv_hbm_gbps", value=first.get("gbps"), unit="GB/s", n_gpus=1,
+                              higher_is_better=True, data="synthetic", dtype="f32",
+                              config=dict(workload="gemv_sustained", K=2048, env=qk_env()),
+                              detail=res)), flush=True)
+        return
+    if a.workload in ("head_bs1", "head_bs16"):   # the LM head alone (for counter runs on its kernel)
+        b = 1 if a.workload == "head_bs1" else 16
+        h = head_workload(qk, 151936, 2048, b, min(a.steps, 40), min(a.warmup, 8))
+        gb = h["bytes_step"] / (h["ms_event"] * 1e-3) / 1e9
+        print(json.dumps(dict(metric="lm_head_argmax_hbm_gbps", value=gb, unit="GB/s", n_gpus=1, steps=h["steps"],
+                              ms_per_step=h["ms_event"], higher_is_better=True, data="synthetic", dtype="f32",
+                              config=dict(workload=a.workload, vocab=151936, n_embd=2048, weights="Q6_K", rows=b),
+                              bytes_per_step=h["bytes_step"], frac_of_hbm_peak=gb / HBM_PEAK_GBPS)), flush=True)
+        return
+    if a.workload == "prefill_gemm":   # the Q8_0 prefill GEMM alone (for counter runs on its kernel)
+        res = {}
+        guarded(res, "prefill_gemm_q8_0_8192x2048x128", lambda: gemm_entry(qk))
+        print(json.dumps(dict(metric="prefill_gemm_tflops", value=res["prefill_gemm_q8_0_8192x2048x128"].get("tflops"),
+                              unit="TFLOP/s", n_gpus=1, higher_is_better=True, data="synthetic", dtype="f16",
+                              config=dict(workload=a.workload, M=8192, K=2048, N=128, weights="Q8_0"), detail=res)), flush=True)
+        return
+    if a.workload == "extras":   # the other BASELINE configs and the rows beside the path, as one JSON object
+        print(json.dumps(dict(extras=extras(qk, a, steps))), flush=True)
+        return
+    if a.workload == "moe_decode_bs1":
+        m = moe_workload(qk, 1, qk.IQ4_XS, a.ring, steps, a.warmup)
+    elif a.workload == "moe_decode_bs16":
+        m = moe_workload(qk, 16, qk.Q6_K, min(a.ring, 8), steps, a.warmup)
+    elif a.workload == "moe_prefill_128":
+        m = moe_workload(qk, 128, qk.IQ4_XS, min(a.ring, 4), min(steps, 400), min(a.warmup, 40))
+    else:
+        sys.exit(f"unknown workload {a.workload}")
+    log(f"[bench] {a.workload}: {m['ms_wall'] * 1e3:.2f} us/step wall, {m['ms_event'] * 1e3:.2f} us/step events, "
+        f"stages {m['stage_ms']}")
+    gbps = m["bytes_step"] / (m["ms_wall"] * 1e-3) / 1e9
+    # dominant kernel = the routed gate/up launch (most bytes of the step); its average launch
+    # duration is measured live with HIP events on the launch stream over a replay of that
+    # stage alone on the same ring (profiles/ holds the rocprofv3 figure for the same kernel)
+    gu_ms = m["stage_ms"]["gateup"]
+    ach = m["gateup_bytes"] / (gu_ms * 1e-3) / 1e9
+    kname, kwhat = {"moe_decode_bs1": ("moe_gateup_kernel", "select + routed IQ3_XXS gate/up + SiLU"),
+                    "moe_decode_bs16": ("moe_gateup_fused_kernel", "routed IQ3_XXS + shared Q8_0 gate/up + SiLU"),
+                    "moe_prefill_128": ("moe_gateup_mfma_kernel", "routed IQ3_XXS gate/up + SiLU; the stage time also "
+                                        "covers the shared expert's launch on the side stream")}[a.workload]
+    roof = dict(bound="hbm", kernel=f"{kname} ({kwhat})", achieved=ach,
+                peak=HBM_PEAK_GBPS, unit="GB/s", frac=ach / HBM_PEAK_GBPS, traffic=TRAFFIC.get(kname),
+                bytes_per_launch=m["gateup_bytes"], us_per_launch=gu_ms * 1e3)
+    out = dict(metric="fused_moe_decode_step_hbm_gbps", value=gbps, unit="GB/s", n_gpus=1, steps=a.steps,
+               warmup=a.warmup, ms_per_step=m["ms_wall"], higher_is_better=True, scaling="weak", vs_baseline=None,
+               dtype="f32", data="synthetic",
+               config=dict(workload=a.workload, n_embd=2048, n_ff=512, n_expert=256, n_used=8,
+                           gate_up="IQ3_XXS", down="Q6_K" if a.workload.endswith("bs16") else "IQ4_XS",
+                           shared="Q8_0", slots={"moe_decode_bs1": 1, "moe_decode_bs16": 16}.get(a.workload, 128),
+                           ring_layers=m["ring"], ring_bytes=m["ring_bytes"],
+                           steps_timed=m["steps"], graph_replays_timed=m["steps"] // m["ring"],
+                           timing=f"hipGraph replays of the ring (one launch set per layer of the ring), at least "
+                                  f"{MIN_REPLAYS} replays whatever --steps asks; value from the host clock over all of them, "
+                                  f"us_per_step_events the median replay by HIP events", env=qk_env()),
+               us_per_step=m["ms_wall"] * 1e3, us_per_step_events=m["ms_event"] * 1e3,
+               bytes_per_step=m["bytes_step"], frac_of_hbm_peak=gbps / HBM_PEAK_GBPS,
+               distinct_experts_per_step=m["distinct_experts"],
+               three_launch_stage_us={k: v * 1e3 for k, v in m["stage_ms"].items()}, roofline=roof, device=info)
+    del m
+    torch.cuda.empty_cache()
 
-            # the ring's tensors carved from one allocation: what the many separate mappings cost, if anything
-            def one_allocation():
-                ms = moe_workload(qk, 1, qk.IQ4_XS, a.ring, min(steps, 800), a.warmup, slab=True)
-                return dict(us=ms["ms_event"] * 1e3, steps_timed=ms["steps"], stage_us={k: v * 1e3 for k, v in ms["stage_ms"].items()})
-            guarded(ex, "moe_decode_bs1_ring_in_one_allocation", one_allocation)
-            torch.cuda.empty_cache()
-            m16 = moe_workload(qk, 16, qk.Q6_K, 4, 200, 20)
-            ex["moe_decode_bs16_q6k_down"] = dict(us=m16["ms_event"] * 1e3, distinct_experts=m16["distinct_experts"],
-                                                  gbps=m16["bytes_step"] / (m16["ms_event"] * 1e-3) / 1e9,
-                                                  frac=m16["bytes_step"] / (m16["ms_event"] * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-                                                  stage_us={k: v * 1e3 for k, v in m16["stage_ms"].items()})
-            log(f"[bench] moe bs16: {ex['moe_decode_bs16_q6k_down']}")
-            torch.cuda.empty_cache()
-            # a few concurrent slots: every row through the one-row launches (grid.y = row)
-            ex["moe_decode_few_rows_q6k_down_us"] = {}
-            for nr in (2, 4, 8):
-                mf = moe_workload(qk, nr, qk.Q6_K, 8, 400, 40)
-                ex["moe_decode_few_rows_q6k_down_us"][f"rows_{nr}"] = mf["ms_event"] * 1e3
-                torch.cuda.empty_cache()
-            log(f"[bench] moe few rows: {ex['moe_decode_few_rows_q6k_down_us']}")
-            # layer glue (add + RMS norm alone, and behind the step in one call)
-            ex["add_rmsnorm_2048"] = dict(us_1_row=norm_workload(qk, 1, 640, 64), us_16_rows=norm_workload(qk, 16, 640, 64))
-            ex["moe_decode_tail_bs1"] = dict(us=moe_tail_workload(qk, 1, qk.IQ4_XS, 8, 400, 40))
-            ex["moe_layer_row_bs1"] = dict(us=moe_tail_workload(qk, 1, qk.IQ4_XS, 8, 400, 40, layer_row=True))
-            torch.cuda.empty_cache()
-            ex["moe_decode_tail_bs16_q6k_down"] = dict(us=moe_tail_workload(qk, 16, qk.Q6_K, 4, 200, 20))
-            log(f"[bench] glue: {ex['add_rmsnorm_2048']} tail bs1 {ex['moe_decode_tail_bs1']} "
-                f"bs16 {ex['moe_decode_tail_bs16_q6k_down']}")
-            torch.cuda.empty_cache()
-            g = gemm_workload(qk, 8192, 2048, 128, 200, 20)
-            ex["prefill_gemm_q8_0_8192x2048x128"] = dict(us=g["ms_event"] * 1e3, tflops=g["flops"] / (g["ms_event"] * 1e-3) / 1e12,
-                                                         frac_mfma_peak=g["flops"] / (g["ms_event"] * 1e-3) / 2.5e15,
-                                                         gbps=g["bytes_step"] / (g["ms_event"] * 1e-3) / 1e9)
-            log(f"[bench] prefill gemm: {ex['prefill_gemm_q8_0_8192x2048x128']}")
-            torch.cuda.empty_cache()
-            pm = prefill_moe_workload(qk, 128, 20, 4)
-            ex["prefill_moe_128_tokens"] = dict(us=pm["ms_event"] * 1e3, tok_per_s=128 / (pm["ms_event"] * 1e-3),
-                                                distinct_experts=pm["distinct_experts"],
-                                                gbps=pm["bytes_step"] / (pm["ms_event"] * 1e-3) / 1e9,
-                                                frac=pm["bytes_step"] / (pm["ms_event"] * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-                                                tflops=pm["flops"] / (pm["ms_event"] * 1e-3) / 1e12)
-            log(f"[bench] prefill moe: {ex['prefill_moe_128_tokens']}")
-            torch.cuda.empty_cache()
-            for b in (1, 16):   # the full-attention mixer's decode step at 4096 cached positions
-                at = attn_workload(qk, b, 4096, 200, 20)
-                gb = at["bytes_step"] / (at["ms_event"] * 1e-3) / 1e9
-                ex[f"attn_decode_ctx4096_bs{b}"] = dict(us=at["ms_event"] * 1e3, gbps=gb, frac=gb / HBM_PEAK_GBPS,
-                                                        ring=at["ring"])
-                torch.cuda.empty_cache()
-            log(f"[bench] attention: {ex['attn_decode_ctx4096_bs1']} {ex['attn_decode_ctx4096_bs16']}")
-            def attn_prefill():   # the attention mixer over a 1,024-position prompt
-                ap = attn_prefill_workload(qk, 1024, 40, 8)
-                return dict(us=ap["ms_event"] * 1e3, tflops=ap["flops"] / (ap["ms_event"] * 1e-3) / 1e12, steps_timed=ap["steps"])
-            guarded(ex, "attn_prefill_1024_positions", attn_prefill)
-            torch.cuda.empty_cache()
-            for b in (1, 16):   # the gated-DeltaNet mixer's decode step
-                dn = deltanet_workload(qk, b, 256, 32)
-                gb = dn["bytes_step"] / (dn["ms_event"] * 1e-3) / 1e9
-                ex[f"deltanet_decode_bs{b}"] = dict(us=dn["ms_event"] * 1e3, gbps=gb, frac=gb / HBM_PEAK_GBPS, ring=dn["ring"])
-                torch.cuda.empty_cache()
-            log(f"[bench] deltanet: {ex['deltanet_decode_bs1']} {ex['deltanet_decode_bs16']}")
-            ex["engine_decode_8_layers"] = engine_workload(qk, 8, (1, 4, 16), 8, 2)
-            log(f"[bench] engine: {ex['engine_decode_8_layers']}")
-            # a whole model: three gated-DeltaNet layers and one full-attention layer, twice (positions 1..320)
-            ex["engine_decode_whole_model_8_layers"] = engine_workload(qk, 8, (1, 16), 8, 2, kinds="RRRARRRA")
-            log(f"[bench] engine, whole model: {ex['engine_decode_whole_model_8_layers']}")
-        out["extras"] = ex
-
+    if a.extras and a.workload == "moe_decode_bs1":
+        out["extras"] = extras_in_child(a)
     if a.cpu:
         guarded(out, "cpu_baseline", lambda: cpu_baseline(qk, entry.load_oracle()))
     print(json.dumps(out), flush=True)

@@ -31,3 +31,125 @@ def test_cpu_baseline_line(qk, orc):
     assert per["C2_moe_decode_bs1"]["bytes"] == 16326656      # the weights one step touches: router, shared gate, 8 experts, shared expert
     assert per["C1_gemv_q8_0_8192x2048"]["bytes"] == 17866752
     assert per["C4_lm_head_q6k_151936_bs1"]["bytes"] == 255252480 + 8192
+
+
+def test_no_function_of_bench_reads_a_name_nothing_binds():
+    """Every name a function of bench.py takes from the module's namespace exists there (or is a
+    builtin): a block that lost the statement that bound its variables cannot come back unnoticed."""
+    import builtins
+    import symtable
+    sys.path.insert(0, ROOT)
+    import bench
+    src = open(os.path.join(ROOT, "bench.py")).read()
+    missing = []
+
+    def walk(tab):
+        for s in tab.get_symbols():
+            if s.is_global() and s.is_referenced() and not hasattr(bench, s.get_name()) and not hasattr(builtins, s.get_name()):
+                missing.append((tab.get_name(), s.get_name()))
+        for c in tab.get_children():
+            walk(c)
+    walk(symtable.symtable(src, "bench.py", "exec"))
+    assert not missing, missing
+
+
+class _FakeCuda:
+    @staticmethod
+    def is_available():
+        return True
+
+    @staticmethod
+    def empty_cache():
+        pass
+
+
+def _bench_with_stub_workloads(monkeypatch, qk):
+    """bench with every GPU workload replaced by a stub of the same signature and result keys, so main()
+    runs from the arguments to the JSON line on the CPU."""
+    sys.path.insert(0, ROOT)
+    import bench
+    import torch
+    monkeypatch.setattr(torch, "cuda", _FakeCuda)
+    monkeypatch.setattr(qk, "lib", lambda: None)
+    monkeypatch.setattr(qk, "device_info", lambda: dict(name="stub"))
+    stage = dict(route=0.004, gateup=0.009, down=0.007)
+    monkeypatch.setattr(bench, "moe_workload", lambda qk_, n, down, ring, steps, warmup, seed=1234, slab=False: dict(
+        ms_wall=0.021, ms_event=0.0205, steps=max(20 * ring, steps), bytes_step=16343200, distinct_experts=8.0, stage_ms=dict(stage),
+        gateup_bytes=6449152, ring=ring, ring_bytes=ring * 351000000))
+    monkeypatch.setattr(bench, "moe_tail_workload", lambda *a, **k: 22.0)
+    monkeypatch.setattr(bench, "norm_workload", lambda *a, **k: 2.1)
+    monkeypatch.setattr(bench, "gemv_workload", lambda qk_, t, M, K, batch, steps, warmup, seed=99, ring=None: dict(
+        ms_wall=0.007, ms_event=0.0068, steps=steps, bytes_step=M * qk.row_bytes(t, K) + batch * (K + M) * 4, ring=ring or 16))
+    monkeypatch.setattr(bench, "head_workload", lambda qk_, V, K, batch, steps, warmup, seed=77: dict(
+        ms_wall=0.06, ms_event=0.059, steps=steps, bytes_step=V * 1680 + batch * (K * 4 + 4), ring=2))
+    monkeypatch.setattr(bench, "gemm_workload", lambda qk_, M, K, N, steps, warmup, seed=55: dict(
+        ms_event=0.032, flops=2.0 * M * K * N, bytes_step=M * K // 32 * 34 + N * (K + M) * 4))
+    monkeypatch.setattr(bench, "prefill_moe_workload", lambda qk_, n, steps, warmup, seed=4242: dict(
+        ms_event=0.21, distinct_experts=251.0, bytes_step=342e6, flops=6.4e9))
+    monkeypatch.setattr(bench, "attn_workload", lambda qk_, b, ctx, steps, warmup, **k: dict(ms_event=0.05, bytes_step=b * 16777216, ring=4))
+    monkeypatch.setattr(bench, "attn_prefill_workload", lambda qk_, n, steps, warmup, **k: dict(ms_event=0.9, flops=1e12, steps=steps))
+    monkeypatch.setattr(bench, "deltanet_workload", lambda qk_, b, steps, warmup, **k: dict(ms_event=0.02, bytes_step=b * 4194304, ring=8))
+    monkeypatch.setattr(bench, "engine_workload", lambda *a, **k: dict(config=dict(layers=8), slots_1=dict(tok_per_s=1.0, prefill_tok_per_s=1.0),
+                                                                      slots_16=dict(tok_per_s=2.0)))
+    monkeypatch.setattr(bench, "cpu_baseline", lambda qk_, orc_: dict(value=0.5, unit="GB/s", cores=8, kind="port", sample="stub", per_config={}))
+    # the side measurements run in a child process; here in this one, on the stubs
+    monkeypatch.setattr(bench, "extras_in_child", lambda a: bench.extras(qk, a, max(a.ring, a.steps // a.ring * a.ring)))
+    return bench
+
+
+def _one_json_line(capsys):
+    lines = [ln for ln in capsys.readouterr().out.splitlines() if ln.strip()]
+    assert len(lines) == 1, lines
+    return json.loads(lines[0])
+
+
+def test_default_run_prints_the_headline_line(monkeypatch, capsys, qk):
+    """The driver's command line, from the arguments to the one JSON line, on stub workloads: the keys the
+    contract names, the roofline and CPU objects, and an entry per BASELINE config among the extras."""
+    bench = _bench_with_stub_workloads(monkeypatch, qk)
+    monkeypatch.setattr(sys, "argv", ["bench.py", "--gpus", "1", "--steps", "20", "--warmup", "5"])
+    bench.main()
+    out = _one_json_line(capsys)
+    for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling", "vs_baseline",
+              "dtype", "data", "config", "roofline", "cpu_baseline", "extras"):
+        assert k in out, k
+    assert out["steps"] == 20 and out["warmup"] == 5 and out["n_gpus"] == 1 and out["vs_baseline"] is None
+    assert out["config"]["workload"] == "moe_decode_bs1" and out["config"]["steps_timed"] >= 20 * out["config"]["ring_layers"]
+    r = out["roofline"]
+    assert r["bound"] == "hbm" and r["peak"] == 8000.0 and abs(r["frac"] - r["achieved"] / r["peak"]) < 1e-12
+    assert abs(r["achieved"] - r["bytes_per_launch"] / r["us_per_launch"] / 1e3) < 1e-6 * r["achieved"] and "traffic" in r
+    assert out["cpu_baseline"]["kind"] == "port"
+    ex = out["extras"]
+    for k in ("gemv_q8_0_8192x2048", "gemv_q6_k_8192x2048", "gemv_iq4_xs_8192x2048", "gemv_iq3_xxs_8192x2048", "gemv_f16_8192x2048",
+              "gemv_q8_0_sustained_256MiB", "gemv_iq3_xxs_sustained_256MiB", "head_q6k_151936_bs1", "head_q6k_151936_bs16",
+              "moe_decode_bs16_q6k_down", "prefill_gemm_q8_0_8192x2048x128", "prefill_moe_128_tokens", "moe_decode_bs1_cache_hot",
+              "moe_decode_bs1_ring_in_one_allocation"):
+        assert k in ex and "error" not in ex[k], (k, ex.get(k))
+    assert ex["gemv_q8_0_8192x2048"]["gbps"] > 0 and ex["prefill_gemm_q8_0_8192x2048x128"]["frac_mfma_peak"] > 0
+
+
+def test_other_workloads_print_one_line_each(monkeypatch, capsys, qk):
+    bench = _bench_with_stub_workloads(monkeypatch, qk)
+    for wl, metric in (("gemv_sustained", "gemv_hbm_gbps"), ("head_bs1", "lm_head_argmax_hbm_gbps"), ("head_bs16", "lm_head_argmax_hbm_gbps"),
+                       ("moe_decode_bs16", "fused_moe_decode_step_hbm_gbps"), ("moe_prefill_128", "fused_moe_decode_step_hbm_gbps"),
+                       ("prefill_gemm", "prefill_gemm_tflops"), ("engine_decode", "engine_decode_tok_per_s")):
+        monkeypatch.setattr(sys, "argv", ["bench.py", "--workload", wl, "--no-cpu", "--no-extras"])
+        bench.main()
+        out = _one_json_line(capsys)
+        assert out["metric"] == metric and out["config"]["workload"] == wl and out["value"] > 0, wl
+    monkeypatch.setattr(sys, "argv", ["bench.py", "--workload", "extras", "--no-cpu"])
+    bench.main()
+    assert "gemv_q8_0_8192x2048" in _one_json_line(capsys)["extras"]
+
+
+def test_a_failing_side_measurement_is_an_entry_of_the_line(monkeypatch, capsys, qk):
+    bench = _bench_with_stub_workloads(monkeypatch, qk)
+
+    def broken(*a, **k):
+        raise RuntimeError("no such kernel")
+    monkeypatch.setattr(bench, "head_workload", broken)
+    monkeypatch.setattr(sys, "argv", ["bench.py", "--steps", "20", "--warmup", "5", "--no-cpu"])
+    bench.main()
+    out = _one_json_line(capsys)
+    assert out["value"] > 0 and "no such kernel" in out["extras"]["head_q6k_151936_bs1"]["error"]
+    assert "error" not in out["extras"]["gemv_q8_0_8192x2048"]
