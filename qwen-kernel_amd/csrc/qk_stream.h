@@ -53,10 +53,16 @@ struct WaveStage {
     __device__ __forceinline__ void commit(uint8_t* lds, int lane) const
     {
         u32x4_a* p = (u32x4_a*)lds;
+        // wavefront-scope fences emit no instruction; they keep the compiler from moving the other
+        // lanes' field reads across the stores (the barrier intrinsic alone orders execution, not memory)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
         for (int j = 0; j < NP; j++) p[lane + 64 * j] = r[j];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
 };
 
