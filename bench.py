@@ -544,6 +544,11 @@ def qk_env():
     return {k: v for k, v in os.environ.items() if k.startswith("QK_")}
 
 
+def kernel_forms(qk):
+    """The library's switches as they stand (which form of each kernel the figures belong to)."""
+    return {n: qk.get_option(n) for n in ("one_row", "dense_reg", "fused_norm", "attn_block", "dn_fused")}
+
+
 def rate(bytes_step, ms, **more):
     gb = bytes_step / (ms * 1e-3) / 1e9
     return dict(us=ms * 1e3, gbps=gb, frac=gb / HBM_PEAK_GBPS, **more)
@@ -586,11 +591,11 @@ def extras(qk, a, steps):
             run(f"gemv_{name}_8192x2048_bs16", lambda t=t: gemv_entry(qk, t, 8192, 2048, 16, es, ew))
     for name, t in fmts:
         run(f"gemv_{name}_sustained_256MiB", lambda t=t: gemv_entry(qk, t, None, 2048, 1, 40, 4))
+    def head(b):
+        h = head_workload(qk, 151936, 2048, b, 40, 8)
+        return rate(h["bytes_step"], h["ms_event"], steps_timed=h["steps"])
     for b in (1, 16):   # C4
-        def head(b=b):
-            h = head_workload(qk, 151936, 2048, b, 40, 8)
-            return rate(h["bytes_step"], h["ms_event"], steps_timed=h["steps"])
-        run(f"head_q6k_151936_bs{b}", head)
+        run(f"head_q6k_151936_bs{b}", lambda b=b: head(b))
 
     def stages(m, **more):
         return dict(us=m["ms_event"] * 1e3, steps_timed=m["steps"], stage_us={k: v * 1e3 for k, v in m["stage_ms"].items()}, **more)
@@ -642,6 +647,18 @@ def extras(qk, a, steps):
             d = deltanet_workload(qk, b, 256, 32)
             return rate(d["bytes_step"], d["ms_event"], ring=d["ring"])
         run(f"deltanet_decode_bs{b}", dn)
+    if a.ab_forms:
+        # both forms of the one-row kernels side by side: block fields loaded per lane (the default) against rows
+        # streamed through LDS; the C1 shapes, the sustained size, the head and the bs = 1 step with its stages
+        for form, on in (("lane", 0), ("stream", 1)):
+            with qk.option("one_row", on), qk.option("dense_reg", on):
+                for name, t in fmts:
+                    run(f"{form}:gemv_{name}_8192x2048", lambda t=t: gemv_entry(qk, t, 8192, 2048, 1, es, ew))
+                    run(f"{form}:gemv_{name}_sustained_256MiB", lambda t=t: gemv_entry(qk, t, None, 2048, 1, 40, 4))
+                run(f"{form}:head_q6k_151936_bs1", lambda: head(1))
+                run(f"{form}:moe_decode_bs1", lambda: stages(moe_workload(qk, 1, qk.IQ4_XS, a.ring, min(steps, 800), a.warmup)))
+                run(f"{form}:moe_decode_bs1_cache_hot", lambda: stages(moe_workload(qk, 1, qk.IQ4_XS, 1, 400, 40)))
+                run(f"{form}:moe_decode_4_rows_q6k_down", lambda: dict(us=moe_workload(qk, 4, qk.Q6_K, 8, 400, 40)["ms_event"] * 1e3))
     run("engine_decode_8_layers", lambda: engine_workload(qk, 8, (1, 4, 16), 8, 2))
     # a whole model: three gated-DeltaNet layers and one full-attention layer, twice (positions 1..320)
     run("engine_decode_whole_model_8_layers", lambda: engine_workload(qk, 8, (1, 16), 8, 2, kinds="RRRARRRA"))
@@ -654,7 +671,7 @@ def extras_in_child(a, timeout_s=1500):
     entry of the object, a process that dies or stalls is an error here -- the line still goes out."""
     import subprocess
     cmd = [sys.executable, os.path.abspath(__file__), "--workload", "extras", "--no-cpu", "--ring", str(a.ring),
-           "--steps", str(a.steps), "--warmup", str(a.warmup)]
+           "--steps", str(a.steps), "--warmup", str(a.warmup)] + (["--ab-forms"] if a.ab_forms else [])
     try:
         r = subprocess.run(cmd, stdout=subprocess.PIPE, text=True, timeout=timeout_s)   # its stderr is this process's
         if r.returncode != 0:
@@ -677,6 +694,8 @@ def main():
                     help="layers of the synthetic model of the engine workloads (40 = the reference model's depth, a 16 GB file)")
     ap.add_argument("--extras", dest="extras", action="store_true", default=True)
     ap.add_argument("--no-extras", dest="extras", action="store_false")
+    ap.add_argument("--ab-forms", action="store_true",
+                    help="extras: also time the one-row kernels in both forms (per-lane loads / rows streamed through LDS)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain 256 MiB device copy (calibrates FETCH_SIZE/WRITE_SIZE counter runs)")
     ap.add_argument("--cpu", dest="cpu", action="store_true", default=True)
@@ -807,7 +826,7 @@ def main():
                            steps_timed=m["steps"], graph_replays_timed=m["steps"] // m["ring"],
                            timing=f"hipGraph replays of the ring (one launch set per layer of the ring), at least "
                                   f"{MIN_REPLAYS} replays whatever --steps asks; value from the host clock over all of them, "
-                                  f"us_per_step_events the median replay by HIP events", env=qk_env()),
+                                  f"us_per_step_events the median replay by HIP events", env=qk_env(), kernel_forms=kernel_forms(qk)),
                us_per_step=m["ms_wall"] * 1e3, us_per_step_events=m["ms_event"] * 1e3,
                bytes_per_step=m["bytes_step"], frac_of_hbm_peak=gbps / HBM_PEAK_GBPS,
                distinct_experts_per_step=m["distinct_experts"],

@@ -82,6 +82,22 @@ const char *qkk_last_error(void);
  * arch_host (e.g. "gfx950") when non-NULL. Never fails. */
 int qkk_device_info(char *arch_host, size_t arch_len, uint32_t *n_cu_host);
 
+/* Switches between two forms of the same operator (no counterpart in the reference, whose pipelines
+ * are chosen when they are built: reference src/main.cpp:3630-3760).  Each is read once from the
+ * environment variable QK_<NAME> on first use; qkk_set_option changes it for the calling process
+ * (launches already captured in a graph keep the form they were captured with).  Names and values:
+ *   "one_row"     0 (env "lane", the default): the one-row GEMV, MoE step and LM head load block
+ *                 fields per lane; 1 (env "stream"): they stream rows as 16-byte pieces through LDS
+ *   "dense_reg"   1: the F16 / F32 GEMV keeps its share of x in registers
+ *   "fused_norm"  1: the engine's one-row step folds each RMS norm into its consumer
+ *   "attn_block"  1: prefill attention over blocks of 16 rows on the matrix cores
+ *   "dn_fused"    1: the gated-DeltaNet decode step as one launch
+ *   "gemv_depth", "head_depth", "rowwise_max": launch-shape sweeps, 0 = built-in value
+ * The default of every switch is the form that has been run and timed on a device.
+ * Returns QKK_EINVAL for an unknown name or a value outside the switch's range. */
+int qkk_set_option(const char *name_host, int value);
+int qkk_get_option(const char *name_host, int *value_host);
+
 /* Bytes of one row of k elements of `type`; 0 if unsupported (reference src/gguf.h:36-46). */
 size_t qkk_row_bytes(int type, uint64_t k);
 

@@ -13,6 +13,7 @@ from .capi import (  # noqa: F401
     rmsnorm, add_rmsnorm, add_rms3, vec_add, embed, moe_decode_tail, moe_layer_rows, ROWWISE_MAX,
     rope_table, attn_prep, attn_workspace_bytes, attn_decode, dn_ab, dn_conv, dn_step, dn_ab_conv,
     moe_decode_static, moe_workspace_status, gemv_norm, head_argmax_norm, dn_step_fused, MOE_STATIC_MAX_SLOTS, MOE_STATIC_BYTES,
+    set_option, get_option, option,
 )
 from . import capi  # noqa: F401
 from . import synth  # noqa: F401

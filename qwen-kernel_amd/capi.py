@@ -49,6 +49,8 @@ def _signatures():
         "qkk_head_workspace_bytes": (sz, [u32, u32]),
         "qkk_attn_workspace_bytes": (sz, [u32, u32, u32]),
         "qkk_device_info": (None, [C.c_char_p, sz, C.POINTER(u32)]),
+        "qkk_set_option": (None, [C.c_char_p, i32]),
+        "qkk_get_option": (None, [C.c_char_p, C.POINTER(i32)]),
         "qkk_dequant": (None, [i32, vp, vp, u64, vp]),
         "qkk_gemv": (None, [i32, vp, vp, vp, u32, u32, u32, vp]),
         "qkk_gemv_norm": (None, [i32, vp, vp, vp, f32, vp, u32, u32, u32, vp]),
@@ -115,6 +117,33 @@ def _check(rc):
     if rc < 0:
         raise QkError(rc, lib().qkk_last_error().decode())
     return rc
+
+
+def set_option(name, value):
+    """Sets one switch of the library (include/qk_kernels.h lists them), e.g. set_option("one_row", 1)."""
+    _check(lib().qkk_set_option(name.encode(), int(value)))
+
+
+def get_option(name):
+    v = C.c_int32(0)
+    _check(lib().qkk_get_option(name.encode(), C.byref(v)))
+    return v.value
+
+
+class option:
+    """with option("one_row", 1): ...  -- a switch set for the block, its previous value afterwards."""
+
+    def __init__(self, name, value):
+        self.name, self.value = name, value
+
+    def __enter__(self):
+        self.old = get_option(self.name)
+        set_option(self.name, self.value)
+        return self
+
+    def __exit__(self, *exc):
+        set_option(self.name, self.old)
+        return False
 
 
 def _ptr(t):

@@ -763,10 +763,9 @@ static int attn_decode_impl(const char* who, const float* qhat, const float* k_c
     // measured 4.5 TB/s with 16 ranges, 4.2 with 32, 3.1 with 128 (the partial results are traffic too);
     // one slot 0.98 TB/s with 64 ranges, 0.80 with 32
     uint32_t n_ranges = std::min(max_ranges(rows), std::max(8u, persistent_blocks() / 2 / (rows * hKV)));
-    // three or more consecutive rows of one slot: blocks of sixteen rows (QK_ATTN_PAIR=1 keeps the pair kernel);
-    // one workgroup per CU (LDS), so about as many (block, KV head, range) triples as there are CUs
-    const bool pair_only = getenv("QK_ATTN_PAIR") != nullptr; // read per call: a test switches it between engines
-    const bool blocked = own == 0 && rows >= 3 && !pair_only;
+    // the "attn_block" switch: three or more consecutive rows of one slot go in blocks of sixteen rows instead of
+    // pairs; one workgroup per CU (LDS), so about as many (block, KV head, range) triples as there are CUs
+    const bool blocked = own == 0 && rows >= 3 && options().attn_block;
     const uint32_t blocks = (rows + BLK_Q - 1) / BLK_Q;
     const uint32_t hgroups = (hQ / hKV + 3) / 4; // four query heads of a KV head per workgroup
     if (blocked) n_ranges = std::min(max_ranges(rows), std::max(1u, persistent_blocks() / 4 / (blocks * hKV * hgroups)));

@@ -1,0 +1,459 @@
+// qk_cli.cpp -- `qk`, the operator test program over libqk.so.
+//
+// The reference's `qk` binary runs its kernels on synthetic tensors from the command line
+// (reference src/main.cpp:6952-6978): `qk suite`, `qk <format> [M] [K] [iters]`,
+// `qk bgemm [M K N iters]`, `qk moe [layer] [iters]`, one line per case with microseconds per
+// iteration, GB/s, GFLOP/s and the bytes moved (src/main.cpp:590-600), and a pass/fail verdict.
+// This program has the same modes over the operator ABI of include/qk_kernels.h:
+//
+//   qk suite                          the five GEMV formats at 8192 x 8192, 200 iterations
+//   qk f16|q8_0|q6_k|iq4_xs|iq3_xxs [M] [K] [iters]     defaults 16384 8192 100
+//   qk bgemm [M] [K] [N] [iters]      the Q8_0 prefill GEMM, defaults 8192 2048 256 40
+//   qk moe [seed] [iters] [slots] [experts]   one fused MoE layer (synthetic weights in place of a
+//                                     model's layer index), defaults 0 200 1 256
+//   qk head [batch] [iters]           the LM head 151936 x 2048 Q6_K with the argmax fused
+//
+// The weights are seeded random valid blocks (every bit pattern of the quant fields is valid; the
+// fp16 scales are |N(0,1)| * 1e-3), the activations N(0,1).  Iterations alternate over a ring of
+// tensors larger than the 256 MB last-level cache, timed with HIP events on the launch stream.
+// The verdict comes from a second computation on the device that shares no kernel with the first:
+// the bit-exact dequantisation kernel followed by the dense fp32 GEMV (1e-3 of the largest output,
+// the bar of the reference's own check, src/main.cpp:548-565); for `moe` the same rows through the
+// expert-major matrix-core path.  No CPU arithmetic takes part.
+#include <hip/hip_runtime.h>
+
+#include <math.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <algorithm>
+#include <string>
+#include <vector>
+
+#include "../../include/qk_kernels.h"
+
+namespace {
+
+constexpr double HBM_PEAK_GBPS = 8000.0, MFMA_F16_PEAK_TFLOPS = 2500.0;
+
+#define HIP_OK(call)                                                                                        \
+    do {                                                                                                    \
+        const hipError_t e_ = (call);                                                                       \
+        if (e_ != hipSuccess) {                                                                             \
+            fprintf(stderr, "qk: %s: %s\n", #call, hipGetErrorString(e_));                                  \
+            exit(2);                                                                                        \
+        }                                                                                                   \
+    } while (0)
+#define QK_OK(call)                                                                                         \
+    do {                                                                                                    \
+        const int rc_ = (call);                                                                             \
+        if (rc_ != QKK_OK) {                                                                                \
+            fprintf(stderr, "qk: %s: %d: %s\n", #call, rc_, qkk_last_error());                              \
+            exit(2);                                                                                        \
+        }                                                                                                   \
+    } while (0)
+
+// splitmix64: seeded, the same stream on every host
+struct Rng {
+    uint64_t s;
+    explicit Rng(uint64_t seed) : s(seed * 0x9E3779B97F4A7C15ull + 0x1234567ull) {}
+    uint64_t next()
+    {
+        uint64_t z = (s += 0x9E3779B97F4A7C15ull);
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        return z ^ (z >> 31);
+    }
+    double uniform() { return (double)(next() >> 11) * (1.0 / 9007199254740992.0); }
+    float normal() // Box-Muller
+    {
+        const double u = std::max(uniform(), 1e-300), v = uniform();
+        return (float)(sqrt(-2.0 * log(u)) * cos(6.283185307179586 * v));
+    }
+};
+
+// float -> IEEE half bits, round to nearest even; values here are far inside the normal range
+uint16_t half_bits(float f)
+{
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    const uint32_t sign = (x >> 16) & 0x8000u;
+    int32_t e = (int32_t)((x >> 23) & 0xFF) - 127 + 15;
+    uint32_t m = x & 0x7FFFFFu;
+    if (e <= 0) {
+        if (e < -10) return (uint16_t)sign;
+        m |= 0x800000u;
+        const int sh = 14 - e;
+        uint32_t r = m >> sh;
+        const uint32_t rem = m & ((1u << sh) - 1), halfway = 1u << (sh - 1);
+        if (rem > halfway || (rem == halfway && (r & 1))) r++;
+        return (uint16_t)(sign | r);
+    }
+    if (e >= 31) return (uint16_t)(sign | 0x7C00u);
+    uint32_t r = ((uint32_t)e << 10) | (m >> 13);
+    const uint32_t rem = m & 0x1FFFu;
+    if (rem > 0x1000u || (rem == 0x1000u && (r & 1))) r++;
+    return (uint16_t)(sign | r);
+}
+
+struct Format {
+    const char* name;
+    int type;
+    uint32_t block_elems, block_bytes, scale_offset; // where the block's fp16 scale lies
+};
+const Format FORMATS[] = {{"f16", QKK_F16, 1, 2, 0},          {"q8_0", QKK_Q8_0, 32, 34, 0},     {"q6_k", QKK_Q6_K, 256, 210, 208},
+                          {"iq4_xs", QKK_IQ4_XS, 256, 136, 0}, {"iq3_xxs", QKK_IQ3_XXS, 256, 98, 0}};
+
+const Format* format_named(const char* n)
+{
+    for (const Format& f : FORMATS)
+        if (!strcmp(f.name, n)) return &f;
+    return nullptr;
+}
+
+// n_elems weights of a format as seeded random valid blocks
+std::vector<uint8_t> random_tensor(const Format& f, uint64_t n_elems, uint64_t seed)
+{
+    Rng rng(seed);
+    if (f.type == QKK_F16) {
+        std::vector<uint8_t> out(n_elems * 2);
+        uint16_t* h = (uint16_t*)out.data();
+        for (uint64_t i = 0; i < n_elems; i++) h[i] = half_bits(rng.normal() * 0.05f);
+        return out;
+    }
+    const uint64_t blocks = n_elems / f.block_elems;
+    std::vector<uint8_t> out(blocks * f.block_bytes);
+    uint64_t* w = (uint64_t*)out.data();
+    for (uint64_t i = 0; i < out.size() / 8; i++) w[i] = rng.next();
+    for (uint64_t i = out.size() / 8 * 8; i < out.size(); i++) out[i] = (uint8_t)rng.next();
+    for (uint64_t b = 0; b < blocks; b++) {
+        const uint16_t d = half_bits(fabsf(rng.normal()) * 1e-3f);
+        memcpy(&out[b * f.block_bytes + f.scale_offset], &d, 2);
+    }
+    return out;
+}
+
+std::vector<float> random_rows(uint64_t n, uint64_t seed, float scale = 1.f)
+{
+    Rng rng(seed);
+    std::vector<float> v(n);
+    for (float& x : v) x = rng.normal() * scale;
+    return v;
+}
+
+template <class T>
+T* to_device(const std::vector<T>& h)
+{
+    T* d = nullptr;
+    HIP_OK(hipMalloc((void**)&d, std::max<size_t>(h.size() * sizeof(T), 16)));
+    HIP_OK(hipMemcpy(d, h.data(), h.size() * sizeof(T), hipMemcpyHostToDevice));
+    return d;
+}
+template <class T>
+T* device_zeros(size_t n)
+{
+    T* d = nullptr;
+    HIP_OK(hipMalloc((void**)&d, std::max<size_t>(n * sizeof(T), 16)));
+    HIP_OK(hipMemset(d, 0, std::max<size_t>(n * sizeof(T), 16)));
+    return d;
+}
+std::vector<float> to_host(const float* d, size_t n)
+{
+    std::vector<float> h(n);
+    HIP_OK(hipMemcpy(h.data(), d, n * 4, hipMemcpyDeviceToHost));
+    return h;
+}
+
+// Microseconds per call of fn(i), i cycling over `ring`, by HIP events on `st` (one warm-up pass first).
+template <class F>
+double time_us(F fn, uint32_t iters, uint32_t ring, hipStream_t st)
+{
+    for (uint32_t i = 0; i < std::min(iters, ring); i++) fn(i % ring);
+    hipEvent_t a, b;
+    HIP_OK(hipEventCreate(&a));
+    HIP_OK(hipEventCreate(&b));
+    HIP_OK(hipStreamSynchronize(st));
+    HIP_OK(hipEventRecord(a, st));
+    for (uint32_t i = 0; i < iters; i++) fn(i % ring);
+    HIP_OK(hipEventRecord(b, st));
+    HIP_OK(hipEventSynchronize(b));
+    float ms = 0.f;
+    HIP_OK(hipEventElapsedTime(&ms, a, b));
+    HIP_OK(hipEventDestroy(a));
+    HIP_OK(hipEventDestroy(b));
+    return (double)ms * 1e3 / iters;
+}
+
+// max |a - b| / max |b|
+double rel_maxabs(const std::vector<float>& a, const std::vector<float>& b)
+{
+    double top = 0, diff = 0;
+    for (size_t i = 0; i < b.size(); i++) {
+        top = std::max(top, (double)fabsf(b[i]));
+        diff = std::max(diff, (double)fabsf(a[i] - b[i]));
+    }
+    return top > 0 ? diff / top : diff;
+}
+
+void print_line(double us, double bytes, double flops)
+{
+    // the reference's line (src/main.cpp:596-599) with the fraction of this device's HBM peak added
+    printf("gpu: %8.1f us/iter | %7.1f GB/s (%4.1f%% of %.0f) | %8.1f GFLOP/s | %.1f MiB/iter\n", us, bytes / us / 1e3,
+           bytes / us / 1e3 / HBM_PEAK_GBPS * 100, HBM_PEAK_GBPS, flops / us / 1e3, bytes / (1 << 20));
+}
+
+bool verdict(const char* what, double err, double bar)
+{
+    printf("check: %s: rel max-abs err %.3g (bar %.0e) -> %s\n", what, err, bar, err <= bar ? "OK" : "FAIL");
+    return err <= bar;
+}
+
+// y = W x for one format: ring of tensors, time, cross-check against dequantise + dense fp32 GEMV
+bool case_gemv(const Format& f, uint32_t M, uint32_t K, uint32_t iters)
+{
+    if (qkk_row_bytes(f.type, K) == 0) {
+        fprintf(stderr, "qk: K=%u is not a multiple of the %s block (%u)\n", K, f.name, f.block_elems);
+        return false;
+    }
+    const size_t wbytes = (size_t)M * qkk_row_bytes(f.type, K);
+    const uint32_t ring = (uint32_t)std::min<size_t>(64, std::max<size_t>(2, (320u << 20) / wbytes + 1));
+    printf("== %s gemv M=%u K=%u iters=%u (ring of %u tensors, %.1f MiB each)\n", f.name, M, K, iters, ring,
+           wbytes / 1048576.0);
+    std::vector<uint8_t*> W(ring);
+    for (uint32_t r = 0; r < ring; r++) W[r] = to_device(random_tensor(f, (uint64_t)M * K, 42 + r));
+    float* x = to_device(random_rows(K, 43));
+    float* y = device_zeros<float>(M);
+    hipStream_t st = nullptr;
+    const double us = time_us([&](uint32_t r) { QK_OK(qkk_gemv(f.type, W[r], x, y, M, K, 1, st)); }, iters, ring, st);
+    print_line(us, (double)wbytes + 4.0 * K + 4.0 * M, 2.0 * M * K);
+    // second opinion: bit-exact dequantisation, then the dense fp32 product (rows in pieces of at most 256 MiB)
+    QK_OK(qkk_gemv(f.type, W[0], x, y, M, K, 1, st));
+    const std::vector<float> got = to_host(y, M);
+    std::vector<float> want(M);
+    const uint32_t piece = (uint32_t)std::max<uint64_t>(1, std::min<uint64_t>(M, (64ull << 20) / K));
+    float* dense = device_zeros<float>((size_t)piece * K);
+    float* y2 = device_zeros<float>(piece);
+    for (uint32_t r0 = 0; r0 < M; r0 += piece) {
+        const uint32_t n = std::min(piece, M - r0);
+        QK_OK(qkk_dequant(f.type, W[0] + (size_t)r0 * qkk_row_bytes(f.type, K), dense, (uint64_t)n * K, st));
+        QK_OK(qkk_gemv(QKK_F32, dense, x, y2, n, K, 1, st));
+        HIP_OK(hipMemcpy(want.data() + r0, y2, (size_t)n * 4, hipMemcpyDeviceToHost));
+    }
+    const bool ok = verdict("against dequantise + dense fp32 product", rel_maxabs(got, want), 1e-3);
+    for (uint8_t* p : W) HIP_OK(hipFree(p));
+    HIP_OK(hipFree(x)); HIP_OK(hipFree(y)); HIP_OK(hipFree(dense)); HIP_OK(hipFree(y2));
+    return ok;
+}
+
+// Y[N][M] = X[N][K] W[M][K]^T, W in Q8_0 (reference caseBGemm, src/main.cpp:5536-5672)
+bool case_bgemm(uint32_t M, uint32_t K, uint32_t N, uint32_t iters)
+{
+    const Format& f = *format_named("q8_0");
+    if (K % 32) {
+        fprintf(stderr, "qk: K=%u is not a multiple of 32\n", K);
+        return false;
+    }
+    const size_t wbytes = (size_t)M * qkk_row_bytes(QKK_Q8_0, K);
+    const uint32_t ring = (uint32_t)std::min<size_t>(64, std::max<size_t>(2, (320u << 20) / wbytes + 1));
+    printf("== q8_0 prefill gemm M=%u K=%u N=%u iters=%u (ring of %u)\n", M, K, N, iters, ring);
+    std::vector<uint8_t*> W(ring);
+    for (uint32_t r = 0; r < ring; r++) W[r] = to_device(random_tensor(f, (uint64_t)M * K, 42 + r));
+    float* X = to_device(random_rows((size_t)N * K, 43));
+    float* Y = device_zeros<float>((size_t)N * M);
+    hipStream_t st = nullptr;
+    const double us = time_us([&](uint32_t r) { QK_OK(qkk_gemm_q8_0(W[r], X, Y, M, K, N, st)); }, iters, ring, st);
+    const double flops = 2.0 * M * K * N, bytes = (double)wbytes + 4.0 * N * K + 4.0 * N * M;
+    print_line(us, bytes, flops);
+    // the reference prints TFLOP/s against its matrix peak (src/main.cpp:5668-5672)
+    printf("     %8.2f TFLOP/s = %.1f%% of the %.0f TFLOP/s dense fp16 matrix peak; %.0f tokens/s\n", flops / us / 1e6,
+           flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS * 100, MFMA_F16_PEAK_TFLOPS, N / us * 1e6);
+    QK_OK(qkk_gemm_q8_0(W[0], X, Y, M, K, N, st));
+    const std::vector<float> got = to_host(Y, (size_t)N * M);
+    // second opinion: one quantised GEMV per token (the one-row kernel, not the matrix cores)
+    std::vector<float> want((size_t)N * M);
+    float* y1 = device_zeros<float>(M);
+    for (uint32_t n = 0; n < N; n++) {
+        QK_OK(qkk_gemv(QKK_Q8_0, W[0], X + (size_t)n * K, y1, M, K, 1, st));
+        HIP_OK(hipMemcpy(want.data() + (size_t)n * M, y1, (size_t)M * 4, hipMemcpyDeviceToHost));
+    }
+    const bool ok = verdict("against one GEMV per token", rel_maxabs(got, want), 1e-3);
+    for (uint8_t* p : W) HIP_OK(hipFree(p));
+    HIP_OK(hipFree(X)); HIP_OK(hipFree(Y)); HIP_OK(hipFree(y1));
+    return ok;
+}
+
+struct Layer {
+    qkk_moe_layer L;
+    std::vector<void*> owned;
+};
+
+// One synthetic Qwen3-MoE layer at the reference model's shape (reference MoeT, src/main.cpp:1258-1311)
+Layer make_layer(uint64_t seed, int down_type, uint32_t E)
+{
+    const uint32_t H = 2048, F = 512, k = 8;
+    Layer out;
+    auto up = [&](const std::vector<uint8_t>& h) { void* p = to_device(h); out.owned.push_back(p); return p; };
+    const Format &iq3 = *format_named("iq3_xxs"), &q8 = *format_named("q8_0");
+    const Format& dn = down_type == QKK_Q6_K ? *format_named("q6_k") : *format_named("iq4_xs");
+    std::vector<float> gi = random_rows((size_t)E * H, seed * 16 + 1, 1.f / sqrtf((float)H)); // logits of order one
+    std::vector<float> gis = random_rows(H, seed * 16 + 2, 1.f / sqrtf((float)H));
+    float* d_gi = to_device(gi);
+    float* d_gis = to_device(gis);
+    out.owned.push_back(d_gi);
+    out.owned.push_back(d_gis);
+    out.L = qkk_moe_layer{H, F, E, k, QKK_IQ3_XXS, down_type, d_gi, d_gis,
+                          up(random_tensor(iq3, (uint64_t)E * F * H, seed * 16 + 3)), up(random_tensor(iq3, (uint64_t)E * F * H, seed * 16 + 4)),
+                          up(random_tensor(dn, (uint64_t)E * H * F, seed * 16 + 5)), up(random_tensor(q8, (uint64_t)F * H, seed * 16 + 6)),
+                          up(random_tensor(q8, (uint64_t)F * H, seed * 16 + 7)), up(random_tensor(q8, (uint64_t)H * F, seed * 16 + 8))};
+    return out;
+}
+
+bool case_moe(uint32_t seed, uint32_t iters, uint32_t slots, uint32_t E)
+{
+    if (slots < 1 || slots > 4096 || E < 8 || E > QKK_MAX_EXPERTS) {
+        fprintf(stderr, "qk: slots %u outside 1..4096 or experts %u outside 8..%u\n", slots, E, QKK_MAX_EXPERTS);
+        return false;
+    }
+    const uint32_t ring = 4, H = 2048;
+    const int down = slots == 1 ? QKK_IQ4_XS : QKK_Q6_K; // the reference's 35B model mixes both down types
+    printf("== fused moe layer (synthetic, seed %u): %u experts, %u slot(s), down %s, iters=%u, ring of %u layers\n", seed, E,
+           slots, down == QKK_Q6_K ? "q6_k" : "iq4_xs", iters, ring);
+    std::vector<Layer> layers;
+    for (uint32_t r = 0; r < ring; r++) layers.push_back(make_layer(seed * 8 + r, down, E));
+    float* X = to_device(random_rows((size_t)ring * slots * H, seed + 43));
+    float* Y = device_zeros<float>((size_t)slots * H);
+    qkk_sel* sel = device_zeros<qkk_sel>(slots);
+    const size_t wsb = qkk_moe_workspace_bytes(&layers[0].L, std::max(slots, 16u));
+    uint8_t* ws = device_zeros<uint8_t>(wsb);
+    hipStream_t st = nullptr;
+    auto step = [&](uint32_t r) { QK_OK(qkk_moe_decode(&layers[r].L, X + (size_t)r * slots * H, Y, sel, ws, wsb, slots, st)); };
+    const double us = time_us(step, iters, ring, st);
+    // bytes: router + shared gate row + shared expert + the distinct experts the rows picked (last step's picks)
+    step(0);
+    std::vector<qkk_sel> hs(slots);
+    HIP_OK(hipMemcpy(hs.data(), sel, slots * sizeof(qkk_sel), hipMemcpyDeviceToHost));
+    std::vector<uint32_t> ids;
+    for (const qkk_sel& s : hs) ids.insert(ids.end(), s.ids, s.ids + 8);
+    std::sort(ids.begin(), ids.end());
+    const size_t distinct = std::unique(ids.begin(), ids.end()) - ids.begin();
+    const double per_expert = 2.0 * 512 * qkk_row_bytes(QKK_IQ3_XXS, 2048) + 2048.0 * qkk_row_bytes(down, 512);
+    const double bytes = (double)E * 2048 * 4 + 2048 * 4 + distinct * per_expert + 2.0 * 512 * qkk_row_bytes(QKK_Q8_0, 2048) +
+                         2048.0 * qkk_row_bytes(QKK_Q8_0, 512) + slots * (2.0 * H * 4 + 160);
+    print_line(us, bytes, slots * (2.0 * E * H + 9 * 3 * 2.0 * 512 * H));
+    printf("     %zu distinct experts; picks of row 0:", distinct);
+    for (int i = 0; i < 8; i++) printf(" %u(%.3f)", hs[0].ids[i], hs[0].w[i]);
+    printf(" shared gate %.3f\n", hs[0].w_shared);
+    // per stage, as the reference's QK_STEP_PROF does (src/main.cpp:4591-4632)
+    for (uint32_t mask : {QKK_STAGE_ROUTE, QKK_STAGE_GATEUP, QKK_STAGE_DOWN}) {
+        const double su = time_us([&](uint32_t r) {
+            QK_OK(qkk_moe_decode_stages(&layers[r].L, X + (size_t)r * slots * H, Y, sel, ws, wsb, slots, mask, st)); }, iters, ring, st);
+        printf("     stage %-7s %7.1f us\n", mask == QKK_STAGE_ROUTE ? "route" : mask == QKK_STAGE_GATEUP ? "gate/up" : "down", su);
+    }
+    // second opinion: the same rows, repeated to fill sixteen, through the expert-major matrix-core path
+    step(0);
+    const std::vector<float> got = to_host(Y, (size_t)slots * H);
+    bool ok = true;
+    if (slots > 10) printf("check: none (above ten rows both calls would take the expert-major path)\n");
+    else {
+        std::vector<float> x0 = to_host(X, (size_t)slots * H), x16((size_t)16 * H);
+        for (uint32_t r = 0; r < 16; r++) memcpy(&x16[(size_t)r * H], &x0[(size_t)(r % slots) * H], H * 4);
+        float* X16 = to_device(x16);
+        float* Y16 = device_zeros<float>((size_t)16 * H);
+        qkk_sel* sel16 = device_zeros<qkk_sel>(16);
+        QK_OK(qkk_moe_decode(&layers[0].L, X16, Y16, sel16, ws, wsb, 16, st));
+        std::vector<float> want = to_host(Y16, (size_t)slots * H);
+        std::vector<qkk_sel> h16(16);
+        HIP_OK(hipMemcpy(h16.data(), sel16, 16 * sizeof(qkk_sel), hipMemcpyDeviceToHost));
+        bool same_ids = true;
+        for (uint32_t r = 0; r < slots; r++) same_ids = same_ids && !memcmp(hs[r].ids, h16[r].ids, 8 * 4);
+        printf("check: picks equal on both paths -> %s\n", same_ids ? "OK" : "FAIL");
+        ok = verdict("row-wise launches against the expert-major path", rel_maxabs(got, want), 1e-3) && same_ids;
+        HIP_OK(hipFree(X16)); HIP_OK(hipFree(Y16)); HIP_OK(hipFree(sel16));
+    }
+    for (Layer& l : layers)
+        for (void* p : l.owned) HIP_OK(hipFree(p));
+    HIP_OK(hipFree(X)); HIP_OK(hipFree(Y)); HIP_OK(hipFree(sel)); HIP_OK(hipFree(ws));
+    return ok;
+}
+
+bool case_head(uint32_t batch, uint32_t iters)
+{
+    const uint32_t V = 151936, K = 2048, ring = 2;
+    if (batch < 1 || batch > 16) {
+        fprintf(stderr, "qk: batch %u outside 1..16\n", batch);
+        return false;
+    }
+    const Format& f = *format_named("q6_k");
+    printf("== lm head + argmax: q6_k %u x %u, batch %u, iters=%u\n", V, K, batch, iters);
+    uint8_t* W[ring];
+    for (uint32_t r = 0; r < ring; r++) W[r] = to_device(random_tensor(f, (uint64_t)V * K, 77 + r));
+    float* X = to_device(random_rows((size_t)batch * K, 43));
+    uint32_t* tok = device_zeros<uint32_t>(batch);
+    float* logits = device_zeros<float>((size_t)batch * V);
+    const size_t wsb = qkk_head_workspace_bytes(V, batch);
+    uint8_t* ws = device_zeros<uint8_t>(wsb);
+    hipStream_t st = nullptr;
+    const double us = time_us([&](uint32_t r) { QK_OK(qkk_head_argmax(W[r], X, tok, nullptr, V, K, batch, ws, wsb, st)); }, iters, ring, st);
+    print_line(us, (double)V * qkk_row_bytes(QKK_Q6_K, K) + batch * (4.0 * K + 4), 2.0 * V * K * batch);
+    // second opinion: the logits written out, the two-pass argmax over them
+    QK_OK(qkk_head_argmax(W[0], X, tok, logits, V, K, batch, ws, wsb, st));
+    uint32_t* tok2 = device_zeros<uint32_t>(batch);
+    QK_OK(qkk_argmax(logits, tok2, V, batch, st));
+    std::vector<uint32_t> a(batch), b(batch);
+    HIP_OK(hipMemcpy(a.data(), tok, batch * 4, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(b.data(), tok2, batch * 4, hipMemcpyDeviceToHost));
+    const bool ok = a == b;
+    printf("check: fused argmax equals the argmax of the written logits (row 0: %u) -> %s\n", a[0], ok ? "OK" : "FAIL");
+    for (uint8_t* p : W) HIP_OK(hipFree(p));
+    HIP_OK(hipFree(X)); HIP_OK(hipFree(tok)); HIP_OK(hipFree(tok2)); HIP_OK(hipFree(logits)); HIP_OK(hipFree(ws));
+    return ok;
+}
+
+void usage()
+{
+    fprintf(stderr, "usage: qk suite\n"
+                    "       qk f16|q8_0|q6_k|iq4_xs|iq3_xxs [M] [K] [iters]\n"
+                    "       qk bgemm [M] [K] [N] [iters]\n"
+                    "       qk moe [seed] [iters] [slots] [experts]\n"
+                    "       qk head [batch] [iters]\n");
+}
+
+} // namespace
+
+int main(int argc, char** argv)
+{
+    if (argc < 2) {
+        usage();
+        return 1;
+    }
+    const std::string mode = argv[1];
+    auto arg_u = [&](int i, uint32_t dflt) { return argc > i ? (uint32_t)strtoul(argv[i], nullptr, 10) : dflt; };
+    const bool known = mode == "suite" || mode == "bgemm" || mode == "moe" || mode == "head" || format_named(mode.c_str());
+    if (!known) {
+        usage();
+        return 1;
+    }
+    char arch[64] = "";
+    uint32_t cus = 0;
+    if (qkk_device_info(arch, sizeof arch, &cus) < 1) {
+        fprintf(stderr, "qk: no HIP device: libqk.so has no CPU path\n");
+        return 2;
+    }
+    printf("device: %s, %u CUs\n", arch, cus);
+    bool ok = true;
+    if (mode == "suite") {
+        for (const Format& f : FORMATS) ok &= case_gemv(f, 8192, 8192, 200);
+    } else if (mode == "bgemm") {
+        ok = case_bgemm(arg_u(2, 8192), arg_u(3, 2048), arg_u(4, 256), arg_u(5, 40));
+    } else if (mode == "moe") {
+        ok = case_moe(arg_u(2, 0), arg_u(3, 200), arg_u(4, 1), arg_u(5, 256));
+    } else if (mode == "head") {
+        ok = case_head(arg_u(2, 1), arg_u(3, 40));
+    } else {
+        ok = case_gemv(*format_named(mode.c_str()), arg_u(2, 16384), arg_u(3, 8192), arg_u(4, 100));
+    }
+    printf("%s\n", ok ? "ALL OK" : "FAILED");
+    return ok ? 0 : 1;
+}

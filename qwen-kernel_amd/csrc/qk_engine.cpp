@@ -105,7 +105,8 @@ struct qk_engine {
     uint32_t pf_rows = 1024;     // positions of one slot a prefill pass carries (whole-model files; QK_PREFILL_ROWS)
     uint32_t cap = MAX_ROWS;     // rows the step's buffers hold (pf_rows for whole-model files)
     bool cat_everywhere = false; // every layer's input projections lie back to back (one product per layer)
-    bool dn_one_launch = false;  // QK_DN_FUSED=1: the gated-DeltaNet decode step as one launch (to be measured against two)
+    bool fused_norm = false;     // the "fused_norm" switch at qk_open: every consumer of a normalised row of the one-row step normalises on the way in
+    bool dn_one_launch = false;  // the "dn_fused" switch at qk_open: the gated-DeltaNet decode step as one launch (to be measured against two)
     uint32_t *d_pf = nullptr, *h_pf = nullptr; // [3][pf_rows] ids, positions, sampled ids of a prefill pass (device / pinned)
     float* d_rope = nullptr;     // [n_ctx][FA_ROT/2][2]
     float *d_big = nullptr, *d_mid = nullptr, *d_kin = nullptr, *d_vin = nullptr, *d_gb = nullptr, *d_conv = nullptr,
@@ -238,7 +239,7 @@ int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool 
     // consumers of a normalised row -- the input projections, the decay / write-strength products, the
     // head -- take the residual row and the norm's weights and normalise on the way in; the MoE
     // launches have done so all along.
-    const bool fuse = rows == 1 && !seq && !final_rows && cat_everywhere && !getenv("QK_NO_FUSED_NORM");
+    const bool fuse = rows == 1 && !seq && !final_rows && cat_everywhere && fused_norm;
     if (!fuse)
         if (int rc = qkk_rmsnorm(x, layers[0].attn_norm, d_xn[0], N_EMBD, rows, eps, st)) return rc;
     int cur = 0;
@@ -759,7 +760,9 @@ bool qk_engine::open(const char* path, const qk_config& cfg, char* err, size_t e
     memset(h_pos, 0, MAX_ROWS * 4);
     if (full_model && !load_mixers(g, err, err_len)) return false;
     cat_everywhere = full_model;
-    dn_one_launch = getenv("QK_DN_FUSED") && atoi(getenv("QK_DN_FUSED")) == 1 && DN_HV == 2 * DN_HK;
+    qk::apply_env_options(qk::options()); // the QK_* switches as the environment holds them now
+    dn_one_launch = qk::options().dn_fused && DN_HV == 2 * DN_HK;
+    fused_norm = qk::options().fused_norm != 0;
     for (const EngineLayer& L : layers) cat_everywhere = cat_everywhere && L.cat.w != nullptr;
     if (hipDeviceSynchronize() != hipSuccess) return bad("qk_open: upload failed"); // fills and uploads are complete
 

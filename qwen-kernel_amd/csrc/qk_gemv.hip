@@ -11,6 +11,7 @@
 #include <stdarg.h>
 
 #include <stdlib.h>
+#include <string.h>
 
 #include <algorithm>
 
@@ -50,6 +51,43 @@ uint32_t persistent_blocks()
         cached = (uint32_t)cus * 4u;
     }
     return cached;
+}
+
+namespace {
+struct OptionDef {
+    const char* name;
+    const char* env;
+    int Options::*field;
+    int lo, hi;
+};
+const OptionDef OPTION_DEFS[] = {
+    {"one_row", "QK_ONE_ROW", &Options::one_row_stream, 0, 1},   {"dense_reg", "QK_DENSE_REG", &Options::dense_reg, 0, 1},
+    {"fused_norm", "QK_FUSED_NORM", &Options::fused_norm, 0, 1}, {"attn_block", "QK_ATTN_BLOCK", &Options::attn_block, 0, 1},
+    {"dn_fused", "QK_DN_FUSED", &Options::dn_fused, 0, 1},       {"gemv_depth", "QK_GEMV_DEPTH", &Options::gemv_depth, 0, 16},
+    {"head_depth", "QK_HEAD_DEPTH", &Options::head_depth, 0, 8}, {"rowwise_max", "QK_ROWWISE_MAX", &Options::rowwise_max, 0, 64},
+};
+} // namespace
+
+// Applies the switches that are set in the environment right now (a value outside its range is ignored).
+void apply_env_options(Options& v)
+{
+    for (const OptionDef& d : OPTION_DEFS) {
+        const char* e = getenv(d.env);
+        if (!e || !*e) continue;
+        int x = atoi(e);
+        if (d.field == &Options::one_row_stream) x = !strcmp(e, "stream") ? 1 : !strcmp(e, "lane") ? 0 : x;
+        if (x >= d.lo && x <= d.hi) v.*d.field = x;
+    }
+}
+
+Options& options()
+{
+    static Options o = [] {
+        Options v;
+        apply_env_options(v);
+        return v;
+    }();
+    return o;
 }
 
 int check_launch(const char* what)
@@ -454,29 +492,40 @@ static void launch_q(const void* W, const float* X, float* Y, uint32_t M, uint32
     const uint32_t cus = persistent_blocks() / 4;
     const uint32_t chunks = M / CH, tail_groups = (M - chunks * CH + WAVE / LPR - 1) / (WAVE / LPR);
     const uint32_t want = (std::max(chunks, tail_groups) + 3) / 4; // one chunk per wave
-    // QK_GEMV_DEPTH=n (1..16): workgroups per CU of the persistent grid, for sweeps on the device
-    static const uint32_t depth_env = [] { const char* e = getenv("QK_GEMV_DEPTH"); const int v = e ? atoi(e) : 0; return v >= 1 && v <= 16 ? (uint32_t)v : 0u; }();
-    const uint32_t depth = depth_env ? std::min(depth_env, RESIDENT) : DEPTH;
+    // the "gemv_depth" switch: workgroups per CU of the persistent grid, for sweeps on the device
+    const uint32_t depth_opt = (uint32_t)options().gemv_depth;
+    const uint32_t depth = depth_opt ? std::min(depth_opt, RESIDENT) : DEPTH;
     const uint32_t blocks = std::max(1u, want <= cus * RESIDENT ? want : cus * depth);
     hipLaunchKernelGGL((gemv_stream_kernel<TYPE, LPR, PASSES, RPC, NORM>), dim3(blocks, batch), dim3(256), 0, st,
                        (const uint8_t*)W, X, Y, M, nw, eps);
 }
 
+bool lane_gemv_launch(int type, const void* W, const float* X, float* Y, uint32_t M, uint32_t K, uint32_t batch, hipStream_t st); // qk_gemv_lane.hip
+
+// The streaming form of one quantised GEMV launch; false for a K outside the tiled shapes.
 template <int TYPE>
-static int dispatch_q(const void* W, const float* X, float* Y, uint32_t M, uint32_t K, uint32_t batch,
-                      hipStream_t st)
+static bool stream_gemv_launch(const void* W, const float* X, float* Y, uint32_t M, uint32_t K, uint32_t batch, hipStream_t st)
 {
-    const uint32_t rb = (uint32_t)qkk_row_bytes(TYPE, K);
     if (K == 2048) launch_q<TYPE, 64, 1>(W, X, Y, M, batch, st);
     else if (K == 4096) launch_q<TYPE, 64, 2>(W, X, Y, M, batch, st);
     else if (K == 8192) launch_q<TYPE, 64, 4>(W, X, Y, M, batch, st);
     else if (K == 1024) launch_q<TYPE, 32, 1>(W, X, Y, M, batch, st);
     else if (K == 512) launch_q<TYPE, 16, 1>(W, X, Y, M, batch, st);
     else if (K == 256) launch_q<TYPE, 8, 1>(W, X, Y, M, batch, st);
-    else {
+    else return false;
+    return true;
+}
+
+template <int TYPE>
+static int dispatch_q(const void* W, const float* X, float* Y, uint32_t M, uint32_t K, uint32_t batch,
+                      hipStream_t st)
+{
+    const bool tiled = options().one_row_stream ? stream_gemv_launch<TYPE>(W, X, Y, M, K, batch, st)
+                                                : lane_gemv_launch(TYPE, W, X, Y, M, K, batch, st);
+    if (!tiled) { // any other K that is a block multiple
         const uint32_t blocks = (uint32_t)std::min<uint64_t>(((uint64_t)M + 3) / 4, 4096);
         hipLaunchKernelGGL((gemv_q_generic_kernel<TYPE>), dim3(blocks, batch), dim3(256), 0, st,
-                           (const uint8_t*)W, X, Y, M, K, rb);
+                           (const uint8_t*)W, X, Y, M, K, (uint32_t)qkk_row_bytes(TYPE, K));
     }
     return check_launch("qkk_gemv");
 }
@@ -497,6 +546,30 @@ void* moe_static_scratch();
 extern "C" {
 
 const char* qkk_last_error(void) { return t_err; }
+
+int qkk_set_option(const char* name, int value)
+{
+    if (!name) return fail(QKK_EINVAL, "qkk_set_option: null name");
+    for (const OptionDef& d : OPTION_DEFS)
+        if (!strcmp(name, d.name)) {
+            if (value < d.lo || value > d.hi)
+                return fail(QKK_EINVAL, "qkk_set_option: %s = %d outside %d..%d", name, value, d.lo, d.hi);
+            options().*d.field = value;
+            return QKK_OK;
+        }
+    return fail(QKK_EINVAL, "qkk_set_option: no switch named '%s'", name);
+}
+
+int qkk_get_option(const char* name, int* value)
+{
+    if (!name || !value) return fail(QKK_EINVAL, "qkk_get_option: null pointer");
+    for (const OptionDef& d : OPTION_DEFS)
+        if (!strcmp(name, d.name)) {
+            *value = options().*d.field;
+            return QKK_OK;
+        }
+    return fail(QKK_EINVAL, "qkk_get_option: no switch named '%s'", name);
+}
 
 int qkk_device_info(char* arch_host, size_t arch_len, uint32_t* n_cu_host)
 {
@@ -618,7 +691,8 @@ int qkk_gemv(int type, const void* W, const float* X, float* Y, uint32_t M, uint
     case QKK_F32: {
         const uint32_t per = type == QKK_F16 ? 8 : 4;
         if (K % per) return fail(QKK_ESHAPE, "qkk_gemv: K=%u must be a multiple of %u for dense rows", K, per);
-        if (type == QKK_F16 ? launch_dense_reg<_Float16>(W, X, Y, M, K, batch, st) : launch_dense_reg<float>(W, X, Y, M, K, batch, st))
+        if (!options().dense_reg) {} // the chunk loop below
+        else if (type == QKK_F16 ? launch_dense_reg<_Float16>(W, X, Y, M, K, batch, st) : launch_dense_reg<float>(W, X, Y, M, K, batch, st))
             return check_launch("qkk_gemv");
         const dim3 grid(std::min((M + 3) / 4, persistent_blocks()), batch);
         if (type == QKK_F16)

@@ -163,6 +163,97 @@ __global__ __launch_bounds__(256) void head_q6k_kernel(const uint8_t* __restrict
     }
 }
 
+// The same head with per-lane block loads: every lane fetches its own block fields from global memory,
+// RIF rows per wave in flight in two register sets.  The form whose results and timings come from runs
+// on an MI355X (59-64 us for the 151,936-row head); used unless the "one_row" switch selects the
+// streaming kernel above.
+template <int PASSES, int RIF>
+__global__ __launch_bounds__(256) void head_q6k_lane_kernel(const uint8_t* __restrict__ W,
+                                                       const float* __restrict__ X,
+                                                       float* __restrict__ logits_out,
+                                                       uint32_t* __restrict__ tok, HeadWs ws, uint32_t V,
+                                                       uint32_t K, uint32_t row_bytes)
+{
+    __shared__ float s_v[256];
+    __shared__ uint32_t s_i[256];
+    __shared__ uint32_t s_last;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t b = blockIdx.y;
+    const float* x = X + (size_t)b * K;
+
+    XSlice xs[PASSES];
+    float xsum[PASSES][4];
+#pragma unroll
+    for (int p = 0; p < PASSES; p++) {
+        load_xslice<QKK_Q6_K>(xs[p], x + p * 2048, lane);
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            float s = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) s += xs[p].v[c * 8 + i];
+            xsum[p][c] = s;
+        }
+    }
+    const uint32_t pass_bytes = row_bytes / PASSES;
+    float bv = ARG_FLOOR;
+    uint32_t bi = 0xFFFFFFFFu;
+    // chunks of RIF rows dealt round-robin to the waves; a wave's rows ascend.  The next
+    // chunk's loads are issued before the arithmetic of the current one.
+    const uint32_t stride = gridDim.x * 4 * RIF;
+    LaneW<QKK_Q6_K> w[2][RIF][PASSES];
+    auto fetch = [&](int set, uint32_t r0) {
+#pragma unroll
+        for (int i = 0; i < RIF; i++) {
+            const uint32_t r = min(r0 + i, V - 1);
+#pragma unroll
+            for (int p = 0; p < PASSES; p++)
+                w[set][i][p].load(W + (size_t)r * row_bytes + (size_t)p * pass_bytes, lane);
+        }
+    };
+    auto reduce = [&](int set, uint32_t r0) {
+#pragma unroll
+        for (int i = 0; i < RIF; i++) {
+            float acc = 0.f;
+#pragma unroll
+            for (int p = 0; p < PASSES; p++) acc += w[set][i][p].dot(xs[p], xsum[p], nullptr, lane);
+            acc = wave_sum(acc);
+            const uint32_t r = r0 + i;
+            if (r < V) {
+                if (logits_out && lane == 0) logits_out[(size_t)b * V + r] = acc;
+                if (acc > bv) { bv = acc; bi = r; } // rows ascend: strict '>' keeps the lowest id
+            }
+        }
+    };
+    uint32_t r0 = (blockIdx.x * 4 + wave) * RIF;
+    fetch(0, r0);
+    for (; r0 < V; r0 += 2 * stride) {
+        fetch(1, r0 + stride);
+        reduce(0, r0);
+        fetch(0, r0 + 2 * stride);
+        reduce(1, r0 + stride);
+    }
+
+    // fold the four waves of the block
+    if (lane == 0) { s_v[wave] = bv; s_i[wave] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int wv = 1; wv < 4; wv++)
+            if (better(s_v[wv], s_i[wv], bv, bi)) { bv = s_v[wv]; bi = s_i[wv]; }
+        publish(&ws.cand_v[(size_t)b * gridDim.x + blockIdx.x], bv);
+        publish(&ws.cand_i[(size_t)b * gridDim.x + blockIdx.x], bi);
+        s_last = arrive_last(&ws.counter[b], gridDim.x) ? 1u : 0u;
+    }
+    __syncthreads();
+    if (s_last) {
+        const uint32_t t = fold_candidates(ws.cand_v + (size_t)b * gridDim.x, ws.cand_i + (size_t)b * gridDim.x,
+                                           gridDim.x, s_v, s_i);
+        if (threadIdx.x == 0) {
+            tok[b] = t;
+            ws.counter[b] = 0u;
+        }
+    }
+}
+
 // One block per row; ties to the lower index.
 __global__ __launch_bounds__(256) void argmax_kernel(const float* __restrict__ logits,
                                                      uint32_t* __restrict__ tok, uint32_t n)
@@ -302,10 +393,20 @@ __global__ __launch_bounds__(CT) void head_q6k_coop_kernel(const uint8_t* __rest
 constexpr uint32_t HEAD_RPC = 2, HEAD_DEPTH = 8;
 static uint32_t head_blocks(uint32_t V, uint32_t rpc)
 {
-    // QK_HEAD_DEPTH=n (1..8): workgroups per CU, for sweeps on the device (never more than the workspace bound's 8)
-    static const uint32_t depth_env = [] { const char* e = getenv("QK_HEAD_DEPTH"); const int v = e ? atoi(e) : 0; return v >= 1 && v <= (int)HEAD_DEPTH ? (uint32_t)v : 0u; }();
+    // the "head_depth" switch (1..8): workgroups per CU, for sweeps on the device (never more than the workspace bound's 8)
+    const uint32_t depth_env = (uint32_t)options().head_depth;
     const uint32_t waves = std::max(V / rpc, V % rpc);
     return std::max(1u, std::min((waves + 3) / 4, persistent_blocks() / 4 * (depth_env ? depth_env : HEAD_DEPTH)));
+}
+
+// Persistent grid of the per-lane kernel.  Measured on the 151,936-row head (two rows in flight per
+// wave, double-buffered): 256 workgroups 65.0 us, 512: 60.0, 768: 62.4, 1024: 63.2, and grids that
+// are not a multiple of the CU count lose 5 us more; four rows in flight (133 VGPRs) 68.3 us.
+constexpr uint32_t HEAD_LANE_RIF = 2;
+static uint32_t head_lane_blocks(uint32_t V, uint32_t rif)
+{
+    const uint32_t waves = (V + rif - 1) / rif;
+    return std::min((waves + 3) / 4, persistent_blocks() / 2);
 }
 
 } // namespace qk
@@ -354,12 +455,21 @@ static int head_argmax_impl(const void* W, const float* X, uint32_t* tok, float*
                            logits, tok, ws, V, batch);
         return check_launch("qkk_head_argmax");
     }
-    const uint32_t blocks = head_blocks(V, K == 2048 ? HEAD_RPC : 1);
+    const bool lane_form = !w_norm && !options().one_row_stream; // the norm in front exists in the streaming form only
+    const uint32_t blocks = lane_form ? head_lane_blocks(V, HEAD_LANE_RIF) : head_blocks(V, K == 2048 ? HEAD_RPC : 1);
     HeadWs ws;
     ws.counter = (uint32_t*)workspace;
     ws.cand_v = (float*)((uint8_t*)workspace + 256);
     ws.cand_i = (uint32_t*)(ws.cand_v + (size_t)batch * blocks);
-    if (w_norm)
+    if (lane_form) {
+        const uint32_t rb = (uint32_t)qkk_row_bytes(QKK_Q6_K, K);
+        if (K == 2048)
+            hipLaunchKernelGGL((head_q6k_lane_kernel<1, HEAD_LANE_RIF>), dim3(blocks, batch), dim3(256), 0, st, (const uint8_t*)W,
+                               X, logits, tok, ws, V, K, rb);
+        else
+            hipLaunchKernelGGL((head_q6k_lane_kernel<2, 2>), dim3(blocks, batch), dim3(256), 0, st, (const uint8_t*)W, X,
+                               logits, tok, ws, V, K, rb);
+    } else if (w_norm)
         hipLaunchKernelGGL((head_q6k_kernel<1, HEAD_RPC, true>), dim3(blocks, batch), dim3(256), 0, st, (const uint8_t*)W,
                            X, logits, tok, ws, V, w_norm, eps);
     else if (K == 2048)

@@ -21,6 +21,23 @@ uint32_t persistent_blocks();
 // Converts the last launch error (if any) into a QKK_EDEVICE failure.
 int check_launch(const char* what);
 
+// Switches of the library, read once from the environment on first use; qkk_set_option changes one at
+// run time (a test or a bench that runs both forms of a kernel in one process).  A form of a kernel
+// that has not yet been run and timed on a device is reached only through its switch: the default
+// of every switch is the form that has.
+struct Options {
+    int one_row_stream = 0; // QK_ONE_ROW=stream: one-row GEMV / MoE step / LM head stream block rows as 16-byte pieces through LDS (default "lane": every lane loads its own block fields)
+    int dense_reg = 0;      // QK_DENSE_REG=1: F16 / F32 GEMV keeps its share of x in registers
+    int fused_norm = 0;     // QK_FUSED_NORM=1: the engine's one-row step folds each RMS norm into its consumer (needs the streaming form)
+    int attn_block = 0;     // QK_ATTN_BLOCK=1: prefill attention over blocks of 16 rows on the matrix cores (default: two rows per workgroup)
+    int dn_fused = 0;       // QK_DN_FUSED=1: the gated-DeltaNet decode step as one launch
+    int gemv_depth = 0;     // QK_GEMV_DEPTH=n (1..16): workgroups per CU of the streaming GEMV's persistent grid, 0 = built-in
+    int head_depth = 0;     // QK_HEAD_DEPTH=n (1..8): the same for the streaming LM head
+    int rowwise_max = 0;    // QK_ROWWISE_MAX=n (1..64): rows up to which the plain MoE step runs row by row, 0 = QKK_ROWWISE_MAX
+};
+Options& options();
+void apply_env_options(Options& v); // qk_open reads the environment again: switches set since the first use take effect for the engine it builds
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }

@@ -594,14 +594,6 @@ static void launch_down(const qkk_moe_layer* L, const MoeWs& ws, const qkk_sel* 
 
 constexpr uint32_t ROWWISE_MAX = QKK_ROWWISE_MAX; // rows up to which each row runs the one-row launches
 
-// One row with the RMS norm in front (weights w) and the residual behind: see qkk_moe_layer_row.
-struct MoeNorm {
-    const float* w;
-    float eps;
-    const float* mix = nullptr; // the row is X + mix ...
-    float* sum = nullptr;       // ... which launch 1 stores here for launches 2 and 3
-};
-
 // Launches 1 and 2 for `rows` activation rows (grid.y); norm given: the variants with the RMS norm
 // in front.
 static void launch_route_gateup(const qkk_moe_layer* L, const float* X, const MoeWs& ws, qkk_sel* sel, const MoeDims& d,
@@ -722,20 +714,25 @@ static int moe_decode_impl(const char* who, const qkk_moe_layer* L, const float*
     // there is little to share: each row runs the one-row launches (grid.y = row), and its result
     // is bit for bit what it is alone.  Measured: 2 rows 26 us against 40 us on the expert-major
     // path, 4 rows 37 / 50, 8 rows 62 / 71, 10 rows 76 / 78, 12 rows 87 / 86: more rows go there.
-    // QK_ROWWISE_MAX=n (1..64) moves the switch between the two paths for the plain step, for measurements on the
-    // device (the limit of the entry points with the norm in front stays QKK_ROWWISE_MAX)
-    static const uint32_t switch_env = [] { const char* e = getenv("QK_ROWWISE_MAX"); const int v = e ? atoi(e) : 0; return v >= 1 && v <= 64 ? (uint32_t)v : 0u; }();
-    if (n_slots > (norm || !switch_env ? ROWWISE_MAX : switch_env)) {
+    // the "rowwise_max" switch moves the change between the two paths for the plain step, for measurements on
+    // the device (the limit of the entry points with the norm in front stays QKK_ROWWISE_MAX)
+    const uint32_t switch_opt = (uint32_t)options().rowwise_max;
+    if (n_slots > (norm || !switch_opt ? ROWWISE_MAX : switch_opt)) {
         if (norm) return fail(QKK_ESHAPE, "%s: %u rows exceed %u (use qkk_moe_decode_tail)", who, n_slots, ROWWISE_MAX);
         return moe_grouped_launch(L, X, Y, sel, workspace, n_slots, stages, st, tail);
     }
     const MoeWs ws = ws_carve(workspace, d, n_slots);
 
-    launch_route_gateup(L, X, ws, sel, d, stages, norm, n_slots, st);
+    // two forms of the three launches: block fields loaded per lane (qk_moe_lane.hip), or rows streamed
+    // as 16-byte pieces through LDS (this file); same arguments, same workspace
+    const bool staged = options().one_row_stream != 0;
+    if (staged) launch_route_gateup(L, X, ws, sel, d, stages, norm, n_slots, st);
+    else lane_route_gateup(L, X, ws, sel, d, stages, norm, n_slots, st);
     if (stages & QKK_STAGE_DOWN) {
         // norm in front: the input row (with the mixer's output, if any) is the residual; Y may be X
         const float* resid = norm ? (norm->mix ? norm->sum : X) : nullptr;
-        if (L->down_type == QKK_IQ4_XS) launch_down<QKK_IQ4_XS>(L, ws, sel, Y, d, resid, n_slots, st);
+        if (!staged) lane_down(L, ws, sel, Y, d, resid, n_slots, st);
+        else if (L->down_type == QKK_IQ4_XS) launch_down<QKK_IQ4_XS>(L, ws, sel, Y, d, resid, n_slots, st);
         else launch_down<QKK_Q6_K>(L, ws, sel, Y, d, resid, n_slots, st);
         // the step's output went to tail->Xn (see qkk_moe_decode_tail); add and norm in place
         if (tail) launch_add_rmsnorm(tail->resid, Y, tail->w_next, tail->S, tail->Xn, d.H, n_slots, tail->eps, st);

@@ -42,6 +42,20 @@ struct MoeTail {
     float* Xn;
 };
 
+// One row with the RMS norm in front (weights w) and the residual behind.
+struct MoeNorm {
+    const float* w;
+    float eps;
+    const float* mix = nullptr; // the row is X + mix ...
+    float* sum = nullptr;       // ... which launch 1 stores here for launches 2 and 3
+};
+
+// The per-lane form of the one-row launches (qk_moe_lane.hip): launches 1 and 2, and launch 3.
+void lane_route_gateup(const qkk_moe_layer* L, const float* X, const MoeWs& ws, qkk_sel* sel, const MoeDims& d,
+                       uint32_t stages, const MoeNorm* norm, uint32_t rows, hipStream_t st);
+void lane_down(const qkk_moe_layer* L, const MoeWs& ws, const qkk_sel* sel, float* Y, const MoeDims& d,
+               const float* resid, uint32_t rows, hipStream_t st);
+
 static inline size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 static inline size_t ws_bytes(const MoeDims& d, uint32_t n)

@@ -55,3 +55,42 @@ def dev(qk):
         pytest.skip("no HIP device")
     print(f"[gpu] {torch.cuda.get_device_name(0)}", flush=True)
     return "cuda:0"
+
+
+SWITCHES = ("one_row", "dense_reg", "fused_norm", "attn_block", "dn_fused", "gemv_depth", "head_depth", "rowwise_max")
+SWITCH_ENV_DEFAULTS = {"QK_ONE_ROW": "lane", "QK_DENSE_REG": "0", "QK_FUSED_NORM": "0", "QK_ATTN_BLOCK": "0", "QK_DN_FUSED": "0"}
+UNRUN = ("a form of the kernels that has not had its first supervised run on a device is reached through a switch "
+         "and tested on hardware only with QK_TEST_UNRUN_FORMS=1 (the host-side build always runs it)")
+
+
+def unrun_forms_allowed(dev):
+    """Kernel forms written after the last run on a device: always tested in the host-side build; on a
+    device only when asked for, so that an unattended run of the suite exercises the forms that have run
+    there before."""
+    return dev == "cpu" or os.environ.get("QK_TEST_UNRUN_FORMS") == "1"
+
+
+@pytest.fixture(params=["lane", "stream"])
+def one_row_form(request, qk, dev):
+    """Both forms of the one-row kernels (GEMV, MoE step, LM head): block fields loaded per lane -- the
+    default -- and rows streamed as 16-byte pieces through LDS (with the dense rows' x in registers)."""
+    on = int(request.param == "stream")
+    if on and not unrun_forms_allowed(dev):
+        pytest.skip(UNRUN)
+    with qk.option("one_row", on), qk.option("dense_reg", on):
+        yield request.param
+
+
+@pytest.fixture
+def switches_back_to_defaults(qk, dev):
+    """qk_open applies the QK_* switches of the environment to the library; this puts the defaults back."""
+    yield
+    for name in SWITCHES:
+        qk.set_option(name, 0)
+
+
+@pytest.fixture
+def unrun_form(dev):
+    """For a test of an entry point or switch whose kernels have not had their first run on a device."""
+    if not unrun_forms_allowed(dev):
+        pytest.skip(UNRUN)

@@ -139,7 +139,16 @@ def test_other_workloads_print_one_line_each(monkeypatch, capsys, qk):
         assert out["metric"] == metric and out["config"]["workload"] == wl and out["value"] > 0, wl
     monkeypatch.setattr(sys, "argv", ["bench.py", "--workload", "extras", "--no-cpu"])
     bench.main()
-    assert "gemv_q8_0_8192x2048" in _one_json_line(capsys)["extras"]
+    ex = _one_json_line(capsys)["extras"]
+    assert "gemv_q8_0_8192x2048" in ex and not any(k.startswith("stream:") for k in ex)
+    # both forms of the one-row kernels side by side, on request only
+    monkeypatch.setattr(sys, "argv", ["bench.py", "--workload", "extras", "--no-cpu", "--ab-forms"])
+    bench.main()
+    ex = _one_json_line(capsys)["extras"]
+    for form in ("lane", "stream"):
+        for k in ("gemv_iq4_xs_8192x2048", "gemv_q6_k_sustained_256MiB", "head_q6k_151936_bs1", "moe_decode_bs1"):
+            assert "error" not in ex[f"{form}:{k}"], (form, k, ex[f"{form}:{k}"])
+    assert qk.get_option("one_row") == 0   # the switch is back at its default
 
 
 def test_a_failing_side_measurement_is_an_entry_of_the_line(monkeypatch, capsys, qk):

@@ -1,0 +1,70 @@
+"""`qk`, the operator test program (qwen-kernel_amd/csrc/qk_cli.cpp; the modes of the reference's binary,
+src/main.cpp:6952-6978).  Without a GPU its logic runs over the host-side build of the kernels (tests/emu/qk_emu:
+the same source against the stand-in runtime); on a device the real binary runs a small case per mode."""
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+QK = os.path.join(ROOT, "qwen-kernel_amd", "qk")
+QK_EMU = os.path.join(ROOT, "tests", "emu", "qk_emu")
+
+
+def run(binary, *args, timeout=300):
+    return subprocess.run([binary, *map(str, args)], capture_output=True, text=True, timeout=timeout)
+
+
+@pytest.fixture(scope="module")
+def qk_emu():
+    if not os.path.exists(QK_EMU):
+        subprocess.run(["make", "-C", os.path.dirname(QK_EMU), "-j", "8"], check=True, stdout=subprocess.DEVNULL)
+    return QK_EMU
+
+
+def test_usage_and_no_device():
+    """No mode, or an unknown one: the usage text and status 1.  A mode without a HIP device: a message that
+    says so and status 2 -- the program has no CPU arithmetic to fall back on."""
+    if not os.path.exists(QK):
+        pytest.skip("qk is not built")
+    for args in ((), ("frobnicate",)):
+        r = run(QK, *args)
+        assert r.returncode == 1 and "usage: qk suite" in r.stderr and not r.stdout
+    import torch
+    if not torch.cuda.is_available():
+        r = run(QK, "q8_0", 64, 256, 1)
+        assert r.returncode == 2 and "no HIP device" in r.stderr
+
+
+@pytest.mark.parametrize("args", [("q8_0", 96, 512, 2), ("q6_k", 33, 2048, 1), ("iq4_xs", 40, 1024, 1), ("iq3_xxs", 40, 2048, 1),
+                                  ("f16", 21, 768, 1), ("bgemm", 48, 512, 20, 1), ("moe", 1, 1, 1, 8), ("moe", 2, 1, 3, 8)],
+                         ids=lambda a: "-".join(map(str, a)))
+def test_modes_in_the_host_build(qk_emu, args):
+    """Every mode on a small shape: the line with the rates, the verdict of the second computation (the
+    dequantise + dense product for the GEMVs, one GEMV per token for the GEMM, the expert-major path for the
+    MoE rows), status 0."""
+    r = run(qk_emu, *args)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "us/iter" in r.stdout and "GB/s" in r.stdout and "-> OK" in r.stdout and "FAIL" not in r.stdout
+    assert r.stdout.strip().endswith("ALL OK")
+
+
+def test_bad_shapes_are_refused(qk_emu):
+    r = run(qk_emu, "q6_k", 8, 100, 1)     # K is not a multiple of the 256-weight block
+    assert r.returncode == 1 and "not a multiple" in r.stderr
+    r = run(qk_emu, "moe", 0, 1, 5000)
+    assert r.returncode == 1 and "outside" in r.stderr
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("args", [("q8_0", 8192, 2048, 50), ("iq3_xxs", 8192, 2048, 50), ("f16", 4096, 4096, 20),
+                                  ("bgemm", 8192, 2048, 128, 10), ("moe", 0, 40, 1), ("moe", 0, 20, 4), ("head", 1, 6)],
+                         ids=lambda a: "-".join(map(str, a)))
+def test_modes_on_the_device(dev, args):
+    if dev == "cpu":
+        pytest.skip("the host-side build has its own cases above")
+    print(f"[case] qk {' '.join(map(str, args))}", flush=True)
+    r = run(QK, *args, timeout=600)
+    print(r.stdout, flush=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "GB/s" in r.stdout and r.stdout.strip().endswith("ALL OK")

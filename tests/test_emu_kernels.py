@@ -18,6 +18,26 @@ def emu(qk):
         yield pool
 
 
+@pytest.fixture(params=["lane", "stream"])
+def form(request, qk, emu):
+    """Both forms of the one-row kernels: block fields loaded per lane (the default), and rows streamed as
+    16-byte pieces through LDS with the dense rows' x in registers (the "one_row" and "dense_reg" switches)."""
+    on = int(request.param == "stream")
+    with qk.option("one_row", on), qk.option("dense_reg", on):
+        yield request.param
+
+
+SWITCHES = ("one_row", "dense_reg", "fused_norm", "attn_block", "dn_fused", "gemv_depth", "head_depth", "rowwise_max")
+
+
+@pytest.fixture
+def switches_back_to_defaults(qk, emu):
+    """qk_open applies the QK_* switches of the environment to the library; this puts the defaults back."""
+    yield
+    for name in SWITCHES:
+        qk.set_option(name, 0)
+
+
 QUANT = ["q8_0", "q6_k", "iq4_xs", "iq3_xxs"]
 
 
@@ -28,7 +48,7 @@ def type_id(qk, name):
 @pytest.mark.parametrize("name", QUANT)
 @pytest.mark.parametrize("K,M", [(2048, 1), (2048, 9), (2048, 67), (4096, 5), (8192, 3), (1024, 11), (512, 23), (256, 70),
                                  (768, 6)])
-def test_gemv_inside_its_tensors(qk, orc, emu, name, K, M):
+def test_gemv_inside_its_tensors(qk, orc, emu, name, K, M, form):
     """Ragged row counts: full chunks go through the staged 16-byte pieces, the rest through per-lane
     loads; the last row ends at the guard page."""
     t = type_id(qk, name)
@@ -93,7 +113,7 @@ def rows_that_pick_the_last_expert(hl, n, seed, scale=None):
 @pytest.mark.parametrize("down", ["iq4_xs", "q6_k"])
 @pytest.mark.parametrize("E,k,F,H,n", [(8, 2, 256, 2048, 1), (8, 2, 512, 2048, 3), (16, 16, 256, 2048, 1), (6, 3, 1024, 2048, 2),
                                        (4, 2, 256, 4096, 2), (20, 10, 512, 2048, 1)])
-def test_moe_step_inside_its_tensors(qk, orc, emu, down, E, k, F, H, n):
+def test_moe_step_inside_its_tensors(qk, orc, emu, down, E, k, F, H, n, form):
     """The three one-row launches with the LAST expert among the picks: its last rows end at the guard
     page (a Q6_K run of rows is not a whole number of 16-byte pieces -- the staging must not fetch the
     piece behind it)."""
@@ -104,7 +124,7 @@ def test_moe_step_inside_its_tensors(qk, orc, emu, down, E, k, F, H, n):
 
 
 @pytest.mark.parametrize("down", ["iq4_xs", "q6_k"])
-def test_moe_block_with_norm_inside_its_tensors(qk, orc, emu, down):
+def test_moe_block_with_norm_inside_its_tensors(qk, orc, emu, down, form):
     """The block with the RMS norm in front and the residual behind, alone and with a mixer's rows
     added on the way, 1 and 3 rows."""
     hl = qk.synth.HostLayer(seed=91, n_ff=256, n_expert=8, n_used=2, down_type=type_id(qk, down))
@@ -117,7 +137,7 @@ def test_moe_block_with_norm_inside_its_tensors(qk, orc, emu, down):
         moe_case(qk, orc, emu, hl, x, norm_w=w, mix=mix)
 
 
-def test_moe_static_workspace_in_the_host_build(qk, orc, emu):
+def test_moe_static_workspace_in_the_host_build(qk, orc, emu, form):
     """qkk_moe_decode_static against qkk_moe_decode, both through the host-side build: same bits."""
     hl = qk.synth.HostLayer(seed=12, n_ff=256, n_expert=8, n_used=2)
     layer = emu_util.layer_in_pool(qk, emu, hl)
@@ -135,7 +155,7 @@ def test_moe_static_workspace_in_the_host_build(qk, orc, emu):
 
 
 @pytest.mark.parametrize("V,batch", [(37, 1), (1000, 1), (300, 3)])
-def test_head_inside_its_tensors(qk, orc, emu, V, batch):
+def test_head_inside_its_tensors(qk, orc, emu, V, batch, form):
     """LM head + argmax on a small vocabulary whose last row ends at the guard page."""
     K = 2048
     W = qk.synth.tensor_host(qk.Q6_K, V, K, seed=V)
@@ -201,7 +221,8 @@ def test_attention_blocks_inside_their_tensors(qk, emu, hq, hkv, base, n_pos):
     ws = emu.workspace(qk.attn_workspace_bytes(n_pos, hq))
     qh = qk.attn_prep(qfd, emu.tensor(kin), emu.tensor(vin), emu.tensor(qn), emu.tensor(kn), emu.tensor(rope), pos, kd, vd, NROT,
                       qhat=emu.zeros((n_pos, hq, DH), np.float32), seq=True)
-    att = qk.attn_decode(qh, kd, vd, qfd, pos, ws, att=emu.zeros((n_pos, hq, DH), np.float32), seq=True).numpy()
+    with qk.option("attn_block", 1):
+        att = qk.attn_decode(qh, kd, vd, qfd, pos, ws, att=emu.zeros((n_pos, hq, DH), np.float32), seq=True).numpy()
     for t in range(n_pos):
         want = OA.attend(OA.prep(qfull[t], kin[t], vin[t], qn, kn, rope, base + t, kc, vc, NROT), kc, vc, qfull[t], base + t)
         err = float(np.max(np.abs(att[t].astype(np.float64) - want)) / np.max(np.abs(want)))
@@ -210,7 +231,7 @@ def test_attention_blocks_inside_their_tensors(qk, emu, hq, hkv, base, n_pos):
 
 @pytest.mark.parametrize("name", ["f16", "f32"])
 @pytest.mark.parametrize("K,M", [(2048, 1), (2048, 9), (4096, 3), (512, 70), (768, 6)])
-def test_dense_gemv_inside_its_tensors(qk, orc, emu, name, K, M):
+def test_dense_gemv_inside_its_tensors(qk, orc, emu, name, K, M, form):
     """Dense rows: K a whole number of 64 sixteen-byte chunks takes the kernel with x in registers (the row
     after the last one is never fetched: the prefetch re-reads the last row), other K the chunk loop."""
     t = {"f16": qk.F16, "f32": qk.F32}[name]
@@ -242,7 +263,9 @@ def test_engine_in_the_host_build_and_its_memory_check(qk, emu, tmp_path, monkey
         assert eng.n_slots == 1
 
 
-def test_whole_model_stream_in_the_host_build(qk, emu, tmp_path):
+@pytest.mark.parametrize("switches", [{}, {"QK_ONE_ROW": "stream", "QK_DENSE_REG": "1", "QK_FUSED_NORM": "1", "QK_ATTN_BLOCK": "1", "QK_DN_FUSED": "1"}],
+                         ids=["defaults", "every_switch_on"])
+def test_whole_model_stream_in_the_host_build(qk, emu, tmp_path, monkeypatch, switches, switches_back_to_defaults):
     """The engine on a small whole model (one gated-DeltaNet layer, one attention layer, a MoE block each)
     through the host-side build: two slots' greedy streams -- prompts prefilled in a pass, then serial steps
     from a replayed graph -- equal the restated state machine driving the CPU oracle of the whole model,
@@ -251,6 +274,8 @@ def test_whole_model_stream_in_the_host_build(qk, emu, tmp_path):
     import sys
     sys.path.insert(0, os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle"))
     import qk_oracle_engine as OE
+    for k_, v_ in {"QK_ONE_ROW": "lane", "QK_DENSE_REG": "0", "QK_FUSED_NORM": "0", "QK_ATTN_BLOCK": "0", "QK_DN_FUSED": "0", **switches}.items():
+        monkeypatch.setenv(k_, v_)   # qk_open reads the switches that are set
     vocab = 96
     model = qk.engine.FullModel(9, kinds="RA", vocab=vocab, n_expert=8, n_ff=256, n_used=2, eos=vocab + 5)
     path = model.write(str(tmp_path / "m.gguf"))

@@ -177,8 +177,8 @@ def test_attention_sequence_forms_equal_the_steps(qk, dev, tmax, base, n_pos):
 
 @pytest.mark.parametrize("hq,hkv,base,n_pos", [(16, 2, 0, 16), (16, 2, 61, 37), (8, 1, 3, 19), (4, 4, 10, 5), (6, 2, 130, 48),
                                                 (2, 2, 0, 3)])
-def test_attention_blocks_of_sixteen_rows(qk, dev, hq, hkv, base, n_pos):
-    """Three or more consecutive rows go through the kernel that takes sixteen rows and four query heads
+def test_attention_blocks_of_sixteen_rows(qk, dev, unrun_form, hq, hkv, base, n_pos):
+    """With the "attn_block" switch three or more consecutive rows go through the kernel that takes sixteen rows and four query heads
     per workgroup (scores and values on the matrix cores): against the CPU mirror row by row, for head
     counts that fill a workgroup's four waves, leave some idle (2, 1 or 3 heads per KV head) or need two
     workgroups per KV head (8), block counts with a ragged last block, and caches that already hold rows."""
@@ -197,7 +197,8 @@ def test_attention_blocks_of_sixteen_rows(qk, dev, hq, hkv, base, n_pos):
     pos = torch.arange(base, base + n_pos, dtype=torch.int32, device=dev)
     ws = torch.empty(qk.attn_workspace_bytes(n_pos, hq), dtype=torch.uint8, device=dev)
     qh = qk.attn_prep(qfd, up(kin), up(vin), up(qn), up(kn), up(rope), pos, kd, vd, NROT, seq=True)
-    att = qk.attn_decode(qh, kd, vd, qfd, pos, ws, seq=True).cpu().numpy()
+    with qk.option("attn_block", 1):
+        att = qk.attn_decode(qh, kd, vd, qfd, pos, ws, seq=True).cpu().numpy()
     for t in range(n_pos):
         want = OA.attend(OA.prep(qfull[t], kin[t], vin[t], qn, kn, rope, base + t, kc, vc, NROT), kc, vc, qfull[t], base + t)
         assert rel(att[t], want) <= TOL, t

@@ -79,7 +79,7 @@ def test_deltanet_steps_match_the_cpu_mirror(qk, dev, n_slots, n_tok, kdiv):
     assert rel(S_gpu, S) <= TOL                  # the states after all tokens
 
 
-def test_deltanet_ab_with_the_norm_in_front(qk, orc, dev):
+def test_deltanet_ab_with_the_norm_in_front(qk, orc, dev, unrun_form):
     """qkk_dn_ab_conv_norm: x is the residual row; decay and write strength come out as from the norm
     launch followed by qkk_dn_ab_conv (to rounding) and match the oracle on the oracle's normalised row;
     the conv half is untouched (bit for bit)."""
@@ -105,7 +105,7 @@ def test_deltanet_ab_with_the_norm_in_front(qk, orc, dev):
 
 
 @pytest.mark.parametrize("n_slots,kdiv,norm", [(1, 0, False), (1, 2, True), (3, 0, True), (16, 2, False)])
-def test_deltanet_one_launch_step(qk, orc, dev, n_slots, kdiv, norm):
+def test_deltanet_one_launch_step(qk, orc, dev, unrun_form, n_slots, kdiv, norm):
     """qkk_dn_step_fused (ab + conv + step of the two value heads of a key head in one workgroup) against
     the two launches it replaces: the same arithmetic in the same order, so attention rows, conv window and
     state come out bit for bit the same, over several tokens; the first token also against the oracle."""

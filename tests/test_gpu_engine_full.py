@@ -79,23 +79,28 @@ def test_whole_model_streams(qk, full):
         print(f"[info] narrowest top-2 gap / largest logit over all steps fed: {chk.narrowest:.2e}", flush=True)
 
 
-def test_whole_model_eager_launches_and_serial_prefill(qk, full, monkeypatch):
+def test_whole_model_eager_launches_and_serial_prefill(qk, full, dev, monkeypatch, switches_back_to_defaults):
     """QK_NO_GRAPH launches the kernels one by one; QK_NO_BATCH feeds every prompt token in a serial
     step instead of at the start; QK_MAXB moves the border between prefilled and serially fed positions,
-    QK_PREFILL_ROWS sets the rows per prefill pass; QK_DN_FUSED, QK_NO_FUSED_NORM and QK_ATTN_PAIR choose
-    between kernel forms of the same step: the same streams."""
+    QK_PREFILL_ROWS sets the rows per prefill pass; QK_DN_FUSED, QK_FUSED_NORM, QK_ATTN_BLOCK and QK_ONE_ROW
+    choose between kernel forms of the same step (on a device only once those forms have had their first
+    run there): the same streams."""
+    from conftest import SWITCH_ENV_DEFAULTS, unrun_forms_allowed
     model, path = full
     print("[case] whole model, eager / serial prefill", flush=True)
     prompt = [int(t) for t in np.random.default_rng(6).integers(0, VOCAB, 18)]
     streams = []
-    for env in ({}, {"QK_NO_GRAPH": "1"}, {"QK_NO_BATCH": "1"}, {"QK_MAXB": "16"},
-                {"QK_PREFILL_ROWS": "16"},    # QK_MAXB 16: 16 positions prefilled, one serial step more; rows 16: two passes
-                {"QK_DN_FUSED": "1"},         # the gated-DeltaNet step as one launch: the same bits
-                {"QK_NO_FUSED_NORM": "1"},    # the norm as launches of its own again: the same sums scaled earlier
-                {"QK_ATTN_PAIR": "1"}):       # the prompt's attention two rows at a time
-        for k in ("QK_NO_GRAPH", "QK_NO_BATCH", "QK_MAXB", "QK_PREFILL_ROWS", "QK_DN_FUSED", "QK_NO_FUSED_NORM", "QK_ATTN_PAIR"):
+    cases = [{}, {"QK_NO_GRAPH": "1"}, {"QK_NO_BATCH": "1"}, {"QK_MAXB": "16"},
+             {"QK_PREFILL_ROWS": "16"}]    # QK_MAXB 16: 16 positions prefilled, one serial step more; rows 16: two passes
+    if unrun_forms_allowed(dev):
+        cases += [{"QK_DN_FUSED": "1"},         # the gated-DeltaNet step as one launch: the same bits
+                  {"QK_ONE_ROW": "stream", "QK_DENSE_REG": "1"},   # block rows streamed through LDS
+                  {"QK_ONE_ROW": "stream", "QK_FUSED_NORM": "1"},  # no norm launches: the same sums scaled later
+                  {"QK_ATTN_BLOCK": "1"}]       # the prompt's attention sixteen rows at a time
+    for env in cases:
+        for k in ("QK_NO_GRAPH", "QK_NO_BATCH", "QK_MAXB", "QK_PREFILL_ROWS"):
             monkeypatch.delenv(k, raising=False)
-        for k, v in env.items():
+        for k, v in {**SWITCH_ENV_DEFAULTS, **env}.items():   # qk_open applies the switches that are set
             monkeypatch.setenv(k, v)
         with qk.engine.Engine(path, n_slots=2, n_ctx=64, chunk=8) as eng:
             assert eng.slot_start(1, prompt, 6) == 0

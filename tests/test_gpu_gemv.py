@@ -4,7 +4,8 @@ scale-aware metric (<= 1e-2) is checked as well."""
 import numpy as np
 import pytest
 
-pytestmark = pytest.mark.gpu
+# every test runs on both forms of the one-row kernels (conftest.one_row_form)
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("one_row_form")]
 
 TYPES = {"q8_0": 8, "q6_k": 14, "iq4_xs": 23, "iq3_xxs": 18, "f16": 1, "f32": 0}
 TOL = 1e-3
@@ -54,7 +55,7 @@ def test_gemv_q8_0_engine_shapes(qk, orc, dev, M, K, batch):
 
 @pytest.mark.parametrize("name", ["q8_0", "q6_k", "iq4_xs", "iq3_xxs"])
 @pytest.mark.parametrize("M,batch", [(12288, 1), (9216, 1), (515, 2), (3, 1)])
-def test_gemv_with_the_norm_in_front(qk, orc, dev, name, M, batch):
+def test_gemv_with_the_norm_in_front(qk, orc, dev, unrun_form, name, M, batch):
     """qkk_gemv_norm: y = W . rmsnorm(x) * w with the norm inside the launch, against the oracle's norm
     (double) followed by its GEMV; 12288 and 9216 rows are a layer's input projections back to back."""
     import torch

@@ -3,7 +3,8 @@ the double-accumulated logits; logits within 1e-3 relative max-abs."""
 import numpy as np
 import pytest
 
-pytestmark = pytest.mark.gpu
+# every test runs on both forms of the one-row kernels (conftest.one_row_form)
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("one_row_form")]
 
 
 def head_case(qk, orc, dev, V, K, batch, seed, want_logits=True):
@@ -45,7 +46,7 @@ def test_head_ragged(qk, orc, dev, V, K, batch):
 
 
 @pytest.mark.parametrize("V", [151936, 4097, 3])
-def test_head_with_the_norm_in_front(qk, orc, dev, V):
+def test_head_with_the_norm_in_front(qk, orc, dev, unrun_form, V):
     """qkk_head_argmax_norm: the output norm inside the head's launch, against the oracle's norm (double)
     followed by its GEMV and argmax."""
     import torch

@@ -4,7 +4,8 @@ weights within 1e-4 (the reference's bar); outputs within 1e-3 relative max-abs.
 import numpy as np
 import pytest
 
-pytestmark = pytest.mark.gpu
+# every test runs on both forms of the one-row kernels (conftest.one_row_form)
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("one_row_form")]
 TOL = 1e-3
 
 

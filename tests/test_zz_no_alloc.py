@@ -8,7 +8,8 @@ point against the oracle.  Collected last: a failure here must not hide the othe
 import numpy as np
 import pytest
 
-pytestmark = pytest.mark.gpu
+# every test runs on both forms of the one-row kernels (conftest.one_row_form)
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("one_row_form")]
 
 
 def run_pair(qk, dev, layer, X):
