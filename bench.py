@@ -581,7 +581,13 @@ def extras(qk, a, steps):
     es, ew = 400, 40
     fmts = (("q8_0", qk.Q8_0), ("q6_k", qk.Q6_K), ("iq4_xs", qk.IQ4_XS), ("iq3_xxs", qk.IQ3_XXS), ("f16", qk.F16))
 
+    t_start = time.perf_counter()
+
     def run(key, fn):
+        # the BASELINE configs come first; whatever is left when the budget is spent is named, not run
+        if time.perf_counter() - t_start > a.extras_seconds:
+            ex[key] = dict(skipped=f"the extras' time budget of {a.extras_seconds} s was spent (--extras-seconds)")
+            return
         guarded(ex, key, fn)
         torch.cuda.empty_cache()
 
@@ -665,15 +671,15 @@ def extras(qk, a, steps):
     return ex
 
 
-def extras_in_child(a, timeout_s=1500):
+def extras_in_child(a, timeout_s=None):
     """Runs `--workload extras` in a child process and returns its object: the headline figure of this
     process is already measured, and whatever happens to a side measurement -- a Python error is an
     entry of the object, a process that dies or stalls is an error here -- the line still goes out."""
     import subprocess
     cmd = [sys.executable, os.path.abspath(__file__), "--workload", "extras", "--no-cpu", "--ring", str(a.ring),
-           "--steps", str(a.steps), "--warmup", str(a.warmup)] + (["--ab-forms"] if a.ab_forms else [])
+           "--steps", str(a.steps), "--warmup", str(a.warmup), "--extras-seconds", str(a.extras_seconds)] + (["--ab-forms"] if a.ab_forms else [])
     try:
-        r = subprocess.run(cmd, stdout=subprocess.PIPE, text=True, timeout=timeout_s)   # its stderr is this process's
+        r = subprocess.run(cmd, stdout=subprocess.PIPE, text=True, timeout=timeout_s or a.extras_seconds + 600)   # its stderr is this process's
         if r.returncode != 0:
             return dict(error=f"the extras process ended with status {r.returncode}")
         return json.loads(r.stdout.strip().splitlines()[-1])["extras"]
@@ -694,6 +700,8 @@ def main():
                     help="layers of the synthetic model of the engine workloads (40 = the reference model's depth, a 16 GB file)")
     ap.add_argument("--extras", dest="extras", action="store_true", default=True)
     ap.add_argument("--no-extras", dest="extras", action="store_false")
+    ap.add_argument("--extras-seconds", type=float, default=240.0,
+                    help="time budget of the side measurements; entries not reached are listed as skipped")
     ap.add_argument("--ab-forms", action="store_true",
                     help="extras: also time the one-row kernels in both forms (per-lane loads / rows streamed through LDS)")
     ap.add_argument("--copy-probe", action="store_true",

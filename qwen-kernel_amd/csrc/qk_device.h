@@ -20,6 +20,12 @@ constexpr int WAVE = 64;
 #ifndef QK_REG
 #define QK_REG(x) "+v"(x)
 #endif
+// A third hook marks the table lookups in LDS (site = a small integer, the address and width of this
+// lane's read): nothing on the device; the host-side build counts bank conflicts per wave instruction.
+#ifndef QK_LDS_PROBE
+#define QK_LDS_PROBE(site, ptr, bytes) ((void)0)
+#endif
+enum { QK_SITE_IQ3_GRID = 0, QK_SITE_IQ3_SIGN = 1, QK_SITE_IQ4_PAIR = 2, QK_SITE_IQ4_FLOAT = 3, QK_SITE_IQ3_GRID_WORD = 4 };
 
 // ---- loads -----------------------------------------------------------------------
 // GGUF blocks are 2-byte (Q8_0, Q6_K, IQ3_XXS) or 8-byte (IQ4_XS) aligned.  gfx950
@@ -408,7 +414,9 @@ struct LaneW<23> { // IQ4_XS
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const uint32_t byte = (qq[i] >> (8 * j)) & 0xFFu;
+                QK_LDS_PROBE(QK_SITE_IQ4_FLOAT, &lut[byte & 15u], 4);
                 s += lut[byte & 15u] * xs.v[i * 4 + j];
+                QK_LDS_PROBE(QK_SITE_IQ4_FLOAT, &lut[byte >> 4], 4);
                 s += lut[byte >> 4] * xs.v[16 + i * 4 + j];
             }
         }
@@ -425,7 +433,11 @@ struct LaneW<23> { // IQ4_XS
         const uint32_t qq[4] = {q.x, q.y, q.z, q.w};
         uint32_t w[16];
 #pragma unroll
-        for (int k = 0; k < 16; k++) w[k] = tab->pair[(qq[k >> 2] >> (8 * (k & 3))) & 0xFFu];
+        for (int k = 0; k < 16; k++) {
+            const uint32_t* e = &tab->pair[(qq[k >> 2] >> (8 * (k & 3))) & 0xFFu];
+            QK_LDS_PROBE(QK_SITE_IQ4_PAIR, e, 4);
+            w[k] = *e;
+        }
         __builtin_amdgcn_sched_barrier(0);
         float s0 = 0.f, s1 = 0.f;
 #pragma unroll
@@ -463,6 +475,7 @@ struct LaneW<18> { // IQ3_XXS
             const uint32_t gw = l < 2 ? g.x : g.y;
 #pragma unroll
             for (int hh = 0; hh < 2; hh++) {
+                QK_LDS_PROBE(QK_SITE_IQ3_GRID_WORD, &grid[(gw >> (16 * (l & 1) + 8 * hh)) & 0xFFu], 4);
                 const uint32_t cw = grid[(gw >> (16 * (l & 1) + 8 * hh)) & 0xFFu];
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
@@ -486,10 +499,16 @@ struct LaneW<18> { // IQ3_XXS
         uint4 sg[4];
 #pragma unroll
         for (int l = 0; l < 4; l++) {
-            sg[l] = tab->sign[(aux >> (7 * l)) & 127u];
+            const uint4* se = &tab->sign[(aux >> (7 * l)) & 127u];
+            QK_LDS_PROBE(QK_SITE_IQ3_SIGN, se, 16);
+            sg[l] = *se;
             const uint32_t gw = l < 2 ? g.x : g.y;
 #pragma unroll
-            for (int hh = 0; hh < 2; hh++) m[l * 2 + hh] = tab->grid[(gw >> (16 * (l & 1) + 8 * hh)) & 0xFFu];
+            for (int hh = 0; hh < 2; hh++) {
+                const uint2* ge = &tab->grid[(gw >> (16 * (l & 1) + 8 * hh)) & 0xFFu];
+                QK_LDS_PROBE(QK_SITE_IQ3_GRID, ge, 8);
+                m[l * 2 + hh] = *ge;
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
         float s0 = 0.f, s1 = 0.f;

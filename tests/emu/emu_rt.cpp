@@ -233,6 +233,41 @@ const uint64_t* exchange(uint64_t v)
 }
 void exchange_done() {} // the values stay valid until the wave's next operation but one
 
+// ---- LDS bank model ------------------------------------------------------------------------------
+bool g_lds_probe_on = false;
+constexpr int PROBE_SITES = 8;
+static std::atomic<uint64_t> g_probe[PROBE_SITES][3]; // wave instructions, cycles in the model, cycles without conflicts
+void lds_probe(int site, const void* p, int bytes)
+{
+    const uint32_t t = t_wg->cur->tid.x;
+    const uint64_t* all = exchange((uint64_t)(uintptr_t)p);
+    if ((t & 63u) == 0 && site >= 0 && site < PROBE_SITES) {
+        const uint32_t lanes = std::min<uint32_t>(64, g_block_dim.x - (t & ~63u));
+        const uint32_t per_pass = bytes <= 4 ? 64 : bytes == 8 ? 32 : 16, dwords = (uint32_t)(bytes + 3) / 4;
+        uint64_t cycles = 0, ideal = 0;
+        for (uint32_t l0 = 0; l0 < lanes; l0 += per_pass) {
+            uint64_t seen[64][16];
+            uint32_t n[64] = {0};
+            for (uint32_t l = l0; l < std::min(lanes, l0 + per_pass); l++)
+                for (uint32_t d = 0; d < dwords; d++) {
+                    const uint64_t dw = (all[l] >> 2) + d;
+                    const uint32_t bank = (uint32_t)(dw & 63u);
+                    bool dup = false;
+                    for (uint32_t k = 0; k < n[bank]; k++) dup = dup || seen[bank][k] == dw;
+                    if (!dup && n[bank] < 16) seen[bank][n[bank]++] = dw; // the same dword is one broadcast read
+                }
+            uint32_t worst = 1;
+            for (uint32_t b = 0; b < 64; b++) worst = std::max(worst, n[b]);
+            cycles += worst;
+            ideal += 1;
+        }
+        g_probe[site][0]++;
+        g_probe[site][1] += cycles;
+        g_probe[site][2] += ideal;
+    }
+    exchange_done();
+}
+
 // Helper threads that live as long as the process (QK_EMU_THREADS, default the host's cores, minus the caller).
 struct Pool {
     unsigned size = 0;
@@ -393,6 +428,18 @@ hipError_t hipFree(void* p)
 
 // C entry points for the tests: buffers that end at a guard page.
 extern "C" {
+void emu_lds_probe_enable(int on)
+{
+    emu::g_lds_probe_on = on != 0;
+    if (on)
+        for (auto& site : emu::g_probe)
+            for (auto& v : site) v = 0;
+}
+// out[0..2] = wave instructions, modelled cycles, conflict-free cycles of the lookups marked `site`
+void emu_lds_probe_read(int site, uint64_t* out)
+{
+    for (int i = 0; i < 3; i++) out[i] = site >= 0 && site < emu::PROBE_SITES ? emu::g_probe[site][i].load() : 0;
+}
 void* emu_guard_alloc(size_t n, size_t align, void** handle)
 {
     auto* g = new emu::GuardBuf(n ? n : 16, align < 16 ? 16 : align);

@@ -31,6 +31,8 @@
 // the kernels' hooks (qk_device.h): dynamic LDS comes from the launch, register pins become memory pins
 #define QK_DYN_LDS(type, name) type* name = (type*)emu::dyn_lds()
 #define QK_REG(x) "+m"(x)
+// table lookups in LDS report this lane's address and width; the runtime models the banks (below)
+#define QK_LDS_PROBE(site, ptr, bytes) do { if (emu::g_lds_probe_on) emu::lds_probe(site, ptr, bytes); } while (0)
 
 struct uint2 { uint32_t x, y; };
 struct __attribute__((aligned(16))) uint4 { uint32_t x, y, z, w; };
@@ -66,6 +68,12 @@ void wave_barrier();
 const uint64_t* exchange(uint64_t v);
 void exchange_done();
 void run(dim3 grid, dim3 block, size_t lds, const std::function<void()>& body);
+// LDS bank model for marked lookups (off unless a test switches it on): a wave instruction's addresses
+// are gathered from its lanes, and it costs, pass by pass (64 lanes of 4 bytes, 32 of 8, 16 of 16), the
+// largest number of distinct dwords that any of the 64 four-byte banks is asked for; a conflict-free
+// pass costs 1.  A proxy for the device's LDS, not a measurement of it.
+extern bool g_lds_probe_on;
+void lds_probe(int site, const void* p, int bytes);
 // Stream capture: between hipStreamBeginCapture and hipStreamEndCapture (per host thread) launches,
 // copies and fills are recorded instead of run; a graph is the recorded list, a launch of it runs
 // the list in order.  submit() runs `op` now, or records it while the calling thread captures.

@@ -373,3 +373,90 @@ def test_deltanet_step_inside_its_tensors(qk, emu, fused):
         g, b = OD.ab(x[s], alpha_w, beta_w, dt_bias, a_vec)
         want = OD.step(OD.conv(st[s].copy(), qkv[s], ker, DS, QK), g, b, S[s].copy(), norm_w, z[s], HK, HV)
         assert float(np.max(np.abs(att.numpy()[s] - want)) / np.max(np.abs(want))) <= 1e-3, s
+
+
+SITES = ["iq3_grid", "iq3_sign", "iq4_pair", "iq4_float", "iq3_grid_word"]
+
+
+def _lds_lookup_cycles(qk, emu, run):
+    """Runs `run()` with the host-side build's LDS bank model on and returns, per marked lookup site,
+    (wave instructions, modelled cycles per instruction, conflict-free cycles per instruction)."""
+    import ctypes as C
+    L = emu_util.emu_lib(qk)
+    L.emu_lds_probe_read.argtypes = [C.c_int, C.POINTER(C.c_uint64)]
+    L.emu_lds_probe_enable(1)
+    try:
+        run()
+    finally:
+        L.emu_lds_probe_enable(0)
+    out = {}
+    for site, name in enumerate(SITES):
+        v = (C.c_uint64 * 3)()
+        L.emu_lds_probe_read(site, v)
+        if v[0]:
+            out[name] = (int(v[0]), v[1] / v[0], v[2] / v[0])
+    return out
+
+
+def _model_cycles(entries, entry_bytes, copies, rng, trials=400):
+    """The same bank model for a table of `entries` entries in `copies` copies, copy r confined to its own
+    64 / copies banks and read by the lanes with lane mod copies = r: mean cycles per wave instruction of 64
+    random lookups."""
+    per_pass = {4: 64, 8: 32, 16: 16}[entry_bytes]
+    dw, banks_per_copy = entry_bytes // 4, 64 // copies
+    slots = max(1, banks_per_copy // dw)          # entries of one copy per 256-byte row
+    total = 0
+    for _ in range(trials):
+        e = rng.integers(0, entries, 64)
+        for l0 in range(0, 64, per_pass):
+            seen = {}
+            for lane in range(l0, l0 + per_pass):
+                r = lane % copies
+                row, slot = divmod(int(e[lane]), slots)
+                for d in range(dw):
+                    bank = r * banks_per_copy + (slot * dw + d) % banks_per_copy
+                    seen.setdefault(bank, set()).add((row, d))
+            total += max(len(v) for v in seen.values())
+    return total / trials
+
+
+def test_lds_bank_model_of_the_table_lookups(qk, orc, emu, capsys):
+    """A PROXY for the device's LDS, not a measurement (64 banks of four bytes; a pass of 64 / 32 / 16 lanes for
+    4 / 8 / 16-byte reads costs the largest number of distinct dwords any bank is asked for).  Counted on the GEMVs
+    in the host-side build, per wave instruction:
+      * the streamed IQ3_XXS product reads 8-byte codebook entries at about three times, and 16-byte sign entries at
+        nearly three times, their conflict-free cost (device counters on the same loop: 58 % of the LDS cycles were
+        bank conflicts); the streamed IQ4_XS pair table at three to four times;
+      * the per-lane IQ4_XS product reads a 16-entry float codebook, whose entries lie in 16 different banks: no
+        conflicts at all, twice the lookups -- one reason why that form measured faster for IQ4_XS;
+      * copies of a table in bank groups of their own do not help until every lane of a pass has a group to itself:
+        8 copies of the codebook still cost nearly three passes, because a wave instruction waits for its worst bank;
+        only 32 copies (64 KB for 256 entries of 8 bytes) are conflict-free -- more LDS than the streaming loop can
+        give up without losing the occupancy that hides its latency."""
+    M, K = 64, 2048
+    x = np.random.default_rng(4).standard_normal((1, K)).astype(np.float32)
+    got = {}
+    for name, form in (("iq3_xxs", 1), ("iq4_xs", 1), ("iq3_xxs", 0), ("iq4_xs", 0)):
+        t = type_id(qk, name)
+        W = qk.synth.tensor_host(t, M, K, seed=3)
+        Wd, Xd, Yd = emu.tensor(W.reshape(-1)), emu.tensor(x), emu.zeros((1, M), np.float32)
+        with qk.option("one_row", form):
+            got[name, form] = _lds_lookup_cycles(qk, emu, lambda: qk.gemv(t, Wd, Xd, M, K, out=Yd))
+        assert orc.rel_maxabs_err(Yd.numpy()[0], orc.gemv(t, W, x[0], M, K)) <= 1e-3
+    with capsys.disabled():
+        print(f"\n[lds model] (instructions, cycles each, conflict-free cycles each): {got}", flush=True)
+    n, c, i = got["iq3_xxs", 1]["iq3_grid"]
+    assert n == M * 8 and i == 2 and 2.5 <= c / i <= 4.0          # 8 lookups per 32 weights, 64 rows of one wave each
+    n, c, i = got["iq3_xxs", 1]["iq3_sign"]
+    assert n == M * 4 and i == 4 and 2.0 <= c / i <= 4.0
+    n, c, i = got["iq4_xs", 1]["iq4_pair"]
+    assert n == M * 16 and i == 1 and 2.5 <= c / i <= 5.0
+    n, c, i = got["iq4_xs", 0]["iq4_float"]
+    assert n == M * 32 and c == i == 1                             # 16 entries in 16 banks: never a conflict
+    n, c, i = got["iq3_xxs", 0]["iq3_grid_word"]
+    assert n == M * 8 and i == 1 and 2.5 <= c / i <= 5.0
+    # what copies per bank group would buy, in the same model
+    rng = np.random.default_rng(0)
+    one, eight, thirty_two = (_model_cycles(256, 8, r, rng) for r in (1, 8, 32))
+    assert abs(one - got["iq3_xxs", 1]["iq3_grid"][1]) < 0.5        # the model in Python agrees with the counted kernel
+    assert eight > 0.85 * one and thirty_two == 2.0
