@@ -127,6 +127,7 @@ struct qk_engine {
     bool open(const char* path, const qk_config& cfg, char* err, size_t err_len);
     bool upload(const qkg_tensor& t, const void** out, char* err, size_t err_len);
     void* dev_alloc(size_t bytes, bool zero);
+    void dev_free(const void* p); // a staging buffer of qk_open that nothing refers to any more
     int launch_rows(uint32_t rows, float** final_rows);
     int launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool want_head, bool seq);
     int prefill(uint32_t slot, const uint32_t* toks, uint32_t n, uint32_t base, uint32_t* ids_out);
@@ -162,6 +163,16 @@ qk_engine::~qk_engine()
 }
 
 // Device memory the engine owns until it closes, 256 spare bytes behind it; nullptr on failure.
+void qk_engine::dev_free(const void* p)
+{
+    for (size_t i = 0; i < dev_allocs.size(); i++)
+        if (dev_allocs[i] == p) {
+            (void)hipFree(dev_allocs[i]);
+            dev_allocs.erase(dev_allocs.begin() + (long)i);
+            return;
+        }
+}
+
 void* qk_engine::dev_alloc(size_t bytes, bool zero)
 {
     void* p = nullptr;
@@ -493,6 +504,9 @@ bool qk_engine::load_mixers(qkg_file* g, char* err, size_t err_len)
                 return set_err(err, err_len, "qk_open: upload failed");
         }
         if (hipStreamSynchronize(st) != hipSuccess) return set_err(err, err_len, "qk_open: upload failed");
+        // the copies are complete: the fused tensor and its dequantised form are not needed again
+        if (rows != (const float*)raw) dev_free(rows);
+        dev_free(raw);
         *alpha = al; *beta = be;
         return true;
     };
