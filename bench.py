@@ -11,7 +11,10 @@ decode do), captured in a HIP graph; inputs are resident in HBM before the timed
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--ring R]
                   [--extras/--no-extras] [--cpu/--no-cpu]
 
-Prints ONE JSON line.  --gpus above 1 is refused: this build drives one GPU.
+Prints ONE JSON line.  --gpus above 1 is refused: this build drives one GPU.  The default run is three
+parts -- the headline workload and the side measurements (`extras`) in a child process each, the CPU baseline
+in this one -- so no side measurement can take the headline with it; with --no-extras, or any other
+--workload, everything runs in this process (the form to put behind `rocprofv3 ... --`).
 """
 import argparse
 import json
@@ -430,14 +433,15 @@ def engine_workload(qk, n_layer, slots_list, chunks, warm_chunks, seed=31, kinds
     return res
 
 
-def guarded(ex, key, fn):
+def guarded(ex, key, fn, quiet=False):
     """Runs one extra measurement; a Python-level failure becomes an entry of the line instead of ending the run
     (the headline figure is already measured by then)."""
     try:
         ex[key] = fn()
     except Exception as e:   # noqa: BLE001 -- whatever it is, the line still goes out
         ex[key] = dict(error=f"{type(e).__name__}: {e}")
-    log(f"[bench] {key}: {ex[key]}")
+    if not quiet or "error" in ex[key]:
+        log(f"[bench] {key}: {ex[key]}")
 
 
 def host_threads():
@@ -671,20 +675,31 @@ def extras(qk, a, steps):
     return ex
 
 
-def extras_in_child(a, timeout_s=None):
-    """Runs `--workload extras` in a child process and returns its object: the headline figure of this
-    process is already measured, and whatever happens to a side measurement -- a Python error is an
-    entry of the object, a process that dies or stalls is an error here -- the line still goes out."""
+def run_child(argv, timeout_s):
+    """Runs this file with `argv` as a child process and returns the object of its JSON line (its stderr
+    is this process's)."""
     import subprocess
-    cmd = [sys.executable, os.path.abspath(__file__), "--workload", "extras", "--no-cpu", "--ring", str(a.ring),
-           "--steps", str(a.steps), "--warmup", str(a.warmup), "--extras-seconds", str(a.extras_seconds)] + (["--ab-forms"] if a.ab_forms else [])
+    r = subprocess.run([sys.executable, os.path.abspath(__file__)] + argv, stdout=subprocess.PIPE, text=True, timeout=timeout_s)
+    if r.returncode != 0:
+        raise RuntimeError(f"`bench.py {' '.join(argv)}` ended with status {r.returncode}")
+    return json.loads(r.stdout.strip().splitlines()[-1])
+
+
+def headline_and_extras(a):
+    """The default run as three parts: the headline workload in a child process, the side measurements in
+    a second one, the CPU baseline here.  This process never touches the GPU, so starting the children is
+    an ordinary process start, and whatever happens to a side measurement -- a Python error is an entry
+    of `extras`, a child that dies or stalls an error for the whole object -- the headline line goes out."""
+    common = ["--ring", str(a.ring), "--steps", str(a.steps), "--warmup", str(a.warmup)]
     try:
-        r = subprocess.run(cmd, stdout=subprocess.PIPE, text=True, timeout=timeout_s or a.extras_seconds + 600)   # its stderr is this process's
-        if r.returncode != 0:
-            return dict(error=f"the extras process ended with status {r.returncode}")
-        return json.loads(r.stdout.strip().splitlines()[-1])["extras"]
-    except Exception as e:   # noqa: BLE001
-        return dict(error=f"{type(e).__name__}: {e}")
+        out = run_child(["--workload", a.workload, "--no-extras", "--no-cpu"] + common, 900)
+    except Exception as e:   # noqa: BLE001 -- no headline, no line
+        sys.exit(f"bench.py: the headline workload did not complete: {type(e).__name__}: {e}")
+    ex_args = ["--workload", "extras", "--no-cpu", "--extras-seconds", str(a.extras_seconds)] + common + (["--ab-forms"] if a.ab_forms else [])
+    guarded(out, "extras", lambda: run_child(ex_args, a.extras_seconds + 600)["extras"], quiet=True)
+    if a.cpu:
+        guarded(out, "cpu_baseline", lambda: cpu_baseline(entry.load_package(), entry.load_oracle()))
+    print(json.dumps(out), flush=True)
 
 
 def main():
@@ -712,6 +727,8 @@ def main():
     if a.gpus != 1:
         sys.exit("bench.py: this build drives ONE GPU (one process, one device); "
                  "--gpus N with N > 1 is not supported")
+    if a.workload == "moe_decode_bs1" and a.extras:
+        return headline_and_extras(a)
     import torch
     qk = entry.load_package()
     if not torch.cuda.is_available():
@@ -842,8 +859,6 @@ def main():
     del m
     torch.cuda.empty_cache()
 
-    if a.extras and a.workload == "moe_decode_bs1":
-        out["extras"] = extras_in_child(a)
     if a.cpu:
         guarded(out, "cpu_baseline", lambda: cpu_baseline(qk, entry.load_oracle()))
     print(json.dumps(out), flush=True)

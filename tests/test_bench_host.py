@@ -12,6 +12,19 @@ def test_more_than_one_gpu_is_refused():
     assert r.returncode != 0 and "ONE GPU" in r.stderr and not r.stdout.strip()
 
 
+def test_default_run_without_a_device_says_so():
+    """The real process tree of the default run on a host without a GPU: the headline child reports the missing
+    device, the parent ends with a message and prints no line (there is no CPU path to fall back on)."""
+    import torch
+    if torch.cuda.is_available():
+        import pytest
+        pytest.skip("a device is present")
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--steps", "20", "--warmup", "5"], capture_output=True, text=True,
+                       timeout=300)
+    assert r.returncode != 0 and not r.stdout.strip()
+    assert "no HIP device" in r.stderr and "headline workload did not complete" in r.stderr
+
+
 def test_cpu_baseline_line(qk, orc):
     """Every BASELINE config has a one-thread and an all-threads figure, the thread count is stated and
     the headline entry is the fused MoE step; the object goes into the JSON line as it is."""
@@ -92,8 +105,19 @@ def _bench_with_stub_workloads(monkeypatch, qk):
     monkeypatch.setattr(bench, "engine_workload", lambda *a, **k: dict(config=dict(layers=8), slots_1=dict(tok_per_s=1.0, prefill_tok_per_s=1.0),
                                                                       slots_16=dict(tok_per_s=2.0)))
     monkeypatch.setattr(bench, "cpu_baseline", lambda qk_, orc_: dict(value=0.5, unit="GB/s", cores=8, kind="port", sample="stub", per_config={}))
-    # the side measurements run in a child process; here in this one, on the stubs
-    monkeypatch.setattr(bench, "extras_in_child", lambda a: bench.extras(qk, a, max(a.ring, a.steps // a.ring * a.ring)))
+    # the default run starts a child process per part; here the parts run in this process, on the stubs
+    def child(argv, timeout_s):
+        import contextlib
+        import io
+        saved, buf = sys.argv, io.StringIO()
+        sys.argv = ["bench.py"] + argv
+        try:
+            with contextlib.redirect_stdout(buf):
+                bench.main()
+        finally:
+            sys.argv = saved
+        return json.loads(buf.getvalue().strip().splitlines()[-1])
+    monkeypatch.setattr(bench, "run_child", child)
     return bench
 
 
