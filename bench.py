@@ -550,7 +550,7 @@ def qk_env():
 
 def kernel_forms(qk):
     """The library's switches as they stand (which form of each kernel the figures belong to)."""
-    return {n: qk.get_option(n) for n in ("one_row", "dense_reg", "fused_norm", "attn_block", "dn_fused")}
+    return {n: qk.get_option(n) for n in ("one_row", "dense_reg", "fused_norm", "attn_block", "dn_fused", "gemm_tiled")}
 
 
 def rate(bytes_step, ms, **more):
@@ -669,6 +669,9 @@ def extras(qk, a, steps):
                 run(f"{form}:moe_decode_bs1", lambda: stages(moe_workload(qk, 1, qk.IQ4_XS, a.ring, min(steps, 800), a.warmup)))
                 run(f"{form}:moe_decode_bs1_cache_hot", lambda: stages(moe_workload(qk, 1, qk.IQ4_XS, 1, 400, 40)))
                 run(f"{form}:moe_decode_4_rows_q6k_down", lambda: dict(us=moe_workload(qk, 4, qk.Q6_K, 8, 400, 40)["ms_event"] * 1e3))
+    if a.ab_forms:   # the prefill product with every weight tile decoded once per 128 rows, beside the default above
+        with qk.option("gemm_tiled", 1):
+            run("gemm_tiled:prefill_gemm_q8_0_8192x2048x128", lambda: gemm_entry(qk))
     run("engine_decode_8_layers", lambda: engine_workload(qk, 8, (1, 4, 16), 8, 2))
     # a whole model: three gated-DeltaNet layers and one full-attention layer, twice (positions 1..320)
     run("engine_decode_whole_model_8_layers", lambda: engine_workload(qk, 8, (1, 16), 8, 2, kinds="RRRARRRA"))

@@ -92,6 +92,8 @@ int qkk_device_info(char *arch_host, size_t arch_len, uint32_t *n_cu_host);
  *   "fused_norm"  1: the engine's one-row step folds each RMS norm into its consumer
  *   "attn_block"  1: prefill attention over blocks of 16 rows on the matrix cores
  *   "dn_fused"    1: the gated-DeltaNet decode step as one launch
+ *   "gemm_tiled"  1: products with 64 and more activation rows (qkk_gemm_q8_0, qkk_gemv) decode every
+ *                 weight tile once per 128 rows instead of once per 32
  *   "gemv_depth", "head_depth", "rowwise_max": launch-shape sweeps, 0 = built-in value
  * The default of every switch is the form that has been run and timed on a device.
  * Returns QKK_EINVAL for an unknown name or a value outside the switch's range. */

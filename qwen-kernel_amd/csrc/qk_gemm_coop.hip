@@ -110,9 +110,13 @@ static bool launch_k(const uint8_t* W, const float* X, float* Y, uint32_t M, uin
     }
 }
 
+bool tiled_gemm_launch(int type, const uint8_t* W, const float* X, float* Y, uint32_t M, uint32_t K, uint32_t N, hipStream_t st); // qk_gemm_tiled.hip
+
 bool coop_gemm_launch(int type, const uint8_t* W, const float* X, float* Y, uint32_t M, uint32_t K, uint32_t N,
                       hipStream_t st)
 {
+    // the "gemm_tiled" switch: 64 rows and more through the kernel that decodes every weight tile once per 128 rows
+    if (options().gemm_tiled && tiled_gemm_launch(type, W, X, Y, M, K, N, st)) return true;
     // the stream copies whole 16-byte pieces: the tensor must end on one
     if (((uint64_t)M * qkk_row_bytes(type, K)) % 16) return false;
     switch (type) {

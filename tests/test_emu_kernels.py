@@ -27,7 +27,7 @@ def form(request, qk, emu):
         yield request.param
 
 
-SWITCHES = ("one_row", "dense_reg", "fused_norm", "attn_block", "dn_fused", "gemv_depth", "head_depth", "rowwise_max")
+SWITCHES = ("one_row", "dense_reg", "fused_norm", "attn_block", "dn_fused", "gemm_tiled", "gemv_depth", "head_depth", "rowwise_max")
 
 
 @pytest.fixture
@@ -263,7 +263,7 @@ def test_engine_in_the_host_build_and_its_memory_check(qk, emu, tmp_path, monkey
         assert eng.n_slots == 1
 
 
-@pytest.mark.parametrize("switches", [{}, {"QK_ONE_ROW": "stream", "QK_DENSE_REG": "1", "QK_FUSED_NORM": "1", "QK_ATTN_BLOCK": "1", "QK_DN_FUSED": "1"}],
+@pytest.mark.parametrize("switches", [{}, {"QK_ONE_ROW": "stream", "QK_DENSE_REG": "1", "QK_FUSED_NORM": "1", "QK_ATTN_BLOCK": "1", "QK_DN_FUSED": "1", "QK_GEMM_TILED": "1"}],
                          ids=["defaults", "every_switch_on"])
 def test_whole_model_stream_in_the_host_build(qk, emu, tmp_path, monkeypatch, switches, switches_back_to_defaults):
     """The engine on a small whole model (one gated-DeltaNet layer, one attention layer, a MoE block each)
@@ -274,7 +274,7 @@ def test_whole_model_stream_in_the_host_build(qk, emu, tmp_path, monkeypatch, sw
     import sys
     sys.path.insert(0, os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle"))
     import qk_oracle_engine as OE
-    for k_, v_ in {"QK_ONE_ROW": "lane", "QK_DENSE_REG": "0", "QK_FUSED_NORM": "0", "QK_ATTN_BLOCK": "0", "QK_DN_FUSED": "0", **switches}.items():
+    for k_, v_ in {"QK_ONE_ROW": "lane", "QK_DENSE_REG": "0", "QK_FUSED_NORM": "0", "QK_ATTN_BLOCK": "0", "QK_DN_FUSED": "0", "QK_GEMM_TILED": "0", **switches}.items():
         monkeypatch.setenv(k_, v_)   # qk_open reads the switches that are set
     vocab = 96
     model = qk.engine.FullModel(9, kinds="RA", vocab=vocab, n_expert=8, n_ff=256, n_used=2, eos=vocab + 5)
@@ -315,6 +315,48 @@ def test_q8_0_gemm_inside_its_tensors(qk, orc, emu, M, K, N):
     qk.gemm_q8_0(emu.tensor(W.reshape(-1)), emu.tensor(X), M, K, out=Y)
     want = orc.gemm_q8_0(W, X, M, K)
     assert orc.rel_maxabs_err(Y.numpy(), want) <= 1e-3
+
+
+@pytest.mark.parametrize("name", QUANT)
+@pytest.mark.parametrize("M,K,N", [(32, 256, 64), (50, 512, 130), (17, 2048, 128), (96, 768, 200)])
+def test_tiled_gemm_inside_its_tensors(qk, orc, emu, name, M, K, N):
+    """The product for 64 and more activation rows with every weight tile decoded once per 128 rows (the
+    "gemm_tiled" switch), all four block formats: weight row counts that leave the last 32-row block partial,
+    activation row counts that leave waves idle or half full, row lengths whose fragments start anywhere
+    inside a 16-byte piece, the tensor ending at the guard page; against the oracle's double-precision rows
+    and against the cooperative stream (the default)."""
+    t = type_id(qk, name)
+    if (M * qk.row_bytes(t, K)) % 16:
+        pytest.skip("the tensor does not end on a 16-byte boundary: neither matrix-core kernel takes it")
+    W = qk.synth.tensor_host(t, M, K, seed=M + N)
+    X = np.random.default_rng(N).standard_normal((N, K)).astype(np.float32)
+    Wd, Xd = emu.tensor(W.reshape(-1)), emu.tensor(X)
+    Y0, Y1 = emu.zeros((N, M), np.float32), emu.zeros((N, M), np.float32)
+    qk.gemv(t, Wd, Xd, M, K, out=Y0)
+    with qk.option("gemm_tiled", 1):
+        qk.gemv(t, Wd, Xd, M, K, out=Y1)
+    want = np.stack([orc.gemv(t, W, X[n], M, K) for n in range(N)])
+    assert orc.rel_maxabs_err(Y1.numpy(), want) <= 1e-3
+    assert orc.rel_maxabs_err(Y1.numpy(), Y0.numpy()) <= 1e-5   # both keep operands exact to 2^-22: rounding of the sums only
+    assert not np.array_equal(Y0.numpy(), np.zeros_like(Y0.numpy()))
+
+
+def test_tiled_gemm_is_the_q8_0_prefill_product(qk, orc, emu):
+    """qkk_gemm_q8_0 with the switch: the reference's acceptance bar (max error below 2e-3 of the result's
+    rms, src/main.cpp:5659-5662) and the per-element bar; fewer than 64 rows keep the cooperative stream."""
+    M, K, N = 64, 1024, 128
+    W = qk.synth.tensor_host(qk.Q8_0, M, K, seed=9)
+    X = np.random.default_rng(1).standard_normal((N, K)).astype(np.float32)
+    Wd, Xd = emu.tensor(W.reshape(-1)), emu.tensor(X)
+    with qk.option("gemm_tiled", 1):
+        Y = emu.zeros((N, M), np.float32)
+        qk.gemm_q8_0(Wd, Xd, M, K, out=Y)
+        Ys = emu.zeros((40, M), np.float32)
+        qk.gemm_q8_0(Wd, emu.tensor(X[:40]), M, K, out=Ys)
+    want = orc.gemm_q8_0(W, X, M, K)
+    err = np.abs(Y.numpy().astype(np.float64) - want)
+    assert err.max() < 2e-3 * np.sqrt(np.mean(want ** 2)) and orc.rel_maxabs_err(Y.numpy(), want) <= 1e-3
+    assert orc.rel_maxabs_err(Ys.numpy(), want[:40]) <= 1e-3
 
 
 def _oracle_module(name):

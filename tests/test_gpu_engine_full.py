@@ -96,7 +96,8 @@ def test_whole_model_eager_launches_and_serial_prefill(qk, full, dev, monkeypatc
         cases += [{"QK_DN_FUSED": "1"},         # the gated-DeltaNet step as one launch: the same bits
                   {"QK_ONE_ROW": "stream", "QK_DENSE_REG": "1"},   # block rows streamed through LDS
                   {"QK_ONE_ROW": "stream", "QK_FUSED_NORM": "1"},  # no norm launches: the same sums scaled later
-                  {"QK_ATTN_BLOCK": "1"}]       # the prompt's attention sixteen rows at a time
+                  {"QK_ATTN_BLOCK": "1"},       # the prompt's attention sixteen rows at a time
+                  {"QK_GEMM_TILED": "1"}]       # (passes of 64 rows and more only: here the same kernels)
     for env in cases:
         for k in ("QK_NO_GRAPH", "QK_NO_BATCH", "QK_MAXB", "QK_PREFILL_ROWS"):
             monkeypatch.delenv(k, raising=False)
@@ -137,12 +138,18 @@ def test_whole_model_stage_run_and_snapshots(qk, full):
         assert eng.state_save(1, 3, 0) == -1 and eng.state_load(2, 0, 0) == -1
 
 
-def test_whole_model_long_prompt_and_long_stage_run(qk, full, monkeypatch):
+@pytest.mark.parametrize("tiled", [False, True], ids=["defaults", "gemm_tiled"])
+def test_whole_model_long_prompt_and_long_stage_run(qk, full, dev, monkeypatch, switches_back_to_defaults, tiled):
     """A prompt longer than one prefill pass (64 positions here go through the projections and the
     MoE blocks together, the mixers through their sequence kernels), then two more passes, then the
     serial steps: the same stream as the oracle fed one token at a time.  qk_stage_run over 40
-    positions returns the oracle's id after every one of them."""
+    positions returns the oracle's id after every one of them.  With the "gemm_tiled" switch the passes
+    of 64 rows run their dense projections through the kernel that decodes a weight tile once per 128 rows."""
+    from conftest import UNRUN, unrun_forms_allowed
+    if tiled and not unrun_forms_allowed(dev):
+        pytest.skip(UNRUN)
     model, path = full
+    monkeypatch.setenv("QK_GEMM_TILED", "1" if tiled else "0")
     monkeypatch.setenv("QK_PREFILL_ROWS", "64")
     print("[case] whole model, 150-token prompt and a 40-position stage run", flush=True)
     rng = np.random.default_rng(21)

@@ -103,6 +103,29 @@ def test_gemm_q8_0(qk, orc, dev, M, K, N):
     assert orc.rel_maxabs_err(Y, want) <= 1e-3
 
 
+@pytest.mark.parametrize("name,M,K,N", [("q8_0", 8192, 2048, 128), ("q8_0", 4096, 4096, 200), ("q6_k", 2048, 2048, 128), ("iq4_xs", 2048, 512, 300),
+                                        ("iq3_xxs", 1000, 2048, 64), ("q8_0", 50, 256, 1024)])
+def test_gemm_with_every_weight_tile_decoded_once(qk, orc, dev, unrun_form, name, M, K, N):
+    """The "gemm_tiled" switch: 64 and more activation rows through the kernel that owns 32 weight rows and
+    128 activation rows per workgroup, against the oracle's double-precision product (the reference's bar for
+    its half-precision tiles, src/main.cpp:5659-5662, and the per-element bar) and against the cooperative
+    stream; the BASELINE shape of the prefill chunk first."""
+    import torch
+    print(f"[case] tiled gemm {name} M={M} K={K} N={N}", flush=True)
+    t = {"q8_0": qk.Q8_0, "q6_k": qk.Q6_K, "iq4_xs": qk.IQ4_XS, "iq3_xxs": qk.IQ3_XXS}[name]
+    W = qk.synth.tensor_host(t, M, K, seed=7)
+    X = np.random.default_rng(8).uniform(-1, 1, (N, K)).astype(np.float32)
+    Wd, Xd = torch.from_numpy(W).to(dev), torch.from_numpy(X).to(dev)
+    base = qk.gemv(t, Wd, Xd, M, K).cpu().numpy()
+    with qk.option("gemm_tiled", 1):
+        Y = (qk.gemm_q8_0(Wd, Xd, M, K) if t == qk.Q8_0 else qk.gemv(t, Wd, Xd, M, K)).cpu().numpy()
+    rows = range(N) if N * M <= 1 << 18 else list(range(0, N, max(1, N // 24))) + [N - 1]   # the oracle is a scalar loop
+    want = np.stack([orc.gemv(t, W, X[n], M, K) for n in rows])
+    assert orc.max_err_over_rms(Y[list(rows)], want) < 2e-3
+    assert orc.rel_maxabs_err(Y[list(rows)], want) <= 1e-3
+    assert orc.rel_maxabs_err(Y, base) <= 1e-5
+
+
 def test_gemm_q8_0_matches_gemv_rows(qk, dev):
     """The GEMM and the GEMV read the same blocks: row by row they agree to fp16-weight rounding."""
     import torch
