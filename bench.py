@@ -32,7 +32,8 @@ MIN_REPLAYS = 20   # graph replays timed at least, whatever --steps says (steps 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by what the same
 # counters read for a plain 256 MiB copy (profiles/); None where no counter run of the CURRENT kernel
 # has been recorded (a figure of an earlier version of a kernel is not carried over).
-TRAFFIC = {"moe_gateup_fused_kernel": 85845150}   # profiles/moe_decode_bs16_hbm_traffic.txt (103 distinct experts)
+TRAFFIC = {"moe_gateup_fused_kernel": 85845150,   # profiles/moe_decode_bs16_hbm_traffic.txt (103 distinct experts)
+           "moe_gateup_kernel": 6722843}          # profiles/moe_decode_bs1_hbm_traffic.txt: the per-lane form (the default)
 
 
 def log(*a):
@@ -842,7 +843,9 @@ def main():
                     "moe_prefill_128": ("moe_gateup_mfma_kernel", "routed IQ3_XXS gate/up + SiLU; the stage time also "
                                         "covers the shared expert's launch on the side stream")}[a.workload]
     roof = dict(bound="hbm", kernel=f"{kname} ({kwhat})", achieved=ach,
-                peak=HBM_PEAK_GBPS, unit="GB/s", frac=ach / HBM_PEAK_GBPS, traffic=TRAFFIC.get(kname),
+                peak=HBM_PEAK_GBPS, unit="GB/s", frac=ach / HBM_PEAK_GBPS,
+                # the counter run is of the per-lane form of the one-row kernel; the streamed form has none yet
+                traffic=TRAFFIC.get(kname) if not (a.workload == "moe_decode_bs1" and qk.get_option("one_row")) else None,
                 bytes_per_launch=m["gateup_bytes"], us_per_launch=gu_ms * 1e3)
     out = dict(metric="fused_moe_decode_step_hbm_gbps", value=gbps, unit="GB/s", n_gpus=1, steps=a.steps,
                warmup=a.warmup, ms_per_step=m["ms_wall"], higher_is_better=True, scaling="weak", vs_baseline=None,
