@@ -200,7 +200,9 @@ __global__ __launch_bounds__(64 * ROUTE_WAVES) void moe_route_kernel(const float
 // and go through the wave's LDS area one after the other.  IQ3_XXS rows of H = 2048*PASSES weights;
 // the product runs on packed halves (two LDS lookups and two XORs per four weights, v_dot2_f32_f16
 // against the activations split into hi + lo halves).  NORM: the RMS norm in front, as in launch 1.
-template <int PASSES, int RPW, bool ROWS, bool NORM>
+// RANKED: the selection by all four waves with select_block (ranks by counting) instead of select_wave's
+// rounds on wave 0.
+template <int PASSES, int RPW, bool ROWS, bool NORM, bool RANKED>
 __global__ __launch_bounds__(256) void moe_gateup_kernel(const uint8_t* __restrict__ gate_exps,
                                                          const uint8_t* __restrict__ up_exps,
                                                          const float* __restrict__ x, MoeWs ws,
@@ -225,7 +227,12 @@ __global__ __launch_bounds__(256) void moe_gateup_kernel(const uint8_t* __restri
     // round trip 1: codebook word, logits (wave 0), activation slice
     const uint32_t grid_word = g_iq3xxs_grid[threadIdx.x];
     float lv[QKK_MAX_EXPERTS / 64 + 1];
-    if (wave == 0) {
+    float l0 = 0.f, l1 = 0.f, lsh = 0.f;
+    if constexpr (RANKED) { // thread t: experts t and t + 256; thread 0 also the shared gate's logit
+        l0 = threadIdx.x < d.E ? ws.logits[threadIdx.x] : 0.f;
+        l1 = threadIdx.x + 256u < d.E ? ws.logits[threadIdx.x + 256u] : 0.f;
+        lsh = threadIdx.x == 0 ? ws.logits[d.E] : 0.f;
+    } else if (wave == 0) {
 #pragma unroll
         for (int i = 0; i <= (int)(QKK_MAX_EXPERTS / 64); i++)
             lv[i] = (uint32_t)(lane + 64 * i) <= d.E ? ws.logits[lane + 64 * i] : 0.f;
@@ -252,7 +259,10 @@ __global__ __launch_bounds__(256) void moe_gateup_kernel(const uint8_t* __restri
     }
 
     fill_iq3_half_entry(tab, threadIdx.x, grid_word);
-    if (wave == 0) {
+    if constexpr (RANKED) {
+        __shared__ SelectScratch s_scr;
+        select_block(l0, l1, lsh, d.E, d.k, &s_sel, s_scr);
+    } else if (wave == 0) {
 #pragma unroll
         for (int i = 0; i <= (int)(QKK_MAX_EXPERTS / 64); i++)
             if ((uint32_t)(lane + 64 * i) <= d.E) s_log[lane + 64 * i] = lv[i];
@@ -627,20 +637,27 @@ static void launch_route_gateup(const qkk_moe_layer* L, const float* X, const Mo
         // FFN rows per wave: four at n_embd 2048, two at 4096 (the same bytes); n_ff is a multiple of both
         const uint32_t rpw = wide ? 2 : 4;
         const dim3 grid((d.k * (d.F / rpw) + 3) / 4, rows), block(256);
-#define QK_GATEUP(PASSES, RPW, ROWS) \
+        const bool ranked = options().select_ranked != 0; // the selection by rank counting on all four waves
+#define QK_GATEUP2(PASSES, RPW, ROWS, RANKED) \
     do { \
         if (norm) \
-            hipLaunchKernelGGL((moe_gateup_kernel<PASSES, RPW, ROWS, true>), grid, block, 0, st, ge, ue, X, ws, sel, d, \
+            hipLaunchKernelGGL((moe_gateup_kernel<PASSES, RPW, ROWS, true, RANKED>), grid, block, 0, st, ge, ue, X, ws, sel, d, \
                                NormArg<true>{norm->w, norm->eps}); \
         else \
-            hipLaunchKernelGGL((moe_gateup_kernel<PASSES, RPW, ROWS, false>), grid, block, 0, st, ge, ue, X, ws, sel, d, \
+            hipLaunchKernelGGL((moe_gateup_kernel<PASSES, RPW, ROWS, false, RANKED>), grid, block, 0, st, ge, ue, X, ws, sel, d, \
                                NormArg<false>{}); \
+    } while (0)
+#define QK_GATEUP(PASSES, RPW, ROWS) \
+    do { \
+        if (ranked) QK_GATEUP2(PASSES, RPW, ROWS, true); \
+        else QK_GATEUP2(PASSES, RPW, ROWS, false); \
     } while (0)
         if (!wide && rows > 1) QK_GATEUP(1, 4, true);
         else if (!wide) QK_GATEUP(1, 4, false);
         else if (rows > 1) QK_GATEUP(2, 2, true);
         else QK_GATEUP(2, 2, false);
 #undef QK_GATEUP
+#undef QK_GATEUP2
     }
 }
 

@@ -193,4 +193,86 @@ __device__ static inline void select_wave(const float* __restrict__ logits, uint
     else select_wave_n<QKK_MAX_EXPERTS / 64>(logits, E, k, out, ids_copy);
 }
 
+// ---- the same selection by a whole workgroup of four waves, without a chain of dependent rounds ------
+// The one-wave selector above is n_used rounds, each a chain of dependent cross-lane steps (about 1.7 us
+// for 8 of 256 on a lone wave).  Here every element finds its RANK by counting, and counting is a stream of
+// independent compares.  An element is (logit key, expert id) packed into 64 bits so that "greater" is
+// "picked earlier" (higher logit first, lower id on equal logits: a strict total order).  Thread t holds the
+// experts t and t + 256; a wave ranks its up to 128 elements among themselves (the others' values come as
+// LDS broadcasts), the n_used best of each wave -- a global pick is always among its own wave's best n_used --
+// are ranked again by wave 0 among the 4 * n_used candidates, and a candidate's rank there is its pick
+// number.  The reference's degenerate case (fewer finite logits than picks: once they are used up every
+// further round finds all entries at the floor and takes entry 0, shaders/moe_select.comp:53-70) is
+// reproduced from the count of finite logits.  Same ids, same weights as select_wave.
+struct SelectScratch {
+    uint64_t elem[QKK_MAX_EXPERTS];
+    uint64_t cand[4 * QKK_MAX_USED];
+    float logit[QKK_MAX_USED];
+    uint32_t finite[4];
+};
+
+// l0 / l1: this thread's logits of experts threadIdx.x and threadIdx.x + 256 (ignored where the id is not
+// below E); shared_logit: the shared gate's logit (thread 0).  All 256 threads call; `out` (LDS) is complete
+// after the caller's next workgroup barrier.
+__device__ static inline void select_block(float l0, float l1, float shared_logit, uint32_t E, uint32_t k,
+                                           qkk_sel* __restrict__ out, SelectScratch& sc)
+{
+    constexpr float FLOOR = -3.4e38f;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t floor_hi = (uint32_t)float_key(FLOOR) ^ 0x80000000u;
+    const auto pack = [&](float l, uint32_t id) -> uint64_t {
+        if (id >= E || isnan(l) || isinf(l)) l = FLOOR;
+        return ((uint64_t)((uint32_t)float_key(l) ^ 0x80000000u) << 32) | (uint32_t)~id;
+    };
+    const bool wide = E > 256; // workgroup-uniform
+    const uint64_t c0 = pack(l0, tid), c1 = pack(l1, tid + 256);
+    sc.elem[tid] = c0;
+    sc.elem[256 + tid] = c1;
+    const uint32_t nf = __builtin_popcountll(__builtin_amdgcn_ballot_w64((uint32_t)(c0 >> 32) > floor_hi)) +
+                        __builtin_popcountll(__builtin_amdgcn_ballot_w64((uint32_t)(c1 >> 32) > floor_hi));
+    if (lane == 0) sc.finite[wave] = nf;
+    __syncthreads();
+    // rank inside the wave
+    uint32_t r0 = 0, r1 = 0;
+#pragma unroll 16
+    for (uint32_t jj = 0; jj < 64; jj++) {
+        const uint64_t o = sc.elem[64 * wave + jj];
+        r0 += o > c0;
+        r1 += o > c1;
+    }
+    if (wide) {
+#pragma unroll 16
+        for (uint32_t jj = 0; jj < 64; jj++) {
+            const uint64_t o = sc.elem[256 + 64 * wave + jj];
+            r0 += o > c0;
+            r1 += o > c1;
+        }
+        if (r1 < k) sc.cand[wave * k + r1] = c1;
+    }
+    if (r0 < k) sc.cand[wave * k + r0] = c0;
+    __syncthreads();
+    if (wave != 0) return;
+    const uint32_t nc = 4 * k;
+    const uint64_t mine = lane < nc ? sc.cand[lane] : 0;
+    uint32_t rank = 0;
+    for (uint32_t jj = 0; jj < nc; jj++) rank += sc.cand[jj] > mine;
+    const uint32_t n_finite = min(sc.finite[0] + sc.finite[1] + sc.finite[2] + sc.finite[3], k);
+    if (lane < nc && (uint32_t)(mine >> 32) > floor_hi && rank < k) {
+        out->ids[rank] = min(~(uint32_t)mine, E - 1);
+        sc.logit[rank] = key_float((int32_t)((uint32_t)(mine >> 32) ^ 0x80000000u));
+    }
+    if (lane >= n_finite && lane < k) { // the finite logits are used up: entry 0, at the floor
+        out->ids[lane] = 0;
+        sc.logit[lane] = FLOOR;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const float p = lane < k ? expf(sc.logit[lane] - sc.logit[0]) : 0.f;
+    float wsum = 0.f;
+    for (uint32_t r = 0; r < k; r++) wsum += readlane_f(p, (int)r); // pick order
+    if (lane < k) out->w[lane] = p / wsum;
+    if (lane == 0) out->w_shared = 1.f / (1.f + expf(-shared_logit));
+}
+
 } // namespace qk

@@ -502,3 +502,48 @@ def test_lds_bank_model_of_the_table_lookups(qk, orc, emu, capsys):
     one, eight, thirty_two = (_model_cycles(256, 8, r, rng) for r in (1, 8, 32))
     assert abs(one - got["iq3_xxs", 1]["iq3_grid"][1]) < 0.5        # the model in Python agrees with the counted kernel
     assert eight > 0.85 * one and thirty_two == 2.0
+
+
+@pytest.mark.parametrize("E,k", [(8, 8), (100, 8), (256, 8), (256, 16), (300, 10), (512, 16), (64, 1)])
+def test_selectors_agree_with_the_oracle_on_exact_logits(qk, orc, emu, E, k):
+    """The router's logits made exact (the activation row is the first unit vector, so logit e is the first
+    element of router row e): ties in clusters, NaN and infinite logits, fewer finite logits than picks, all
+    logits non-finite.  Ids and weights of the one-wave selector (per-lane form, and the streamed form with
+    "select_ranked" off) and of the rank-counting selector (the streamed form's default) against the oracle's
+    restatement of the reference's rounds (shaders/moe_select.comp:28-34, 53-76): ids bit for bit in pick order."""
+    hl = qk.synth.HostLayer(seed=E + k, n_ff=256, n_expert=E, n_used=k)
+    rng = np.random.default_rng(E * 31 + k)
+    x = np.zeros((1, 2048), np.float32)
+    x[0, 0] = 1.0
+    cases = []
+    cases.append(rng.standard_normal(E))                                   # plain
+    cases.append(np.round(rng.standard_normal(E) * 2) / 2)                 # many ties
+    t = rng.standard_normal(E); t[rng.integers(0, E, max(1, E // 3))] = np.nan; t[rng.integers(0, E, 3)] = np.inf; cases.append(t)
+    t = np.full(E, np.nan); t[rng.choice(E, min(E, max(1, k // 2)), replace=False)] = rng.standard_normal(min(E, max(1, k // 2))); cases.append(t)  # fewer finite than picks
+    cases.append(np.full(E, np.nan))                                       # nothing finite
+    cases.append(np.full(E, 0.25))                                         # all equal
+    t = -np.abs(rng.standard_normal(E)); t[E - 1] = 0.0; t[0] = -0.0; cases.append(t)   # signed zeros tie
+    import contextlib
+    hl.gate_inp[:, :] = 0
+    layer = emu_util.layer_in_pool(qk, emu, hl)           # once: the cases rewrite the router's first column in place
+    router = layer.tensors["gate_inp"].numpy()
+    ws = emu.workspace(qk.moe_workspace_bytes(layer, 1))
+    X = emu.tensor(x)
+    for ci, logits in enumerate(cases):
+        router[:, 0] = logits.astype(np.float32)
+        want = orc.select_f32(logits.astype(np.float32), k)
+        got = {}
+        for name, opts in (("lane", {"one_row": 0}), ("stream_rounds", {"one_row": 1, "select_ranked": 0}),
+                           ("stream_ranked", {"one_row": 1, "select_ranked": 1})):
+            sel = emu.zeros((1, 160), np.uint8)
+            Y = emu.zeros((1, 2048), np.float32)
+            with contextlib.ExitStack() as st:
+                for o, v in opts.items():
+                    st.enter_context(qk.option(o, v))
+                qk.moe_decode(layer, X, ws, Y=Y, sel=sel, stages=3)   # route + select/gate/up
+            raw = sel.numpy().reshape(-1)
+            ids = raw[:64].view(np.uint32)[:k].tolist()
+            w = raw[64:128].view(np.float32)[:k]
+            got[name] = ids
+            assert ids == list(want.ids[:k]), (ci, name, ids, list(want.ids[:k]))
+            assert np.allclose(w, np.array(want.w[:k]), rtol=0, atol=1e-6, equal_nan=True), (ci, name, w, list(want.w[:k]))
