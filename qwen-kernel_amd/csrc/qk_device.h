@@ -493,6 +493,29 @@ struct LaneW<18> { // IQ3_XXS
     // XORs per four weights, each v_dot2_f32_f16 takes two weights (products exact, fp32 sums).  All
     // twelve lookups are issued before the first product, so that their latencies overlap (one at a
     // time, as the compiler had scheduled them, a lone lookup's latency was paid twelve times).
+    // The product as the per-lane gate/up launch runs it (the form its device results and timings belong
+    // to): lookups where they are used, the compiler's schedule.
+    __device__ __forceinline__ float dot_h_inline(const XSliceH& xh, const Iq3HalfTables* tab) const
+    {
+        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+        for (int l = 0; l < 4; l++) {
+            const uint4 sm = tab->sign[(aux >> (7 * l)) & 127u];
+            const uint32_t gw = l < 2 ? g.x : g.y;
+#pragma unroll
+            for (int hh = 0; hh < 2; hh++) {
+                const uint2 m = tab->grid[(gw >> (16 * (l & 1) + 8 * hh)) & 0xFFu];
+                const qk_half2 w01 = __builtin_bit_cast(qk_half2, m.x ^ (hh ? sm.z : sm.x));
+                const qk_half2 w23 = __builtin_bit_cast(qk_half2, m.y ^ (hh ? sm.w : sm.y));
+                const int q = l * 4 + hh * 2;
+                s0 = __builtin_amdgcn_fdot2(w01, xh.hi[q], s0, false);
+                s1 = __builtin_amdgcn_fdot2(w23, xh.hi[q + 1], s1, false);
+                s0 = __builtin_amdgcn_fdot2(w01, xh.lo[q], s0, false);
+                s1 = __builtin_amdgcn_fdot2(w23, xh.lo[q + 1], s1, false);
+            }
+        }
+        return h2f(d) * (0.5f + (float)(aux >> 28)) * 0.5f * (s0 + s1);
+    }
     __device__ __forceinline__ float dot_h(const XSliceH& xh, const Iq3HalfTables* tab) const
     {
         uint2 m[8];

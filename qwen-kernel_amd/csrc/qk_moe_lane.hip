@@ -277,8 +277,8 @@ __global__ __launch_bounds__(256) void moe_gateup_kernel(const uint8_t* __restri
             float g = 0.f, u = 0.f;
 #pragma unroll
             for (int p = 0; p < PASSES; p++) {
-                g += wg[i][p].dot_h(xs[p], &tab);
-                u += wu[i][p].dot_h(xs[p], &tab);
+                g += wg[i][p].dot_h_inline(xs[p], &tab);
+                u += wu[i][p].dot_h_inline(xs[p], &tab);
             }
             g = wave_sum(g);
             u = wave_sum(u);
@@ -385,8 +385,8 @@ __global__ __launch_bounds__(256) void moe_gateup_norm_kernel(const uint8_t* __r
             float g = 0.f, u = 0.f;
 #pragma unroll
             for (int p = 0; p < PASSES; p++) {
-                g += wg[i][p].dot_h(xs[p], &tab);
-                u += wu[i][p].dot_h(xs[p], &tab);
+                g += wg[i][p].dot_h_inline(xs[p], &tab);
+                u += wu[i][p].dot_h_inline(xs[p], &tab);
             }
             g = wave_sum(g) * scale;
             u = wave_sum(u) * scale;
