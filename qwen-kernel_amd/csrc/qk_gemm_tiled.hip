@@ -35,24 +35,53 @@ __device__ __forceinline__ void load_araw(ARaw& r, const float* __restrict__ row
 {
 #pragma unroll
     for (int i = 0; i < 8; i++) {
-        const uint32_t k = LAYOUT == 0 ? 64 * g + 8 * i : 128 * (g >> 1) + 32 * (i >> 1) + 16 * (g & 1) + 8 * (i & 1);
+        // LAYOUT 2: K in its natural order, step i = weights 32 i .. 32 i + 31 (one Q8_0 block), group g eight of them
+        const uint32_t k = LAYOUT == 2 ? 32 * i + 8 * g
+                         : LAYOUT == 0 ? 64 * g + 8 * i : 128 * (g >> 1) + 32 * (i >> 1) + 16 * (g & 1) + 8 * (i & 1);
         r.v[i][0] = *(const float4*)(row + k0 + k);
         r.v[i][1] = *(const float4*)(row + k0 + k + 4);
     }
 }
-__device__ __forceinline__ void split_araw(AFrag& a, const ARaw& r, float keep)
+// x = hi + lo.  Rows behind the last activation row repeat it (the loads are clamped): an output depends on
+// its own activation row only and those outputs are not stored, so nothing needs to be zeroed.
+// `one` is 1.0 in a register the compiler cannot see through: x * one - hi is then a genuine fused
+// multiply-add with mixed operands, which has a one-instruction form with a half result (v_fma_mixlo_f16);
+// written as x - hi it becomes a conversion, a subtraction and another conversion.
+__device__ __forceinline__ void split_araw(AFrag& a, const ARaw& r, float one)
 {
 #pragma unroll
     for (int i = 0; i < 8; i++) {
         const float f[8] = {r.v[i][0].x, r.v[i][0].y, r.v[i][0].z, r.v[i][0].w, r.v[i][1].x, r.v[i][1].y, r.v[i][1].z, r.v[i][1].w};
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            const float x = f[e] * keep;
-            a.hi[i][e] = (_Float16)x;
-            a.lo[i][e] = (_Float16)(x - (float)a.hi[i][e]);
+            a.hi[i][e] = (_Float16)f[e];
+            a.lo[i][e] = (_Float16)__builtin_fmaf(f[e], one, -(float)a.hi[i][e]);
         }
     }
 }
+
+// Q8_0 has a cut of its own: one matrix instruction's K = 32 is exactly one block, so the operand holds the
+// block's integers as they are (exact in a half, no residual operand), two instructions (activations hi, lo)
+// fill a fresh 16 x 16 result, and the block's scale multiplies that result in fp32 -- two matrix instructions
+// per product instead of three and a decode of 6 vector operations per block and tile instead of 18.
+struct Q8Rows {
+    uint2 q[8];     // this lane's eight weights of each of the fragment's eight blocks
+    uint32_t d[8];  // the blocks' scales (half bits)
+    __device__ __forceinline__ void load(const uint8_t* frag, int g)
+    {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            d[i] = ldg<uint16_t>(frag + i * Q8_0_BYTES);
+            q[i] = ldg<uint2>(frag + i * Q8_0_BYTES + 2 + 8 * g);
+        }
+    }
+    __device__ __forceinline__ half8 block(int i) const
+    {
+        const half4 a = bytes_to_half4(q[i].x ^ 0x80808080u, 128.f), b = bytes_to_half4(q[i].y ^ 0x80808080u, 128.f);
+        return half8{a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+    }
+    __device__ __forceinline__ float scale(int i) const { return h2f((uint16_t)d[i]); }
+};
 
 template <int TYPE>
 __global__ __launch_bounds__(GT_THREADS) void gemm_tiled_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X,
@@ -73,8 +102,9 @@ __global__ __launch_bounds__(GT_THREADS) void gemm_tiled_kernel(const uint8_t* _
     const uint32_t row0 = blockIdx.x * GT_BM;
     const uint32_t tok = blockIdx.y * GT_BN + wave * 16 + j; // this lane's activation row of the A operand
     const bool wave_live = blockIdx.y * GT_BN + wave * 16 < N; // wave-uniform: its 16 rows exist at least in part
-    const float keep = tok < N ? 1.f : 0.f;
     const float* xrow = X + (size_t)min(tok, N - 1) * K;
+    float one = 1.f; // in a register the compiler cannot see through (see split_araw)
+    asm volatile("" : QK_REG(one));
 
     // piece p of a K step: row p / NPW of the block, piece p % NPW of that row's window; rows behind the
     // matrix repeat its last row, pieces behind the tensor its last piece (neither is used)
@@ -111,9 +141,10 @@ __global__ __launch_bounds__(GT_THREADS) void gemm_tiled_kernel(const uint8_t* _
     fetch(0);
     ARaw raw;
     AFrag a;
-    if (wave_live) load_araw<F::LAYOUT>(raw, xrow, 0, g);
+    constexpr int CUT = TYPE == QKK_Q8_0 ? 2 : F::LAYOUT; // how K is dealt to the steps and lane groups
+    if (wave_live) load_araw<CUT>(raw, xrow, 0, g);
     commit(0);
-    if (wave_live) split_araw(a, raw, keep);
+    if (wave_live) split_araw(a, raw, one);
     __syncthreads();
 
     float4v acc[2] = {float4v{0.f, 0.f, 0.f, 0.f}, float4v{0.f, 0.f, 0.f, 0.f}};
@@ -121,8 +152,32 @@ __global__ __launch_bounds__(GT_THREADS) void gemm_tiled_kernel(const uint8_t* _
     for (uint32_t f = 0; f < nfrag; f++) {
         const uint32_t buf = f & 1u, fn = min(f + 1, nfrag - 1); // past the end: a harmless re-read
         fetch(fn);
-        if (wave_live) load_araw<F::LAYOUT>(raw, xrow, 256 * fn, g);
-        if (wave_live) {
+        if (wave_live) load_araw<CUT>(raw, xrow, 256 * fn, g);
+        if constexpr (TYPE == QKK_Q8_0) {
+            if (wave_live) {
+                Q8Rows w[2];
+#pragma unroll
+                for (int t = 0; t < 2; t++) w[t].load(frag_at(buf, t, f), g);
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const float4v zero = {0.f, 0.f, 0.f, 0.f};
+                    half8 b[2];
+                    float4v blk[2];
+#pragma unroll
+                    for (int t = 0; t < 2; t++) b[t] = w[t].block(i);
+#pragma unroll
+                    for (int t = 0; t < 2; t++) blk[t] = mfma16x32(a.hi[i], b[t], zero);
+#pragma unroll
+                    for (int t = 0; t < 2; t++) blk[t] = mfma16x32(a.lo[i], b[t], blk[t]);
+#pragma unroll
+                    for (int t = 0; t < 2; t++) {
+                        const float sc = w[t].scale(i);
+                        acc[t] += float4v{sc * blk[t][0], sc * blk[t][1], sc * blk[t][2], sc * blk[t][3]};
+                    }
+                }
+                split_araw(a, raw, one);
+            }
+        } else if (wave_live) {
             F w[2];
 #pragma unroll
             for (int t = 0; t < 2; t++) w[t].load(frag_at(buf, t, f), 0, g);
@@ -148,7 +203,7 @@ __global__ __launch_bounds__(GT_THREADS) void gemm_tiled_kernel(const uint8_t* _
                 const float sc = w[t].post(); // the row's fp16 scale of this fragment, in fp32
                 acc[t] += float4v{sc * part[t][0], sc * part[t][1], sc * part[t][2], sc * part[t][3]};
             }
-            split_araw(a, raw, keep); // the next step's operand
+            split_araw(a, raw, one); // the next step's operand
         }
         commit(buf ^ 1u);
         __syncthreads(); // step f is read, step f + 1 is in place
