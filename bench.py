@@ -551,7 +551,7 @@ def qk_env():
 
 def kernel_forms(qk):
     """The library's switches as they stand (which form of each kernel the figures belong to)."""
-    return {n: qk.get_option(n) for n in ("one_row", "dense_reg", "fused_norm", "attn_block", "dn_fused", "gemm_tiled")}
+    return {n: qk.get_option(n) for n in ("one_row", "dense_reg", "fused_norm", "attn_block", "dn_fused", "gemm_tiled", "moe_rows", "select_ranked")}
 
 
 def rate(bytes_step, ms, **more):
@@ -673,6 +673,9 @@ def extras(qk, a, steps):
     if a.ab_forms:   # the prefill product with every weight tile decoded once per 128 rows, beside the default above
         with qk.option("gemm_tiled", 1):
             run("gemm_tiled:prefill_gemm_q8_0_8192x2048x128", lambda: gemm_entry(qk))
+        with qk.option("moe_rows", 1):   # the routed experts with the waves splitting the weight rows, beside C3 and C5b above
+            run("moe_rows:moe_decode_bs16_q6k_down", moe16)
+            run("moe_rows:prefill_moe_128_tokens", prefill_moe)
     run("engine_decode_8_layers", lambda: engine_workload(qk, 8, (1, 4, 16), 8, 2))
     # a whole model: three gated-DeltaNet layers and one full-attention layer, twice (positions 1..320)
     run("engine_decode_whole_model_8_layers", lambda: engine_workload(qk, 8, (1, 16), 8, 2, kinds="RRRARRRA"))

@@ -273,6 +273,9 @@ __global__ __launch_bounds__(1024) void moe_select_group_kernel(MoeWs ws, qkk_se
 
 void moe_mfma_launch_shared(const qkk_moe_layer* L, const float* X, const qkk_sel* sel, const MoeWs& ws,
                             const MoeDims& d, uint32_t N, uint32_t stages, hipStream_t st);
+bool moe_rows_covers(const qkk_moe_layer* L, const MoeDims& d); // qk_moe_rows.hip
+void moe_rows_launch_routed(const qkk_moe_layer* L, const float* X, const qkk_sel* sel, const MoeWs& ws, const MoeDims& d,
+                            uint32_t N, uint32_t stages, hipStream_t st);
 void moe_mfma_launch_routed(const qkk_moe_layer* L, const float* X, const qkk_sel* sel, const MoeWs& ws,
                             const MoeDims& d, uint32_t N, uint32_t stages, hipStream_t st);
 void moe_mfma_launch_fold(float* Y, const qkk_sel* sel, const MoeWs& ws, const MoeDims& d, uint32_t N, hipStream_t st);
@@ -336,7 +339,10 @@ int moe_grouped_launch(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel
     if (d.H != 2048) return fail(QKK_ESHAPE, "moe: several rows need n_embd = 2048 (got %u)", d.H);
     const MoeWs ws = ws_carve(workspace, d, N);
     const uint32_t experts_stages = stages & (QKK_STAGE_GATEUP | QKK_STAGE_DOWN);
-    const bool split = N > FUSED_MAX_ROWS;
+    // the "moe_rows" switch: the routed experts through the row-split kernels (qk_moe_rows.hip); the shared expert
+    // then always takes its own launches
+    const bool rows = options().moe_rows != 0 && moe_rows_covers(L, d);
+    const bool split = N > FUSED_MAX_ROWS || rows;
     // fork: the shared expert needs only X (and its own h), so it starts right away
     SideStream* side = experts_stages && split ? side_stream(st) : nullptr;
     if (experts_stages && split) {
@@ -373,7 +379,8 @@ int moe_grouped_launch(const qkk_moe_layer* L, const float* X, float* Y, qkk_sel
         }
     }
     if (experts_stages) {
-        if (split) moe_mfma_launch_routed(L, X, sel, ws, d, N, stages, st);
+        if (rows) moe_rows_launch_routed(L, X, sel, ws, d, N, stages, st);
+        else if (split) moe_mfma_launch_routed(L, X, sel, ws, d, N, stages, st);
         else moe_mfma_launch_fused(L, X, sel, ws, d, N, stages, st);
     }
     if (side) { // join

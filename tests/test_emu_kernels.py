@@ -27,7 +27,7 @@ def form(request, qk, emu):
         yield request.param
 
 
-SWITCHES = ("one_row", "dense_reg", "fused_norm", "attn_block", "dn_fused", "gemm_tiled", "gemv_depth", "head_depth", "rowwise_max")
+SWITCHES = ("one_row", "dense_reg", "fused_norm", "attn_block", "dn_fused", "gemm_tiled", "moe_rows", "gemv_depth", "head_depth", "rowwise_max")
 
 
 @pytest.fixture
@@ -303,6 +303,22 @@ def test_expert_major_moe_inside_its_tensors(qk, orc, emu, down, n):
     ids = moe_case(qk, orc, emu, hl, x)
     assert ids.shape == (n, 2) and set(np.unique(ids)) <= set(range(8))
     qk.moe_workspace_status()   # the cleared workspace raised no flag
+
+
+@pytest.mark.parametrize("down,n,E,k,F", [("iq4_xs", 16, 8, 2, 256), ("q6_k", 40, 8, 2, 256), ("iq4_xs", 70, 4, 2, 512), ("q6_k", 12, 16, 8, 1024)])
+def test_row_split_expert_kernels_inside_their_tensors(qk, orc, emu, down, n, E, k, F):
+    """The routed experts' projections with the waves splitting the weight rows (the "moe_rows" switch): 12 to 70
+    rows, so that experts hold from a few pairs to several tiles of 16 (70 rows x 2 picks on 4 experts: three
+    tiles, the last one partial), n_ff of two to eight blocks of 128 rows, the LAST expert among the picks and the
+    tensors ending at guard pages; against the oracle, and the same ids and (to rounding of the sums) the same
+    outputs as the K-split kernels."""
+    hl = qk.synth.HostLayer(seed=31 + n, n_ff=F, n_expert=E, n_used=k, down_type=type_id(qk, down))
+    x = rows_that_pick_the_last_expert(hl, n, seed=n)
+    base = moe_case(qk, orc, emu, hl, x)
+    with qk.option("moe_rows", 1):
+        ids = moe_case(qk, orc, emu, hl, x)
+    assert np.array_equal(ids, base) and all(E - 1 in row for row in ids)
+    qk.moe_workspace_status()
 
 
 @pytest.mark.parametrize("M,K,N", [(48, 2048, 20), (33, 512, 9), (16, 4096, 128)])

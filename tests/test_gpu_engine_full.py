@@ -97,7 +97,8 @@ def test_whole_model_eager_launches_and_serial_prefill(qk, full, dev, monkeypatc
                   {"QK_ONE_ROW": "stream", "QK_DENSE_REG": "1"},   # block rows streamed through LDS
                   {"QK_ONE_ROW": "stream", "QK_FUSED_NORM": "1"},  # no norm launches: the same sums scaled later
                   {"QK_ATTN_BLOCK": "1"},       # the prompt's attention sixteen rows at a time
-                  {"QK_GEMM_TILED": "1"}]       # (passes of 64 rows and more only: here the same kernels)
+                  {"QK_GEMM_TILED": "1"},       # (passes of 64 rows and more only: here the same kernels)
+                  {"QK_MOE_ROWS": "1"}]         # the prompt's 17 positions through the row-split expert kernels
     for env in cases:
         for k in ("QK_NO_GRAPH", "QK_NO_BATCH", "QK_MAXB", "QK_PREFILL_ROWS"):
             monkeypatch.delenv(k, raising=False)

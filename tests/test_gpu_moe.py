@@ -114,6 +114,20 @@ def test_moe_decode_bs16_q6k_down(qk, orc, dev, layer_q6k):
     check(qk, orc, dev, layer_q6k, X, refs)
 
 
+def test_moe_decode_bs16_with_the_waves_splitting_the_rows(qk, orc, dev, unrun_form, layer_q6k, layer_iq4):
+    """Sixteen rows through the row-split expert kernels (the "moe_rows" switch): against the oracle, both
+    down formats, and twice on one workspace with identical bits."""
+    import torch
+    print("[case] moe bs=16, row-split experts", flush=True)
+    with qk.option("moe_rows", 1):
+        for hl, seed in ((layer_q6k, 2), (layer_iq4, 5)):
+            X, refs = pick_inputs(orc, hl, 16, seed=seed)
+            layer, ws, Y, sel = check(qk, orc, dev, hl, X, refs)
+            Y2, sel2 = qk.moe_decode(layer, torch.from_numpy(X).to(dev), ws)
+            torch.cuda.synchronize()
+            assert np.array_equal(Y2.cpu().numpy().view(np.uint32), Y.view(np.uint32)) and torch.equal(sel2, sel)
+
+
 def test_moe_decode_bs3_iq4_down_repeatable(qk, orc, dev, layer_iq4):
     import torch
     print("[case] moe bs=3 repeat on one workspace", flush=True)

@@ -52,6 +52,27 @@ def test_moe_prefill_small_layer_many_pairs_per_expert(qk, orc, dev):
     prefill_case(qk, orc, dev, hl, 96, seed=23)
 
 
+@pytest.mark.parametrize("down,n,E,k", [("iq4", 128, 256, 8), ("q6k", 40, 256, 8), ("iq4", 96, 16, 4)])
+def test_moe_prefill_with_the_waves_splitting_the_rows(qk, orc, dev, unrun_form, down, n, E, k):
+    """The "moe_rows" switch: the routed experts' gate/up and down projections with a wave owning 16 weight
+    rows for all of K and the pairs' activations shared through LDS.  The oracle's ids, weights and outputs
+    per token, and the ids of the default (K-split) kernels; experts with a few pairs (256 experts) and with
+    several tiles of 16 (16 experts)."""
+    import torch
+    print(f"[case] moe prefill, row-split experts: {n} tokens, {E} experts, {down} down", flush=True)
+    hl = qk.synth.HostLayer(seed=400 + n, n_expert=E, n_used=k, down_type=qk.IQ4_XS if down == "iq4" else qk.Q6_K)
+    with qk.option("moe_rows", 1):
+        prefill_case(qk, orc, dev, hl, n, seed=24)
+        X, _ = pick_inputs(orc, hl, n, seed=24)
+        layer = hl.to_device(dev)
+        ws = torch.zeros(qk.moe_prefill_workspace_bytes(layer, n), dtype=torch.uint8, device=dev)
+        _, sel_rows = qk.moe_prefill(layer, torch.from_numpy(X).to(dev), ws)
+        sel_rows = sel_rows.clone()
+    _, sel_k = qk.moe_prefill(layer, torch.from_numpy(X).to(dev), ws)
+    torch.cuda.synchronize()
+    assert torch.equal(sel_rows, sel_k)
+
+
 def test_moe_step_in_hip_graph_matches_eager(qk, dev):
     """The many-row step forks the shared expert onto a side stream of the library and joins it back
     with events: captured into a HIP graph it must replay to the eager result every time, with
