@@ -551,7 +551,7 @@ def qk_env():
 
 def kernel_forms(qk):
     """The library's switches as they stand (which form of each kernel the figures belong to)."""
-    return {n: qk.get_option(n) for n in ("one_row", "dense_reg", "fused_norm", "attn_block", "dn_fused", "gemm_tiled", "moe_rows", "select_ranked")}
+    return {n: qk.get_option(n) for n in ("one_row", "dense_reg", "fused_norm", "attn_block", "dn_fused", "gemm_tiled", "moe_rows", "head_rows", "select_ranked")}
 
 
 def rate(bytes_step, ms, **more):
@@ -676,6 +676,8 @@ def extras(qk, a, steps):
         with qk.option("moe_rows", 1):   # the routed experts with the waves splitting the weight rows, beside C3 and C5b above
             run("moe_rows:moe_decode_bs16_q6k_down", moe16)
             run("moe_rows:prefill_moe_128_tokens", prefill_moe)
+        with qk.option("head_rows", 1):  # the 16-row head with the waves splitting the vocabulary rows, beside C4 above
+            run("head_rows:head_q6k_151936_bs16", lambda: head(16))
     run("engine_decode_8_layers", lambda: engine_workload(qk, 8, (1, 4, 16), 8, 2))
     # a whole model: three gated-DeltaNet layers and one full-attention layer, twice (positions 1..320)
     run("engine_decode_whole_model_8_layers", lambda: engine_workload(qk, 8, (1, 16), 8, 2, kinds="RRRARRRA"))

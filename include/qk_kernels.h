@@ -96,6 +96,7 @@ int qkk_device_info(char *arch_host, size_t arch_len, uint32_t *n_cu_host);
  *                 weight tile once per 128 rows instead of once per 32
  *   "moe_rows"    1: the routed experts' projections for more than ten rows (qkk_moe_decode, qkk_moe_prefill)
  *                 with each wave owning 16 weight rows for all of K, instead of the waves splitting K
+ *   "head_rows"   1: qkk_head_argmax for 2..16 rows with each wave owning 16 vocabulary rows for all of K
  *   "select_ranked" (default 1; matters with "one_row" = 1 only) 0: the streamed gate/up launch picks the experts
  *                 in n_used rounds on one wave, as the per-lane form does, instead of by rank counting on four
  *   "gemv_depth", "head_depth", "rowwise_max": launch-shape sweeps, 0 = built-in value

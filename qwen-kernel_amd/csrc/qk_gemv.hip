@@ -66,7 +66,7 @@ const OptionDef OPTION_DEFS[] = {
     {"dn_fused", "QK_DN_FUSED", &Options::dn_fused, 0, 1},       {"gemv_depth", "QK_GEMV_DEPTH", &Options::gemv_depth, 0, 16},
     {"head_depth", "QK_HEAD_DEPTH", &Options::head_depth, 0, 8}, {"rowwise_max", "QK_ROWWISE_MAX", &Options::rowwise_max, 0, 64},
     {"gemm_tiled", "QK_GEMM_TILED", &Options::gemm_tiled, 0, 1}, {"select_ranked", "QK_SELECT_RANKED", &Options::select_ranked, 0, 1},
-    {"moe_rows", "QK_MOE_ROWS", &Options::moe_rows, 0, 1},
+    {"moe_rows", "QK_MOE_ROWS", &Options::moe_rows, 0, 1}, {"head_rows", "QK_HEAD_ROWS", &Options::head_rows, 0, 1},
 };
 } // namespace
 

@@ -6,6 +6,7 @@
 // token id.  Ties go to the lower id; a logit must beat -3.4e38 to be chosen
 // (reference shaders/argmax1.comp:25-33, argmax2.comp:20-28).
 #include "qk_coop.h"
+#include "qk_rows.h"
 #include "qk_device.h"
 #include "qk_host.h"
 #include "qk_stream.h"
@@ -387,6 +388,98 @@ __global__ __launch_bounds__(CT) void head_q6k_coop_kernel(const uint8_t* __rest
     }
 }
 
+// ---- 2..16 rows with the waves splitting the vocabulary rows (the "head_rows" switch) ----
+// The cooperative stream above splits K over the waves: per batch of 32 vocabulary rows partial tiles go through
+// LDS, one wave sums them and a barrier closes the batch -- 4,748 batches for the 151,936-row head, and it is
+// that fixed cost per batch which holds 16 rows at a third of the memory roofline.  Here a work item is a block
+// of 128 vocabulary rows and a wave owns 16 of them for all of K (rows_tile, qk_rows.h): its accumulators are
+// logits, a thread keeps the best (logit, id) of each of its four activation rows across its items (its rows
+// ascend, so `>` keeps the lowest id), and the fold over the workgroup, the candidates and the last workgroup are
+// those of the kernel above.  64 KB of LDS, two workgroups per CU.
+__global__ __launch_bounds__(MR_THREADS, 4) void head_q6k_rows_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X,
+                                                                      float* __restrict__ logits_out, uint32_t* __restrict__ tok,
+                                                                      HeadWs ws, uint32_t V, uint32_t batch)
+{
+    using G = RowsGeo<QKK_Q6_K, 1>;
+    constexpr uint32_t K = 2048, ROW = (K / 256) * G::FB;
+    QK_DYN_LDS(uint8_t, smem);
+    __shared__ MfmaTables tab; // Q6_K reads no table; rows_tile takes the reference
+    __shared__ uint32_t s_last;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, j = lane & 15, g = lane >> 4;
+    const uint8_t* tens[1] = {W};
+    const size_t last_piece = (size_t)V * ROW - 16; // a Q6_K row of 2048 is 105 pieces: the tensor ends on one
+    const uint32_t items = (V + MR_ROWS - 1) / MR_ROWS;
+    const float* arow = X + (size_t)min((uint32_t)j, batch - 1) * K; // operand rows behind the batch repeat its last row
+    float bv[4];
+    uint32_t bi[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) { bv[e] = ARG_FLOOR; bi[e] = 0xFFFFFFFFu; }
+    for (uint32_t item = blockIdx.x; item < items; item += gridDim.x) {
+        __syncthreads(); // the previous item's LDS is consumed
+        float4v acc[1];
+        rows_tile<QKK_Q6_K, 1>(tens, (size_t)item * MR_ROWS * ROW, ROW, last_piece, K / 256, arow, smem, tab, tid, acc);
+        const uint32_t row = item * MR_ROWS + 16 * wave + j; // rows behind V were read from clamped addresses: dropped here
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const uint32_t t = 4 * g + e;
+            if (t < batch && row < V) {
+                if (logits_out) logits_out[(size_t)t * V + row] = acc[0][e];
+                if (acc[0][e] > bv[e]) { bv[e] = acc[0][e]; bi[e] = row; }
+            }
+        }
+    }
+    __syncthreads();
+    // per activation row: the 128 threads that hold its outputs (16 rows x 8 waves), then the workgroups
+    float* s_v = (float*)smem;
+    uint32_t* s_i = (uint32_t*)(smem + MR_THREADS * 4 * 4);
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        s_v[tid * 4 + e] = bv[e];
+        s_i[tid * 4 + e] = bi[e];
+    }
+    __syncthreads();
+    if ((uint32_t)tid < batch) {
+        float v = ARG_FLOOR;
+        uint32_t i = 0xFFFFFFFFu;
+        const uint32_t tg = tid >> 2, te = tid & 3u;
+        for (uint32_t w = 0; w < MR_THREADS / 64; w++)
+            for (uint32_t jj = 0; jj < 16; jj++) {
+                const uint32_t o = (w * 64 + tg * 16 + jj) * 4 + te;
+                if (better(s_v[o], s_i[o], v, i)) { v = s_v[o]; i = s_i[o]; }
+            }
+        publish(&ws.cand_v[(size_t)tid * gridDim.x + blockIdx.x], v);
+        publish(&ws.cand_i[(size_t)tid * gridDim.x + blockIdx.x], i);
+        publish_wait(); // acknowledged before the barrier and the arrival count
+    }
+    __syncthreads();
+    if (tid == 0) s_last = arrive_last(&ws.counter[0], gridDim.x) ? 1u : 0u;
+    __syncthreads();
+    if (s_last) {
+        // one wave per activation row folds the workgroups' candidates
+        for (uint32_t t = wave; t < batch; t += MR_THREADS / 64) {
+            float v = ARG_FLOOR;
+            uint32_t i = 0xFFFFFFFFu;
+            for (uint32_t c = lane; c < gridDim.x; c += 64) {
+                const float cv = ws.cand_v[(size_t)t * gridDim.x + c];
+                const uint32_t ci = ws.cand_i[(size_t)t * gridDim.x + c];
+                if (better(cv, ci, v, i)) { v = cv; i = ci; }
+            }
+            dpp_better(v, i);
+            // four rows of 16 lanes remain
+            float fv = readlane_f(v, 0);
+            uint32_t fi = (uint32_t)__builtin_amdgcn_readlane((int)i, 0);
+#pragma unroll
+            for (int r = 16; r < 64; r += 16) {
+                const float ov = readlane_f(v, r);
+                const uint32_t oi = (uint32_t)__builtin_amdgcn_readlane((int)i, r);
+                if (better(ov, oi, fv, fi)) { fv = ov; fi = oi; }
+            }
+            if (lane == 0) tok[t] = fi == 0xFFFFFFFFu ? 0u : fi;
+        }
+        if (tid == 0) ws.counter[0] = 0u;
+    }
+}
+
 // Grid of the one-row kernel: one chunk per wave for a small vocabulary, else a persistent grid eight
 // workgroups deep per CU (16 KB of LDS each), the depth at which the same streaming loop read Q6_K
 // fastest as a plain GEMV.
@@ -418,7 +511,7 @@ extern "C" {
 size_t qkk_head_workspace_bytes(uint32_t V, uint32_t batch)
 {
     if (V == 0 || batch == 0) return 0;
-    const size_t blocks = std::max<size_t>(head_blocks(V, 1), persistent_blocks() / 4); // upper bound over the kernels
+    const size_t blocks = std::max<size_t>(head_blocks(V, 1), persistent_blocks() / 2); // upper bound over the kernels
     return 256 + (size_t)batch * blocks * 8;
 }
 
@@ -439,6 +532,21 @@ static int head_argmax_impl(const void* W, const float* X, uint32_t* tok, float*
     hipStream_t st = as_stream(stream);
     if (w_norm && (batch != 1 || K != 2048))
         return fail(QKK_ESHAPE, "qkk_head_argmax_norm: one row of 2048 (got %u rows of %u)", batch, K);
+    if (batch >= 2 && batch <= 16 && K == 2048 && options().head_rows) {
+        // the "head_rows" switch: blocks of 128 vocabulary rows, a wave owning 16 of them for all of K
+        using RG = RowsGeo<QKK_Q6_K, 1>;
+        HeadWs ws;
+        const uint32_t blocks = std::min((V + MR_ROWS - 1) / MR_ROWS, persistent_blocks() / 2); // two workgroups per CU (LDS)
+        ws.counter = (uint32_t*)workspace;
+        ws.cand_v = (float*)((uint8_t*)workspace + 256);
+        ws.cand_i = (uint32_t*)(ws.cand_v + (size_t)batch * blocks);
+        static const bool raised = ((void)hipFuncSetAttribute((const void*)head_q6k_rows_kernel,
+                                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)RG::LDS_BYTES), true);
+        (void)raised;
+        hipLaunchKernelGGL(head_q6k_rows_kernel, dim3(blocks), dim3(MR_THREADS), RG::LDS_BYTES, st, (const uint8_t*)W, X, logits,
+                           tok, ws, V, batch);
+        return check_launch("qkk_head_argmax");
+    }
     if (batch >= 2 && batch <= 16 && K == 2048) {
         HeadWs ws;
         const uint32_t blocks = persistent_blocks() / 4; // one workgroup per CU (LDS)

@@ -33,6 +33,7 @@ struct Options {
     int dn_fused = 0;       // QK_DN_FUSED=1: the gated-DeltaNet decode step as one launch
     int gemm_tiled = 0;     // QK_GEMM_TILED=1: 64 and more activation rows go through the kernel that decodes every weight tile once per 128 rows
     int select_ranked = 1;  // QK_SELECT_RANKED=0: the streamed gate/up launch selects with wave 0's rounds (as the per-lane form does) instead of by rank counting on all four waves
+    int head_rows = 0;      // QK_HEAD_ROWS=1: the LM head for 2..16 rows with the waves splitting the vocabulary rows instead of K
     int moe_rows = 0;       // QK_MOE_ROWS=1: the routed experts' projections for more than ten rows with the waves splitting the weight rows instead of K
     int gemv_depth = 0;     // QK_GEMV_DEPTH=n (1..16): workgroups per CU of the streaming GEMV's persistent grid, 0 = built-in
     int head_depth = 0;     // QK_HEAD_DEPTH=n (1..8): the same for the streaming LM head

@@ -18,26 +18,12 @@
 // Behind the "moe_rows" switch until it has been run and timed on a device; the shared expert keeps the
 // kernels of qk_moe_mfma.hip (it is one dense expert for every token).
 // (reference shaders/moe_gateup_iq3_grouped_coopmat.comp:46-217, moe_down_iq4_grouped_coopmat.comp:45-166.)
-#include "qk_coop.h"
 #include "qk_moe_common.h"
+#include "qk_rows.h"
 
 #include <algorithm>
 
 namespace qk {
-
-constexpr uint32_t MR_THREADS = 512, MR_ROWS = 128; // threads of a workgroup; weight rows of a work item
-
-template <int TYPE, bool GATEUP>
-struct RowsGeo {
-    using F = BFrag<TYPE>;
-    static constexpr uint32_t FB = F::BYTES;                       // bytes of a row's 256-weight fragment
-    static constexpr uint32_t NPW = (FB + 15 + 15) / 16, WIN = NPW * 16; // pieces / bytes of a row's window
-    static constexpr uint32_t SLOTS = GATEUP ? 2 * MR_ROWS : MR_ROWS;    // row fragments of a K step in LDS
-    static constexpr uint32_t PIECES = SLOTS * NPW;
-    static constexpr int NLD = (PIECES + MR_THREADS - 1) / MR_THREADS;
-    static constexpr uint32_t W_BYTES = SLOTS * WIN + 16, A_BYTES = 8 * 2 * 64 * 16; // one K step each
-    static constexpr uint32_t LDS_BYTES = W_BYTES + 2 * A_BYTES;
-};
 
 // GATEUP: W0 = gate_exps, W1 = up_exps (IQ3_XXS rows of n_embd), activations X [N][n_embd], outputs h.
 // else:   W0 = down_exps (rows of n_ff), activations h [N][k+1][n_ff], outputs contrib, weighted by the router.
@@ -46,13 +32,9 @@ __global__ __launch_bounds__(MR_THREADS, 4) void moe_rows_kernel(const uint8_t* 
                                                                  const float* __restrict__ X, MoeWs ws,
                                                                  const qkk_sel* __restrict__ sel, MoeDims d, uint32_t N)
 {
-    using G = RowsGeo<TYPE, GATEUP>;
-    using F = typename G::F;
-    constexpr uint32_t FB = G::FB, NPW = G::NPW, WIN = G::WIN, PIECES = G::PIECES;
-    constexpr int NLD = G::NLD, NT = GATEUP ? 2 : 1;
+    constexpr int NT = GATEUP ? 2 : 1;
+    using G = RowsGeo<TYPE, NT>;
     QK_DYN_LDS(uint8_t, smem);
-    uint8_t* s_w = smem;                 // [SLOTS][WIN]
-    uint8_t* s_a = smem + G::W_BYTES;    // [2][step 8][hi, lo][lane 64] half8
     __shared__ MfmaTables tab;
     __shared__ uint32_t s_tok[16], s_slot[16];
     __shared__ float s_wt[16];
@@ -60,42 +42,17 @@ __global__ __launch_bounds__(MR_THREADS, 4) void moe_rows_kernel(const uint8_t* 
     fill_mfma_tables_for<TYPE>(tab, tid, MR_THREADS); // in place before the first barrier below
     const uint32_t K = GATEUP ? d.H : d.F, R = GATEUP ? d.F : d.H; // weights per row, rows per expert
     const uint32_t nfrag = K / 256, blocks_per_expert = R / MR_ROWS;
-    const size_t stride = (size_t)nfrag * FB;                          // bytes of a weight row
+    const size_t stride = (size_t)nfrag * G::FB;                       // bytes of a weight row
     const size_t last_piece = (size_t)d.E * R * stride - 16;           // the tensors end on 16-byte boundaries (E * R * stride: R is a multiple of 128)
     const uint32_t n_active = active_count(ws, d);
-    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const uint8_t* tens[NT];
+    tens[0] = W0;
+    if constexpr (GATEUP) tens[1] = W1;
 
     for (uint32_t item = blockIdx.x; item < n_active * blocks_per_expert; item += gridDim.x) {
         const ActiveExpert ae = active_expert(ws, item / blocks_per_expert, d, N);
         const uint32_t row0 = (item % blocks_per_expert) * MR_ROWS;
         const size_t base = ((size_t)ae.expert * R + row0) * stride; // the block's first row, both tensors
-
-        // piece p of a K step: row slot p / NPW (gate rows, then up rows), piece p % NPW of its window.  Addresses
-        // are formed anew at every use (the thread index passes through an opaque register, or the compiler
-        // forms the row offsets once per kernel and keeps them): four of them kept per thread across the
-        // arithmetic cost more registers than the dozen integer operations they take.
-        u32x4 ld[NLD];
-        const auto fetch = [&](uint32_t f) {
-            uint32_t me = (uint32_t)tid;
-            asm volatile("" : QK_REG(me));
-#pragma unroll
-            for (int n = 0; n < NLD; n++) {
-                const uint32_t p = min(me + MR_THREADS * n, PIECES - 1);
-                const uint32_t slot = p / NPW, q = p % NPW;
-                const uint8_t* tens = GATEUP && slot >= MR_ROWS ? W1 : W0;
-                const size_t at = base + (size_t)(slot % MR_ROWS) * stride + (size_t)f * FB; // the row's fragment f
-                ld[n] = *(const u32x4*)(tens + min((at & ~(size_t)15) + 16u * q, last_piece));   // its window starts at the 16-byte boundary below
-            }
-        };
-        const auto commit = [&]() {
-#pragma unroll
-            for (int n = 0; n < NLD; n++) {
-                const uint32_t p = tid + MR_THREADS * n;
-                if (PIECES % MR_THREADS == 0 || n + 1 < NLD || p < PIECES) *(u32x4*)(s_w + (p / NPW) * WIN + (p % NPW) * 16) = ld[n];
-            }
-        };
-        // this lane's weight rows: row 16 wave + j of the block (gate tile, and for gate/up the up tile)
-        const size_t my_at = base + (size_t)(16 * wave + j) * stride;
 
         for (uint32_t t0 = 0; t0 < ae.count; t0 += 16) {
             const uint32_t np = min(16u, ae.count - t0);
@@ -108,72 +65,9 @@ __global__ __launch_bounds__(MR_THREADS, 4) void moe_rows_kernel(const uint8_t* 
                 s_tok[tid] = tok; s_slot[tid] = slot; s_wt[tid] = wt;
             }
             __syncthreads();
-            // thread (step i = wave, lane): the operand of lane (pair j, group g) for step i of a K step
             const float* arow = GATEUP ? X + (size_t)s_tok[j] * d.H : ws.h + ((size_t)s_tok[j] * (d.k + 1) + s_slot[j]) * d.F;
-            const uint32_t acut = F::LAYOUT == 0 ? 64 * g + 8 * wave : 128 * (g >> 1) + 32 * (wave >> 1) + 16 * (g & 1) + 8 * (wave & 1);
-            float4 ar[2];
-            const auto load_a = [&](uint32_t f) {
-                ar[0] = *(const float4*)(arow + 256 * f + acut);
-                ar[1] = *(const float4*)(arow + 256 * f + acut + 4);
-            };
-            const auto commit_a = [&](uint32_t buf) {
-                const float x[8] = {ar[0].x, ar[0].y, ar[0].z, ar[0].w, ar[1].x, ar[1].y, ar[1].z, ar[1].w};
-                half8 hi, lo;
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    hi[e] = (_Float16)x[e];
-                    lo[e] = (_Float16)(x[e] - (float)hi[e]);
-                }
-                half8* dstp = (half8*)(s_a + buf * G::A_BYTES) + (size_t)(wave * 2) * 64 + lane;
-                dstp[0] = hi;
-                dstp[64] = lo;
-            };
-            fetch(0);
-            load_a(0);
-            commit();
-            commit_a(0);
-            __syncthreads();
-
             float4v acc[NT];
-#pragma unroll
-            for (int t = 0; t < NT; t++) acc[t] = float4v{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 1
-            for (uint32_t f = 0; f < nfrag; f++) {
-                const uint32_t buf = f & 1u;
-                const bool more = f + 1 < nfrag; // workgroup-uniform
-                if (more) {
-                    fetch(f + 1);
-                    load_a(f + 1);
-                }
-                // one tile after the other (gate, then up): one set of fragment registers and decode temporaries
-                // alive at a time; the waves of the SIMD fill each other's matrix-instruction latencies
-                const half8* ap = (const half8*)(s_a + buf * G::A_BYTES) + lane;
-#pragma unroll
-                for (int t = 0; t < NT; t++) {
-                    asm volatile("" ::: "memory"); // the second tile reads its activation operands again rather than keeping the first's 64 registers
-                    F w;
-                    w.load(s_w + (size_t)(t * MR_ROWS + 16 * wave + j) * WIN + ((my_at + (size_t)f * FB) & 15), 0, g);
-                    float4v part = float4v{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int i = 0; i < 8; i++) {
-                        const half8 ahi = ap[(size_t)(i * 2) * 64], alo = ap[(size_t)(i * 2 + 1) * 64];
-                        half8 bl;
-                        const half8 bh = w.step(i, g, tab, bl);
-                        part = mfma16x32(ahi, bh, part);
-                        part = mfma16x32(alo, bh, part);
-                        if constexpr (F::SPLIT) part = mfma16x32(ahi, bl, part);
-                        __builtin_amdgcn_sched_barrier(0); // keep the decode of later steps from piling up in registers
-                    }
-                    const float sc = w.post();
-                    acc[t] += float4v{sc * part[0], sc * part[1], sc * part[2], sc * part[3]};
-                }
-                if (more) {
-                    __syncthreads(); // every wave has read this step's rows
-                    commit();
-                    commit_a(buf ^ 1u);
-                    __syncthreads(); // the next step's rows and activations are in place
-                }
-            }
+            rows_tile<TYPE, NT>(tens, base, stride, last_piece, nfrag, arow, smem, tab, tid, acc);
             // D[4 g + e][j]: pair 4 g + e of the tile, row 16 wave + j of the block
             const uint32_t row = row0 + 16 * wave + j;
 #pragma unroll
@@ -193,7 +87,7 @@ template <int TYPE, bool GATEUP>
 static void launch_rows(const uint8_t* W0, const uint8_t* W1, const float* X, const MoeWs& ws, const qkk_sel* sel,
                         const MoeDims& d, uint32_t N, uint32_t experts, hipStream_t st)
 {
-    using G = RowsGeo<TYPE, GATEUP>;
+    using G = RowsGeo<TYPE, GATEUP ? 2 : 1>;
     static const bool raised = ((void)hipFuncSetAttribute((const void*)moe_rows_kernel<TYPE, GATEUP>,
                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)G::LDS_BYTES), true);
     (void)raised;

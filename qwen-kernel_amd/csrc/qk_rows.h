@@ -1,0 +1,139 @@
+// qk_rows.h -- a tile of 16 activation rows against a block of 128 weight rows (or 128 rows each of two
+// tensors), with the eight waves of a workgroup splitting the weight ROWS: a wave owns 16 rows for all of K,
+// so its accumulators are its outputs.  The activation operand of the 16 rows lives in LDS in operand order,
+// converted to hi + lo halves once per workgroup and K step of 256 weights and read by every wave; the rows'
+// fragments of a K step reach LDS as the aligned 16-byte pieces that cover them, the next step's pieces and
+// activations in flight in registers during the arithmetic.  Decoder: BFrag<TYPE>::step, the cooperative
+// stream's (qk_coop.h), so the same exactness (activations hi + lo, weights hi (+ lo)).
+// Users: the routed experts' projections (qk_moe_rows.hip), the LM head for 2..16 rows (qk_head.hip).
+#pragma once
+#include "qk_coop.h"
+
+namespace qk {
+
+constexpr uint32_t MR_THREADS = 512, MR_ROWS = 128; // threads of a workgroup; weight rows of a work item
+
+template <int TYPE, int NT>
+struct RowsGeo {
+    using F = BFrag<TYPE>;
+    static constexpr uint32_t FB = F::BYTES;                             // bytes of a row's 256-weight fragment
+    static constexpr uint32_t NPW = (FB + 15 + 15) / 16, WIN = NPW * 16; // pieces / bytes of a row's window
+    static constexpr uint32_t SLOTS = NT * MR_ROWS;                      // row fragments of a K step in LDS
+    static constexpr uint32_t PIECES = SLOTS * NPW;
+    static constexpr int NLD = (PIECES + MR_THREADS - 1) / MR_THREADS;
+    static constexpr uint32_t W_BYTES = SLOTS * WIN + 16, A_BYTES = 8 * 2 * 64 * 16; // one K step each
+    static constexpr uint32_t LDS_BYTES = W_BYTES + 2 * A_BYTES;
+};
+
+// acc[t][e] = sum over K of (row 16 wave + j of tensor t's block) . (activation row 4 g + e), lane = 16 g + j.
+// tens[t] + base: the block's first row in tensor t (rows `stride` bytes apart, nfrag fragments each); reads are
+// clamped to the 16-byte piece at `last_piece`, the tensors' last one.  arow: the activation row of THIS
+// thread's lane j (thread (wave, lane) converts the operand of lane `lane` for instruction `wave` of a step).
+// smem: RowsGeo::LDS_BYTES; the caller has a barrier between the previous user of smem and this call, and one
+// between this call and the next user.
+template <int TYPE, int NT>
+__device__ __forceinline__ void rows_tile(const uint8_t* const (&tens)[NT], size_t base, size_t stride, size_t last_piece,
+                                          uint32_t nfrag, const float* arow, uint8_t* smem, const MfmaTables& tab, int tid,
+                                          float4v (&acc)[NT])
+{
+    using G = RowsGeo<TYPE, NT>;
+    using F = typename G::F;
+    constexpr uint32_t FB = G::FB, NPW = G::NPW, WIN = G::WIN, PIECES = G::PIECES;
+    constexpr int NLD = G::NLD;
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    uint8_t* s_w = smem;              // [SLOTS][WIN]
+    uint8_t* s_a = smem + G::W_BYTES; // [2][step 8][hi, lo][lane 64] half8
+    const int lane = tid & 63, wave = tid >> 6, j = lane & 15, g = lane >> 4;
+
+    // piece p of a K step: row slot p / NPW (the first tensor's rows, then the second's), piece p % NPW of its
+    // window.  Addresses are formed anew at every use (the thread index passes through an opaque register, or
+    // the compiler forms the row offsets once per kernel and keeps them): four of them kept per thread across
+    // the arithmetic cost more registers than the dozen integer operations they take.
+    u32x4 ld[NLD];
+    const auto fetch = [&](uint32_t f) {
+        uint32_t me = (uint32_t)tid;
+        asm volatile("" : QK_REG(me));
+#pragma unroll
+        for (int n = 0; n < NLD; n++) {
+            const uint32_t p = min(me + MR_THREADS * n, PIECES - 1);
+            const uint32_t slot = p / NPW, q = p % NPW;
+            const uint8_t* t = tens[NT > 1 && slot >= MR_ROWS ? NT - 1 : 0];
+            const size_t at = base + (size_t)(slot % MR_ROWS) * stride + (size_t)f * FB; // the row's fragment f
+            ld[n] = *(const u32x4*)(t + min((at & ~(size_t)15) + 16u * q, last_piece)); // its window starts at the 16-byte boundary below
+        }
+    };
+    const auto commit = [&]() {
+#pragma unroll
+        for (int n = 0; n < NLD; n++) {
+            const uint32_t p = tid + MR_THREADS * n;
+            if (PIECES % MR_THREADS == 0 || n + 1 < NLD || p < PIECES) *(u32x4*)(s_w + (p / NPW) * WIN + (p % NPW) * 16) = ld[n];
+        }
+    };
+    // this lane's weight rows: row 16 wave + j of the block, in every tensor
+    const size_t my_at = base + (size_t)(16 * wave + j) * stride;
+    const uint32_t acut = F::LAYOUT == 0 ? 64 * g + 8 * wave : 128 * (g >> 1) + 32 * (wave >> 1) + 16 * (g & 1) + 8 * (wave & 1);
+    float4 ar[2];
+    const auto load_a = [&](uint32_t f) {
+        ar[0] = *(const float4*)(arow + 256 * f + acut);
+        ar[1] = *(const float4*)(arow + 256 * f + acut + 4);
+    };
+    const auto commit_a = [&](uint32_t buf) {
+        const float x[8] = {ar[0].x, ar[0].y, ar[0].z, ar[0].w, ar[1].x, ar[1].y, ar[1].z, ar[1].w};
+        half8 hi, lo;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            hi[e] = (_Float16)x[e];
+            lo[e] = (_Float16)(x[e] - (float)hi[e]);
+        }
+        half8* dstp = (half8*)(s_a + buf * G::A_BYTES) + (size_t)(wave * 2) * 64 + lane;
+        dstp[0] = hi;
+        dstp[64] = lo;
+    };
+    fetch(0);
+    load_a(0);
+    commit();
+    commit_a(0);
+    __syncthreads();
+
+#pragma unroll
+    for (int t = 0; t < NT; t++) acc[t] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+    for (uint32_t f = 0; f < nfrag; f++) {
+        const uint32_t buf = f & 1u;
+        const bool more = f + 1 < nfrag; // workgroup-uniform
+        if (more) {
+            fetch(f + 1);
+            load_a(f + 1);
+        }
+        // one tensor's tile after the other: one set of fragment registers and decode temporaries alive at a
+        // time; the waves of the SIMD fill each other's matrix-instruction latencies
+        const half8* ap = (const half8*)(s_a + buf * G::A_BYTES) + lane;
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            asm volatile("" ::: "memory"); // the second tile reads its activation operands again rather than keeping the first's 64 registers
+            F w;
+            w.load(s_w + (size_t)(t * MR_ROWS + 16 * wave + j) * WIN + ((my_at + (size_t)f * FB) & 15), 0, g);
+            float4v part = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const half8 ahi = ap[(size_t)(i * 2) * 64], alo = ap[(size_t)(i * 2 + 1) * 64];
+                half8 bl;
+                const half8 bh = w.step(i, g, tab, bl);
+                part = mfma16x32(ahi, bh, part);
+                part = mfma16x32(alo, bh, part);
+                if constexpr (F::SPLIT) part = mfma16x32(ahi, bl, part);
+                __builtin_amdgcn_sched_barrier(0); // keep the decode of later steps from piling up in registers
+            }
+            const float sc = w.post();
+            acc[t] += float4v{sc * part[0], sc * part[1], sc * part[2], sc * part[3]};
+        }
+        if (more) {
+            __syncthreads(); // every wave has read this step's rows
+            commit();
+            commit_a(buf ^ 1u);
+            __syncthreads(); // the next step's rows and activations are in place
+        }
+    }
+}
+
+} // namespace qk

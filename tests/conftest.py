@@ -57,8 +57,8 @@ def dev(qk):
     return "cuda:0"
 
 
-SWITCHES = ("one_row", "dense_reg", "fused_norm", "attn_block", "dn_fused", "gemm_tiled", "moe_rows", "gemv_depth", "head_depth", "rowwise_max")
-SWITCH_ENV_DEFAULTS = {"QK_ONE_ROW": "lane", "QK_DENSE_REG": "0", "QK_FUSED_NORM": "0", "QK_ATTN_BLOCK": "0", "QK_DN_FUSED": "0", "QK_GEMM_TILED": "0", "QK_MOE_ROWS": "0"}
+SWITCHES = ("one_row", "dense_reg", "fused_norm", "attn_block", "dn_fused", "gemm_tiled", "moe_rows", "head_rows", "gemv_depth", "head_depth", "rowwise_max")
+SWITCH_ENV_DEFAULTS = {"QK_ONE_ROW": "lane", "QK_DENSE_REG": "0", "QK_FUSED_NORM": "0", "QK_ATTN_BLOCK": "0", "QK_DN_FUSED": "0", "QK_GEMM_TILED": "0", "QK_MOE_ROWS": "0", "QK_HEAD_ROWS": "0"}
 UNRUN = ("a form of the kernels that has not had its first supervised run on a device is reached through a switch "
          "and tested on hardware only with QK_TEST_UNRUN_FORMS=1 (the host-side build always runs it)")
 

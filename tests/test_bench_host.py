@@ -172,7 +172,7 @@ def test_other_workloads_print_one_line_each(monkeypatch, capsys, qk):
     for form in ("lane", "stream"):
         for k in ("gemv_iq4_xs_8192x2048", "gemv_q6_k_sustained_256MiB", "head_q6k_151936_bs1", "moe_decode_bs1"):
             assert "error" not in ex[f"{form}:{k}"], (form, k, ex[f"{form}:{k}"])
-    for k in ("gemm_tiled:prefill_gemm_q8_0_8192x2048x128", "moe_rows:moe_decode_bs16_q6k_down", "moe_rows:prefill_moe_128_tokens"):
+    for k in ("gemm_tiled:prefill_gemm_q8_0_8192x2048x128", "moe_rows:moe_decode_bs16_q6k_down", "moe_rows:prefill_moe_128_tokens", "head_rows:head_q6k_151936_bs16"):
         assert "error" not in ex[k], (k, ex[k])
     assert qk.get_option("one_row") == 0 and qk.get_option("moe_rows") == 0   # the switches are back at their defaults
 

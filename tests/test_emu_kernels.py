@@ -27,7 +27,7 @@ def form(request, qk, emu):
         yield request.param
 
 
-SWITCHES = ("one_row", "dense_reg", "fused_norm", "attn_block", "dn_fused", "gemm_tiled", "moe_rows", "gemv_depth", "head_depth", "rowwise_max")
+SWITCHES = ("one_row", "dense_reg", "fused_norm", "attn_block", "dn_fused", "gemm_tiled", "moe_rows", "head_rows", "gemv_depth", "head_depth", "rowwise_max")
 
 
 @pytest.fixture
@@ -168,6 +168,38 @@ def test_head_inside_its_tensors(qk, orc, emu, V, batch, form):
         top2 = np.sort(want)[-2:]
         if top2[1] - top2[0] > 2e-3 * abs(top2[1]):
             assert int(tok.numpy()[b]) == int(np.argmax(want))
+
+
+@pytest.mark.parametrize("V,batch", [(300, 3), (128, 16), (1000, 2), (2049, 9)])
+def test_head_with_the_waves_splitting_the_rows(qk, orc, emu, V, batch):
+    """The LM head for 2..16 rows with a wave owning 16 vocabulary rows for all of K (the "head_rows" switch):
+    vocabularies that end inside a block of 128 rows, on one, or one row behind one, the tensor at the guard
+    page; logits and ids against the oracle, ids and (to rounding of the sums) logits as the default kernel's,
+    the winning row copied to a lower and a higher id so that equal logits meet across waves and workgroups,
+    and a second call on the same workspace."""
+    K = 2048
+    W = qk.synth.tensor_host(qk.Q6_K, V, K, seed=V).reshape(V, -1).copy()
+    x = np.random.default_rng(V).standard_normal((batch, K)).astype(np.float32)
+    ws = emu.workspace(qk.head_workspace_bytes(V, batch))
+    xd = emu.tensor(x)
+    tok0, logits0 = qk.head_argmax(emu.tensor(W.reshape(-1)), xd, V, K, ws, want_logits=True)
+    tok0, logits0 = tok0.numpy().copy(), logits0.numpy().copy()
+    with qk.option("head_rows", 1):
+        tok, logits = qk.head_argmax(emu.tensor(W.reshape(-1)), xd, V, K, ws, want_logits=True)
+        tok, logits = tok.numpy().copy(), logits.numpy().copy()
+        for b in range(batch):
+            want = orc.gemv(qk.Q6_K, W.reshape(-1), x[b], V, K)
+            assert orc.rel_maxabs_err(logits[b], want) <= 1e-3
+            assert int(tok[b]) == int(np.argmax(logits[b]))
+        assert orc.rel_maxabs_err(logits, logits0) <= 1e-5
+        # ties: row 0's winner copied to the last row and to row 1 (or 0): the lowest id must win
+        best = int(tok[0])
+        lo = 1 if best != 1 else 0
+        W[V - 1] = W[best]
+        W[lo] = W[best]
+        tok2, _ = qk.head_argmax(emu.tensor(W.reshape(-1)), xd, V, K, ws)
+        assert int(tok2.numpy()[0]) == min(best, lo)
+    assert qk.get_option("head_rows") == 0
 
 
 @pytest.mark.parametrize("name", QUANT)

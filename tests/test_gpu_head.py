@@ -45,6 +45,13 @@ def test_head_ragged(qk, orc, dev, V, K, batch):
     head_case(qk, orc, dev, V, K, batch, seed=12 + V)
 
 
+@pytest.mark.parametrize("V,batch", [(151936, 16), (151936, 2), (4097, 16), (128, 5), (33, 9)])
+def test_head_with_the_waves_splitting_the_rows(qk, orc, dev, unrun_form, V, batch):
+    """The "head_rows" switch: 2..16 rows with a wave owning 16 vocabulary rows for all of K."""
+    with qk.option("head_rows", 1):
+        head_case(qk, orc, dev, V, 2048, batch, seed=40 + batch)
+
+
 @pytest.mark.parametrize("V", [151936, 4097, 3])
 def test_head_with_the_norm_in_front(qk, orc, dev, unrun_form, V):
     """qkk_head_argmax_norm: the output norm inside the head's launch, against the oracle's norm (double)
