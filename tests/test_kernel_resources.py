@@ -60,6 +60,14 @@ def test_streaming_kernels_keep_two_waves_per_simd(usage):
     assert not low, low
 
 
+def test_row_split_kernels_keep_four_waves_per_simd(usage):
+    """The kernels whose waves split the weight rows (512 threads, 64 KB of LDS) are meant to run two workgroups to
+    a CU: four waves per SIMD, so at most 128 registers per lane -- and none of them in scratch memory."""
+    rows = {k: v for k, v in usage.items() if "moe_rows_kernel" in k or "head_q6k_rows_kernel" in k}
+    assert len(rows) == 4, sorted(rows)
+    assert all(v["occupancy"] >= 4 and v["vgprs"] <= 128 and v["scratch"] == 0 for v in rows.values()), rows
+
+
 def isa_of(path):
     import tempfile
     with tempfile.TemporaryDirectory() as tmp:
