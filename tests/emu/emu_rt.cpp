@@ -15,6 +15,7 @@
 #include <atomic>
 #include <condition_variable>
 #include <mutex>
+#include <string>
 #include <thread>
 #include <vector>
 
@@ -47,6 +48,25 @@ extern "C" void emu_ctx_switch(void** save_sp, void* load_sp);
 namespace emu {
 
 Idx g_block_dim, g_grid_dim;
+
+// Order in which a sweep of the scheduler visits the fibers of a workgroup: 0 ascending thread index, 1 descending,
+// 2 a fresh random permutation per sweep.  Between two barriers the threads of a workgroup run one after the other
+// in that order, so a pair of accesses that needs a barrier and has none sees the writer first under one order and
+// the reader first under another: results that differ between orders are a race.
+std::atomic<int> g_order_mode{0};
+std::atomic<uint64_t> g_order_seed{1};
+// QK_EMU_ORDER=reverse | random[:seed] sets the order for a whole process (a test file run on the host-side build)
+static const bool g_order_from_env = [] {
+    const char* e = getenv("QK_EMU_ORDER");
+    if (!e) return false;
+    const std::string v(e);
+    if (v == "reverse") g_order_mode = 1;
+    else if (v.rfind("random", 0) == 0) {
+        g_order_mode = 2;
+        if (v.size() > 7) g_order_seed = strtoull(v.c_str() + 7, nullptr, 10) | 1u;
+    }
+    return true;
+}();
 
 namespace {
 constexpr int MAX_WAVES = 16;
@@ -166,18 +186,43 @@ void run_workgroup(Workgroup& g, Idx block, int n, size_t lds, const std::functi
     delete g.dyn;
     g.dyn = new GuardBuf(lds ? lds : 16);
     int live = n;
+    const int mode = g_order_mode.load();
+    uint64_t rng = g_order_seed.load() * 0x9E3779B97F4A7C15ull + (((uint64_t)block.z << 40) ^ ((uint64_t)block.y << 20) ^ block.x) + 1;
+    std::vector<int> order((size_t)n);
+    for (int t = 0; t < n; t++) order[(size_t)t] = mode == 1 ? n - 1 - t : t;
+    // mode 2 also holds waves back: now and then a wave sits out up to 48 sweeps (a sweep is about one
+    // cross-lane operation or matrix instruction of every other wave), so the waves of a workgroup drift apart
+    // between two workgroup barriers as far as they may on a device
+    int hold[MAX_WAVES] = {};
     while (live > 0) {
-        bool ran = false;
-        for (int t = 0; t < n; t++) {
+        bool ran = false, held = false;
+        if (mode == 2) {
+            for (int t = n - 1; t > 0; t--) { // Fisher-Yates on a xorshift stream
+                rng ^= rng << 13; rng ^= rng >> 7; rng ^= rng << 17;
+                std::swap(order[(size_t)t], order[(size_t)(rng % (uint64_t)(t + 1))]);
+            }
+            for (int w = 0; w < n / 64; w++) {
+                rng ^= rng << 13; rng ^= rng >> 7; rng ^= rng << 17;
+                if (hold[w] > 0) hold[w]--;
+                else if ((rng & 7u) == 0) hold[w] = 1 + (int)((rng >> 8) % 48u);
+            }
+        }
+        for (int k = 0; k < n; k++) {
+            const int t = order[(size_t)k];
             Fiber& fb = g.f[t];
             if (fb.done) continue;
             if (fb.wait_kind == 1 && g.wave_gen[t >> 6] == fb.wait_gen) continue;
             if (fb.wait_kind == 2 && g.block_gen == fb.wait_gen) continue;
+            if (hold[t >> 6] > 0) { held = true; continue; }
             fb.wait_kind = 0;
             g.cur = &fb;
             emu_ctx_switch(&g.main_sp, fb.sp);
             ran = true;
             if (fb.done) live--;
+        }
+        if (!ran && held) { // only held waves could run: let them
+            for (int w = 0; w < MAX_WAVES; w++) hold[w] = 0;
+            continue;
         }
         if (!ran) {
             int at_wave = 0, at_block = 0;
@@ -193,6 +238,7 @@ void run_workgroup(Workgroup& g, Idx block, int n, size_t lds, const std::functi
 
 std::mutex g_launch_mu; // one launch at a time
 } // namespace
+
 
 const Idx& cur_thread() { return t_wg->cur->tid; }
 const Idx& cur_block() { return t_wg->block; }
@@ -428,6 +474,12 @@ hipError_t hipFree(void* p)
 
 // C entry points for the tests: buffers that end at a guard page.
 extern "C" {
+// mode 0: threads of a workgroup run in ascending order between barriers, 1: descending, 2: random per sweep (seed)
+void emu_set_schedule(int mode, uint64_t seed)
+{
+    emu::g_order_mode = mode < 0 || mode > 2 ? 0 : mode;
+    emu::g_order_seed = seed ? seed : 1;
+}
 void emu_lds_probe_enable(int on)
 {
     emu::g_lds_probe_on = on != 0;

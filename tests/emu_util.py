@@ -31,6 +31,8 @@ def emu_lib(qk):
         L.emu_guard_alloc.restype = C.c_void_p
         L.emu_guard_alloc.argtypes = [C.c_size_t, C.c_size_t, C.POINTER(C.c_void_p)]
         L.emu_guard_free.argtypes = [C.c_void_p]
+        L.emu_set_schedule.argtypes = [C.c_int, C.c_uint64]
+        L.emu_set_schedule.restype = None
         _emu = L
     return _emu
 

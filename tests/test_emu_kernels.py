@@ -595,3 +595,85 @@ def test_selectors_agree_with_the_oracle_on_exact_logits(qk, orc, emu, E, k):
             got[name] = ids
             assert ids == list(want.ids[:k]), (ci, name, ids, list(want.ids[:k]))
             assert np.allclose(w, np.array(want.w[:k]), rtol=0, atol=1e-6, equal_nan=True), (ci, name, w, list(want.w[:k]))
+
+
+def _snapshot(*arrays):
+    return [np.ascontiguousarray(a.numpy()).view(np.uint8).copy() for a in arrays]
+
+
+def _order_cases(qk, emu):
+    """Small launches of every kernel family, each returning the bytes it produced."""
+    K = 2048
+    cases = {}
+    for name in QUANT:
+        t = type_id(qk, name)
+        W = qk.synth.tensor_host(t, 67, K, seed=7)
+        x1 = np.random.default_rng(1).standard_normal((1, K)).astype(np.float32)
+        x5 = np.random.default_rng(5).standard_normal((5, K)).astype(np.float32)
+        x70 = np.random.default_rng(70).standard_normal((70, K)).astype(np.float32)
+
+        def gemv(x, W=W, t=t):
+            Y = emu.zeros((x.shape[0], 67), np.float32)
+            qk.gemv(t, emu.tensor(W.reshape(-1)), emu.tensor(x), 67, K, out=Y)
+            return _snapshot(Y)
+        cases[f"gemv {name} one row"] = lambda x1=x1, gemv=gemv: gemv(x1)
+        cases[f"gemv {name} five rows"] = lambda x5=x5, gemv=gemv: gemv(x5)
+        if name in ("q8_0", "iq3_xxs"):
+            cases[f"gemv {name} seventy rows"] = lambda x70=x70, gemv=gemv: gemv(x70)
+    Wf = np.random.default_rng(3).standard_normal((40, K)).astype(np.float16)
+    xf = np.random.default_rng(4).standard_normal((1, K)).astype(np.float32)
+
+    def dense():
+        Y = emu.zeros((1, 40), np.float32)
+        qk.gemv(qk.F16, emu.tensor(Wf.reshape(-1)), emu.tensor(xf), 40, K, out=Y)
+        return _snapshot(Y)
+    cases["gemv f16"] = dense
+    for down, E, k, F in (("iq4_xs", 8, 2, 256), ("q6_k", 16, 4, 512)):
+        hl = qk.synth.HostLayer(seed=E, n_ff=F, n_expert=E, n_used=k, down_type=type_id(qk, down))
+        for n in (1, 3, 12, 40):
+            x = np.random.default_rng(n).standard_normal((n, K)).astype(np.float32)
+
+            def moe(hl=hl, x=x, n=n):
+                layer = emu_util.layer_in_pool(qk, emu, hl)
+                ws = emu.workspace(qk.moe_workspace_bytes(layer, n))
+                sel, Y = emu.zeros((n, 160), np.uint8), emu.zeros((n, K), np.float32)
+                qk.moe_decode(layer, emu.tensor(x), ws, Y=Y, sel=sel)
+                return _snapshot(Y, sel)
+            cases[f"moe {down} {n} rows"] = moe
+    Wh = qk.synth.tensor_host(qk.Q6_K, 300, K, seed=300)
+    for b in (1, 3):
+        xh = np.random.default_rng(b).standard_normal((b, K)).astype(np.float32)
+
+        def head(xh=xh, b=b):
+            ws = emu.workspace(qk.head_workspace_bytes(300, b))
+            tok, logits = qk.head_argmax(emu.tensor(Wh.reshape(-1)), emu.tensor(xh), 300, K, ws, want_logits=True)
+            return _snapshot(tok, logits)
+        cases[f"head {b} rows"] = head
+    return cases
+
+
+FORMS = [{}, {"one_row": 1, "dense_reg": 1}, {"one_row": 1, "select_ranked": 0}, {"gemm_tiled": 1, "moe_rows": 1, "head_rows": 1}]
+
+
+@pytest.mark.parametrize("form_switches", FORMS, ids=["defaults", "streamed", "streamed-rounds", "tiled-rows"])
+def test_results_do_not_depend_on_the_order_of_the_threads(qk, emu, switches_back_to_defaults, form_switches):
+    """Between two barriers the host-side build runs the threads of a workgroup one after the other.  Two accesses
+    to LDS (or to a workspace) by different threads that need a barrier between them and have none are seen
+    writer-first under one order and reader-first under another, so every family of kernels, in every form, has to
+    give the same bits with the threads visited in ascending order, in descending order and in two random orders
+    drawn anew at every sweep.  (What this cannot see: orderings inside a wave that the hardware's lockstep
+    provides and the device compiler must keep.)"""
+    L = emu_util.emu_lib(qk)
+    for name_, v in form_switches.items():
+        qk.set_option(name_, v)
+    cases = _order_cases(qk, emu)
+    try:
+        L.emu_set_schedule(0, 1)
+        want = {k_: run() for k_, run in cases.items()}
+        for mode, seed in ((1, 1), (2, 11), (2, 12)):
+            L.emu_set_schedule(mode, seed)
+            for k_, run in cases.items():
+                got = run()
+                assert all(np.array_equal(a, b) for a, b in zip(got, want[k_])), (k_, mode, seed)
+    finally:
+        L.emu_set_schedule(0, 1)
