@@ -392,7 +392,7 @@ __global__ __launch_bounds__(CT) void head_q6k_coop_kernel(const uint8_t* __rest
 // The cooperative stream above splits K over the waves: per batch of 32 vocabulary rows partial tiles go through
 // LDS, one wave sums them and a barrier closes the batch -- 4,748 batches for the 151,936-row head, and it is
 // that fixed cost per batch which holds 16 rows at a third of the memory roofline.  Here a work item is a block
-// of 128 vocabulary rows and a wave owns 16 of them for all of K (rows_tile, qk_rows.h): its accumulators are
+// of 128 vocabulary rows and a wave owns 16 of them for all of K (rows_stream, qk_rows.h): its accumulators are
 // logits, a thread keeps the best (logit, id) of each of its four activation rows across its items (its rows
 // ascend, so `>` keeps the lowest id), and the fold over the workgroup, the candidates and the last workgroup are
 // those of the kernel above.  64 KB of LDS, two workgroups per CU.
@@ -403,7 +403,7 @@ __global__ __launch_bounds__(MR_THREADS, 4) void head_q6k_rows_kernel(const uint
     using G = RowsGeo<QKK_Q6_K, 1>;
     constexpr uint32_t K = 2048, ROW = (K / 256) * G::FB;
     QK_DYN_LDS(uint8_t, smem);
-    __shared__ MfmaTables tab; // Q6_K reads no table; rows_tile takes the reference
+    __shared__ MfmaTables tab; // Q6_K reads no table; rows_stream takes the reference
     __shared__ uint32_t s_last;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, j = lane & 15, g = lane >> 4;
     const uint8_t* tens[1] = {W};
@@ -414,20 +414,22 @@ __global__ __launch_bounds__(MR_THREADS, 4) void head_q6k_rows_kernel(const uint
     uint32_t bi[4];
 #pragma unroll
     for (int e = 0; e < 4; e++) { bv[e] = ARG_FLOOR; bi[e] = 0xFFFFFFFFu; }
-    for (uint32_t item = blockIdx.x; item < items; item += gridDim.x) {
-        __syncthreads(); // the previous item's LDS is consumed
-        float4v acc[1];
-        rows_tile<QKK_Q6_K, 1>(tens, (size_t)item * MR_ROWS * ROW, ROW, last_piece, K / 256, arow, smem, tab, tid, acc);
-        const uint32_t row = item * MR_ROWS + 16 * wave + j; // rows behind V were read from clamped addresses: dropped here
+    // this workgroup's items blockIdx.x, blockIdx.x + gridDim.x, ... as one pipeline
+    const uint32_t mine = blockIdx.x < items ? (items - blockIdx.x + gridDim.x - 1) / gridDim.x : 0u;
+    if (mine)
+        rows_stream<QKK_Q6_K, 1>(
+            tens, mine, [&](uint32_t b) { return (size_t)(blockIdx.x + b * gridDim.x) * MR_ROWS * ROW; }, ROW, last_piece, K / 256,
+            arow, smem, tab, tid, [&](uint32_t b, const float4v(&acc)[1]) {
+                const uint32_t row = (blockIdx.x + b * gridDim.x) * MR_ROWS + 16 * wave + j; // rows behind V were read from clamped addresses: dropped here
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const uint32_t t = 4 * g + e;
-            if (t < batch && row < V) {
-                if (logits_out) logits_out[(size_t)t * V + row] = acc[0][e];
-                if (acc[0][e] > bv[e]) { bv[e] = acc[0][e]; bi[e] = row; }
-            }
-        }
-    }
+                for (int e = 0; e < 4; e++) {
+                    const uint32_t t = 4 * g + e;
+                    if (t < batch && row < V) {
+                        if (logits_out) logits_out[(size_t)t * V + row] = acc[0][e];
+                        if (acc[0][e] > bv[e]) { bv[e] = acc[0][e]; bi[e] = row; }
+                    }
+                }
+            });
     __syncthreads();
     // per activation row: the 128 threads that hold its outputs (16 rows x 8 waves), then the workgroups
     float* s_v = (float*)smem;

@@ -14,7 +14,8 @@
 // qk_gemm_tiled.hip), the next step's pieces and activations in flight in registers during the arithmetic;
 // 64 KB of LDS and under 128 registers per lane, so two workgroups share a CU.  Decoder: BFrag<TYPE>::step, the
 // cooperative stream's, so the same exactness (activations hi + lo, weights hi (+ lo)).
-// Work item = (active expert, block of 128 rows); its pair tiles of 16 follow one another.
+// Work item = (active expert, 1, 2 or 4 consecutive blocks of 128 rows); its pair tiles of 16 follow one another,
+// and within a tile the K steps of all its blocks are one pipeline (rows_stream, qk_rows.h).
 // Behind the "moe_rows" switch until it has been run and timed on a device; the shared expert keeps the
 // kernels of qk_moe_mfma.hip (it is one dense expert for every token).
 // (reference shaders/moe_gateup_iq3_grouped_coopmat.comp:46-217, moe_down_iq4_grouped_coopmat.comp:45-166.)
@@ -30,7 +31,7 @@ namespace qk {
 template <int TYPE, bool GATEUP>
 __global__ __launch_bounds__(MR_THREADS, 4) void moe_rows_kernel(const uint8_t* __restrict__ W0, const uint8_t* __restrict__ W1,
                                                                  const float* __restrict__ X, MoeWs ws,
-                                                                 const qkk_sel* __restrict__ sel, MoeDims d, uint32_t N)
+                                                                 const qkk_sel* __restrict__ sel, MoeDims d, uint32_t N, uint32_t bpi)
 {
     constexpr int NT = GATEUP ? 2 : 1;
     using G = RowsGeo<TYPE, NT>;
@@ -49,10 +50,12 @@ __global__ __launch_bounds__(MR_THREADS, 4) void moe_rows_kernel(const uint8_t* 
     tens[0] = W0;
     if constexpr (GATEUP) tens[1] = W1;
 
-    for (uint32_t item = blockIdx.x; item < n_active * blocks_per_expert; item += gridDim.x) {
-        const ActiveExpert ae = active_expert(ws, item / blocks_per_expert, d, N);
-        const uint32_t row0 = (item % blocks_per_expert) * MR_ROWS;
-        const size_t base = ((size_t)ae.expert * R + row0) * stride; // the block's first row, both tensors
+    const uint32_t groups = blocks_per_expert / bpi; // a work item: bpi consecutive blocks of an active expert
+
+    for (uint32_t item = blockIdx.x; item < n_active * groups; item += gridDim.x) {
+        const ActiveExpert ae = active_expert(ws, item / groups, d, N);
+        const uint32_t row0 = (item % groups) * bpi * MR_ROWS;
+        const size_t base = ((size_t)ae.expert * R + row0) * stride; // the item's first row, both tensors
 
         for (uint32_t t0 = 0; t0 < ae.count; t0 += 16) {
             const uint32_t np = min(16u, ae.count - t0);
@@ -66,19 +69,21 @@ __global__ __launch_bounds__(MR_THREADS, 4) void moe_rows_kernel(const uint8_t* 
             }
             __syncthreads();
             const float* arow = GATEUP ? X + (size_t)s_tok[j] * d.H : ws.h + ((size_t)s_tok[j] * (d.k + 1) + s_slot[j]) * d.F;
-            float4v acc[NT];
-            rows_tile<TYPE, NT>(tens, base, stride, last_piece, nfrag, arow, smem, tab, tid, acc);
-            // D[4 g + e][j]: pair 4 g + e of the tile, row 16 wave + j of the block
-            const uint32_t row = row0 + 16 * wave + j;
+            rows_stream<TYPE, NT>(
+                tens, bpi, [&](uint32_t b) { return base + (size_t)b * MR_ROWS * stride; }, stride, last_piece, nfrag, arow, smem,
+                tab, tid, [&](uint32_t b, const float4v(&acc)[NT]) {
+                    // D[4 g + e][j]: pair 4 g + e of the tile, row 16 wave + j of block b
+                    const uint32_t row = row0 + b * MR_ROWS + 16 * wave + j;
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const uint32_t r = 4 * g + e;
-                if (r < np) {
-                    const size_t rec = (size_t)s_tok[r] * (d.k + 1) + s_slot[r];
-                    if constexpr (GATEUP) ws.h[rec * d.F + row] = (acc[0][e] / (1.f + expf(-acc[0][e]))) * acc[NT - 1][e];
-                    else ws.contrib[rec * d.H + row] = s_wt[r] * acc[0][e];
-                }
-            }
+                    for (int e = 0; e < 4; e++) {
+                        const uint32_t r = 4 * g + e;
+                        if (r < np) {
+                            const size_t rec = (size_t)s_tok[r] * (d.k + 1) + s_slot[r];
+                            if constexpr (GATEUP) ws.h[rec * d.F + row] = (acc[0][e] / (1.f + expf(-acc[0][e]))) * acc[NT - 1][e];
+                            else ws.contrib[rec * d.H + row] = s_wt[r] * acc[0][e];
+                        }
+                    }
+                });
         }
     }
 }
@@ -91,9 +96,14 @@ static void launch_rows(const uint8_t* W0, const uint8_t* W1, const float* X, co
     static const bool raised = ((void)hipFuncSetAttribute((const void*)moe_rows_kernel<TYPE, GATEUP>,
                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)G::LDS_BYTES), true);
     (void)raised;
-    const uint32_t items = experts * ((GATEUP ? d.F : d.H) / MR_ROWS); // an upper bound: the active experts are known on the device
-    const uint32_t blocks = std::max(1u, std::min(items, 2 * (persistent_blocks() / 4)));
-    hipLaunchKernelGGL((moe_rows_kernel<TYPE, GATEUP>), dim3(blocks), dim3(MR_THREADS), G::LDS_BYTES, st, W0, W1, X, ws, sel, d, N);
+    // Work items of 4, 2 or 1 consecutive blocks of an expert: as long as there are items for every resident
+    // workgroup (two per CU), fewer and longer ones -- the wait for the first fragments is paid once per item.
+    // `experts` is an upper bound, the active ones are known on the device only.
+    const uint32_t per_expert = (GATEUP ? d.F : d.H) / MR_ROWS, slots = persistent_blocks() / 2;
+    uint32_t bpi = 4;
+    while (bpi > 1 && (per_expert % bpi || experts * (per_expert / bpi) < slots)) bpi /= 2;
+    const uint32_t blocks = std::max(1u, std::min(experts * (per_expert / bpi), slots));
+    hipLaunchKernelGGL((moe_rows_kernel<TYPE, GATEUP>), dim3(blocks), dim3(MR_THREADS), G::LDS_BYTES, st, W0, W1, X, ws, sel, d, N, bpi);
 }
 
 // Whether the row-split form covers the layer: whole K steps of 256 weights, whole blocks of 128 rows, the

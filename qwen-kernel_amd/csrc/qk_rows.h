@@ -3,7 +3,7 @@
 // so its accumulators are its outputs.  The activation operand of the 16 rows lives in LDS in operand order,
 // converted to hi + lo halves once per workgroup and K step of 256 weights and read by every wave; the rows'
 // fragments of a K step reach LDS as the aligned 16-byte pieces that cover them, the next step's pieces and
-// activations in flight in registers during the arithmetic.  Decoder: BFrag<TYPE>::step, the cooperative
+// activations in flight in registers during the arithmetic, from one block of rows into the next.  Decoder: BFrag<TYPE>::step, the cooperative
 // stream's (qk_coop.h), so the same exactness (activations hi + lo, weights hi (+ lo)).
 // Users: the routed experts' projections (qk_moe_rows.hip), the LM head for 2..16 rows (qk_head.hip).
 #pragma once
@@ -25,16 +25,20 @@ struct RowsGeo {
     static constexpr uint32_t LDS_BYTES = W_BYTES + 2 * A_BYTES;
 };
 
-// acc[t][e] = sum over K of (row 16 wave + j of tensor t's block) . (activation row 4 g + e), lane = 16 g + j.
-// tens[t] + base: the block's first row in tensor t (rows `stride` bytes apart, nfrag fragments each); reads are
-// clamped to the 16-byte piece at `last_piece`, the tensors' last one.  arow: the activation row of THIS
-// thread's lane j (thread (wave, lane) converts the operand of lane `lane` for instruction `wave` of a step).
+// For each of `nblk` blocks of 128 weight rows in turn: acc[t][e] = sum over K of (row 16 wave + j of the block in
+// tensor t) . (activation row 4 g + e), lane = 16 g + j, handed to done(b, acc).  base_of(b): byte offset of block
+// b's first row in every tensor (rows `stride` bytes apart, nfrag fragments each); reads are clamped to the
+// 16-byte piece at `last_piece`, the tensors' last one.  arow: the activation row of THIS thread's lane j (thread
+// (wave, lane) converts the operand of lane `lane` for instruction `wave` of a K step).  The K steps of all blocks
+// form ONE pipeline: the first fragments of block b + 1 are in flight during the last step of block b, so the
+// wait for memory at the head is paid once per call, not once per block.  With nfrag <= 2 the activation operand
+// of every K step fits the two buffers and is converted once per call.
 // smem: RowsGeo::LDS_BYTES; the caller has a barrier between the previous user of smem and this call, and one
 // between this call and the next user.
-template <int TYPE, int NT>
-__device__ __forceinline__ void rows_tile(const uint8_t* const (&tens)[NT], size_t base, size_t stride, size_t last_piece,
-                                          uint32_t nfrag, const float* arow, uint8_t* smem, const MfmaTables& tab, int tid,
-                                          float4v (&acc)[NT])
+template <int TYPE, int NT, class BaseOf, class Done>
+__device__ __forceinline__ void rows_stream(const uint8_t* const (&tens)[NT], uint32_t nblk, BaseOf base_of, size_t stride,
+                                            size_t last_piece, uint32_t nfrag, const float* arow, uint8_t* smem,
+                                            const MfmaTables& tab, int tid, Done done)
 {
     using G = RowsGeo<TYPE, NT>;
     using F = typename G::F;
@@ -50,9 +54,10 @@ __device__ __forceinline__ void rows_tile(const uint8_t* const (&tens)[NT], size
     // the compiler forms the row offsets once per kernel and keeps them): four of them kept per thread across
     // the arithmetic cost more registers than the dozen integer operations they take.
     u32x4 ld[NLD];
-    const auto fetch = [&](uint32_t f) {
+    const auto fetch = [&](uint32_t b, uint32_t f) {
         uint32_t me = (uint32_t)tid;
         asm volatile("" : QK_REG(me));
+        const size_t base = base_of(b);
 #pragma unroll
         for (int n = 0; n < NLD; n++) {
             const uint32_t p = min(me + MR_THREADS * n, PIECES - 1);
@@ -69,8 +74,6 @@ __device__ __forceinline__ void rows_tile(const uint8_t* const (&tens)[NT], size
             if (PIECES % MR_THREADS == 0 || n + 1 < NLD || p < PIECES) *(u32x4*)(s_w + (p / NPW) * WIN + (p % NPW) * 16) = ld[n];
         }
     };
-    // this lane's weight rows: row 16 wave + j of the block, in every tensor
-    const size_t my_at = base + (size_t)(16 * wave + j) * stride;
     const uint32_t acut = F::LAYOUT == 0 ? 64 * g + 8 * wave : 128 * (g >> 1) + 32 * (wave >> 1) + 16 * (g & 1) + 8 * (wave & 1);
     float4 ar[2];
     const auto load_a = [&](uint32_t f) {
@@ -89,30 +92,39 @@ __device__ __forceinline__ void rows_tile(const uint8_t* const (&tens)[NT], size
         dstp[0] = hi;
         dstp[64] = lo;
     };
-    fetch(0);
+    const bool a_stays = nfrag <= 2; // step s reads buffer s & 1 = fragment s % nfrag for every block: filled by steps 0 and 1
+    fetch(0, 0);
     load_a(0);
     commit();
     commit_a(0);
     __syncthreads();
 
-#pragma unroll
-    for (int t = 0; t < NT; t++) acc[t] = float4v{0.f, 0.f, 0.f, 0.f};
+    float4v acc[NT];
+    const uint32_t steps = nblk * nfrag;
+    uint32_t b = 0, f = 0; // block and fragment of step s
 #pragma unroll 1
-    for (uint32_t f = 0; f < nfrag; f++) {
-        const uint32_t buf = f & 1u;
-        const bool more = f + 1 < nfrag; // workgroup-uniform
-        if (more) {
-            fetch(f + 1);
-            load_a(f + 1);
+    for (uint32_t s = 0; s < steps; s++) {
+        const uint32_t buf = s & 1u;
+        const bool more = s + 1 < steps;                  // workgroup-uniform
+        const bool wrap = f + 1 == nfrag;                 // this step closes its block
+        const uint32_t nb = wrap ? b + 1 : b, nf = wrap ? 0u : f + 1;
+        const bool conv = more && !(a_stays && s + 1 >= 2); // the next step's activations still have to be converted
+        if (more) fetch(nb, nf);
+        if (conv) load_a(nf);
+        if (f == 0) {
+#pragma unroll
+            for (int t = 0; t < NT; t++) acc[t] = float4v{0.f, 0.f, 0.f, 0.f};
         }
-        // one tensor's tile after the other: one set of fragment registers and decode temporaries alive at a
-        // time; the waves of the SIMD fill each other's matrix-instruction latencies
+        // this lane's weight rows: row 16 wave + j of the block, in every tensor.  One tensor's tile after the
+        // other: one set of fragment registers and decode temporaries alive at a time; the waves of the SIMD
+        // fill each other's matrix-instruction latencies
+        const uint32_t skew = (uint32_t)((base_of(b) + (size_t)(16 * wave + j) * stride + (size_t)f * FB) & 15);
         const half8* ap = (const half8*)(s_a + buf * G::A_BYTES) + lane;
 #pragma unroll
         for (int t = 0; t < NT; t++) {
             asm volatile("" ::: "memory"); // the second tile reads its activation operands again rather than keeping the first's 64 registers
             F w;
-            w.load(s_w + (size_t)(t * MR_ROWS + 16 * wave + j) * WIN + ((my_at + (size_t)f * FB) & 15), 0, g);
+            w.load(s_w + (size_t)(t * MR_ROWS + 16 * wave + j) * WIN + skew, 0, g);
             float4v part = float4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int i = 0; i < 8; i++) {
@@ -127,12 +139,15 @@ __device__ __forceinline__ void rows_tile(const uint8_t* const (&tens)[NT], size
             const float sc = w.post();
             acc[t] += float4v{sc * part[0], sc * part[1], sc * part[2], sc * part[3]};
         }
+        if (wrap) done(b, acc);
         if (more) {
             __syncthreads(); // every wave has read this step's rows
             commit();
-            commit_a(buf ^ 1u);
+            if (conv) commit_a(buf ^ 1u);
             __syncthreads(); // the next step's rows and activations are in place
         }
+        b = nb;
+        f = nf;
     }
 }
 

@@ -337,13 +337,15 @@ def test_expert_major_moe_inside_its_tensors(qk, orc, emu, down, n):
     qk.moe_workspace_status()   # the cleared workspace raised no flag
 
 
-@pytest.mark.parametrize("down,n,E,k,F", [("iq4_xs", 16, 8, 2, 256), ("q6_k", 40, 8, 2, 256), ("iq4_xs", 70, 4, 2, 512), ("q6_k", 12, 16, 8, 1024)])
+@pytest.mark.parametrize("down,n,E,k,F", [("iq4_xs", 16, 8, 2, 256), ("q6_k", 40, 8, 2, 256), ("iq4_xs", 70, 4, 2, 512), ("q6_k", 12, 16, 8, 1024),
+                                          ("iq4_xs", 20, 2, 1, 256)])
 def test_row_split_expert_kernels_inside_their_tensors(qk, orc, emu, down, n, E, k, F):
     """The routed experts' projections with the waves splitting the weight rows (the "moe_rows" switch): 12 to 70
     rows, so that experts hold from a few pairs to several tiles of 16 (70 rows x 2 picks on 4 experts: three
     tiles, the last one partial), n_ff of two to eight blocks of 128 rows, the LAST expert among the picks and the
-    tensors ending at guard pages; against the oracle, and the same ids and (to rounding of the sums) the same
-    outputs as the K-split kernels."""
+    tensors ending at guard pages; work items of four, two and one block of rows (the host-side build's "device" has
+    four CUs, so eight resident workgroups decide); against the oracle, and the same ids and (to rounding of the sums)
+    the same outputs as the K-split kernels."""
     hl = qk.synth.HostLayer(seed=31 + n, n_ff=F, n_expert=E, n_used=k, down_type=type_id(qk, down))
     x = rows_that_pick_the_last_expert(hl, n, seed=n)
     base = moe_case(qk, orc, emu, hl, x)
