@@ -12,6 +12,11 @@
 //   qk moe [seed] [iters] [slots] [experts]   one fused MoE layer (synthetic weights in place of a
 //                                     model's layer index), defaults 0 200 1 256
 //   qk head [batch] [iters]           the LM head 151936 x 2048 Q6_K with the argmax fused
+// and, on the tensors of a model file named by QK_GGUF (reference src/main.cpp:846-915, 920-1254):
+//   qk list [prefix]                  the file's tensors: name, type, dimensions
+//   qk gguf <tensor> [iters]          y = W x on a named tensor (a 3-D tensor: its first slice, expert 0)
+//   qk layer [layer] [iters] [slots]  the fused MoE step on the tensors blk.<layer>.ffn_* (the reference's
+//                                     `qk moe [layer]`; `moe` here keeps its synthetic weights)
 //
 // The weights are seeded random valid blocks (every bit pattern of the quant fields is valid; the
 // fp16 scales are |N(0,1)| * 1e-3), the activations N(0,1).  Iterations alternate over a ring of
@@ -32,6 +37,7 @@
 #include <string>
 #include <vector>
 
+#include "../../include/qk_gguf.h"
 #include "../../include/qk_kernels.h"
 
 namespace {
@@ -210,6 +216,25 @@ bool verdict(const char* what, double err, double bar)
     return err <= bar;
 }
 
+// Second opinion on y = W x: bit-exact dequantisation, then the dense fp32 product (rows in pieces of at most 256 MiB)
+bool check_gemv(int type, const uint8_t* W, const float* x, float* y, uint32_t M, uint32_t K, hipStream_t st)
+{
+    QK_OK(qkk_gemv(type, W, x, y, M, K, 1, st));
+    const std::vector<float> got = to_host(y, M);
+    std::vector<float> want(M);
+    const uint32_t piece = (uint32_t)std::max<uint64_t>(1, std::min<uint64_t>(M, (64ull << 20) / K));
+    float* dense = device_zeros<float>((size_t)piece * K);
+    float* y2 = device_zeros<float>(piece);
+    for (uint32_t r0 = 0; r0 < M; r0 += piece) {
+        const uint32_t n = std::min(piece, M - r0);
+        QK_OK(qkk_dequant(type, W + (size_t)r0 * qkk_row_bytes(type, K), dense, (uint64_t)n * K, st));
+        QK_OK(qkk_gemv(QKK_F32, dense, x, y2, n, K, 1, st));
+        HIP_OK(hipMemcpy(want.data() + r0, y2, (size_t)n * 4, hipMemcpyDeviceToHost));
+    }
+    HIP_OK(hipFree(dense)); HIP_OK(hipFree(y2));
+    return verdict("against dequantise + dense fp32 product", rel_maxabs(got, want), 1e-3);
+}
+
 // y = W x for one format: ring of tensors, time, cross-check against dequantise + dense fp32 GEMV
 bool case_gemv(const Format& f, uint32_t M, uint32_t K, uint32_t iters)
 {
@@ -228,22 +253,9 @@ bool case_gemv(const Format& f, uint32_t M, uint32_t K, uint32_t iters)
     hipStream_t st = nullptr;
     const double us = time_us([&](uint32_t r) { QK_OK(qkk_gemv(f.type, W[r], x, y, M, K, 1, st)); }, iters, ring, st);
     print_line(us, (double)wbytes + 4.0 * K + 4.0 * M, 2.0 * M * K);
-    // second opinion: bit-exact dequantisation, then the dense fp32 product (rows in pieces of at most 256 MiB)
-    QK_OK(qkk_gemv(f.type, W[0], x, y, M, K, 1, st));
-    const std::vector<float> got = to_host(y, M);
-    std::vector<float> want(M);
-    const uint32_t piece = (uint32_t)std::max<uint64_t>(1, std::min<uint64_t>(M, (64ull << 20) / K));
-    float* dense = device_zeros<float>((size_t)piece * K);
-    float* y2 = device_zeros<float>(piece);
-    for (uint32_t r0 = 0; r0 < M; r0 += piece) {
-        const uint32_t n = std::min(piece, M - r0);
-        QK_OK(qkk_dequant(f.type, W[0] + (size_t)r0 * qkk_row_bytes(f.type, K), dense, (uint64_t)n * K, st));
-        QK_OK(qkk_gemv(QKK_F32, dense, x, y2, n, K, 1, st));
-        HIP_OK(hipMemcpy(want.data() + r0, y2, (size_t)n * 4, hipMemcpyDeviceToHost));
-    }
-    const bool ok = verdict("against dequantise + dense fp32 product", rel_maxabs(got, want), 1e-3);
+    const bool ok = check_gemv(f.type, W[0], x, y, M, K, st);
     for (uint8_t* p : W) HIP_OK(hipFree(p));
-    HIP_OK(hipFree(x)); HIP_OK(hipFree(y)); HIP_OK(hipFree(dense)); HIP_OK(hipFree(y2));
+    HIP_OK(hipFree(x)); HIP_OK(hipFree(y));
     return ok;
 }
 
@@ -310,22 +322,16 @@ Layer make_layer(uint64_t seed, int down_type, uint32_t E)
     return out;
 }
 
-bool case_moe(uint32_t seed, uint32_t iters, uint32_t slots, uint32_t E)
+// The fused step on a ring of layers of one shape: time, per stage, and the row-wise launches against the
+// expert-major path (reference caseMoe, src/main.cpp:920-1254)
+bool run_moe(std::vector<Layer>& layers, uint32_t iters, uint32_t slots, uint64_t seed)
 {
-    if (slots < 1 || slots > 4096 || E < 8 || E > QKK_MAX_EXPERTS) {
-        fprintf(stderr, "qk: slots %u outside 1..4096 or experts %u outside 8..%u\n", slots, E, QKK_MAX_EXPERTS);
-        return false;
-    }
-    const uint32_t ring = 4, H = 2048;
-    const int down = slots == 1 ? QKK_IQ4_XS : QKK_Q6_K; // the reference's 35B model mixes both down types
-    printf("== fused moe layer (synthetic, seed %u): %u experts, %u slot(s), down %s, iters=%u, ring of %u layers\n", seed, E,
-           slots, down == QKK_Q6_K ? "q6_k" : "iq4_xs", iters, ring);
-    std::vector<Layer> layers;
-    for (uint32_t r = 0; r < ring; r++) layers.push_back(make_layer(seed * 8 + r, down, E));
+    const qkk_moe_layer& L0 = layers[0].L;
+    const uint32_t ring = (uint32_t)layers.size(), H = L0.n_embd, F = L0.n_ff, E = L0.n_expert, k = L0.n_used;
     float* X = to_device(random_rows((size_t)ring * slots * H, seed + 43));
     float* Y = device_zeros<float>((size_t)slots * H);
     qkk_sel* sel = device_zeros<qkk_sel>(slots);
-    const size_t wsb = qkk_moe_workspace_bytes(&layers[0].L, std::max(slots, 16u));
+    const size_t wsb = qkk_moe_workspace_bytes(&L0, std::max(slots, 16u));
     uint8_t* ws = device_zeros<uint8_t>(wsb);
     hipStream_t st = nullptr;
     auto step = [&](uint32_t r) { QK_OK(qkk_moe_decode(&layers[r].L, X + (size_t)r * slots * H, Y, sel, ws, wsb, slots, st)); };
@@ -335,15 +341,15 @@ bool case_moe(uint32_t seed, uint32_t iters, uint32_t slots, uint32_t E)
     std::vector<qkk_sel> hs(slots);
     HIP_OK(hipMemcpy(hs.data(), sel, slots * sizeof(qkk_sel), hipMemcpyDeviceToHost));
     std::vector<uint32_t> ids;
-    for (const qkk_sel& s : hs) ids.insert(ids.end(), s.ids, s.ids + 8);
+    for (const qkk_sel& s : hs) ids.insert(ids.end(), s.ids, s.ids + k);
     std::sort(ids.begin(), ids.end());
     const size_t distinct = std::unique(ids.begin(), ids.end()) - ids.begin();
-    const double per_expert = 2.0 * 512 * qkk_row_bytes(QKK_IQ3_XXS, 2048) + 2048.0 * qkk_row_bytes(down, 512);
-    const double bytes = (double)E * 2048 * 4 + 2048 * 4 + distinct * per_expert + 2.0 * 512 * qkk_row_bytes(QKK_Q8_0, 2048) +
-                         2048.0 * qkk_row_bytes(QKK_Q8_0, 512) + slots * (2.0 * H * 4 + 160);
-    print_line(us, bytes, slots * (2.0 * E * H + 9 * 3 * 2.0 * 512 * H));
+    const double per_expert = 2.0 * F * qkk_row_bytes(L0.gu_type, H) + (double)H * qkk_row_bytes(L0.down_type, F);
+    const double bytes = (double)E * H * 4 + H * 4 + distinct * per_expert + 2.0 * F * qkk_row_bytes(QKK_Q8_0, H) +
+                         (double)H * qkk_row_bytes(QKK_Q8_0, F) + slots * (2.0 * H * 4 + 160);
+    print_line(us, bytes, slots * (2.0 * E * H + (k + 1) * 3 * 2.0 * F * H));
     printf("     %zu distinct experts; picks of row 0:", distinct);
-    for (int i = 0; i < 8; i++) printf(" %u(%.3f)", hs[0].ids[i], hs[0].w[i]);
+    for (uint32_t i = 0; i < k; i++) printf(" %u(%.3f)", hs[0].ids[i], hs[0].w[i]);
     printf(" shared gate %.3f\n", hs[0].w_shared);
     // per stage, as the reference's QK_STEP_PROF does (src/main.cpp:4591-4632)
     for (uint32_t mask : {QKK_STAGE_ROUTE, QKK_STAGE_GATEUP, QKK_STAGE_DOWN}) {
@@ -356,18 +362,19 @@ bool case_moe(uint32_t seed, uint32_t iters, uint32_t slots, uint32_t E)
     const std::vector<float> got = to_host(Y, (size_t)slots * H);
     bool ok = true;
     if (slots > 10) printf("check: none (above ten rows both calls would take the expert-major path)\n");
+    else if (H != 2048) printf("check: none (the expert-major path takes n_embd = 2048 only)\n");
     else {
         std::vector<float> x0 = to_host(X, (size_t)slots * H), x16((size_t)16 * H);
         for (uint32_t r = 0; r < 16; r++) memcpy(&x16[(size_t)r * H], &x0[(size_t)(r % slots) * H], H * 4);
         float* X16 = to_device(x16);
         float* Y16 = device_zeros<float>((size_t)16 * H);
         qkk_sel* sel16 = device_zeros<qkk_sel>(16);
-        QK_OK(qkk_moe_decode(&layers[0].L, X16, Y16, sel16, ws, wsb, 16, st));
+        QK_OK(qkk_moe_decode(&L0, X16, Y16, sel16, ws, wsb, 16, st));
         std::vector<float> want = to_host(Y16, (size_t)slots * H);
         std::vector<qkk_sel> h16(16);
         HIP_OK(hipMemcpy(h16.data(), sel16, 16 * sizeof(qkk_sel), hipMemcpyDeviceToHost));
         bool same_ids = true;
-        for (uint32_t r = 0; r < slots; r++) same_ids = same_ids && !memcmp(hs[r].ids, h16[r].ids, 8 * 4);
+        for (uint32_t r = 0; r < slots; r++) same_ids = same_ids && !memcmp(hs[r].ids, h16[r].ids, k * 4);
         printf("check: picks equal on both paths -> %s\n", same_ids ? "OK" : "FAIL");
         ok = verdict("row-wise launches against the expert-major path", rel_maxabs(got, want), 1e-3) && same_ids;
         HIP_OK(hipFree(X16)); HIP_OK(hipFree(Y16)); HIP_OK(hipFree(sel16));
@@ -376,6 +383,137 @@ bool case_moe(uint32_t seed, uint32_t iters, uint32_t slots, uint32_t E)
         for (void* p : l.owned) HIP_OK(hipFree(p));
     HIP_OK(hipFree(X)); HIP_OK(hipFree(Y)); HIP_OK(hipFree(sel)); HIP_OK(hipFree(ws));
     return ok;
+}
+
+bool case_moe(uint32_t seed, uint32_t iters, uint32_t slots, uint32_t E)
+{
+    if (slots < 1 || slots > 4096 || E < 8 || E > QKK_MAX_EXPERTS) {
+        fprintf(stderr, "qk: slots %u outside 1..4096 or experts %u outside 8..%u\n", slots, E, QKK_MAX_EXPERTS);
+        return false;
+    }
+    const uint32_t ring = 4;
+    const int down = slots == 1 ? QKK_IQ4_XS : QKK_Q6_K; // the reference's 35B model mixes both down types
+    printf("== fused moe layer (synthetic, seed %u): %u experts, %u slot(s), down %s, iters=%u, ring of %u layers\n", seed, E,
+           slots, down == QKK_Q6_K ? "q6_k" : "iq4_xs", iters, ring);
+    std::vector<Layer> layers;
+    for (uint32_t r = 0; r < ring; r++) layers.push_back(make_layer(seed * 8 + r, down, E));
+    return run_moe(layers, iters, slots, seed);
+}
+
+// ---- the tensors of a model file ----------------------------------------------------------------
+
+const char* type_name(uint32_t t)
+{
+    switch (t) {
+    case QKK_F32: return "f32";
+    case QKK_F16: return "f16";
+    case QKK_Q8_0: return "q8_0";
+    case QKK_Q6_K: return "q6_k";
+    case QKK_IQ4_XS: return "iq4_xs";
+    case QKK_IQ3_XXS: return "iq3_xxs";
+    default: return "other";
+    }
+}
+
+// The model file: QK_GGUF, as in the reference (src/main.cpp:846-856: no compiled-in default)
+qkg_file* open_model()
+{
+    const char* path = getenv("QK_GGUF");
+    if (!path || !*path) {
+        fprintf(stderr, "qk: no model path. Set QK_GGUF=/path/to/model.gguf\n");
+        exit(1);
+    }
+    qkg_file* f = qkg_open(path);
+    if (!f) {
+        fprintf(stderr, "qk: %s: %s\n", path, qkk_last_error());
+        exit(1);
+    }
+    return f;
+}
+
+bool case_list(const char* prefix)
+{
+    qkg_file* f = open_model();
+    printf("gguf v%u, %u shard(s), %llu tensors\n", qkg_version(f), qkg_n_shards(f), (unsigned long long)qkg_n_tensors(f));
+    for (uint64_t i = 0; i < qkg_n_tensors(f); i++) {
+        qkg_tensor t;
+        if (qkg_tensor_at(f, i, &t) != QKK_OK) continue;
+        if (prefix && strncmp(t.name, prefix, strlen(prefix))) continue;
+        printf("%-40s %-8s [%llu, %llu, %llu, %llu] %.1f MiB\n", t.name, type_name(t.type), (unsigned long long)t.ne[0],
+               (unsigned long long)t.ne[1], (unsigned long long)t.ne[2], (unsigned long long)t.ne[3], t.nbytes / 1048576.0);
+    }
+    qkg_close(f);
+    return true;
+}
+
+// y = W x on a tensor of the file (reference caseGguf, src/main.cpp:858-915)
+bool case_gguf(const char* name, uint32_t iters)
+{
+    qkg_file* f = open_model();
+    qkg_tensor t;
+    if (qkg_find(f, name, &t) != QKK_OK) {
+        fprintf(stderr, "qk: tensor '%s' not found (try: qk list)\n", name);
+        qkg_close(f);
+        return false;
+    }
+    const uint32_t K = (uint32_t)t.ne[0], M = (uint32_t)t.ne[1];
+    const size_t row = qkk_row_bytes((int)t.type, K);
+    printf("== gguf %s  %s  ne=[%llu,%llu,%llu]\n", name, type_name(t.type), (unsigned long long)t.ne[0],
+           (unsigned long long)t.ne[1], (unsigned long long)t.ne[2]);
+    if (!row || t.n_dims < 2) {
+        fprintf(stderr, "qk: no kernel for a %u-dimensional tensor of type %s\n", t.n_dims, type_name(t.type));
+        qkg_close(f);
+        return false;
+    }
+    if (t.ne[2] > 1) printf("3-D tensor: its first slice (expert 0)\n");
+    const size_t wbytes = (size_t)M * row;
+    printf("gemv M=%u K=%u, W %.1f MiB\n", M, K, wbytes / 1048576.0);
+    uint8_t* W = nullptr;
+    HIP_OK(hipMalloc((void**)&W, std::max<size_t>(wbytes, 16)));
+    HIP_OK(hipMemcpy(W, t.data, wbytes, hipMemcpyHostToDevice));
+    qkg_close(f);
+    float* x = to_device(random_rows(K, 43));
+    float* y = device_zeros<float>(M);
+    hipStream_t st = nullptr;
+    const double us = time_us([&](uint32_t) { QK_OK(qkk_gemv((int)t.type, W, x, y, M, K, 1, st)); }, iters, 1, st);
+    print_line(us, (double)wbytes + 4.0 * K + 4.0 * M, 2.0 * M * K);
+    bool ok = true;
+    if (t.type == QKK_F32) printf("check: none (the dense fp32 product is the second opinion of the others)\n");
+    else ok = check_gemv((int)t.type, W, x, y, M, K, st);
+    HIP_OK(hipFree(W)); HIP_OK(hipFree(x)); HIP_OK(hipFree(y));
+    return ok;
+}
+
+// The fused MoE step on the tensors of one layer of the file (reference caseMoe, src/main.cpp:920-1254)
+bool case_layer(uint32_t layer, uint32_t iters, uint32_t slots)
+{
+    if (slots < 1 || slots > 4096) {
+        fprintf(stderr, "qk: slots %u outside 1..4096\n", slots);
+        return false;
+    }
+    qkg_file* f = open_model();
+    qkg_moe_tensors mt;
+    if (qkg_moe_layer(f, layer, &mt) != QKK_OK) {
+        fprintf(stderr, "qk: layer %u: %s\n", layer, qkk_last_error());
+        qkg_close(f);
+        return false;
+    }
+    printf("== fused moe layer blk.%u: n_embd %u, n_ff %u, %u experts, %u used, down %s, %u slot(s), iters=%u\n", layer, mt.n_embd,
+           mt.n_ff, mt.n_expert, mt.n_used, type_name((uint32_t)mt.down_type), slots, iters);
+    std::vector<Layer> layers(1);
+    Layer& out = layers[0];
+    auto up = [&](const qkg_tensor& t) {
+        void* p = nullptr;
+        HIP_OK(hipMalloc(&p, std::max<size_t>(t.nbytes, 16)));
+        HIP_OK(hipMemcpy(p, t.data, t.nbytes, hipMemcpyHostToDevice));
+        out.owned.push_back(p);
+        return p;
+    };
+    out.L = qkk_moe_layer{mt.n_embd, mt.n_ff, mt.n_expert, mt.n_used, mt.gu_type, mt.down_type,
+                          (const float*)up(mt.gate_inp), (const float*)up(mt.gate_inp_shexp), up(mt.gate_exps), up(mt.up_exps),
+                          up(mt.down_exps), up(mt.gate_shexp), up(mt.up_shexp), up(mt.down_shexp)};
+    qkg_close(f);
+    return run_moe(layers, iters, slots, layer);
 }
 
 bool case_head(uint32_t batch, uint32_t iters)
@@ -417,7 +555,8 @@ void usage()
                     "       qk f16|q8_0|q6_k|iq4_xs|iq3_xxs [M] [K] [iters]\n"
                     "       qk bgemm [M] [K] [N] [iters]\n"
                     "       qk moe [seed] [iters] [slots] [experts]\n"
-                    "       qk head [batch] [iters]\n");
+                    "       qk head [batch] [iters]\n"
+                    "       QK_GGUF=model.gguf qk list [prefix] | gguf <tensor> [iters] | layer [layer] [iters] [slots]\n");
 }
 
 } // namespace
@@ -430,11 +569,13 @@ int main(int argc, char** argv)
     }
     const std::string mode = argv[1];
     auto arg_u = [&](int i, uint32_t dflt) { return argc > i ? (uint32_t)strtoul(argv[i], nullptr, 10) : dflt; };
-    const bool known = mode == "suite" || mode == "bgemm" || mode == "moe" || mode == "head" || format_named(mode.c_str());
-    if (!known) {
+    const bool known = mode == "suite" || mode == "bgemm" || mode == "moe" || mode == "head" || mode == "list" || mode == "gguf" ||
+                       mode == "layer" || format_named(mode.c_str());
+    if (!known || (mode == "gguf" && argc < 3)) {
         usage();
         return 1;
     }
+    if (mode == "list") return case_list(argc > 2 ? argv[2] : nullptr) ? 0 : 1; // host only
     char arch[64] = "";
     uint32_t cus = 0;
     if (qkk_device_info(arch, sizeof arch, &cus) < 1) {
@@ -451,6 +592,10 @@ int main(int argc, char** argv)
         ok = case_moe(arg_u(2, 0), arg_u(3, 200), arg_u(4, 1), arg_u(5, 256));
     } else if (mode == "head") {
         ok = case_head(arg_u(2, 1), arg_u(3, 40));
+    } else if (mode == "gguf") {
+        ok = case_gguf(argv[2], arg_u(3, 100));
+    } else if (mode == "layer") {
+        ok = case_layer(arg_u(2, 0), arg_u(3, 200), arg_u(4, 1));
     } else {
         ok = case_gemv(*format_named(mode.c_str()), arg_u(2, 16384), arg_u(3, 8192), arg_u(4, 100));
     }

@@ -11,8 +11,9 @@ QK = os.path.join(ROOT, "qwen-kernel_amd", "qk")
 QK_EMU = os.path.join(ROOT, "tests", "emu", "qk_emu")
 
 
-def run(binary, *args, timeout=300):
-    return subprocess.run([binary, *map(str, args)], capture_output=True, text=True, timeout=timeout)
+def run(binary, *args, timeout=300, env=None):
+    return subprocess.run([binary, *map(str, args)], capture_output=True, text=True, timeout=timeout,
+                          env=None if env is None else {**os.environ, **env})
 
 
 @pytest.fixture(scope="module")
@@ -56,6 +57,53 @@ def test_bad_shapes_are_refused(qk_emu):
     assert r.returncode == 1 and "outside" in r.stderr
 
 
+@pytest.fixture(scope="module")
+def model_file(qk, tmp_path_factory):
+    """A GGUF file with one MoE layer under the reference's tensor names (blk.3.ffn_*) and an F16 tensor."""
+    import numpy as np
+    hl = qk.synth.HostLayer(seed=5, n_embd=2048, n_ff=256, n_expert=8, n_used=2, down_type=qk.Q6_K)
+    path = str(tmp_path_factory.mktemp("gguf") / "model.gguf")
+    half = np.random.default_rng(1).standard_normal((24, 512)).astype(np.float16)
+    qk.gguf.write(path, {"general.architecture": "qwen3next", "qwen3next.expert_used_count": 2},
+                  qk.gguf.layer_tensors(hl, 3) + [("token_embd.weight", qk.F16, (512, 24), half)])
+    return path
+
+
+def test_modes_on_a_model_file_in_the_host_build(qk_emu, model_file):
+    """The reference's real-weight modes (src/main.cpp:846-915, 920-1254) on a file named by QK_GGUF: the tensor
+    list, y = W x on named tensors (a 3-D expert tensor: its first slice) with the dequantise + dense verdict,
+    and the fused step on a layer's tensors, one row and three, with the expert-major path as second opinion."""
+    env = {"QK_GGUF": model_file}
+    r = run(qk_emu, "list", "blk.3.ffn_down", env=env)
+    assert r.returncode == 0 and "9 tensors" in r.stdout, r.stdout + r.stderr
+    lines = [ln for ln in r.stdout.splitlines() if ln.startswith("blk.")]
+    assert len(lines) == 2 and "q6_k" in lines[0] and "[256, 2048, 8, 1]" in lines[0] and "q8_0" in lines[1]
+    for tensor, typ in (("blk.3.ffn_gate_exps.weight", "iq3_xxs"), ("blk.3.ffn_down_shexp.weight", "q8_0"),
+                        ("token_embd.weight", "f16")):
+        r = run(qk_emu, "gguf", tensor, 1, env=env)
+        assert r.returncode == 0 and typ in r.stdout and "-> OK" in r.stdout and r.stdout.strip().endswith("ALL OK"), r.stdout + r.stderr
+    r = run(qk_emu, "gguf", "blk.3.ffn_gate_inp.weight", 1, env=env)
+    assert r.returncode == 0 and "check: none" in r.stdout
+    for slots in (1, 3):
+        r = run(qk_emu, "layer", 3, 1, slots, env=env)
+        assert r.returncode == 0, r.stdout + r.stderr
+        assert "8 experts, 2 used, down q6_k" in r.stdout and "picks equal on both paths -> OK" in r.stdout
+        assert r.stdout.strip().endswith("ALL OK")
+
+
+def test_model_file_errors(qk_emu, model_file):
+    r = run(qk_emu, "gguf", "x", env={"QK_GGUF": ""})
+    assert r.returncode == 1 and "Set QK_GGUF" in r.stderr
+    r = run(qk_emu, "list", env={"QK_GGUF": model_file + ".missing"})
+    assert r.returncode == 1 and "model.gguf.missing" in r.stderr
+    r = run(qk_emu, "gguf", "blk.9.nothing", env={"QK_GGUF": model_file})
+    assert r.returncode == 1 and "not found" in r.stderr
+    r = run(qk_emu, "layer", 4, 1, env={"QK_GGUF": model_file})
+    assert r.returncode == 1 and "layer 4" in r.stderr
+    r = run(qk_emu, "gguf")
+    assert r.returncode == 1 and "usage" in r.stderr
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("args", [("q8_0", 8192, 2048, 50), ("iq3_xxs", 8192, 2048, 50), ("f16", 4096, 4096, 20),
                                   ("bgemm", 8192, 2048, 128, 10), ("moe", 0, 40, 1), ("moe", 0, 20, 4), ("head", 1, 6)],
@@ -68,3 +116,17 @@ def test_modes_on_the_device(dev, args):
     print(r.stdout, flush=True)
     assert r.returncode == 0, r.stdout + r.stderr
     assert "GB/s" in r.stdout and r.stdout.strip().endswith("ALL OK")
+
+
+@pytest.mark.gpu
+def test_modes_on_a_model_file_on_the_device(dev, model_file):
+    if dev == "cpu":
+        pytest.skip("the host-side build has its own cases above")
+    env = {"QK_GGUF": model_file}
+    for args in (("gguf", "blk.3.ffn_gate_exps.weight", 20), ("gguf", "blk.3.ffn_down_exps.weight", 20), ("layer", 3, 20, 1),
+                 ("layer", 3, 10, 4)):
+        print(f"[case] QK_GGUF=... qk {' '.join(map(str, args))}", flush=True)
+        r = run(QK, *args, timeout=300, env=env)
+        print(r.stdout, flush=True)
+        assert r.returncode == 0, r.stdout + r.stderr
+        assert r.stdout.strip().endswith("ALL OK")
