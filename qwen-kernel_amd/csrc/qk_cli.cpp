@@ -17,6 +17,11 @@
 //   qk gguf <tensor> [iters]          y = W x on a named tensor (a 3-D tensor: its first slice, expert 0)
 //   qk layer [layer] [iters] [slots]  the fused MoE step on the tensors blk.<layer>.ffn_* (the reference's
 //                                     `qk moe [layer]`; `moe` here keeps its synthetic weights)
+//   qk token <ids-file> <nGen> [tmax] [batch]   the whole model through the engine ABI of include/qk.h: the
+//                                     prompt's ids from a file, nGen greedy tokens on `batch` slots fed the same
+//                                     prompt (their streams must be identical), prefill and decode rates
+//   qk warm <ids-file> <nGen> [tmax]  the same stream twice: after a prefill, and after restoring a snapshot of
+//                                     the slot's state taken behind the prompt (reference src/main.cpp:2500-3062)
 //
 // The weights are seeded random valid blocks (every bit pattern of the quant fields is valid; the
 // fp16 scales are |N(0,1)| * 1e-3), the activations N(0,1).  Iterations alternate over a ring of
@@ -34,9 +39,11 @@
 #include <string.h>
 
 #include <algorithm>
+#include <chrono>
 #include <string>
 #include <vector>
 
+#include "../../include/qk.h"
 #include "../../include/qk_gguf.h"
 #include "../../include/qk_kernels.h"
 
@@ -549,6 +556,171 @@ bool case_head(uint32_t batch, uint32_t iters)
     return ok;
 }
 
+// ---- the whole model through the engine ABI ---------------------------------------------------
+
+double ms_since(std::chrono::steady_clock::time_point t0)
+{
+    return std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+}
+
+// ids separated by commas, blanks or newlines (reference src/main.cpp:2502-2509)
+bool read_ids(const char* path, std::vector<uint32_t>& out)
+{
+    FILE* f = fopen(path, "r");
+    if (!f) {
+        perror(path);
+        return false;
+    }
+    long v;
+    while (fscanf(f, "%ld%*[, \n\r\t]", &v) == 1) out.push_back((uint32_t)std::max(0l, v));
+    fclose(f);
+    return true;
+}
+
+qk_engine* open_engine(uint32_t slots, uint32_t tmax)
+{
+    const char* path = getenv("QK_GGUF");
+    if (!path || !*path) {
+        fprintf(stderr, "qk: no model path. Set QK_GGUF=/path/to/model.gguf\n");
+        exit(1);
+    }
+    const qk_config cfg{slots, std::max(64u, tmax), 8};
+    char err[512] = "";
+    qk_engine* e = qk_open(path, &cfg, err, sizeof err);
+    if (!e) {
+        fprintf(stderr, "qk: %s: %s\n", path, err);
+        exit(1);
+    }
+    return e;
+}
+
+// reference caseToken (src/main.cpp:2500-3062): prefill, nGen greedy steps on nB identical streams
+bool case_token(const char* ids_file, uint32_t n_gen, uint32_t tmax, uint32_t nb)
+{
+    std::vector<uint32_t> prompt;
+    if (!read_ids(ids_file, prompt)) return false;
+    if (prompt.empty() || n_gen == 0 || prompt.size() + n_gen > tmax) {
+        fprintf(stderr, "qk: bad prompt (%zu ids, %u to generate, tmax %u)\n", prompt.size(), n_gen, tmax);
+        return false;
+    }
+    if (nb < 1 || nb > 16) {
+        fprintf(stderr, "qk: batch must be 1..16\n");
+        return false;
+    }
+    qk_engine* e = open_engine(nb, tmax);
+    const uint32_t chunk = qk_chunk(e);
+    printf("token mode: %zu prompt ids, gen %u, vocab %u, tmax %u, batch %u\n", prompt.size(), n_gen, qk_n_vocab(e), tmax, nb);
+    auto t0 = std::chrono::steady_clock::now();
+    for (uint32_t s = 0; s < nb; s++) {
+        const int rc = qk_slot_start(e, s, prompt.data(), (uint32_t)prompt.size(), n_gen, 0);
+        if (rc != 0) {
+            fprintf(stderr, "qk: qk_slot_start(slot %u) returned %d\n", s, rc);
+            qk_close(e);
+            return false;
+        }
+    }
+    const double prefill_ms = ms_since(t0);
+    printf("prefill: %zu tokens x %u streams in %.1f ms (%.2f ms/token)\n", prompt.size(), nb, prefill_ms,
+           prefill_ms / (prompt.size() * nb));
+    std::vector<std::vector<uint32_t>> gen(nb);
+    std::vector<uint32_t> toks((size_t)nb * chunk), counts(nb);
+    uint32_t finished = 0, calls = 0;
+    t0 = std::chrono::steady_clock::now();
+    for (;;) {
+        const int active = qk_step_chunk(e, toks.data(), counts.data(), &finished);
+        if (active < 0) {
+            fprintf(stderr, "qk: qk_step_chunk returned %d\n", active);
+            qk_close(e);
+            return false;
+        }
+        if (active == 0) break;
+        calls++;
+        for (uint32_t s = 0; s < nb; s++) gen[s].insert(gen[s].end(), &toks[(size_t)s * chunk], &toks[(size_t)s * chunk] + counts[s]);
+    }
+    const double gen_ms = ms_since(t0);
+    const size_t n0 = gen[0].size();
+    bool same = true;
+    for (uint32_t s = 1; s < nb; s++) same = same && gen[s] == gen[0];
+    printf("decode: %zu tokens x %u streams in %.1f ms (%u calls of %u steps) -> %.2f ms/step | per-stream %.1f tok/s | aggregate %.1f tok/s\n",
+           n0, nb, gen_ms, calls, chunk, n0 ? gen_ms / n0 : 0.0, n0 * 1000.0 / gen_ms, (double)n0 * nb * 1000.0 / gen_ms);
+    if (n0 < n_gen) printf("the stream ended at the end-of-sequence token %u after %zu tokens\n", qk_eos_token(e), n0);
+    if (nb > 1) printf("streams identical: %s\n", same ? "YES" : "NO");
+    printf("GEN:");
+    for (uint32_t id : gen[0]) printf(" %u", id);
+    printf("\n");
+    qk_close(e);
+    return same;
+}
+
+// reference caseToken with warmDemo (src/main.cpp:2975-3050): the cost of a cached prefix against a prefill
+bool case_warm(const char* ids_file, uint32_t n_gen, uint32_t tmax)
+{
+    std::vector<uint32_t> prompt;
+    if (!read_ids(ids_file, prompt)) return false;
+    if (prompt.empty() || n_gen == 0 || prompt.size() + n_gen > tmax) {
+        fprintf(stderr, "qk: bad prompt (%zu ids, %u to generate, tmax %u)\n", prompt.size(), n_gen, tmax);
+        return false;
+    }
+    qk_engine* e = open_engine(1, tmax);
+    const uint32_t n = (uint32_t)prompt.size();
+    if (qk_state_n(e) == 0) {
+        fprintf(stderr, "qk: the engine keeps no state snapshots\n");
+        qk_close(e);
+        return false;
+    }
+    printf("warm mode: %u prompt ids, gen %u, tmax %u, %u snapshot entries\n", n, n_gen, tmax, qk_state_n(e));
+    std::vector<uint32_t> ids(n);
+    auto t0 = std::chrono::steady_clock::now();
+    int rc = qk_stage_run(e, 0, prompt.data(), nullptr, n, 0, nullptr, ids.data());
+    const double prefill_ms = ms_since(t0);
+    if (rc != 0) {
+        fprintf(stderr, "qk: qk_stage_run returned %d\n", rc);
+        qk_close(e);
+        return false;
+    }
+    const uint32_t first = ids[n - 1]; // the token behind the prompt: kept with the snapshot, as the reference keeps its logits
+    t0 = std::chrono::steady_clock::now();
+    rc = qk_state_save(e, 0, 0, n);
+    const double snap_ms = ms_since(t0);
+    auto decode = [&](std::vector<uint32_t>& out, double& ms) {
+        out.assign(1, first);
+        const auto t1 = std::chrono::steady_clock::now();
+        for (uint32_t i = 1; i < n_gen && rc == 0; i++) {
+            uint32_t next = 0;
+            rc = qk_stage_run(e, 0, &out.back(), nullptr, 1, n + i - 1, nullptr, &next);
+            out.push_back(next);
+        }
+        ms = ms_since(t1);
+    };
+    std::vector<uint32_t> cold, warm;
+    double cold_ms = 0, warm_ms = 0;
+    if (rc == 0) decode(cold, cold_ms);
+    t0 = std::chrono::steady_clock::now();
+    if (rc == 0) rc = qk_state_load(e, 0, 0, n); // a "new request" with the same prefix
+    const double restore_ms = ms_since(t0);
+    if (rc == 0) decode(warm, warm_ms);
+    if (rc != 0) {
+        fprintf(stderr, "qk: a state or stage call returned %d\n", rc);
+        qk_close(e);
+        return false;
+    }
+    const bool eq = warm == cold;
+    printf("cold start: prefill %u tokens = %.1f ms before the first token\n", n, prefill_ms);
+    printf("warm start: restore the snapshot = %.1f ms before the first token (snapshot %.1f ms, paid once)\n", restore_ms, snap_ms);
+    printf("decode: cold %.1f ms, warm %.1f ms for %u tokens; warm stream identical to cold: %s\n", cold_ms, warm_ms, n_gen,
+           eq ? "YES" : "NO");
+    printf("GEN:");
+    for (uint32_t id : cold) printf(" %u", id);
+    printf("\n");
+    if (!eq) {
+        printf("WARM:");
+        for (uint32_t id : warm) printf(" %u", id);
+        printf("\n");
+    }
+    qk_close(e);
+    return eq;
+}
+
 void usage()
 {
     fprintf(stderr, "usage: qk suite\n"
@@ -556,7 +728,8 @@ void usage()
                     "       qk bgemm [M] [K] [N] [iters]\n"
                     "       qk moe [seed] [iters] [slots] [experts]\n"
                     "       qk head [batch] [iters]\n"
-                    "       QK_GGUF=model.gguf qk list [prefix] | gguf <tensor> [iters] | layer [layer] [iters] [slots]\n");
+                    "       QK_GGUF=model.gguf qk list [prefix] | gguf <tensor> [iters] | layer [layer] [iters] [slots]\n"
+                    "       QK_GGUF=model.gguf qk token <ids-file> <nGen> [tmax] [batch] | warm <ids-file> <nGen> [tmax]\n");
 }
 
 } // namespace
@@ -570,8 +743,8 @@ int main(int argc, char** argv)
     const std::string mode = argv[1];
     auto arg_u = [&](int i, uint32_t dflt) { return argc > i ? (uint32_t)strtoul(argv[i], nullptr, 10) : dflt; };
     const bool known = mode == "suite" || mode == "bgemm" || mode == "moe" || mode == "head" || mode == "list" || mode == "gguf" ||
-                       mode == "layer" || format_named(mode.c_str());
-    if (!known || (mode == "gguf" && argc < 3)) {
+                       mode == "layer" || mode == "token" || mode == "warm" || format_named(mode.c_str());
+    if (!known || (mode == "gguf" && argc < 3) || ((mode == "token" || mode == "warm") && argc < 4)) {
         usage();
         return 1;
     }
@@ -596,6 +769,10 @@ int main(int argc, char** argv)
         ok = case_gguf(argv[2], arg_u(3, 100));
     } else if (mode == "layer") {
         ok = case_layer(arg_u(2, 0), arg_u(3, 200), arg_u(4, 1));
+    } else if (mode == "token") {
+        ok = case_token(argv[2], arg_u(3, 12), arg_u(4, 128), arg_u(5, 1));
+    } else if (mode == "warm") {
+        ok = case_warm(argv[2], arg_u(3, 12), arg_u(4, 128));
     } else {
         ok = case_gemv(*format_named(mode.c_str()), arg_u(2, 16384), arg_u(3, 8192), arg_u(4, 100));
     }

@@ -118,6 +118,65 @@ def test_modes_on_the_device(dev, args):
     assert "GB/s" in r.stdout and r.stdout.strip().endswith("ALL OK")
 
 
+@pytest.fixture(scope="module")
+def whole_model(qk, tmp_path_factory):
+    """A small whole model of the reference's family (a gated-DeltaNet layer and a full-attention layer) and a prompt."""
+    d = tmp_path_factory.mktemp("whole")
+    path = qk.engine.FullModel(23, kinds="RA", vocab=192, eos=197).write(str(d / "model.gguf"))
+    ids = d / "prompt.txt"
+    ids.write_text("5, 17 3\n44,9\n120 7")
+    return path, str(ids)
+
+
+def gen_of(out):
+    return [ln for ln in out.splitlines() if ln.startswith("GEN:")][0].split()[1:]
+
+
+def test_whole_model_modes_in_the_host_build(qk_emu, whole_model):
+    """`qk token` and `qk warm` (reference src/main.cpp:2500-3062) over the engine ABI: the prompt's ids from a
+    file, greedy tokens on one slot and on three slots fed the same prompt (identical streams, and the stream of
+    the single slot), and the stream behind a restored snapshot equal to the one behind the prefill."""
+    path, ids = whole_model
+    env = {"QK_GGUF": path}
+    one = run(qk_emu, "token", ids, 5, 64, env=env)
+    assert one.returncode == 0 and "token mode: 7 prompt ids, gen 5, vocab 192" in one.stdout, one.stdout + one.stderr
+    assert len(gen_of(one.stdout)) == 5 and one.stdout.strip().endswith("ALL OK")
+    three = run(qk_emu, "token", ids, 5, 64, 3, env=env)
+    assert three.returncode == 0 and "streams identical: YES" in three.stdout, three.stdout + three.stderr
+    assert gen_of(three.stdout) == gen_of(one.stdout)
+    warm = run(qk_emu, "warm", ids, 5, 64, env=env)
+    assert warm.returncode == 0 and "warm stream identical to cold: YES" in warm.stdout, warm.stdout + warm.stderr
+    assert gen_of(warm.stdout) == gen_of(one.stdout)
+    # refusals: a prompt that does not fit, a batch the engine has no slots for, a missing file, no model
+    r = run(qk_emu, "token", ids, 60, 64, env=env)
+    assert r.returncode == 1 and "bad prompt" in r.stderr
+    r = run(qk_emu, "token", ids, 5, 64, 17, env=env)
+    assert r.returncode == 1 and "batch must be" in r.stderr
+    r = run(qk_emu, "token", ids + ".missing", 5, env=env)
+    assert r.returncode == 1
+    r = run(qk_emu, "token", ids, 5, env={"QK_GGUF": ""})
+    assert r.returncode == 1 and "Set QK_GGUF" in r.stderr
+    r = run(qk_emu, "warm", ids)
+    assert r.returncode == 1 and "usage" in r.stderr
+
+
+@pytest.mark.gpu
+def test_whole_model_modes_on_the_device(dev, whole_model):
+    if dev == "cpu":
+        pytest.skip("the host-side build has its own cases above")
+    path, ids = whole_model
+    outs = []
+    for args in (("token", ids, 8, 64), ("token", ids, 8, 64, 4), ("warm", ids, 8, 64)):
+        print(f"[case] QK_GGUF=... qk {' '.join(map(str, args))}", flush=True)
+        r = run(QK, *args, timeout=300, env={"QK_GGUF": path})
+        print(r.stdout, flush=True)
+        assert r.returncode == 0 and r.stdout.strip().endswith("ALL OK"), r.stdout + r.stderr
+        outs.append(gen_of(r.stdout))
+    # one slot twice: the same kernels, the same stream (four slots run other kernel families, whose sums differ
+    # in the last bits: their streams are compared with each other inside the program, not with the single slot's)
+    assert outs[0] == outs[2]
+
+
 @pytest.mark.gpu
 def test_modes_on_a_model_file_on_the_device(dev, model_file):
     if dev == "cpu":
