@@ -345,7 +345,8 @@ __device__ __forceinline__ void coop_stream(const uint8_t* __restrict__ base0, c
         {   // next batch: lands during the MFMA phase
             const size_t adv = adv_of(b + 1);
 #pragma unroll
-            for (int n = 0; n < NLD; n++) ld[n] = *(const u32x4*)(src[n] + (CLAMP ? min(adv, room[n]) : adv));
+            for (int n = 0; n < NLD; n++) // a signed step: with two tensors the way from one to the other may lead down
+                ld[n] = *(const u32x4*)(src[n] + (ptrdiff_t)(CLAMP ? min(adv, room[n]) : adv));
         }
         // this wave's fragments of the batch: tiles tg*TG .. +TG of every tensor in it
         BFrag<TYPE> f[NTL];

@@ -160,6 +160,33 @@ def test_whole_model_modes_in_the_host_build(qk_emu, whole_model):
     assert r.returncode == 1 and "usage" in r.stderr
 
 
+SWITCH_SETS = [{}, {"QK_ONE_ROW": "stream", "QK_DENSE_REG": "1", "QK_FUSED_NORM": "1", "QK_DN_FUSED": "1", "QK_ATTN_BLOCK": "1"},
+               {"QK_ONE_ROW": "stream", "QK_SELECT_RANKED": "0"},
+               {"QK_GEMM_TILED": "1", "QK_MOE_ROWS": "1", "QK_HEAD_ROWS": "1", "QK_PREFILL_ROWS": "16"}]
+
+
+@pytest.mark.skipif(os.environ.get("QK_TEST_SANITIZE") != "1", reason="set QK_TEST_SANITIZE=1: builds every kernel under "
+                    "AddressSanitizer + UndefinedBehaviorSanitizer (minutes) and runs the program's modes through it")
+def test_modes_under_the_sanitizers(model_file, whole_model):
+    """The host-side build of every kernel, the engine and the test program as ONE executable under ASan and UBSan
+    (tests/emu/Makefile, target qk_emu_san): each mode under each set of switches must end with its verdict and
+    without a report -- static LDS arrays, arrays on a thread's stack and the kernels' address arithmetic are
+    what the guard pages of the other tests cannot see."""
+    subprocess.run(["make", "-C", os.path.dirname(QK_EMU), "-j", "8", "qk_emu_san"], check=True, stdout=subprocess.DEVNULL)
+    san = os.path.join(os.path.dirname(QK_EMU), "qk_emu_san")
+    path, ids = whole_model
+    base = {"ASAN_OPTIONS": "detect_stack_use_after_return=0:detect_leaks=0", "UBSAN_OPTIONS": "print_stacktrace=1"}
+    cases = [((f, 67, 2048, 1), {}) for f in ("q8_0", "q6_k", "iq4_xs", "iq3_xxs")] + [(("iq4_xs", 9, 768, 1), {}), (("f16", 40, 2048, 1), {}),
+             (("bgemm", 48, 512, 20, 1), {}), (("bgemm", 64, 2048, 130, 1), {}), (("moe", 1, 1, 1, 8), {}), (("moe", 2, 1, 3, 8), {}),
+             (("moe", 3, 1, 16, 8), {}), (("moe", 3, 1, 40, 16), {}), (("layer", 3, 1, 1), {"QK_GGUF": model_file}),
+             (("layer", 3, 1, 12), {"QK_GGUF": model_file}), (("token", ids, 4, 64, 1), {"QK_GGUF": path}),
+             (("token", ids, 4, 64, 3), {"QK_GGUF": path}), (("warm", ids, 4, 64), {"QK_GGUF": path})]
+    for sw in SWITCH_SETS:
+        for args, env in cases:
+            r = run(san, *args, timeout=1500, env={**base, **sw, **env})
+            assert r.returncode == 0 and "runtime error" not in r.stderr and "Sanitizer" not in r.stderr, (sw, args, r.stdout[-500:], r.stderr[-3000:])
+
+
 @pytest.mark.gpu
 def test_whole_model_modes_on_the_device(dev, whole_model):
     if dev == "cpu":
