@@ -25,7 +25,11 @@
  * Environment, as in the reference: QK_MAXB (batch-prefill chunk, 16..1024, default 128),
  * QK_NO_BATCH (serial prefill of the whole prompt); and QK_PREFILL_ROWS (rows of one prefill
  * pass, 16..1024, default 1024: how the prefilled positions are cut, not which are prefilled),
- * QK_NO_GRAPH (launch the step's kernels one by one instead of replaying the graph).
+ * QK_NO_GRAPH (launch the step's kernels one by one instead of replaying the graph);
+ * QK_STEP_PROF, as in the reference (src/main.cpp:4591-4632): the first decode step of slot 0 alone is launched
+ * kernel by kernel with an event behind every stage and the stages' times go to stderr once
+ * ("[prof] decode step: ... us on-GPU across N stages", one line per stage name; QK_STEP_PROF_DETAIL adds every
+ * interval in launch order).
  */
 #ifndef QK_H
 #define QK_H

@@ -114,6 +114,12 @@ struct qk_engine {
     void* d_aws = nullptr;       // attention workspace
     size_t aws_bytes = 0;
     std::vector<std::vector<float*>> snaps; // [N_STATE][2 * layer]: one slot's state stripes
+    // QK_STEP_PROF (reference src/main.cpp:3300-3305, 4591-4632): the first pure decode step at depth 1 is launched
+    // kernel by kernel with an event behind every stage, and the stages' times are printed once to stderr
+    bool prof_on = false, prof_armed = false, prof_printed = false;
+    std::vector<std::pair<const char*, hipEvent_t>> prof_ev;
+    void stamp(const char* label);
+    void prof_report();
 
     // host side (reference src/main.cpp:3153-3175, Slot)
     struct Slot {
@@ -152,6 +158,7 @@ static bool set_err(char* err, size_t n, const char* msg)
 qk_engine::~qk_engine()
 {
     if (st) (void)hipStreamSynchronize(st);
+    for (auto& p : prof_ev) (void)hipEventDestroy(p.second);
     for (hipGraphExec_t g : graphs)
         if (g) (void)hipGraphExecDestroy(g);
     for (void* p : dev_allocs) (void)hipFree(p);
@@ -196,19 +203,70 @@ bool qk_engine::upload(const qkg_tensor& t, const void** out, char* err, size_t 
 
 // The launches of one device step over `rows` rows: d_ids -> d_tok.  *final_rows receives the
 // buffer that holds the rows normalised with output_norm (the LM head's input).
+// An event behind what has been launched so far, named for the stage it closes (only while the profiled step runs).
+void qk_engine::stamp(const char* label)
+{
+    if (!prof_armed) return;
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) return;
+    if (hipEventRecord(e, st) != hipSuccess) { (void)hipEventDestroy(e); return; }
+    prof_ev.emplace_back(label, e);
+}
+
+// The profiled step has been waited for: per stage name the launches, their time and their share, longest first
+// (the reference's lines, src/main.cpp:4609-4615; QK_STEP_PROF_DETAIL adds every interval in launch order).
+void qk_engine::prof_report()
+{
+    struct Row { const char* name; uint32_t n; double us; };
+    std::vector<Row> rows;
+    std::vector<double> each;
+    double total = 0;
+    for (size_t i = 1; i < prof_ev.size(); i++) {
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, prof_ev[i - 1].second, prof_ev[i].second) != hipSuccess) ms = 0.f;
+        const double us = (double)ms * 1e3;
+        each.push_back(us);
+        total += us;
+        auto it = std::find_if(rows.begin(), rows.end(), [&](const Row& r) { return !strcmp(r.name, prof_ev[i].first); });
+        if (it == rows.end()) rows.push_back(Row{prof_ev[i].first, 1, us});
+        else { it->n++; it->us += us; }
+    }
+    std::sort(rows.begin(), rows.end(), [](const Row& a, const Row& b) { return a.us > b.us; });
+    fprintf(stderr, "[prof] decode step: %.0f us on-GPU across %zu stages\n", total, each.size());
+    for (const Row& r : rows)
+        fprintf(stderr, "[prof]   %-10s n=%-3u tot=%8.1f us  avg=%6.2f us  %4.1f%%\n", r.name, r.n, r.us, r.us / r.n,
+                total > 0 ? 100.0 * r.us / total : 0.0);
+    if (getenv("QK_STEP_PROF_DETAIL")) {
+        uint32_t layer = 0;
+        for (size_t i = 1; i < prof_ev.size(); i++) {
+            fprintf(stderr, "[prof-detail] seq=%-3zu layer=%-2u %-10s %8.2f us\n", i, layer, prof_ev[i].first, each[i - 1]);
+            if (!strcmp(prof_ev[i].first, "moe") || !strcmp(prof_ev[i].first, "moe+tail")) layer++;
+        }
+    }
+    for (auto& p : prof_ev) (void)hipEventDestroy(p.second);
+    prof_ev.clear();
+}
+
 int qk_engine::launch_rows(uint32_t rows, float** final_rows)
 {
     if (rows < 1 || rows > MAX_ROWS) return QKK_ESHAPE;
+    stamp("t0");
     if (int rc = qkk_embed(embd_type, d_embd, embd_rows, N_EMBD, d_ids, MAX_ROWS, 0, 1, d_x, rows, st)) return rc;
+    stamp("emb");
     if (rows <= QKK_ROWWISE_MAX) {
         // few rows: each layer's norm runs inside its MoE launches and the residual is added by the
         // last of them -- three launches per layer, then the output norm and the head.  Every row
         // goes through the one-row kernels, so a slot's tokens do not depend on its company.
-        for (const EngineLayer& L : layers)
+        for (const EngineLayer& L : layers) {
             if (int rc = qkk_moe_layer_rows(&L.moe, d_x, L.post_norm, eps, d_sel, d_ws, ws_bytes, rows, st)) return rc;
+            stamp("moe");
+        }
         if (int rc = qkk_rmsnorm(d_x, d_onorm, d_xn[0], N_EMBD, rows, eps, st)) return rc;
+        stamp("rms");
         if (final_rows) *final_rows = d_xn[0];
-        return qkk_head_argmax(d_head, d_xn[0], d_tok, nullptr, vocab, N_EMBD, rows, d_hws, hws_bytes, st);
+        const int rc = qkk_head_argmax(d_head, d_xn[0], d_tok, nullptr, vocab, N_EMBD, rows, d_hws, hws_bytes, st);
+        stamp("head");
+        return rc;
     }
     if (int rc = qkk_rmsnorm(d_x, layers[0].post_norm, d_xn[0], N_EMBD, rows, eps, st)) return rc;
     int cur = 0;
@@ -244,15 +302,19 @@ int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool 
     const uint32_t* ids = seq ? d_pf : d_ids;
     const uint32_t* pos = seq ? d_pf + pf_rows : d_pos + s0;
     uint32_t* tok = seq ? d_pf + 2 * pf_rows : d_tok + s0;
+    stamp("t0");
     if (int rc = qkk_embed(embd_type, d_embd, embd_rows, N_EMBD, ids, seq ? pf_rows : MAX_ROWS, seq ? 0 : s0, 1, x, rows, st))
         return rc;
+    stamp("emb");
     // One row of a decode step (no caller wants the normalised rows): no norm launches at all.  The
     // consumers of a normalised row -- the input projections, the decay / write-strength products, the
     // head -- take the residual row and the norm's weights and normalise on the way in; the MoE
     // launches have done so all along.
     const bool fuse = rows == 1 && !seq && !final_rows && cat_everywhere && fused_norm;
-    if (!fuse)
+    if (!fuse) {
         if (int rc = qkk_rmsnorm(x, layers[0].attn_norm, d_xn[0], N_EMBD, rows, eps, st)) return rc;
+        stamp("rms0");
+    }
     int cur = 0;
     for (size_t l = 0; l < layers.size(); l++) {
         const EngineLayer& L = layers[l];
@@ -264,12 +326,14 @@ int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool 
             if (int rc = qkk_gemv_norm(L.cat.type, L.cat.w, x, L.attn_norm, eps, d_big, L.cat.M, L.cat.K, 1, st)) return rc;
         } else if (one)
             if (int rc = dense(L.cat, xn, d_big, 1, st)) return rc;
-        if (L.kind == EngineLayer::RECURRENT) {
+        const bool rec = L.kind == EngineLayer::RECURRENT;
+        if (rec) {
             float* d_mid = one ? d_big + DN_CH : this->d_mid;
             if (!one) {
                 if (int rc = dense(L.p1, xn, d_big, rows, st)) return rc;
                 if (int rc = dense(L.p2, xn, d_mid, rows, st)) return rc;
             }
+            stamp("dn.proj");
             if (seq) {
                 if (int rc = qkk_dn_ab(xn, L.alpha_w, L.beta_w, L.dt_bias, L.a_vec, d_gb, N_EMBD, DN_HV, rows, st)) return rc;
                 if (int rc = qkk_dn_conv_seq(s1, d_big, L.ker, d_conv, DN_CH, DN_DS, 2 * DN_HK * DN_DS, eps, rows, st)) return rc;
@@ -290,9 +354,11 @@ int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool 
                                   : qkk_dn_ab_conv(xn, L.alpha_w, L.beta_w, L.dt_bias, L.a_vec, d_gb, N_EMBD, DN_HV, s1, d_big,
                                                    L.ker, d_conv, DN_CH, DN_DS, 2 * DN_HK * DN_DS, eps, rows, st))
                     return rc;
+                stamp("dn.ab+conv");
                 if (int rc = qkk_dn_step(d_conv, d_gb, s2, L.ssm_norm, d_mid, d_att, DN_DS, DN_HK, DN_HV, dn_kdiv, eps, rows, st))
                     return rc;
             }
+            stamp("dn.step");
         } else {
             float* d_kin = one ? d_big + FA_HQ * 2 * FA_DH : this->d_kin;
             float* d_vin = one ? d_kin + FA_HKV * FA_DH : this->d_vin;
@@ -301,6 +367,7 @@ int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool 
                 if (int rc = dense(L.p2, xn, d_kin, rows, st)) return rc;
                 if (int rc = dense(L.p3, xn, d_vin, rows, st)) return rc;
             }
+            stamp("at.proj");
             if (seq) {
                 if (int rc = qkk_attn_prep_seq(d_big, d_kin, d_vin, L.q_norm, L.k_norm, d_rope, pos, d_qhat, s1, s2, rows, FA_HQ,
                                                FA_HKV, FA_DH, FA_ROT, n_ctx, eps, st))
@@ -312,35 +379,48 @@ int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool 
                 if (int rc = qkk_attn_prep(d_big, d_kin, d_vin, L.q_norm, L.k_norm, d_rope, pos, d_qhat, s1, s2, rows, FA_HQ,
                                            FA_HKV, FA_DH, FA_ROT, n_ctx, eps, st))
                     return rc;
+                stamp("at.prep");
                 if (int rc = qkk_attn_decode(d_qhat, s1, s2, d_big, pos, d_att, d_aws, aws_bytes, rows, FA_HQ, FA_HKV, FA_DH,
                                              n_ctx, st))
                     return rc;
             }
+            stamp("at.attn");
         }
         if (int rc = dense(L.out, d_att, d_mix, rows, st)) return rc;
+        stamp(rec ? "dn.out" : "at.out");
         const float* w_next = l + 1 < layers.size() ? layers[l + 1].attn_norm : d_onorm;
         if (rows <= QKK_ROWWISE_MAX) {
             // x <- (x + mixer) + MoE(norm(x + mixer)) in three launches (xn, read by now, takes the sum), then
             // the next layer's norm
             if (int rc = qkk_moe_layer_rows_add(&L.moe, x, d_mix, xn, L.post_norm, eps, d_sel, d_ws, ws_bytes, rows, st))
                 return rc;
-            if (!fuse)
+            stamp("moe");
+            if (!fuse) {
                 if (int rc = qkk_rmsnorm(x, w_next, d_xn[cur ^ 1], N_EMBD, rows, eps, st)) return rc;
+                stamp("rms");
+            }
         } else {
             // y = x + mixer, normalised for the MoE block; then x = y + MoE, normalised for the next layer
             if (int rc = qkk_add_rmsnorm(x, d_mix, L.post_norm, x, xn, N_EMBD, rows, eps, st)) return rc;
+            stamp("addN");
             if (int rc = qkk_moe_decode_tail(&L.moe, xn, x, w_next, eps, x, d_xn[cur ^ 1], d_sel, d_ws, ws_bytes, rows, st))
                 return rc;
+            stamp("moe+tail");
         }
         cur ^= 1;
     }
     if (final_rows) *final_rows = d_xn[cur];
     if (!want_head) return QKK_OK;
-    if (fuse) return qkk_head_argmax_norm(d_head, x, d_onorm, eps, tok, nullptr, vocab, N_EMBD, d_hws, hws_bytes, st);
+    if (fuse) {
+        const int rc = qkk_head_argmax_norm(d_head, x, d_onorm, eps, tok, nullptr, vocab, N_EMBD, d_hws, hws_bytes, st);
+        stamp("head");
+        return rc;
+    }
     for (uint32_t r0 = 0; r0 < rows; r0 += MAX_ROWS) // the head takes sixteen rows at a time
         if (int rc = qkk_head_argmax(d_head, d_xn[cur] + (size_t)r0 * N_EMBD, tok + r0, nullptr, vocab, N_EMBD,
                                      std::min(MAX_ROWS, rows - r0), d_hws, hws_bytes, st))
             return rc;
+    stamp("head");
     return QKK_OK;
 }
 
@@ -783,6 +863,7 @@ bool qk_engine::open(const char* path, const qk_config& cfg, char* err, size_t e
     // One graph per dispatch depth z = highest active slot + 1 (the reference records one
     // command buffer per z, src/main.cpp:4169-4422).  Each depth runs once eagerly first, so
     // that whatever a launcher sets up on its first call is not part of a capture.
+    prof_on = getenv("QK_STEP_PROF") != nullptr;
     const bool use_graphs = !getenv("QK_NO_GRAPH");
     graphs.assign(use_graphs ? n_slots : 0, nullptr);
     for (uint32_t z = 1; z <= n_slots; z++) {
@@ -845,7 +926,16 @@ int qk_engine::step_chunk(uint32_t* out_tok, uint32_t* out_cnt, uint32_t* out_fi
             }
         }
         if (!n_act || !need) break;
-        if (int rc = run_rows(max_z, true)) return rc;
+        // QK_STEP_PROF: the first pure decode step at depth 1 goes out kernel by kernel with an event behind each stage
+        const bool profile = prof_on && !prof_printed && max_z == 1 && slots[0].active && slots[0].cursor >= slots[0].prompt.size();
+        prof_armed = profile;
+        const int rc_step = run_rows(max_z, !profile);
+        prof_armed = false;
+        if (rc_step) return rc_step;
+        if (profile) {
+            prof_report();
+            prof_printed = true;
+        }
 
         for (uint32_t s = 0; s < n_slots; s++) {
             Slot& sl = slots[s];

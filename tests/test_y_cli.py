@@ -147,6 +147,13 @@ def test_whole_model_modes_in_the_host_build(qk_emu, whole_model):
     warm = run(qk_emu, "warm", ids, 5, 64, env=env)
     assert warm.returncode == 0 and "warm stream identical to cold: YES" in warm.stdout, warm.stdout + warm.stderr
     assert gen_of(warm.stdout) == gen_of(one.stdout)
+    # QK_STEP_PROF (reference src/main.cpp:4591-4632): the first decode step's stages on stderr, once, the stream unchanged
+    prof = run(qk_emu, "token", ids, 5, 64, env={**env, "QK_STEP_PROF": "1", "QK_STEP_PROF_DETAIL": "1"})
+    assert prof.returncode == 0 and gen_of(prof.stdout) == gen_of(one.stdout), prof.stdout + prof.stderr
+    assert prof.stderr.count("[prof] decode step:") == 1 and "across 15 stages" in prof.stderr, prof.stderr
+    for stage in ("emb", "rms0", "dn.proj", "dn.ab+conv", "dn.step", "dn.out", "at.proj", "at.prep", "at.attn", "at.out", "moe", "rms", "head"):
+        assert f"[prof]   {stage:<10s} n=" in prof.stderr, (stage, prof.stderr)
+    assert prof.stderr.count("[prof-detail]") == 15 and "[prof]   moe        n=2" in prof.stderr
     # refusals: a prompt that does not fit, a batch the engine has no slots for, a missing file, no model
     r = run(qk_emu, "token", ids, 60, 64, env=env)
     assert r.returncode == 1 and "bad prompt" in r.stderr
