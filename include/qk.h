@@ -29,7 +29,9 @@
  * QK_STEP_PROF, as in the reference (src/main.cpp:4591-4632): the first decode step of slot 0 alone is launched
  * kernel by kernel with an event behind every stage and the stages' times go to stderr once
  * ("[prof] decode step: ... us on-GPU across N stages", one line per stage name; QK_STEP_PROF_DETAIL adds every
- * interval in launch order).
+ * interval in launch order); QK_COUNTERS (src/main.cpp:5250-5281): the same for the first prefill pass of more
+ * than one row ("[qk counters] HIP batched prefill N=... span=... ms", one line per stage; QK_COUNTER_RAW adds
+ * every interval).
  */
 #ifndef QK_H
 #define QK_H

@@ -117,9 +117,12 @@ struct qk_engine {
     // QK_STEP_PROF (reference src/main.cpp:3300-3305, 4591-4632): the first pure decode step at depth 1 is launched
     // kernel by kernel with an event behind every stage, and the stages' times are printed once to stderr
     bool prof_on = false, prof_armed = false, prof_printed = false;
+    // QK_COUNTERS (reference src/main.cpp:3307-3313, 5250-5281): the same for the first prefill pass of more than one row
+    bool counters_on = false, counters_printed = false;
     std::vector<std::pair<const char*, hipEvent_t>> prof_ev;
     void stamp(const char* label);
     void prof_report();
+    void counters_report(uint32_t rows, uint32_t base);
 
     // host side (reference src/main.cpp:3153-3175, Slot)
     struct Slot {
@@ -247,6 +250,30 @@ void qk_engine::prof_report()
     prof_ev.clear();
 }
 
+// The profiled prefill pass has been waited for: per stage name its time, share and launches, in launch order
+// (the reference's lines, src/main.cpp:5276-5281; QK_COUNTER_RAW adds every interval).
+void qk_engine::counters_report(uint32_t rows, uint32_t base)
+{
+    struct Agg { const char* name; double ms; uint32_t count; };
+    std::vector<Agg> agg;
+    double total = 0;
+    for (size_t i = 1; i < prof_ev.size(); i++) {
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, prof_ev[i - 1].second, prof_ev[i].second) != hipSuccess) ms = 0.f;
+        total += ms;
+        auto it = std::find_if(agg.begin(), agg.end(), [&](const Agg& a) { return !strcmp(a.name, prof_ev[i].first); });
+        if (it == agg.end()) agg.push_back(Agg{prof_ev[i].first, ms, 1});
+        else { it->ms += ms; it->count++; }
+        if (getenv("QK_COUNTER_RAW")) fprintf(stderr, "[qk counter raw] %03zu %-22s %9.3f ms\n", i, prof_ev[i].first, ms);
+    }
+    fprintf(stderr, "[qk counters] HIP batched prefill N=%u base=%u span=%.3f ms markers=%zu\n", rows, base, total, prof_ev.size());
+    for (const Agg& a : agg)
+        fprintf(stderr, "[qk counters] %-22s %9.3f ms %6.2f%%  (%u passes)\n", a.name, a.ms, total > 0 ? 100.0 * a.ms / total : 0.0,
+                a.count);
+    for (auto& p : prof_ev) (void)hipEventDestroy(p.second);
+    prof_ev.clear();
+}
+
 int qk_engine::launch_rows(uint32_t rows, float** final_rows)
 {
     if (rows < 1 || rows > MAX_ROWS) return QKK_ESHAPE;
@@ -337,6 +364,7 @@ int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool 
             if (seq) {
                 if (int rc = qkk_dn_ab(xn, L.alpha_w, L.beta_w, L.dt_bias, L.a_vec, d_gb, N_EMBD, DN_HV, rows, st)) return rc;
                 if (int rc = qkk_dn_conv_seq(s1, d_big, L.ker, d_conv, DN_CH, DN_DS, 2 * DN_HK * DN_DS, eps, rows, st)) return rc;
+                stamp("dn.ab+conv");
                 if (int rc = qkk_dn_step_seq(d_conv, d_gb, s2, L.ssm_norm, d_mid, d_att, DN_DS, DN_HK, DN_HV, dn_kdiv, eps, rows,
                                              st))
                     return rc;
@@ -372,6 +400,7 @@ int qk_engine::launch_full(uint32_t rows, uint32_t s0, float** final_rows, bool 
                 if (int rc = qkk_attn_prep_seq(d_big, d_kin, d_vin, L.q_norm, L.k_norm, d_rope, pos, d_qhat, s1, s2, rows, FA_HQ,
                                                FA_HKV, FA_DH, FA_ROT, n_ctx, eps, st))
                     return rc;
+                stamp("at.prep");
                 if (int rc = qkk_attn_seq(d_qhat, s1, s2, d_big, pos, d_att, d_aws, aws_bytes, rows, FA_HQ, FA_HKV, FA_DH, n_ctx,
                                           st))
                     return rc;
@@ -438,13 +467,21 @@ int qk_engine::prefill(uint32_t slot, const uint32_t* toks, uint32_t n, uint32_t
         if (hipMemcpyAsync(d_pf, h_pf, 2 * pf_rows * sizeof(uint32_t), hipMemcpyHostToDevice, st) != hipSuccess)
             return ERR_DEVICE;
         float* fin = nullptr;
-        if (launch_full(rows, slot, &fin, ids_out != nullptr, true) != QKK_OK) return ERR_DEVICE;
+        const bool trace = counters_on && !counters_printed && rows > 1;
+        prof_armed = trace;
+        const int rc_pass = launch_full(rows, slot, &fin, ids_out != nullptr, true);
+        prof_armed = false;
+        if (rc_pass != QKK_OK) return ERR_DEVICE;
         if (ids_out && (hipMemcpyAsync(h_pf + 2 * pf_rows, d_pf + 2 * pf_rows, rows * sizeof(uint32_t), hipMemcpyDeviceToHost,
                                        st) != hipSuccess ||
                         hipMemcpyAsync(d_last, fin + (size_t)(rows - 1) * N_EMBD, N_EMBD * sizeof(float),
                                        hipMemcpyDeviceToDevice, st) != hipSuccess))
             return ERR_DEVICE;
         if (hipStreamSynchronize(st) != hipSuccess) return ERR_DEVICE;
+        if (trace) {
+            counters_report(rows, base + off);
+            counters_printed = true;
+        }
         if (ids_out) memcpy(ids_out + off, h_pf + 2 * pf_rows, rows * sizeof(uint32_t));
     }
     return 0;
@@ -864,6 +901,7 @@ bool qk_engine::open(const char* path, const qk_config& cfg, char* err, size_t e
     // command buffer per z, src/main.cpp:4169-4422).  Each depth runs once eagerly first, so
     // that whatever a launcher sets up on its first call is not part of a capture.
     prof_on = getenv("QK_STEP_PROF") != nullptr;
+    counters_on = getenv("QK_COUNTERS") != nullptr;
     const bool use_graphs = !getenv("QK_NO_GRAPH");
     graphs.assign(use_graphs ? n_slots : 0, nullptr);
     for (uint32_t z = 1; z <= n_slots; z++) {

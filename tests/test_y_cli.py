@@ -154,6 +154,19 @@ def test_whole_model_modes_in_the_host_build(qk_emu, whole_model):
     for stage in ("emb", "rms0", "dn.proj", "dn.ab+conv", "dn.step", "dn.out", "at.proj", "at.prep", "at.attn", "at.out", "moe", "rms", "head"):
         assert f"[prof]   {stage:<10s} n=" in prof.stderr, (stage, prof.stderr)
     assert prof.stderr.count("[prof-detail]") == 15 and "[prof]   moe        n=2" in prof.stderr
+    # QK_COUNTERS (reference src/main.cpp:5250-5281): the stages of the first prefill pass (a prompt of 20 ids: 19
+    # positions are prefilled together, the last one is a serial step)
+    long_ids = os.path.join(os.path.dirname(ids), "long.txt")
+    with open(long_ids, "w") as f:
+        f.write(" ".join(str(3 + 7 * i) for i in range(20)))
+    plain = run(qk_emu, "token", long_ids, 3, 64, env=env)
+    cnt = run(qk_emu, "token", long_ids, 3, 64, env={**env, "QK_COUNTERS": "1", "QK_COUNTER_RAW": "1"})
+    assert cnt.returncode == 0 and gen_of(cnt.stdout) == gen_of(plain.stdout), cnt.stdout + cnt.stderr
+    assert cnt.stderr.count("[qk counters] HIP batched prefill N=19 base=0") == 1, cnt.stderr
+    for stage in ("emb", "rms0", "dn.proj", "dn.ab+conv", "dn.step", "dn.out", "at.proj", "at.prep", "at.attn", "at.out", "addN",
+                  "moe+tail"):   # more than ten rows: the add + norm launch and the MoE step with its tail
+        assert f"[qk counters] {stage:<22s}" in cnt.stderr, (stage, cnt.stderr)
+    assert "[qk counter raw] 001 emb" in cnt.stderr
     # refusals: a prompt that does not fit, a batch the engine has no slots for, a missing file, no model
     r = run(qk_emu, "token", ids, 60, 64, env=env)
     assert r.returncode == 1 and "bad prompt" in r.stderr
