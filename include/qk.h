@@ -18,12 +18,13 @@
  * Every entry point behaves as the reference's: argument checks and return codes, the serial-step
  * state machine of qk_step_chunk (one captured hipGraph per dispatch depth), greedy sampling,
  * EOS / max_gen / n_ctx endings, qk_stage_run / qk_stage_topk on the unsplit engine, state
- * snapshots (three entries).  qk_slot_start prefills the positions the reference batch-prefills,
+ * snapshots (three entries, or QK_PCACHE).  qk_slot_start prefills the positions the reference batch-prefills,
  * and qk_stage_run feeds its positions, in passes of up to QK_PREFILL_ROWS rows on the slot
  * alone.  Not part of this library: the prefix cache, speculative decoding, QK_LAYERS pipeline
  * stages (refused: one GPU runs every layer).  A device failure inside a call returns -6.
  * Environment, as in the reference: QK_MAXB (batch-prefill chunk, 16..1024, default 128),
- * QK_NO_BATCH (serial prefill of the whole prompt); and QK_PREFILL_ROWS (rows of one prefill
+ * QK_NO_BATCH (serial prefill of the whole prompt), QK_PCACHE (state snapshot entries, 1..256, default 3);
+ * and QK_PREFILL_ROWS (rows of one prefill
  * pass, 16..1024, default 1024: how the prefilled positions are cut, not which are prefilled),
  * QK_NO_GRAPH (launch the step's kernels one by one instead of replaying the graph);
  * QK_STEP_PROF, as in the reference (src/main.cpp:4591-4632): the first decode step of slot 0 alone is launched

@@ -35,7 +35,7 @@ namespace {
 
 constexpr uint32_t N_EMBD = 2048;           // reference src/main.cpp:3086 (compile-time there too)
 constexpr uint32_t MAX_ROWS = QKK_MAX_SLOTS; // rows one device step carries
-constexpr uint32_t N_STATE = 3;             // snapshot entries (reference default, stub/qk_stub.c:98)
+constexpr uint32_t N_STATE_DEFAULT = 3;     // snapshot entries (reference default, stub/qk_stub.c:98; QK_PCACHE sets 1..256, src/main.cpp:4121-4125)
 constexpr int ERR_DEVICE = -6;              // a launch, copy or synchronisation failed
 
 // The mixers' shapes are fixed, as in the reference engine (src/main.cpp:3085-3090).
@@ -113,7 +113,8 @@ struct qk_engine {
           *d_qhat = nullptr, *d_att = nullptr, *d_mix = nullptr; // per-step rows of the mixers
     void* d_aws = nullptr;       // attention workspace
     size_t aws_bytes = 0;
-    std::vector<std::vector<float*>> snaps; // [N_STATE][2 * layer]: one slot's state stripes
+    uint32_t n_state = N_STATE_DEFAULT;     // snapshot entries (QK_PCACHE)
+    std::vector<std::vector<float*>> snaps; // [n_state][2 * layer]: one slot's state stripes
     // QK_STEP_PROF (reference src/main.cpp:3300-3305, 4591-4632): the first pure decode step at depth 1 is launched
     // kernel by kernel with an event behind every stage, and the stages' times are printed once to stderr
     bool prof_on = false, prof_armed = false, prof_printed = false;
@@ -679,7 +680,7 @@ bool qk_engine::load_mixers(qkg_file* g, char* err, size_t err_len)
         hipMemcpy(d_rope, rope.data(), rope.size() * sizeof(float), hipMemcpyHostToDevice) != hipSuccess)
         return bad("qk_open: upload failed");
     // snapshot entries: one slot's state stripes each (reference src/main.cpp:3435-3487, copyStripes)
-    snaps.assign(N_STATE, std::vector<float*>(2 * n_layer, nullptr));
+    snaps.assign(n_state, std::vector<float*>(2 * n_layer, nullptr));
     for (auto& sn : snaps)
         for (uint32_t l = 0; l < n_layer; l++) {
             sn[2 * l] = (float*)dev_alloc(layers[l].ps1 * sizeof(float), true);
@@ -758,6 +759,10 @@ bool qk_engine::open(const char* path, const qk_config& cfg, char* err, size_t e
         if (x >= 16 && x <= 1024) pf_rows = (uint32_t)x;
         else fprintf(stderr, "QK_PREFILL_ROWS=%s out of range [16,1024]; using %u\n", pr, pf_rows);
     }
+    if (const char* pc = getenv("QK_PCACHE")) { // reference src/main.cpp:4121-4125
+        const long v = strtol(pc, nullptr, 10);
+        if (v >= 1 && v <= 256) n_state = (uint32_t)v;
+    }
     if (const char* mb = getenv("QK_MAXB")) { // reference src/main.cpp:3834-3838
         const long x = atol(mb);
         if (x >= 16 && x <= 1024) max_b = (uint32_t)x;
@@ -828,7 +833,7 @@ bool qk_engine::open(const char* path, const qk_config& cfg, char* err, size_t e
         const uint64_t per_slot = kinds[l] == EngineLayer::RECURRENT
                                       ? (uint64_t)DN_CH * 3 + (uint64_t)DN_HV * DN_DS * DN_DS
                                       : 2ull * FA_HKV * n_ctx * FA_DH;
-        need += (n_slots + N_STATE) * per_slot * sizeof(float);
+        need += (n_slots + n_state) * per_slot * sizeof(float);
     }
     need += (uint64_t)(with_mixers ? pf_rows : MAX_ROWS) * (64u << 10) * sizeof(float) + (uint64_t)vocab * 80;
     size_t free_b = 0, total_b = 0;
@@ -1155,15 +1160,15 @@ int qk_stage_topk(qk_engine* e, uint32_t k, uint32_t* ids, float* vals)
 }
 
 // reference src/main.cpp:5428-5445.  A MoE-only model has no per-position state: bounds only.
-uint32_t qk_state_n(const qk_engine* e) { return e ? N_STATE : 0; }
+uint32_t qk_state_n(const qk_engine* e) { return e ? e->n_state : 0; }
 int qk_state_save(qk_engine* e, uint32_t slot, uint32_t idx, uint32_t n_tok)
 {
-    if (!e || slot >= e->n_slots || idx >= N_STATE) return -1;
+    if (!e || slot >= e->n_slots || idx >= e->n_state) return -1;
     return e->full_model ? e->copy_state(slot, idx, true, n_tok) : 0;
 }
 int qk_state_load(qk_engine* e, uint32_t slot, uint32_t idx, uint32_t n_tok)
 {
-    if (!e || slot >= e->n_slots || idx >= N_STATE) return -1;
+    if (!e || slot >= e->n_slots || idx >= e->n_state) return -1;
     return e->full_model ? e->copy_state(slot, idx, false, n_tok) : 0;
 }
 

@@ -144,8 +144,9 @@ def test_whole_model_modes_in_the_host_build(qk_emu, whole_model):
     three = run(qk_emu, "token", ids, 5, 64, 3, env=env)
     assert three.returncode == 0 and "streams identical: YES" in three.stdout, three.stdout + three.stderr
     assert gen_of(three.stdout) == gen_of(one.stdout)
-    warm = run(qk_emu, "warm", ids, 5, 64, env=env)
+    warm = run(qk_emu, "warm", ids, 5, 64, env={**env, "QK_PCACHE": "5"})   # the reference's knob for the snapshot entries
     assert warm.returncode == 0 and "warm stream identical to cold: YES" in warm.stdout, warm.stdout + warm.stderr
+    assert "5 snapshot entries" in warm.stdout
     assert gen_of(warm.stdout) == gen_of(one.stdout)
     # QK_STEP_PROF (reference src/main.cpp:4591-4632): the first decode step's stages on stderr, once, the stream unchanged
     prof = run(qk_emu, "token", ids, 5, 64, env={**env, "QK_STEP_PROF": "1", "QK_STEP_PROF_DETAIL": "1"})
