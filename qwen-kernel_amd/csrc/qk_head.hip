@@ -406,7 +406,6 @@ __global__ __launch_bounds__(MR_THREADS, 4) void head_q6k_rows_kernel(const uint
     __shared__ MfmaTables tab; // Q6_K reads no table; rows_stream takes the reference
     __shared__ uint32_t s_last;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, j = lane & 15, g = lane >> 4;
-    const uint8_t* tens[1] = {W};
     const size_t last_piece = (size_t)V * ROW - 16; // a Q6_K row of 2048 is 105 pieces: the tensor ends on one
     const uint32_t items = (V + MR_ROWS - 1) / MR_ROWS;
     const float* arow = X + (size_t)min((uint32_t)j, batch - 1) * K; // operand rows behind the batch repeat its last row
@@ -418,7 +417,7 @@ __global__ __launch_bounds__(MR_THREADS, 4) void head_q6k_rows_kernel(const uint
     const uint32_t mine = blockIdx.x < items ? (items - blockIdx.x + gridDim.x - 1) / gridDim.x : 0u;
     if (mine)
         rows_stream<QKK_Q6_K, 1>(
-            tens, mine, [&](uint32_t b) { return (size_t)(blockIdx.x + b * gridDim.x) * MR_ROWS * ROW; }, ROW, last_piece, K / 256,
+            W, nullptr, mine, [&](uint32_t b) { return (size_t)(blockIdx.x + b * gridDim.x) * MR_ROWS * ROW; }, ROW, last_piece, K / 256,
             arow, smem, tab, tid, [&](uint32_t b, const float4v(&acc)[1]) {
                 const uint32_t row = (blockIdx.x + b * gridDim.x) * MR_ROWS + 16 * wave + j; // rows behind V were read from clamped addresses: dropped here
 #pragma unroll

@@ -46,9 +46,6 @@ __global__ __launch_bounds__(MR_THREADS, 4) void moe_rows_kernel(const uint8_t* 
     const size_t stride = (size_t)nfrag * G::FB;                       // bytes of a weight row
     const size_t last_piece = (size_t)d.E * R * stride - 16;           // the tensors end on 16-byte boundaries (E * R * stride: R is a multiple of 128)
     const uint32_t n_active = active_count(ws, d);
-    const uint8_t* tens[NT];
-    tens[0] = W0;
-    if constexpr (GATEUP) tens[1] = W1;
 
     const uint32_t groups = blocks_per_expert / bpi; // a work item: bpi consecutive blocks of an active expert
 
@@ -70,7 +67,7 @@ __global__ __launch_bounds__(MR_THREADS, 4) void moe_rows_kernel(const uint8_t* 
             __syncthreads();
             const float* arow = GATEUP ? X + (size_t)s_tok[j] * d.H : ws.h + ((size_t)s_tok[j] * (d.k + 1) + s_slot[j]) * d.F;
             rows_stream<TYPE, NT>(
-                tens, bpi, [&](uint32_t b) { return base + (size_t)b * MR_ROWS * stride; }, stride, last_piece, nfrag, arow, smem,
+                W0, W1, bpi, [&](uint32_t b) { return base + (size_t)b * MR_ROWS * stride; }, stride, last_piece, nfrag, arow, smem,
                 tab, tid, [&](uint32_t b, const float4v(&acc)[NT]) {
                     // D[4 g + e][j]: pair 4 g + e of the tile, row 16 wave + j of block b
                     const uint32_t row = row0 + b * MR_ROWS + 16 * wave + j;

@@ -26,7 +26,7 @@ struct RowsGeo {
 };
 
 // For each of `nblk` blocks of 128 weight rows in turn: acc[t][e] = sum over K of (row 16 wave + j of the block in
-// tensor t) . (activation row 4 g + e), lane = 16 g + j, handed to done(b, acc).  base_of(b): byte offset of block
+// tensor t: w0, and with NT = 2 also w1) . (activation row 4 g + e), lane = 16 g + j, handed to done(b, acc).  base_of(b): byte offset of block
 // b's first row in every tensor (rows `stride` bytes apart, nfrag fragments each); reads are clamped to the
 // 16-byte piece at `last_piece`, the tensors' last one.  arow: the activation row of THIS thread's lane j (thread
 // (wave, lane) converts the operand of lane `lane` for instruction `wave` of a K step).  The K steps of all blocks
@@ -36,7 +36,7 @@ struct RowsGeo {
 // smem: RowsGeo::LDS_BYTES; the caller has a barrier between the previous user of smem and this call, and one
 // between this call and the next user.
 template <int TYPE, int NT, class BaseOf, class Done>
-__device__ __forceinline__ void rows_stream(const uint8_t* const (&tens)[NT], uint32_t nblk, BaseOf base_of, size_t stride,
+__device__ __forceinline__ void rows_stream(const uint8_t* w0, const uint8_t* w1, uint32_t nblk, BaseOf base_of, size_t stride,
                                             size_t last_piece, uint32_t nfrag, const float* arow, uint8_t* smem,
                                             const MfmaTables& tab, int tid, Done done)
 {
@@ -62,7 +62,7 @@ __device__ __forceinline__ void rows_stream(const uint8_t* const (&tens)[NT], ui
         for (int n = 0; n < NLD; n++) {
             const uint32_t p = min(me + MR_THREADS * n, PIECES - 1);
             const uint32_t slot = p / NPW, q = p % NPW;
-            const uint8_t* t = tens[NT > 1 && slot >= MR_ROWS ? NT - 1 : 0];
+            const uint8_t* t = NT > 1 && slot >= MR_ROWS ? w1 : w0; // a choice between two kernel arguments: the loads stay global loads
             const size_t at = base + (size_t)(slot % MR_ROWS) * stride + (size_t)f * FB; // the row's fragment f
             ld[n] = *(const u32x4*)(t + min((at & ~(size_t)15) + 16u * q, last_piece)); // its window starts at the 16-byte boundary below
         }

@@ -108,3 +108,25 @@ def test_one_row_kernels_fetch_the_weights_as_16_byte_pieces():
         assert wide >= 8, (k, wide, narrow)
         if "gemv_stream" in k or "head_q6k" in k:   # the MoE launches also fetch logits, picks and h: scalars and short rows
             assert narrow * 3 <= wide, (k, wide, narrow, sorted(set(loads)))
+
+
+def test_matrix_kernels_keep_their_loads_in_the_global_address_space():
+    """The tiled GEMM and the row-split expert / head kernels: every weight fetch is a global_load_dwordx4.  A
+    pointer that loses its address space on the way (a tensor chosen through an array of pointers did) becomes a
+    flat load, which also counts against the LDS counter -- every wait for an LDS read then waits for the
+    fetches in flight, and the overlap of fetch and arithmetic is gone.  Flat loads are allowed only where a
+    kernel reads other workgroups' candidates with system scope (the head's last fold)."""
+    if not os.path.exists(HIPCC):
+        pytest.skip("no hipcc")
+    files = [os.path.join(CSRC, f) for f in ("qk_moe_rows.hip", "qk_gemm_tiled.hip", "qk_head.hip")]
+    with concurrent.futures.ThreadPoolExecutor(max_workers=3) as pool:
+        funcs = {}
+        for d in pool.map(isa_of, files):
+            funcs.update(d)
+    hot = [k for k in funcs if "moe_rows_kernel" in k or "gemm_tiled_kernel" in k or "head_q6k_rows_kernel" in k]
+    assert len(hot) == 8, sorted(hot)
+    for k in hot:
+        flat = re.findall(r"\bflat_load_\w+[^\n]*", funcs[k])
+        assert all("sc0 sc1" in f for f in flat) and len(flat) <= 2, (k, flat)
+        assert len(re.findall(r"\bglobal_load_dwordx4", funcs[k])) >= 4, k
+        assert "scratch_" not in funcs[k], k
