@@ -115,29 +115,35 @@ __device__ __forceinline__ void rows_stream(const uint8_t* w0, const uint8_t* w1
 #pragma unroll
             for (int t = 0; t < NT; t++) acc[t] = float4v{0.f, 0.f, 0.f, 0.f};
         }
-        // this lane's weight rows: row 16 wave + j of the block, in every tensor.  One tensor's tile after the
-        // other: one set of fragment registers and decode temporaries alive at a time; the waves of the SIMD
-        // fill each other's matrix-instruction latencies
+        // this lane's weight rows: row 16 wave + j of the block, in every tensor.  The tensors' tiles go through a
+        // matrix-instruction step side by side: the activation operand of the step is read from LDS once for
+        // both (its 2 KB per wave and step are the largest share of the workgroup's LDS traffic)
         const uint32_t skew = (uint32_t)((base_of(b) + (size_t)(16 * wave + j) * stride + (size_t)f * FB) & 15);
         const half8* ap = (const half8*)(s_a + buf * G::A_BYTES) + lane;
+        F w[NT];
+        float4v part[NT];
 #pragma unroll
         for (int t = 0; t < NT; t++) {
-            asm volatile("" ::: "memory"); // the second tile reads its activation operands again rather than keeping the first's 64 registers
-            F w;
-            w.load(s_w + (size_t)(t * MR_ROWS + 16 * wave + j) * WIN + skew, 0, g);
-            float4v part = float4v{0.f, 0.f, 0.f, 0.f};
+            w[t].load(s_w + (size_t)(t * MR_ROWS + 16 * wave + j) * WIN + skew, 0, g);
+            part[t] = float4v{0.f, 0.f, 0.f, 0.f};
+        }
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const half8 ahi = ap[(size_t)(i * 2) * 64], alo = ap[(size_t)(i * 2 + 1) * 64];
+        for (int i = 0; i < 8; i++) {
+            const half8 ahi = ap[(size_t)(i * 2) * 64], alo = ap[(size_t)(i * 2 + 1) * 64];
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
                 half8 bl;
-                const half8 bh = w.step(i, g, tab, bl);
-                part = mfma16x32(ahi, bh, part);
-                part = mfma16x32(alo, bh, part);
-                if constexpr (F::SPLIT) part = mfma16x32(ahi, bl, part);
-                __builtin_amdgcn_sched_barrier(0); // keep the decode of later steps from piling up in registers
+                const half8 bh = w[t].step(i, g, tab, bl);
+                part[t] = mfma16x32(ahi, bh, part[t]);
+                part[t] = mfma16x32(alo, bh, part[t]);
+                if constexpr (F::SPLIT) part[t] = mfma16x32(ahi, bl, part[t]);
             }
-            const float sc = w.post();
-            acc[t] += float4v{sc * part[0], sc * part[1], sc * part[2], sc * part[3]};
+            __builtin_amdgcn_sched_barrier(0); // keep the decode of later steps from piling up in registers
+        }
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const float sc = w[t].post();
+            acc[t] += float4v{sc * part[t][0], sc * part[t][1], sc * part[t][2], sc * part[t][3]};
         }
         if (wrap) done(b, acc);
         if (more) {
