@@ -679,3 +679,21 @@ def test_results_do_not_depend_on_the_order_of_the_threads(qk, emu, switches_bac
                 assert all(np.array_equal(a, b) for a, b in zip(got, want[k_])), (k_, mode, seed)
     finally:
         L.emu_set_schedule(0, 1)
+
+
+def test_mixers_and_engine_under_a_random_thread_order(qk, emu, tmp_path, monkeypatch, switches_back_to_defaults):
+    """The attention and gated-DeltaNet kernels (both forms each) and the engine's captured steps with every switch
+    on, once more with the threads of a workgroup visited in a random order and waves held back at random: the same
+    checks against the CPU mirrors and the oracle's state machine as in ascending order."""
+    L = emu_util.emu_lib(qk)
+    L.emu_set_schedule(2, 21)
+    try:
+        test_attention_blocks_inside_their_tensors(qk, emu, 8, 2, 45, 19)
+        test_attention_decode_inside_its_tensors(qk, emu)
+        for fused in (False, True):
+            test_deltanet_step_inside_its_tensors(qk, emu, fused)
+        every = {"QK_ONE_ROW": "stream", "QK_DENSE_REG": "1", "QK_FUSED_NORM": "1", "QK_ATTN_BLOCK": "1", "QK_DN_FUSED": "1",
+                 "QK_GEMM_TILED": "1", "QK_MOE_ROWS": "1", "QK_HEAD_ROWS": "1"}
+        test_whole_model_stream_in_the_host_build(qk, emu, tmp_path, monkeypatch, every, None)
+    finally:
+        L.emu_set_schedule(0, 1)
