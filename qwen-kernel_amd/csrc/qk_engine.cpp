@@ -760,8 +760,8 @@ bool qk_engine::open(const char* path, const qk_config& cfg, char* err, size_t e
         else fprintf(stderr, "QK_PREFILL_ROWS=%s out of range [16,1024]; using %u\n", pr, pf_rows);
     }
     if (const char* pc = getenv("QK_PCACHE")) { // reference src/main.cpp:4121-4125
-        const long v = strtol(pc, nullptr, 10);
-        if (v >= 1 && v <= 256) n_state = (uint32_t)v;
+        const long entries = strtol(pc, nullptr, 10);
+        if (entries >= 1 && entries <= 256) n_state = (uint32_t)entries;
     }
     if (const char* mb = getenv("QK_MAXB")) { // reference src/main.cpp:3834-3838
         const long x = atol(mb);
