@@ -26,7 +26,8 @@
  * QK_NO_BATCH (serial prefill of the whole prompt), QK_PCACHE (state snapshot entries, 1..256, default 3);
  * and QK_PREFILL_ROWS (rows of one prefill
  * pass, 16..1024, default 1024: how the prefilled positions are cut, not which are prefilled),
- * QK_NO_GRAPH (launch the step's kernels one by one instead of replaying the graph);
+ * QK_NO_GRAPH (launch the step's kernels one by one instead of replaying the graph), QK_WEIGHT_SLAB=1 (the file's
+ * tensors carved from one device allocation instead of one each);
  * QK_STEP_PROF, as in the reference (src/main.cpp:4591-4632): the first decode step of slot 0 alone is launched
  * kernel by kernel with an event behind every stage and the stages' times go to stderr once
  * ("[prof] decode step: ... us on-GPU across N stages", one line per stage name; QK_STEP_PROF_DETAIL adds every

@@ -78,6 +78,10 @@ struct qk_engine {
     // device side
     hipStream_t st = nullptr;
     std::vector<void*> dev_allocs;
+    // QK_WEIGHT_SLAB=1: the tensors of the file are carved from ONE allocation instead of one each (whether many
+    // separate mappings cost the one-row step address translations is a question for a device; default off)
+    uint8_t* slab = nullptr;
+    size_t slab_bytes = 0, slab_used = 0;
     const void* d_embd = nullptr;
     const void* d_head = nullptr;
     const float* d_onorm = nullptr;
@@ -176,6 +180,7 @@ qk_engine::~qk_engine()
 // Device memory the engine owns until it closes, 256 spare bytes behind it; nullptr on failure.
 void qk_engine::dev_free(const void* p)
 {
+    if (slab && (const uint8_t*)p >= slab && (const uint8_t*)p < slab + slab_bytes) return; // carved from the slab: stays until close
     for (size_t i = 0; i < dev_allocs.size(); i++)
         if (dev_allocs[i] == p) {
             (void)hipFree(dev_allocs[i]);
@@ -187,6 +192,13 @@ void qk_engine::dev_free(const void* p)
 void* qk_engine::dev_alloc(size_t bytes, bool zero)
 {
     void* p = nullptr;
+    const size_t take = (bytes + 256 + 255) & ~(size_t)255; // the slab hands out 256-byte aligned pieces, the spare bytes included
+    if (slab && slab_used + take <= slab_bytes) {
+        p = slab + slab_used;
+        slab_used += take;
+        if (zero && hipMemset(p, 0, bytes + 256) != hipSuccess) return nullptr;
+        return p;
+    }
     if (hipMalloc(&p, bytes + 256) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
     dev_allocs.push_back(p);
     if (zero && hipMemset(p, 0, bytes + 256) != hipSuccess) return nullptr;
@@ -845,6 +857,18 @@ bool qk_engine::open(const char* path, const qk_config& cfg, char* err, size_t e
         return false;
     }
     if (hipStreamCreateWithFlags(&st, hipStreamNonBlocking) != hipSuccess) return bad("qk_open: cannot create a stream");
+    if (const char* sl = getenv("QK_WEIGHT_SLAB"); sl && atoi(sl) == 1) {
+        uint64_t tensors = 0; // every tensor of the file at most once, each with its spare bytes and alignment
+        for (uint64_t i = 0; i < qkg_n_tensors(g); i++) {
+            qkg_tensor t;
+            if (qkg_tensor_at(g, i, &t) == 0) tensors += t.nbytes + 512;
+        }
+        void* sp = nullptr;
+        if (hipMalloc(&sp, tensors) != hipSuccess) { (void)hipGetLastError(); return bad("qk_open: device memory exhausted"); }
+        dev_allocs.push_back(sp);
+        slab = (uint8_t*)sp;
+        slab_bytes = tensors;
+    }
 
     const void* p = nullptr;
     if (!upload(t_embd, &d_embd, err, err_len) || !upload(t_head, &d_head, err, err_len) ||

@@ -153,6 +153,9 @@ def test_whole_model_modes_in_the_host_build(qk_emu, whole_model):
     many = run(qk_emu, "token", ids, 3, 64, 12, env={**env, "QK_MOE_ROWS": "1", "QK_HEAD_ROWS": "1"}, timeout=600)
     assert many.returncode == 0 and "streams identical: YES" in many.stdout, many.stdout + many.stderr
     assert gen_of(many.stdout) == gen_of(one.stdout)[:3]
+    # QK_WEIGHT_SLAB=1: the file's tensors carved from one device allocation; the same stream
+    slab = run(qk_emu, "token", ids, 5, 64, env={**env, "QK_WEIGHT_SLAB": "1"})
+    assert slab.returncode == 0 and gen_of(slab.stdout) == gen_of(one.stdout), slab.stdout + slab.stderr
     # QK_STEP_PROF (reference src/main.cpp:4591-4632): the first decode step's stages on stderr, once, the stream unchanged
     prof = run(qk_emu, "token", ids, 5, 64, env={**env, "QK_STEP_PROF": "1", "QK_STEP_PROF_DETAIL": "1"})
     assert prof.returncode == 0 and gen_of(prof.stdout) == gen_of(one.stdout), prof.stdout + prof.stderr
